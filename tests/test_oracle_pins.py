@@ -1,0 +1,308 @@
+"""Pins for the CPU oracle: each check is independent of the oracle's own formula
+(float64 brute force, a library routine, or a mathematical invariant), chosen so that a
+dropped term, wrong sign/index or transposed operand fails it."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import flashsvd_oracle as O
+
+torch.manual_seed(1234)
+
+
+def _rand(*shape, dtype=torch.float32, scale=1.0, seed=None):
+    g = torch.Generator().manual_seed(seed if seed is not None else int(np.prod(shape)) % 9973)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+# ---------------------------------------------------------------- linear pair
+def test_lin_matches_float64_loops():
+    x, w = _rand(3, 7), _rand(5, 7)
+    ref = np.zeros((3, 5))
+    for i in range(3):
+        for o in range(5):
+            for k in range(7):
+                ref[i, o] += float(x[i, k]) * float(w[o, k])
+    assert np.allclose(O.lin(x, w).numpy(), ref, atol=1e-6)
+
+
+def test_lowrank_pair_full_rank_is_dense_linear():
+    d = 16
+    q, _ = torch.linalg.qr(_rand(d, d))
+    W = _rand(24, d)
+    # v = Q^T (orthonormal, [R=d, in]), u = W Q -> u v = W
+    y = O.lowrank_pair(_rand(4, d, seed=5), q.t().contiguous(), (W @ q).contiguous())
+    assert torch.allclose(y, torch.nn.functional.linear(_rand(4, d, seed=5), W), atol=1e-5)
+
+
+def test_lin_bf16_rounds_once_from_fp32():
+    x, w = _rand(2, 64, dtype=torch.bfloat16), _rand(8, 64, dtype=torch.bfloat16)
+    exact = (x.double() @ w.double().t())
+    y = O.lin(x, w)
+    assert y.dtype == torch.bfloat16
+    # one bf16 rounding of an (almost) exact sum: error <= 1/2 ulp (2^-9 relative) + fp32 noise
+    assert torch.all((y.double() - exact).abs() <= exact.abs() * 2 ** -8 + 1e-6)
+
+
+# ---------------------------------------------------------------- rmsnorm
+def test_rms_norm_matches_transformers():
+    from transformers.models.llama.modeling_llama import LlamaRMSNorm
+    for dt in (torch.float32, torch.bfloat16):
+        n = LlamaRMSNorm(32, eps=1e-6).to(dt)
+        with torch.no_grad():
+            n.weight.copy_(_rand(32, seed=3).to(dt))
+        x = _rand(2, 3, 32, dtype=dt, seed=4)
+        assert torch.equal(O.rms_norm(x, n.weight.detach(), 1e-6), n(x).detach())
+
+
+# ---------------------------------------------------------------- rope
+def test_rope_tables_closed_form():
+    cos, sin = O.rope_tables(9, 8, 10000.0)
+    for p in (0, 1, 8):
+        for i in range(4):
+            a = p * 10000.0 ** (-i / 4)
+            assert abs(float(cos[p, i]) - math.cos(a)) < 1e-5
+            assert abs(float(sin[p, i]) - math.sin(a)) < 1e-5
+    assert torch.all(cos[0] == 1) and torch.all(sin[0] == 0)
+
+
+def test_rope_invariants():
+    Dh = 16
+    cos, sin = O.rope_tables(40, Dh)
+    q, k = _rand(Dh, seed=1), _rand(Dh, seed=2)
+    # position 0 is the identity
+    assert torch.equal(O.apply_rope(q, cos[0], sin[0]), q)
+    # norm preserved per (i, i+half) pair
+    r = O.apply_rope(q, cos[17], sin[17])
+    assert torch.allclose(r[:8] ** 2 + r[8:] ** 2, q[:8] ** 2 + q[8:] ** 2, atol=1e-5)
+    # <rope(q,m), rope(k,n)> depends only on n-m
+    d1 = O.apply_rope(q, cos[3], sin[3]) @ O.apply_rope(k, cos[10], sin[10])
+    d2 = O.apply_rope(q, cos[23], sin[23]) @ O.apply_rope(k, cos[30], sin[30])
+    assert abs(float(d1 - d2)) < 1e-4
+    # and differs for another offset (a sign error in sin keeps norms but breaks this)
+    d3 = O.apply_rope(q, cos[3], sin[3]) @ O.apply_rope(k, cos[11], sin[11])
+    assert abs(float(d1 - d3)) > 1e-4
+
+
+def test_rope_matches_transformers_apply_rotary():
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    Dh, T = 16, 6
+    for dt in (torch.float32, torch.bfloat16):
+        cos_h, sin_h = O.rope_tables(T, Dh, dtype=dt)
+        cos = torch.cat([cos_h, cos_h], -1)[None]
+        sin = torch.cat([sin_h, sin_h], -1)[None]
+        q = _rand(1, 2, T, Dh, dtype=dt, seed=7)  # [B,H,T,Dh]
+        k = _rand(1, 2, T, Dh, dtype=dt, seed=8)
+        qe, ke = apply_rotary_pos_emb(q, k, cos, sin)
+        mine = O.apply_rope(q, cos_h[None, None], sin_h[None, None])
+        assert torch.allclose(mine.float(), qe.float(), atol=0 if dt == torch.float32 else 2 ** -7 * 4)
+        if dt == torch.float32:
+            assert torch.allclose(O.apply_rope_fp32(k, cos_h[None, None], sin_h[None, None]), ke, atol=1e-6)
+
+
+# ---------------------------------------------------------------- reconstruct
+def test_reconstruct_variants_agree_and_match_flat_gemm():
+    B, H, Hk, R, Dh = 2, 4, 2, 24, 8
+    Pq, Pk, Pv = _rand(B, R, seed=1), _rand(B, R, seed=2), _rand(B, R, seed=3)
+    Vq, Vk, Vv = _rand(H, R, Dh, seed=4), _rand(Hk, R, Dh, seed=5), _rand(Hk, R, Dh, seed=6)
+    bq, bk, bv = _rand(H, Dh, seed=7), _rand(Hk, Dh, seed=8), _rand(Hk, Dh, seed=9)
+    Qs, Ks, Vs = O.reconstruct_qkv_token_shared(Pq, Pk, Pv, Vq, Vk, Vv, bq, bk, bv)
+    # brute force
+    ref = np.zeros((B, H, Dh))
+    for b in range(B):
+        for h in range(H):
+            for d in range(Dh):
+                ref[b, h, d] = sum(float(Pq[b, r]) * float(Vq[h, r, d]) for r in range(R)) + float(bq[h, d])
+    assert np.allclose(Qs.numpy(), ref, atol=1e-5)
+    # headwise with broadcast P == shared
+    Qh, Kh, Vh = O.reconstruct_qkv_token(Pq[:, None].expand(B, H, R), Pk[:, None].expand(B, Hk, R),
+                                         Pv[:, None].expand(B, Hk, R), Vq, Vk, Vv, bq, bk, bv)
+    assert torch.allclose(Qh, Qs, atol=1e-6) and torch.allclose(Kh, Ks, atol=1e-6) and torch.allclose(Vh, Vs, atol=1e-6)
+    # prepacked == shared; flat identity
+    fq, fk, fv = O.pack_qkv_shared_bases(Vq, Vk, Vv)
+    assert fq.shape == (R, H * Dh)
+    Qp, Kp, Vp = O.reconstruct_qkv_token_shared_prepacked(Pq, Pk, Pv, fq, fk, fv, H=H, Hk=Hk, Dh=Dh, bq=bq, bk=bk, bv=bv)
+    assert torch.allclose(Qp, Qs, atol=1e-5) and torch.allclose(Kp, Ks, atol=1e-5) and torch.allclose(Vp, Vs, atol=1e-5)
+    assert torch.allclose((Pk @ fk)[:, Dh:2 * Dh] + bk[1], Ks[:, 1], atol=1e-5)
+    # hetero ranks
+    Q2, K2, V2 = O.reconstruct_qkv_token_shared_hetero(Pq, Pk[:, :16], Pv[:, :8], Vq, Vk[:, :16], Vv[:, :8])
+    assert torch.allclose(K2, torch.einsum("br,hrd->bhd", Pk[:, :16], Vk[:, :16]), atol=1e-5)
+    assert torch.allclose(V2, torch.einsum("br,hrd->bhd", Pv[:, :8], Vv[:, :8]), atol=1e-5)
+
+
+# ---------------------------------------------------------------- decode attention
+def test_dense_decode_attn_matches_sdpa_gqa():
+    B, H, Hk, L, Dh = 2, 4, 2, 9, 8
+    q, k, v = _rand(B, H, Dh, seed=1), _rand(B, L, Hk, Dh, seed=2), _rand(B, L, Hk, Dh, seed=3)
+    out = O.dense_decode_attn(q, k, v)
+    kk = k.permute(0, 2, 1, 3).repeat_interleave(H // Hk, dim=1)
+    vv = v.permute(0, 2, 1, 3).repeat_interleave(H // Hk, dim=1)
+    ref = torch.nn.functional.scaled_dot_product_attention(q[:, :, None], kk, vv)[:, :, 0]
+    assert torch.allclose(out, ref, atol=1e-5)
+
+
+def test_flash_attn_with_kvcache_append_then_attend():
+    B, H, Hk, Dh, S = 2, 4, 2, 8, 12
+    cos, sin = O.rope_tables(S, Dh)
+    kraw, vraw = _rand(B, S, Hk, Dh, seed=1), _rand(B, S, Hk, Dh, seed=2)
+    qraw = _rand(B, S, H, Dh, seed=3)
+    n = 7
+    kc = torch.zeros(B, S, Hk, Dh)
+    vc = torch.zeros(B, S, Hk, Dh)
+    kc[:, :n] = O.apply_rope_fp32(kraw[:, :n], cos[:n][None, :, None], sin[:n][None, :, None])
+    vc[:, :n] = vraw[:, :n]
+    seqlens = torch.full((B,), n, dtype=torch.int32)
+    out = O.flash_attn_with_kvcache(qraw[:, n:n + 1], kc, vc, k=kraw[:, n:n + 1], v=vraw[:, n:n + 1],
+                                    cache_seqlens=seqlens, rotary_cos=cos, rotary_sin=sin, causal=True)
+    # cache mutated at position n
+    assert torch.allclose(kc[:, n], O.apply_rope_fp32(kraw[:, n], cos[n], sin[n]))
+    assert torch.equal(vc[:, n], vraw[:, n]) and torch.all(kc[:, n + 1:] == 0)
+    # equals last row of full causal SDPA over n+1 rotated tokens
+    qr = O.apply_rope_fp32(qraw[:, :n + 1], cos[:n + 1][None, :, None], sin[:n + 1][None, :, None])
+    kr = O.apply_rope_fp32(kraw[:, :n + 1], cos[:n + 1][None, :, None], sin[:n + 1][None, :, None])
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        qr.permute(0, 2, 1, 3), kr.permute(0, 2, 1, 3).repeat_interleave(2, 1),
+        vraw[:, :n + 1].permute(0, 2, 1, 3).repeat_interleave(2, 1), is_causal=True)
+    assert torch.allclose(out[:, 0], ref[:, :, -1], atol=1e-5)
+
+
+def test_rank_decode_equals_dense_on_reconstructed_kv_and_is_block_invariant():
+    B, H, Hk, L, R, Dh = 2, 4, 2, 37, 12, 8
+    cos, sin = O.rope_tables(L, Dh)
+    q = _rand(B, H, Dh, seed=1)
+    Pk, Pv = _rand(B, L, R, seed=2), _rand(B, L, R, seed=3)
+    Vk, Vv = _rand(Hk, R, Dh, seed=4), _rand(Hk, R, Dh, seed=5)
+    K = torch.einsum("blr,krd->blkd", Pk, Vk)
+    V = torch.einsum("blr,krd->blkd", Pv, Vv)
+    Kr = O.apply_rope_fp32(K, cos[None, :, None], sin[None, :, None])
+    ref = O.dense_decode_attn(q, Kr, V)
+    outs = [O.rank_decode_attn(q, Pk, Pv, Vk, Vv, cos, sin, BN=bn) for bn in (1, 5, 16, 64)]
+    for o in outs:
+        assert torch.allclose(o, ref, atol=2e-5)
+    # V-absorption identity: sum_n p_n (Pv_n Vv) == (sum_n p_n Pv_n) Vv
+    scores = torch.einsum("bkgd,blkd->bkgl", q.reshape(B, Hk, 2, Dh), Kr) / math.sqrt(Dh)
+    p = torch.softmax(scores, -1)
+    absorbed = torch.einsum("bkgr,krd->bkgd", torch.einsum("bkgl,blr->bkgr", p, Pv), Vv).reshape(B, H, Dh)
+    assert torch.allclose(absorbed, ref, atol=2e-5)
+    # headwise variant with expanded shared P agrees
+    hw = O.rank_decode_attn_headwise(q, Pk[:, :, None].expand(B, L, Hk, R), Pv[:, :, None].expand(B, L, Hk, R), Vk, Vv, cos, sin)
+    assert torch.allclose(hw, ref, atol=2e-5)
+
+
+# ---------------------------------------------------------------- fused prefill
+def test_rope_sdpa_prefill_equals_reconstruct_rope_sdpa():
+    B, H, Hk, M, R, dh = 2, 4, 2, 11, 6, 8
+    cos, sin = O.rope_tables(M, dh)
+    Pq, Pk, Pv = _rand(B, H, M, R, seed=1), _rand(B, Hk, M, R, seed=2), _rand(B, Hk, M, R, seed=3)
+    Vq, Vk, Vv = _rand(H, R, dh, seed=4), _rand(Hk, R, dh, seed=5), _rand(Hk, R, dh, seed=6)
+    out = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin)
+    q = O.apply_rope_fp32(torch.einsum("bhmr,hrd->bhmd", Pq, Vq), cos[None, None], sin[None, None])
+    k = O.apply_rope_fp32(torch.einsum("bhmr,hrd->bhmd", Pk, Vk), cos[None, None], sin[None, None])
+    v = torch.einsum("bhmr,hrd->bhmd", Pv, Vv)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k.repeat_interleave(2, 1), v.repeat_interleave(2, 1), is_causal=True)
+    assert torch.allclose(out, ref.permute(0, 2, 1, 3), atol=1e-5)
+    # last row == decode over the same keys
+    dec = O.dense_decode_attn(q[:, :, -1], k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3))
+    assert torch.allclose(out[:, -1], dec, atol=1e-5)
+    # left-padded batch row: padded keys masked; a query whose keys are all masked gives 0
+    pad = torch.ones(B, M, dtype=torch.long)
+    pad[1, :3] = 0
+    outp = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin, pad_mask=pad)
+    assert torch.all(outp[1, :3] == 0)
+    assert torch.allclose(outp[0], out[0], atol=1e-6)
+    ref1 = torch.nn.functional.scaled_dot_product_attention(
+        q[1:, :, 3:], k[1:, :, 3:].repeat_interleave(2, 1), v[1:, :, 3:].repeat_interleave(2, 1), is_causal=True)
+    assert torch.allclose(outp[1, 3:], ref1[0].permute(1, 0, 2), atol=1e-5)
+
+
+# ---------------------------------------------------------------- MLP
+def test_dual_split_closed_form_and_partition_invariance():
+    B, L, R, D, Hd = 2, 1, 10, 37, 12
+    PUp, PGate = _rand(B, L, R, seed=1), _rand(B, L, R, seed=2)
+    GateU, UpU = _rand(R, D, seed=3), _rand(R, D, seed=4)
+    DownV, DownU, b2 = _rand(D, R, seed=5), _rand(R, Hd, seed=6), _rand(Hd, seed=7)
+    y = O.dual_split_mlp(PUp, PGate, GateU, UpU, DownV, DownU, b2)
+    g = (PGate.double() @ GateU.double())
+    u = (PUp.double() @ UpU.double())
+    ref = ((g / (1 + torch.exp(-g))) * u) @ DownV.double() @ DownU.double() + b2.double()
+    assert torch.allclose(y.double(), ref, atol=1e-5)
+    # swapping gate/up must change the answer (catches transposed operands)
+    assert not torch.allclose(O.dual_split_mlp(PGate, PUp, GateU, UpU, DownV, DownU, b2).double(), ref, atol=1e-3)
+    for bd in (1, 8, 16, 64):
+        assert torch.allclose(O.dual_split_mlp(PUp, PGate, GateU, UpU, DownV, DownU, b2, BD=bd), y, atol=1e-5)
+    assert torch.allclose(O.dual_split_mlp_pcat(torch.cat([PUp, PGate], -1), GateU, UpU, DownV, DownU, b2), y, atol=1e-6)
+    assert torch.allclose(O.dual_split_mlp_v3(PUp, PGate, GateU, UpU, DownV, DownU, b2, BD=16, BR2=4), y, atol=1e-5)
+
+
+def test_mlp_forward_full_rank_is_hf_llama_mlp():
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaMLP
+    d, ffn = 16, 24
+    cfg = LlamaConfig(hidden_size=d, intermediate_size=ffn, hidden_act="silu", mlp_bias=False, num_attention_heads=2)
+    mlp = LlamaMLP(cfg)
+    R = d  # full rank factors: v orthonormal [R,in], u = W v^T
+    qd, _ = torch.linalg.qr(_rand(d, d, seed=1))
+    qf, _ = torch.linalg.qr(_rand(ffn, ffn, seed=2))
+    Wg, Wu, Wd = mlp.gate_proj.weight.detach(), mlp.up_proj.weight.detach(), mlp.down_proj.weight.detach()
+    z = torch.zeros(1)
+    bw = O.BlockWeights(q_v=z, q_u=z, k_v=z, k_u=z, v_v=z, v_u=z, o_v=z, o_u=z,
+                        gate_v=qd.t().contiguous(), gate_u=Wg @ qd, up_v=qd.t().contiguous(), up_u=Wu @ qd,
+                        down_v=qf.t().contiguous(), down_u=Wd @ qf, ln1=z, ln2=z)
+    x = _rand(3, d, seed=3)
+    assert torch.allclose(O.mlp_forward(bw, x), mlp(x).detach(), atol=1e-5)
+
+
+# ---------------------------------------------------------------- whole model
+def _tiny(dtype=torch.float32, n_layers=2, kvh=2):
+    return O.make_model(d=32, n_heads=4, n_kv_heads=kvh, head_dim=8, ffn=48, attn_rank=12, mlp_rank=16,
+                        n_layers=n_layers, vocab=50, dtype=dtype, seed=0, std=0.3)
+
+
+def test_model_matches_transformers_llama_with_dense_weights():
+    from transformers import LlamaConfig, LlamaForCausalLM
+    mw = _tiny()
+    cfg = LlamaConfig(vocab_size=50, hidden_size=32, intermediate_size=48, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=2, head_dim=8, rms_norm_eps=1e-6,
+                      rope_theta=10000.0, attention_bias=False, mlp_bias=False, tie_word_embeddings=False,
+                      max_position_embeddings=64, attn_implementation="eager")
+    hf = LlamaForCausalLM(cfg).eval()
+    with torch.no_grad():
+        hf.model.embed_tokens.weight.copy_(mw.embed)
+        hf.lm_head.weight.copy_(mw.lm_head)
+        hf.model.norm.weight.copy_(mw.norm)
+        for layer, b in zip(hf.model.layers, mw.blocks):
+            a, m = layer.self_attn, layer.mlp
+            a.q_proj.weight.copy_(b.q_u @ b.q_v); a.k_proj.weight.copy_(b.k_u @ b.k_v)
+            a.v_proj.weight.copy_(b.v_u @ b.v_v); a.o_proj.weight.copy_(b.o_u @ b.o_v)
+            m.gate_proj.weight.copy_(b.gate_u @ b.gate_v); m.up_proj.weight.copy_(b.up_u @ b.up_v)
+            m.down_proj.weight.copy_(b.down_u @ b.down_v)
+            layer.input_layernorm.weight.copy_(b.ln1); layer.post_attention_layernorm.weight.copy_(b.ln2)
+    ids = torch.randint(0, 50, (2, 9), generator=torch.Generator().manual_seed(3))
+    with torch.no_grad():
+        ref = hf(input_ids=ids).logits
+    mine = O.model_forward(mw, ids, last_only=False)
+    assert torch.allclose(mine, ref, atol=2e-4, rtol=1e-3)
+
+
+@pytest.mark.parametrize("cache_kind", ["dense", "rank"])
+def test_cached_greedy_decode_equals_full_recompute(cache_kind):
+    mw = _tiny()
+    prompt = torch.randint(0, 50, (2, 6), generator=torch.Generator().manual_seed(5))
+    toks, hid, _ = O.greedy_decode(mw, prompt, 5, cache_kind=cache_kind, return_hidden=True)
+    seq = prompt
+    for step in range(5):
+        logits, h = O.model_forward(mw, seq, return_hidden=True)
+        assert torch.allclose(h[:, -1], hid[:, step], atol=1e-4)
+        nxt = logits[:, -1].argmax(-1, keepdim=True)
+        assert torch.equal(nxt, toks[:, step:step + 1])
+        seq = torch.cat([seq, nxt], 1)
+
+
+def test_rank_cache_and_dense_cache_agree_bf16():
+    mw = _tiny(torch.bfloat16)
+    prompt = torch.randint(0, 50, (1, 8), generator=torch.Generator().manual_seed(6))
+    _, hd, _ = O.greedy_decode(mw, prompt, 4, "dense", return_hidden=True)
+    _, hr, _ = O.greedy_decode(mw, prompt, 4, "rank", return_hidden=True)
+    assert (hd.float() - hr.float()).abs().max() < 0.15  # bf16 noise only; same algebra
