@@ -1,0 +1,215 @@
+// Single-query attention over a dense KV cache [B,S,Hk,Dh] (K stored post-RoPE), split over
+// the key axis so that B*H*nsplit workgroups cover the chip.  Each workgroup scores its key
+// range (16-byte K loads, V_DOT2 against the query chunk held in registers, DPP fold over the
+// lanes that share a key), does a two-pass softmax through LDS, accumulates p*V per lane and
+// writes an un-normalised partial (acc, m, l).  The last workgroup to arrive for a (b,h)
+// merges the partials in split order, so the result does not depend on arrival order.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace fsvd {
+
+constexpr int kAttnThreads = 256;
+constexpr int kMaxKeysPerSplit = 2048;
+
+__device__ __forceinline__ void decode_work_item(int B, int H, int nsplit, int& b, int& h, int& s) {
+  // Consecutive workgroup ids go round-robin over the 8 XCDs; remap so that the splits of one
+  // head (which meet again in the merge) run on the same XCD and share its L2.
+  const int total = B * H * nsplit;
+  int id = blockIdx.x;
+  if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+  s = id % nsplit;
+  h = (id / nsplit) % H;
+  b = id / (nsplit * H);
+}
+
+template <int DH>
+__global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArgs a) {
+  constexpr int LPK = DH / 8;                 // lanes that share one key (8 bf16 each)
+  constexpr int KPB = kAttnThreads / LPK;     // keys per block pass
+  __shared__ float sc[kMaxKeysPerSplit];
+  __shared__ __align__(16) float accs[KPB * DH];
+  __shared__ __align__(16) uint16_t qs[DH];
+  __shared__ float red[8];
+  __shared__ int last_flag;
+
+  int b, h, s;
+  decode_work_item(a.B, a.H, a.nsplit, b, h, s);
+  const int tid = threadIdx.x;
+  const int hk = h / (a.H / a.Hk);
+  int n_keys = a.seqlens[b] + a.seqlen_add;
+  n_keys = max(0, min(n_keys, a.S));
+  int per = (n_keys + a.nsplit - 1) / a.nsplit;
+  per = (per + KPB - 1) / KPB * KPB;
+  const int k0 = min(s * per, n_keys);
+  const int k1 = min(n_keys, k0 + per);
+  const int nk = k1 - k0;
+
+  // query chunk (optionally rotated at position seqlens[b], fp32 math, one rounding)
+  const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)h * a.sq_h;
+  if (tid < DH / 2) {
+    float x0 = bf16_bits_to_f32(qp[tid]), x1 = bf16_bits_to_f32(qp[tid + DH / 2]);
+    if (a.cos) {
+      const int tp = min(max(a.seqlens[b], 0), a.rope_len - 1);
+      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * (DH / 2) + tid]);
+      const float sn = bf16_bits_to_f32(a.sin[(int64_t)tp * (DH / 2) + tid]);
+      const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
+      x0 = r0; x1 = r1;
+    }
+    qs[tid] = (uint16_t)f32_to_bf16_bits(x0);
+    qs[tid + DH / 2] = (uint16_t)f32_to_bf16_bits(x1);
+  }
+  __syncthreads();
+  const int part = tid % LPK, slot = tid / LPK;
+  const u32x4_t qv = *reinterpret_cast<const u32x4_t*>(qs + part * 8);
+
+  // pass 1: scaled scores into LDS
+  const uint16_t* kbase = a.k_cache + (int64_t)b * a.sc_b + (int64_t)hk * a.sc_h + part * 8;
+  float lmax = -INFINITY;
+  for (int j = slot; j < nk; j += KPB) {
+    const u32x4_t kv = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)(k0 + j) * a.sc_s);
+    float d = dot8_bf16(kv, qv, 0.f);
+    d += dpp_f32<0xB1>(d);
+    d += dpp_f32<0x4E>(d);
+    d += dpp_f32<0x141>(d);
+    if (LPK == 16) d += dpp_f32<0x140>(d);
+    d *= a.scale;
+    if (part == 0) sc[j] = d;
+    lmax = fmaxf(lmax, d);
+  }
+  lmax = wave_max(lmax);
+  if ((tid & 63) == 0) red[tid >> 6] = lmax;
+  __syncthreads();
+  float m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  // pass 2: p = exp(s - m), l = sum p
+  float lsum = 0.f;
+  for (int j = tid; j < nk; j += kAttnThreads) {
+    const float p = __expf(sc[j] - m);
+    sc[j] = p;
+    lsum += p;
+  }
+  lsum = wave_sum(lsum);
+  if ((tid & 63) == 0) red[4 + (tid >> 6)] = lsum;
+  __syncthreads();
+  const float l = (red[4] + red[5]) + (red[6] + red[7]);
+
+  // pass 3: acc[d] = sum_j p_j V[j,d]
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  const uint16_t* vbase = a.v_cache + (int64_t)b * a.sc_b + (int64_t)hk * a.sc_h + part * 8;
+  for (int j = slot; j < nk; j += KPB) {
+    const u32x4_t vv = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)(k0 + j) * a.sc_s);
+    const float p = sc[j];
+    acc[0] += p * bf16_lo(vv.x); acc[1] += p * bf16_hi(vv.x);
+    acc[2] += p * bf16_lo(vv.y); acc[3] += p * bf16_hi(vv.y);
+    acc[4] += p * bf16_lo(vv.z); acc[5] += p * bf16_hi(vv.z);
+    acc[6] += p * bf16_lo(vv.w); acc[7] += p * bf16_hi(vv.w);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) accs[slot * DH + part * 8 + i] = acc[i];
+  __syncthreads();
+  float o = 0.f;
+  if (tid < DH) {
+#pragma unroll 8
+    for (int j = 0; j < KPB; ++j) o += accs[j * DH + tid];
+  }
+
+  uint16_t* outp = a.out + (int64_t)b * a.so_b + (int64_t)h * a.so_h;
+  if (a.nsplit == 1) {
+    if (tid < DH) outp[tid] = (uint16_t)f32_to_bf16_bits(l > 0.f ? o / l : 0.f);
+    return;
+  }
+  float* part_ws = a.ws_part + ((int64_t)(b * a.H + h) * a.nsplit) * (DH + 2);
+  float* mine = part_ws + (int64_t)s * (DH + 2);
+  if (tid < DH) mine[tid] = o;
+  if (tid == 0) { mine[DH] = m; mine[DH + 1] = l; }
+  __threadfence();
+  __syncthreads();
+  if (tid == 0) {
+    const int old = atomicAdd(&a.ws_count[b * a.H + h], 1);
+    last_flag = (old == a.nsplit - 1);
+  }
+  __syncthreads();
+  if (!last_flag) return;
+  __threadfence();
+  if (tid < DH) {
+    float M = -INFINITY;
+    for (int i = 0; i < a.nsplit; ++i) M = fmaxf(M, __builtin_nontemporal_load(part_ws + (int64_t)i * (DH + 2) + DH));
+    float num = 0.f, den = 0.f;
+    for (int i = 0; i < a.nsplit; ++i) {
+      const float* pw = part_ws + (int64_t)i * (DH + 2);
+      const float mi = __builtin_nontemporal_load(pw + DH);
+      const float w = (mi == -INFINITY) ? 0.f : __expf(mi - M);
+      num += w * __builtin_nontemporal_load(pw + tid);
+      den += w * __builtin_nontemporal_load(pw + DH + 1);
+    }
+    outp[tid] = (uint16_t)f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
+  }
+  if (tid == 0) a.ws_count[b * a.H + h] = 0;
+}
+
+// rotate k_new at position seqlens[b] (fp32 math, one rounding) and write k/v into the caches
+__global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
+  const int half = a.Dh >> 1;
+  const int total = a.B * a.Hk * half;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+    const int d = i % half, hk = (i / half) % a.Hk, b = i / (half * a.Hk);
+    const int pos = a.seqlens[b];
+    if (pos < 0 || pos >= a.S) continue;
+    const uint16_t* kp = a.k_new + (int64_t)b * a.sk_b + (int64_t)hk * a.sk_h;
+    const uint16_t* vp = a.v_new + (int64_t)b * a.sv_b + (int64_t)hk * a.sv_h;
+    float x0 = bf16_bits_to_f32(kp[d]), x1 = bf16_bits_to_f32(kp[d + half]);
+    if (a.cos) {
+      const int tp = min(pos, a.rope_len - 1);
+      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * half + d]);
+      const float s = bf16_bits_to_f32(a.sin[(int64_t)tp * half + d]);
+      const float r0 = x0 * c - x1 * s, r1 = x0 * s + x1 * c;
+      x0 = r0; x1 = r1;
+    }
+    const int64_t off = (int64_t)b * a.sc_b + (int64_t)pos * a.sc_s + (int64_t)hk * a.sc_h;
+    a.k_cache[off + d] = (uint16_t)f32_to_bf16_bits(x0);
+    a.k_cache[off + d + half] = (uint16_t)f32_to_bf16_bits(x1);
+    a.v_cache[off + d] = vp[d];
+    a.v_cache[off + d + half] = vp[d + half];
+  }
+}
+
+size_t attn_decode_ws_floats(int B, int H, int nsplit, int Dh) { return (size_t)B * H * nsplit * (Dh + 2); }
+
+int launch_attn_decode(const AttnDecodeArgs& a, hipStream_t st) {
+  if (a.B <= 0 || a.H <= 0 || a.Hk <= 0 || a.H % a.Hk != 0 || a.S <= 0 || a.nsplit <= 0) {
+    set_last_error("fsvd_attn_decode_densekv: bad shape B=%d H=%d Hk=%d S=%d nsplit=%d", a.B, a.H, a.Hk, a.S, a.nsplit);
+    return kErrBadShape;
+  }
+  if (a.Dh != 64 && a.Dh != 128) { set_last_error("fsvd_attn_decode_densekv: head_dim %d not in {64,128}", a.Dh); return kErrBadShape; }
+  const int kpb = kAttnThreads / (a.Dh / 8);
+  const int per = ((a.S + a.nsplit - 1) / a.nsplit + kpb - 1) / kpb * kpb;
+  if (per > kMaxKeysPerSplit) {
+    set_last_error("fsvd_attn_decode_densekv: %d keys per split exceeds %d; raise nsplit", per, kMaxKeysPerSplit);
+    return kErrBadShape;
+  }
+  if ((a.sc_s % 8) || (a.sc_h % 8) || (a.sc_b % 8) || (reinterpret_cast<uintptr_t>(a.k_cache) & 15) ||
+      (reinterpret_cast<uintptr_t>(a.v_cache) & 15)) {
+    set_last_error("fsvd_attn_decode_densekv: cache strides/pointers must be 16-byte aligned");
+    return kErrBadAlign;
+  }
+  if (a.nsplit > 1 && (!a.ws_part || !a.ws_count)) { set_last_error("fsvd_attn_decode_densekv: workspace missing"); return kErrWorkspace; }
+  dim3 grid(a.B * a.H * a.nsplit);
+  if (a.Dh == 128) hipLaunchKernelGGL(attn_decode_kernel<128>, grid, dim3(kAttnThreads), 0, st, a);
+  else hipLaunchKernelGGL(attn_decode_kernel<64>, grid, dim3(kAttnThreads), 0, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("fsvd_attn_decode_densekv: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
+int launch_kv_append(const KvAppendArgs& a, hipStream_t st) {
+  if (a.B <= 0 || a.Hk <= 0 || a.Dh <= 0 || (a.Dh & 1) || a.S <= 0) { set_last_error("fsvd_kv_append: bad shape"); return kErrBadShape; }
+  const int total = a.B * a.Hk * (a.Dh / 2);
+  hipLaunchKernelGGL(kv_append_kernel, dim3((total + 255) / 256), dim3(256), 0, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("fsvd_kv_append: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
+}  // namespace fsvd

@@ -1,0 +1,94 @@
+// Shared device helpers for the gfx950 kernels: bf16 packing, wave64 reductions,
+// status codes of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fsvd {
+
+constexpr int kWave = 64;
+
+// status codes returned by every extern "C" entry point (0 == ok)
+enum Status : int {
+  kOk = 0,
+  kErrBadShape = -1,     // a dimension is out of the supported range
+  kErrBadAlign = -2,     // pointer / stride alignment the kernel needs is missing
+  kErrBadDtype = -3,
+  kErrNullPtr = -4,
+  kErrLaunch = -5,       // hipGetLastError() after the launch
+  kErrWorkspace = -6,    // caller workspace too small
+};
+
+void set_last_error(const char* fmt, ...);
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+
+// round-to-nearest-even fp32 -> bf16 (bit pattern in the low 16 bits)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  __bf16 h = static_cast<__bf16>(f);
+  return static_cast<uint32_t>(__builtin_bit_cast(unsigned short, h));
+}
+// value after one bf16 rounding
+__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// acc += a.lo*b.lo + a.hi*b.hi with fp32 accumulation (V_DOT2_F32_BF16)
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc, false);
+}
+__device__ __forceinline__ float dot8_bf16(const u32x4_t& w, const u32x4_t& x, float acc) {
+  acc = dot2_bf16(w.x, x.x, acc);
+  acc = dot2_bf16(w.y, x.y, acc);
+  acc = dot2_bf16(w.z, x.z, acc);
+  acc = dot2_bf16(w.w, x.w, acc);
+  return acc;
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+// sum over each aligned group of 16 lanes; every lane of the group gets the sum
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f32<0x141>(v);  // row_half_mirror
+  v += dpp_f32<0x140>(v);  // row_mirror
+  return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_f32<0xB1>(v));
+  v = fmaxf(v, dpp_f32<0x4E>(v));
+  v = fmaxf(v, dpp_f32<0x141>(v));
+  v = fmaxf(v, dpp_f32<0x140>(v));
+  return v;
+}
+// sum over the 64 lanes of the wave; the result is wave-uniform
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return (a + b) + (c + d);
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = row16_max(v);
+  float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+
+}  // namespace fsvd

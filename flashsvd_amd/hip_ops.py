@@ -1,0 +1,224 @@
+"""Tensor-level wrappers over the C ABI: shape/dtype/device checks in Python, raw pointers and
+the current torch stream handed to libflashsvd_hip.  PyTorch only provides device memory and
+streams here; every arithmetic step runs in the HIP library."""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_BF16 = torch.bfloat16
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need(t: torch.Tensor, name: str, *, dtype=_BF16) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor, got device {t.device}")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+
+
+def _rows(t: torch.Tensor, name: str) -> torch.Tensor:
+    """View as [rows, last] with unit stride on the last axis (copies only if it must)."""
+    if t.stride(-1) != 1:
+        t = t.contiguous()
+    if t.dim() == 1:
+        return t.unsqueeze(0)
+    if t.dim() == 2:
+        return t
+    try:
+        return t.view(-1, t.shape[-1])
+    except RuntimeError:
+        return t.reshape(-1, t.shape[-1])
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
+           norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
+           residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:
+    """out = (residual +) linear(rmsnorm?(x), weight, bias); weight is nn.Linear layout [N, K]."""
+    _need(x, "x"); _need(weight, "weight")
+    if weight.dim() != 2 or weight.stride(1) != 1:
+        raise ValueError(f"weight must be [N, K] with unit inner stride, got {tuple(weight.shape)} strides {weight.stride()}")
+    N, K = weight.shape
+    if x.shape[-1] != K:
+        raise ValueError(f"x last dim {x.shape[-1]} != weight in_features {K}")
+    x2 = _rows(x, "x")
+    B = x2.shape[0]
+    if out is None:
+        out = torch.empty(*x.shape[:-1], N, device=x.device, dtype=_BF16)
+    o2 = _rows(out, "out")
+    if o2.shape != (B, N) or o2.data_ptr() != out.data_ptr():
+        raise ValueError("out must be a dense [..., N] tensor matching x")
+    r2 = None
+    if residual is not None:
+        _need(residual, "residual")
+        r2 = _rows(residual, "residual")
+        if r2.shape != (B, N):
+            raise ValueError(f"residual shape {tuple(residual.shape)} does not match output [{B}, {N}]")
+    for t, nm, n in ((bias, "bias", N), (norm_weight, "norm_weight", K)):
+        if t is not None:
+            _need(t, nm)
+            if t.shape != (n,) or not t.is_contiguous():
+                raise ValueError(f"{nm} must be a contiguous [{n}] tensor")
+    lib = _lib.load()
+    rc = lib.fsvd_linear(x2.data_ptr(), x2.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias), _ptr(norm_weight),
+                         float(eps), _ptr(r2), 0 if r2 is None else r2.stride(0), o2.data_ptr(), o2.stride(0),
+                         B, N, K, int(cfg), _stream())
+    _lib.check("fsvd_linear", rc)
+    return out
+
+
+def swiglu_linear(p: torch.Tensor, gate_u: torch.Tensor, up_u: torch.Tensor, *, up_off: int, mode: int = 0,
+                  out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:
+    """h = silu(p[..., :R] @ gate_u.T) * (p[..., up_off:up_off+R] @ up_u.T); gate_u/up_u are [D, R]."""
+    _need(p, "p"); _need(gate_u, "gate_u"); _need(up_u, "up_u")
+    if gate_u.dim() != 2 or gate_u.shape != up_u.shape or gate_u.stride() != up_u.stride() or gate_u.stride(1) != 1:
+        raise ValueError(f"gate_u/up_u must be matching [D, R] weights, got {tuple(gate_u.shape)} / {tuple(up_u.shape)}")
+    D, R = gate_u.shape
+    p2 = _rows(p, "p")
+    if p2.shape[1] < up_off + R:
+        raise ValueError(f"p last dim {p2.shape[1]} too small for up_off {up_off} + R {R}")
+    B = p2.shape[0]
+    if out is None:
+        out = torch.empty(*p.shape[:-1], D, device=p.device, dtype=_BF16)
+    o2 = _rows(out, "out")
+    lib = _lib.load()
+    rc = lib.fsvd_swiglu_linear(p2.data_ptr(), p2.stride(0), int(up_off), gate_u.data_ptr(), up_u.data_ptr(),
+                                gate_u.stride(0), o2.data_ptr(), o2.stride(0), B, D, R, int(mode), int(cfg), _stream())
+    _lib.check("fsvd_swiglu_linear", rc)
+    return out
+
+
+def qkv_rope_append(p: torch.Tensor, q_u: torch.Tensor, k_u: torch.Tensor, v_u: torch.Tensor,
+                    cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
+                    k_cache: torch.Tensor, v_cache: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int,
+                    q_out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:
+    """q (rotated) -> q_out [B,H,Dh]; rotated k and v written into the caches [B,S,Hk,Dh] at positions[b]."""
+    for t, nm in ((p, "p"), (q_u, "q_u"), (k_u, "k_u"), (v_u, "v_u"), (k_cache, "k_cache"), (v_cache, "v_cache")):
+        _need(t, nm)
+    _need(positions, "positions", dtype=torch.int32)
+    H, Hk, Dh = int(num_heads), int(num_kv_heads), int(head_dim)
+    Rq, Rk, Rv = q_u.shape[1], k_u.shape[1], v_u.shape[1]
+    if q_u.shape[0] != H * Dh or k_u.shape[0] != Hk * Dh or v_u.shape[0] != Hk * Dh:
+        raise ValueError(f"u_proj rows do not match heads: {tuple(q_u.shape)}/{tuple(k_u.shape)}/{tuple(v_u.shape)} "
+                         f"for H={H} Hk={Hk} Dh={Dh}")
+    p2 = _rows(p, "p")
+    B = p2.shape[0]
+    if p2.shape[1] != Rq + Rk + Rv:
+        raise ValueError(f"p last dim {p2.shape[1]} != Rq+Rk+Rv = {Rq + Rk + Rv}")
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.stride() != v_cache.stride() \
+            or k_cache.shape[2:] != (Hk, Dh) or k_cache.shape[0] < B or k_cache.stride(3) != 1:
+        raise ValueError(f"caches must be matching [B>={B}, S, {Hk}, {Dh}] tensors, got {tuple(k_cache.shape)}")
+    if positions.numel() != B or not positions.is_contiguous():
+        raise ValueError(f"positions must be a contiguous int32 [{B}] tensor")
+    rope_len = 0
+    if cos is not None:
+        _need(cos, "cos"); _need(sin, "sin")
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2 or not cos.is_contiguous() or not sin.is_contiguous():
+            raise ValueError(f"cos/sin must be contiguous [len, {Dh // 2}] tables")
+        rope_len = cos.shape[0]
+    if q_out is None:
+        q_out = torch.empty(B, H, Dh, device=p.device, dtype=_BF16)
+    elif q_out.shape != (B, H, Dh) or not q_out.is_contiguous():
+        raise ValueError("q_out must be contiguous [B,H,Dh]")
+    lib = _lib.load()
+    rc = lib.fsvd_qkv_rope_append(p2.data_ptr(), p2.stride(0), q_u.data_ptr(), q_u.stride(0), k_u.data_ptr(), k_u.stride(0),
+                                  v_u.data_ptr(), v_u.stride(0), _ptr(cos), _ptr(sin), rope_len, positions.data_ptr(),
+                                  q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                  k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+                                  B, H, Hk, Dh, Rq, Rk, Rv, k_cache.shape[1], int(cfg), _stream())
+    _lib.check("fsvd_qkv_rope_append", rc)
+    return q_out
+
+
+def pick_nsplit(max_len: int, batch: int, heads: int, head_dim: int = 128) -> int:
+    """Key-axis split so that batch*heads*nsplit workgroups fill 256 CUs, within the per-split key cap."""
+    want = max(1, math.ceil(512 / max(1, batch * heads)))
+    need = math.ceil(max_len / 1024)
+    n = max(want, need)
+    return int(min(n, max(1, math.ceil(max_len / 16))))
+
+
+def attn_workspace(batch: int, heads: int, head_dim: int, nsplit: int, device) -> torch.Tensor:
+    lib = _lib.load()
+    nbytes = lib.fsvd_attn_decode_workspace_bytes(batch, heads, head_dim, nsplit)
+    return torch.zeros(max(1, (nbytes + 3) // 4), dtype=torch.int32, device=device)
+
+
+def attn_decode_densekv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cache_seqlens: torch.Tensor, *,
+                        k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
+                        cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, seqlen_add: int = 0,
+                        nsplit: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
+                        out: Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None) -> torch.Tensor:
+    """q [B,H,Dh] over caches [B,S,Hk,Dh]; see fsvd_attn_decode_densekv in include/flashsvd_hip.h."""
+    _need(q, "q"); _need(k_cache, "k_cache"); _need(v_cache, "v_cache")
+    _need(cache_seqlens, "cache_seqlens", dtype=torch.int32)
+    if q.dim() != 3 or q.stride(2) != 1:
+        raise ValueError(f"q must be [B,H,Dh] with unit inner stride, got {tuple(q.shape)}")
+    B, H, Dh = q.shape
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.stride() != v_cache.stride() \
+            or k_cache.shape[3] != Dh or k_cache.shape[0] < B or k_cache.stride(3) != 1:
+        raise ValueError(f"caches must be matching [B>={B}, S, Hk, {Dh}] tensors, got {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
+    S, Hk = k_cache.shape[1], k_cache.shape[2]
+    if H % Hk != 0:
+        raise ValueError(f"H={H} is not a multiple of Hk={Hk}")
+    if cache_seqlens.numel() != B or not cache_seqlens.is_contiguous():
+        raise ValueError(f"cache_seqlens must be a contiguous int32 [{B}] tensor")
+    sn_b = sn_h = 0
+    if k_new is not None:
+        _need(k_new, "k_new"); _need(v_new, "v_new")
+        if k_new.shape != (B, Hk, Dh) or v_new.shape != (B, Hk, Dh) or k_new.stride() != v_new.stride() or k_new.stride(2) != 1:
+            raise ValueError(f"k_new/v_new must be matching [B,Hk,Dh] tensors, got {tuple(k_new.shape)} / {tuple(v_new.shape)}")
+        sn_b, sn_h = k_new.stride(0), k_new.stride(1)
+    rope_len = 0
+    if cos is not None:
+        _need(cos, "cos"); _need(sin, "sin")
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2 or not cos.is_contiguous() or not sin.is_contiguous():
+            raise ValueError(f"cos/sin must be contiguous [len, {Dh // 2}] tables")
+        rope_len = cos.shape[0]
+    if nsplit is None:
+        nsplit = pick_nsplit(S, B, H, Dh)
+    if out is None:
+        out = torch.empty(B, H, Dh, device=q.device, dtype=_BF16)
+    elif out.shape != (B, H, Dh) or out.stride(2) != 1:
+        raise ValueError("out must be [B,H,Dh] with unit inner stride")
+    lib = _lib.load()
+    ws_ptr, ws_bytes = None, 0
+    if nsplit > 1:
+        if workspace is None:
+            workspace = attn_workspace(B, H, Dh, nsplit, q.device)
+        ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    rc = lib.fsvd_attn_decode_densekv(q.data_ptr(), q.stride(0), q.stride(1), k_cache.data_ptr(), v_cache.data_ptr(),
+                                      k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+                                      _ptr(k_new), _ptr(v_new), sn_b, sn_h, cache_seqlens.data_ptr(), int(seqlen_add),
+                                      _ptr(cos), _ptr(sin), rope_len, out.data_ptr(), out.stride(0), out.stride(1),
+                                      ws_ptr, ws_bytes, B, H, Hk, Dh, S, int(nsplit),
+                                      float(softmax_scale) if softmax_scale else 0.0, _stream())
+    _lib.check("fsvd_attn_decode_densekv", rc)
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _need(x, "x"); _need(weight, "weight")
+    K = x.shape[-1]
+    if weight.shape != (K,) or not weight.is_contiguous():
+        raise ValueError(f"weight must be contiguous [{K}]")
+    x2 = _rows(x, "x")
+    if out is None:
+        out = torch.empty_like(x, memory_format=torch.contiguous_format)
+    o2 = _rows(out, "out")
+    lib = _lib.load()
+    rc = lib.fsvd_rmsnorm(x2.data_ptr(), x2.stride(0), weight.data_ptr(), float(eps), o2.data_ptr(), o2.stride(0),
+                          x2.shape[0], K, _stream())
+    _lib.check("fsvd_rmsnorm", rc)
+    return out

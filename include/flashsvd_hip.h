@@ -1,0 +1,99 @@
+/*
+ * libflashsvd_hip — C ABI of the MI355X (gfx950) low-rank decode kernels.
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless it says "host";
+ *   - tensors are bf16 (uint16 bit patterns) unless a dtype argument says otherwise;
+ *   - leading dimensions / strides are in ELEMENTS;
+ *   - `stream` is a hipStream_t (NULL = the default stream); launches are asynchronous;
+ *   - the return value is 0 on success and a negative FSVD_ERR_* code otherwise, with a
+ *     human-readable message available from fsvd_last_error() (thread-local);
+ *   - no entry point allocates or frees device memory: scratch is passed in by the caller.
+ *
+ * Reference paths cited below are relative to the FlashSVD checkout.
+ */
+#ifndef FLASHSVD_HIP_H_
+#define FLASHSVD_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FSVD_OK 0
+#define FSVD_ERR_BAD_SHAPE (-1)
+#define FSVD_ERR_BAD_ALIGN (-2)
+#define FSVD_ERR_BAD_DTYPE (-3)
+#define FSVD_ERR_NULL_PTR (-4)
+#define FSVD_ERR_LAUNCH (-5)
+#define FSVD_ERR_WORKSPACE (-6)
+
+/* dtype codes for the entry points that take one (the reference kernels switch on
+ * USE_BF16 / USE_FP32, kernels/attn/decode/densekv_reconstruct_triton.py:427-428) */
+#define FSVD_BF16 0
+#define FSVD_FP16 1
+#define FSVD_FP32 2
+
+int fsvd_version(void);
+const char* fsvd_last_error(void);
+
+/* y[b,n] = (res[b,n] +) bf16( W[n,:] . norm(x[b,:]) (+ bias[n]) ),  W is an nn.Linear weight [N,K].
+ * norm_w != NULL fuses the RMSNorm of x (w * bf16(x * rsqrt(mean(x^2)+eps))) in front.
+ * Replaces the factor GEMVs the reference issues through torch: rank projection
+ * `hidden @ packed_qkv_rank` (benchmark/attn/decode_compare.py:1538), `o_u_proj(o_v_proj(.))`
+ * (utils/model_utils.py:332-341), `up_v_proj/gate_v_proj` (benchmark/mlp/bench_svd_llama_decode_graph.py:133),
+ * phase-2 `matmul(S, DownU)` (kernels/mlp/decode/dual_split_triton.py:719-721) and RMSNorm
+ * (benchmark/mlp/bench_svd_llama_decode_graph.py:78-83).  cfg = 0 picks the tiling. */
+int fsvd_linear(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* bias,
+                const void* norm_w, float eps, const void* res, int64_t ldres,
+                void* y, int64_t ldy, int B, int N, int K, int cfg, void* stream);
+
+/* h[b,n] = silu(gate_u[n,:] . p[b,0:R]) * (up_u[n,:] . p[b,up_off:up_off+R]),  gate_u/up_u [D,R].
+ * mode 0 rounds like a chain of bf16 nn.Linear modules, mode 1 like the fused reference kernel
+ * (h = bf16(silu(g32)*u32), kernels/mlp/decode/dual_split_triton.py:207). */
+int fsvd_swiglu_linear(const void* p, int64_t ldp, int64_t up_off, const void* gate_u, const void* up_u,
+                       int64_t ldw, void* h, int64_t ldh, int B, int D, int R, int mode, int cfg, void* stream);
+
+/* Current-token q/k/v from packed rank coefficients p[b] = [Pq|Pk|Pv] and nn.Linear-layout
+ * u_proj weights, rotate-half RoPE on q and k at positions[b] (eager bf16 arithmetic), q to
+ * q_out [B,H,Dh], k/v appended to the dense caches [B,S,Hk,Dh] at positions[b].
+ * Fuses reconstruct_qkv_token_shared* (kernels/attn/decode/densekv_reconstruct_triton.py:464-659)
+ * with the rotary + cache write the reference leaves to flash_attn_with_kvcache
+ * (runtime/attn/decode_registry.py:177-211) and prepare_fa2_direct_write_step
+ * (runtime/cache/attn_dense_kv.py:258-311).  cos/sin [rope_len, Dh/2] may be NULL (no rotation). */
+int fsvd_qkv_rope_append(const void* p, int64_t ldp, const void* q_u, int64_t ldq, const void* k_u, int64_t ldk,
+                         const void* v_u, int64_t ldv, const void* cos, const void* sin, int rope_len,
+                         const int32_t* positions, void* q_out, void* k_cache, void* v_cache,
+                         int64_t sc_b, int64_t sc_s, int64_t sc_h,
+                         int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int S, int cfg, void* stream);
+
+/* Bytes of scratch fsvd_attn_decode_densekv needs: fp32 partials followed by int32 counters.
+ * The counters must be zero before the first call; the kernel leaves them zero. */
+size_t fsvd_attn_decode_workspace_bytes(int B, int H, int Dh, int nsplit);
+
+/* Single-query attention over a dense KV cache; the role of flash-attn's
+ * flash_attn_with_kvcache in the reference (runtime/attn/decode_registry.py:177-211,
+ * benchmark/attn/decode_compare.py:530-566).  q [B,H,Dh]; caches [B,S,Hk,Dh];
+ * if k_new/v_new [B,Hk,Dh] are given they are rotated (cos/sin given) and written at
+ * cache_seqlens[b] first, then attention runs over cache_seqlens[b]+1 keys; otherwise over
+ * cache_seqlens[b]+seqlen_add keys.  cos/sin != NULL also rotates q at cache_seqlens[b].
+ * softmax scale = 1/sqrt(Dh) when scale <= 0.  out [B,H,Dh]. */
+int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h,
+                             void* k_cache, void* v_cache, int64_t sc_b, int64_t sc_s, int64_t sc_h,
+                             const void* k_new, const void* v_new, int64_t sn_b, int64_t sn_h,
+                             const int32_t* cache_seqlens, int seqlen_add,
+                             const void* cos, const void* sin, int rope_len,
+                             void* out, int64_t so_b, int64_t so_h,
+                             void* workspace, size_t workspace_bytes,
+                             int B, int H, int Hk, int Dh, int S, int nsplit, float scale, void* stream);
+
+/* y = w * bf16(x * rsqrt(mean(x^2)+eps)) over rows of length K.
+ * benchmark/mlp/bench_svd_llama_decode_graph.py:78-83. */
+int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHSVD_HIP_H_ */

@@ -1,0 +1,154 @@
+"""GPU parity of the projection / attention primitives against the CPU oracle, called through
+the C ABI (flashsvd_amd.hip_ops -> libflashsvd_hip.so).  Tolerance: bf16 outputs within
+max-abs 2e-2 and max-rel 1e-2 of the oracle on the same seeded inputs."""
+import math
+
+import pytest
+import torch
+
+from oracle import flashsvd_oracle as O
+from tests.util import assert_close_bf16, rand_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from flashsvd_amd import hip_ops
+    return hip_ops
+
+
+@pytest.mark.parametrize("B,N,K", [(1, 3072, 4096), (1, 1536, 11008), (1, 4096, 1536), (1, 4096, 1024),
+                                   (2, 257, 512), (3, 64, 264), (5, 33, 1492), (1, 7, 100), (8, 128, 4096)])
+def test_linear_plain(ops, B, N, K):
+    x, w = rand_bf16(B, K, seed=1), rand_bf16(N, K, std=0.02, seed=2)
+    y = ops.linear(x.cuda(), w.cuda())
+    assert_close_bf16(y, O.lin(x, w), f"linear {B}x{N}x{K}")
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 4, 0x101, 0x102])
+def test_linear_tilings_agree(ops, cfg):
+    x, w = rand_bf16(1, 2048, seed=3), rand_bf16(515, 2048, std=0.02, seed=4)
+    y = ops.linear(x.cuda(), w.cuda(), cfg=cfg)
+    assert_close_bf16(y, O.lin(x, w), f"cfg {cfg:#x}")
+
+
+def test_linear_norm_bias_residual(ops):
+    B, N, K = 2, 512, 4096
+    x, w = rand_bf16(B, K, seed=1), rand_bf16(N, K, std=0.02, seed=2)
+    nw, bias, res = rand_bf16(K, seed=3) * 0.1 + 1, rand_bf16(N, std=0.1, seed=4), rand_bf16(B, N, seed=5)
+    y = ops.linear(x.cuda(), w.cuda(), bias.cuda(), norm_weight=nw.cuda(), eps=1e-6, residual=res.cuda())
+    ref = res + O.lin(O.rms_norm(x, nw, 1e-6), w, bias)
+    assert_close_bf16(y, ref, "norm+bias+residual")
+
+
+def test_linear_strided_rows(ops):
+    # x and out are row slices of wider buffers; weight is a row slice of a packed matrix
+    xw = rand_bf16(2, 3000, seed=1).cuda()
+    W = rand_bf16(300, 1024, std=0.02, seed=2).cuda()
+    outw = torch.zeros(2, 500, dtype=torch.bfloat16, device="cuda")
+    y = ops.linear(xw[:, 8:8 + 1024], W[100:228])
+    assert_close_bf16(y, O.lin(xw[:, 8:1032].cpu(), W[100:228].cpu()), "strided")
+
+
+def test_rmsnorm(ops):
+    x, w = rand_bf16(3, 4096, seed=1), rand_bf16(4096, seed=2) * 0.1 + 1
+    assert_close_bf16(ops.rmsnorm(x.cuda(), w.cuda(), 1e-6), O.rms_norm(x, w, 1e-6), "rmsnorm")
+
+
+@pytest.mark.parametrize("B,D,R,mode", [(1, 11008, 1536, 0), (1, 11008, 1536, 1), (3, 1376, 256, 0), (2, 100, 52, 1)])
+def test_swiglu_linear(ops, B, D, R, mode):
+    p = rand_bf16(B, 2 * R, seed=1)
+    gu, uu = rand_bf16(D, R, std=0.05, seed=2), rand_bf16(D, R, std=0.05, seed=3)
+    h = ops.swiglu_linear(p.cuda(), gu.cuda(), uu.cuda(), up_off=R, mode=mode)
+    g, u = p[:, :R].float() @ gu.float().t(), p[:, R:].float() @ uu.float().t()
+    if mode == 0:
+        ref = torch.nn.functional.silu(g.to(torch.bfloat16)) * u.to(torch.bfloat16)
+    else:
+        ref = ((g * torch.sigmoid(g)) * u).to(torch.bfloat16)
+    assert_close_bf16(h, ref, f"swiglu mode {mode}")
+
+
+@pytest.mark.parametrize("B,H,Hk,Dh,Rq,Rk,Rv", [(1, 32, 32, 128, 1024, 1024, 1024), (2, 8, 2, 64, 128, 96, 72), (3, 4, 4, 64, 52, 52, 52)])
+def test_qkv_rope_append(ops, B, H, Hk, Dh, Rq, Rk, Rv):
+    S = 40
+    p = rand_bf16(B, Rq + Rk + Rv, seed=1)
+    qu, ku, vu = rand_bf16(H * Dh, Rq, std=0.05, seed=2), rand_bf16(Hk * Dh, Rk, std=0.05, seed=3), rand_bf16(Hk * Dh, Rv, std=0.05, seed=4)
+    cos, sin = O.rope_tables(S, Dh, dtype=torch.bfloat16)
+    pos = torch.tensor([(7 * b + 5) % S for b in range(B)], dtype=torch.int32)
+    kc = torch.zeros(B, S, Hk, Dh, dtype=torch.bfloat16, device="cuda")
+    vc = torch.zeros_like(kc)
+    q = ops.qkv_rope_append(p.cuda(), qu.cuda(), ku.cuda(), vu.cuda(), cos.cuda(), sin.cuda(), pos.cuda(), kc, vc,
+                            num_heads=H, num_kv_heads=Hk, head_dim=Dh)
+    pq, pk, pv = p[:, :Rq], p[:, Rq:Rq + Rk], p[:, Rq + Rk:]
+    for b in range(B):
+        c, s = cos[pos[b]], sin[pos[b]]
+        qr = O.apply_rope(O.lin(pq[b:b + 1], qu).reshape(H, Dh), c, s)
+        kr = O.apply_rope(O.lin(pk[b:b + 1], ku).reshape(Hk, Dh), c, s)
+        vr = O.lin(pv[b:b + 1], vu).reshape(Hk, Dh)
+        assert_close_bf16(q[b], qr, "q")
+        assert_close_bf16(kc[b, pos[b]], kr, "k row")
+        assert_close_bf16(vc[b, pos[b]], vr, "v row")
+    # nothing else in the caches was touched
+    mask = torch.ones(B, S, dtype=torch.bool)
+    for b in range(B):
+        mask[b, pos[b]] = False
+    assert torch.all(kc.cpu()[mask] == 0) and torch.all(vc.cpu()[mask] == 0)
+
+
+@pytest.mark.parametrize("B,H,Hk,Dh,L,S,nsplit", [(1, 32, 32, 128, 512, 560, 8), (1, 32, 32, 128, 513, 560, 16),
+                                                 (2, 8, 2, 64, 37, 64, 3), (3, 4, 4, 128, 1, 16, 2),
+                                                 (1, 32, 8, 128, 4096, 4100, 16), (2, 4, 4, 64, 100, 128, 1)])
+def test_attn_decode_densekv_prerotated(ops, B, H, Hk, Dh, L, S, nsplit):
+    q = rand_bf16(B, H, Dh, seed=1)
+    kc, vc = rand_bf16(B, S, Hk, Dh, seed=2), rand_bf16(B, S, Hk, Dh, seed=3)
+    lens = torch.tensor([max(1, L - 3 * b) for b in range(B)], dtype=torch.int32)
+    out = ops.attn_decode_densekv(q.cuda(), kc.cuda(), vc.cuda(), lens.cuda(), nsplit=nsplit)
+    for b in range(B):
+        n = int(lens[b])
+        ref = O.dense_decode_attn(q[b:b + 1], kc[b:b + 1, :n], vc[b:b + 1, :n])
+        assert_close_bf16(out[b:b + 1], ref, f"attn b={b}")
+
+
+def test_attn_decode_two_calls_same_workspace(ops):
+    # counters must return to zero so that a second call (smaller) is still right
+    B, H, Hk, Dh, S = 1, 8, 8, 128, 300
+    ws = ops.attn_workspace(B, H, Dh, 8, "cuda")
+    q = rand_bf16(B, H, Dh, seed=1)
+    kc, vc = rand_bf16(B, S, Hk, Dh, seed=2), rand_bf16(B, S, Hk, Dh, seed=3)
+    for n in (290, 17):
+        lens = torch.tensor([n], dtype=torch.int32)
+        out = ops.attn_decode_densekv(q.cuda(), kc.cuda(), vc.cuda(), lens.cuda(), nsplit=8, workspace=ws)
+        assert_close_bf16(out, O.dense_decode_attn(q, kc[:, :n], vc[:, :n]), f"n={n}")
+
+
+def test_attn_decode_flash_attn_kvcache_contract(ops):
+    B, H, Hk, Dh, S = 2, 8, 4, 128, 96
+    cos, sin = O.rope_tables(S, Dh, dtype=torch.bfloat16)
+    q, kn, vn = rand_bf16(B, H, Dh, seed=1), rand_bf16(B, Hk, Dh, seed=2), rand_bf16(B, Hk, Dh, seed=3)
+    kc, vc = rand_bf16(B, S, Hk, Dh, seed=4), rand_bf16(B, S, Hk, Dh, seed=5)
+    lens = torch.tensor([70, 33], dtype=torch.int32)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    ref = O.flash_attn_with_kvcache(q[:, None], kc_ref, vc_ref, k=kn[:, None], v=vn[:, None], cache_seqlens=lens,
+                                    rotary_cos=cos, rotary_sin=sin, causal=True)
+    kcg, vcg = kc.cuda(), vc.cuda()
+    out = ops.attn_decode_densekv(q.cuda(), kcg, vcg, lens.cuda(), k_new=kn.cuda(), v_new=vn.cuda(), cos=cos.cuda(), sin=sin.cuda(), nsplit=4)
+    assert_close_bf16(out, ref[:, 0], "fa2 contract out")
+    assert_close_bf16(kcg, kc_ref, "k cache after append")
+    assert torch.equal(vcg.cpu(), vc_ref)
+
+
+def test_errors_are_python_exceptions(ops):
+    x, w = rand_bf16(1, 64).cuda(), rand_bf16(8, 32).cuda()
+    with pytest.raises(ValueError):
+        ops.linear(x, w)
+    with pytest.raises(ValueError):
+        ops.linear(x.float(), rand_bf16(8, 64).cuda())
+    with pytest.raises(ValueError):
+        ops.linear(x.cpu(), rand_bf16(8, 64).cuda())
+    from flashsvd_amd._lib import FlashSVDHipError
+    q = rand_bf16(1, 2, 32).cuda()  # head_dim 32 unsupported
+    kc = rand_bf16(1, 8, 2, 32).cuda()
+    with pytest.raises(FlashSVDHipError):
+        ops.attn_decode_densekv(q, kc, kc.clone(), torch.tensor([4], dtype=torch.int32).cuda(), nsplit=1)
