@@ -551,7 +551,7 @@ def model_forward(mw: ModelWeights, ids: torch.Tensor, pos0: int = 0, cache=None
 
 
 def greedy_decode(mw: ModelWeights, prompt: torch.Tensor, n_new: int, cache_kind: str = "dense",
-                  return_hidden: bool = False):
+                  return_hidden: bool = False, return_logits: bool = False):
     """Prefill yields token 0; each later token is one decode forward at
     cache_position = prompt_len + step.  scripts/demo_support/api.py:285-312,
     benchmark/decode/check_flashsvd_decode_correctness.py:277-322."""
@@ -562,14 +562,18 @@ def greedy_decode(mw: ModelWeights, prompt: torch.Tensor, n_new: int, cache_kind
     cos, sin = rope_tables(max_len, mw.head_dim, mw.rope_theta, dtype)
     logits, hid = model_forward(mw, prompt, 0, cache, cos, sin, return_hidden=True)
     hiddens = [hid[:, -1]]
+    all_logits = [logits[:, -1]]
     tok = logits[:, -1].float().argmax(-1, keepdim=True)
     toks = [tok]
     for step in range(n_new - 1):
         logits, hid = model_forward(mw, tok, Lp + step, cache, cos, sin, return_hidden=True)
         hiddens.append(hid[:, -1])
+        all_logits.append(logits[:, -1])
         tok = logits[:, -1].float().argmax(-1, keepdim=True)
         toks.append(tok)
     out = torch.cat(toks, dim=1)
+    if return_logits:
+        return out, torch.stack(hiddens, dim=1), cache, torch.stack(all_logits, dim=1)
     return (out, torch.stack(hiddens, dim=1), cache) if return_hidden else out
 
 
