@@ -1,0 +1,360 @@
+#!/usr/bin/env python3
+"""Decode benchmark of the low-rank Llama path on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): a 32-layer Llama-2-7B-shaped
+low-rank model (d 4096, 32x128 heads, ffn 11008, attention rank 1024, MLP rank 1536, vocab
+32000, ~0.5 parameter ratio), bf16, random-init factors N(0, 0.02), batch 1, random-token prompt
+of 512, greedy decode with the whole step captured as one HIP graph.
+
+A "step" is one decoded token (one graph replay).  Protocol follows the reference's
+decode_kvcache_eval (utils/evaluator.py:486-522): prefill, W untimed warm-up tokens, then exactly
+K timed tokens between two device synchronisations.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel (gate/up u-projection + SwiGLU,
+67.6 MB of factor bytes per launch), timed live with events around graph replays that launch it
+once per layer over all 32 layers' weights.  `cpu_baseline` is the CPU oracle (fp32, the reference's
+CPU precision) timed on this host on a 2-layer sample and scaled to 32 layers.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+CFG = dict(hidden_size=4096, num_heads=32, num_kv_heads=32, head_dim=128, intermediate_size=11008,
+           num_layers=32, vocab_size=32000, attn_rank=1024, mlp_rank=1536)
+PROMPT_LEN = 512
+HBM_PEAK_GBS = 8000.0
+
+
+def _parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=CFG["num_layers"], help="debug only: fewer layers => INVALID as a headline number")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense bf16 comparator leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kernel-breakdown", action="store_true", help="also time every kernel type of the step")
+    return ap.parse_args()
+
+
+def _median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def time_graph_ms(graph, reps: int, warm: int = 3) -> float:
+    """Median over `reps` of the event time of one replay (events on the current stream)."""
+    import torch
+    for _ in range(warm):
+        graph.replay()
+    torch.cuda.synchronize()
+    out = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        out.append(e0.elapsed_time(e1))
+    return _median(out)
+
+
+def per_layer_kernel_us(fn_per_layer, n_layers: int, reps: int = 10) -> float:
+    """Capture `fn_per_layer(i)` for i in range(n_layers) (cold weights for every launch) into a
+    graph and return the average microseconds per launch, launch gaps included."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(n_layers):
+            fn_per_layer(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(n_layers):
+            fn_per_layer(i)
+    # subtract the replay's fixed cost measured on an empty-ish graph of one launch? no: keep it in (conservative)
+    return time_graph_ms(g, reps) * 1000.0 / n_layers
+
+
+def kernel_legs(model, cache, dec):
+    """name -> (launch closure over layer index, algorithmic bytes per launch)."""
+    import torch
+    from flashsvd_amd import hip_ops
+    L = model.model.layers
+    dev = "cuda"
+    d, R, Ra, D = CFG["hidden_size"], CFG["mlp_rank"], CFG["attn_rank"], CFG["intermediate_size"]
+    H, Dh = CFG["num_heads"], CFG["head_dim"]
+    bf = torch.bfloat16
+    x = torch.randn(1, d, device=dev).to(bf)
+    p_attn = torch.randn(1, 3 * Ra, device=dev).to(bf)
+    a_in = torch.randn(1, H * Dh, device=dev).to(bf)
+    po = torch.randn(1, Ra, device=dev).to(bf)
+    p_mlp = torch.randn(1, 2 * R, device=dev).to(bf)
+    h = torch.randn(1, D, device=dev).to(bf)
+    s = torch.randn(1, R, device=dev).to(bf)
+    q = torch.randn(1, H, Dh, device=dev).to(bf)
+    pos = dec.positions
+    outs = dict(p_attn=torch.empty_like(p_attn), q=torch.empty_like(q), a=torch.empty(1, H, Dh, device=dev, dtype=bf),
+                po=torch.empty_like(po), x=torch.empty_like(x), p_mlp=torch.empty_like(p_mlp), h=torch.empty_like(h),
+                s=torch.empty_like(s))
+    for l in L:
+        l.self_attn._ensure_runtime_state()
+        l.mlp._ensure_runtime_state()
+    n_ctx = PROMPT_LEN
+    legs = {
+        "attn_rank_proj(norm+[q_v;k_v;v_v])": (
+            lambda i: hip_ops.linear(x, L[i].self_attn._packed_qkv_v, norm_weight=L[i].input_layernorm.weight, out=outs["p_attn"]),
+            3 * Ra * d * 2 + d * 2 + 3 * Ra * 2),
+        "attn_qkv_u+rope+append": (
+            lambda i: hip_ops.qkv_rope_append(p_attn, L[i].self_attn.q_u_proj.weight, L[i].self_attn.k_u_proj.weight,
+                                              L[i].self_attn.v_u_proj.weight, dec.rope[0], dec.rope[1], pos,
+                                              cache.key_cache[i], cache.value_cache[i], num_heads=H, num_kv_heads=H,
+                                              head_dim=Dh, q_out=outs["q"]),
+            3 * H * Dh * Ra * 2 + 3 * Ra * 2 + 3 * H * Dh * 2),
+        "attn_decode_densekv(L=%d)" % n_ctx: (
+            lambda i: hip_ops.attn_decode_densekv(q, cache.key_cache[i], cache.value_cache[i], pos, seqlen_add=1,
+                                                  nsplit=dec.nsplit, workspace=dec.attn_ws, out=outs["a"]),
+            2 * (n_ctx + 1) * H * Dh * 2 + 2 * H * Dh * 2),
+        "attn_o_v": (lambda i: hip_ops.linear(a_in, L[i].self_attn.o_v_proj.weight, out=outs["po"]), Ra * H * Dh * 2 + H * Dh * 2 + Ra * 2),
+        "attn_o_u+residual": (lambda i: hip_ops.linear(po, L[i].self_attn.o_u_proj.weight, residual=x, out=outs["x"]), d * Ra * 2 + Ra * 2 + 2 * d * 2),
+        "mlp_rank_proj(norm+[gate_v;up_v])": (
+            lambda i: hip_ops.linear(x, L[i].mlp._packed_gu_v, norm_weight=L[i].post_attention_layernorm.weight, out=outs["p_mlp"]),
+            2 * R * d * 2 + d * 2 + 2 * R * 2),
+        "mlp_gate_up_u+swiglu": (
+            lambda i: hip_ops.swiglu_linear(p_mlp, L[i].mlp.gate_u_proj.weight, L[i].mlp.up_u_proj.weight, up_off=R, out=outs["h"]),
+            2 * D * R * 2 + 2 * R * 2 + D * 2),
+        "mlp_down_v": (lambda i: hip_ops.linear(h, L[i].mlp.down_v_proj.weight, out=outs["s"]), R * D * 2 + D * 2 + R * 2),
+        "mlp_down_u+residual": (lambda i: hip_ops.linear(s, L[i].mlp.down_u_proj.weight, residual=x, out=outs["x"]), d * R * 2 + R * 2 + 2 * d * 2),
+    }
+    return legs
+
+
+def run_lowrank(args):
+    import torch
+    from flashsvd_amd import llama
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+
+    cfg = dict(CFG, num_layers=args.layers)
+    model = llama.materialize(llama.build_model(**cfg), "cuda", torch.bfloat16, seed=0)
+    B = 1
+    max_len = PROMPT_LEN + args.warmup + args.steps + 8
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=torch.bfloat16)
+    prompt = torch.randint(0, cfg["vocab_size"], (B, PROMPT_LEN), generator=torch.Generator().manual_seed(1)).cuda()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = model(prompt, past_key_values=cache, cache_position=torch.arange(PROMPT_LEN), logits_to_keep=1)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    tok = out.logits[:, -1].float().argmax(-1, keepdim=True)
+    dec = GraphedDecoder(model, cache, B)
+    dec.set_state(tok, PROMPT_LEN)
+    dec.capture()
+    for _ in range(args.warmup):
+        dec.step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        dec.step()
+    torch.cuda.synchronize()
+    t_decode = time.perf_counter() - t1
+    res = dict(tok_s=B * args.steps / t_decode, ms_per_step=t_decode * 1000.0 / args.steps, prefill_s=t_prefill,
+               last_token=int(dec.tokens[0, 0]))
+    legs = kernel_legs(model, cache, dec)
+    name = "mlp_gate_up_u+swiglu"
+    fn, nbytes = legs[name]
+    us = per_layer_kernel_us(fn, args.layers)
+    res["roofline"] = {"kernel": "swiglu_kernel (" + name + ")", "bound": "hbm", "achieved": nbytes / us / 1e3,
+                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / us / 1e3 / HBM_PEAK_GBS,
+                       "traffic": _traffic("swiglu_kernel"), "bytes_per_launch": nbytes, "us_per_launch": us}
+    if args.kernel_breakdown:
+        kb = {}
+        for nm, (f, nb) in legs.items():
+            u = per_layer_kernel_us(f, args.layers)
+            kb[nm] = {"us": round(u, 3), "bytes": nb, "GB/s": round(nb / u / 1e3, 1), "frac": round(nb / u / 1e3 / HBM_PEAK_GBS, 4)}
+        res["kernels"] = kb
+        tot_b = sum(v["bytes"] for v in kb.values())
+        tot_u = sum(v["us"] for v in kb.values())
+        res["layer_sum"] = {"us": round(tot_u, 2), "bytes": tot_b, "GB/s": round(tot_b / tot_u / 1e3, 1)}
+    # whole-step effective bandwidth: every factor byte + lm_head + KV read once per token
+    n_ctx = PROMPT_LEN + args.warmup + args.steps // 2
+    per_layer = 8 * CFG["hidden_size"] * CFG["attn_rank"] * 2 + 3 * (CFG["hidden_size"] + 2 * CFG["intermediate_size"]) * CFG["mlp_rank"] * 2
+    step_bytes = args.layers * (per_layer + 2 * n_ctx * CFG["num_heads"] * CFG["head_dim"] * 2) + CFG["vocab_size"] * CFG["hidden_size"] * 2
+    res["step_bytes"] = step_bytes
+    res["step_GBs"] = step_bytes / (res["ms_per_step"] * 1e-3) / 1e9
+    del dec, cache, model
+    torch.cuda.empty_cache()
+    return res
+
+
+def _traffic(kernel: str):
+    """HBM bytes per launch from the committed rocprofv3 --pmc summaries, if present."""
+    f = ROOT / "profiles" / "hbm_traffic.json"
+    try:
+        return json.loads(f.read_text())[kernel]["traffic_bytes_per_launch"]
+    except Exception:
+        return None
+
+
+def run_dense(args):
+    """Same model shape with dense bf16 weights, vendor GEMV (torch.matmul -> hipBLASLt) for the
+    projections, torch ops for norm/rotary/SwiGLU, the same HIP decode-attention kernel, whole step
+    captured as one graph.  This is the "same model run as dense bf16 on the same GPU" comparator."""
+    import torch
+    import torch.nn.functional as F
+    from flashsvd_amd import hip_ops
+    from types import SimpleNamespace
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    d, H, Dh, D, V, NL = CFG["hidden_size"], CFG["num_heads"], CFG["head_dim"], CFG["intermediate_size"], CFG["vocab_size"], args.layers
+    bf = torch.bfloat16
+    gen = torch.Generator(device="cuda").manual_seed(0)
+
+    def rn(*s):
+        return (torch.randn(*s, generator=gen, device="cuda") * 0.02).to(bf)
+
+    layers = [dict(wqkv=rn(3 * d, d), wo=rn(d, d), wgu=rn(2 * D, d), wd=rn(d, D), n1=torch.ones(d, device="cuda", dtype=bf),
+                   n2=torch.ones(d, device="cuda", dtype=bf)) for _ in range(NL)]
+    embed, head, nf = rn(V, d), rn(V, d), torch.ones(d, device="cuda", dtype=bf)
+    max_len = PROMPT_LEN + args.warmup + args.steps + 8
+    cfg = SimpleNamespace(num_hidden_layers=NL, rope_theta=10000.0)
+    cache = FlashSVDV15DenseKVCache(cfg, max_batch_size=1, max_cache_len=max_len, device="cuda", dtype=bf)
+    for i in range(NL):
+        cache._ensure_layer_spec(i, h=H, dh=Dh)
+        cache.key_cache[i][:, :PROMPT_LEN].normal_()
+        cache.value_cache[i][:, :PROMPT_LEN].normal_()
+    cos, sin = cache.get_rope_tables(seqlen=max_len, head_dim=Dh, device="cuda", dtype=bf)
+    nsplit = hip_ops.pick_nsplit(max_len, 1, H, Dh)
+    ws = hip_ops.attn_workspace(1, H, Dh, nsplit, "cuda")
+    tokens = torch.zeros(1, 1, dtype=torch.long, device="cuda")
+    positions = torch.full((1,), PROMPT_LEN, dtype=torch.int32, device="cuda")
+
+    def rms(x, w):
+        x32 = x.float()
+        return w * (x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + 1e-6)).to(bf)
+
+    def step():
+        x = embed[tokens[:, 0]]
+        for i, L in enumerate(layers):
+            qkv = F.linear(rms(x, L["n1"]), L["wqkv"]).view(1, 3, H, Dh)
+            c, s = cos[positions.long()][:, None], sin[positions.long()][:, None]
+            q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]
+
+            def rot(t):
+                t0, t1 = t[..., :Dh // 2], t[..., Dh // 2:]
+                return torch.cat([t0 * c - t1 * s, t1 * c + t0 * s], -1)
+            a = hip_ops.attn_decode_densekv(rot(q).contiguous(), cache.key_cache[i], cache.value_cache[i], positions,
+                                            k_new=rot(k).contiguous(), v_new=v.contiguous(), nsplit=nsplit, workspace=ws)
+            x = x + F.linear(a.view(1, d), L["wo"])
+            gu = F.linear(rms(x, L["n2"]), L["wgu"])
+            x = x + F.linear(F.silu(gu[:, :D]) * gu[:, D:], L["wd"])
+        logits = F.linear(rms(x, nf), head)
+        tokens.copy_(logits.argmax(-1, keepdim=True))
+        positions.add_(1)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+            positions.fill_(PROMPT_LEN)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    positions.fill_(PROMPT_LEN)
+    for _ in range(args.warmup):
+        g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        g.replay()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return dict(tok_s=args.steps / dt, ms_per_step=dt * 1000.0 / args.steps)
+
+
+def run_cpu_baseline():
+    """The CPU oracle in fp32 (the precision of the reference's CPU path) on a bounded sample:
+    2 of the 32 layers + final norm + lm_head, prompt 16, 6 greedy tokens; per-token decode time is
+    scaled to 32 layers."""
+    import torch
+    from oracle import flashsvd_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    n_s = 2
+    mw = O.make_model(d=CFG["hidden_size"], n_heads=CFG["num_heads"], n_kv_heads=CFG["num_kv_heads"], head_dim=CFG["head_dim"],
+                      ffn=CFG["intermediate_size"], attn_rank=CFG["attn_rank"], mlp_rank=CFG["mlp_rank"], n_layers=n_s,
+                      vocab=CFG["vocab_size"], dtype=torch.float32, seed=0)
+    prompt = torch.randint(0, CFG["vocab_size"], (1, 16), generator=torch.Generator().manual_seed(1))
+    n_new = 6
+    cache = O.DenseCache(mw, 1, 64, torch.float32)
+    cos, sin = O.rope_tables(64, mw.head_dim, mw.rope_theta, torch.float32)
+    logits = O.model_forward(mw, prompt, 0, cache, cos, sin)
+    tok = logits[:, -1].argmax(-1, keepdim=True)
+    t_layers = t_head = 0.0
+    for s in range(n_new):
+        t0 = time.perf_counter()
+        x = mw.embed[tok]
+        for li in range(n_s):
+            x = O.block_forward(mw, li, x, 16 + s, cache, cos, sin)
+        t1 = time.perf_counter()
+        logits = O.lin(O.rms_norm(x[:, -1:], mw.norm, mw.eps), mw.lm_head)
+        tok = logits[:, -1].argmax(-1, keepdim=True)
+        t2 = time.perf_counter()
+        if s > 0:  # first token warms the allocator
+            t_layers += t1 - t0
+            t_head += t2 - t1
+    per_tok = (t_layers / n_s * CFG["num_layers"] + t_head) / (n_new - 1)
+    return {"value": 1.0 / per_tok, "unit": "tok/s", "cores": int(torch.get_num_threads()), "kind": "port",
+            "sample": f"CPU oracle fp32, {n_s} of 32 layers + lm_head, context 16-21, {n_new - 1} timed greedy tokens, "
+                      f"per-layer time x32 + head time ({per_tok * 1e3:.1f} ms/token)"}
+
+
+def main():
+    args = _parse()
+    if args.gpus != 1:
+        print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); no multi-GPU path exists", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from flashsvd_amd import _lib
+    _lib.load()
+    lr = run_lowrank(args)
+    line = {
+        "metric": "decode tok/s, 7B-shape rank-0.5 bs1", "value": lr["tok_s"], "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": lr["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "32-layer Llama-2-7B-shaped low-rank decode (attn rank 1024, MLP rank 1536, vocab 32000), "
+                               "bs1, prompt 512, greedy, whole step in one HIP graph", "layers": args.layers,
+                   "prompt_len": PROMPT_LEN, "batch": 1, "kv_cache": "dense"},
+        "roofline": lr["roofline"],
+        "step_hbm": {"bytes_per_token": lr["step_bytes"], "GB/s": lr["step_GBs"], "frac_of_peak": lr["step_GBs"] / HBM_PEAK_GBS},
+        "prefill_s": lr["prefill_s"],
+    }
+    if "kernels" in lr:
+        line["kernels"] = lr["kernels"]
+        line["layer_sum"] = lr["layer_sum"]
+    if not args.no_dense:
+        dn = run_dense(args)
+        line["dense_bf16"] = {"tok_s": dn["tok_s"], "ms_per_step": dn["ms_per_step"], "speedup_lowrank_vs_dense": lr["tok_s"] / dn["tok_s"],
+                              "how": "same shape, dense bf16 weights, torch.matmul (hipBLASLt) projections, same attention kernel, one HIP graph"}
+    line["cpu_baseline"] = None if args.no_cpu else run_cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

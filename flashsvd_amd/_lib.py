@@ -29,7 +29,7 @@ SIGNATURES = {
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_attn_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "fsvd_attn_decode_densekv": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
-                                         c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int,
+                                         c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int,
                                          c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
                                          c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "fsvd_rmsnorm": (c_int, [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int, c_int, c_void_p]),

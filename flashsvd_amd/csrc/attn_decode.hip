@@ -1,16 +1,18 @@
 // Single-query attention over a dense KV cache [B,S,Hk,Dh] (K stored post-RoPE), split over
 // the key axis so that B*H*nsplit workgroups cover the chip.  Each workgroup scores its key
-// range (16-byte K loads, V_DOT2 against the query chunk held in registers, DPP fold over the
-// lanes that share a key), does a two-pass softmax through LDS, accumulates p*V per lane and
-// writes an un-normalised partial (acc, m, l).  The last workgroup to arrive for a (b,h)
-// merges the partials in split order, so the result does not depend on arrival order.
+// range in passes of 128 keys: every K and V row of a pass is requested up front (16-byte loads,
+// 16 in flight per lane), scores come from V_DOT2 against the query chunk held in registers with
+// a DPP fold over the lanes that share a key, the softmax is the online (running max / sum)
+// form and p*V accumulates per lane.  The workgroup writes an un-normalised partial (acc, m, l)
+// with write-through stores; the last workgroup to arrive for a (b,h) merges the partials in
+// split order, so the result does not depend on arrival order.
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace fsvd {
 
 constexpr int kAttnThreads = 256;
-constexpr int kMaxKeysPerSplit = 2048;
+constexpr int kMaxKeysPerSplit = 1 << 20;  // the key loop is streamed; only a sanity bound
 
 __device__ __forceinline__ void decode_work_item(int B, int H, int nsplit, int& b, int& h, int& s) {
   // Consecutive workgroup ids go round-robin over the 8 XCDs; remap so that the splits of one
@@ -23,14 +25,20 @@ __device__ __forceinline__ void decode_work_item(int B, int H, int nsplit, int& 
   b = id / (nsplit * H);
 }
 
-template <int DH>
+// coherent (L2-bypassing) scalar accessors for the cross-workgroup partials: the producers write
+// through to memory and the merging workgroup reads from memory, so no L2 write-back / invalidate
+// fence is needed (those serialise per XCD and cost more than the whole kernel)
+__device__ __forceinline__ void st_agent(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float ld_agent(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+template <int DH, int U>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArgs a) {
   constexpr int LPK = DH / 8;                 // lanes that share one key (8 bf16 each)
   constexpr int KPB = kAttnThreads / LPK;     // keys per block pass
-  __shared__ float sc[kMaxKeysPerSplit];
+  constexpr int CH = KPB * U;                 // keys in flight per workgroup
   __shared__ __align__(16) float accs[KPB * DH];
   __shared__ __align__(16) uint16_t qs[DH];
-  __shared__ float red[8];
+  __shared__ float red[2][4];
   __shared__ int last_flag;
 
   int b, h, s;
@@ -43,7 +51,6 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
   per = (per + KPB - 1) / KPB * KPB;
   const int k0 = min(s * per, n_keys);
   const int k1 = min(n_keys, k0 + per);
-  const int nk = k1 - k0;
 
   // query chunk (optionally rotated at position seqlens[b], fp32 math, one rounding)
   const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)h * a.sq_h;
@@ -59,56 +66,74 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
     qs[tid] = (uint16_t)f32_to_bf16_bits(x0);
     qs[tid + DH / 2] = (uint16_t)f32_to_bf16_bits(x1);
   }
-  __syncthreads();
   const int part = tid % LPK, slot = tid / LPK;
-  const u32x4_t qv = *reinterpret_cast<const u32x4_t*>(qs + part * 8);
-
-  // pass 1: scaled scores into LDS
   const uint16_t* kbase = a.k_cache + (int64_t)b * a.sc_b + (int64_t)hk * a.sc_h + part * 8;
-  float lmax = -INFINITY;
-  for (int j = slot; j < nk; j += KPB) {
-    const u32x4_t kv = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)(k0 + j) * a.sc_s);
-    float d = dot8_bf16(kv, qv, 0.f);
-    d += dpp_f32<0xB1>(d);
-    d += dpp_f32<0x4E>(d);
-    d += dpp_f32<0x141>(d);
-    if (LPK == 16) d += dpp_f32<0x140>(d);
-    d *= a.scale;
-    if (part == 0) sc[j] = d;
-    lmax = fmaxf(lmax, d);
-  }
-  lmax = wave_max(lmax);
-  if ((tid & 63) == 0) red[tid >> 6] = lmax;
-  __syncthreads();
-  float m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  // pass 2: p = exp(s - m), l = sum p
-  float lsum = 0.f;
-  for (int j = tid; j < nk; j += kAttnThreads) {
-    const float p = __expf(sc[j] - m);
-    sc[j] = p;
-    lsum += p;
-  }
-  lsum = wave_sum(lsum);
-  if ((tid & 63) == 0) red[4 + (tid >> 6)] = lsum;
-  __syncthreads();
-  const float l = (red[4] + red[5]) + (red[6] + red[7]);
+  const uint16_t* vbase = a.v_cache + (int64_t)b * a.sc_b + (int64_t)hk * a.sc_h + part * 8;
 
-  // pass 3: acc[d] = sum_j p_j V[j,d]
+  float m_run = -INFINITY, l_thr = 0.f;
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  const uint16_t* vbase = a.v_cache + (int64_t)b * a.sc_b + (int64_t)hk * a.sc_h + part * 8;
-  for (int j = slot; j < nk; j += KPB) {
-    const u32x4_t vv = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)(k0 + j) * a.sc_s);
-    const float p = sc[j];
-    acc[0] += p * bf16_lo(vv.x); acc[1] += p * bf16_hi(vv.x);
-    acc[2] += p * bf16_lo(vv.y); acc[3] += p * bf16_hi(vv.y);
-    acc[4] += p * bf16_lo(vv.z); acc[5] += p * bf16_hi(vv.z);
-    acc[6] += p * bf16_lo(vv.w); acc[7] += p * bf16_hi(vv.w);
+  int it = 0;
+  for (int c0 = k0; c0 < k1; c0 += CH, ++it) {
+    // all K and V rows of this pass are requested before anything is consumed
+    u32x4_t kv[U], vv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = min(c0 + u * KPB + slot, k1 - 1);
+      kv[u] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)key * a.sc_s);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = min(c0 + u * KPB + slot, k1 - 1);
+      vv[u] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)key * a.sc_s);
+    }
+    if (it == 0) __syncthreads();  // qs ready
+    const u32x4_t qv = *reinterpret_cast<const u32x4_t*>(qs + part * 8);
+    float sc[U];
+    float lmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float d = dot8_bf16(kv[u], qv, 0.f);
+      d += dpp_f32<0xB1>(d);
+      d += dpp_f32<0x4E>(d);
+      d += dpp_f32<0x141>(d);
+      if (LPK == 16) d += dpp_f32<0x140>(d);
+      sc[u] = (c0 + u * KPB + slot < k1) ? d * a.scale : -INFINITY;
+      lmax = fmaxf(lmax, sc[u]);
+    }
+    lmax = wave_max(lmax);
+    const int rb = it & 1;
+    if ((tid & 63) == 0) red[rb][tid >> 6] = lmax;
+    __syncthreads();
+    const float m_c = fmaxf(fmaxf(red[rb][0], red[rb][1]), fmaxf(red[rb][2], red[rb][3]));
+    const float m_new = fmaxf(m_run, m_c);
+    const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float p = (sc[u] == -INFINITY) ? 0.f : __expf(sc[u] - m_new);
+      psum += p;
+      acc[0] += p * bf16_lo(vv[u].x); acc[1] += p * bf16_hi(vv[u].x);
+      acc[2] += p * bf16_lo(vv[u].y); acc[3] += p * bf16_hi(vv[u].y);
+      acc[4] += p * bf16_lo(vv[u].z); acc[5] += p * bf16_hi(vv[u].z);
+      acc[6] += p * bf16_lo(vv[u].w); acc[7] += p * bf16_hi(vv[u].w);
+    }
+    l_thr = l_thr * alpha + (part == 0 ? psum : 0.f);
+    m_run = m_new;
   }
+  if (it == 0) __syncthreads();
+  // fold the key slots and the per-thread sums
 #pragma unroll
   for (int i = 0; i < 8; ++i) accs[slot * DH + part * 8 + i] = acc[i];
+  float lw = wave_sum(l_thr);
+  __syncthreads();  // red[] of the last pass consumed; accs written
+  if ((tid & 63) == 0) red[0][tid >> 6] = lw;
   __syncthreads();
+  const float l = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+  const float m = m_run;
   float o = 0.f;
   if (tid < DH) {
 #pragma unroll 8
@@ -122,31 +147,31 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
   }
   float* part_ws = a.ws_part + ((int64_t)(b * a.H + h) * a.nsplit) * (DH + 2);
   float* mine = part_ws + (int64_t)s * (DH + 2);
-  if (tid < DH) mine[tid] = o;
-  if (tid == 0) { mine[DH] = m; mine[DH + 1] = l; }
-  __threadfence();
+  if (tid < DH) st_agent(mine + tid, o);
+  if (tid == 0) { st_agent(mine + DH, m); st_agent(mine + DH + 1, l); }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (tid == 0) {
-    const int old = atomicAdd(&a.ws_count[b * a.H + h], 1);
+    const int old = __hip_atomic_fetch_add(&a.ws_count[b * a.H + h], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     last_flag = (old == a.nsplit - 1);
   }
   __syncthreads();
   if (!last_flag) return;
-  __threadfence();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   if (tid < DH) {
     float M = -INFINITY;
-    for (int i = 0; i < a.nsplit; ++i) M = fmaxf(M, __builtin_nontemporal_load(part_ws + (int64_t)i * (DH + 2) + DH));
+    for (int i = 0; i < a.nsplit; ++i) M = fmaxf(M, ld_agent(part_ws + (int64_t)i * (DH + 2) + DH));
     float num = 0.f, den = 0.f;
     for (int i = 0; i < a.nsplit; ++i) {
       const float* pw = part_ws + (int64_t)i * (DH + 2);
-      const float mi = __builtin_nontemporal_load(pw + DH);
+      const float mi = ld_agent(pw + DH);
       const float w = (mi == -INFINITY) ? 0.f : __expf(mi - M);
-      num += w * __builtin_nontemporal_load(pw + tid);
-      den += w * __builtin_nontemporal_load(pw + DH + 1);
+      num += w * ld_agent(pw + tid);
+      den += w * ld_agent(pw + DH + 1);
     }
     outp[tid] = (uint16_t)f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
   }
-  if (tid == 0) a.ws_count[b * a.H + h] = 0;
+  if (tid == 0) __hip_atomic_store(&a.ws_count[b * a.H + h], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // rotate k_new at position seqlens[b] (fp32 math, one rounding) and write k/v into the caches
@@ -196,8 +221,8 @@ int launch_attn_decode(const AttnDecodeArgs& a, hipStream_t st) {
   }
   if (a.nsplit > 1 && (!a.ws_part || !a.ws_count)) { set_last_error("fsvd_attn_decode_densekv: workspace missing"); return kErrWorkspace; }
   dim3 grid(a.B * a.H * a.nsplit);
-  if (a.Dh == 128) hipLaunchKernelGGL(attn_decode_kernel<128>, grid, dim3(kAttnThreads), 0, st, a);
-  else hipLaunchKernelGGL(attn_decode_kernel<64>, grid, dim3(kAttnThreads), 0, st, a);
+  if (a.Dh == 128) hipLaunchKernelGGL((attn_decode_kernel<128, 8>), grid, dim3(kAttnThreads), 0, st, a);
+  else hipLaunchKernelGGL((attn_decode_kernel<64, 4>), grid, dim3(kAttnThreads), 0, st, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("fsvd_attn_decode_densekv: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
   return kOk;

@@ -81,7 +81,7 @@ size_t fsvd_attn_decode_workspace_bytes(int B, int H, int Dh, int nsplit) {
 }
 
 int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h, void* k_cache, void* v_cache, int64_t sc_b,
-                             int64_t sc_s, int64_t sc_h, const void* k_new, const void* v_new, int64_t sn_b, int64_t sn_h,
+                             int64_t sc_s, int64_t sc_h, const void* k_new, int64_t sk_b, int64_t sk_h, const void* v_new, int64_t sv_b, int64_t sv_h,
                              const int32_t* cache_seqlens, int seqlen_add, const void* cos, const void* sin, int rope_len,
                              void* out, int64_t so_b, int64_t so_h, void* workspace, size_t workspace_bytes, int B, int H,
                              int Hk, int Dh, int S, int nsplit, float scale, void* stream) {
@@ -104,7 +104,7 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h, void* k_
     ws_count = reinterpret_cast<int32_t*>(ws_part + attn_decode_ws_floats(B, H, nsplit, Dh));
   }
   if (k_new) {
-    KvAppendArgs ka{cu16(k_new), cu16(v_new), sn_b, sn_h, sn_b, sn_h, u16(k_cache), u16(v_cache), sc_b, sc_s, sc_h,
+    KvAppendArgs ka{cu16(k_new), cu16(v_new), sk_b, sk_h, sv_b, sv_h, u16(k_cache), u16(v_cache), sc_b, sc_s, sc_h,
                     cache_seqlens, cu16(cos), cu16(sin), rope_len, B, Hk, Dh, S};
     int rc = launch_kv_append(ka, st);
     if (rc != kOk) return rc;

@@ -37,10 +37,20 @@ __device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int64_t 
       continue;
     }
     // RMSNorm: y = w * bf16(x * rsqrt(mean(x^2) + eps)), sum in fp32
+    const bool vnorm = vec && ((reinterpret_cast<uintptr_t>(norm_w) & 15) == 0);
     float ss = 0.f;
-    for (int k = tid; k < K; k += kThreads) {
-      float v = bf16_bits_to_f32(src[k]);
-      ss += v * v;
+    if (vnorm) {
+      for (int k = tid * 8; k < K; k += kThreads * 8) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + k);
+        const float a0 = bf16_lo(v.x), a1 = bf16_hi(v.x), a2 = bf16_lo(v.y), a3 = bf16_hi(v.y);
+        const float a4 = bf16_lo(v.z), a5 = bf16_hi(v.z), a6 = bf16_lo(v.w), a7 = bf16_hi(v.w);
+        ss += ((a0 * a0 + a1 * a1) + (a2 * a2 + a3 * a3)) + ((a4 * a4 + a5 * a5) + (a6 * a6 + a7 * a7));
+      }
+    } else {
+      for (int k = tid; k < K; k += kThreads) {
+        float v = bf16_bits_to_f32(src[k]);
+        ss += v * v;
+      }
     }
     ss = wave_sum(ss);
     __syncthreads();  // red[] free
@@ -50,13 +60,26 @@ __device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int64_t 
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) tot += red[w];
     const float rs = rsqrtf(tot / (float)K + eps);
-    for (int k = tid; k < Kp; k += kThreads) {
-      uint16_t o = 0;
-      if (k < K) {
-        float v = round_bf16(bf16_bits_to_f32(src[k]) * rs);
-        o = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(norm_w[k]) * v);
+    if (vnorm) {
+      for (int k = tid * 8; k < K; k += kThreads * 8) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + k);
+        const u32x4_t g = *reinterpret_cast<const u32x4_t*>(norm_w + k);
+        u32x4_t o;
+        o.x = pack_bf16x2(bf16_lo(g.x) * round_bf16(bf16_lo(v.x) * rs), bf16_hi(g.x) * round_bf16(bf16_hi(v.x) * rs));
+        o.y = pack_bf16x2(bf16_lo(g.y) * round_bf16(bf16_lo(v.y) * rs), bf16_hi(g.y) * round_bf16(bf16_hi(v.y) * rs));
+        o.z = pack_bf16x2(bf16_lo(g.z) * round_bf16(bf16_lo(v.z) * rs), bf16_hi(g.z) * round_bf16(bf16_hi(v.z) * rs));
+        o.w = pack_bf16x2(bf16_lo(g.w) * round_bf16(bf16_lo(v.w) * rs), bf16_hi(g.w) * round_bf16(bf16_hi(v.w) * rs));
+        *reinterpret_cast<u32x4_t*>(dst + k) = o;
       }
-      dst[k] = o;
+    } else {
+      for (int k = tid; k < Kp; k += kThreads) {
+        uint16_t o = 0;
+        if (k < K) {
+          float v = round_bf16(bf16_bits_to_f32(src[k]) * rs);
+          o = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(norm_w[k]) * v);
+        }
+        dst[k] = o;
+      }
     }
   }
   __syncthreads();
@@ -79,6 +102,39 @@ __device__ __forceinline__ void dot_rows_vec8(const uint16_t* const (&wrow)[NR],
         u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xrow[r] + b * Kp + k);
         acc[r][b] = dot8_bf16(w[r], xv, acc[r][b]);
       }
+    }
+  }
+}
+
+// the first PF chunks of every row, requested before the activations are staged so that the
+// weight stream is already in flight while the block normalises / copies x
+template <int NR, int PF>
+__device__ __forceinline__ void prefetch_rows(const uint16_t* const (&wrow)[NR], int K, int first, int step,
+                                              u32x4_t (&w)[NR][PF]) {
+#pragma unroll
+  for (int c = 0; c < PF; ++c) {
+    const int k = first + c * step;
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      if (k < K) w[r][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wrow[r] + k));
+      else w[r][c] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+  }
+}
+template <int NR, int PF, int BATCH>
+__device__ __forceinline__ void consume_rows(const u32x4_t (&w)[NR][PF], const uint16_t* const (&xrow)[NR], int Kp, int K,
+                                             int first, int step, float (&acc)[NR][BATCH]) {
+#pragma unroll
+  for (int c = 0; c < PF; ++c) {
+    const int k = first + c * step;
+    if (k < K) {
+#pragma unroll
+      for (int r = 0; r < NR; ++r)
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) {
+          const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xrow[r] + b * Kp + k);
+          acc[r][b] = dot8_bf16(w[r][c], xv, acc[r][b]);
+        }
     }
   }
 }
@@ -133,34 +189,52 @@ template <int BATCH, int ROWS, bool BLOCKROW, bool VEC>
 __global__ __launch_bounds__(kThreads) void linear_kernel(LinearArgs a) {
   extern __shared__ __align__(16) uint16_t smem[];
   __shared__ float red[kWaves * ROWS * BATCH > kWaves ? kWaves * ROWS * BATCH : kWaves];
+  constexpr int PF = (8 / ROWS) > 1 ? (8 / ROWS) : 2;
   const int Kp = (a.K + 7) & ~7;
   const int b0 = blockIdx.y * BATCH;
   const int nb = min(BATCH, a.B - b0);
-  stage_x<BATCH>(a.x + (int64_t)b0 * a.ldx, a.ldx, nb, a.K, Kp, a.norm_w, a.eps, smem, red);
-
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int group = BLOCKROW ? blockIdx.x : blockIdx.x * kWaves + wave;
   const int ngroups = BLOCKROW ? gridDim.x : gridDim.x * kWaves;
   const int first = (BLOCKROW ? tid : lane) * (VEC ? 8 : 1);
   const int step = (BLOCKROW ? kThreads : kWave) * (VEC ? 8 : 1);
   const int ngrp_rows = (a.N + ROWS - 1) / ROWS;
-  // BLOCKROW needs every thread of the block in the loop (barriers inside reduce_acc)
-  for (int g = group; g < ngrp_rows; g += ngroups) {
-    const int n0 = g * ROWS;
-    const uint16_t* wrow[ROWS];
-    const uint16_t* xrow[ROWS];
+
+  const uint16_t* wrow[ROWS];
+  const uint16_t* xrow[ROWS];
+  int g = group;
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      wrow[r] = a.W + (int64_t)min(n0 + r, a.N - 1) * a.ldw;
-      xrow[r] = smem;
-    }
+  for (int r = 0; r < ROWS; ++r) {
+    wrow[r] = a.W + (int64_t)min(max(g, 0) * ROWS + r, a.N - 1) * a.ldw;
+    xrow[r] = smem;
+  }
+  u32x4_t pf[ROWS][PF];
+  bool have_pf = false;
+  if (VEC && g < ngrp_rows) {
+    prefetch_rows<ROWS, PF>(wrow, a.K, first, step, pf);
+    have_pf = true;
+  }
+  stage_x<BATCH>(a.x + (int64_t)b0 * a.ldx, a.ldx, nb, a.K, Kp, a.norm_w, a.eps, smem, red);
+
+  // BLOCKROW needs every thread of the block in the loop (barriers inside reduce_acc)
+  for (; g < ngrp_rows; g += ngroups) {
+    const int n0 = g * ROWS;
     float acc[ROWS][BATCH];
 #pragma unroll
     for (int r = 0; r < ROWS; ++r)
 #pragma unroll
       for (int b = 0; b < BATCH; ++b) acc[r][b] = 0.f;
-    if (VEC) dot_rows_vec8<ROWS, BATCH>(wrow, xrow, Kp, a.K, first, step, acc);
-    else dot_rows_scalar<ROWS, BATCH>(wrow, xrow, Kp, a.K, first, step, acc);
+    int kstart = first;
+    if (have_pf) {
+      consume_rows<ROWS, PF, BATCH>(pf, xrow, Kp, a.K, first, step, acc);
+      kstart = first + PF * step;
+      have_pf = false;
+    } else {
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) wrow[r] = a.W + (int64_t)min(n0 + r, a.N - 1) * a.ldw;
+    }
+    if (VEC) dot_rows_vec8<ROWS, BATCH>(wrow, xrow, Kp, a.K, kstart, step, acc);
+    else dot_rows_scalar<ROWS, BATCH>(wrow, xrow, Kp, a.K, kstart, step, acc);
     reduce_acc<ROWS, BATCH, BLOCKROW>(acc, red);
     // epilogue: lane/thread (r*BATCH+b) stores one value
     const int who = BLOCKROW ? tid : lane;
@@ -192,34 +266,55 @@ __global__ __launch_bounds__(kThreads) void swiglu_kernel(SwigluArgs a) {
   const int Kp = (a.R + 7) & ~7;
   const int b0 = blockIdx.y * BATCH;
   const int nb = min(BATCH, a.B - b0);
-  // two staged vectors per batch row: gate input then up input
-  stage_x<BATCH>(a.p + (int64_t)b0 * a.ldp, a.ldp, nb, a.R, Kp, nullptr, 0.f, smem, red);
-  stage_x<BATCH>(a.p + (int64_t)b0 * a.ldp + a.up_off, a.ldp, nb, a.R, Kp, nullptr, 0.f, smem + BATCH * Kp, red);
-
+  constexpr int PF = (4 / ROWS) > 1 ? (4 / ROWS) : 2;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int group = blockIdx.x * kWaves + wave;
   const int ngroups = gridDim.x * kWaves;
   const int first = lane * (VEC ? 8 : 1), step = kWave * (VEC ? 8 : 1);
   const int ngrp_rows = (a.D + ROWS - 1) / ROWS;
-  for (int g = group; g < ngrp_rows; g += ngroups) {
-    const int n0 = g * ROWS;
-    const uint16_t* wrow[2 * ROWS];
-    const uint16_t* xrow[2 * ROWS];
+  const uint16_t* wrow[2 * ROWS];
+  const uint16_t* xrow[2 * ROWS];
+  int g = group;
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int64_t off = (int64_t)min(n0 + r, a.D - 1) * a.ldw;
-      wrow[r] = a.gate_u + off;
-      wrow[ROWS + r] = a.up_u + off;
-      xrow[r] = smem;
-      xrow[ROWS + r] = smem + BATCH * Kp;
-    }
+  for (int r = 0; r < ROWS; ++r) {
+    const int64_t off = (int64_t)min(g * ROWS + r, a.D - 1) * a.ldw;
+    wrow[r] = a.gate_u + off;
+    wrow[ROWS + r] = a.up_u + off;
+    xrow[r] = smem;
+    xrow[ROWS + r] = smem + BATCH * Kp;
+  }
+  u32x4_t pf[2 * ROWS][PF];
+  bool have_pf = false;
+  if (VEC && g < ngrp_rows) {
+    prefetch_rows<2 * ROWS, PF>(wrow, a.R, first, step, pf);
+    have_pf = true;
+  }
+  // two staged vectors per batch row: gate input then up input
+  stage_x<BATCH>(a.p + (int64_t)b0 * a.ldp, a.ldp, nb, a.R, Kp, nullptr, 0.f, smem, red);
+  stage_x<BATCH>(a.p + (int64_t)b0 * a.ldp + a.up_off, a.ldp, nb, a.R, Kp, nullptr, 0.f, smem + BATCH * Kp, red);
+
+  for (; g < ngrp_rows; g += ngroups) {
+    const int n0 = g * ROWS;
     float acc[2 * ROWS][BATCH];
 #pragma unroll
     for (int r = 0; r < 2 * ROWS; ++r)
 #pragma unroll
       for (int b = 0; b < BATCH; ++b) acc[r][b] = 0.f;
-    if (VEC) dot_rows_vec8<2 * ROWS, BATCH>(wrow, xrow, Kp, a.R, first, step, acc);
-    else dot_rows_scalar<2 * ROWS, BATCH>(wrow, xrow, Kp, a.R, first, step, acc);
+    int kstart = first;
+    if (have_pf) {
+      consume_rows<2 * ROWS, PF, BATCH>(pf, xrow, Kp, a.R, first, step, acc);
+      kstart = first + PF * step;
+      have_pf = false;
+    } else {
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        const int64_t off = (int64_t)min(n0 + r, a.D - 1) * a.ldw;
+        wrow[r] = a.gate_u + off;
+        wrow[ROWS + r] = a.up_u + off;
+      }
+    }
+    if (VEC) dot_rows_vec8<2 * ROWS, BATCH>(wrow, xrow, Kp, a.R, kstart, step, acc);
+    else dot_rows_scalar<2 * ROWS, BATCH>(wrow, xrow, Kp, a.R, kstart, step, acc);
     reduce_acc<2 * ROWS, BATCH, false>(acc, red);
 #pragma unroll
     for (int r = 0; r < ROWS; ++r)
@@ -392,8 +487,7 @@ static int launch_linear_b(const LinearArgs& a, int cfg, hipStream_t st) {
   bool blockrow = (cfg >> 8) & 1;
   if (cfg == 0) {
     blockrow = a.K >= 8192;
-    if (blockrow) rows = 1;
-    else rows = ((int64_t)a.N * a.K >= (int64_t)12 << 20 && a.K <= 4096) ? 2 : 1;
+    rows = (!blockrow && a.N >= 16384) ? 4 : 1;   // long outputs (lm_head) amortise the x reads over 4 rows
   }
   if (BATCH > 1 && rows > 2) rows = 2;
 #define FSVD_LAUNCH_LIN(R, BR)                                                                   \
@@ -468,7 +562,7 @@ static int launch_qkv_b(const QkvArgs& a, int cfg, hipStream_t st) {
   const int nby = (a.B + BATCH - 1) / BATCH;
   const int npairs = (a.H + 2 * a.Hk) * (a.Dh / 2);
   int pairs = cfg & 0xff;
-  if (pairs == 0) pairs = 1;
+  if (pairs == 0) pairs = 2;
 #define FSVD_LAUNCH_QKV(P)                                                                          \
   {                                                                                                 \
     const int groups = (npairs + P - 1) / P;                                                        \

@@ -142,11 +142,12 @@ def qkv_rope_append(p: torch.Tensor, q_u: torch.Tensor, k_u: torch.Tensor, v_u: 
 
 
 def pick_nsplit(max_len: int, batch: int, heads: int, head_dim: int = 128) -> int:
-    """Key-axis split so that batch*heads*nsplit workgroups fill 256 CUs, within the per-split key cap."""
-    want = max(1, math.ceil(512 / max(1, batch * heads)))
-    need = math.ceil(max_len / 1024)
-    n = max(want, need)
-    return int(min(n, max(1, math.ceil(max_len / 16))))
+    """Key-axis split: about 128 keys per workgroup (one pass of loads in flight), bounded so that
+    batch*heads*nsplit stays within ~2048 workgroups."""
+    per_pass = 128 if head_dim >= 128 else 128
+    n = max(1, math.ceil(max_len / per_pass))
+    cap = max(1, 2048 // max(1, batch * heads))
+    return int(max(1, min(n, cap)))
 
 
 def attn_workspace(batch: int, heads: int, head_dim: int, nsplit: int, device) -> torch.Tensor:
@@ -174,12 +175,12 @@ def attn_decode_densekv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
         raise ValueError(f"H={H} is not a multiple of Hk={Hk}")
     if cache_seqlens.numel() != B or not cache_seqlens.is_contiguous():
         raise ValueError(f"cache_seqlens must be a contiguous int32 [{B}] tensor")
-    sn_b = sn_h = 0
+    sk_b = sk_h = sv_b = sv_h = 0
     if k_new is not None:
         _need(k_new, "k_new"); _need(v_new, "v_new")
-        if k_new.shape != (B, Hk, Dh) or v_new.shape != (B, Hk, Dh) or k_new.stride() != v_new.stride() or k_new.stride(2) != 1:
-            raise ValueError(f"k_new/v_new must be matching [B,Hk,Dh] tensors, got {tuple(k_new.shape)} / {tuple(v_new.shape)}")
-        sn_b, sn_h = k_new.stride(0), k_new.stride(1)
+        if k_new.shape != (B, Hk, Dh) or v_new.shape != (B, Hk, Dh) or k_new.stride(2) != 1 or v_new.stride(2) != 1:
+            raise ValueError(f"k_new/v_new must be [B,Hk,Dh] tensors with unit inner stride, got {tuple(k_new.shape)} / {tuple(v_new.shape)}")
+        sk_b, sk_h, sv_b, sv_h = k_new.stride(0), k_new.stride(1), v_new.stride(0), v_new.stride(1)
     rope_len = 0
     if cos is not None:
         _need(cos, "cos"); _need(sin, "sin")
@@ -200,7 +201,7 @@ def attn_decode_densekv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
         ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     rc = lib.fsvd_attn_decode_densekv(q.data_ptr(), q.stride(0), q.stride(1), k_cache.data_ptr(), v_cache.data_ptr(),
                                       k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
-                                      _ptr(k_new), _ptr(v_new), sn_b, sn_h, cache_seqlens.data_ptr(), int(seqlen_add),
+                                      _ptr(k_new), sk_b, sk_h, _ptr(v_new), sv_b, sv_h, cache_seqlens.data_ptr(), int(seqlen_add),
                                       _ptr(cos), _ptr(sin), rope_len, out.data_ptr(), out.stride(0), out.stride(1),
                                       ws_ptr, ws_bytes, B, H, Hk, Dh, S, int(nsplit),
                                       float(softmax_scale) if softmax_scale else 0.0, _stream())

@@ -82,7 +82,7 @@ size_t fsvd_attn_decode_workspace_bytes(int B, int H, int Dh, int nsplit);
  * softmax scale = 1/sqrt(Dh) when scale <= 0.  out [B,H,Dh]. */
 int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h,
                              void* k_cache, void* v_cache, int64_t sc_b, int64_t sc_s, int64_t sc_h,
-                             const void* k_new, const void* v_new, int64_t sn_b, int64_t sn_h,
+                             const void* k_new, int64_t sk_b, int64_t sk_h, const void* v_new, int64_t sv_b, int64_t sv_h,
                              const int32_t* cache_seqlens, int seqlen_add,
                              const void* cos, const void* sin, int rope_len,
                              void* out, int64_t so_b, int64_t so_h,
