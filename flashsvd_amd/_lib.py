@@ -33,6 +33,17 @@ SIGNATURES = {
                                          c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
                                          c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "fsvd_rmsnorm": (c_int, [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "fsvd_xw_linear_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "fsvd_xw_linear": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int,
+                               c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "fsvd_reconstruct_qkv_workspace_bytes": (c_size_t, [c_int] * 8),
+    "fsvd_reconstruct_qkv_token": (c_int, [c_void_p, c_int64, c_int64, c_int64] * 3 + [c_void_p, c_int64, c_int64] * 3
+                                   + [c_void_p, c_int64] * 3 + [c_void_p, c_int64, c_int64] * 3 + [c_int] * 8
+                                   + [c_void_p, c_size_t, c_void_p]),
+    "fsvd_mlp_dual_split_workspace_bytes": (c_size_t, [c_int] * 6),
+    "fsvd_mlp_dual_split": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
+                                    c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
 }
 
 

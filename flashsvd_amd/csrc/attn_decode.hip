@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
   float* mine = part_ws + (int64_t)s * (DH + 2);
   if (tid < DH) st_agent(mine + tid, o);
   if (tid == 0) { st_agent(mine + DH, m); st_agent(mine + DH + 1, l); }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  wait_stores_acked();
   __syncthreads();
   if (tid == 0) {
     const int old = __hip_atomic_fetch_add(&a.ws_count[b * a.H + h], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -2,6 +2,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
 
 #include "../../include/flashsvd_hip.h"
 #include "common.hpp"
@@ -75,9 +76,13 @@ int fsvd_qkv_rope_append(const void* p, int64_t ldp, const void* q_u, int64_t ld
   return launch_qkv(a, cfg, static_cast<hipStream_t>(stream));
 }
 
+// arrival counters (one per (b,h), zero at rest) sit in a fixed-size block at the front of the
+// attention workspace, the fp32 partials behind it
+static constexpr size_t kAttnCounterBytes = 256 * 1024;
+
 size_t fsvd_attn_decode_workspace_bytes(int B, int H, int Dh, int nsplit) {
   if (B <= 0 || H <= 0 || Dh <= 0 || nsplit <= 0) return 0;
-  return attn_decode_ws_floats(B, H, nsplit, Dh) * sizeof(float) + (size_t)B * H * sizeof(int32_t);
+  return kAttnCounterBytes + attn_decode_ws_floats(B, H, nsplit, Dh) * sizeof(float);
 }
 
 int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h, void* k_cache, void* v_cache, int64_t sc_b,
@@ -100,8 +105,12 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h, void* k_
       set_last_error("%s: workspace of %zu bytes needed, %zu given", fn, need, workspace_bytes);
       return kErrWorkspace;
     }
-    ws_part = static_cast<float*>(workspace);
-    ws_count = reinterpret_cast<int32_t*>(ws_part + attn_decode_ws_floats(B, H, nsplit, Dh));
+    if ((size_t)B * H * sizeof(int32_t) > kAttnCounterBytes) {
+      set_last_error("%s: B*H = %d exceeds the %zu arrival counters of the workspace", fn, B * H, kAttnCounterBytes / 4);
+      return kErrBadShape;
+    }
+    ws_count = static_cast<int32_t*>(workspace);
+    ws_part = reinterpret_cast<float*>(static_cast<char*>(workspace) + kAttnCounterBytes);
   }
   if (k_new) {
     KvAppendArgs ka{cu16(k_new), cu16(v_new), sk_b, sk_h, sv_b, sv_h, u16(k_cache), u16(v_cache), sc_b, sc_s, sc_h,
@@ -119,6 +128,228 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h, void* k_
 int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, void* stream) {
   FSVD_REQUIRE_PTR(x, "fsvd_rmsnorm"); FSVD_REQUIRE_PTR(w, "fsvd_rmsnorm"); FSVD_REQUIRE_PTR(y, "fsvd_rmsnorm");
   return launch_rmsnorm(cu16(x), ldx, cu16(w), eps, u16(y), ldy, rows, K, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------
+// reference operand layouts
+// ---------------------------------------------------------------------------------------------
+namespace {
+inline size_t align16(size_t n) { return (n + 15) / 16 * 16; }
+inline int esize(int dtype) { return dtype == FSVD_FP32 ? 4 : 2; }
+
+struct XwPlan { XwArgs a; int tx, bt; };
+
+// Workspace layout shared by every split-K entry point: a fixed block of arrival counters at the
+// front (zero at rest: each launch leaves its counters at zero) and the fp32 partials behind it.
+// The counter block has a fixed size so that calls of different shapes that reuse one workspace
+// never see each other's partials as counters.
+constexpr size_t kCounterBytes = 64 * 1024;
+
+int run_xw(XwPlan& p, int dtype, char* ws, size_t ws_bytes, const char* fn, hipStream_t st) {
+  const size_t pbytes = xw_partial_floats(p.a, p.tx * 8, p.bt) * sizeof(float);
+  if (xw_num_tiles(p.a) * sizeof(int32_t) > kCounterBytes) {
+    set_last_error("%s: %zu output tiles exceed the %zu arrival counters of the workspace", fn, xw_num_tiles(p.a), kCounterBytes / 4);
+    return kErrBadShape;
+  }
+  if (p.a.ksplit > 1 && (ws == nullptr || ws_bytes < kCounterBytes + pbytes)) {
+    set_last_error("%s: workspace of %zu bytes needed, %zu given", fn, kCounterBytes + pbytes, ws_bytes);
+    return kErrWorkspace;
+  }
+  return launch_xw(p.a, dtype, p.tx, p.bt, reinterpret_cast<int32_t*>(ws), reinterpret_cast<float*>(ws + kCounterBytes), st);
+}
+size_t xw_bytes(const XwPlan& p) {
+  return kCounterBytes + xw_partial_floats(p.a, p.tx * 8, p.bt) * sizeof(float);
+}
+
+int plan_linear(XwPlan& p, const void* x, int64_t sx_b, int64_t sx_k, int x_fp32, const void* W, int64_t sw_k, const void* bias,
+                int bias_post, void* y, int64_t sy_b, int out_fp32, int B, int K, int N, int dtype, int kslice_fixed,
+                int round_partials) {
+  p.a = XwArgs{};
+  p.a.nprob = 1; p.a.B = B; p.a.x_fp32 = x_fp32; p.a.out_fp32 = out_fp32; p.a.round_partials = round_partials; p.a.bias_post = bias_post;
+  XwProblem& P = p.a.prob[0];
+  P.x = x; P.sx_b = sx_b; P.sx_h = 0; P.sx_k = sx_k; P.W = W; P.sw_h = 0; P.sw_k = sw_k; P.bias = bias; P.sbias_h = 0;
+  P.y = y; P.sy_b = sy_b; P.sy_h = 0; P.K = K; P.N = N; P.heads = 1;
+  return plan_xw(p.a, dtype, 0, kslice_fixed, &p.tx, &p.bt);
+}
+
+int plan_reconstruct(XwPlan& p, const void* const Pm[3], const int64_t sP[3][3], const void* const Vm[3], const int64_t sV[3][2],
+                     const void* const bm[3], const int64_t sb[3], void* const Om[3], const int64_t sO[3][2], int B,
+                     const int heads[3], int Dh, const int R[3], int dtype) {
+  p.a = XwArgs{};
+  p.a.nprob = 3; p.a.B = B;
+  for (int i = 0; i < 3; ++i) {
+    XwProblem& P = p.a.prob[i];
+    P.x = Pm[i]; P.sx_b = sP[i][0]; P.sx_h = sP[i][1]; P.sx_k = sP[i][2];
+    P.W = Vm[i]; P.sw_h = sV[i][0]; P.sw_k = sV[i][1];
+    P.bias = bm[i]; P.sbias_h = sb[i];
+    P.y = Om[i]; P.sy_b = sO[i][0]; P.sy_h = sO[i][1];
+    P.K = R[i]; P.N = Dh; P.heads = heads[i];
+  }
+  return plan_xw(p.a, dtype, 0, 0, &p.tx, &p.bt);
+}
+}  // namespace
+
+extern "C" {
+
+size_t fsvd_xw_linear_workspace_bytes(int B, int K, int N, int dtype) {
+  XwPlan p;
+  if (plan_linear(p, nullptr, K, 1, 0, nullptr, N, nullptr, 0, nullptr, N, 0, B, K, N, dtype, 0, 0) != kOk) return 0;
+  return xw_bytes(p);
+}
+
+int fsvd_xw_linear(const void* x, int64_t sx_b, int64_t sx_k, int x_fp32, const void* W, int64_t sw_k, const void* bias,
+                   int bias_post, void* y, int64_t sy_b, int out_fp32, int B, int K, int N, int dtype, void* workspace,
+                   size_t workspace_bytes, void* stream) {
+  const char* fn = "fsvd_xw_linear";
+  FSVD_REQUIRE_PTR(x, fn); FSVD_REQUIRE_PTR(W, fn); FSVD_REQUIRE_PTR(y, fn);
+  if (dtype < 0 || dtype > 2) { set_last_error("%s: dtype code %d not in {0,1,2}", fn, dtype); return kErrBadDtype; }
+  if (sw_k < N || sy_b < N) { set_last_error("%s: leading dimension smaller than N=%d", fn, N); return kErrBadShape; }
+  XwPlan p;
+  int rc = plan_linear(p, x, sx_b, sx_k, x_fp32, W, sw_k, bias, bias_post, y, sy_b, out_fp32, B, K, N, dtype, 0, 0);
+  if (rc != kOk) return rc;
+  return run_xw(p, dtype, static_cast<char*>(workspace), workspace_bytes, fn, static_cast<hipStream_t>(stream));
+}
+
+size_t fsvd_reconstruct_qkv_workspace_bytes(int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int dtype) {
+  XwPlan p;
+  const void* nul[3] = {nullptr, nullptr, nullptr};
+  void* nulo[3] = {nullptr, nullptr, nullptr};
+  const int64_t sP[3][3] = {{Rq, 0, 1}, {Rk, 0, 1}, {Rv, 0, 1}};
+  const int64_t sV[3][2] = {{(int64_t)Rq * Dh, Dh}, {(int64_t)Rk * Dh, Dh}, {(int64_t)Rv * Dh, Dh}};
+  const int64_t sb[3] = {Dh, Dh, Dh};
+  const int64_t sO[3][2] = {{(int64_t)H * Dh, Dh}, {(int64_t)Hk * Dh, Dh}, {(int64_t)Hk * Dh, Dh}};
+  const int heads[3] = {H, Hk, Hk};
+  const int R[3] = {Rq, Rk, Rv};
+  if (plan_reconstruct(p, nul, sP, nul, sV, nul, sb, nulo, sO, B, heads, Dh, R, dtype) != kOk) return 0;
+  return xw_bytes(p);
+}
+
+int fsvd_reconstruct_qkv_token(const void* Pq, int64_t sPq_b, int64_t sPq_h, int64_t sPq_r, const void* Pk, int64_t sPk_b,
+                               int64_t sPk_h, int64_t sPk_r, const void* Pv, int64_t sPv_b, int64_t sPv_h, int64_t sPv_r,
+                               const void* Vq, int64_t sVq_h, int64_t sVq_r, const void* Vk, int64_t sVk_h, int64_t sVk_r,
+                               const void* Vv, int64_t sVv_h, int64_t sVv_r, const void* bq, int64_t sbq_h, const void* bk,
+                               int64_t sbk_h, const void* bv, int64_t sbv_h, void* Q, int64_t sQ_b, int64_t sQ_h, void* K,
+                               int64_t sK_b, int64_t sK_h, void* V, int64_t sV_b, int64_t sV_h, int B, int H, int Hk, int Dh,
+                               int Rq, int Rk, int Rv, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  const char* fn = "fsvd_reconstruct_qkv_token";
+  FSVD_REQUIRE_PTR(Pq, fn); FSVD_REQUIRE_PTR(Pk, fn); FSVD_REQUIRE_PTR(Pv, fn);
+  FSVD_REQUIRE_PTR(Vq, fn); FSVD_REQUIRE_PTR(Vk, fn); FSVD_REQUIRE_PTR(Vv, fn);
+  FSVD_REQUIRE_PTR(Q, fn); FSVD_REQUIRE_PTR(K, fn); FSVD_REQUIRE_PTR(V, fn);
+  if (dtype < 0 || dtype > 2) { set_last_error("%s: dtype code %d not in {0,1,2}", fn, dtype); return kErrBadDtype; }
+  if (B <= 0 || H <= 0 || Hk <= 0 || Dh <= 0 || Rq <= 0 || Rk <= 0 || Rv <= 0) {
+    set_last_error("%s: bad shape B=%d H=%d Hk=%d Dh=%d R=(%d,%d,%d)", fn, B, H, Hk, Dh, Rq, Rk, Rv);
+    return kErrBadShape;
+  }
+  if (sVq_r < Dh || sVk_r < Dh || sVv_r < Dh || sQ_h < Dh || sK_h < Dh || sV_h < Dh) {
+    set_last_error("%s: a row stride is smaller than head_dim %d", fn, Dh);
+    return kErrBadShape;
+  }
+  const void* Pm[3] = {Pq, Pk, Pv};
+  const int64_t sP[3][3] = {{sPq_b, sPq_h, sPq_r}, {sPk_b, sPk_h, sPk_r}, {sPv_b, sPv_h, sPv_r}};
+  const void* Vm[3] = {Vq, Vk, Vv};
+  const int64_t sVm[3][2] = {{sVq_h, sVq_r}, {sVk_h, sVk_r}, {sVv_h, sVv_r}};
+  const void* bm[3] = {bq, bk, bv};
+  const int64_t sb[3] = {sbq_h, sbk_h, sbv_h};
+  void* Om[3] = {Q, K, V};
+  const int64_t sO[3][2] = {{sQ_b, sQ_h}, {sK_b, sK_h}, {sV_b, sV_h}};
+  const int heads[3] = {H, Hk, Hk};
+  const int R[3] = {Rq, Rk, Rv};
+  XwPlan p;
+  int rc = plan_reconstruct(p, Pm, sP, Vm, sVm, bm, sb, Om, sO, B, heads, Dh, R, dtype);
+  if (rc != kOk) return rc;
+  return run_xw(p, dtype, static_cast<char*>(workspace), workspace_bytes, fn, static_cast<hipStream_t>(stream));
+}
+
+namespace {
+struct MlpPlan { XwPlan gu, dv, du; size_t off_h, off_s, off_xw, cbytes, total; };
+
+int plan_mlp(MlpPlan& m, const void* PUp, int64_t sPUp_t, const void* PGate, int64_t sPGate_t, const void* GateU, int64_t ldGateU,
+             const void* UpU, int64_t ldUpU, const void* DownV, int64_t ldDownV, const void* DownU, int64_t ldDownU, const void* b2,
+             void* Y, int64_t ldY, int T, int R, int D, int Hd, int dtype, int variant, int bd, int partials_fp32, char* ws) {
+  const int es = esize(dtype);
+  m.off_h = kCounterBytes;
+  m.off_s = m.off_h + align16((size_t)T * D * es);
+  m.off_xw = m.off_s + align16((size_t)T * R * sizeof(float));
+  void* h = ws ? ws + m.off_h : nullptr;
+  float* S = ws ? reinterpret_cast<float*>(ws + m.off_s) : nullptr;
+  // stage 1: h = silu(PGate @ GateU) * (PUp @ UpU)
+  m.gu.a = XwArgs{};
+  m.gu.a.nprob = 1; m.gu.a.B = T; m.gu.a.dual = 1;
+  XwProblem& G = m.gu.a.prob[0];
+  if (ldGateU != ldUpU) { set_last_error("fsvd_mlp_dual_split: GateU and UpU must share a row stride"); return kErrBadShape; }
+  G.x = PGate; G.x2 = PUp; G.sx_b = sPGate_t; G.sx_h = 0; G.sx_k = 1; G.W = GateU; G.W2 = UpU; G.sw_h = 0; G.sw_k = ldGateU;
+  G.y = h; G.sy_b = D; G.sy_h = 0; G.K = R; G.N = D; G.heads = 1;
+  if (sPGate_t != sPUp_t) { set_last_error("fsvd_mlp_dual_split: PUp and PGate must share a row stride"); return kErrBadShape; }
+  int rc = plan_xw(m.gu.a, dtype, 0, 0, &m.gu.tx, &m.gu.bt);
+  if (rc != kOk) return rc;
+  // stage 2: S = h @ DownV, one K slice per D tile of bd rows
+  const bool s_fp32 = variant != 1;   // v1 keeps S in dtype (sum of dtype partials); v2/v3 carry fp32
+  rc = plan_linear(m.dv, h, D, 1, 0, DownV, ldDownV, nullptr, 0, S, R, s_fp32 ? 1 : 0, T, D, R, dtype, bd,
+                   variant == 3 || (variant == 1 && !partials_fp32));
+  if (rc != kOk) return rc;
+  // stage 3: Y = S @ DownU (+ b2)
+  // v1: S already in dtype.  v2: fp32 S rounded to dtype while it is staged.  v3: fp32 S used as is.
+  rc = plan_linear(m.du, S, R, 1, s_fp32 ? 1 : 0, DownU, ldDownU, b2, variant == 3 ? 1 : 0, Y, ldY, 0, T, R, Hd, dtype, 0, 0);
+  if (rc != kOk) return rc;
+  m.du.a.x_round = variant == 2 ? 1 : 0;
+  // the three stages run one after another and share the counter block at the front of the
+  // workspace and one partials block behind the h and S buffers
+  const size_t cbytes = 0;
+  if (std::max(xw_num_tiles(m.gu.a), std::max(xw_num_tiles(m.dv.a), xw_num_tiles(m.du.a))) * sizeof(int32_t) > kCounterBytes) {
+    set_last_error("fsvd_mlp_dual_split: too many output tiles for the workspace counters");
+    return kErrBadShape;
+  }
+  const size_t pfloats = std::max(xw_partial_floats(m.gu.a, m.gu.tx * 8, m.gu.bt),
+                                  std::max(xw_partial_floats(m.dv.a, m.dv.tx * 8, m.dv.bt), xw_partial_floats(m.du.a, m.du.tx * 8, m.du.bt)));
+  m.cbytes = cbytes;
+  m.total = m.off_xw + cbytes + pfloats * sizeof(float);
+  return kOk;
+}
+}  // namespace
+
+size_t fsvd_mlp_dual_split_workspace_bytes(int T, int R, int D, int Hd, int dtype, int bd) {
+  MlpPlan m;
+  if (bd <= 0) bd = 128;
+  if (plan_mlp(m, nullptr, R, nullptr, R, nullptr, D, nullptr, D, nullptr, R, nullptr, Hd, nullptr, nullptr, Hd, T, R, D, Hd,
+               dtype, 2, bd, 1, nullptr) != kOk) return 0;
+  return m.total;
+}
+
+int fsvd_mlp_dual_split(const void* PUp, int64_t sPUp_t, const void* PGate, int64_t sPGate_t, const void* GateU, int64_t ldGateU,
+                        const void* UpU, int64_t ldUpU, const void* DownV, int64_t ldDownV, const void* DownU, int64_t ldDownU,
+                        const void* b2, void* Y, int64_t ldY, float* S_out, int T, int R, int D, int Hd, int dtype, int variant,
+                        int bd, int partials_fp32, void* workspace, size_t workspace_bytes, void* stream) {
+  const char* fn = "fsvd_mlp_dual_split";
+  FSVD_REQUIRE_PTR(PUp, fn); FSVD_REQUIRE_PTR(PGate, fn); FSVD_REQUIRE_PTR(GateU, fn); FSVD_REQUIRE_PTR(UpU, fn);
+  FSVD_REQUIRE_PTR(DownV, fn); FSVD_REQUIRE_PTR(DownU, fn); FSVD_REQUIRE_PTR(Y, fn); FSVD_REQUIRE_PTR(workspace, fn);
+  if (dtype < 0 || dtype > 2) { set_last_error("%s: dtype code %d not in {0,1,2}", fn, dtype); return kErrBadDtype; }
+  if (variant < 1 || variant > 3) { set_last_error("%s: variant %d not in {1,2,3}", fn, variant); return kErrBadShape; }
+  if (T <= 0 || R <= 0 || D <= 0 || Hd <= 0) { set_last_error("%s: bad shape T=%d R=%d D=%d Hd=%d", fn, T, R, D, Hd); return kErrBadShape; }
+  if (ldGateU < D || ldUpU < D || ldDownV < R || ldDownU < Hd || ldY < Hd || sPUp_t < R) {
+    set_last_error("%s: a leading dimension is smaller than its row", fn);
+    return kErrBadShape;
+  }
+  if (bd <= 0) bd = 128;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  char* ws = static_cast<char*>(workspace);
+  MlpPlan m;
+  int rc = plan_mlp(m, PUp, sPUp_t, PGate, sPGate_t, GateU, ldGateU, UpU, ldUpU, DownV, ldDownV, DownU, ldDownU, b2, Y, ldY, T, R,
+                    D, Hd, dtype, variant, bd, partials_fp32, ws);
+  if (rc != kOk) return rc;
+  if (workspace_bytes < m.total) { set_last_error("%s: workspace of %zu bytes needed, %zu given", fn, m.total, workspace_bytes); return kErrWorkspace; }
+  int32_t* counters = reinterpret_cast<int32_t*>(ws);
+  float* partials = reinterpret_cast<float*>(ws + m.off_xw);
+  rc = launch_xw(m.gu.a, dtype, m.gu.tx, m.gu.bt, counters, partials, st);
+  if (rc != kOk) return rc;
+  rc = launch_xw(m.dv.a, dtype, m.dv.tx, m.dv.bt, counters, partials, st);
+  if (rc != kOk) return rc;
+  if (variant != 1 && S_out) {
+    hipError_t e = hipMemcpyAsync(S_out, ws + m.off_s, (size_t)T * R * sizeof(float), hipMemcpyDeviceToDevice, st);
+    if (e != hipSuccess) { set_last_error("%s: copy of S failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+  }
+  return launch_xw(m.du.a, dtype, m.du.tx, m.du.bt, counters, partials, st);
 }
 
 }  // extern "C"

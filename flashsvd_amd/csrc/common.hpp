@@ -89,6 +89,15 @@ __device__ __forceinline__ float wave_max(float v) {
   return fmaxf(fmaxf(a, b), fmaxf(c, d));
 }
 
+// Cross-workgroup hand-off without L2 write-back/invalidate fences: producers use write-through
+// (agent-scope) stores, wait until the memory system has acknowledged them, then signal through an
+// agent-scope atomic; consumers read with agent-scope loads.  A workgroup-scope release fence does
+// not wait for outstanding stores on this target, hence the explicit wait.
+__device__ __forceinline__ void wait_stores_acked() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);   // vmcnt(0) expcnt(0) lgkmcnt(0)
+}
+
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
 }  // namespace fsvd

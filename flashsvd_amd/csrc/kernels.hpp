@@ -60,6 +60,38 @@ struct KvAppendArgs {
   int B, Hk, Dh, S;
 };
 
+// one x @ W problem of the input-major GEMV (a launch carries up to three: q, k, v)
+struct XwProblem {
+  const void* x; const void* x2;         // [B, (heads), K]; x2 feeds W2 in dual mode
+  int64_t sx_b, sx_h, sx_k;
+  const void* W; const void* W2;         // [(heads), K, N], unit stride along N
+  int64_t sw_h, sw_k;
+  const void* bias; int64_t sbias_h;     // [(heads), N] or null
+  void* y; int64_t sy_b, sy_h;           // [B, (heads), N]
+  int K, N, heads;
+  int kslice;                            // filled by plan_xw
+  int vec;                               // filled by plan_xw: 16-byte loads are legal
+};
+
+struct XwArgs {
+  XwProblem prob[3];
+  int nprob;
+  int B;
+  int dual;            // 1: y = silu(x@W) * (x2@W2)
+  int x_fp32;          // activations are fp32 even though W is 16-bit
+  int x_round;         // round the staged activations to the element type (fp32 S -> dtype S)
+  int out_fp32;        // store y as fp32
+  int round_partials;  // round each K-slice partial to the element type before the final sum
+  int bias_post;       // y = round(round(x@W) + bias) instead of round(x@W + bias)
+  int ksplit, ntiles_n, grid_x, grid_z;   // filled by plan_xw
+  float* ws; int32_t* counters;           // filled by launch_xw
+};
+
+int plan_xw(XwArgs& a, int dtype, int want_ksplit, int kslice_fixed, int* tx_out, int* batch_tile_out);
+size_t xw_num_tiles(const XwArgs& a);
+size_t xw_partial_floats(const XwArgs& a, int tn, int batch_tile);
+int launch_xw(XwArgs& a, int dtype, int tx, int batch_tile, int32_t* counters, float* partials, hipStream_t st);
+
 int launch_linear(const LinearArgs& a, int cfg, hipStream_t st);
 int launch_swiglu(const SwigluArgs& a, int cfg, hipStream_t st);
 int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st);

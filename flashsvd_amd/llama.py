@@ -24,6 +24,8 @@ from . import hip_ops
 from .runtime.cache import FlashSVDLegacySparseKVCache, FlashSVDV15DenseKVCache
 
 _TRUE = {"1", "true", "yes", "y", "on"}
+# set by api.enable_flashsvd_llama_layer_tail_cuda_graph(); read at call time together with the env flags
+LAYER_TAIL_GRAPH_ENABLED = False
 
 
 def _env_truthy(name: str) -> bool:
@@ -423,7 +425,27 @@ class SVDLlamaDecoderLayer(nn.Module):
         n1, n2 = self.input_layernorm, self.post_attention_layernorm
         x2 = self.self_attn.decode_token(x, cache, positions, norm_weight=n1.weight, eps=n1.variance_epsilon,
                                          residual=x, rope=rope, attn_ws=attn_ws, nsplit=nsplit)
-        return self.mlp.run(x2, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=x2)
+        return self._layer_tail(x2)
+
+    def _layer_tail(self, x2: torch.Tensor) -> torch.Tensor:
+        """residual + post-attention norm + MLP + residual; replayed from a captured graph when the
+        layer-tail scope is enabled and no outer capture is running."""
+        n2 = self.post_attention_layernorm
+        want_graph = (LAYER_TAIL_GRAPH_ENABLED and _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH")
+                      and os.getenv("FLASH_SVD_MLP_CUDA_GRAPH_SCOPE", "auto").strip().lower() in ("auto", "layer_tail")
+                      and not torch.cuda.is_current_stream_capturing())
+        if not want_graph:
+            return self.mlp.run(x2, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=x2)
+        from .graphs import GraphedCallable
+        mode = mlp_rounding_mode()
+        cache = self.mlp._flashsvd_layer_graph_cache
+        key = (tuple(x2.shape), x2.dtype, x2.device, mode)
+        g = cache.get(key)
+        if g is None:
+            g = GraphedCallable(lambda t: self.mlp.run(t, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=t, mode=mode), x2)
+            cache[key] = g
+        out = g(x2)
+        return out if _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH_ALIAS_OUTPUT") else out.clone()
 
     def forward(self, hidden_states: torch.Tensor, attention_mask=None, position_ids=None, past_key_values=None,
                 cache_position=None, position_embeddings=None, **kwargs):

@@ -306,7 +306,7 @@ class FlashSVDLegacySparseKVCache(_CacheBase):
         if ws is None:
             if head_dim % 2:
                 raise ValueError(f"head_dim must be even, got {head_dim}")
-            b, h, s, r = key[:4]
+            b, h, r, s = key[:4]
             f32 = dict(device=device, dtype=torch.float32)
             ws = _DecodeWorkspace(M=torch.empty((b, h, s), **f32), L=torch.empty((b, h, s), **f32),
                                   Acc=torch.empty((b, h, s, r), **f32),

@@ -69,8 +69,9 @@ int fsvd_qkv_rope_append(const void* p, int64_t ldp, const void* q_u, int64_t ld
                          int64_t sc_b, int64_t sc_s, int64_t sc_h,
                          int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int S, int cfg, void* stream);
 
-/* Bytes of scratch fsvd_attn_decode_densekv needs: fp32 partials followed by int32 counters.
- * The counters must be zero before the first call; the kernel leaves them zero. */
+/* Bytes of scratch fsvd_attn_decode_densekv needs for nsplit > 1: a 256 KiB block of int32 arrival
+ * counters followed by the fp32 partials.  The workspace must be zero-filled before its first use;
+ * every call leaves the counters at zero, so it can be reused by later calls of any shape that fits. */
 size_t fsvd_attn_decode_workspace_bytes(int B, int H, int Dh, int nsplit);
 
 /* Single-query attention over a dense KV cache; the role of flash-attn's
@@ -92,6 +93,59 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h,
 /* y = w * bf16(x * rsqrt(mean(x^2)+eps)) over rows of length K.
  * benchmark/mlp/bench_svd_llama_decode_graph.py:78-83. */
 int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Reference operand layouts ("x @ W", W is [K, N]).  dtype is FSVD_BF16 / FSVD_FP16 / FSVD_FP32;
+ * accumulation is fp32 with one rounding at the store.  Workspaces: bytes from the matching
+ * *_workspace_bytes call; the first use needs the workspace zero-filled, later calls keep it valid.
+ * ------------------------------------------------------------------------------------------- */
+
+/* y[b,:] = x[b,:] @ W (+ bias).  Replaces torch.matmul(hidden, packed_qkv_rank)
+ * (benchmark/attn/decode_compare.py:1538), the three matmuls of
+ * reconstruct_qkv_token_shared_prepacked (kernels/attn/decode/densekv_reconstruct_triton.py:739-741)
+ * and phase 2 of the dual-split MLP, matmul/addmm(S, DownU) (kernels/mlp/decode/dual_split_triton.py:623,721).
+ * x_fp32 / out_fp32: activations / result held in fp32 while W is `dtype`.  bias_post != 0 adds the
+ * bias after the product has been rounded (`Q = Q + bq`, densekv_reconstruct_triton.py:747-758). */
+size_t fsvd_xw_linear_workspace_bytes(int B, int K, int N, int dtype);
+int fsvd_xw_linear(const void* x, int64_t sx_b, int64_t sx_k, int x_fp32, const void* W, int64_t sw_k,
+                   const void* bias, int bias_post, void* y, int64_t sy_b, int out_fp32,
+                   int B, int K, int N, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Current-token reconstruction Q[b,h,:] = Pq[b,(h),:] @ Vq[h] (+ bq[h]) and the same for K, V over
+ * Hk heads.  One entry point for the three reference kernels: headwise P [B,H,R] (sP*_h = R stride),
+ * shared P [B,R] (sP*_h = 0) and hetero ranks (Rq, Rk, Rv differ).
+ * kernels/attn/decode/densekv_reconstruct_triton.py:11-357 (kernels), :360-659 (wrappers).
+ * Bases V* are [heads, R, Dh] with unit stride along Dh; biases [heads, Dh] or NULL. */
+size_t fsvd_reconstruct_qkv_workspace_bytes(int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int dtype);
+int fsvd_reconstruct_qkv_token(const void* Pq, int64_t sPq_b, int64_t sPq_h, int64_t sPq_r,
+                               const void* Pk, int64_t sPk_b, int64_t sPk_h, int64_t sPk_r,
+                               const void* Pv, int64_t sPv_b, int64_t sPv_h, int64_t sPv_r,
+                               const void* Vq, int64_t sVq_h, int64_t sVq_r,
+                               const void* Vk, int64_t sVk_h, int64_t sVk_r,
+                               const void* Vv, int64_t sVv_h, int64_t sVv_r,
+                               const void* bq, int64_t sbq_h, const void* bk, int64_t sbk_h, const void* bv, int64_t sbv_h,
+                               void* Q, int64_t sQ_b, int64_t sQ_h, void* K, int64_t sK_b, int64_t sK_h,
+                               void* V, int64_t sV_b, int64_t sV_h,
+                               int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int dtype,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+/* Dual-split low-rank SwiGLU MLP on the reference operands: PUp, PGate [T,R] (row strides given),
+ * GateU, UpU [R,D], DownV [D,R], DownU [R,Hd], optional b2 [Hd]; Y [T,Hd].
+ *   h = dtype(silu(PGate@GateU) * (PUp@UpU));  S = sum over D tiles of bd rows of h[:,tile] @ DownV[tile,:];
+ *   Y = dtype(S) @ DownU (+ b2).
+ * variant 1: tile partials pass through a workspace of `dtype` (or fp32 when partials_fp32 != 0) before
+ *            the sum (flashsvd_mlp_dual_split_triton_v1, kernels/mlp/decode/dual_split_triton.py:535-624);
+ * variant 2: fp32 partials summed into S, which is then rounded (v2 / v2_sm80 / pcat_s, :627-855 and
+ *            dual_split_triton_pcat_s.py:123-218); S_out, if given, receives the fp32 S [T,R];
+ * variant 3: tile partials rounded to dtype, Y accumulated in fp32 from them and rounded once, b2 added
+ *            afterwards in dtype (v3, dual_split_triton.py:427-532,858-966).
+ * The summation over D tiles is in tile order (deterministic), unlike the reference's atomics. */
+size_t fsvd_mlp_dual_split_workspace_bytes(int T, int R, int D, int Hd, int dtype, int bd);
+int fsvd_mlp_dual_split(const void* PUp, int64_t sPUp_t, const void* PGate, int64_t sPGate_t,
+                        const void* GateU, int64_t ldGateU, const void* UpU, int64_t ldUpU,
+                        const void* DownV, int64_t ldDownV, const void* DownU, int64_t ldDownU, const void* b2,
+                        void* Y, int64_t ldY, float* S_out, int T, int R, int D, int Hd, int dtype,
+                        int variant, int bd, int partials_fp32, void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -164,3 +164,86 @@ def test_cpu_tensors_raise():
     mlp = llama.SVD_LlamaMLP(64, 128, "silu", ratio=0.5)
     with pytest.raises(RuntimeError):
         mlp(torch.zeros(1, 1, 64, dtype=BF16))
+
+
+def test_registry_flash_attn_with_kvcache_callable():
+    """The attend-with-append callable resolved by the registry follows the flash-attn keyword contract."""
+    from flashsvd_amd.runtime import decode_registry as R
+    from tests.util import rand_bf16
+    B, H, Hk, Dh, S = 2, 8, 8, 128, 64
+    cos, sin = O.rope_tables(S, Dh, dtype=BF16)
+    q, kn, vn = rand_bf16(B, 1, H, Dh, seed=1), rand_bf16(B, 1, Hk, Dh, seed=2), rand_bf16(B, 1, Hk, Dh, seed=3)
+    kc, vc = rand_bf16(B, S, Hk, Dh, seed=4), rand_bf16(B, S, Hk, Dh, seed=5)
+    lens = torch.tensor([40, 7], dtype=torch.int32)
+    kr, vr = kc.clone(), vc.clone()
+    ref = O.flash_attn_with_kvcache(q, kr, vr, k=kn, v=vn, cache_seqlens=lens, rotary_cos=cos, rotary_sin=sin, causal=True)
+    fn = R.get_flash_attn_with_kvcache()
+    kg, vg = kc.cuda(), vc.cuda()
+    out = R.call_flash_attn_with_kvcache(fn, q.cuda(), kg, vg, k_bmhd=kn.cuda(), v_bmhd=vn.cuda(), cache_seqlens=lens.cuda(),
+                                         rotary_cos=cos.cuda(), rotary_sin=sin.cuda(), causal=True)
+    assert out.shape == (B, 1, H, Dh)
+    assert_close_bf16(out, ref, "registry fa2 call")
+    assert_close_bf16(kg, kr, "k cache")
+
+
+def test_module_decode_entry_and_layer_tail_graph():
+    """_flashsvd_dense_decode_token_from_hidden and the layer-tail / MLP graph scopes give the eager result."""
+    from flashsvd_amd import api
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    mw, prompt = O.config_c1(BF16)
+    model = model_from_oracle(mw)
+    layer = model.model.layers[0]
+    x = mw.embed[prompt[:, :9]].cuda()
+
+    def run():
+        cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=16, device="cuda", dtype=BF16)
+        layer(x[:, :8], past_key_values=cache, cache_position=torch.arange(8))
+        return layer(x[:, 8:9], past_key_values=cache, cache_position=torch.tensor([8])).clone(), cache
+
+    api.configure_runtime("flashsvd", enable_mlp_graph=False)
+    eager, cache = run()
+    # the attention entry point on normed hidden states == oracle attention block
+    oc = O.DenseCache(mw, 1, 16, BF16)
+    cos, sin = O.rope_tables(16, mw.head_dim, dtype=BF16)
+    O.block_forward(mw, 0, mw.embed[prompt[:, :8]], 0, oc, cos, sin)
+    ref = O.block_forward(mw, 0, mw.embed[prompt[:, 8:9]], 8, oc, cos, sin)
+    assert_close_bf16(eager, ref, "layer decode")
+    assert cache.get_seq_length() == 9
+    api.enable_flashsvd_llama_layer_tail_cuda_graph()
+    api.configure_runtime("flashsvd", enable_mlp_graph=True, mlp_graph_scope="layer_tail")
+    for _ in range(3):    # capture, then replays
+        got, _ = run()
+        assert torch.equal(got, eager)
+    assert len(layer.mlp._flashsvd_layer_graph_cache) == 1
+    api.configure_runtime("flashsvd", enable_mlp_graph=True, mlp_graph_scope="mlp")
+    h2 = torch.randn(1, 1, 512, device="cuda").to(BF16)
+    a = layer.mlp(h2).clone()
+    b = layer.mlp(h2).clone()
+    api.configure_runtime("flashsvd", enable_mlp_graph=False)
+    c = layer.mlp(h2)
+    assert torch.equal(a, b) and torch.equal(a, c) and len(layer.mlp._flashsvd_graph_cache) == 1
+    api.configure_runtime("flashsvd")
+
+
+def test_generate_text_and_decode_eval():
+    from flashsvd_amd import api
+
+    class Tok:
+        pad_token_id, eos_token_id, eos_token, pad_token = 0, None, "<eos>", "<pad>"
+
+        def __call__(self, text, return_tensors="pt", add_special_tokens=False):
+            return {"input_ids": torch.tensor([[1, 5, 7, 11, 13]], dtype=torch.long)}
+
+        def decode(self, ids, skip_special_tokens=False):
+            return " ".join(str(int(i)) for i in ids)
+
+    mw, _ = O.config_c1(BF16)
+    model = model_from_oracle(mw)
+    ref = O.greedy_decode(mw, torch.tensor([[1, 5, 7, 11, 13]]), 6)
+    api.configure_runtime("flashsvd")
+    for graph in (False, True):
+        res = api.generate_text(model, Tok(), prompt="x", max_new_tokens=6, device="cuda", use_graph=graph)
+        assert res["prompt_token_count"] == 5 and res["generated_token_count"] == 6 and len(res["output_ids"]) == 11
+        assert res["completion_ids"] == ref[0].tolist()
+    out = api.decode_kvcache_eval(model, prompt_len=16, new_tokens=4, warmup=2, batch_size=2)
+    assert out["new_tokens"] == 4 and out["decode_tok_s"] > 0 and out["flashsvd_dense_cache"]
