@@ -33,6 +33,10 @@ SIGNATURES = {
                                          c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
                                          c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "fsvd_rmsnorm": (c_int, [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "fsvd_attn_decode_rankkv": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
+                                        c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                        c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                        c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "fsvd_xw_linear_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "fsvd_xw_linear": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int,
                                c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -92,6 +92,23 @@ size_t xw_num_tiles(const XwArgs& a);
 size_t xw_partial_floats(const XwArgs& a, int tn, int batch_tile);
 int launch_xw(XwArgs& a, int dtype, int tx, int batch_tile, int32_t* counters, float* partials, hipStream_t st);
 
+struct RankDecodeArgs {
+  const uint16_t* q; int64_t sq_b, sq_h;            // [B,H,Dh] current-token query (bf16)
+  const uint16_t* pk; int64_t spk_b, spk_s, spk_h;  // rank-space key cache   [B,S,(Hk),Rk]; head stride 0 when shared
+  const uint16_t* pv; int64_t spv_b, spv_s, spv_h;  // rank-space value cache [B,S,(Hk),Rv]
+  const uint16_t* k_u; int64_t ldku;                // [Hk*Dh, Rk] nn.Linear layout
+  const uint16_t* v_u; int64_t ldvu;                // [Hk*Dh, Rv]
+  const uint16_t* bv;                               // [Hk*Dh] or null
+  const uint16_t* cos; const uint16_t* sin; int rope_len;   // [rope_len, Dh/2] or null (no rotation of K)
+  int rotate_q;                                     // also rotate q at position n_keys-1
+  const int32_t* seqlens; int seqlen_add;
+  float* ws_m; float* ws_l; float* ws_acc;          // [B,H,nsplit], [B,H,nsplit], [B,H,nsplit,Rv]
+  uint16_t* out; int64_t so_b, so_h;                // [B,H,Dh]
+  int B, H, Hk, Dh, S, Rk, Rv, nsplit;
+  float scale;
+};
+int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st);
+
 int launch_linear(const LinearArgs& a, int cfg, hipStream_t st);
 int launch_swiglu(const SwigluArgs& a, int cfg, hipStream_t st);
 int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st);

@@ -1,0 +1,272 @@
+// Single-query attention over a RANK-SPACE KV cache: the cache holds the pre-RoPE rank
+// coefficients Pk, Pv [B,S,R] (shared by all heads); K is rebuilt per key tile inside the kernel
+// as Pk_tile @ k_u[h]^T on the matrix cores, rotated at the keys' absolute positions, scored
+// against the (already rebuilt and rotated) query, and V is never rebuilt per key: the softmax
+// weights are applied to Pv in rank space, t = sum_n p_n Pv_n, and one product t @ v_u[h]^T per
+// head finishes the job (the Acc[B,H,S,R] workspace idea of the reference's split-K design).
+//
+// Stage 1, grid (nsplit, Hk*groups, B), 4 waves: each wave owns 16 keys of a 64-key tile.
+//   MFMA 16x16x32 bf16: A = Pk[16 keys x 32 r] and B = k_u[16 d x 32 r] are both contiguous along
+//   r, so both operands are plain 16-byte global loads in the instruction's native lane layout.
+//   The 8 accumulator tiles of a wave hold K[16 keys x 128 d]; d and d+64 sit in the same lane,
+//   so the rotate-half RoPE is register-local; scores fold over the 16 lanes of a DPP row.
+// Stage 2, grid (H, B): merge the splits in order, normalise, multiply by v_u[h].
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace fsvd {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kRdThreads = 256;
+constexpr int kRdTileKeys = 64;   // 4 waves x 16 keys
+constexpr int kRdMaxChunks = 4;   // rank-space accumulator: R <= 4 * 512
+
+__device__ __forceinline__ bf16x8_t ld_frag(const uint16_t* p) {
+  return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(p));
+}
+__device__ __forceinline__ bf16x8_t zero_frag() { return __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u}); }
+
+template <int REP>
+__global__ __launch_bounds__(kRdThreads) void rank_decode_partial_kernel(RankDecodeArgs a) {
+  constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
+  __shared__ float qs[REP][DH];
+  __shared__ float wm[4][REP], wl[4][REP];
+  __shared__ float tbuf[4][kRdMaxChunks * 512];
+
+  const int s = blockIdx.x, b = blockIdx.z;
+  const int groups = a.H / a.Hk / REP;             // q-head groups per kv head handled by separate blocks
+  const int hk = blockIdx.y / groups, grp = blockIdx.y % groups;
+  const int h0 = hk * (a.H / a.Hk) + grp * REP;    // first q head of this block
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;        // column-in-tile / row group
+
+  int n_keys = a.seqlens[b] + a.seqlen_add;
+  n_keys = max(0, min(n_keys, a.S));
+  int per = (n_keys + a.nsplit - 1) / a.nsplit;
+  per = (per + kRdTileKeys - 1) / kRdTileKeys * kRdTileKeys;
+  const int k0 = min(s * per, n_keys), k1 = min(n_keys, k0 + per);
+
+  // queries of this block as fp32 in LDS, rotated at position n_keys-1 when asked to
+  for (int i = tid; i < REP * HALF; i += kRdThreads) {
+    const int g = i / HALF, d = i % HALF;
+    const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)(h0 + g) * a.sq_h;
+    float x0 = bf16_bits_to_f32(qp[d]), x1 = bf16_bits_to_f32(qp[d + HALF]);
+    if (a.rotate_q) {
+      const int tp = min(max(n_keys - 1, 0), a.rope_len - 1);
+      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * HALF + d]), sn = bf16_bits_to_f32(a.sin[(int64_t)tp * HALF + d]);
+      const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
+      x0 = r0; x1 = r1;
+    }
+    qs[g][d] = x0 * a.scale;
+    qs[g][d + HALF] = x1 * a.scale;
+  }
+  __syncthreads();
+  float qv[REP][NT];
+#pragma unroll
+  for (int g = 0; g < REP; ++g)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) qv[g][t] = qs[g][t * 16 + lr];
+
+  const int nchunk = (a.Rv + 511) / 512;
+  float m_run[REP], l_run[REP];
+  float tacc[REP][kRdMaxChunks][8];
+#pragma unroll
+  for (int g = 0; g < REP; ++g) {
+    m_run[g] = -INFINITY; l_run[g] = 0.f;
+#pragma unroll
+    for (int c = 0; c < kRdMaxChunks; ++c)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) tacc[g][c][i] = 0.f;
+  }
+
+  const uint16_t* pk_b = a.pk + (int64_t)b * a.spk_b + (int64_t)hk * a.spk_h;
+  const uint16_t* pv_b = a.pv + (int64_t)b * a.spv_b + (int64_t)hk * a.spv_h;
+  const uint16_t* ku_h = a.k_u + (int64_t)hk * DH * a.ldku;
+
+  for (int kt = k0; kt < k1; kt += kRdTileKeys) {
+    const int wkey0 = kt + wave * 16;              // first key of this wave
+    if (wkey0 >= k1) continue;                     // whole wave past the end (no block barrier in the loop)
+    // ---- K tile = Pk[16 keys, R] @ k_u[h]^T on the matrix cores
+    f32x4_t acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int akey = min(wkey0 + lr, k1 - 1);
+    const uint16_t* arow = pk_b + (int64_t)akey * a.spk_s + lg * 8;
+    const uint16_t* brow = ku_h + (int64_t)lr * a.ldku + lg * 8;
+#pragma unroll 2
+    for (int r0 = 0; r0 < a.Rk; r0 += 32) {
+      const bool in = r0 + lg * 8 < a.Rk;
+      const bf16x8_t af = in ? ld_frag(arow + r0) : zero_frag();
+      bf16x8_t bf[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) bf[t] = in ? ld_frag(brow + (int64_t)t * 16 * a.ldku + r0) : zero_frag();
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bf[t], acc[t], 0, 0, 0);
+    }
+    // ---- rotate-half RoPE at absolute key positions (register-local: tiles t and t+4 pair up)
+    if (a.cos) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int pos = min(wkey0 + lg * 4 + i, a.rope_len - 1);
+#pragma unroll
+        for (int t = 0; t < NT / 2; ++t) {
+          const int idx = t * 16 + lr;
+          const float c = bf16_bits_to_f32(a.cos[(int64_t)pos * HALF + idx]), sn = bf16_bits_to_f32(a.sin[(int64_t)pos * HALF + idx]);
+          const float x0 = acc[t][i], x1 = acc[t + NT / 2][i];
+          acc[t][i] = x0 * c - x1 * sn;
+          acc[t + NT / 2][i] = x0 * sn + x1 * c;
+        }
+      }
+    }
+    // ---- scores, online softmax and the rank-space accumulation, per query head of the group
+#pragma unroll
+    for (int g = 0; g < REP; ++g) {
+      float sc[4];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float d = 0.f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) d += qv[g][t] * acc[t][i];
+        d = row16_sum(d);
+        sc[i] = (wkey0 + lg * 4 + i < k1) ? d : -INFINITY;
+        tmax = fmaxf(tmax, sc[i]);
+      }
+      tmax = wave_max(tmax);
+      const float m_new = fmaxf(m_run[g], tmax);
+      const float alpha = (m_run[g] == -INFINITY) ? 0.f : __expf(m_run[g] - m_new);
+      float p[4], psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { p[i] = (sc[i] == -INFINITY) ? 0.f : __expf(sc[i] - m_new); psum += p[i]; }
+      // every lane of a row group holds the same p; one lane per group contributes to the sum
+      float pl = (lr == 0) ? psum : 0.f;
+      pl = wave_sum(pl);
+      l_run[g] = l_run[g] * alpha + pl;
+      m_run[g] = m_new;
+      // p of all 16 keys as wave-uniform values
+      float pk16[16];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pk16[j * 4 + i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p[i]), j * 16));
+#pragma unroll
+      for (int c = 0; c < kRdMaxChunks; ++c) {
+        const int r = c * 512 + lane * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) tacc[g][c][i] *= alpha;
+        if (c < nchunk && r < a.Rv) {
+#pragma unroll
+          for (int kk = 0; kk < 16; ++kk) {
+            const int key = min(wkey0 + kk, k1 - 1);   // p is 0 for clamped keys
+            const u32x4_t v = *reinterpret_cast<const u32x4_t*>(pv_b + (int64_t)key * a.spv_s + r);
+            const float pw = pk16[kk];
+            tacc[g][c][0] += pw * bf16_lo(v.x); tacc[g][c][1] += pw * bf16_hi(v.x);
+            tacc[g][c][2] += pw * bf16_lo(v.y); tacc[g][c][3] += pw * bf16_hi(v.y);
+            tacc[g][c][4] += pw * bf16_lo(v.z); tacc[g][c][5] += pw * bf16_hi(v.z);
+            tacc[g][c][6] += pw * bf16_lo(v.w); tacc[g][c][7] += pw * bf16_hi(v.w);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- merge the 4 waves (each has its own running max) and write the split's partial
+#pragma unroll
+  for (int g = 0; g < REP; ++g) {
+    __syncthreads();
+    if (lane == 0) { wm[wave][g] = m_run[g]; wl[wave][g] = l_run[g]; }
+#pragma unroll
+    for (int c = 0; c < kRdMaxChunks; ++c) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) tbuf[wave][c * 512 + lane * 8 + i] = tacc[g][c][i];
+    }
+    __syncthreads();
+    const float M = fmaxf(fmaxf(wm[0][g], wm[1][g]), fmaxf(wm[2][g], wm[3][g]));
+    float w[4], L = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { w[j] = (wm[j][g] == -INFINITY) ? 0.f : __expf(wm[j][g] - M); L += w[j] * wl[j][g]; }
+    const int64_t slot = ((int64_t)b * a.H + h0 + g) * a.nsplit + s;
+    for (int r = tid; r < a.Rv; r += kRdThreads)
+      a.ws_acc[slot * a.Rv + r] = w[0] * tbuf[0][r] + w[1] * tbuf[1][r] + w[2] * tbuf[2][r] + w[3] * tbuf[3][r];
+    if (tid == 0) { a.ws_m[slot] = M; a.ws_l[slot] = L; }
+  }
+}
+
+// out[b,h,:] = (sum_s w_s Acc_s / max(sum_s w_s L_s, 1e-20)) @ v_u[h]^T (+ bv[h])
+__global__ __launch_bounds__(kRdThreads) void rank_decode_merge_kernel(RankDecodeArgs a) {
+  constexpr int DH = 128;
+  __shared__ float ts[kRdMaxChunks * 512];
+  __shared__ float wsc[64];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int hk = h / (a.H / a.Hk);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t slot0 = ((int64_t)b * a.H + h) * a.nsplit;
+  float M = -INFINITY;
+  for (int s = 0; s < a.nsplit; ++s) M = fmaxf(M, a.ws_m[slot0 + s]);
+  float den = 0.f;
+  for (int s = 0; s < a.nsplit; ++s) {
+    const float m = a.ws_m[slot0 + s];
+    den += ((m == -INFINITY) ? 0.f : __expf(m - M)) * a.ws_l[slot0 + s];
+  }
+  const float inv = 1.0f / fmaxf(den, 1e-20f);
+  for (int r = tid; r < a.Rv; r += kRdThreads) {
+    float t = 0.f;
+    for (int s = 0; s < a.nsplit; ++s) {
+      const float m = a.ws_m[slot0 + s];
+      const float w = (m == -INFINITY) ? 0.f : __expf(m - M);
+      t += w * a.ws_acc[(slot0 + s) * a.Rv + r];
+    }
+    ts[r] = t * inv;
+  }
+  __syncthreads();
+  (void)wsc;
+  uint16_t* outp = a.out + (int64_t)b * a.so_b + (int64_t)h * a.so_h;
+  for (int d = wave; d < DH; d += kRdThreads / 64) {
+    const uint16_t* row = a.v_u + (int64_t)(hk * DH + d) * a.ldvu;
+    float acc = 0.f;
+    for (int r = lane * 8; r < a.Rv; r += 512) {
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(row + r);
+      acc += ts[r] * bf16_lo(v.x) + ts[r + 1] * bf16_hi(v.x) + ts[r + 2] * bf16_lo(v.y) + ts[r + 3] * bf16_hi(v.y) +
+             ts[r + 4] * bf16_lo(v.z) + ts[r + 5] * bf16_hi(v.z) + ts[r + 6] * bf16_lo(v.w) + ts[r + 7] * bf16_hi(v.w);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      if (a.bv) acc += bf16_bits_to_f32(a.bv[hk * DH + d]);
+      outp[d] = (uint16_t)f32_to_bf16_bits(acc);
+    }
+  }
+}
+
+int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
+  const char* fn = "fsvd_attn_decode_rankkv";
+  if (a.B <= 0 || a.H <= 0 || a.Hk <= 0 || a.H % a.Hk != 0 || a.S <= 0 || a.nsplit <= 0) {
+    set_last_error("%s: bad shape B=%d H=%d Hk=%d S=%d nsplit=%d", fn, a.B, a.H, a.Hk, a.S, a.nsplit);
+    return kErrBadShape;
+  }
+  if (a.Dh != 128) { set_last_error("%s: head_dim %d is not 128", fn, a.Dh); return kErrBadShape; }
+  if (a.Rk <= 0 || a.Rv <= 0 || (a.Rk % 8) || (a.Rv % 8) || a.Rv > kRdMaxChunks * 512) {
+    set_last_error("%s: ranks must be multiples of 8 with Rv <= %d (got Rk=%d Rv=%d); pad the factors", fn, kRdMaxChunks * 512, a.Rk, a.Rv);
+    return kErrBadShape;
+  }
+  const auto mis = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+  if (mis(a.pk) || mis(a.pv) || mis(a.k_u) || mis(a.v_u) || (a.spk_s % 8) || (a.spv_s % 8) || (a.spk_b % 8) || (a.spv_b % 8) || (a.spk_h % 8) || (a.spv_h % 8) ||
+      (a.ldku % 8) || (a.ldvu % 8)) {
+    set_last_error("%s: cache / factor pointers and strides must be 16-byte aligned", fn);
+    return kErrBadAlign;
+  }
+  const int rep = a.H / a.Hk;
+  dim3 block(kRdThreads);
+  if (rep % 4 == 0) hipLaunchKernelGGL(rank_decode_partial_kernel<4>, dim3(a.nsplit, a.Hk * (rep / 4), a.B), block, 0, st, a);
+  else if (rep % 2 == 0) hipLaunchKernelGGL(rank_decode_partial_kernel<2>, dim3(a.nsplit, a.Hk * (rep / 2), a.B), block, 0, st, a);
+  else hipLaunchKernelGGL(rank_decode_partial_kernel<1>, dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: stage 1 launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+  hipLaunchKernelGGL(rank_decode_merge_kernel, dim3(a.H, a.B), block, 0, st, a);
+  e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: stage 2 launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
+}  // namespace fsvd

@@ -248,8 +248,10 @@ class SVD_LlamaAttention(nn.Module):
         self._ensure_runtime_state()
         B = x.shape[0]
         H, Hk, Dh = self.num_heads, self.num_key_value_heads, self.head_dim
+        if isinstance(cache, FlashSVDLegacySparseKVCache):
+            return self._decode_token_rank(x, cache, positions, norm_weight=norm_weight, eps=eps, residual=residual, rope=rope)
         if not isinstance(cache, FlashSVDV15DenseKVCache):
-            raise TypeError(f"dense-KV decode needs a FlashSVDV15DenseKVCache, got {type(cache).__name__}")
+            raise TypeError(f"decode needs a FlashSVDV15DenseKVCache or FlashSVDLegacySparseKVCache, got {type(cache).__name__}")
         cache._ensure_layer_spec(self.layer_idx, h=Hk, dh=Dh)
         kc, vc = cache.key_cache[self.layer_idx], cache.value_cache[self.layer_idx]
         if rope is None:
@@ -261,6 +263,28 @@ class SVD_LlamaAttention(nn.Module):
         if nsplit is None:
             nsplit = hip_ops.pick_nsplit(cache.max_cache_len, B, H, Dh)
         a = hip_ops.attn_decode_densekv(q, kc[:B], vc[:B], positions, seqlen_add=1, nsplit=nsplit, workspace=attn_ws)
+        po = hip_ops.linear(a.view(B, H * Dh), self.o_v_proj.weight)
+        return hip_ops.linear(po, self.o_u_proj.weight, residual=residual)
+
+    def _decode_token_rank(self, x, cache, positions, *, norm_weight=None, eps=1e-6, residual=None, rope=None):
+        """Rank-space cache: append Pk, Pv (pre-RoPE coefficients) and attend with in-kernel K rebuild."""
+        from .kernels.rank_decode import rank_decode
+        B = x.shape[0]
+        H, Hk, Dh = self.num_heads, self.num_key_value_heads, self.head_dim
+        rq, rk, rv = self._qkv_rank_tuple()
+        cache.ensure_layer_ranks(self.layer_idx, rk, rv)
+        pkc, pvc = cache.key_cache[self.layer_idx], cache.value_cache[self.layer_idx]
+        if rope is None:
+            rope = cache.get_rope_tables(seqlen=cache.max_cache_len, head_dim=Dh, device=x.device, dtype=x.dtype)
+        p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)       # [B, rq+rk+rv]
+        rows = torch.arange(B, device=x.device)
+        pos = positions.long()
+        pkc[rows, pos] = p[:, rq:rq + rk]        # device-side scatter of the new coefficients (data movement only)
+        pvc[rows, pos] = p[:, rq + rk:]
+        cache._layer_initialized[self.layer_idx] = True
+        q = hip_ops.linear(p[:, :rq], self.q_u_proj.weight).view(B, H, Dh)
+        a = rank_decode(q, pkc[:B], pvc[:B], self.k_u_proj.weight, self.v_u_proj.weight, rope[0], rope[1], positions,
+                        num_kv_heads=Hk, seqlen_add=1, rotate_q=True)
         po = hip_ops.linear(a.view(B, H * Dh), self.o_v_proj.weight)
         return hip_ops.linear(po, self.o_u_proj.weight, residual=residual)
 
@@ -303,6 +327,8 @@ class SVD_LlamaAttention(nn.Module):
         self._ensure_runtime_state()
         B, T, d = x.shape
         H, Hk, Dh = self.num_heads, self.num_key_value_heads, self.head_dim
+        if isinstance(cache, FlashSVDLegacySparseKVCache):
+            return self._prefill_tokens_rank(x, cache, cache_position, norm_weight=norm_weight, eps=eps, residual=residual)
         # no cache_position means "prefill from slot 0", as in the reference caches' update()
         start = 0 if cache_position is None else int(cache_position.reshape(-1)[0])
         if start < 0 or start + T > cache.max_cache_len:
@@ -325,6 +351,38 @@ class SVD_LlamaAttention(nn.Module):
         po = hip_ops.linear(a, self.o_v_proj.weight)
         return hip_ops.linear(po, self.o_u_proj.weight, residual=residual)
 
+
+def _prefill_tokens_rank(self, x, cache, cache_position=None, *, norm_weight=None, eps=1e-6, residual=None):
+    """Rank-space prefill with the decode kernel: coefficients of all T tokens go into the cache,
+    then the tokens of a sequence are the kernel's batch rows bound to one cache row (batch stride 0)
+    with key counts start+t+1.  K tiles are rebuilt once per query, so this is meant for short prompts."""
+    from .kernels.rank_decode import rank_decode
+    B, T, d = x.shape
+    H, Hk, Dh = self.num_heads, self.num_key_value_heads, self.head_dim
+    rq, rk, rv = self._qkv_rank_tuple()
+    start = 0 if cache_position is None else int(cache_position.reshape(-1)[0])
+    if start < 0 or start + T > cache.max_cache_len:
+        raise IndexError(f"{type(cache).__name__} write position out of range: start={start} q_len={T} max={cache.max_cache_len}")
+    cache.ensure_layer_ranks(self.layer_idx, rk, rv)
+    pkc, pvc = cache.key_cache[self.layer_idx], cache.value_cache[self.layer_idx]
+    rope = cache.get_rope_tables(seqlen=cache.max_cache_len, head_dim=Dh, device=x.device, dtype=x.dtype)
+    p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)           # [B,T,R*]
+    pkc[:B, start:start + T] = p[..., rq:rq + rk]
+    pvc[:B, start:start + T] = p[..., rq + rk:]
+    cache._layer_initialized[self.layer_idx] = True
+    cache._note_seen(self.layer_idx, T, cache_position)
+    q = hip_ops.linear(p[..., :rq].contiguous(), self.q_u_proj.weight).view(B, T, H, Dh)
+    lens = torch.arange(start + 1, start + T + 1, device=x.device, dtype=torch.int32)
+    a = torch.empty(B, T, H * Dh, device=x.device, dtype=x.dtype)
+    for b in range(B):
+        # the rotation position of query t is its own key count - 1, which rotate_q uses
+        rank_decode(q[b], pkc[b:b + 1].expand(T, -1, -1), pvc[b:b + 1].expand(T, -1, -1), self.k_u_proj.weight,
+                    self.v_u_proj.weight, rope[0], rope[1], lens, num_kv_heads=Hk, rotate_q=True, out=a[b].view(T, H, Dh))
+    po = hip_ops.linear(a, self.o_v_proj.weight)
+    return hip_ops.linear(po, self.o_u_proj.weight, residual=residual)
+
+
+SVD_LlamaAttention._prefill_tokens_rank = _prefill_tokens_rank
 
 _FUSED_ROUNDING_BACKENDS = {
     "flashsvd_mlp_dual_split_prod", "flashsvd_mlp_dual_split_cutlass", "flashsvd_mlp_dual_split_triton_v1",

@@ -147,6 +147,27 @@ int fsvd_mlp_dual_split(const void* PUp, int64_t sPUp_t, const void* PGate, int6
                         void* Y, int64_t ldY, float* S_out, int T, int R, int D, int Hd, int dtype,
                         int variant, int bd, int partials_fp32, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Single-query attention over a rank-space KV cache (pre-RoPE coefficients Pk, Pv [B,S,R] shared
+ * by all heads; runtime/cache/attn_legacy_sparse_kv.py:22-35).  K tiles are rebuilt in-kernel as
+ * Pk @ k_u[h]^T on the matrix cores and rotated at absolute key positions, the softmax weights are
+ * applied to Pv in rank space and one product with v_u[h] finishes each head.  Semantics of the
+ * reference's streaming decode, benchmark/attn/decode_compare.py:675-750, and of the (absent) fused
+ * kernels behind flashsvd_attn_decode_packed (:823-948): q [B,H,Dh] is the current token's query
+ * (rotate_q != 0 rotates it at position n_keys-1), k_u / v_u are nn.Linear-layout u_proj weights
+ * [Hk*Dh, R] (= per-head bases V[h][r][d] = u[h*Dh+d][r]), workspaces are the reference's split-K
+ * buffers M, L [B,H,nsplit] and Acc [B,H,nsplit,Rv] (fp32), n_keys = cache_seqlens[b] + seqlen_add.
+ * spk_h / spv_h are the kv-head strides of head-wise coefficient caches [B,S,Hk,R] (0 when shared).
+ * bf16 only; head_dim 128; ranks multiples of 8, Rv <= 2048. */
+int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,
+                            const void* pk_cache, int64_t spk_b, int64_t spk_s, int64_t spk_h,
+                            const void* pv_cache, int64_t spv_b, int64_t spv_s, int64_t spv_h,
+                            const void* k_u, int64_t ldku, const void* v_u, int64_t ldvu, const void* bv,
+                            const void* cos, const void* sin, int rope_len, int rotate_q,
+                            const int32_t* cache_seqlens, int seqlen_add,
+                            float* ws_m, float* ws_l, float* ws_acc,
+                            void* out, int64_t so_b, int64_t so_h,
+                            int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit, float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
