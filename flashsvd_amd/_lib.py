@@ -37,6 +37,12 @@ SIGNATURES = {
                                         c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                         c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                         c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
+    "fsvd_lowrank_expand_heads": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
+                                          c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
+                                          c_int, c_void_p]),
+    "fsvd_attn_prefill": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p,
+                                  c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
+                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "fsvd_xw_linear_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "fsvd_xw_linear": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int,
                                c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -371,4 +371,29 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h, const voi
   return launch_rank_decode(a, static_cast<hipStream_t>(stream));
 }
 
+int fsvd_lowrank_expand_heads(const void* p, int64_t sp_b, int64_t sp_m, int64_t sp_h, const void* u, int64_t ldu, const void* bias,
+                              const void* cos, const void* sin, int rope_len, const int32_t* positions, void* y, int64_t sy_b,
+                              int64_t sy_m, int64_t sy_h, int dst_by_position, int dst_rows, int B, int M, int heads, int Dh, int R,
+                              void* stream) {
+  const char* fn = "fsvd_lowrank_expand_heads";
+  FSVD_REQUIRE_PTR(p, fn); FSVD_REQUIRE_PTR(u, fn); FSVD_REQUIRE_PTR(y, fn);
+  if ((cos == nullptr) != (sin == nullptr) || (cos && rope_len <= 0)) { set_last_error("%s: cos/sin must both be set with rope_len > 0", fn); return kErrBadShape; }
+  if (ldu < R || sy_h < Dh || dst_rows <= 0) { set_last_error("%s: inconsistent strides (ldu=%lld R=%d sy_h=%lld dst_rows=%d)", fn, (long long)ldu, R, (long long)sy_h, dst_rows); return kErrBadShape; }
+  ExpandArgs a{cu16(p), sp_b, sp_m, sp_h, cu16(u), ldu, cu16(bias), cu16(cos), cu16(sin), rope_len, positions, u16(y), sy_b, sy_m,
+               sy_h, dst_by_position, dst_rows, B, M, heads, Dh, R};
+  return launch_expand(a, static_cast<hipStream_t>(stream));
+}
+
+int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h, const void* k, const void* v, int64_t sk_b,
+                      int64_t sk_s, int64_t sk_h, const int32_t* q_pos0, const uint8_t* pad_mask, int64_t spm_b,
+                      const float* add_mask, int64_t sam_b, int64_t sam_q, void* out, int64_t so_b, int64_t so_m, int64_t so_h,
+                      int B, int M, int H, int Hk, int Dh, int S, int causal, float scale, void* stream) {
+  const char* fn = "fsvd_attn_prefill";
+  FSVD_REQUIRE_PTR(q, fn); FSVD_REQUIRE_PTR(k, fn); FSVD_REQUIRE_PTR(v, fn); FSVD_REQUIRE_PTR(out, fn);
+  if (S <= 0 || (!q_pos0 && M > S)) { set_last_error("%s: %d queries do not fit %d cache rows", fn, M, S); return kErrBadShape; }
+  PrefillAttnArgs a{cu16(q), sq_b, sq_m, sq_h, cu16(k), cu16(v), sk_b, sk_s, sk_h, q_pos0, pad_mask, spm_b, add_mask, sam_b, sam_q,
+                    u16(out), so_b, so_m, so_h, B, M, H, Hk, Dh, S, causal, scale > 0.f ? scale : 1.0f / sqrtf((float)Dh)};
+  return launch_prefill_attn(a, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

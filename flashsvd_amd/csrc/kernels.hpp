@@ -109,6 +109,30 @@ struct RankDecodeArgs {
 };
 int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st);
 
+struct ExpandArgs {
+  const uint16_t* p; int64_t sp_b, sp_m, sp_h;      // rank coefficients [B,M,(heads),R]; sp_h = 0 when shared
+  const uint16_t* u; int64_t ldu;                   // [heads*Dh, R] nn.Linear layout
+  const uint16_t* bias;                             // [heads*Dh] or null
+  const uint16_t* cos; const uint16_t* sin; int rope_len;   // rotation tables or null
+  const int32_t* positions;                         // [B] absolute position of token 0 of each row (null = 0)
+  uint16_t* y; int64_t sy_b, sy_m, sy_h;            // destination [B, rows, heads, Dh]
+  int dst_by_position;                              // 1: destination row = absolute position (cache), 0: row = m
+  int dst_rows;                                     // rows the destination has (bounds check)
+  int B, M, heads, Dh, R;
+};
+struct PrefillAttnArgs {
+  const uint16_t* q; int64_t sq_b, sq_m, sq_h;      // [B,M,H,Dh], rotated
+  const uint16_t* k; const uint16_t* v; int64_t sk_b, sk_s, sk_h;   // [B,S,Hk,Dh]
+  const int32_t* q_pos0;                            // [B] absolute position of query row 0 (null = 0)
+  const uint8_t* pad_mask; int64_t spm_b;           // [B, keys] 1 = valid, or null
+  const float* add_mask; int64_t sam_b, sam_q;      // [B, M, keys] additive, or null
+  uint16_t* out; int64_t so_b, so_m, so_h;          // [B,M,H,Dh]
+  int B, M, H, Hk, Dh, S, causal;
+  float scale;
+};
+int launch_expand(const ExpandArgs& a, hipStream_t st);
+int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st);
+
 int launch_linear(const LinearArgs& a, int cfg, hipStream_t st);
 int launch_swiglu(const SwigluArgs& a, int cfg, hipStream_t st);
 int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st);

@@ -1,0 +1,266 @@
+// Full-sequence (prefill) side of the low-rank RoPE attention, split the way a 288 GB part wants it:
+//
+//  1. lowrank_expand_kernel — Y = P @ u^T on the matrix cores for all tokens at once, with the head
+//     epilogue fused: bias, rotate-half RoPE at the token's absolute position, and a strided store
+//     straight into its destination (the query buffer [B,M,H,dh], or the dense KV cache rows
+//     [B,S,Hk,dh] the decode kernels read later).  Both MFMA operands are contiguous along the rank
+//     axis (P rows, nn.Linear-layout u rows), so they are plain 16-byte global loads in the
+//     instruction's native lane layout; a wave owns 32 tokens x 128 head columns (16 accumulator
+//     tiles) and d / d+64 of a head sit in the same lane, which keeps the rotation register-local.
+//     K and V are rebuilt exactly once per token (the reference's fused kernel rebuilds every key
+//     tile once per query tile to avoid the HBM round trip; with 288 GB that trade goes the other way).
+//
+//  2. attn_prefill_kernel — causal flash attention over the rotated q and the cache rows: S = Q K^T
+//     and O += P V on MFMA 16x16x32 bf16, online softmax in fp32 on the accumulator layout, P passed
+//     through LDS to become an A operand, V tile transposed through LDS to become a B operand.
+//     Key padding mask, additive mask and "fully masked row -> 0" follow the reference kernel.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace fsvd {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kPfThreads = 256;
+
+__device__ __forceinline__ bf16x8_t pf_ld(const uint16_t* p) {
+  return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(p));
+}
+__device__ __forceinline__ bf16x8_t pf_zero() { return __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u}); }
+
+// ---------------------------------------------------------------------------------------------
+// 1. Y[token, head, :] = epilogue( P[token, (head), :] @ u[head*128 + :, :]^T )
+//    grid (ceil(T/128), heads), 4 waves x 32 tokens
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kPfThreads) void lowrank_expand_kernel(ExpandArgs a) {
+  constexpr int DH = 128, NT = 8, HALF = 64;
+  const int head = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int T = a.B * a.M;
+  const int row0 = blockIdx.x * 128 + wave * 32;
+  if (row0 >= T) return;
+
+  const uint16_t* arow[2];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+    const int r = min(row0 + mi * 16 + lr, T - 1);
+    const int b = r / a.M, m = r % a.M;
+    arow[mi] = a.p + (int64_t)b * a.sp_b + (int64_t)m * a.sp_m + (int64_t)head * a.sp_h + lg * 8;
+  }
+  const uint16_t* brow = a.u + (int64_t)(head * DH + lr) * a.ldu + lg * 8;
+
+  f32x4_t acc[2][NT];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mi][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int r0 = 0; r0 < a.R; r0 += 32) {
+    const bool in = r0 + lg * 8 < a.R;
+    bf16x8_t af[2], bf[NT];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) af[mi] = in ? pf_ld(arow[mi] + r0) : pf_zero();
+#pragma unroll
+    for (int t = 0; t < NT; ++t) bf[t] = in ? pf_ld(brow + (int64_t)t * 16 * a.ldu + r0) : pf_zero();
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mi], bf[t], acc[mi][t], 0, 0, 0);
+  }
+
+  // epilogue on the accumulator layout: lane holds rows lg*4+i, column t*16+lr of each tile
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = row0 + mi * 16 + lg * 4 + i;
+      if (r >= T) continue;
+      const int b = r / a.M, m = r % a.M;
+      const int pos = (a.positions ? a.positions[b] : 0) + m;
+      float x[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        float v = acc[mi][t][i];
+        if (a.bias) v += bf16_bits_to_f32(a.bias[head * DH + t * 16 + lr]);
+        x[t] = round_bf16(v);                       // the projection's own rounding point
+      }
+      if (a.cos) {
+        // eager bf16 arithmetic: x0*c - x1*s and x1*c + x0*s, one rounding per op
+        const int tp = min(max(pos, 0), a.rope_len - 1);
+#pragma unroll
+        for (int t = 0; t < NT / 2; ++t) {
+          const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * HALF + t * 16 + lr]);
+          const float s = bf16_bits_to_f32(a.sin[(int64_t)tp * HALF + t * 16 + lr]);
+          const float x0 = x[t], x1 = x[t + NT / 2];
+          x[t] = round_bf16(round_bf16(x0 * c) - round_bf16(x1 * s));
+          x[t + NT / 2] = round_bf16(round_bf16(x1 * c) + round_bf16(x0 * s));
+        }
+      }
+      const int slot = a.dst_by_position ? pos : m;
+      if (slot < 0 || slot >= a.dst_rows) continue;   // outside the destination: dropped
+      uint16_t* dst = a.y + (int64_t)b * a.sy_b + (int64_t)slot * a.sy_m + (int64_t)head * a.sy_h;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) dst[t * 16 + lr] = (uint16_t)f32_to_bf16_bits(x[t]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 2. causal flash attention, head_dim 128, 64 queries per workgroup (16 per wave), 64-key tiles
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArgs a) {
+  constexpr int DH = 128, BN = 64, PSTR = BN + 8, VSTR = BN + 8;
+  __shared__ __align__(16) uint16_t Ps[4][16][PSTR];
+  __shared__ __align__(16) uint16_t Vt[DH][VSTR];
+
+  const int mt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int hk = h / (a.H / a.Hk);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int q0 = a.q_pos0 ? a.q_pos0[b] : 0;          // absolute position of query row 0
+  const int m_base = mt * 64 + wave * 16;             // first query row of this wave
+  const int n_keys_all = max(1, min(q0 + a.M, a.S));  // keys that exist once the block is appended
+
+  // Q fragments (A operand): row m_base+lr, d = step*32 + lg*8
+  bf16x8_t qf[4];
+  {
+    const int m = min(m_base + lr, a.M - 1);
+    const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)m * a.sq_m + (int64_t)h * a.sq_h + lg * 8;
+#pragma unroll
+    for (int st = 0; st < 4; ++st) qf[st] = pf_ld(qp + st * 32);
+  }
+  float m_run[4], l_run[4];
+  f32x4_t o[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m_run[i] = -INFINITY; l_run[i] = 0.f; }
+#pragma unroll
+  for (int t = 0; t < 8; ++t) o[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  // last key any row of this workgroup may see (causal): position of its last valid query
+  const int last_m = min(mt * 64 + 63, a.M - 1);
+  const int k_end = a.causal ? min(n_keys_all, q0 + last_m + 1) : n_keys_all;
+  const uint16_t* kb = a.k + (int64_t)b * a.sk_b + (int64_t)hk * a.sk_h;
+  const uint16_t* vb = a.v + (int64_t)b * a.sk_b + (int64_t)hk * a.sk_h;
+
+  for (int n0 = 0; n0 < k_end; n0 += BN) {
+    // ---- stage V tile transposed: thread -> key n0 + tid/16 (+16 per pass), d0 = (tid%16)*8
+    __syncthreads();   // previous tile's Vt / Ps fully consumed
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+      const int kk = pass * 16 + (tid >> 4);
+      const int key = min(n0 + kk, n_keys_all - 1);
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(vb + (int64_t)key * a.sk_s + (tid & 15) * 8);
+      const int d0 = (tid & 15) * 8;
+      Vt[d0 + 0][kk] = (uint16_t)(v.x & 0xffff); Vt[d0 + 1][kk] = (uint16_t)(v.x >> 16);
+      Vt[d0 + 2][kk] = (uint16_t)(v.y & 0xffff); Vt[d0 + 3][kk] = (uint16_t)(v.y >> 16);
+      Vt[d0 + 4][kk] = (uint16_t)(v.z & 0xffff); Vt[d0 + 5][kk] = (uint16_t)(v.z >> 16);
+      Vt[d0 + 6][kk] = (uint16_t)(v.w & 0xffff); Vt[d0 + 7][kk] = (uint16_t)(v.w >> 16);
+    }
+    // ---- S = Q K^T for 16 rows x 64 keys (4 tiles); K rows are B operands straight from memory
+    f32x4_t s[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      s[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const int key = min(n0 + j * 16 + lr, n_keys_all - 1);
+      const uint16_t* kp = kb + (int64_t)key * a.sk_s + lg * 8;
+#pragma unroll
+      for (int st = 0; st < 4; ++st) s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[st], pf_ld(kp + st * 32), s[j], 0, 0, 0);
+    }
+    // ---- masks + online softmax on the accumulator layout (rows lg*4+i, key column j*16+lr)
+    float p[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m_base + lg * 4 + i;
+      const int qpos = q0 + m;
+      float rmax = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int key = n0 + j * 16 + lr;
+        float v = s[j][i];
+        bool ok = key < n_keys_all && m < a.M;
+        if (a.causal) ok = ok && key <= qpos;
+        v = ok ? v * a.scale : -INFINITY;            // mask first, then scale, as the reference kernel
+        if (ok && a.pad_mask) ok = a.pad_mask[(int64_t)b * a.spm_b + key] != 0;
+        if (!ok) v = -INFINITY;
+        if (ok && a.add_mask) v += a.add_mask[(int64_t)b * a.sam_b + (int64_t)m * a.sam_q + key];
+        p[j][i] = v;
+        rmax = fmaxf(rmax, v);
+      }
+      rmax = row16_max(rmax);
+      const float m_new = fmaxf(m_run[i], rmax);
+      const float alpha = (m_run[i] == -INFINITY) ? 0.f : __expf(m_run[i] - m_new);
+      float rsum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float e = (p[j][i] == -INFINITY || m_new == -INFINITY) ? 0.f : __expf(p[j][i] - m_new);
+        p[j][i] = e;
+        rsum += e;
+      }
+      rsum = row16_sum(rsum);
+      l_run[i] = l_run[i] * alpha + rsum;
+      m_run[i] = m_new;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) o[t][i] *= alpha;
+    }
+    // ---- P (bf16) to LDS in row-major so that it can be re-read as an A operand
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) Ps[wave][lg * 4 + i][j * 16 + lr] = (uint16_t)f32_to_bf16_bits(p[j][i]);
+    __syncthreads();   // Vt and Ps visible
+    // ---- O += P V : A = Ps[row lr][keys st*32 + lg*8 ..], B = Vt[d = t*16+lr][keys st*32 + lg*8 ..]
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const bf16x8_t pa = pf_ld(&Ps[wave][lr][st * 32 + lg * 8]);
+#pragma unroll
+      for (int t = 0; t < 8; ++t)
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, pf_ld(&Vt[t * 16 + lr][st * 32 + lg * 8]), o[t], 0, 0, 0);
+    }
+  }
+
+  // ---- normalise and store; rows with no visible key give 0
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m_base + lg * 4 + i;
+    if (m >= a.M) continue;
+    const float inv = l_run[i] > 0.f ? 1.0f / l_run[i] : 0.f;
+    uint16_t* op = a.out + (int64_t)b * a.so_b + (int64_t)m * a.so_m + (int64_t)h * a.so_h;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) op[t * 16 + lr] = (uint16_t)f32_to_bf16_bits(o[t][i] * inv);
+  }
+}
+
+int launch_expand(const ExpandArgs& a, hipStream_t st) {
+  const char* fn = "fsvd_lowrank_expand_heads";
+  if (a.B <= 0 || a.M <= 0 || a.heads <= 0 || a.R <= 0) { set_last_error("%s: empty shape", fn); return kErrBadShape; }
+  if (a.Dh != 128) { set_last_error("%s: head_dim %d is not 128", fn, a.Dh); return kErrBadShape; }
+  if (a.R % 8) { set_last_error("%s: rank %d is not a multiple of 8; pad the factors", fn, a.R); return kErrBadShape; }
+  const auto mis = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+  if (mis(a.p) || mis(a.u) || (a.sp_b % 8) || (a.sp_m % 8) || (a.sp_h % 8) || (a.ldu % 8)) {
+    set_last_error("%s: coefficient / factor pointers and strides must be 16-byte aligned", fn);
+    return kErrBadAlign;
+  }
+  const int T = a.B * a.M;
+  hipLaunchKernelGGL(lowrank_expand_kernel, dim3((T + 127) / 128, a.heads), dim3(kPfThreads), 0, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
+int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
+  const char* fn = "fsvd_attn_prefill";
+  if (a.B <= 0 || a.M <= 0 || a.H <= 0 || a.Hk <= 0 || a.H % a.Hk) { set_last_error("%s: bad shape", fn); return kErrBadShape; }
+  if (a.Dh != 128) { set_last_error("%s: head_dim %d is not 128", fn, a.Dh); return kErrBadShape; }
+  const auto mis = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+  if (mis(a.q) || mis(a.k) || mis(a.v) || (a.sq_b % 8) || (a.sq_m % 8) || (a.sq_h % 8) || (a.sk_b % 8) || (a.sk_s % 8) || (a.sk_h % 8)) {
+    set_last_error("%s: q / k / v pointers and strides must be 16-byte aligned", fn);
+    return kErrBadAlign;
+  }
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), 0, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
+}  // namespace fsvd

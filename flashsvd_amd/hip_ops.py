@@ -223,3 +223,84 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, out: Optio
                           x2.shape[0], K, _stream())
     _lib.check("fsvd_rmsnorm", rc)
     return out
+
+
+def lowrank_expand_heads(p: torch.Tensor, u: torch.Tensor, *, num_heads: int, head_dim: int, out: torch.Tensor,
+                         cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                         positions: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+                         dst_by_position: bool = False, head_stride: Optional[int] = None) -> torch.Tensor:
+    """out[b, row, h, :] = rope(p[b, m, (h), :] @ u[h*Dh:(h+1)*Dh].T + bias); see fsvd_lowrank_expand_heads.
+    p is [B, M, R] (shared by all heads) or [B, M, heads, R]; out is [B, rows, heads, Dh]."""
+    _need(p, "p"); _need(u, "u"); _need(out, "out")
+    heads, Dh = int(num_heads), int(head_dim)
+    if p.dim() == 3:
+        B, M, R = p.shape
+        sp = (p.stride(0), p.stride(1), 0 if head_stride is None else int(head_stride))
+    elif p.dim() == 4:
+        B, M, hp, R = p.shape
+        if hp != heads:
+            raise ValueError(f"p has {hp} heads, expected {heads}")
+        sp = (p.stride(0), p.stride(1), p.stride(2))
+    else:
+        raise ValueError(f"p must be [B,M,R] or [B,M,heads,R], got {tuple(p.shape)}")
+    if p.stride(-1) != 1 or u.stride(1) != 1 or out.stride(-1) != 1:
+        raise ValueError("p, u and out need unit stride on the last axis")
+    if u.shape != (heads * Dh, R):
+        raise ValueError(f"u must be [{heads * Dh}, {R}], got {tuple(u.shape)}")
+    if out.dim() != 4 or out.shape[0] < B or out.shape[2] != heads or out.shape[3] != Dh:
+        raise ValueError(f"out must be [B>={B}, rows, {heads}, {Dh}], got {tuple(out.shape)}")
+    rope_len = 0
+    if cos is not None:
+        _need(cos, "cos"); _need(sin, "sin")
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2 or not cos.is_contiguous() or not sin.is_contiguous():
+            raise ValueError(f"cos/sin must be contiguous [len, {Dh // 2}] tables")
+        rope_len = cos.shape[0]
+    if positions is not None:
+        _need(positions, "positions", dtype=torch.int32)
+        if positions.numel() != B:
+            raise ValueError(f"positions must be int32 [{B}]")
+    if bias is not None:
+        _need(bias, "bias")
+        if bias.numel() != heads * Dh or not bias.is_contiguous():
+            raise ValueError(f"bias must be contiguous [{heads * Dh}]")
+    lib = _lib.load()
+    rc = lib.fsvd_lowrank_expand_heads(p.data_ptr(), sp[0], sp[1], sp[2], u.data_ptr(), u.stride(0), _ptr(bias), _ptr(cos), _ptr(sin),
+                                       rope_len, _ptr(positions), out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+                                       int(bool(dst_by_position)), out.shape[1], B, M, heads, Dh, R, _stream())
+    _lib.check("fsvd_lowrank_expand_heads", rc)
+    return out
+
+
+def attn_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, q_pos0: Optional[torch.Tensor] = None, causal: bool = True,
+                 pad_mask: Optional[torch.Tensor] = None, add_mask: Optional[torch.Tensor] = None,
+                 out: Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None) -> torch.Tensor:
+    """q [B,M,H,Dh] (rotated), k/v [B,S,Hk,Dh] -> out [B,M,H,Dh]; keys n < q_pos0[b]+M, causal n <= q_pos0[b]+m."""
+    _need(q, "q"); _need(k, "k"); _need(v, "v")
+    if q.dim() != 4 or k.dim() != 4 or k.shape != v.shape or k.stride() != v.stride():
+        raise ValueError(f"q must be [B,M,H,Dh] and k/v matching [B,S,Hk,Dh], got {tuple(q.shape)} {tuple(k.shape)} {tuple(v.shape)}")
+    B, M, H, Dh = q.shape
+    S, Hk = k.shape[1], k.shape[2]
+    if k.shape[0] < B or k.shape[3] != Dh or H % Hk:
+        raise ValueError("k/v do not match q")
+    if q.stride(3) != 1 or k.stride(3) != 1:
+        raise ValueError("q, k, v need unit stride on the last axis")
+    if out is None:
+        out = torch.empty(B, M, H, Dh, device=q.device, dtype=_BF16)
+    spm = sam_b = sam_q = 0
+    if pad_mask is not None:
+        if pad_mask.dtype != torch.uint8 or pad_mask.dim() != 2 or pad_mask.shape[0] != B or pad_mask.stride(1) != 1:
+            raise ValueError("pad_mask must be uint8 [B, keys]")
+        spm = pad_mask.stride(0)
+    if add_mask is not None:
+        if add_mask.dtype != torch.float32 or add_mask.dim() != 3 or add_mask.shape[0] != B or add_mask.shape[1] != M or add_mask.stride(2) != 1:
+            raise ValueError("add_mask must be float32 [B, M, keys]")
+        sam_b, sam_q = add_mask.stride(0), add_mask.stride(1)
+    if q_pos0 is not None:
+        _need(q_pos0, "q_pos0", dtype=torch.int32)
+    lib = _lib.load()
+    rc = lib.fsvd_attn_prefill(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), k.data_ptr(), v.data_ptr(), k.stride(0),
+                               k.stride(1), k.stride(2), _ptr(q_pos0), _ptr(pad_mask), spm, _ptr(add_mask), sam_b, sam_q,
+                               out.data_ptr(), out.stride(0), out.stride(1), out.stride(2), B, M, H, Hk, Dh, S, int(bool(causal)),
+                               float(softmax_scale) if softmax_scale else 0.0, _stream())
+    _lib.check("fsvd_attn_prefill", rc)
+    return out

@@ -321,9 +321,12 @@ class SVD_LlamaAttention(nn.Module):
 
     def prefill_tokens(self, x: torch.Tensor, cache, cache_position=None, *, norm_weight=None, eps: float = 1e-6,
                        residual: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Causal full-sequence pass expressed with the decode kernels: the T tokens of one
-        sequence are the kernel's batch rows, all bound to the same cache row (batch stride 0),
-        token t written at start+t and attending over start+t+1 keys."""
+        """Causal full-sequence pass; T tokens are appended at start..start+T-1.
+        head_dim 128 with ranks that are multiples of 8 takes the matrix-core route (q/k/v rebuilt once
+        per token with the rotation fused, then causal flash attention over the cache).  Other shapes
+        (or FLASHSVD_AMD_PREFILL=decode) reuse the decode kernels: the T tokens of one sequence are the
+        kernel's batch rows, all bound to the same cache row (batch stride 0), token t written at
+        start+t and attending over start+t+1 keys."""
         self._ensure_runtime_state()
         B, T, d = x.shape
         H, Hk, Dh = self.num_heads, self.num_key_value_heads, self.head_dim
@@ -337,15 +340,31 @@ class SVD_LlamaAttention(nn.Module):
         cache._ensure_layer_spec(self.layer_idx, h=Hk, dh=Dh)
         kc, vc = cache.key_cache[self.layer_idx], cache.value_cache[self.layer_idx]
         rope = cache.get_rope_tables(seqlen=cache.max_cache_len, head_dim=Dh, device=x.device, dtype=x.dtype)
-        positions = torch.arange(start, start + T, device=x.device, dtype=torch.int32)
         p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)       # [B,T,Rtot]
-        nsplit = hip_ops.pick_nsplit(cache.max_cache_len, T, H, Dh)
+        rq, rk, rv = self._qkv_rank_tuple()
+        mfma_ok = Dh == 128 and rq % 8 == 0 and rk % 8 == 0 and rv % 8 == 0 and T >= 16 \
+            and os.getenv("FLASHSVD_AMD_PREFILL", "mfma").strip().lower() != "decode"
         a = torch.empty(B, T, H * Dh, device=x.device, dtype=x.dtype)
-        for b in range(B):
-            kb, vb = kc[b:b + 1].expand(T, -1, -1, -1), vc[b:b + 1].expand(T, -1, -1, -1)
-            q = hip_ops.qkv_rope_append(p[b], self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight,
-                                        rope[0], rope[1], positions, kb, vb, num_heads=H, num_kv_heads=Hk, head_dim=Dh)
-            hip_ops.attn_decode_densekv(q, kb, vb, positions, seqlen_add=1, nsplit=nsplit, out=a[b].view(T, H, Dh))
+        if mfma_ok:
+            # matrix-core route: q/k/v rebuilt once per token with the rotation fused (k, v land in the
+            # cache rows start..start+T-1), then causal flash attention over the cache
+            pos0 = torch.full((B,), start, device=x.device, dtype=torch.int32)
+            q = torch.empty(B, T, H, Dh, device=x.device, dtype=x.dtype)
+            hip_ops.lowrank_expand_heads(p[..., :rq], self.q_u_proj.weight, num_heads=H, head_dim=Dh, out=q,
+                                         cos=rope[0], sin=rope[1], positions=pos0)
+            hip_ops.lowrank_expand_heads(p[..., rq:rq + rk], self.k_u_proj.weight, num_heads=Hk, head_dim=Dh, out=kc[:B],
+                                         cos=rope[0], sin=rope[1], positions=pos0, dst_by_position=True)
+            hip_ops.lowrank_expand_heads(p[..., rq + rk:], self.v_u_proj.weight, num_heads=Hk, head_dim=Dh, out=vc[:B],
+                                         positions=pos0, dst_by_position=True)
+            hip_ops.attn_prefill(q, kc[:B], vc[:B], q_pos0=pos0, causal=True, out=a.view(B, T, H, Dh))
+        else:
+            positions = torch.arange(start, start + T, device=x.device, dtype=torch.int32)
+            nsplit = hip_ops.pick_nsplit(cache.max_cache_len, T, H, Dh)
+            for b in range(B):
+                kb, vb = kc[b:b + 1].expand(T, -1, -1, -1), vc[b:b + 1].expand(T, -1, -1, -1)
+                q = hip_ops.qkv_rope_append(p[b], self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight,
+                                            rope[0], rope[1], positions, kb, vb, num_heads=H, num_kv_heads=Hk, head_dim=Dh)
+                hip_ops.attn_decode_densekv(q, kb, vb, positions, seqlen_add=1, nsplit=nsplit, out=a[b].view(T, H, Dh))
         cache._layer_initialized[self.layer_idx] = True
         cache._note_seen(self.layer_idx, T, cache_position)
         po = hip_ops.linear(a, self.o_v_proj.weight)

@@ -168,6 +168,31 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,
                             void* out, int64_t so_b, int64_t so_h,
                             int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit, float scale, void* stream);
 
+/* Full-sequence low-rank RoPE attention = the role of the fused Triton kernel flashsvd_rope_sdpa
+ * (kernels/attn/prefill/rope_sdpa.py:67-248, wrapper FlashSVDRoPEAttention :254-427), as two launches:
+ *
+ * fsvd_lowrank_expand_heads: y[b, row, head, :] = P[b,m,(head),:] @ u[head*Dh:(head+1)*Dh, :]^T
+ *   (+ bias), rounded to bf16, then rotate-half RoPE at position positions[b]+m when cos/sin are given,
+ *   stored at row = m (dst_by_position = 0: a query buffer [B,M,H,Dh]) or row = positions[b]+m
+ *   (dst_by_position = 1: the dense KV cache [B,S,Hk,Dh]; rows outside [0,dst_rows) are dropped).
+ *   P is [B,M,heads,R] with sp_h = 0 for coefficients shared by all heads; u is the nn.Linear-layout
+ *   u_proj weight [heads*Dh, R] (per-head basis V[h][r][d] = u[h*Dh+d][r]).  bf16, Dh = 128, R % 8 == 0.
+ *
+ * fsvd_attn_prefill: out[b,m,h,:] = softmax_n(q[b,m,h,:] . k[b,n,hk,:] * scale + masks) v[b,n,hk,:]
+ *   over keys n < q_pos0[b] + M, causal (n <= q_pos0[b] + m) when causal != 0; pad_mask [B,keys] (0 =
+ *   masked key), add_mask [B,M,keys] fp32 added to the scaled scores; rows with no visible key give 0
+ *   (rope_sdpa.py:195-209,244-246).  q is already rotated; k is the post-RoPE cache. */
+int fsvd_lowrank_expand_heads(const void* p, int64_t sp_b, int64_t sp_m, int64_t sp_h, const void* u, int64_t ldu,
+                              const void* bias, const void* cos, const void* sin, int rope_len, const int32_t* positions,
+                              void* y, int64_t sy_b, int64_t sy_m, int64_t sy_h, int dst_by_position, int dst_rows,
+                              int B, int M, int heads, int Dh, int R, void* stream);
+int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
+                      const void* k, const void* v, int64_t sk_b, int64_t sk_s, int64_t sk_h,
+                      const int32_t* q_pos0, const uint8_t* pad_mask, int64_t spm_b,
+                      const float* add_mask, int64_t sam_b, int64_t sam_q,
+                      void* out, int64_t so_b, int64_t so_m, int64_t so_h,
+                      int B, int M, int H, int Hk, int Dh, int S, int causal, float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,121 @@
+"""GPU parity of the full-sequence low-rank RoPE attention (matrix-core rebuild of q/k/v + causal flash
+attention) against the CPU oracle; bf16 within max-abs 2e-2 / max-rel 1e-2."""
+import os
+
+import pytest
+import torch
+
+from oracle import flashsvd_oracle as O
+from tests.util import assert_close_bf16, bounds, model_from_oracle, rand_bf16
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+class _Rot:
+    def __init__(self, dh, theta=10000.0):
+        half = dh // 2
+        self.inv_freq = 1.0 / (theta ** (torch.arange(0, half, dtype=torch.float32) / half))
+
+
+def _factors(B, H, Hk, M, R, dh, shared, seed=0):
+    if shared:
+        pq, pk, pv = (rand_bf16(B, 1, M, R, seed=seed + i) for i in range(3))
+        Pq, Pk, Pv = pq.expand(B, H, M, R), pk.expand(B, Hk, M, R), pv.expand(B, Hk, M, R)
+    else:
+        Pq, Pk, Pv = rand_bf16(B, H, M, R, seed=seed), rand_bf16(B, Hk, M, R, seed=seed + 1), rand_bf16(B, Hk, M, R, seed=seed + 2)
+    s = R ** -0.5
+    Vq, Vk, Vv = rand_bf16(H, R, dh, std=s, seed=seed + 3), rand_bf16(Hk, R, dh, std=s, seed=seed + 4), rand_bf16(Hk, R, dh, std=s, seed=seed + 5)
+    return Pq, Pk, Pv, Vq, Vk, Vv
+
+
+@pytest.mark.parametrize("B,H,Hk,M,R,shared", [(1, 32, 32, 512, 1024, True), (2, 4, 2, 100, 40, False), (3, 2, 2, 1, 16, True),
+                                               (1, 8, 8, 333, 1664, True), (2, 4, 4, 65, 8, False)])
+def test_rope_attention_module_vs_oracle(B, H, Hk, M, R, shared):
+    from flashsvd_amd.kernels.flashsvdropeattn import FlashSVDRoPEAttention, QKVFactors
+    dh = 128
+    Pq, Pk, Pv, Vq, Vk, Vv = _factors(B, H, Hk, M, R, dh, shared)
+    cos, sin = O.rope_tables(M, dh, dtype=BF16)
+    ref = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin)
+    mod = FlashSVDRoPEAttention(H, dh, _Rot(dh), bm=64, bn=64, br=64)
+    g = [t.cuda() for t in (Pq, Pk, Pv, Vq, Vk, Vv)]
+    out = mod(QKVFactors(*g), None, torch.arange(M, device="cuda")[None])
+    assert out.shape == (B, M, H, dh) and out.dtype == BF16
+    assert_close_bf16(out, ref, "prefill", **bounds(ref))
+
+
+def test_rope_attention_masks_biases_positions():
+    from flashsvd_amd.kernels.rope_attn import FlashSVDRoPEAttention, QKVFactors
+    B, H, Hk, M, R, dh = 2, 4, 4, 70, 48, 128
+    Pq, Pk, Pv, Vq, Vk, Vv = _factors(B, H, Hk, M, R, dh, False, seed=10)
+    bq, bk, bv = rand_bf16(H * dh, std=0.1, seed=20), rand_bf16(H * dh, std=0.1, seed=21), rand_bf16(H * dh, std=0.1, seed=22)
+    # left-padded second row, per-row positions
+    pad = torch.ones(B, M, dtype=torch.long)
+    pad[1, :9] = 0
+    pos = torch.stack([torch.arange(M), (torch.arange(M) - 9).clamp_min(0)])
+    ang = pos.float()[..., None] * _Rot(dh).inv_freq
+    cos, sin = torch.cos(ang).to(BF16), torch.sin(ang).to(BF16)
+    ref = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin, bq=bq, bk=bk, bv=bv, pad_mask=pad)
+    mod = FlashSVDRoPEAttention(H, dh, _Rot(dh))
+    g = [t.cuda() for t in (Pq, Pk, Pv, Vq, Vk, Vv)]
+    out = mod(QKVFactors(*g, bq=bq.cuda(), bk=bk.cuda(), bv=bv.cuda()), pad.cuda(), pos.cuda())
+    assert torch.all(out[1, :9] == 0)                     # rows whose keys are all padded give 0
+    assert_close_bf16(out, ref, "pad + bias + positions", **bounds(ref))
+    # additive mask that forbids a band of keys for every query
+    add = torch.zeros(B, 1, M, M)
+    add[:, :, :, 5:12] = float("-inf")
+    add[0, :, :, 0] = -1.5
+    ref2 = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos[:1].expand(B, M, dh // 2), sin[:1].expand(B, M, dh // 2), add_mask=add)
+    out2 = mod(QKVFactors(*g), add.to(BF16).cuda(), pos[:1].cuda())
+    assert_close_bf16(out2, ref2, "additive mask", **bounds(ref2))
+    with pytest.raises(ValueError, match=r"expects Pq \[B,H,M,R\]"):
+        mod(QKVFactors(g[0][0], *g[1:]), None, pos.cuda())
+    with pytest.raises(ValueError, match="position_ids last dim"):
+        mod(QKVFactors(*g), None, pos[:, :5].cuda())
+    with pytest.raises(NotImplementedError):
+        mod(QKVFactors(*[t.float() for t in g]), None, pos.cuda())
+
+
+def test_expand_and_prefill_attention_primitives():
+    from flashsvd_amd import hip_ops
+    B, M, H, Hk, dh, R, S, start = 2, 40, 4, 2, 128, 72, 96, 13
+    cos, sin = O.rope_tables(S, dh, dtype=BF16)
+    p = rand_bf16(B, M, R, seed=1)
+    u = rand_bf16(Hk * dh, R, std=R ** -0.5, seed=2)
+    kc = torch.zeros(B, S, Hk, dh, dtype=BF16, device="cuda")
+    pos0 = torch.full((B,), start, dtype=torch.int32, device="cuda")
+    hip_ops.lowrank_expand_heads(p.cuda(), u.cuda(), num_heads=Hk, head_dim=dh, out=kc, cos=cos.cuda(), sin=sin.cuda(),
+                                 positions=pos0, dst_by_position=True)
+    ref = O.apply_rope(O.lin(p, u).reshape(B, M, Hk, dh), cos[start:start + M][None, :, None], sin[start:start + M][None, :, None])
+    assert_close_bf16(kc[:, start:start + M], ref, "expand into cache rows", **bounds(ref))
+    assert torch.all(kc[:, :start] == 0) and torch.all(kc[:, start + M:] == 0)
+    # chunked prefill: queries at positions start.. attend over the prefix already in the cache
+    kfull, vfull = rand_bf16(B, S, Hk, dh, seed=3), rand_bf16(B, S, Hk, dh, seed=4)
+    q = rand_bf16(B, M, H, dh, seed=5)
+    out = hip_ops.attn_prefill(q.cuda(), kfull.cuda(), vfull.cuda(), q_pos0=pos0, causal=True)
+    for m in (0, 17, M - 1):
+        n = start + m + 1
+        refm = O.dense_decode_attn(q[:, m], kfull[:, :n], vfull[:, :n])
+        assert_close_bf16(out[:, m], refm, f"row {m}", **bounds(refm))
+
+
+def test_model_prefill_mfma_equals_decode_route():
+    mw = O.make_model(d=512, n_heads=4, n_kv_heads=2, head_dim=128, ffn=1024, attn_rank=96, mlp_rank=128, n_layers=2,
+                      vocab=300, dtype=BF16, seed=7, std=0.05)
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    model = model_from_oracle(mw)
+    ids = torch.randint(0, 300, (2, 50), generator=torch.Generator().manual_seed(3))
+    outs = {}
+    for route in ("mfma", "decode"):
+        os.environ["FLASHSVD_AMD_PREFILL"] = route
+        try:
+            cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=2, max_cache_len=64, device="cuda", dtype=BF16)
+            o = model(ids.cuda(), past_key_values=cache, cache_position=torch.arange(50))
+            outs[route] = (o.logits.clone(), o.hidden_states.clone(), cache.key_cache[0][:, :50].clone(), cache.value_cache[1][:, :50].clone())
+        finally:
+            del os.environ["FLASHSVD_AMD_PREFILL"]
+    ref_logits, ref_hidden = O.model_forward(mw, ids, last_only=False, return_hidden=True)
+    for route, (lg, hid, k0, v1) in outs.items():
+        assert_close_bf16(hid, ref_hidden, f"{route} hidden", rel_tol=3e-2)
+    assert_close_bf16(outs["mfma"][2], outs["decode"][2], "layer-0 K rows of the two routes", abs_tol=float("inf"), rel_tol=1e-2)
+    assert (outs["mfma"][2] != outs["decode"][2]).float().mean() < 0.01   # same rounding points: all but a few ulp flips identical

@@ -51,3 +51,10 @@ def model_from_oracle(mw, device="cuda"):
                               vocab_size=meta["vocab"], attn_rank=meta["attn_rank"], mlp_rank=meta["mlp_rank"],
                               rope_theta=mw.rope_theta, rms_norm_eps=mw.eps)
     return load_oracle_weights(model, mw, device)
+
+
+def bounds(ref):
+    """(abs_tol, rel_tol): 2e-2 / 1e-2, except that where max|ref| >= 2 one bf16 ulp already exceeds
+    1.5e-2, so the absolute bound becomes two ulps at max|ref|."""
+    m = float(ref.float().abs().max())
+    return dict(abs_tol=2e-2 if m < 2.0 else 2.0 * m * 2.0 ** -7, rel_tol=1e-2)
