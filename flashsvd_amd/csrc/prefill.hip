@@ -12,7 +12,7 @@
 //
 //  2. attn_prefill_kernel — causal flash attention over the rotated q and the cache rows: S = Q K^T
 //     and O += P V on MFMA 16x16x32 bf16, online softmax in fp32 on the accumulator layout, P passed
-//     through LDS to become an A operand, V tile transposed through LDS to become a B operand.
+//     through LDS (as a bf16 high part plus a bf16 residual) to become an A operand, V tile transposed through LDS to become a B operand.
 //     Key padding mask, additive mask and "fully masked row -> 0" follow the reference kernel.
 #include "common.hpp"
 #include "kernels.hpp"
@@ -111,7 +111,8 @@ __global__ __launch_bounds__(kPfThreads) void lowrank_expand_kernel(ExpandArgs a
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArgs a) {
   constexpr int DH = 128, BN = 64, PSTR = BN + 8, VSTR = BN + 8;
-  __shared__ __align__(16) uint16_t Ps[4][16][PSTR];
+  __shared__ __align__(16) uint16_t Ps[4][16][PSTR];    // softmax weights, bf16 high part
+  __shared__ __align__(16) uint16_t Pl[4][16][PSTR];    // and the bf16 residual, so that P carries ~16 mantissa bits
   __shared__ __align__(16) uint16_t Vt[DH][VSTR];
 
   const int mt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -207,15 +208,23 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) Ps[wave][lg * 4 + i][j * 16 + lr] = (uint16_t)f32_to_bf16_bits(p[j][i]);
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t hi = f32_to_bf16_bits(p[j][i]);
+        Ps[wave][lg * 4 + i][j * 16 + lr] = (uint16_t)hi;
+        Pl[wave][lg * 4 + i][j * 16 + lr] = (uint16_t)f32_to_bf16_bits(p[j][i] - bf16_bits_to_f32(hi));
+      }
     __syncthreads();   // Vt and Ps visible
     // ---- O += P V : A = Ps[row lr][keys st*32 + lg*8 ..], B = Vt[d = t*16+lr][keys st*32 + lg*8 ..]
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
       const bf16x8_t pa = pf_ld(&Ps[wave][lr][st * 32 + lg * 8]);
+      const bf16x8_t pb = pf_ld(&Pl[wave][lr][st * 32 + lg * 8]);
 #pragma unroll
-      for (int t = 0; t < 8; ++t)
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, pf_ld(&Vt[t * 16 + lr][st * 32 + lg * 8]), o[t], 0, 0, 0);
+      for (int t = 0; t < 8; ++t) {
+        const bf16x8_t vf = pf_ld(&Vt[t * 16 + lr][st * 32 + lg * 8]);
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vf, o[t], 0, 0, 0);
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pb, vf, o[t], 0, 0, 0);
+      }
     }
   }
 
