@@ -43,6 +43,9 @@ def _parse():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense bf16 comparator leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-breakdown", action="store_true", help="also time every kernel type of the step")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 256 MiB device copy 10 times (the known-size kernel that FETCH_SIZE / WRITE_SIZE "
+                         "counters are scaled against) and exit")
     return ap.parse_args()
 
 
@@ -331,6 +334,15 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.calibrate_copy:
+        n = 256 << 20
+        src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "torch device copy", "bytes_read": n, "bytes_written": n, "launches": 10}))
+        return
     from flashsvd_amd import _lib
     _lib.load()
     lr = run_lowrank(args)
