@@ -43,6 +43,9 @@ def _parse():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense bf16 comparator leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-breakdown", action="store_true", help="also time every kernel type of the step")
+    ap.add_argument("--engine", choices=["persistent", "graph", "both"], default="both",
+                    help="persistent: one resident kernel per token (fsvd_decode_step); graph: one HIP graph of the "
+                         "per-operator kernels per token; both: time both, the headline value is the persistent step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device copy 10 times (the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counters are scaled against) and exit")
@@ -161,19 +164,42 @@ def run_lowrank(args):
     torch.cuda.synchronize()
     t_prefill = time.perf_counter() - t0
     tok = out.logits[:, -1].float().argmax(-1, keepdim=True)
+    res = dict(prefill_s=t_prefill)
     dec = GraphedDecoder(model, cache, B)
     dec.set_state(tok, PROMPT_LEN)
-    dec.capture()
-    for _ in range(args.warmup):
-        dec.step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    for _ in range(args.steps):
-        dec.step()
-    torch.cuda.synchronize()
-    t_decode = time.perf_counter() - t1
-    res = dict(tok_s=B * args.steps / t_decode, ms_per_step=t_decode * 1000.0 / args.steps, prefill_s=t_prefill,
-               last_token=int(dec.tokens[0, 0]))
+    if args.engine in ("graph", "both"):
+        dec.capture()
+        for _ in range(args.warmup):
+            dec.step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            dec.step()
+        torch.cuda.synchronize()
+        t_decode = time.perf_counter() - t1
+        res["graph"] = dict(tok_s=B * args.steps / t_decode, ms_per_step=t_decode * 1000.0 / args.steps)
+    if args.engine in ("persistent", "both"):
+        from flashsvd_amd.step import PersistentDecoder
+        cache._seen_tokens = PROMPT_LEN
+        pdec = PersistentDecoder(model, cache)
+        pdec.set_state(tok, PROMPT_LEN)
+        pdec.step(args.warmup)
+        pdec.check()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        e0.record()
+        pdec.step(args.steps)
+        e1.record()
+        torch.cuda.synchronize()
+        t_decode = time.perf_counter() - t1
+        pdec.check()
+        res["persistent"] = dict(tok_s=B * args.steps / t_decode, ms_per_step=t_decode * 1000.0 / args.steps,
+                                 kernel_us_per_launch=e0.elapsed_time(e1) * 1000.0 / args.steps,
+                                 workgroups=pdec.nwg, last_token=int(pdec.tokens()[-1]))
+        del pdec
+    best = res.get("persistent") or res["graph"]
+    res["tok_s"], res["ms_per_step"] = best["tok_s"], best["ms_per_step"]
     legs = kernel_legs(model, cache, dec)
     name = "mlp_gate_up_u+swiglu"
     fn, nbytes = legs[name]
@@ -192,10 +218,19 @@ def run_lowrank(args):
         res["layer_sum"] = {"us": round(tot_u, 2), "bytes": tot_b, "GB/s": round(tot_b / tot_u / 1e3, 1)}
     # whole-step effective bandwidth: every factor byte + lm_head + KV read once per token
     n_ctx = PROMPT_LEN + args.warmup + args.steps // 2
-    per_layer = 8 * CFG["hidden_size"] * CFG["attn_rank"] * 2 + 3 * (CFG["hidden_size"] + 2 * CFG["intermediate_size"]) * CFG["mlp_rank"] * 2
+    per_layer = 8 * CFG["hidden_size"] * CFG["attn_rank"] * 2 + 3 * (CFG["hidden_size"] + CFG["intermediate_size"]) * CFG["mlp_rank"] * 2
     step_bytes = args.layers * (per_layer + 2 * n_ctx * CFG["num_heads"] * CFG["head_dim"] * 2) + CFG["vocab_size"] * CFG["hidden_size"] * 2
     res["step_bytes"] = step_bytes
     res["step_GBs"] = step_bytes / (res["ms_per_step"] * 1e-3) / 1e9
+    if "persistent" in res:
+        # the resident step kernel is the dominant (only) kernel of the token: its algorithmic bytes are the
+        # step's — every factor, the lm_head and the KV rows read once — over its event-timed launch duration
+        us_launch = res["persistent"]["kernel_us_per_launch"]
+        res["swiglu_roofline"] = res["roofline"]
+        res["roofline"] = {"kernel": "decode_step_kernel (whole token: 32 layers + lm_head + argmax)", "bound": "hbm",
+                           "achieved": step_bytes / us_launch / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": step_bytes / us_launch / 1e3 / HBM_PEAK_GBS, "traffic": _traffic("decode_step_kernel"),
+                           "bytes_per_launch": step_bytes, "us_per_launch": us_launch}
     del dec, cache, model
     torch.cuda.empty_cache()
     return res
@@ -351,12 +386,16 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": lr["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "32-layer Llama-2-7B-shaped low-rank decode (attn rank 1024, MLP rank 1536, vocab 32000), "
-                               "bs1, prompt 512, greedy, whole step in one HIP graph", "layers": args.layers,
+                               "bs1, prompt 512, greedy, " + ("one resident kernel launch per token" if "persistent" in lr
+                                                              else "whole step in one HIP graph"), "layers": args.layers,
                    "prompt_len": PROMPT_LEN, "batch": 1, "kv_cache": "dense"},
         "roofline": lr["roofline"],
         "step_hbm": {"bytes_per_token": lr["step_bytes"], "GB/s": lr["step_GBs"], "frac_of_peak": lr["step_GBs"] / HBM_PEAK_GBS},
         "prefill_s": lr["prefill_s"],
     }
+    for k in ("persistent", "graph", "swiglu_roofline"):
+        if k in lr:
+            line[k if k != "graph" else "per_operator_graph"] = lr[k]
     if "kernels" in lr:
         line["kernels"] = lr["kernels"]
         line["layer_sum"] = lr["layer_sum"]

@@ -15,6 +15,35 @@ _lib = None
 
 _i32p = ctypes.POINTER(ctypes.c_int32)
 
+
+class TagBuf(ctypes.Structure):
+    """fsvd_tagbuf: a tagged hand-off vector and which of its per-step uses a phase touches."""
+    _fields_ = [("ptr", c_void_p), ("uses_per_step", ctypes.c_int32), ("use", ctypes.c_int32)]
+
+
+class Phase(ctypes.Structure):
+    """fsvd_phase (include/flashsvd_hip.h), field for field."""
+    _fields_ = [("type", ctypes.c_int32), ("epilogue", ctypes.c_int32),
+                ("N", ctypes.c_int32), ("K", ctypes.c_int32), ("nmat", ctypes.c_int32), ("mode", ctypes.c_int32),
+                ("H", ctypes.c_int32), ("Hk", ctypes.c_int32), ("Dh", ctypes.c_int32), ("nsplit", ctypes.c_int32),
+                ("rope_len", ctypes.c_int32), ("S", ctypes.c_int32),
+                ("fparam", c_float),
+                ("W", c_void_p * 3), ("norm_w", c_void_p), ("cos", c_void_p), ("sin", c_void_p),
+                ("k_cache", c_void_p), ("v_cache", c_void_p), ("sc_s", c_int64), ("sc_h", c_int64),
+                ("plain_out", c_void_p),
+                ("inp", TagBuf), ("aux0", TagBuf), ("aux1", TagBuf), ("out0", TagBuf), ("out1", TagBuf), ("out2", TagBuf),
+                ("share_q", ctypes.c_int32), ("share_r", ctypes.c_int32), ("m_kp", ctypes.c_uint32), ("m_pps", ctypes.c_uint32)]
+
+
+class StepState(ctypes.Structure):
+    """fsvd_step_state."""
+    _fields_ = [("epoch", ctypes.c_int32), ("err", ctypes.c_int32), ("pos", ctypes.c_int32), ("step", ctypes.c_int32),
+                ("token", c_int64), ("err_wg", ctypes.c_int32), ("spin_limit", ctypes.c_int32)]
+
+
+PH_EMBED, PH_GEMV, PH_QKV, PH_ATTN, PH_MERGE, PH_ARGMAX = range(6)
+EP_STORE, EP_RESID, EP_SWIGLU, EP_LOGITS = range(4)
+
 # name -> (restype, argtypes); mirrors include/flashsvd_hip.h declaration by declaration
 SIGNATURES = {
     "fsvd_version": (c_int, []),
@@ -51,6 +80,10 @@ SIGNATURES = {
                                    + [c_void_p, c_int64] * 3 + [c_void_p, c_int64, c_int64] * 3 + [c_int] * 8
                                    + [c_void_p, c_size_t, c_void_p]),
     "fsvd_mlp_dual_split_workspace_bytes": (c_size_t, [c_int] * 6),
+    "fsvd_decode_step_workgroups": (c_int, []),
+    "fsvd_decode_step_prepare": (c_int, [c_void_p, c_int, c_int]),
+    "fsvd_decode_step": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
+    "fsvd_decode_step_trace": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "fsvd_mlp_dual_split": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                     c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -396,4 +396,41 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h, c
   return launch_prefill_attn(a, static_cast<hipStream_t>(stream));
 }
 
+int fsvd_decode_step_workgroups(void) { return decode_step_workgroups(); }
+
+int fsvd_decode_step_prepare(fsvd_phase* phases_host, int nphase, int workgroups) {
+  const char* fn = "fsvd_decode_step_prepare";
+  FSVD_REQUIRE_PTR(phases_host, fn);
+  if (nphase <= 0 || workgroups <= 0) { set_last_error("%s: bad arguments", fn); return kErrBadShape; }
+  return prepare_decode_step(phases_host, nphase, workgroups);
+}
+
+int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase, fsvd_step_state* state,
+                     int validate, void* stream) {
+  const char* fn = "fsvd_decode_step";
+  FSVD_REQUIRE_PTR(phases_dev, fn); FSVD_REQUIRE_PTR(state, fn);
+  if (nphase <= 0) { set_last_error("%s: empty phase list", fn); return kErrBadShape; }
+  if (validate) {
+    FSVD_REQUIRE_PTR(phases_host, fn);
+    const int nwg = decode_step_workgroups();
+    if (nwg <= 0) { set_last_error("%s: cannot query the device", fn); return kErrLaunch; }
+    const int rc = validate_decode_step(phases_host, nphase, nwg);
+    if (rc != kOk) return rc;
+  }
+  return launch_decode_step(phases_dev, nphase, state, nullptr, 1, static_cast<hipStream_t>(stream));
+}
+
+int fsvd_decode_step_trace(const fsvd_phase* phases_dev, int nphase, fsvd_step_state* state, uint64_t* trace,
+                           size_t trace_words, int wg_stride, void* stream) {
+  const char* fn = "fsvd_decode_step_trace";
+  FSVD_REQUIRE_PTR(phases_dev, fn); FSVD_REQUIRE_PTR(state, fn); FSVD_REQUIRE_PTR(trace, fn);
+  const int nwg = decode_step_workgroups();
+  if (nwg <= 0) { set_last_error("%s: cannot query the device", fn); return kErrLaunch; }
+  if (nphase <= 0 || wg_stride <= 0) { set_last_error("%s: bad arguments", fn); return kErrBadShape; }
+  const size_t need = (size_t)((nwg + wg_stride - 1) / wg_stride) * nphase * 4;
+  if (trace_words < need) { set_last_error("%s: trace buffer holds %zu words, %zu needed", fn, trace_words, need); return kErrWorkspace; }
+  return launch_decode_step(phases_dev, nphase, state, reinterpret_cast<unsigned long long*>(trace), wg_stride,
+                            static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -143,3 +143,15 @@ int launch_kv_append(const KvAppendArgs& a, hipStream_t st);
 size_t attn_decode_ws_floats(int B, int H, int nsplit, int Dh);
 
 }  // namespace fsvd
+
+// persistent decode step (decode_step.hip); the argument structs are part of the public header
+struct fsvd_phase;
+struct fsvd_step_state;
+namespace fsvd {
+int decode_step_workgroups();
+int prepare_decode_step(fsvd_phase* host_phases, int nph, int nwg);
+int validate_decode_step(const fsvd_phase* host_phases, int nph, int nwg);
+int launch_decode_step(const fsvd_phase* dev_phases, int nph, fsvd_step_state* state, unsigned long long* trace,
+                       int trace_stride, hipStream_t stream);
+}  // namespace fsvd
+

@@ -1,0 +1,261 @@
+"""Greedy batch-1 decoding with ONE persistent launch per token (C ABI: fsvd_decode_step).
+
+The per-token module walk of the reference (utils/evaluator.py:39-82 ``_manual_llama_decode_step``,
+scripts/demo_support/api.py:238-322) issues ~10 dependent kernels per layer; at batch 1 each of them
+is a few microseconds of weight streaming behind a launch gap of the same size.  Here the whole step
+is a list of phases handed to one kernel that keeps one workgroup per compute unit resident, passes
+activations between workgroups through tagged vectors and keeps the weight stream of the next phase
+in flight while it waits (flashsvd_amd/csrc/decode_step.hip).  Token id, position and the tag epoch
+live on the device, so N tokens are N launches without host synchronisation.
+
+Arithmetic and rounding points are those of the stand-alone kernels (hip_ops.linear,
+swiglu_linear, qkv_rope_append, attn_decode_densekv); only fp32 summation order differs.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+from ._lib import (EP_LOGITS, EP_RESID, EP_STORE, EP_SWIGLU, PH_ARGMAX, PH_ATTN, PH_EMBED, PH_GEMV, PH_MERGE, PH_QKV,
+                   Phase, TagBuf)
+from .runtime.cache import FlashSVDV15DenseKVCache
+
+
+class DecodeStepError(RuntimeError):
+    """The persistent step gave up waiting for a hand-off (state.err != 0)."""
+
+
+def _tb(t: torch.Tensor, uses: int, use: int) -> TagBuf:
+    return TagBuf(t.data_ptr(), int(uses), int(use))
+
+
+class PersistentDecoder:
+    """``PersistentDecoder(model, cache)`` then ``set_state(token, position)``, ``step(n)``, ``tokens()``.
+
+    Requirements (checked): batch 1, bf16, dense KV cache, head_dim 128, equal q/k/v ranks, every
+    matrix row length a multiple of 128, and a device whose compute-unit count is a multiple of the
+    number of heads.  Models outside these limits decode through ``graphs.GraphedDecoder``.
+    """
+
+    def __init__(self, model, cache, *, mode: int | None = None, max_new_tokens: int = 4096):
+        from .llama import mlp_rounding_mode
+        if not isinstance(cache, FlashSVDV15DenseKVCache):
+            raise TypeError("PersistentDecoder needs a FlashSVDV15DenseKVCache")
+        lib = _lib.load()
+        self.lib = lib
+        self.model, self.cache = model, cache
+        inner = model.model
+        cfg = model.config
+        dev = model.lm_head.weight.device
+        if model.lm_head.weight.dtype != torch.bfloat16:
+            raise ValueError("PersistentDecoder is bf16 only")
+        self.nwg = int(lib.fsvd_decode_step_workgroups())
+        if self.nwg <= 0:
+            raise RuntimeError("fsvd_decode_step_workgroups: cannot query the device")
+        H = int(cfg.num_attention_heads)
+        Hk = int(getattr(cfg, "num_key_value_heads", H))
+        Dh = int(getattr(cfg, "head_dim", None) or cfg.hidden_size // H)
+        d = int(cfg.hidden_size)
+        L = len(inner.layers)
+        V = int(model.lm_head.weight.shape[0])
+        if self.nwg % H != 0:
+            raise ValueError(f"{self.nwg} workgroups are not a multiple of {H} heads")
+        nsplit = self.nwg // H
+        S = int(cache.max_cache_len)
+        mode = mlp_rounding_mode() if mode is None else int(mode)
+        self.H, self.Hk, self.Dh, self.d, self.L, self.V, self.S, self.nsplit = H, Hk, Dh, d, L, V, S, nsplit
+
+        def tagged(n):  # uint32 words: tag << 16 | bf16
+            return torch.zeros(n, dtype=torch.int32, device=dev)
+
+        def tagged64(n):
+            return torch.zeros(n, dtype=torch.int64, device=dev)
+
+        a0 = inner.layers[0].self_attn
+        m0 = inner.layers[0].mlp
+        Rq, Rk, Rv = a0._qkv_rank_tuple()
+        Ro = int(a0.o_v_proj.out_features)
+        Rm = int(m0.gate_v_proj.out_features)
+        D = int(m0.gate_u_proj.out_features)
+        if not (Rq == Rk == Rv):
+            raise ValueError("PersistentDecoder needs equal q/k/v ranks (pad them to a common multiple of 128)")
+        self.XA, self.XB = tagged(d), tagged(d)
+        self.P, self.Q, self.KN, self.VN = tagged(3 * Rq), tagged(H * Dh), tagged(Hk * Dh), tagged(Hk * Dh)
+        self.PART, self.A = tagged64(H * nsplit * (Dh + 2)), tagged(H * Dh)
+        self.PO, self.PM, self.HB, self.SB = tagged(Ro), tagged(2 * Rm), tagged(D), tagged(Rm)
+        self.CAND = tagged64(self.nwg)
+        self.logits = torch.zeros(V, dtype=torch.bfloat16, device=dev)
+        self.token_log = torch.zeros(int(max_new_tokens), dtype=torch.int64, device=dev)
+        self.state = torch.zeros(8, dtype=torch.int32, device=dev)   # fsvd_step_state
+        self.rope = cache.get_rope_tables(seqlen=S, head_dim=Dh, device=dev, dtype=torch.bfloat16)
+        cos, sin = self.rope
+        self._keep = []   # tensors whose storage the phase list points into
+
+        ph: list[Phase] = []
+
+        def gemv(W, N, K, inp, out, *, nmat=1, norm=None, eps=0.0, epi=EP_STORE, aux=None, plain=None):
+            p = Phase()
+            p.type, p.epilogue, p.N, p.K, p.nmat, p.mode = PH_GEMV, epi, N, K, nmat, mode
+            for i, w in enumerate(W):
+                if tuple(w.shape) != (N, K) or not w.is_contiguous():
+                    raise ValueError(f"weight {tuple(w.shape)} is not a contiguous [{N},{K}] matrix")
+                p.W[i] = w.data_ptr()
+                self._keep.append(w)
+            if norm is not None:
+                p.norm_w, p.fparam = norm.data_ptr(), float(eps)
+                self._keep.append(norm)
+            p.inp, p.out0 = inp, out
+            if aux is not None:
+                p.aux0 = aux
+            if plain is not None:
+                p.plain_out = plain.data_ptr()
+            ph.append(p)
+
+        e = Phase()
+        e.type, e.N = PH_EMBED, d
+        emb = inner.embed_tokens.weight
+        if tuple(emb.shape)[1] != d or not emb.is_contiguous():
+            raise ValueError("embedding table must be a contiguous [V, hidden] matrix")
+        e.W[0] = emb.data_ptr()
+        e.out0 = _tb(self.XA, L + 1, 0)
+        ph.append(e)
+        for l, layer in enumerate(inner.layers):
+            at, mlp = layer.self_attn, layer.mlp
+            at._ensure_runtime_state()
+            mlp._ensure_runtime_state()
+            if at._qkv_rank_tuple() != (Rq, Rk, Rv) or int(at.o_v_proj.out_features) != Ro or \
+                    int(mlp.gate_v_proj.out_features) != Rm or int(mlp.up_v_proj.out_features) != Rm:
+                raise ValueError("PersistentDecoder needs the same ranks in every layer")
+            cache._ensure_layer_spec(l, h=Hk, dh=Dh)
+            kc, vc = cache.key_cache[l][0], cache.value_cache[l][0]      # [S, Hk, Dh]
+            n1, n2 = layer.input_layernorm, layer.post_attention_layernorm
+            xin, xmid, xout = _tb(self.XA, L + 1, l), _tb(self.XB, L, l), _tb(self.XA, L + 1, l + 1)
+            gemv([at._packed_qkv_v], 3 * Rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
+            q = Phase()
+            q.type, q.K, q.H, q.Hk, q.Dh, q.S = PH_QKV, Rq, H, Hk, Dh, S
+            for i, w in enumerate((at.q_u_proj.weight, at.k_u_proj.weight, at.v_u_proj.weight)):
+                if not w.is_contiguous() or w.shape[1] != Rq:
+                    raise ValueError("u_proj weights must be contiguous [heads*Dh, R]")
+                q.W[i] = w.data_ptr()
+                self._keep.append(w)
+            q.cos, q.sin, q.rope_len = cos.data_ptr(), sin.data_ptr(), int(cos.shape[0])
+            q.k_cache, q.v_cache, q.sc_s, q.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
+            q.inp, q.out0, q.out1, q.out2 = _tb(self.P, L, l), _tb(self.Q, L, l), _tb(self.KN, L, l), _tb(self.VN, L, l)
+            ph.append(q)
+            a = Phase()
+            a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
+            a.fparam = 1.0 / math.sqrt(Dh)
+            a.k_cache, a.v_cache, a.sc_s, a.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
+            a.inp, a.aux0, a.aux1, a.out0 = _tb(self.Q, L, l), _tb(self.KN, L, l), _tb(self.VN, L, l), _tb(self.PART, L, l)
+            ph.append(a)
+            m = Phase()
+            m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
+            m.inp, m.out0 = _tb(self.PART, L, l), _tb(self.A, L, l)
+            ph.append(m)
+            gemv([at.o_v_proj.weight], Ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
+            gemv([at.o_u_proj.weight], d, Ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
+            gemv([mlp._packed_gu_v], 2 * Rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
+            gemv([mlp.gate_u_proj.weight, mlp.up_u_proj.weight], D, Rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2,
+                 epi=EP_SWIGLU)
+            gemv([mlp.down_v_proj.weight], Rm, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
+            gemv([mlp.down_u_proj.weight], d, Rm, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
+            cache._layer_initialized[l] = True
+        fn = inner.norm
+        gemv([model.lm_head.weight], V, d, _tb(self.XA, L + 1, L), _tb(self.CAND, 1, 0), norm=fn.weight,
+             eps=fn.variance_epsilon, epi=EP_LOGITS, plain=self.logits)
+        g = Phase()
+        g.type = PH_ARGMAX
+        g.inp = _tb(self.CAND, 1, 0)
+        g.plain_out = self.token_log.data_ptr()
+        ph.append(g)
+
+        self.nph = len(ph)
+        self.host_phases = (Phase * self.nph)(*ph)
+        _lib.check("fsvd_decode_step_prepare", lib.fsvd_decode_step_prepare(ctypes.addressof(self.host_phases), self.nph, self.nwg))
+        raw = bytes(self.host_phases)
+        self.dev_phases = torch.frombuffer(bytearray(raw), dtype=torch.uint8).to(dev)
+        self._validated = False
+        self._host_pos = 0
+        self._host_steps = 0
+
+    # ------------------------------------------------------------------ state
+    def set_state(self, token, position: int) -> None:
+        """Next input token and its position (= number of keys already in the cache)."""
+        if position < 0 or position >= self.S:
+            raise IndexError(f"decode position {position} outside the cache (max {self.S})")
+        tok = int(token.reshape(-1)[0].item()) if torch.is_tensor(token) else int(token)
+        st = self.state
+        st[2] = int(position)
+        st[3] = 0
+        st.view(torch.int64)[2] = tok
+        self._host_pos = int(position)
+        self._host_steps = 0
+
+    def step(self, n: int = 1) -> None:
+        """Decode ``n`` tokens greedily (asynchronous; read them with ``tokens()``)."""
+        if self._host_pos + n > self.S:
+            raise IndexError(f"decode position {self._host_pos + n - 1} outside the cache (max {self.S})")
+        if self._host_steps + n > self.token_log.numel():
+            raise IndexError(f"token log holds {self.token_log.numel()} tokens")
+        stream = torch.cuda.current_stream().cuda_stream
+        for _ in range(int(n)):
+            rc = self.lib.fsvd_decode_step(self.dev_phases.data_ptr(), ctypes.addressof(self.host_phases), self.nph,
+                                           self.state.data_ptr(), 0 if self._validated else 1, stream)
+            _lib.check("fsvd_decode_step", rc)
+            self._validated = True
+        self._host_pos += int(n)
+        self._host_steps += int(n)
+        self.cache._seen_tokens += int(n)
+
+    PHASE_NAMES = ("embed", "attn_rank_proj", "qkv_rope", "attn", "attn_merge", "o_v", "o_u", "mlp_rank_proj", "swiglu",
+                   "down_v", "down_u")
+
+    def trace_step(self, wg_stride: int = 32) -> torch.Tensor:
+        """Run ONE step with per-phase time stamps; returns int64 [workgroups/stride, phases, 4] in
+        microseconds relative to the earliest stamp (0 entered, 1 input staged, 2 weights consumed,
+        3 epilogue done).  The step counts like any other (token, position and cache advance)."""
+        if not self._validated:
+            raise RuntimeError("run step() once before tracing")
+        if self._host_pos + 1 > self.S or self._host_steps + 1 > self.token_log.numel():
+            raise IndexError("no room for another step")
+        nt = (self.nwg + wg_stride - 1) // wg_stride
+        buf = torch.zeros(nt * self.nph * 4, dtype=torch.int64, device=self.state.device)
+        rc = self.lib.fsvd_decode_step_trace(self.dev_phases.data_ptr(), self.nph, self.state.data_ptr(), buf.data_ptr(),
+                                             buf.numel(), int(wg_stride), torch.cuda.current_stream().cuda_stream)
+        _lib.check("fsvd_decode_step_trace", rc)
+        self._host_pos += 1
+        self._host_steps += 1
+        self.cache._seen_tokens += 1
+        self.check()
+        t = buf.view(nt, self.nph, 4).cpu()
+        t0 = t[t > 0].min()
+        return (t - t0).clamp_min(0).float() / 100.0
+
+    def check(self) -> None:
+        """Synchronise and raise if a step timed out waiting for a hand-off."""
+        st = self.state.cpu()
+        if int(st[1]) != 0:
+            raise DecodeStepError(f"decode step gave up in phase {int(st[1]) - 1} (workgroup {int(st[6])}); "
+                                  "clear with reset_error() after finding the cause")
+
+    def reset_error(self) -> None:
+        """Clear a time-out.  The failed step left half-written vectors that carry its tags, so the
+        epoch moves on and every tag of the next step differs from them."""
+        self.state[1] = 0
+        self.state[0] += 1
+
+    def set_spin_limit(self, polls: int) -> None:
+        """Polls before a workgroup gives up waiting (0 = default, about a second)."""
+        self.state[7] = int(polls)
+
+    def tokens(self) -> torch.Tensor:
+        """Tokens generated since ``set_state`` (synchronises)."""
+        self.check()
+        return self.token_log[: self._host_steps].clone()
+
+    def hidden(self) -> torch.Tensor:
+        """Final-layer hidden state of the last step, bf16 [hidden]."""
+        return ((self.XA & 0xFFFF) << 16).view(torch.float32).to(torch.bfloat16)

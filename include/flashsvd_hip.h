@@ -193,6 +193,91 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
                       void* out, int64_t so_b, int64_t so_m, int64_t so_h,
                       int B, int M, int H, int Hk, int Dh, int S, int causal, float scale, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Persistent decode step (batch 1): ONE launch walks a caller-built list of phases — embedding row,
+ * low-rank projections with fused RMSNorm / residual / SwiGLU, q/k/v head expansion with RoPE and
+ * cache append, split-KV attention and its merge, lm_head and greedy argmax — on one workgroup per
+ * compute unit.  Workgroups hand activations to each other through "tagged" vectors: every 32-bit
+ * word carries a bf16 value and a 16-bit tag (fp32 partials: 64-bit words with a 32-bit tag) that
+ * changes with every use of the buffer, so a consumer polls the data itself and no grid barrier, L2
+ * write-back or counter is needed; while a workgroup waits, the first weights of its next phase are
+ * already in flight.  It replaces, for greedy batch-1 decoding, the per-token module walk of
+ * utils/evaluator.py:39-82 (_manual_llama_decode_step) and scripts/demo_support/api.py:238-322 together
+ * with the per-layer operators listed above; arithmetic and rounding points are those of the
+ * stand-alone entry points (fsvd_linear, fsvd_swiglu_linear mode 0/1, fsvd_qkv_rope_append,
+ * fsvd_attn_decode_densekv).
+ *
+ * Rules for the phase list (checked by fsvd_decode_step): every matrix has K % 128 == 0 and at least
+ * one row per workgroup; a tagged buffer is written by one phase per step position and must not be
+ * written again until a later GEMV phase has consumed a vector that every workgroup helped to write
+ * (use separate buffers per role and two alternating hidden-state buffers).  All tagged buffers and
+ * the state block start zero-filled.  Polls are bounded: on a time-out the step sets state->err and
+ * every workgroup leaves; later launches return immediately until the caller clears err.
+ * ------------------------------------------------------------------------------------------- */
+#define FSVD_PH_EMBED 0   /* out0[n] = W[0][token, n]                                   (N = hidden)        */
+#define FSVD_PH_GEMV 1    /* out0 = epilogue(W[m] . norm(in)), m < nmat                                      */
+#define FSVD_PH_QKV 2     /* q/k/v head expansion from in = [Pq|Pk|Pv], RoPE, cache append; out0/1/2 = q/k/v */
+#define FSVD_PH_ATTN 3    /* split-KV attention of in = q over the cache + (aux0, aux1) = new k, v           */
+#define FSVD_PH_MERGE 4   /* out0 = merged attention output from in = partials                               */
+#define FSVD_PH_ARGMAX 5  /* token = argmax of the per-workgroup candidates in `in`; advances the state      */
+
+#define FSVD_EP_STORE 0   /* out0[n] = bf16(dot)                                                              */
+#define FSVD_EP_RESID 1   /* out0[n] = bf16(aux0[n] + bf16(dot))                                              */
+#define FSVD_EP_SWIGLU 2  /* nmat = 2: out0[n] = silu(W[0][n].in[0:K]) * (W[1][n].in[K:2K]), rounding `mode`  */
+#define FSVD_EP_LOGITS 3  /* plain_out[n] = bf16(dot) and out0[wg] = (best value, best index) of the workgroup */
+
+typedef struct fsvd_tagbuf {
+  void* ptr;              /* uint32 [len] (bf16 payload) or uint64 [len] (fp32 / candidate payload)           */
+  int32_t uses_per_step;  /* how many phases of one step write this buffer                                    */
+  int32_t use;            /* which of those uses this phase writes (out*) or reads (in, aux*)                 */
+} fsvd_tagbuf;
+
+typedef struct fsvd_phase {
+  int32_t type, epilogue;
+  int32_t N, K, nmat, mode;     /* rows per matrix, row length, matrices, SwiGLU rounding mode; the staged     */
+                                /* input has nmat * K elements (QKV: 3 * K)                                    */
+  int32_t H, Hk, Dh, nsplit, rope_len, S;
+  float fparam;                 /* GEMV with norm_w: RMSNorm eps; ATTN: softmax scale                          */
+  const void* W[3];             /* nn.Linear-layout weights [N, K] (QKV: q_u, k_u, v_u; EMBED: table [V, N]) */
+  const void* norm_w;           /* RMSNorm weight over `in` or NULL                                            */
+  const void* cos; const void* sin;   /* [rope_len, Dh/2]                                                      */
+  void* k_cache; void* v_cache; /* batch row of the dense cache, [S, Hk, Dh] with strides sc_s, sc_h          */
+  int64_t sc_s, sc_h;
+  void* plain_out;              /* EP_LOGITS: bf16 logits [N]; ARGMAX: int64 token log indexed by state->step */
+  fsvd_tagbuf in, aux0, aux1, out0, out1, out2;
+  /* derived by fsvd_decode_step_prepare (do not fill by hand): work items (rows, or 16-row q/k/v groups)
+   * are dealt as share_q per workgroup plus one more for the first share_r workgroups; m_kp, m_pps are
+   * 32-bit reciprocals of K/8 and of the pieces per q/k/v segment */
+  int32_t share_q, share_r;
+  uint32_t m_kp, m_pps;
+} fsvd_phase;
+
+typedef struct fsvd_step_state {
+  int32_t epoch;      /* advanced by every completed step; seeds the tags                                     */
+  int32_t err;        /* 0 ok; else 1 + index of the phase whose input never arrived                          */
+  int32_t pos;        /* position of the token being decoded = number of keys already in the cache            */
+  int32_t step;       /* tokens generated so far (index into the token log)                                   */
+  int64_t token;      /* input token of the next step (written by ARGMAX)                                     */
+  int32_t err_wg;     /* workgroup that raised err                                                            */
+  int32_t spin_limit; /* polls before a workgroup gives up; 0 = default (about a second)                       */
+} fsvd_step_state;
+
+/* Workgroups the step kernel runs with on the current device (one per compute unit). */
+int fsvd_decode_step_workgroups(void);
+/* Fill the derived fields of a host-side phase list for `workgroups` workgroups (call before uploading it). */
+int fsvd_decode_step_prepare(fsvd_phase* phases_host, int nphase, int workgroups);
+/* phases_dev: the list in device memory; phases_host: the same list in host memory (validated on every
+ * call unless validate == 0); state: device.  Launch is asynchronous on `stream`. */
+int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase,
+                     fsvd_step_state* state, int validate, void* stream);
+/* The same step with per-phase time stamps (the hipEvent-per-module decode profiler of the reference,
+ * utils/evaluator.py:553-689, cannot see inside one launch): workgroups 0, wg_stride, 2*wg_stride, ...
+ * write trace[(wg / wg_stride) * nphase * 4 + phase * 4 + k], k = 0 phase entered, 1 input staged,
+ * 2 weights consumed, 3 epilogue done, in ticks of the 100 MHz device wall clock.  The list must have
+ * passed fsvd_decode_step's validation before. */
+int fsvd_decode_step_trace(const fsvd_phase* phases_dev, int nphase, fsvd_step_state* state, uint64_t* trace,
+                           size_t trace_words, int wg_stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,174 @@
+"""Persistent decode step (fsvd_decode_step through flashsvd_amd.step.PersistentDecoder) against the CPU
+oracle and against the per-kernel decode path on identical seeded weights.
+
+Tolerances as in test_gpu_model.py: hidden states within max-rel 1e-2 per teacher-forced step
+(abs bound two bf16 ulps at max|ref| once max|ref| >= 2), free-running states 3e-2, greedy tokens
+identical on the small model and tie-aware at 7B width.
+"""
+import pytest
+import torch
+
+from oracle import flashsvd_oracle as O
+from tests.util import assert_close_bf16, bounds, model_from_oracle
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+def _prefill(model, prompt, extra):
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    B, Lp = prompt.shape
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=Lp + extra, device="cuda", dtype=BF16)
+    out = model(prompt.cuda(), past_key_values=cache, cache_position=torch.arange(Lp))
+    tok = out.logits[:, -1].float().argmax(-1, keepdim=True)
+    return cache, tok
+
+
+def _small():
+    # GQA (8 query heads over 4 kv heads), 3 layers, every row length a multiple of 128
+    mw = O.make_model(d=1024, n_heads=8, n_kv_heads=4, head_dim=128, ffn=2048, attn_rank=256, mlp_rank=384,
+                      n_layers=3, vocab=2048, dtype=BF16, seed=3)
+    prompt = torch.randint(0, 2048, (1, 37), generator=torch.Generator().manual_seed(5))
+    return mw, prompt
+
+
+def _tie_aware(g, o, ref_logits_row, what):
+    """Tokens must agree unless the oracle itself holds the two candidates within bf16 resolution."""
+    if g == o:
+        return True
+    rl = ref_logits_row.float()
+    gap = float(rl[o] - rl[g])
+    assert gap <= 1e-2 * float(rl.abs().max()), f"{what}: token {g} vs oracle {o}, oracle logit gap {gap}"
+    return False
+
+
+def test_small_model_teacher_forced_against_oracle():
+    from flashsvd_amd.step import PersistentDecoder
+    mw, prompt = _small()
+    n_new = 12
+    model = model_from_oracle(mw)
+    ref_tok, ref_hid, _, ref_logits = O.greedy_decode(mw, prompt, n_new, "dense", return_logits=True)
+    cache, tok0 = _prefill(model, prompt, n_new + 4)
+    assert int(tok0) == int(ref_tok[0, 0])
+    dec = PersistentDecoder(model, cache)
+    Lp = prompt.shape[1]
+    n_equal = 0
+    for s in range(1, n_new):
+        dec.set_state(ref_tok[:, s - 1], Lp + s - 1)
+        dec.step(1)
+        g = int(dec.tokens()[0])
+        # three layers run back to back inside one step: the multi-layer (free-running) bound applies
+        assert_close_bf16(dec.hidden()[None].cpu(), ref_hid[:, s], f"hidden state at step {s}",
+                          abs_tol=3 * bounds(ref_hid[:, s])["abs_tol"], rel_tol=3e-2)
+        rl = ref_logits[:, s].float()
+        assert_close_bf16(dec.logits[None].cpu(), rl, f"logits at step {s}", abs_tol=3 * bounds(rl)["abs_tol"], rel_tol=3e-2)
+        n_equal += _tie_aware(g, int(ref_tok[0, s]), ref_logits[0, s], f"step {s}")
+    assert n_equal >= n_new - 3
+
+
+def test_small_model_free_running_matches_kernel_path():
+    """16 launches queued without host synchronisation: same greedy tokens and cache rows as the
+    per-kernel decode path (both GPU paths, identical rounding points)."""
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.step import PersistentDecoder
+    mw, prompt = _small()
+    n_new = 17
+    model = model_from_oracle(mw)
+    Lp = prompt.shape[1]
+    cache_k, tok0 = _prefill(model, prompt, n_new + 4)
+    dec_k = GraphedDecoder(model, cache_k, 1)
+    dec_k.set_state(tok0, Lp)
+    toks_k = [tok0.clone()]
+    for _ in range(n_new - 1):
+        toks_k.append(dec_k.eager_step().clone())
+    toks_k = torch.cat(toks_k, 1).cpu()
+    cache_p, tok0p = _prefill(model, prompt, n_new + 4)
+    dec = PersistentDecoder(model, cache_p)
+    dec.set_state(tok0p, Lp)
+    dec.step(n_new - 1)
+    toks_p = torch.cat([tok0p.cpu(), dec.tokens().cpu()[None, :]], 1)
+    assert torch.equal(toks_p, toks_k), f"step kernel {toks_p.tolist()} vs per-kernel path {toks_k.tolist()}"
+    assert cache_p.get_seq_length() == cache_k.get_seq_length()
+    for li in range(3):
+        for got, ref, nm in ((cache_p.key_cache[li], cache_k.key_cache[li], "K"), (cache_p.value_cache[li], cache_k.value_cache[li], "V")):
+            assert_close_bf16(got[:, Lp:Lp + n_new - 1], ref[:, Lp:Lp + n_new - 1], f"{nm} rows layer {li}", abs_tol=float("inf"), rel_tol=3e-2)
+    assert_close_bf16(dec.logits[None].cpu(), dec_k.logits[:, -1].float().cpu(), "logits of the last step", rel_tol=3e-2,
+                      abs_tol=3 * bounds(dec_k.logits.float())["abs_tol"])
+
+
+def test_7b_width_two_layers_teacher_forced_tie_aware():
+    from flashsvd_amd.step import PersistentDecoder
+    mw = O.make_model(d=4096, n_heads=32, n_kv_heads=32, head_dim=128, ffn=11008, attn_rank=1024, mlp_rank=1536,
+                      n_layers=2, vocab=32000, dtype=BF16, seed=0)
+    prompt = torch.randint(0, 32000, (1, 48), generator=torch.Generator().manual_seed(1))
+    n_new = 12
+    model = model_from_oracle(mw)
+    ref_tok, ref_hid, _, ref_logits = O.greedy_decode(mw, prompt, n_new, "dense", return_logits=True)
+    cache, _ = _prefill(model, prompt, n_new + 4)
+    dec = PersistentDecoder(model, cache)
+    n_equal = 0
+    for s in range(1, n_new):
+        dec.set_state(ref_tok[:, s - 1], prompt.shape[1] + s - 1)      # teacher forcing: the oracle's token
+        dec.step(1)
+        g = int(dec.tokens()[0])
+        b = bounds(ref_hid[:, s])
+        assert_close_bf16(dec.hidden()[None].cpu(), ref_hid[:, s], f"hidden state at step {s}", abs_tol=3 * b["abs_tol"], rel_tol=3e-2)
+        n_equal += _tie_aware(g, int(ref_tok[0, s]), ref_logits[0, s], f"step {s}")
+    assert n_equal >= n_new - 3
+
+
+def test_timeout_path_leaves_cleanly_and_recovers():
+    """A spin limit of one poll makes workgroups give up instead of waiting: the step must end, report the
+    error, and decode correctly again after reset_error()."""
+    from flashsvd_amd.step import DecodeStepError, PersistentDecoder
+    mw, prompt = _small()
+    model = model_from_oracle(mw)
+    ref_tok, _, _ = O.greedy_decode(mw, prompt, 5, "dense", return_hidden=True)
+    cache, tok0 = _prefill(model, prompt, 12)
+    dec = PersistentDecoder(model, cache)
+    dec.set_state(tok0, prompt.shape[1])
+    dec.set_spin_limit(1)
+    dec.step(1)
+    torch.cuda.synchronize()
+    gave_up = int(dec.state.cpu()[1]) != 0
+    if gave_up:
+        with pytest.raises(DecodeStepError):
+            dec.check()
+        dec.step(1)                       # a launch with err set returns immediately
+        torch.cuda.synchronize()
+        dec.reset_error()
+    dec.set_spin_limit(0)
+    cache._seen_tokens = prompt.shape[1]
+    dec.set_state(tok0, prompt.shape[1])
+    dec.step(4)
+    toks = torch.cat([tok0.cpu(), dec.tokens().cpu()[None, :]], 1)
+    assert torch.equal(toks, ref_tok), f"after recovery: {toks.tolist()} vs {ref_tok.tolist()}"
+
+
+def test_phase_list_validation():
+    """The host check rejects lists the kernel cannot run (no launch happens)."""
+    import ctypes
+    from flashsvd_amd import _lib
+    from flashsvd_amd.step import PersistentDecoder
+    mw, prompt = _small()
+    model = model_from_oracle(mw)
+    cache, tok0 = _prefill(model, prompt, 8)
+    dec = PersistentDecoder(model, cache)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    saved = dec.host_phases[1].K
+    dec.host_phases[1].K = saved + 8          # row length not a multiple of 128
+    rc = lib.fsvd_decode_step(dec.dev_phases.data_ptr(), ctypes.addressof(dec.host_phases), dec.nph, dec.state.data_ptr(), 1, stream)
+    assert rc == -1 and b"fsvd_decode_step_prepare" in lib.fsvd_last_error()   # derived fields are stale
+    assert lib.fsvd_decode_step_prepare(ctypes.addressof(dec.host_phases), dec.nph, dec.nwg) == 0
+    rc = lib.fsvd_decode_step(dec.dev_phases.data_ptr(), ctypes.addressof(dec.host_phases), dec.nph, dec.state.data_ptr(), 1, stream)
+    assert rc == -1 and b"multiple of 128" in lib.fsvd_last_error()
+    dec.host_phases[1].K = saved
+    assert lib.fsvd_decode_step_prepare(ctypes.addressof(dec.host_phases), dec.nph, dec.nwg) == 0
+    saved_use = dec.host_phases[2].inp.use
+    dec.host_phases[2].inp.use = saved_use + 1   # consumer expects a tag its producer never writes
+    rc = lib.fsvd_decode_step(dec.dev_phases.data_ptr(), ctypes.addressof(dec.host_phases), dec.nph, dec.state.data_ptr(), 1, stream)
+    assert rc == -1 and b"tag schedule" in lib.fsvd_last_error()
+    dec.host_phases[2].inp.use = saved_use
+    rc = lib.fsvd_decode_step(None, ctypes.addressof(dec.host_phases), dec.nph, dec.state.data_ptr(), 1, stream)
+    assert rc == -4
