@@ -32,7 +32,7 @@ class Phase(ctypes.Structure):
                 ("k_cache", c_void_p), ("v_cache", c_void_p), ("sc_s", c_int64), ("sc_h", c_int64),
                 ("plain_out", c_void_p),
                 ("inp", TagBuf), ("aux0", TagBuf), ("aux1", TagBuf), ("out0", TagBuf), ("out1", TagBuf), ("out2", TagBuf),
-                ("share_q", ctypes.c_int32), ("share_r", ctypes.c_int32), ("m_kp", ctypes.c_uint32), ("m_pps", ctypes.c_uint32)]
+                ("share_q", ctypes.c_int32), ("share_r", ctypes.c_int32), ("m_kp", ctypes.c_uint32), ("dk", ctypes.c_int32)]
 
 
 class StepState(ctypes.Structure):
@@ -41,7 +41,7 @@ class StepState(ctypes.Structure):
                 ("token", c_int64), ("err_wg", ctypes.c_int32), ("spin_limit", ctypes.c_int32)]
 
 
-PH_EMBED, PH_GEMV, PH_QKV, PH_ATTN, PH_MERGE, PH_ARGMAX = range(6)
+PH_EMBED, PH_GEMV, _PH_RESERVED, PH_ATTN, PH_MERGE, PH_ARGMAX = range(6)
 EP_STORE, EP_RESID, EP_SWIGLU, EP_LOGITS = range(4)
 
 # name -> (restype, argtypes); mirrors include/flashsvd_hip.h declaration by declaration

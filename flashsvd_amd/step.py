@@ -19,8 +19,7 @@ import math
 import torch
 
 from . import _lib
-from ._lib import (EP_LOGITS, EP_RESID, EP_STORE, EP_SWIGLU, PH_ARGMAX, PH_ATTN, PH_EMBED, PH_GEMV, PH_MERGE, PH_QKV,
-                   Phase, TagBuf)
+from ._lib import EP_LOGITS, EP_RESID, EP_STORE, EP_SWIGLU, PH_ARGMAX, PH_ATTN, PH_EMBED, PH_GEMV, PH_MERGE, Phase, TagBuf
 from .runtime.cache import FlashSVDV15DenseKVCache
 
 
@@ -41,7 +40,7 @@ class PersistentDecoder:
     """
 
     def __init__(self, model, cache, *, mode: int | None = None, max_new_tokens: int = 4096):
-        from .llama import mlp_rounding_mode
+        from .llama import _packed_rows, mlp_rounding_mode
         if not isinstance(cache, FlashSVDV15DenseKVCache):
             raise TypeError("PersistentDecoder needs a FlashSVDV15DenseKVCache")
         lib = _lib.load()
@@ -83,7 +82,7 @@ class PersistentDecoder:
         if not (Rq == Rk == Rv):
             raise ValueError("PersistentDecoder needs equal q/k/v ranks (pad them to a common multiple of 128)")
         self.XA, self.XB = tagged(d), tagged(d)
-        self.P, self.Q, self.KN, self.VN = tagged(3 * Rq), tagged(H * Dh), tagged(Hk * Dh), tagged(Hk * Dh)
+        self.P, self.QKV = tagged(3 * Rq), tagged((H + 2 * Hk) * Dh)
         self.PART, self.A = tagged64(H * nsplit * (Dh + 2)), tagged(H * Dh)
         self.PO, self.PM, self.HB, self.SB = tagged(Ro), tagged(2 * Rm), tagged(D), tagged(Rm)
         self.CAND = tagged64(self.nwg)
@@ -96,9 +95,11 @@ class PersistentDecoder:
 
         ph: list[Phase] = []
 
-        def gemv(W, N, K, inp, out, *, nmat=1, norm=None, eps=0.0, epi=EP_STORE, aux=None, plain=None):
+        def gemv(W, N, K, inp, out, *, nmat=1, norm=None, eps=0.0, epi=EP_STORE, aux=None, plain=None, groups=None):
             p = Phase()
             p.type, p.epilogue, p.N, p.K, p.nmat, p.mode = PH_GEMV, epi, N, K, nmat, mode
+            if groups is not None:          # rows are q | k | v heads, each group reads its own K-long input
+                p.H, p.Hk, p.Dh = groups
             for i, w in enumerate(W):
                 if tuple(w.shape) != (N, K) or not w.is_contiguous():
                     raise ValueError(f"weight {tuple(w.shape)} is not a contiguous [{N},{K}] matrix")
@@ -134,22 +135,17 @@ class PersistentDecoder:
             n1, n2 = layer.input_layernorm, layer.post_attention_layernorm
             xin, xmid, xout = _tb(self.XA, L + 1, l), _tb(self.XB, L, l), _tb(self.XA, L + 1, l + 1)
             gemv([at._packed_qkv_v], 3 * Rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
-            q = Phase()
-            q.type, q.K, q.H, q.Hk, q.Dh, q.S = PH_QKV, Rq, H, Hk, Dh, S
-            for i, w in enumerate((at.q_u_proj.weight, at.k_u_proj.weight, at.v_u_proj.weight)):
-                if not w.is_contiguous() or w.shape[1] != Rq:
-                    raise ValueError("u_proj weights must be contiguous [heads*Dh, R]")
-                q.W[i] = w.data_ptr()
-                self._keep.append(w)
-            q.cos, q.sin, q.rope_len = cos.data_ptr(), sin.data_ptr(), int(cos.shape[0])
-            q.k_cache, q.v_cache, q.sc_s, q.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
-            q.inp, q.out0, q.out1, q.out2 = _tb(self.P, L, l), _tb(self.Q, L, l), _tb(self.KN, L, l), _tb(self.VN, L, l)
-            ph.append(q)
+            # q, k, v head expansion as one GEMV over the row-packed [q_u; k_u; v_u] (the three module
+            # weights become views of one buffer); RoPE and the cache append happen in the attention phase
+            qkv_u = _packed_rows([at.q_u_proj, at.k_u_proj, at.v_u_proj])
+            self._keep.append(qkv_u)
+            gemv([qkv_u], (H + 2 * Hk) * Dh, Rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
             a = Phase()
             a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
             a.fparam = 1.0 / math.sqrt(Dh)
+            a.cos, a.sin, a.rope_len = cos.data_ptr(), sin.data_ptr(), int(cos.shape[0])
             a.k_cache, a.v_cache, a.sc_s, a.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
-            a.inp, a.aux0, a.aux1, a.out0 = _tb(self.Q, L, l), _tb(self.KN, L, l), _tb(self.VN, L, l), _tb(self.PART, L, l)
+            a.inp, a.out0 = _tb(self.QKV, L, l), _tb(self.PART, L, l)
             ph.append(a)
             m = Phase()
             m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
@@ -210,7 +206,7 @@ class PersistentDecoder:
         self._host_steps += int(n)
         self.cache._seen_tokens += int(n)
 
-    PHASE_NAMES = ("embed", "attn_rank_proj", "qkv_rope", "attn", "attn_merge", "o_v", "o_u", "mlp_rank_proj", "swiglu",
+    PHASE_NAMES = ("embed", "attn_rank_proj", "qkv_u", "attn", "attn_merge", "o_v", "o_u", "mlp_rank_proj", "swiglu",
                    "down_v", "down_u")
 
     def trace_step(self, wg_stride: int = 32) -> torch.Tensor:

@@ -216,8 +216,9 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
  * ------------------------------------------------------------------------------------------- */
 #define FSVD_PH_EMBED 0   /* out0[n] = W[0][token, n]                                   (N = hidden)        */
 #define FSVD_PH_GEMV 1    /* out0 = epilogue(W[m] . norm(in)), m < nmat                                      */
-#define FSVD_PH_QKV 2     /* q/k/v head expansion from in = [Pq|Pk|Pv], RoPE, cache append; out0/1/2 = q/k/v */
-#define FSVD_PH_ATTN 3    /* split-KV attention of in = q over the cache + (aux0, aux1) = new k, v           */
+#define FSVD_PH_ATTN 3    /* in = un-rotated [q | k | v] of the current token ((H + 2*Hk) * Dh values, the   */
+                          /* output of a GEMV over the row-packed [q_u; k_u; v_u]): rotate-half RoPE on q, k */
+                          /* at state->pos, append k, v to the cache, split-KV attention; out0 = partials    */
 #define FSVD_PH_MERGE 4   /* out0 = merged attention output from in = partials                               */
 #define FSVD_PH_ARGMAX 5  /* token = argmax of the per-workgroup candidates in `in`; advances the state      */
 
@@ -235,21 +236,23 @@ typedef struct fsvd_tagbuf {
 typedef struct fsvd_phase {
   int32_t type, epilogue;
   int32_t N, K, nmat, mode;     /* rows per matrix, row length, matrices, SwiGLU rounding mode; the staged     */
-                                /* input has nmat * K elements (QKV: 3 * K)                                    */
-  int32_t H, Hk, Dh, nsplit, rope_len, S;
+                                /* input has nmat * K elements                                                 */
+  int32_t H, Hk, Dh, nsplit, rope_len, S;   /* on a GEMV, H > 0 marks the q | k | v head expansion: N = (H + 2*Hk) * Dh  */
+                                /* rows in three groups that read in[0:K], in[K:2K], in[2K:3K]                 */
   float fparam;                 /* GEMV with norm_w: RMSNorm eps; ATTN: softmax scale                          */
-  const void* W[3];             /* nn.Linear-layout weights [N, K] (QKV: q_u, k_u, v_u; EMBED: table [V, N]) */
+  const void* W[3];             /* nn.Linear-layout weights [N, K] (EMBED: table [V, N]); W[2] unused         */
   const void* norm_w;           /* RMSNorm weight over `in` or NULL                                            */
   const void* cos; const void* sin;   /* [rope_len, Dh/2]                                                      */
   void* k_cache; void* v_cache; /* batch row of the dense cache, [S, Hk, Dh] with strides sc_s, sc_h          */
   int64_t sc_s, sc_h;
   void* plain_out;              /* EP_LOGITS: bf16 logits [N]; ARGMAX: int64 token log indexed by state->step */
-  fsvd_tagbuf in, aux0, aux1, out0, out1, out2;
-  /* derived by fsvd_decode_step_prepare (do not fill by hand): work items (rows, or 16-row q/k/v groups)
-   * are dealt as share_q per workgroup plus one more for the first share_r workgroups; m_kp, m_pps are
-   * 32-bit reciprocals of K/8 and of the pieces per q/k/v segment */
+  fsvd_tagbuf in, aux0, aux1, out0, out1, out2;   /* aux0: residual of EP_RESID; aux1, out1, out2 reserved */
+  /* derived by fsvd_decode_step_prepare (do not fill by hand): work items (rows, merge outputs) are
+   * dealt as share_q per workgroup plus one more for the first share_r workgroups; m_kp is the 32-bit
+   * reciprocal of K/8 and dk = (threads per workgroup) mod (K/8) */
   int32_t share_q, share_r;
-  uint32_t m_kp, m_pps;
+  uint32_t m_kp;
+  int32_t dk;
 } fsvd_phase;
 
 typedef struct fsvd_step_state {
