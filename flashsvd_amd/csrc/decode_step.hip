@@ -567,15 +567,16 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     } else if (type == FSVD_PH_ATTN) {
       // fold the key slots and publish this split's (acc, m, l)
       const int Dh = 128;
-      float* wts = cp + kSlots * (Dh + 2);
-      float M = -INFINITY;
-      for (int j = 0; j < kSlots; ++j) M = fmaxf(M, cp[j * (Dh + 2) + Dh]);
-      if (tid < kSlots) {
-        const float mj = cp[tid * (Dh + 2) + Dh];
-        wts[tid] = (mj == -INFINITY) ? 0.f : __expf(mj - M);
+      float* wts = cp + kSlots * (Dh + 2);     // kSlots weights, then the maximum
+      if (tid < 64) {
+        const float mj = tid < kSlots ? cp[tid * (Dh + 2) + Dh] : -INFINITY;
+        const float M0 = wave_max(mj);
+        if (tid < kSlots) wts[tid] = (mj == -INFINITY) ? 0.f : __expf(mj - M0);
+        if (tid == 0) wts[kSlots] = M0;
       }
       __syncthreads();
       if (tid < Dh + 2) {
+        const float M = wts[kSlots];
         float o = M;
         if (tid != Dh) {
           const int col = tid < Dh ? tid : Dh + 1;
@@ -791,7 +792,7 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         if ((d.sc_s % 8) || (d.sc_h % 8) || (reinterpret_cast<uintptr_t>(d.k_cache) & 15) || (reinterpret_cast<uintptr_t>(d.v_cache) & 15))
           return bad("cache strides/pointers must be 16-byte aligned", p);
         if (d.S <= 0) return bad("cache length missing", p);
-        if (kSlots * (d.Dh + 2) + kSlots > kMaxChunks) return bad("internal: slot buffer", p);
+        if (kSlots * (d.Dh + 2) + kSlots + 1 > kMaxChunks) return bad("internal: slot buffer", p);
         writes_all[p] = 1;
         break;
       case FSVD_PH_MERGE:
