@@ -214,17 +214,25 @@ def generate_text(model, tokenizer, *, prompt: str, max_new_tokens: int = 64, de
     if use_graph is None:
         use_graph = _env_truthy("FLASH_SVD_DENSE_DECODE_GRAPH") or _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH")
     dec = None
+    pdec = None
     if use_graph and not do_sample and hasattr(model, "decode_step"):
         from .graphs import GraphedDecoder
-        dec = GraphedDecoder(model, cache, 1)
-        dec.set_state(next_token, prompt_len)
-        dec.capture()
+        from .step import make_persistent_decoder
+        pdec = make_persistent_decoder(model, cache, 1, max_new_tokens=int(max_new_tokens) + 1)
+        if pdec is not None:
+            pdec.set_state(next_token, prompt_len)
+        else:
+            dec = GraphedDecoder(model, cache, 1)
+            dec.set_state(next_token, prompt_len)
+            dec.capture()
     for step in range(int(max_new_tokens)):
         tid = int(next_token.item())
         output_ids.append(tid)
         if (eos is not None and tid == int(eos)) or step + 1 >= int(max_new_tokens):
             break
-        if dec is not None:
+        if pdec is not None:
+            next_token = pdec.step_token()
+        elif dec is not None:
             next_token = dec.step()
         else:
             out = _manual_llama_decode_step(model, next_token, past_key_values=cache,
@@ -263,11 +271,17 @@ def decode_kvcache_eval(model, *, prompt_len: int = 2048, new_tokens: int = 128,
     torch.cuda.synchronize()
     t_prefill = time.perf_counter() - t0
     next_token = out.logits[:, -1, :].argmax(dim=-1, keepdim=True)
-    dec = GraphedDecoder(model, cache, int(batch_size))
-    dec.set_state(next_token, int(prompt_len))
-    if use_graph:
-        dec.capture()
-    step = dec.step if use_graph else dec.eager_step
+    from .step import make_persistent_decoder
+    pdec = make_persistent_decoder(model, cache, int(batch_size), max_new_tokens=int(max_cache_len)) if use_graph else None
+    if pdec is not None:
+        pdec.set_state(next_token, int(prompt_len))
+        step = pdec.step_token
+    else:
+        dec = GraphedDecoder(model, cache, int(batch_size))
+        dec.set_state(next_token, int(prompt_len))
+        if use_graph:
+            dec.capture()
+        step = dec.step if use_graph else dec.eager_step
     for _ in range(max(0, int(warmup))):
         step()
     torch.cuda.synchronize()
@@ -276,7 +290,10 @@ def decode_kvcache_eval(model, *, prompt_len: int = 2048, new_tokens: int = 128,
         step()
     torch.cuda.synchronize()
     t_decode = time.perf_counter() - t1
+    if pdec is not None:
+        pdec.check()
     result = {
+        "decode_engine": "persistent" if pdec is not None else ("graph" if use_graph else "eager"),
         "prompt_len": int(prompt_len), "new_tokens": int(new_tokens), "batch_size": int(batch_size),
         "prefill_time_s": float(t_prefill), "decode_time_s": float(t_decode),
         "prefill_tok_s": float(batch_size * prompt_len / t_prefill) if t_prefill > 0 else float("inf"),
@@ -285,6 +302,10 @@ def decode_kvcache_eval(model, *, prompt_len: int = 2048, new_tokens: int = 128,
         "lowrank_cache": bool(lowrank_cache), "flashsvd_dense_cache": bool(flashsvd_dense_cache),
         "baseline_dense_kvcache": bool(baseline_dense_kvcache),
     }
+    if profile_decode and pdec is not None:
+        # one traced token: where the time of a step goes, phase by phase (the hipEvent-per-module profile of
+        # the reference, utils/evaluator.py:553-689, cannot look inside a single launch)
+        result["decode_profile_us"] = pdec.phase_profile()
     print("=== KV-Cache Prefill/Decode Benchmark ===")
     print(f"Prefill: prompt_len={prompt_len} | time {t_prefill:.3f}s | {result['prefill_tok_s']:,.0f} tok/s")
     print(f"Decode : new_tokens={new_tokens} | time {t_decode:.3f}s | {result['decode_ms_per_token']:.3f} ms/token | "

@@ -255,3 +255,52 @@ class PersistentDecoder:
     def hidden(self) -> torch.Tensor:
         """Final-layer hidden state of the last step, bf16 [hidden]."""
         return ((self.XA & 0xFFFF) << 16).view(torch.float32).to(torch.bfloat16)
+
+
+    # ------------------------------------------------------------------ GraphedDecoder-compatible face
+    def step_token(self) -> torch.Tensor:
+        """One token; returns the device tensor [1, 1] that holds the next token id (no synchronisation)."""
+        self.step(1)
+        return self.state.view(torch.int64)[2].reshape(1, 1)
+
+    def phase_profile(self, wg_stride: int = 32) -> dict:
+        """Per-phase microseconds of one traced step, averaged over layers and traced workgroups:
+        {phase name: {"wait": input wait, "stream": weight stream, "publish": epilogue, "total": ...}}."""
+        t = self.trace_step(wg_stride)
+        names = ["embed"] + [n for _ in range(self.L) for n in self.PHASE_NAMES[1:]] + ["lm_head", "argmax"]
+        acc: dict = {}
+        for p, nm in enumerate(names):
+            e, s_, c, d_ = (t[:, p, k] for k in range(4))
+            staged = torch.where(s_ > 0, s_, e)
+            row = acc.setdefault(nm, {"wait": 0.0, "stream": 0.0, "publish": 0.0, "total": 0.0, "n": 0})
+            row["wait"] += float((staged - e).mean())
+            row["stream"] += float((c - staged).mean())
+            row["publish"] += float((d_ - c).mean())
+            row["total"] += float((d_ - e).mean())
+            row["n"] += 1
+        return {k: {m: v[m] / v["n"] for m in ("wait", "stream", "publish", "total")} for k, v in acc.items()}
+
+
+def decode_engine_choice() -> str:
+    """FLASHSVD_AMD_DECODE_ENGINE = auto (default) | persistent | graph."""
+    import os
+    v = os.getenv("FLASHSVD_AMD_DECODE_ENGINE", "auto").strip().lower()
+    if v not in ("auto", "persistent", "graph"):
+        raise ValueError(f"FLASHSVD_AMD_DECODE_ENGINE={v!r}: expected auto, persistent or graph")
+    return v
+
+
+def make_persistent_decoder(model, cache, batch_size: int, *, max_new_tokens: int = 4096):
+    """A PersistentDecoder when the engine choice and the model allow it, else None (the caller then uses
+    graphs.GraphedDecoder).  With the choice "persistent" an unsupported model raises instead."""
+    choice = decode_engine_choice()
+    if choice == "graph":
+        return None
+    try:
+        if int(batch_size) != 1:
+            raise ValueError("the persistent step decodes one sequence")
+        return PersistentDecoder(model, cache, max_new_tokens=max_new_tokens)
+    except (ValueError, TypeError, _lib.FlashSVDHipError):
+        if choice == "persistent":
+            raise
+        return None

@@ -172,3 +172,48 @@ def test_phase_list_validation():
     dec.host_phases[2].inp.use = saved_use
     rc = lib.fsvd_decode_step(None, ctypes.addressof(dec.host_phases), dec.nph, dec.state.data_ptr(), 1, stream)
     assert rc == -4
+
+
+def test_decode_driver_picks_the_persistent_engine(monkeypatch):
+    """decode_kvcache_eval (the reference's timing protocol) runs on the persistent step when the model allows
+    it, reports the per-phase profile, and falls back to the graph engine on request."""
+    from flashsvd_amd import api
+    mw, _ = _small()
+    model = model_from_oracle(mw)
+    monkeypatch.setenv("FLASHSVD_AMD_DECODE_ENGINE", "auto")
+    r = api.decode_kvcache_eval(model, prompt_len=40, new_tokens=6, warmup=2, profile_decode=True, profile_decode_steps=1)
+    assert r["decode_engine"] == "persistent" and r["decode_tok_s"] > 0
+    prof = r["decode_profile_us"]
+    assert {"attn_rank_proj", "qkv_u", "attn", "attn_merge", "o_v", "o_u", "mlp_rank_proj", "swiglu", "down_v", "down_u",
+            "lm_head"} <= set(prof)
+    assert all(v["total"] >= 0 for v in prof.values())
+    monkeypatch.setenv("FLASHSVD_AMD_DECODE_ENGINE", "graph")
+    r2 = api.decode_kvcache_eval(model, prompt_len=40, new_tokens=6, warmup=2)
+    assert r2["decode_engine"] == "graph"
+    monkeypatch.setenv("FLASHSVD_AMD_DECODE_ENGINE", "sideways")
+    with pytest.raises(ValueError):
+        api.decode_kvcache_eval(model, prompt_len=40, new_tokens=2, warmup=1)
+
+
+def test_generate_text_same_tokens_on_both_engines(monkeypatch):
+    from flashsvd_amd import api
+
+    class Tok:
+        eos_token_id = None
+        pad_token_id = 0
+
+        def __call__(self, prompt, return_tensors="pt", add_special_tokens=False):
+            g = torch.Generator().manual_seed(len(prompt))
+            return {"input_ids": torch.randint(0, 2048, (1, 23), generator=g)}
+
+        def decode(self, ids, skip_special_tokens=False):
+            return " ".join(str(i) for i in ids)
+
+    mw, _ = _small()
+    model = model_from_oracle(mw)
+    outs = {}
+    for eng in ("persistent", "graph"):
+        monkeypatch.setenv("FLASHSVD_AMD_DECODE_ENGINE", eng)
+        outs[eng] = api.generate_text(model, Tok(), prompt="a seeded prompt", max_new_tokens=10, use_graph=True)
+    assert outs["persistent"]["generated_token_count"] == 10
+    assert outs["persistent"]["completion_ids"] == outs["graph"]["completion_ids"]
