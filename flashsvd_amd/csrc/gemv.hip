@@ -508,6 +508,7 @@ static int launch_linear_b(const LinearArgs& a, int cfg, hipStream_t st) {
 
 int launch_linear(const LinearArgs& a, int cfg, hipStream_t st) {
   if (a.B <= 0 || a.N <= 0 || a.K <= 0) { set_last_error("fsvd_linear: empty shape B=%d N=%d K=%d", a.B, a.N, a.K); return kErrBadShape; }
+  if (cfg == 0 && mfma_linear_applies(a)) return launch_linear_mfma(a, st);
   if (a.K > 32768) { set_last_error("fsvd_linear: K=%d exceeds the 32768 LDS staging limit", a.K); return kErrBadShape; }
   const bool vec = (a.K % 8 == 0) && (a.ldw % 8 == 0) && aligned16(a.W);
   const int batch = a.B >= 4 && a.K <= 16384 ? 4 : (a.B >= 2 ? 2 : 1);
@@ -542,6 +543,7 @@ static int launch_swiglu_b(const SwigluArgs& a, int cfg, hipStream_t st) {
 
 int launch_swiglu(const SwigluArgs& a, int cfg, hipStream_t st) {
   if (a.B <= 0 || a.D <= 0 || a.R <= 0) { set_last_error("fsvd_swiglu_linear: empty shape"); return kErrBadShape; }
+  if (cfg == 0 && mfma_swiglu_applies(a)) return launch_swiglu_mfma(a, st);
   if (a.R > 16384) { set_last_error("fsvd_swiglu_linear: R=%d exceeds 16384", a.R); return kErrBadShape; }
   const bool vec = (a.R % 8 == 0) && (a.ldw % 8 == 0) && aligned16(a.gate_u) && aligned16(a.up_u);
   const int batch = a.B >= 4 && a.R <= 4096 ? 4 : (a.B >= 2 ? 2 : 1);

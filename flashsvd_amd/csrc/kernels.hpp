@@ -134,6 +134,11 @@ int launch_expand(const ExpandArgs& a, hipStream_t st);
 int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st);
 
 int launch_linear(const LinearArgs& a, int cfg, hipStream_t st);
+// matrix-core path for 5+ rows (mfma_gemv.hip); launch_linear / launch_swiglu route to it when cfg == 0
+bool mfma_linear_applies(const LinearArgs& a);
+int launch_linear_mfma(const LinearArgs& a, hipStream_t st);
+bool mfma_swiglu_applies(const SwigluArgs& a);
+int launch_swiglu_mfma(const SwigluArgs& a, hipStream_t st);
 int launch_swiglu(const SwigluArgs& a, int cfg, hipStream_t st);
 int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st);
 int launch_rmsnorm(const uint16_t* x, int64_t ldx, const uint16_t* w, float eps, uint16_t* y, int64_t ldy, int rows,

@@ -71,6 +71,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             if t.shape != (n,) or not t.is_contiguous():
                 raise ValueError(f"{nm} must be a contiguous [{n}] tensor")
     lib = _lib.load()
+    if norm_weight is not None and B >= 5 and cfg == 0 and K % 32 == 0:
+        # five rows and more run on the matrix cores, which take the activations as they are: normalise once
+        # up front (same rounding points as the fused prologue)
+        x2 = rmsnorm(x2, norm_weight, eps)
+        norm_weight = None
     rc = lib.fsvd_linear(x2.data_ptr(), x2.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias), _ptr(norm_weight),
                          float(eps), _ptr(r2), 0 if r2 is None else r2.stride(0), o2.data_ptr(), o2.stride(0),
                          B, N, K, int(cfg), _stream())

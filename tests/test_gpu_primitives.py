@@ -152,3 +152,37 @@ def test_errors_are_python_exceptions(ops):
     kc = rand_bf16(1, 8, 2, 32).cuda()
     with pytest.raises(FlashSVDHipError):
         ops.attn_decode_densekv(q, kc, kc.clone(), torch.tensor([4], dtype=torch.int32).cuda(), nsplit=1)
+
+
+# ---- five rows and more: the matrix-core path (csrc/mfma_gemv.hip) behind the same entry points
+@pytest.mark.parametrize("B,N,K", [(5, 48, 1024), (8, 3072, 4096), (16, 1536, 11008), (17, 100, 2048), (32, 4096, 1536),
+                                   (64, 256, 512), (70, 33, 256), (8, 40, 96)])
+def test_linear_batched_matrix_cores(ops, B, N, K):
+    x, w = rand_bf16(B, K, seed=1), rand_bf16(N, K, std=0.02, seed=2)
+    bias, res = rand_bf16(N, std=0.1, seed=4), rand_bf16(B, N, seed=5)
+    y = ops.linear(x.cuda(), w.cuda(), bias.cuda(), residual=res.cuda())
+    assert_close_bf16(y, res + O.lin(x, w, bias), f"batched linear {B}x{N}x{K}")
+    # the vector kernels (explicit tiling) give the same rounding points
+    y_vec = ops.linear(x.cuda(), w.cuda(), bias.cuda(), residual=res.cuda(), cfg=1)
+    assert_close_bf16(y, y_vec.cpu(), "matrix-core vs vector path")
+
+
+def test_linear_batched_with_norm(ops):
+    B, N, K = 8, 512, 4096
+    x, w = rand_bf16(B, K, seed=1), rand_bf16(N, K, std=0.02, seed=2)
+    nw = rand_bf16(K, seed=3) * 0.1 + 1
+    y = ops.linear(x.cuda(), w.cuda(), norm_weight=nw.cuda(), eps=1e-6)
+    assert_close_bf16(y, O.lin(O.rms_norm(x, nw, 1e-6), w), "batched norm + linear")
+
+
+@pytest.mark.parametrize("B,D,R,mode", [(8, 11008, 1536, 0), (32, 1376, 256, 1), (5, 100, 64, 0), (33, 64, 96, 1)])
+def test_swiglu_batched_matrix_cores(ops, B, D, R, mode):
+    p = rand_bf16(B, 2 * R, seed=1)
+    gu, uu = rand_bf16(D, R, std=0.05, seed=2), rand_bf16(D, R, std=0.05, seed=3)
+    h = ops.swiglu_linear(p.cuda(), gu.cuda(), uu.cuda(), up_off=R, mode=mode)
+    g, u = p[:, :R].float() @ gu.float().t(), p[:, R:].float() @ uu.float().t()
+    if mode == 0:
+        ref = torch.nn.functional.silu(g.to(torch.bfloat16)) * u.to(torch.bfloat16)
+    else:
+        ref = ((g * torch.sigmoid(g)) * u).to(torch.bfloat16)
+    assert_close_bf16(h, ref, f"batched swiglu mode {mode}")
