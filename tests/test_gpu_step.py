@@ -217,3 +217,38 @@ def test_generate_text_same_tokens_on_both_engines(monkeypatch):
         outs[eng] = api.generate_text(model, Tok(), prompt="a seeded prompt", max_new_tokens=10, use_graph=True)
     assert outs["persistent"]["generated_token_count"] == 10
     assert outs["persistent"]["completion_ids"] == outs["graph"]["completion_ids"]
+
+
+def test_checkpoint_round_trip_decodes_identically(tmp_path):
+    """A directory checkpoint in the wrapped factor-pair naming, loaded straight to the GPU, gives the tokens
+    of the model it was written from (loader + persistent step on loaded, unpacked weights)."""
+    import json
+    from safetensors.torch import save_file
+    from flashsvd_amd import checkpoint as ck
+    from flashsvd_amd.step import PersistentDecoder
+    mw, prompt = _small()
+    model = model_from_oracle(mw)
+    sd = {}
+    for k, v in model.state_dict().items():
+        parts = k.split(".")
+        if len(parts) == 6 and parts[3] in ("self_attn", "mlp"):
+            proj, factor = parts[4].split("_")[:2]
+            parts[4:5] = [f"{proj}_proj", f"{factor}_proj"]
+        sd[".".join(parts)] = v.detach().cpu().contiguous().clone()
+    cfg = model.config
+    (tmp_path / "config.json").write_text(json.dumps(dict(
+        hidden_size=cfg.hidden_size, num_attention_heads=cfg.num_attention_heads, num_key_value_heads=cfg.num_key_value_heads,
+        head_dim=cfg.head_dim, intermediate_size=cfg.intermediate_size, num_hidden_layers=cfg.num_hidden_layers,
+        vocab_size=cfg.vocab_size, rope_theta=cfg.rope_theta, rms_norm_eps=cfg.rms_norm_eps, torch_dtype="bfloat16",
+        max_position_embeddings=getattr(cfg, "max_position_embeddings", 4096))))
+    save_file(sd, str(tmp_path / "model.safetensors"))
+    loaded = ck.load_lowrank_model_from_dir(tmp_path, device="cuda")
+    n_new, Lp = 9, prompt.shape[1]
+    toks = []
+    for m in (model, loaded):
+        cache, tok0 = _prefill(m, prompt, n_new + 4)
+        dec = PersistentDecoder(m, cache)
+        dec.set_state(tok0, Lp)
+        dec.step(n_new - 1)
+        toks.append([int(tok0)] + dec.tokens().cpu().tolist())
+    assert toks[0] == toks[1]
