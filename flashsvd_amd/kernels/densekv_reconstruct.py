@@ -152,6 +152,16 @@ def _xw(x: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], bias_pos
     return y
 
 
+def xw_linear(x: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ W`` for x [B,K] and a row-major [K,N] matrix such as the packed rank projection
+    (the product the reference issues as torch.matmul, benchmark/attn/decode_compare.py:1538)."""
+    if not _all_cuda(x, W):
+        raise ValueError("xw_linear expects all tensors on CUDA.")
+    if x.ndim != 2 or W.ndim != 2 or x.shape[1] != W.shape[0]:
+        raise ValueError(f"xw_linear: x {tuple(x.shape)} does not chain with W {tuple(W.shape)}")
+    return _xw(x, W, bias, False)
+
+
 def reconstruct_qkv_token_shared_prepacked(Pq, Pk, Pv, Vq_flat, Vk_flat, Vv_flat, *, H: int, Hk: int, Dh: int,
                                            bq=None, bk=None, bv=None):
     """Q = Pq @ Vq_flat etc. on the prepacked [R, heads*Dh] bases; the bias is added after the
@@ -178,4 +188,4 @@ def reconstruct_qkv_token_shared_prepacked(Pq, Pk, Pv, Vq_flat, Vk_flat, Vv_flat
 
 
 __all__ = ["reconstruct_qkv_token", "reconstruct_qkv_token_shared", "reconstruct_qkv_token_shared_hetero",
-           "pack_qkv_shared_bases", "reconstruct_qkv_token_shared_prepacked"]
+           "pack_qkv_shared_bases", "reconstruct_qkv_token_shared_prepacked", "xw_linear"]

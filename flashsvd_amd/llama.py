@@ -217,6 +217,22 @@ class SVD_LlamaAttention(nn.Module):
         return out
 
     # ---- decode ---------------------------------------------------------------------------------
+    def _dense_decode_backend(self, cache=None) -> str:
+        """"exact" or "packed" for the current token: the entry an applied decode plan holds for this layer
+        (per bucket of cached keys, read from the cache's host-side count, so a captured graph keeps the
+        choice it was captured with), else FLASH_SVD_DENSE_DECODE_BACKEND (auto = packed)."""
+        entry = getattr(self, "_dense_decode_plan", None)
+        if entry:
+            from .plan import plan_choice
+            past = None
+            if cache is not None and isinstance(entry.get("buckets"), dict):
+                past = int(cache.get_seq_length())
+            return plan_choice(entry, past)
+        raw = os.getenv("FLASH_SVD_DENSE_DECODE_BACKEND", "auto").strip().lower() or "auto"
+        if raw not in ("auto", "exact", "packed"):
+            raise ValueError(f"FLASH_SVD_DENSE_DECODE_BACKEND={raw!r}: expected auto, exact or packed")
+        return "exact" if raw == "exact" else "packed"
+
     def _positions_for(self, cache, batch: int, cache_position, device) -> torch.Tensor:
         """int32 [B] device tensor holding the write position of the current token."""
         if isinstance(cache_position, torch.Tensor) and cache_position.is_cuda and cache_position.dtype == torch.int32 \
@@ -256,13 +272,23 @@ class SVD_LlamaAttention(nn.Module):
         kc, vc = cache.key_cache[self.layer_idx], cache.value_cache[self.layer_idx]
         if rope is None:
             rope = cache.get_rope_tables(seqlen=cache.max_cache_len, head_dim=Dh, device=x.device, dtype=x.dtype)
-        p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)
-        q = hip_ops.qkv_rope_append(p, self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight, rope[0], rope[1],
-                                    positions, kc[:B], vc[:B], num_heads=H, num_kv_heads=Hk, head_dim=Dh)
-        cache._layer_initialized[self.layer_idx] = True
         if nsplit is None:
             nsplit = hip_ops.pick_nsplit(cache.max_cache_len, B, H, Dh)
-        a = hip_ops.attn_decode_densekv(q, kc[:B], vc[:B], positions, seqlen_add=1, nsplit=nsplit, workspace=attn_ws)
+        if self._dense_decode_backend(cache) == "exact":
+            # module by module: three rank projections, three head expansions, rotary + append inside attention
+            xn = x if norm_weight is None else hip_ops.rmsnorm(x, norm_weight, eps)
+            q = hip_ops.linear(hip_ops.linear(xn, self.q_v_proj.weight), self.q_u_proj.weight).view(B, H, Dh)
+            k = hip_ops.linear(hip_ops.linear(xn, self.k_v_proj.weight), self.k_u_proj.weight).view(B, Hk, Dh)
+            v = hip_ops.linear(hip_ops.linear(xn, self.v_v_proj.weight), self.v_u_proj.weight).view(B, Hk, Dh)
+            a = hip_ops.attn_decode_densekv(q, kc[:B], vc[:B], positions, k_new=k, v_new=v, cos=rope[0], sin=rope[1],
+                                            nsplit=nsplit, workspace=attn_ws)
+            cache._layer_initialized[self.layer_idx] = True
+        else:
+            p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)
+            q = hip_ops.qkv_rope_append(p, self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight, rope[0], rope[1],
+                                        positions, kc[:B], vc[:B], num_heads=H, num_kv_heads=Hk, head_dim=Dh)
+            cache._layer_initialized[self.layer_idx] = True
+            a = hip_ops.attn_decode_densekv(q, kc[:B], vc[:B], positions, seqlen_add=1, nsplit=nsplit, workspace=attn_ws)
         po = hip_ops.linear(a.view(B, H * Dh), self.o_v_proj.weight)
         return hip_ops.linear(po, self.o_u_proj.weight, residual=residual)
 

@@ -73,18 +73,27 @@ class PersistentDecoder:
         def tagged64(n):
             return torch.zeros(n, dtype=torch.int64, device=dev)
 
-        a0 = inner.layers[0].self_attn
-        m0 = inner.layers[0].mlp
-        Rq, Rk, Rv = a0._qkv_rank_tuple()
-        Ro = int(a0.o_v_proj.out_features)
-        Rm = int(m0.gate_v_proj.out_features)
-        D = int(m0.gate_u_proj.out_features)
-        if not (Rq == Rk == Rv):
-            raise ValueError("PersistentDecoder needs equal q/k/v ranks (pad them to a common multiple of 128)")
+        # ranks may differ from layer to layer (buffers take the largest); within a layer q, k and v share
+        # one rank because their head expansion is a single grouped product
+        ranks = []
+        for li, layer in enumerate(inner.layers):
+            at, mlp = layer.self_attn, layer.mlp
+            rq, rk, rv = at._qkv_rank_tuple()
+            if not (rq == rk == rv):
+                raise ValueError(f"PersistentDecoder needs equal q/k/v ranks in layer {li} (got {rq}/{rk}/{rv}; pad them "
+                                 "to a common multiple of 128)")
+            rm = int(mlp.gate_v_proj.out_features)
+            if int(mlp.up_v_proj.out_features) != rm:
+                raise ValueError(f"PersistentDecoder needs equal gate/up ranks in layer {li}")
+            ranks.append((rq, int(at.o_v_proj.out_features), rm, int(mlp.down_v_proj.out_features)))
+        if not ranks:
+            raise ValueError("PersistentDecoder needs at least one layer")
+        Rq, Ro, Rm, Rd = (max(r[i] for r in ranks) for i in range(4))
+        D = int(inner.layers[0].mlp.gate_u_proj.out_features)
         self.XA, self.XB = tagged(d), tagged(d)
         self.P, self.QKV = tagged(3 * Rq), tagged((H + 2 * Hk) * Dh)
         self.PART, self.A = tagged64(H * nsplit * (Dh + 2)), tagged(H * Dh)
-        self.PO, self.PM, self.HB, self.SB = tagged(Ro), tagged(2 * Rm), tagged(D), tagged(Rm)
+        self.PO, self.PM, self.HB, self.SB = tagged(Ro), tagged(2 * Rm), tagged(D), tagged(Rd)
         self.CAND = tagged64(self.nwg)
         self.logits = torch.zeros(V, dtype=torch.bfloat16, device=dev)
         self.token_log = torch.zeros(int(max_new_tokens), dtype=torch.int64, device=dev)
@@ -127,19 +136,17 @@ class PersistentDecoder:
             at, mlp = layer.self_attn, layer.mlp
             at._ensure_runtime_state()
             mlp._ensure_runtime_state()
-            if at._qkv_rank_tuple() != (Rq, Rk, Rv) or int(at.o_v_proj.out_features) != Ro or \
-                    int(mlp.gate_v_proj.out_features) != Rm or int(mlp.up_v_proj.out_features) != Rm:
-                raise ValueError("PersistentDecoder needs the same ranks in every layer")
+            rq, ro, rm, rd = ranks[l]
             cache._ensure_layer_spec(l, h=Hk, dh=Dh)
             kc, vc = cache.key_cache[l][0], cache.value_cache[l][0]      # [S, Hk, Dh]
             n1, n2 = layer.input_layernorm, layer.post_attention_layernorm
             xin, xmid, xout = _tb(self.XA, L + 1, l), _tb(self.XB, L, l), _tb(self.XA, L + 1, l + 1)
-            gemv([at._packed_qkv_v], 3 * Rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
+            gemv([at._packed_qkv_v], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
             # q, k, v head expansion as one GEMV over the row-packed [q_u; k_u; v_u] (the three module
             # weights become views of one buffer); RoPE and the cache append happen in the attention phase
             qkv_u = _packed_rows([at.q_u_proj, at.k_u_proj, at.v_u_proj])
             self._keep.append(qkv_u)
-            gemv([qkv_u], (H + 2 * Hk) * Dh, Rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
+            gemv([qkv_u], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
             a = Phase()
             a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
             a.fparam = 1.0 / math.sqrt(Dh)
@@ -151,13 +158,13 @@ class PersistentDecoder:
             m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
             m.inp, m.out0 = _tb(self.PART, L, l), _tb(self.A, L, l)
             ph.append(m)
-            gemv([at.o_v_proj.weight], Ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
-            gemv([at.o_u_proj.weight], d, Ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
-            gemv([mlp._packed_gu_v], 2 * Rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
-            gemv([mlp.gate_u_proj.weight, mlp.up_u_proj.weight], D, Rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2,
+            gemv([at.o_v_proj.weight], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
+            gemv([at.o_u_proj.weight], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
+            gemv([mlp._packed_gu_v], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
+            gemv([mlp.gate_u_proj.weight, mlp.up_u_proj.weight], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2,
                  epi=EP_SWIGLU)
-            gemv([mlp.down_v_proj.weight], Rm, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
-            gemv([mlp.down_u_proj.weight], d, Rm, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
+            gemv([mlp.down_v_proj.weight], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
+            gemv([mlp.down_u_proj.weight], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
             cache._layer_initialized[l] = True
         fn = inner.norm
         gemv([model.lm_head.weight], V, d, _tb(self.XA, L + 1, L), _tb(self.CAND, 1, 0), norm=fn.weight,

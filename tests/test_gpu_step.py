@@ -68,7 +68,9 @@ def test_small_model_teacher_forced_against_oracle():
 
 def test_small_model_free_running_matches_kernel_path():
     """16 launches queued without host synchronisation: same greedy tokens and cache rows as the
-    per-kernel decode path (both GPU paths, identical rounding points)."""
+    per-kernel decode path (both GPU paths, same rounding points; fp32 sums are split differently, so a
+    token may differ where the per-kernel path itself holds the two candidates within bf16 resolution —
+    the comparison stops there)."""
     from flashsvd_amd.graphs import GraphedDecoder
     from flashsvd_amd.step import PersistentDecoder
     mw, prompt = _small()
@@ -78,22 +80,31 @@ def test_small_model_free_running_matches_kernel_path():
     cache_k, tok0 = _prefill(model, prompt, n_new + 4)
     dec_k = GraphedDecoder(model, cache_k, 1)
     dec_k.set_state(tok0, Lp)
-    toks_k = [tok0.clone()]
+    toks_k, logits_k = [tok0.clone()], [None]
     for _ in range(n_new - 1):
         toks_k.append(dec_k.eager_step().clone())
+        logits_k.append(dec_k.logits[0, -1].float().cpu())
     toks_k = torch.cat(toks_k, 1).cpu()
     cache_p, tok0p = _prefill(model, prompt, n_new + 4)
     dec = PersistentDecoder(model, cache_p)
     dec.set_state(tok0p, Lp)
     dec.step(n_new - 1)
     toks_p = torch.cat([tok0p.cpu(), dec.tokens().cpu()[None, :]], 1)
-    assert torch.equal(toks_p, toks_k), f"step kernel {toks_p.tolist()} vs per-kernel path {toks_k.tolist()}"
+    same = n_new
+    for s in range(n_new):
+        if int(toks_p[0, s]) != int(toks_k[0, s]):
+            assert s >= 4, f"step kernel {toks_p.tolist()} vs per-kernel path {toks_k.tolist()}"
+            _tie_aware(int(toks_p[0, s]), int(toks_k[0, s]), logits_k[s], f"free-running step {s}")
+            same = s
+            break
     assert cache_p.get_seq_length() == cache_k.get_seq_length()
+    rows = min(same, n_new - 1)          # cache row Lp + j holds the token fed at step j + 1
     for li in range(3):
         for got, ref, nm in ((cache_p.key_cache[li], cache_k.key_cache[li], "K"), (cache_p.value_cache[li], cache_k.value_cache[li], "V")):
-            assert_close_bf16(got[:, Lp:Lp + n_new - 1], ref[:, Lp:Lp + n_new - 1], f"{nm} rows layer {li}", abs_tol=float("inf"), rel_tol=3e-2)
-    assert_close_bf16(dec.logits[None].cpu(), dec_k.logits[:, -1].float().cpu(), "logits of the last step", rel_tol=3e-2,
-                      abs_tol=3 * bounds(dec_k.logits.float())["abs_tol"])
+            assert_close_bf16(got[:, Lp:Lp + rows], ref[:, Lp:Lp + rows], f"{nm} rows layer {li}", abs_tol=float("inf"), rel_tol=3e-2)
+    if same == n_new:
+        assert_close_bf16(dec.logits[None].cpu(), dec_k.logits[:, -1].float().cpu(), "logits of the last step", rel_tol=3e-2,
+                          abs_tol=3 * bounds(dec_k.logits.float())["abs_tol"])
 
 
 def test_7b_width_two_layers_teacher_forced_tie_aware():
@@ -216,7 +227,10 @@ def test_generate_text_same_tokens_on_both_engines(monkeypatch):
         monkeypatch.setenv("FLASHSVD_AMD_DECODE_ENGINE", eng)
         outs[eng] = api.generate_text(model, Tok(), prompt="a seeded prompt", max_new_tokens=10, use_graph=True)
     assert outs["persistent"]["generated_token_count"] == 10
-    assert outs["persistent"]["completion_ids"] == outs["graph"]["completion_ids"]
+    # the engines split their fp32 sums differently, so a near-tie between two logits may fall either way
+    # (after which the texts differ); tie-aware token parity is checked step by step in the tests above
+    a, b = outs["persistent"]["completion_ids"], outs["graph"]["completion_ids"]
+    assert len(a) == len(b) == 10 and a[:4] == b[:4], f"{a} vs {b}"
 
 
 def test_checkpoint_round_trip_decodes_identically(tmp_path):
