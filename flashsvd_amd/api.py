@@ -302,15 +302,115 @@ def decode_kvcache_eval(model, *, prompt_len: int = 2048, new_tokens: int = 128,
         "lowrank_cache": bool(lowrank_cache), "flashsvd_dense_cache": bool(flashsvd_dense_cache),
         "baseline_dense_kvcache": bool(baseline_dense_kvcache),
     }
+    profile = None
     if profile_decode and pdec is not None:
-        # one traced token: where the time of a step goes, phase by phase (the hipEvent-per-module profile of
-        # the reference, utils/evaluator.py:553-689, cannot look inside a single launch)
+        # one traced token: where the time of a step goes, phase by phase (events around modules, as in
+        # utils/evaluator.py:553-689, cannot look inside a single launch), folded into the same categories
         result["decode_profile_us"] = pdec.phase_profile()
+        profile = decode_profile_from_phases(result["decode_profile_us"], len(model.model.layers),
+                                             float(result["decode_ms_per_token"]))
+    elif profile_decode:
+        profile = profile_decode_modules(dec, int(profile_decode_steps))
+    if profile is not None:
+        result["decode_profile"] = profile
     print("=== KV-Cache Prefill/Decode Benchmark ===")
     print(f"Prefill: prompt_len={prompt_len} | time {t_prefill:.3f}s | {result['prefill_tok_s']:,.0f} tok/s")
     print(f"Decode : new_tokens={new_tokens} | time {t_decode:.3f}s | {result['decode_ms_per_token']:.3f} ms/token | "
           f"{result['decode_tok_s']:,.0f} tok/s")
+    if profile is not None:
+        print("\n".join(format_decode_profile(profile)))
     return result
+
+
+_PROFILE_CATEGORIES = ("attn_total", "mlp_total", "ln1_total", "ln2_total", "embed_tokens", "final_norm", "lm_head")
+
+
+def _finish_profile(per_mod: dict, total_ms_per_tok: float, steps: int, seq: int, source: str) -> dict:
+    """Fold per-module milliseconds into the reference's categories (utils/evaluator.py:646-660).  Both
+    RMSNorms of a layer and the final norm run inside the projection that consumes them, so their own rows
+    read zero and their time sits in attn / mlp / lm_head."""
+    def suffix(sfx):
+        return sum(v for k, v in per_mod.items() if k.endswith(sfx))
+    breakdown = {"attn_total": suffix(".attn"), "mlp_total": suffix(".mlp"), "ln1_total": suffix(".ln1"),
+                 "ln2_total": suffix(".ln2"), "embed_tokens": per_mod.get("embed_tokens", 0.0),
+                 "final_norm": per_mod.get("final_norm", 0.0), "lm_head": per_mod.get("lm_head", 0.0)}
+    other = max(0.0, float(total_ms_per_tok) - float(sum(breakdown.values())))
+    return {"source": source, "steps": int(steps), "seq": int(seq), "total_forward_ms_per_token": float(total_ms_per_tok),
+            "breakdown_ms": breakdown, "other_ms": other, "per_module_ms": dict(per_mod)}
+
+
+def decode_profile_from_phases(phases_us: dict, n_layers: int, total_ms_per_tok: float) -> dict:
+    """The persistent step's per-phase microseconds (averages over layers) as a per-token module profile."""
+    def ms(*names):
+        return sum(float(phases_us.get(n, {}).get("total", 0.0)) for n in names) / 1000.0
+    attn = ms("attn_rank_proj", "qkv_u", "attn", "attn_merge", "o_v", "o_u")
+    mlp = ms("mlp_rank_proj", "swiglu", "down_v", "down_u")
+    per_mod = {"embed_tokens": ms("embed"), "lm_head": ms("lm_head", "argmax")}
+    for i in range(int(n_layers)):
+        per_mod[f"layer{i}.attn"] = attn
+        per_mod[f"layer{i}.mlp"] = mlp
+    return _finish_profile(per_mod, total_ms_per_tok, 1, 0, "persistent step, one traced token")
+
+
+def profile_decode_modules(dec, steps: int) -> dict:
+    """Per-module device time of ``steps`` un-captured per-kernel decode tokens, measured with events recorded
+    around each module's kernels on the current stream (the reference does this with forward hooks)."""
+    from . import hip_ops
+    model, cache = dec.model, dec.cache
+    inner = model.model
+    pairs: dict = {}
+
+    def timed(name, fn):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        out = fn()
+        b.record()
+        pairs.setdefault(name, []).append((a, b))
+        return out
+
+    totals = []
+    start_pos = int(getattr(dec, "_host_pos", 0))
+    for _ in range(int(steps)):
+        if getattr(dec, "_host_pos", 0) + 1 > cache.max_cache_len:
+            raise IndexError(f"decode position {dec._host_pos} outside the cache (max {cache.max_cache_len})")
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        x = timed("embed_tokens", lambda: inner.embed_tokens(dec.tokens)[:, 0])
+        for i, layer in enumerate(inner.layers):
+            n1 = layer.input_layernorm
+            x2 = timed(f"layer{i}.attn", lambda: layer.self_attn.decode_token(
+                x, cache, dec.positions, norm_weight=n1.weight, eps=n1.variance_epsilon, residual=x, rope=dec.rope,
+                attn_ws=dec.attn_ws, nsplit=dec.nsplit))
+            x = timed(f"layer{i}.mlp", lambda: layer._layer_tail(x2))
+        logits = timed("lm_head", lambda: hip_ops.linear(x, model.lm_head.weight, norm_weight=inner.norm.weight,
+                                                          eps=inner.norm.variance_epsilon))
+        dec.tokens.copy_(logits.argmax(dim=-1, keepdim=True))
+        dec.positions.add_(1)
+        t1.record()
+        totals.append((t0, t1))
+        dec._host_pos = getattr(dec, "_host_pos", 0) + 1
+        cache._seen_tokens += 1
+    torch.cuda.synchronize()
+    n = float(max(1, int(steps)))
+    per_mod = {k: sum(float(a.elapsed_time(b)) for a, b in v) / n for k, v in pairs.items()}
+    total = sum(float(a.elapsed_time(b)) for a, b in totals) / n
+    return _finish_profile(per_mod, total, int(steps), start_pos, "per-kernel path, events around modules")
+
+
+def format_decode_profile(profile: dict, topk: int = 10) -> list[str]:
+    total = float(profile["total_forward_ms_per_token"])
+    pct = (lambda v: 100.0 * v / total if total > 0 else 0.0)
+    lines = ["", "=== Decode Profile (module device time) ===",
+             f"Avg over {profile['steps']} steps @ seq≈{profile['seq']} | total_forward {total:.3f} ms/token ({profile['source']})"]
+    for k, v in sorted(profile["breakdown_ms"].items(), key=lambda kv: kv[1], reverse=True):
+        lines.append(f"  {k:12s}: {v:8.3f} ms ({pct(v):5.1f}%)")
+    lines.append(f"  {'other':12s}: {profile['other_ms']:8.3f} ms ({pct(profile['other_ms']):5.1f}%)")
+    top = sorted(((k, v) for k, v in profile["per_module_ms"].items() if v > 0), key=lambda kv: kv[1], reverse=True)[:topk]
+    if top:
+        lines.append(f"Top {len(top)}/{topk} modules:")
+        lines += [f"  {name:16s}: {ms:8.3f} ms ({pct(ms):5.1f}%)" for name, ms in top]
+    lines.append("")
+    return lines
 
 
 def enable_flashsvd_llama_layer_tail_cuda_graph() -> None:
