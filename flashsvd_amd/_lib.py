@@ -52,6 +52,11 @@ SIGNATURES = {
                             c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_swiglu_linear": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                                    c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "fsvd_linear_q4": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p,
+                               c_float, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
+    "fsvd_dequant_q4": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "fsvd_swiglu_linear_q4": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                      c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int64, c_int64, c_int64,

@@ -140,6 +140,21 @@ int launch_linear_mfma(const LinearArgs& a, hipStream_t st);
 bool mfma_swiglu_applies(const SwigluArgs& a);
 int launch_swiglu_mfma(const SwigluArgs& a, hipStream_t st);
 int launch_swiglu(const SwigluArgs& a, int cfg, hipStream_t st);
+
+// group-wise int4 weights (q4_gemv.hip): one matrix (linear) or the gate/up pair of the SwiGLU
+struct Q4Args {
+  const uint16_t* x; int64_t ldx; int64_t up_off;   // [B, >= K] bf16; the second matrix reads x + up_off
+  const uint8_t* qw[2]; int64_t ldq;                // [N, ldq] bytes, two columns per byte (even column low nibble)
+  const uint16_t* sc[2]; const int16_t* zr[2]; int64_t ldg;   // fp16 scales / int16 zero points [N, ldg]
+  int group;                                        // columns per group (power of two >= 32), <= 0 or >= K: one per row
+  const uint16_t* bias; const uint16_t* norm_w; float eps;
+  const uint16_t* res; int64_t ldres;
+  uint16_t* y; int64_t ldy;
+  int B, N, K, nmat, mode;
+};
+int launch_linear_q4(const Q4Args& a, hipStream_t st);
+int launch_dequant_q4(const uint8_t* qw, int64_t ldq, const uint16_t* sc, const int16_t* zr, int64_t ldg, int group, uint16_t* w,
+                      int64_t ldw, int N, int K, hipStream_t st);
 int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st);
 int launch_rmsnorm(const uint16_t* x, int64_t ldx, const uint16_t* w, float eps, uint16_t* y, int64_t ldy, int rows,
                    int K, hipStream_t st);

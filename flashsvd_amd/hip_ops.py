@@ -104,6 +104,97 @@ def swiglu_linear(p: torch.Tensor, gate_u: torch.Tensor, up_u: torch.Tensor, *, 
     return out
 
 
+def _q4_check(qweight, scales, zeros, N: int, K: int, group_size: int, name: str) -> int:
+    """Validate one int4 matrix; returns the group width the kernel is given (0 = one group per row)."""
+    if qweight.dtype != torch.uint8 or scales.dtype != torch.float16 or zeros.dtype != torch.int16:
+        raise TypeError(f"{name}: expected uint8 weights, float16 scales and int16 zeros, got {qweight.dtype}, {scales.dtype}, "
+                        f"{zeros.dtype}")
+    if not (qweight.is_cuda and scales.is_cuda and zeros.is_cuda):
+        raise ValueError(f"{name}: quantised buffers must be on the GPU")
+    if qweight.dim() != 2 or qweight.shape != (N, (K + 1) // 2) or qweight.stride(1) != 1:
+        raise ValueError(f"{name}: packed weight must be [{N}, {(K + 1) // 2}] bytes, got {tuple(qweight.shape)}")
+    group = 0 if group_size <= 0 or group_size >= K else int(group_size)
+    G = 1 if group == 0 else -(-K // group)
+    if scales.shape != (N, G) or zeros.shape != (N, G) or scales.stride() != zeros.stride() or scales.stride(1) != 1:
+        raise ValueError(f"{name}: scales / zeros must be matching [{N}, {G}] tensors, got {tuple(scales.shape)} / {tuple(zeros.shape)}")
+    return group
+
+
+def linear_q4(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor, *, group_size: int,
+              bias: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
+              residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = (residual +) linear(rmsnorm?(x), s * (q - z), bias) on group-wise int4 weights [N, K/2] bytes."""
+    _need(x, "x")
+    N, K = qweight.shape[0], x.shape[-1]
+    group = _q4_check(qweight, scales, zeros, N, K, group_size, "linear_q4")
+    x2 = _rows(x, "x")
+    B = x2.shape[0]
+    if out is None:
+        out = torch.empty(*x.shape[:-1], N, device=x.device, dtype=_BF16)
+    o2 = out if out.dim() == 2 else _rows(out, "out")
+    if o2.shape != (B, N) or o2.stride(1) != 1:
+        raise ValueError("out must be a [rows, N] tensor with unit inner stride matching x")
+    r2 = None
+    if residual is not None:
+        _need(residual, "residual")
+        r2 = _rows(residual, "residual")
+        if r2.shape != (B, N):
+            raise ValueError(f"residual shape {tuple(residual.shape)} does not match output [{B}, {N}]")
+    for t, nm, n in ((bias, "bias", N), (norm_weight, "norm_weight", K)):
+        if t is not None:
+            _need(t, nm)
+            if t.shape != (n,) or not t.is_contiguous():
+                raise ValueError(f"{nm} must be a contiguous [{n}] tensor")
+    lib = _lib.load()
+    rc = lib.fsvd_linear_q4(x2.data_ptr(), x2.stride(0), qweight.data_ptr(), qweight.stride(0), scales.data_ptr(), zeros.data_ptr(),
+                            scales.stride(0), group, _ptr(bias), _ptr(norm_weight), float(eps), _ptr(r2),
+                            0 if r2 is None else r2.stride(0), o2.data_ptr(), o2.stride(0), B, N, K, _stream())
+    _lib.check("fsvd_linear_q4", rc)
+    return out
+
+
+def swiglu_linear_q4(p: torch.Tensor, gate: tuple, up: tuple, *, up_off: int, group_size: int, mode: int = 0,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h = silu(p[..., :R] @ Wg.T) * (p[..., up_off:up_off+R] @ Wu.T); gate / up are (qweight, scales, zeros) of [D, R]."""
+    _need(p, "p")
+    (gq, gs, gz), (uq, us, uz) = gate, up
+    D = gq.shape[0]
+    R = 2 * gq.shape[1]
+    p2 = _rows(p, "p")
+    if p2.shape[1] < up_off + R:
+        raise ValueError(f"p last dim {p2.shape[1]} too small for up_off {up_off} + R {R}")
+    group = _q4_check(gq, gs, gz, D, R, group_size, "swiglu_linear_q4 gate")
+    _q4_check(uq, us, uz, D, R, group_size, "swiglu_linear_q4 up")
+    if gq.stride() != uq.stride() or gs.stride() != us.stride():
+        raise ValueError("gate and up must share one layout")
+    B = p2.shape[0]
+    if out is None:
+        out = torch.empty(*p.shape[:-1], D, device=p.device, dtype=_BF16)
+    o2 = _rows(out, "out")
+    lib = _lib.load()
+    rc = lib.fsvd_swiglu_linear_q4(p2.data_ptr(), p2.stride(0), int(up_off), gq.data_ptr(), gs.data_ptr(), gz.data_ptr(),
+                                   uq.data_ptr(), us.data_ptr(), uz.data_ptr(), gq.stride(0), gs.stride(0), group,
+                                   o2.data_ptr(), o2.stride(0), B, D, R, int(mode), _stream())
+    _lib.check("fsvd_swiglu_linear_q4", rc)
+    return out
+
+
+def dequant_q4(qweight: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor, *, in_features: int, group_size: int,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16 [N, K] = s * (q - z)."""
+    N, K = qweight.shape[0], int(in_features)
+    group = _q4_check(qweight, scales, zeros, N, K, group_size, "dequant_q4")
+    if out is None:
+        out = torch.empty(N, K, device=qweight.device, dtype=_BF16)
+    elif out.shape != (N, K) or out.dtype != _BF16 or out.stride(1) != 1:
+        raise ValueError(f"out must be a bf16 [{N}, {K}] tensor with unit inner stride")
+    lib = _lib.load()
+    rc = lib.fsvd_dequant_q4(qweight.data_ptr(), qweight.stride(0), scales.data_ptr(), zeros.data_ptr(), scales.stride(0), group,
+                             out.data_ptr(), out.stride(0), N, K, _stream())
+    _lib.check("fsvd_dequant_q4", rc)
+    return out
+
+
 def qkv_rope_append(p: torch.Tensor, q_u: torch.Tensor, k_u: torch.Tensor, v_u: torch.Tensor,
                     cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                     k_cache: torch.Tensor, v_cache: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int,

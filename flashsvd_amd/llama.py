@@ -148,6 +148,10 @@ class SVD_LlamaAttention(nn.Module):
         self._dense_decode_backend_cache: dict = {}
         self._packed_qkv_v = None
 
+    def _factor_modules(self):
+        return (self.q_v_proj, self.q_u_proj, self.k_v_proj, self.k_u_proj, self.v_v_proj, self.v_u_proj, self.o_v_proj,
+                self.o_u_proj)
+
     def _ensure_runtime_state(self) -> None:
         """Idempotent.  Packs [q_v; k_v; v_v] into one row-contiguous buffer (the module weights
         become views of it) so the three rank projections are a single weight stream."""
@@ -157,6 +161,9 @@ class SVD_LlamaAttention(nn.Module):
         for name in ("_dense_decode_prepacked_cache", "_dense_decode_backend_cache"):
             if not isinstance(getattr(self, name, None), dict):
                 setattr(self, name, {})
+        from .quant import is_quantized
+        if is_quantized(*self._factor_modules()):
+            return                      # int4 factors are read where they lie, nothing is packed
         mods = [self.q_v_proj, self.k_v_proj, self.v_v_proj]
         key = tuple((m.weight.data_ptr(), m.weight.dtype, m.weight.device) for m in mods)
         if self._packed_qkv_v is None or self._decode_ptrs != key:
@@ -274,15 +281,20 @@ class SVD_LlamaAttention(nn.Module):
             rope = cache.get_rope_tables(seqlen=cache.max_cache_len, head_dim=Dh, device=x.device, dtype=x.dtype)
         if nsplit is None:
             nsplit = hip_ops.pick_nsplit(cache.max_cache_len, B, H, Dh)
-        if self._dense_decode_backend(cache) == "exact":
+        from .quant import apply_linear, is_quantized
+        quantized = is_quantized(*self._factor_modules())
+        if quantized or self._dense_decode_backend(cache) == "exact":
             # module by module: three rank projections, three head expansions, rotary + append inside attention
+            # (the only form for int4 factors, whose bytes cannot be row-packed with their neighbours')
             xn = x if norm_weight is None else hip_ops.rmsnorm(x, norm_weight, eps)
-            q = hip_ops.linear(hip_ops.linear(xn, self.q_v_proj.weight), self.q_u_proj.weight).view(B, H, Dh)
-            k = hip_ops.linear(hip_ops.linear(xn, self.k_v_proj.weight), self.k_u_proj.weight).view(B, Hk, Dh)
-            v = hip_ops.linear(hip_ops.linear(xn, self.v_v_proj.weight), self.v_u_proj.weight).view(B, Hk, Dh)
+            q = apply_linear(self.q_u_proj, apply_linear(self.q_v_proj, xn)).view(B, H, Dh)
+            k = apply_linear(self.k_u_proj, apply_linear(self.k_v_proj, xn)).view(B, Hk, Dh)
+            v = apply_linear(self.v_u_proj, apply_linear(self.v_v_proj, xn)).view(B, Hk, Dh)
             a = hip_ops.attn_decode_densekv(q, kc[:B], vc[:B], positions, k_new=k, v_new=v, cos=rope[0], sin=rope[1],
                                             nsplit=nsplit, workspace=attn_ws)
             cache._layer_initialized[self.layer_idx] = True
+            po = apply_linear(self.o_v_proj, a.view(B, H * Dh))
+            return apply_linear(self.o_u_proj, po, residual=residual)
         else:
             p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)
             q = hip_ops.qkv_rope_append(p, self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight, rope[0], rope[1],
@@ -295,6 +307,9 @@ class SVD_LlamaAttention(nn.Module):
     def _decode_token_rank(self, x, cache, positions, *, norm_weight=None, eps=1e-6, residual=None, rope=None):
         """Rank-space cache: append Pk, Pv (pre-RoPE coefficients) and attend with in-kernel K rebuild."""
         from .kernels.rank_decode import rank_decode
+        from .quant import is_quantized
+        if is_quantized(*self._factor_modules()):
+            raise NotImplementedError("the rank-space cache reads bf16 head bases; int4 factors decode through the dense cache")
         B = x.shape[0]
         H, Hk, Dh = self.num_heads, self.num_key_value_heads, self.head_dim
         rq, rk, rv = self._qkv_rank_tuple()
@@ -366,7 +381,16 @@ class SVD_LlamaAttention(nn.Module):
         cache._ensure_layer_spec(self.layer_idx, h=Hk, dh=Dh)
         kc, vc = cache.key_cache[self.layer_idx], cache.value_cache[self.layer_idx]
         rope = cache.get_rope_tables(seqlen=cache.max_cache_len, head_dim=Dh, device=x.device, dtype=x.dtype)
-        p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)       # [B,T,Rtot]
+        from .quant import PackedQuantLinear, apply_linear, is_quantized
+        if is_quantized(*self._factor_modules()):
+            # int4 factors: rank projections module by module, head bases expanded to bf16 for this call
+            xn = x if norm_weight is None else hip_ops.rmsnorm(x, norm_weight, eps)
+            p = torch.cat([apply_linear(m, xn) for m in (self.q_v_proj, self.k_v_proj, self.v_v_proj)], dim=-1)
+            wq, wk, wv = (m.dequantize(dtype=x.dtype) if isinstance(m, PackedQuantLinear) else m.weight
+                          for m in (self.q_u_proj, self.k_u_proj, self.v_u_proj))
+        else:
+            p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)   # [B,T,Rtot]
+            wq, wk, wv = self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight
         rq, rk, rv = self._qkv_rank_tuple()
         mfma_ok = Dh == 128 and rq % 8 == 0 and rk % 8 == 0 and rv % 8 == 0 and T >= 16 \
             and os.getenv("FLASHSVD_AMD_PREFILL", "mfma").strip().lower() != "decode"
@@ -376,11 +400,11 @@ class SVD_LlamaAttention(nn.Module):
             # cache rows start..start+T-1), then causal flash attention over the cache
             pos0 = torch.full((B,), start, device=x.device, dtype=torch.int32)
             q = torch.empty(B, T, H, Dh, device=x.device, dtype=x.dtype)
-            hip_ops.lowrank_expand_heads(p[..., :rq], self.q_u_proj.weight, num_heads=H, head_dim=Dh, out=q,
+            hip_ops.lowrank_expand_heads(p[..., :rq], wq, num_heads=H, head_dim=Dh, out=q,
                                          cos=rope[0], sin=rope[1], positions=pos0)
-            hip_ops.lowrank_expand_heads(p[..., rq:rq + rk], self.k_u_proj.weight, num_heads=Hk, head_dim=Dh, out=kc[:B],
+            hip_ops.lowrank_expand_heads(p[..., rq:rq + rk], wk, num_heads=Hk, head_dim=Dh, out=kc[:B],
                                          cos=rope[0], sin=rope[1], positions=pos0, dst_by_position=True)
-            hip_ops.lowrank_expand_heads(p[..., rq + rk:], self.v_u_proj.weight, num_heads=Hk, head_dim=Dh, out=vc[:B],
+            hip_ops.lowrank_expand_heads(p[..., rq + rk:], wv, num_heads=Hk, head_dim=Dh, out=vc[:B],
                                          positions=pos0, dst_by_position=True)
             hip_ops.attn_prefill(q, kc[:B], vc[:B], q_pos0=pos0, causal=True, out=a.view(B, T, H, Dh))
         else:
@@ -388,13 +412,13 @@ class SVD_LlamaAttention(nn.Module):
             nsplit = hip_ops.pick_nsplit(cache.max_cache_len, T, H, Dh)
             for b in range(B):
                 kb, vb = kc[b:b + 1].expand(T, -1, -1, -1), vc[b:b + 1].expand(T, -1, -1, -1)
-                q = hip_ops.qkv_rope_append(p[b], self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight,
+                q = hip_ops.qkv_rope_append(p[b], wq, wk, wv,
                                             rope[0], rope[1], positions, kb, vb, num_heads=H, num_kv_heads=Hk, head_dim=Dh)
                 hip_ops.attn_decode_densekv(q, kb, vb, positions, seqlen_add=1, nsplit=nsplit, out=a[b].view(T, H, Dh))
         cache._layer_initialized[self.layer_idx] = True
         cache._note_seen(self.layer_idx, T, cache_position)
-        po = hip_ops.linear(a, self.o_v_proj.weight)
-        return hip_ops.linear(po, self.o_u_proj.weight, residual=residual)
+        po = apply_linear(self.o_v_proj, a)
+        return apply_linear(self.o_u_proj, po, residual=residual)
 
 
 def _prefill_tokens_rank(self, x, cache, cache_position=None, *, norm_weight=None, eps=1e-6, residual=None):
@@ -402,6 +426,9 @@ def _prefill_tokens_rank(self, x, cache, cache_position=None, *, norm_weight=Non
     then the tokens of a sequence are the kernel's batch rows bound to one cache row (batch stride 0)
     with key counts start+t+1.  K tiles are rebuilt once per query, so this is meant for short prompts."""
     from .kernels.rank_decode import rank_decode
+    from .quant import is_quantized
+    if is_quantized(*self._factor_modules()):
+        raise NotImplementedError("the rank-space cache reads bf16 head bases; int4 factors decode through the dense cache")
     B, T, d = x.shape
     H, Hk, Dh = self.num_heads, self.num_key_value_heads, self.head_dim
     rq, rk, rv = self._qkv_rank_tuple()
@@ -470,6 +497,12 @@ class SVD_LlamaMLP(nn.Module):
         self._packed_key = None
 
     def _ensure_runtime_state(self) -> None:
+        from .quant import is_quantized
+        for name in ("_flashsvd_graph_cache", "_flashsvd_layer_graph_cache"):
+            if not isinstance(getattr(self, name, None), dict):
+                setattr(self, name, {})
+        if is_quantized(*self._factor_modules()):
+            return                      # int4 factors are read where they lie, nothing is packed
         mods = [self.gate_v_proj, self.up_v_proj]
         key = tuple((m.weight.data_ptr(), m.weight.dtype, m.weight.device) for m in mods)
         if getattr(self, "_packed_gu_v", None) is None or self._packed_key != key:
@@ -481,8 +514,39 @@ class SVD_LlamaMLP(nn.Module):
             if not isinstance(getattr(self, name, None), dict):
                 setattr(self, name, {})
 
+    def _factor_modules(self):
+        return (self.gate_v_proj, self.gate_u_proj, self.up_v_proj, self.up_u_proj, self.down_v_proj, self.down_u_proj)
+
+    def _run_quantized(self, x: torch.Tensor, *, norm_weight=None, eps: float = 1e-6, residual=None, mode: Optional[int] = None):
+        """The same four stages with int4 factors: each projection through the kernel that fits its module."""
+        from .quant import PackedQuantLinear, apply_linear
+        gu, uu = self.gate_u_proj, self.up_u_proj
+        r = int(self.gate_v_proj.out_features)
+        if int(self.up_v_proj.out_features) != r:
+            raise ValueError("gate and up factors must share one rank")
+        xn = x if norm_weight is None else hip_ops.rmsnorm(x, norm_weight, eps)
+        p = torch.empty(*x.shape[:-1], 2 * r, device=x.device, dtype=x.dtype)
+        p2 = p.view(-1, 2 * r)
+        apply_linear(self.gate_v_proj, xn.reshape(-1, xn.shape[-1]), out=p2[:, :r])
+        apply_linear(self.up_v_proj, xn.reshape(-1, xn.shape[-1]), out=p2[:, r:])
+        mode = mlp_rounding_mode() if mode is None else mode
+        rows = p2.shape[0]
+        both_q = isinstance(gu, PackedQuantLinear) and isinstance(uu, PackedQuantLinear)
+        if both_q and gu.streams_int4(rows) and uu.streams_int4(rows) and gu.group_size == uu.group_size:
+            h = hip_ops.swiglu_linear_q4(p, (gu.qweight, gu.scales, gu.zeros), (uu.qweight, uu.scales, uu.zeros), up_off=r,
+                                         group_size=gu.group_size, mode=mode)
+        else:
+            wg = gu.dequantize(dtype=x.dtype) if isinstance(gu, PackedQuantLinear) else gu.weight
+            wu = uu.dequantize(dtype=x.dtype) if isinstance(uu, PackedQuantLinear) else uu.weight
+            h = hip_ops.swiglu_linear(p, wg, wu, up_off=r, mode=mode)
+        s = apply_linear(self.down_v_proj, h)
+        return apply_linear(self.down_u_proj, s, residual=residual)
+
     def run(self, x: torch.Tensor, *, norm_weight=None, eps: float = 1e-6, residual=None, mode: Optional[int] = None):
         """x [..., d] -> (residual +) down_u(down_v(silu(gate(x)) * up(x))); four weight streams."""
+        from .quant import is_quantized
+        if is_quantized(*self._factor_modules()):
+            return self._run_quantized(x, norm_weight=norm_weight, eps=eps, residual=residual, mode=mode)
         self._ensure_runtime_state()
         r = self.gate_v_proj.out_features
         p = hip_ops.linear(x, self._packed_gu_v, norm_weight=norm_weight, eps=eps)      # [.., 2R] = [PGate | PUp]

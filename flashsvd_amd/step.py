@@ -73,6 +73,10 @@ class PersistentDecoder:
         def tagged64(n):
             return torch.zeros(n, dtype=torch.int64, device=dev)
 
+        from .quant import is_quantized
+        for li, layer in enumerate(inner.layers):
+            if is_quantized(*layer.self_attn._factor_modules(), *layer.mlp._factor_modules()):
+                raise ValueError(f"PersistentDecoder streams bf16 factors; layer {li} holds int4 modules")
         # ranks may differ from layer to layer (buffers take the largest); within a layer q, k and v share
         # one rank because their head expansion is a single grouped product
         ranks = []

@@ -56,6 +56,27 @@ int fsvd_linear(const void* x, int64_t ldx, const void* W, int64_t ldw, const vo
 int fsvd_swiglu_linear(const void* p, int64_t ldp, int64_t up_off, const void* gate_u, const void* up_u,
                        int64_t ldw, void* h, int64_t ldh, int B, int D, int R, int mode, int cfg, void* stream);
 
+/* The same projection on group-wise int4 weights: y[b,n] = (res[b,n] +) bf16( sum_k norm(x)[b,k] * s[n,g(k)] *
+ * (q[n,k] - z[n,g(k)]) (+ bias[n]) ).  qweight [N, ldq] bytes holds two columns per byte (even column in the low
+ * nibble), scales fp16 and zeros int16 are [N, ldg] with one entry per group_size columns (a power of two >= 32;
+ * <= 0 means one group per row): the buffers of the reference's PackedQuantLinear as they are
+ * (src/quant/packed_quant_linear.py:18-26 packing, :126-172 quantisation, :284-299 dequantisation, :301-312 forward).
+ * The sum runs on the un-rounded s * (q - z) in fp32, which the reference rounds to the activation type first.
+ * K must be a multiple of 256; B rows go in slices of four. */
+int fsvd_linear_q4(const void* x, int64_t ldx, const void* qweight, int64_t ldq, const void* scales, const void* zeros,
+                   int64_t ldg, int group_size, const void* bias, const void* norm_w, float eps, const void* res,
+                   int64_t ldres, void* y, int64_t ldy, int B, int N, int K, void* stream);
+
+/* w[n,k] = bf16(s[n,g(k)] * (q[n,k] - z[n,g(k)])): PackedQuantLinear.dequantize for 4 bits and a bf16 result
+ * (src/quant/packed_quant_linear.py:284-299); any K and group size. */
+int fsvd_dequant_q4(const void* qweight, int64_t ldq, const void* scales, const void* zeros, int64_t ldg, int group_size,
+                    void* w, int64_t ldw, int N, int K, void* stream);
+
+/* fsvd_swiglu_linear on int4 gate_u / up_u [D, R] (same layout for both; rounding modes as above). */
+int fsvd_swiglu_linear_q4(const void* p, int64_t ldp, int64_t up_off, const void* gate_q, const void* gate_scales,
+                          const void* gate_zeros, const void* up_q, const void* up_scales, const void* up_zeros, int64_t ldq,
+                          int64_t ldg, int group_size, void* h, int64_t ldh, int B, int D, int R, int mode, void* stream);
+
 /* Current-token q/k/v from packed rank coefficients p[b] = [Pq|Pk|Pv] and nn.Linear-layout
  * u_proj weights, rotate-half RoPE on q and k at positions[b] (eager bf16 arithmetic), q to
  * q_out [B,H,Dh], k/v appended to the dense caches [B,S,Hk,Dh] at positions[b].

@@ -29,6 +29,9 @@ Pinning status (see tests/test_oracle_pins.py):
   dual_split_mlp             closed form, D-tile partition invariance, HF LlamaMLP
   LowRankLlama (block/model) transformers LlamaForCausalLM built from W = U @ V
   greedy_decode              cached decode == full-sequence recompute
+  pack_int4 / quantize_weight / dequantize_weight / quant_linear
+                             hand-worked vectors, pack/unpack round trip, |w - dequant| <= scale/2,
+                             symmetric zero point, all-zero group, fp64 closed form of the linear
 parity unpinned (source absent from the reference checkout, behaviour defined here):
   the op order / rounding points of models/llama.py (SVD_LlamaAttention.forward,
   SVD_LlamaMLP.forward) and the bit-level behaviour of flash-attn 2.8.3.
@@ -575,6 +578,74 @@ def greedy_decode(mw: ModelWeights, prompt: torch.Tensor, n_new: int, cache_kind
     if return_logits:
         return out, torch.stack(hiddens, dim=1), cache, torch.stack(all_logits, dim=1)
     return (out, torch.stack(hiddens, dim=1), cache) if return_hidden else out
+
+
+# ----------------------------------------------------------------------------
+# group-wise int4 / int8 weights (src/quant/packed_quant_linear.py)
+# ----------------------------------------------------------------------------
+def pack_int4(q: torch.Tensor) -> torch.Tensor:
+    """[N, K] values 0..15 -> [N, ceil(K/2)] bytes, even column in the low nibble.
+    src/quant/packed_quant_linear.py:18-26."""
+    q = q.to(torch.uint8)
+    if q.shape[1] % 2:
+        q = torch.cat([q, torch.zeros((q.shape[0], 1), dtype=torch.uint8)], dim=1)
+    return (q[:, 0::2] & 0x0F) | ((q[:, 1::2] & 0x0F) << 4)
+
+
+def unpack_int4(packed: torch.Tensor, in_features: int) -> torch.Tensor:
+    """src/quant/packed_quant_linear.py:29-36."""
+    out = torch.empty((packed.shape[0], packed.shape[1] * 2), dtype=torch.uint8)
+    out[:, 0::2] = packed & 0x0F
+    out[:, 1::2] = (packed >> 4) & 0x0F
+    return out[:, :in_features]
+
+
+def quantize_weight(weight: torch.Tensor, *, bits: int = 4, group_size: int = 128, sym: bool = False):
+    """Min/max group quantisation of an nn.Linear weight [N, K] along K.
+    Returns (qweight uint8 [N, K/2] for 4 bits or [N, K] for 8, scales fp16 [N, G], zeros int16 [N, G]);
+    w ~= scale * (q - zero).  An all-zero group is given the range [-1, 1]; ``sym`` centres the range and fixes
+    zero = 2^(bits-1).  src/quant/packed_quant_linear.py:126-172."""
+    w = weight.detach().to(torch.float32)
+    N, K = w.shape
+    group = K if group_size <= 0 else int(group_size)
+    maxq = float((1 << bits) - 1)
+    qs, ss, zs = [], [], []
+    for g0 in range(0, K, group):
+        chunk = w[:, g0:min(K, g0 + group)]
+        xmin, xmax = chunk.min(dim=1).values, chunk.max(dim=1).values
+        if sym:
+            xmax = torch.maximum(xmax.abs(), xmin.abs())
+            xmin = -xmax
+        dead = (xmin == 0) & (xmax == 0)
+        xmin = torch.where(dead, torch.full_like(xmin, -1.0), xmin)
+        xmax = torch.where(dead, torch.full_like(xmax, 1.0), xmax)
+        scale = (xmax - xmin) / maxq
+        scale = torch.where(scale == 0, torch.ones_like(scale), scale)
+        zero = torch.full_like(scale, int((maxq + 1) / 2)) if sym else torch.round(-xmin / scale)
+        qs.append(torch.clamp(torch.round(chunk / scale.unsqueeze(1)) + zero.unsqueeze(1), 0, maxq).to(torch.uint8))
+        ss.append(scale.to(torch.float16))
+        zs.append(zero.to(torch.int16))
+    q = torch.cat(qs, dim=1).contiguous()
+    return (pack_int4(q) if bits == 4 else q), torch.stack(ss, dim=1).contiguous(), torch.stack(zs, dim=1).contiguous()
+
+
+def dequantize_weight(qweight, scales, zeros, *, in_features: int, bits: int = 4, group_size: int = 128,
+                      dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """scale * (q - zero) in fp32, then ONE rounding to ``dtype``.  src/quant/packed_quant_linear.py:284-299."""
+    q = (unpack_int4(qweight, in_features) if bits == 4 else qweight).to(torch.float32)
+    group = in_features if group_size <= 0 else int(group_size)
+    cols = []
+    for gi in range(scales.shape[1]):
+        g0, g1 = gi * group, min(in_features, (gi + 1) * group)
+        cols.append(scales[:, gi].float().unsqueeze(1) * (q[:, g0:g1] - zeros[:, gi].float().unsqueeze(1)))
+    return torch.cat(cols, dim=1).to(dtype)
+
+
+def quant_linear(x, qweight, scales, zeros, bias=None, *, bits: int = 4, group_size: int = 128) -> torch.Tensor:
+    """The module's reference forward: dequantise to the activation dtype, then an ordinary linear.
+    src/quant/packed_quant_linear.py:301-312."""
+    w = dequantize_weight(qweight, scales, zeros, in_features=x.shape[-1], bits=bits, group_size=group_size, dtype=x.dtype)
+    return lin(x, w, bias)
 
 
 # ----------------------------------------------------------------------------

@@ -306,3 +306,63 @@ def test_rank_cache_and_dense_cache_agree_bf16():
     _, hd, _ = O.greedy_decode(mw, prompt, 4, "dense", return_hidden=True)
     _, hr, _ = O.greedy_decode(mw, prompt, 4, "rank", return_hidden=True)
     assert (hd.float() - hr.float()).abs().max() < 0.15  # bf16 noise only; same algebra
+
+
+# ---- group-wise int4 weights (src/quant/packed_quant_linear.py) --------------------------------
+def test_int4_pack_layout_by_hand():
+    q = torch.tensor([[1, 2, 3, 15, 0, 7, 9]], dtype=torch.uint8)            # odd length: one padding nibble
+    packed = O.pack_int4(q)
+    assert packed.tolist() == [[0x21, 0xF3, 0x70, 0x09]]                       # even column low nibble, odd column high
+    assert O.unpack_int4(packed, 7).tolist() == q.tolist()
+    g = torch.Generator().manual_seed(0)
+    q = torch.randint(0, 16, (5, 64), generator=g, dtype=torch.uint8)
+    assert torch.equal(O.unpack_int4(O.pack_int4(q), 64), q)
+
+
+def test_int4_quantize_by_hand():
+    # one row, two groups of 4.  group 0: min -1.5, max 6 -> scale 0.5, zero = round(3) = 3
+    # group 1: all zero -> range [-1, 1]: scale 2/15, zero = round(1 / fp32(2/15)) = round(7.4999996) = 7
+    w = torch.tensor([[-1.5, 0.0, 6.0, 2.26, 0.0, 0.0, 0.0, 0.0]])
+    qw, sc, zr = O.quantize_weight(w, bits=4, group_size=4, sym=False)
+    assert sc.dtype == torch.float16 and zr.dtype == torch.int16 and qw.dtype == torch.uint8
+    assert sc.tolist() == [[0.5, float(torch.tensor(2 / 15).half())]] and zr.tolist() == [[3, 7]]
+    assert O.unpack_int4(qw, 8).tolist() == [[0, 3, 15, 8, 7, 7, 7, 7]]        # 2.26/0.5 = 4.52 -> 5, + 3
+    deq = O.dequantize_weight(qw, sc, zr, in_features=8, group_size=4)
+    assert deq.tolist() == [[-1.5, 0.0, 6.0, 2.5, 0.0, 0.0, 0.0, 0.0]]
+    # symmetric: zero point 8, scale = 2*max|w|/15, clamp keeps q within 0..15
+    qw, sc, zr = O.quantize_weight(w, bits=4, group_size=-1, sym=True)
+    assert zr.tolist() == [[8]] and sc.shape == (1, 1) and float(sc[0, 0]) == float(torch.tensor(12 / 15).half())
+    assert O.unpack_int4(qw, 8).tolist() == [[6, 8, 15, 11, 8, 8, 8, 8]]       # 6/0.8 = 7.5 -> 8 (even) + 8 = 16 -> clamp 15
+    # 8 bits keep one byte per weight
+    qw8, sc8, zr8 = O.quantize_weight(w, bits=8, group_size=4)
+    assert qw8.shape == (1, 8) and int(qw8.max()) == 255 and int(qw8.min()) == 0
+
+
+def test_int4_round_trip_error_bound_and_linear_closed_form():
+    g = torch.Generator().manual_seed(1)
+    w = torch.randn(24, 96, generator=g) * 0.05
+    for group, sym in ((32, False), (32, True), (-1, False), (40, False)):       # 40: ragged last group
+        qw, sc, zr = O.quantize_weight(w, group_size=group, sym=sym)
+        G = 1 if group <= 0 else -(-96 // group)
+        assert sc.shape == (24, G) and zr.shape == (24, G) and qw.shape == (24, 48)
+        deq = O.dequantize_weight(qw, sc, zr, in_features=96, group_size=group)
+        width = 96 if group <= 0 else group
+        bound = sc.float().repeat_interleave(width, dim=1)[:, :96]
+        # rounding to the grid costs at most half a step; the scale is stored in fp16 (2^-11 relative) and
+        # multiplies a level distance |q - z| of at most 15
+        assert bool(((w - deq).abs() <= bound * (0.5 + 15 * 2 ** -11) * (1 + 2 ** -10) + 1e-7).all()), (group, sym)
+    # the linear is x @ (s * (q - z))^T: check against float64 arithmetic written out element by element
+    qw, sc, zr = O.quantize_weight(w, group_size=32)
+    x = torch.randn(3, 96, generator=g)
+    y = O.quant_linear(x, qw, sc, zr, group_size=32)
+    q = O.unpack_int4(qw, 96).double()
+    ref = torch.zeros(3, 24, dtype=torch.float64)
+    for n in range(24):
+        for k in range(96):
+            ref[:, n] += x[:, k].double() * (sc[n, k // 32].double() * (q[n, k] - zr[n, k // 32].double()))
+    assert torch.allclose(y.double(), ref, rtol=1e-5, atol=1e-6)
+    # bf16 activations: the dequantised weight is rounded to bf16 before the product
+    xb = x.to(torch.bfloat16)
+    yb = O.quant_linear(xb, qw, sc, zr, group_size=32)
+    wb = O.dequantize_weight(qw, sc, zr, in_features=96, group_size=32, dtype=torch.bfloat16)
+    assert yb.dtype == torch.bfloat16 and torch.equal(yb, (xb.float() @ wb.float().t()).to(torch.bfloat16))
