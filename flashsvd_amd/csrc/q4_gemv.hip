@@ -47,6 +47,41 @@ __device__ __forceinline__ float dot32_q4(const u32x4_t& q, const u32x4_t* xs) {
   return acc;
 }
 
+// NU pieces per thread of matrix m, starting at item i0: all loads first, then the products
+template <int BATCH, int NU>
+__device__ __forceinline__ void q4_trip(const Q4Args& a, int m, int i0, int items, int r0, int PPR, int K, int nchunk,
+                                        uint32_t ppr_magic, int gshift, const uint16_t* xs, const float* xsum, float* cp) {
+  const int tid = threadIdx.x;
+  const uint8_t* qw = a.qw[m];
+  const uint16_t* sc = a.sc[m];
+  const int16_t* zr = a.zr[m];
+  u32x4_t q[NU];
+  float s[NU], zz[NU];
+  int piece[NU];
+#pragma unroll
+  for (int u = 0; u < NU; ++u) {
+    const int i = min(i0 + u * kQT + tid, items - 1);
+    const int row = (int)__umulhi((uint32_t)i, ppr_magic);
+    piece[u] = i - row * PPR;
+    const int64_t n = r0 + row;
+    q[u] = __builtin_nontemporal_load((q4_gptr_t)(uintptr_t)(qw + n * a.ldq + (int64_t)piece[u] * 16));
+    const int64_t gi = n * a.ldg + (piece[u] >> gshift);
+    s[u] = half_bits_to_f32(sc[gi]);
+    zz[u] = (float)((int)zr[gi] + 128);
+  }
+#pragma unroll
+  for (int u = 0; u < NU; ++u) {
+    const int i = i0 + u * kQT + tid;
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const size_t xo = (size_t)m * BATCH + b;
+      const float d = dot32_q4(q[u], reinterpret_cast<const u32x4_t*>(xs + xo * K + (size_t)piece[u] * 32));
+      const float part = row8_sum(s[u] * (d - zz[u] * xsum[xo * PPR + piece[u]]));
+      if ((tid & 7) == 0 && i < items) cp[xo * nchunk + (i >> 3)] = part;
+    }
+  }
+}
+
 // BATCH activation rows, NMAT = 1 (linear) or 2 (gate and up of the SwiGLU, each with its own input)
 template <int BATCH, int NMAT>
 __global__ __launch_bounds__(kQT) void q4_linear_kernel(Q4Args a, int rows_per_wg, uint32_t ppr_magic, int gshift) {
@@ -129,36 +164,11 @@ __global__ __launch_bounds__(kQT) void q4_linear_kernel(Q4Args a, int rows_per_w
   const int items = nrows * PPR;
 #pragma unroll
   for (int m = 0; m < NMAT; ++m) {
-    const uint8_t* qw = a.qw[m];
-    const uint16_t* sc = a.sc[m];
-    const int16_t* zr = a.zr[m];
-    for (int i0 = 0; i0 < items; i0 += kQT * kQUnroll) {
-      u32x4_t q[kQUnroll];
-      float s[kQUnroll], zz[kQUnroll];
-      int piece[kQUnroll];
-#pragma unroll
-      for (int u = 0; u < kQUnroll; ++u) {
-        const int i = min(i0 + u * kQT + tid, items - 1);
-        const int row = (int)__umulhi((uint32_t)i, ppr_magic);
-        piece[u] = i - row * PPR;
-        const int64_t n = r0 + row;
-        q[u] = __builtin_nontemporal_load((q4_gptr_t)(uintptr_t)(qw + n * a.ldq + (int64_t)piece[u] * 16));
-        const int64_t gi = n * a.ldg + (piece[u] >> gshift);
-        s[u] = half_bits_to_f32(sc[gi]);
-        zz[u] = (float)((int)zr[gi] + 128);
-      }
-#pragma unroll
-      for (int u = 0; u < kQUnroll; ++u) {
-        const int i = i0 + u * kQT + tid;
-#pragma unroll
-        for (int b = 0; b < BATCH; ++b) {
-          const size_t xo = (size_t)m * BATCH + b;
-          const float d = dot32_q4(q[u], reinterpret_cast<const u32x4_t*>(xs + xo * K + (size_t)piece[u] * 32));
-          const float part = row8_sum(s[u] * (d - zz[u] * xsum[xo * PPR + piece[u]]));
-          if ((tid & 7) == 0 && i < items) cp[xo * nchunk + (i >> 3)] = part;
-        }
-      }
-    }
+    int i0 = 0;
+    for (; i0 + kQT * kQUnroll <= items; i0 += kQT * kQUnroll)     // full trips: kQUnroll pieces in flight per thread
+      q4_trip<BATCH, kQUnroll>(a, m, i0, items, r0, PPR, K, nchunk, ppr_magic, gshift, xs, xsum, cp);
+    for (; i0 < items; i0 += kQT)                                  // tail: one piece per thread
+      q4_trip<BATCH, 1>(a, m, i0, items, r0, PPR, K, nchunk, ppr_magic, gshift, xs, xsum, cp);
   }
   __syncthreads();
 

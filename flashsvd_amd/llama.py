@@ -161,9 +161,15 @@ class SVD_LlamaAttention(nn.Module):
         for name in ("_dense_decode_prepacked_cache", "_dense_decode_backend_cache"):
             if not isinstance(getattr(self, name, None), dict):
                 setattr(self, name, {})
-        from .quant import is_quantized
+        from .quant import is_quantized, pack_quant_rows
         if is_quantized(*self._factor_modules()):
-            return                      # int4 factors are read where they lie, nothing is packed
+            # int4 factors: the three rank projections share their input, so their rows are packed into one stream
+            mods = [self.q_v_proj, self.k_v_proj, self.v_v_proj]
+            key = tuple(m.qweight.data_ptr() if is_quantized(m) else m.weight.data_ptr() for m in mods)
+            if getattr(self, "_q4_key", None) != key:
+                self._q4_qkv_v = pack_quant_rows(mods)
+                self._q4_key = tuple(m.qweight.data_ptr() if is_quantized(m) else m.weight.data_ptr() for m in mods)
+            return
         mods = [self.q_v_proj, self.k_v_proj, self.v_v_proj]
         key = tuple((m.weight.data_ptr(), m.weight.dtype, m.weight.device) for m in mods)
         if self._packed_qkv_v is None or self._decode_ptrs != key:
@@ -286,10 +292,17 @@ class SVD_LlamaAttention(nn.Module):
         if quantized or self._dense_decode_backend(cache) == "exact":
             # module by module: three rank projections, three head expansions, rotary + append inside attention
             # (the only form for int4 factors, whose bytes cannot be row-packed with their neighbours')
-            xn = x if norm_weight is None else hip_ops.rmsnorm(x, norm_weight, eps)
-            q = apply_linear(self.q_u_proj, apply_linear(self.q_v_proj, xn)).view(B, H, Dh)
-            k = apply_linear(self.k_u_proj, apply_linear(self.k_v_proj, xn)).view(B, Hk, Dh)
-            v = apply_linear(self.v_u_proj, apply_linear(self.v_v_proj, xn)).view(B, Hk, Dh)
+            pk = getattr(self, "_q4_qkv_v", None) if quantized else None
+            if pk is not None and self.q_v_proj.streams_int4(B):
+                rq, rk, rv = self._qkv_rank_tuple()
+                p = hip_ops.linear_q4(x, *pk, group_size=self.q_v_proj.group_size, norm_weight=norm_weight, eps=eps)
+                pq, pkk, pv = p[:, :rq], p[:, rq:rq + rk], p[:, rq + rk:]
+            else:
+                xn = x if norm_weight is None else hip_ops.rmsnorm(x, norm_weight, eps)
+                pq, pkk, pv = (apply_linear(m, xn) for m in (self.q_v_proj, self.k_v_proj, self.v_v_proj))
+            q = apply_linear(self.q_u_proj, pq).view(B, H, Dh)
+            k = apply_linear(self.k_u_proj, pkk).view(B, Hk, Dh)
+            v = apply_linear(self.v_u_proj, pv).view(B, Hk, Dh)
             a = hip_ops.attn_decode_densekv(q, kc[:B], vc[:B], positions, k_new=k, v_new=v, cos=rope[0], sin=rope[1],
                                             nsplit=nsplit, workspace=attn_ws)
             cache._layer_initialized[self.layer_idx] = True
@@ -502,7 +515,13 @@ class SVD_LlamaMLP(nn.Module):
             if not isinstance(getattr(self, name, None), dict):
                 setattr(self, name, {})
         if is_quantized(*self._factor_modules()):
-            return                      # int4 factors are read where they lie, nothing is packed
+            from .quant import pack_quant_rows
+            mods = [self.gate_v_proj, self.up_v_proj]
+            key = tuple(m.qweight.data_ptr() if is_quantized(m) else m.weight.data_ptr() for m in mods)
+            if getattr(self, "_q4_key", None) != key:
+                self._q4_gu_v = pack_quant_rows(mods)       # gate and up rank projections as one int4 stream
+                self._q4_key = tuple(m.qweight.data_ptr() if is_quantized(m) else m.weight.data_ptr() for m in mods)
+            return
         mods = [self.gate_v_proj, self.up_v_proj]
         key = tuple((m.weight.data_ptr(), m.weight.dtype, m.weight.device) for m in mods)
         if getattr(self, "_packed_gu_v", None) is None or self._packed_key != key:
@@ -524,13 +543,18 @@ class SVD_LlamaMLP(nn.Module):
         r = int(self.gate_v_proj.out_features)
         if int(self.up_v_proj.out_features) != r:
             raise ValueError("gate and up factors must share one rank")
-        xn = x if norm_weight is None else hip_ops.rmsnorm(x, norm_weight, eps)
-        p = torch.empty(*x.shape[:-1], 2 * r, device=x.device, dtype=x.dtype)
-        p2 = p.view(-1, 2 * r)
-        apply_linear(self.gate_v_proj, xn.reshape(-1, xn.shape[-1]), out=p2[:, :r])
-        apply_linear(self.up_v_proj, xn.reshape(-1, xn.shape[-1]), out=p2[:, r:])
+        self._ensure_runtime_state()
+        rows = x.numel() // x.shape[-1]
+        pk = getattr(self, "_q4_gu_v", None)
+        if pk is not None and self.gate_v_proj.streams_int4(rows):
+            p = hip_ops.linear_q4(x, *pk, group_size=self.gate_v_proj.group_size, norm_weight=norm_weight, eps=eps)
+        else:
+            xn = x if norm_weight is None else hip_ops.rmsnorm(x, norm_weight, eps)
+            p = torch.empty(*x.shape[:-1], 2 * r, device=x.device, dtype=x.dtype)
+            p2 = p.view(-1, 2 * r)
+            apply_linear(self.gate_v_proj, xn.reshape(-1, xn.shape[-1]), out=p2[:, :r])
+            apply_linear(self.up_v_proj, xn.reshape(-1, xn.shape[-1]), out=p2[:, r:])
         mode = mlp_rounding_mode() if mode is None else mode
-        rows = p2.shape[0]
         both_q = isinstance(gu, PackedQuantLinear) and isinstance(uu, PackedQuantLinear)
         if both_q and gu.streams_int4(rows) and uu.streams_int4(rows) and gu.group_size == uu.group_size:
             h = hip_ops.swiglu_linear_q4(p, (gu.qweight, gu.scales, gu.zeros), (uu.qweight, uu.scales, uu.zeros), up_off=r,

@@ -181,6 +181,41 @@ def apply_linear(mod: nn.Module, x: torch.Tensor, *, norm_weight=None, eps: floa
     return hip_ops.linear(x, mod.weight, getattr(mod, "bias", None), norm_weight=norm_weight, eps=eps, residual=residual, out=out)
 
 
+def pack_quant_rows(mods) -> Optional[tuple]:
+    """(qweight, scales, zeros) with the rows of all ``mods`` one below the other, so that projections sharing their input
+    are one weight stream; the modules' buffers become row slices of the packed tensors (no second copy).  None when the
+    modules cannot share a launch (mixed types, widths, group sizes, or a bias)."""
+    mods = list(mods)
+    if not mods or not all(isinstance(m, PackedQuantLinear) for m in mods):
+        return None
+    m0 = mods[0]
+    if m0.bits != 4 or any(m.bits != 4 or m.in_features != m0.in_features or m.group_size != m0.group_size or m.bias is not None
+                           or m.qweight.device != m0.qweight.device for m in mods):
+        return None
+    packed = []
+    for name in ("qweight", "scales", "zeros"):
+        parts = [getattr(m, name) for m in mods]
+        base, row, shared = parts[0], 0, True
+        for t in parts:
+            if t.untyped_storage().data_ptr() != base.untyped_storage().data_ptr() or not t.is_contiguous() or \
+                    t.storage_offset() != base.storage_offset() + row * base.shape[1]:
+                shared = False
+                break
+            row += t.shape[0]
+        if shared:
+            packed.append(torch.as_strided(base, (row, base.shape[1]), (base.shape[1], 1), base.storage_offset()))
+            continue
+        cat = torch.cat(parts, dim=0).contiguous()
+        row = 0
+        for m, t in zip(mods, parts):
+            setattr(m, name, cat[row:row + t.shape[0]])
+            row += t.shape[0]
+        packed.append(cat)
+    for m in mods:
+        m._dense = None
+    return tuple(packed)
+
+
 def is_quantized(*mods) -> bool:
     return any(isinstance(m, PackedQuantLinear) for m in mods)
 
