@@ -443,6 +443,13 @@ int fsvd_decode_step_prepare(fsvd_phase* phases_host, int nphase, int workgroups
   return prepare_decode_step(phases_host, nphase, workgroups);
 }
 
+int fsvd_decode_step_validate(const fsvd_phase* phases_host, int nphase, int workgroups) {
+  const char* fn = "fsvd_decode_step_validate";
+  FSVD_REQUIRE_PTR(phases_host, fn);
+  if (nphase <= 0 || workgroups <= 0) { set_last_error("%s: bad arguments", fn); return kErrBadShape; }
+  return validate_decode_step(phases_host, nphase, workgroups);
+}
+
 int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase, fsvd_step_state* state,
                      int validate, void* stream) {
   const char* fn = "fsvd_decode_step";

@@ -145,6 +145,9 @@ def pad_mlp_ranks(mlp, multiple: int = 1, *, _shared: Optional[dict] = None) -> 
         pad_factor_pair(getattr(mlp, f"{p}_v_proj"), getattr(mlp, f"{p}_u_proj"), t, _shared)
     mlp._packed_gu_v = None
     mlp._packed_key = None
+    for name in ("_flashsvd_graph_cache", "_flashsvd_layer_graph_cache"):     # captured graphs point at the old weights
+        if isinstance(getattr(mlp, name, None), dict):
+            getattr(mlp, name).clear()
     return {"gate": (rg, tg), "up": (ru, tu), "down": (rd, td)}
 
 

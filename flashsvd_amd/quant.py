@@ -287,4 +287,7 @@ def replace_linears_with_packed_quant_inplace(model: nn.Module, *, module_names:
         if hasattr(layer.mlp, "_packed_gu_v"):
             layer.mlp._packed_gu_v = None
             layer.mlp._packed_key = None
+        for name in ("_flashsvd_graph_cache", "_flashsvd_layer_graph_cache"):  # captured graphs point at the old weights
+            if isinstance(getattr(layer.mlp, name, None), dict):
+                getattr(layer.mlp, name).clear()
     return replaced

@@ -182,6 +182,8 @@ class PersistentDecoder:
         self.nph = len(ph)
         self.host_phases = (Phase * self.nph)(*ph)
         _lib.check("fsvd_decode_step_prepare", lib.fsvd_decode_step_prepare(ctypes.addressof(self.host_phases), self.nph, self.nwg))
+        # reject a model the kernel cannot run here, not at the first step (the driver then takes the other engine)
+        _lib.check("fsvd_decode_step_validate", lib.fsvd_decode_step_validate(ctypes.addressof(self.host_phases), self.nph, self.nwg))
         raw = bytes(self.host_phases)
         self.dev_phases = torch.frombuffer(bytearray(raw), dtype=torch.uint8).to(dev)
         self._validated = False

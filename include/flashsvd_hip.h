@@ -290,6 +290,8 @@ typedef struct fsvd_step_state {
 int fsvd_decode_step_workgroups(void);
 /* Fill the derived fields of a host-side phase list for `workgroups` workgroups (call before uploading it). */
 int fsvd_decode_step_prepare(fsvd_phase* phases_host, int nphase, int workgroups);
+/* The host-side check of fsvd_decode_step alone (no launch): 0, or a negative status with fsvd_last_error(). */
+int fsvd_decode_step_validate(const fsvd_phase* phases_host, int nphase, int workgroups);
 /* phases_dev: the list in device memory; phases_host: the same list in host memory (validated on every
  * call unless validate == 0); state: device.  Launch is asynchronous on `stream`. */
 int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase,
