@@ -133,6 +133,18 @@ struct PrefillAttnArgs {
 int launch_expand(const ExpandArgs& a, hipStream_t st);
 int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st);
 
+// matrix-core projections: y = epilogue(x . W^T) with the rounding points of the vector kernels
+struct MfmaArgs {
+  const uint16_t* x; int64_t ldx;            // [B, >= K] activations; DUAL: gate input at 0, up input at up_off
+  int64_t up_off;
+  const uint16_t* W; const uint16_t* W2; int64_t ldw;   // [N, K] (DUAL: gate_u, up_u)
+  const uint16_t* bias; const uint16_t* res; int64_t ldres;
+  uint16_t* y; int64_t ldy;
+  int B, N, K, mode;
+};
+bool gemm_tiles_apply(const MfmaArgs& a);                                   // mfma_gemm.hip: 128 rows and more
+int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* who);
+
 int launch_linear(const LinearArgs& a, int cfg, hipStream_t st);
 // matrix-core path for 5+ rows (mfma_gemv.hip); launch_linear / launch_swiglu route to it when cfg == 0
 bool mfma_linear_applies(const LinearArgs& a);

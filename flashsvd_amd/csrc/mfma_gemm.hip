@@ -1,0 +1,185 @@
+// Prefill projections: y[M, N] = epilogue(x[M, K] . W[N, K]^T) for 128 rows and more, on the matrix cores.
+//
+// Both operands are K-contiguous, which is the layout V_MFMA_F32_16X16X32_BF16 wants for its two inputs (each lane
+// holds 8 consecutive k of one row).  A workgroup of four waves owns a 128 x 128 output tile (a wave 64 x 64: 4 x 4
+// accumulator tiles), walks K in steps of 64 through a double-buffered LDS stage (rows padded to 72 elements so that
+// the 16-byte fragment reads of 16 consecutive rows fall on different banks) and overlaps the global loads of step
+// k + 1 with the products of step k.  Epilogue as in the vector kernels: bias, ONE rounding to bf16, residual — or,
+// for the gate / up pair, SwiGLU in either rounding mode.  Every weight is read once per 128 rows of x.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace fsvd {
+
+typedef __bf16 gm_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float gm_f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kGT = 256;            // threads: 2 x 2 waves
+constexpr int kGBK = 64;
+constexpr int kGLd = kGBK + 8;      // LDS row stride in elements (144 bytes)
+
+// WT: 16 x 16 accumulator tiles per wave and dimension: 4 -> 128 x 128 per workgroup, 2 -> 64 x 64 (problems with
+// few output tiles, where more workgroups matter more than reuse)
+template <bool DUAL, int WT, int PF>
+__global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a) {
+  constexpr int NM = DUAL ? 2 : 1;
+  constexpr int kGBM = 32 * WT, kGBN = 32 * WT;
+  extern __shared__ __align__(16) unsigned char gm_smem[];
+  // [stage][operand: x0, (x1), W0, (W1)][128 rows][kGLd]
+  uint16_t* lds = reinterpret_cast<uint16_t*>(gm_smem);
+  constexpr int kTile = kGBM * kGLd;                 // elements per operand tile
+  constexpr int kStage = 2 * NM * kTile;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * kGBM, n0 = blockIdx.x * kGBN;
+  const int ksteps = a.K / kGBK;
+
+  // global -> register staging: a tile row is 128 bytes = 8 16-byte pieces; WT pieces per thread and operand
+  const int ld_row = tid >> 3, ld_chunk = tid & 7;   // rows ld_row + 32 * j, j = 0..WT-1
+  const uint16_t* gx[NM][WT];
+  const uint16_t* gw[NM][WT];
+#pragma unroll
+  for (int j = 0; j < WT; ++j) {
+    const int64_t xr = min(m0 + ld_row + 32 * j, a.B - 1), wr = min(n0 + ld_row + 32 * j, a.N - 1);
+    gx[0][j] = a.x + xr * a.ldx + ld_chunk * 8;
+    gw[0][j] = a.W + wr * a.ldw + ld_chunk * 8;
+    if (DUAL) {
+      gx[NM - 1][j] = a.x + xr * a.ldx + a.up_off + ld_chunk * 8;
+      gw[NM - 1][j] = a.W2 + wr * a.ldw + ld_chunk * 8;
+    }
+  }
+  // PF register sets hold the global loads of the next PF steps (set s % PF belongs to step s); a set is written
+  // to the idle LDS stage one step before its products and refilled at once with the loads of step s + PF
+  u32x4_t rx[PF][NM][WT], rw[PF][NM][WT];
+  auto load_regs = [&](int set, int ks) {
+    const int k = min(ks, ksteps - 1) * kGBK;        // past the end: a valid address, never used
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+      for (int j = 0; j < WT; ++j) {
+        rx[set][m][j] = *reinterpret_cast<const u32x4_t*>(gx[m][j] + k);
+        rw[set][m][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(gw[m][j] + k));
+      }
+  };
+  auto store_lds = [&](int set, int stage) {
+    uint16_t* base = lds + stage * kStage;
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+      for (int j = 0; j < WT; ++j) {
+        const int off = (ld_row + 32 * j) * kGLd + ld_chunk * 8;
+        *reinterpret_cast<u32x4_t*>(base + m * kTile + off) = rx[set][m][j];
+        *reinterpret_cast<u32x4_t*>(base + (NM + m) * kTile + off) = rw[set][m][j];
+      }
+  };
+
+  gm_f32x4_t acc[NM][WT][WT];
+#pragma unroll
+  for (int m = 0; m < NM; ++m)
+#pragma unroll
+    for (int i = 0; i < WT; ++i)
+#pragma unroll
+      for (int j = 0; j < WT; ++j) acc[m][i][j] = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int u = 0; u < PF; ++u) load_regs(u, u);
+  store_lds(0, 0);
+  load_regs(0, PF);
+  __syncthreads();
+  for (int ks0 = 0; ks0 < ksteps; ks0 += PF) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      const int ks = ks0 + u;
+      if (ks >= ksteps) break;
+      const uint16_t* base = lds + (ks & 1) * kStage;
+#pragma unroll
+      for (int kk = 0; kk < kGBK / 32; ++kk) {
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+          gm_bf16x8_t fx[WT], fw[WT];
+#pragma unroll
+          for (int i = 0; i < WT; ++i) {
+            fx[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + m * kTile + (wm * 16 * WT + i * 16 + lr) * kGLd + kk * 32 + lg * 8);
+            fw[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + (NM + m) * kTile + (wn * 16 * WT + i * 16 + lr) * kGLd + kk * 32 + lg * 8);
+          }
+#pragma unroll
+          for (int i = 0; i < WT; ++i)
+#pragma unroll
+            for (int j = 0; j < WT; ++j)
+              acc[m][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fx[i], fw[j], acc[m][i][j], 0, 0, 0);
+        }
+      }
+      if (ks + 1 < ksteps) {
+        // the other stage was last read before the barrier that ended step ks - 1
+        store_lds((u + 1) % PF, (ks + 1) & 1);
+        load_regs((u + 1) % PF, ks + 1 + PF);
+        __syncthreads();
+      }
+    }
+  }
+
+  // element e of lane l of tile (i, j): row m = i*16 + (l/16)*4 + e of x, column n = j*16 + l%16 of W
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int m = m0 + wm * 16 * WT + i * 16 + lg * 4 + e;
+      if (m >= a.B) continue;
+#pragma unroll
+      for (int j = 0; j < WT; ++j) {
+        const int n = n0 + wn * 16 * WT + j * 16 + lr;
+        if (n >= a.N) continue;
+        float v0 = acc[0][i][j][e];
+        float v;
+        if (DUAL) {
+          float v1 = acc[NM - 1][i][j][e];
+          if (a.mode == 0) {
+            v0 = round_bf16(v0);
+            v1 = round_bf16(v1);
+            v = round_bf16(round_bf16(silu_f32(v0)) * v1);
+          } else {
+            v = round_bf16((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
+          }
+        } else {
+          if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
+          v = round_bf16(v0);
+          if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)m * a.ldres + n]) + v);
+        }
+        a.y[(int64_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+      }
+    }
+}
+
+bool gemm_tiles_apply(const MfmaArgs& a) {
+  return a.B >= 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0;
+}
+
+template <bool DUAL, int WT>
+static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* who) {
+  static bool granted = false;
+  constexpr int BM = 32 * WT;
+  // register sets in flight: deep for the small single tile (few workgroups, latency-bound), two where a deeper
+  // pipeline would cost a resident wave per SIMD
+  constexpr int PF = (!DUAL && WT == 2) ? 4 : 2;
+  const size_t lds = (size_t)2 * 2 * (DUAL ? 2 : 1) * BM * kGLd * 2;
+  if (lds > 64 * 1024 && !granted) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, PF>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
+    granted = true;
+  }
+  const dim3 grid((a.N + BM - 1) / BM, (a.B + BM - 1) / BM);
+  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, PF>), grid, dim3(kGT), lds, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
+int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
+  // 128 x 128 tiles when they give every compute unit work, else 64 x 64
+  const int64_t big = (int64_t)((a.N + 127) / 128) * ((a.B + 127) / 128);
+  if (big >= 192) return dual ? launch_gemm_tiles_t<true, 4>(a, st, who) : launch_gemm_tiles_t<false, 4>(a, st, who);
+  return dual ? launch_gemm_tiles_t<true, 2>(a, st, who) : launch_gemm_tiles_t<false, 2>(a, st, who);
+}
+
+}  // namespace fsvd

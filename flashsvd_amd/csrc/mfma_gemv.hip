@@ -27,14 +27,6 @@ __device__ __forceinline__ bf16x8_t ldx_frag(const uint16_t* p) {
   return __builtin_bit_cast(bf16x8_t, *(gp16_t)(uintptr_t)p);
 }
 
-struct MfmaArgs {
-  const uint16_t* x; int64_t ldx;            // [B, >= K] activations; DUAL: gate input at 0, up input at up_off
-  int64_t up_off;
-  const uint16_t* W; const uint16_t* W2; int64_t ldw;   // [N, K] (DUAL: gate_u, up_u)
-  const uint16_t* bias; const uint16_t* res; int64_t ldres;
-  uint16_t* y; int64_t ldy;
-  int B, N, K, mode;
-};
 
 // NB: 16-row batch tiles (B <= 16 * NB); KS: waves that split K for one 16-row weight tile, so a workgroup
 // of 8 waves covers 8 / KS weight tiles
@@ -143,6 +135,8 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
   int ks = 8;
   for (int c = 2; c <= 8; c *= 2)
     if ((tiles * c + 7) / 8 >= 256 && ksteps / c >= 4) { ks = c; break; }
+  // many rows (prefill): the tiled kernel reads every weight once per 128 rows instead of once per 64
+  if (gemm_tiles_apply(a0)) return launch_gemm_tiles(a0, DUAL, st, who);
   // batches above 64 rows go in slices of 64
   for (int b0 = 0; b0 < a0.B; b0 += 64) {
     MfmaArgs a = a0;

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import flashsvd_oracle as O
-from tests.util import assert_close_bf16, rand_bf16
+from tests.util import assert_close_bf16, bounds, rand_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -186,3 +186,36 @@ def test_swiglu_batched_matrix_cores(ops, B, D, R, mode):
     else:
         ref = ((g * torch.sigmoid(g)) * u).to(torch.bfloat16)
     assert_close_bf16(h, ref, f"batched swiglu mode {mode}")
+
+
+# ---- 128 rows and more (prefill): the tiled matrix-core kernel (csrc/mfma_gemm.hip) behind the same entry points
+@pytest.mark.parametrize("B,N,K", [(512, 3072, 4096), (128, 128, 64), (200, 1000, 1536), (129, 130, 192), (384, 1536, 11008),
+                                   (1024, 64, 1024)])
+def test_linear_prefill_rows_tiled_kernel(ops, B, N, K):
+    x, w = rand_bf16(B, K, seed=1), rand_bf16(N, K, std=0.02, seed=2)
+    bias, res = rand_bf16(N, std=0.1, seed=4), rand_bf16(B, N, seed=5)
+    y = ops.linear(x.cuda(), w.cuda(), bias.cuda(), residual=res.cuda())
+    ref = res + O.lin(x, w, bias)
+    assert_close_bf16(y, ref, f"tiled linear {B}x{N}x{K}", **bounds(ref))
+    y_plain = ops.linear(x.cuda(), w.cuda())
+    ref = O.lin(x, w)
+    assert_close_bf16(y_plain, ref, f"tiled linear, no epilogue {B}x{N}x{K}", **bounds(ref))
+    # strided operands: x a column slice, y a column slice of wider buffers
+    xw = torch.zeros(B, K + 64, dtype=torch.bfloat16)
+    xw[:, 64:] = x
+    out = torch.zeros(B, N + 8, dtype=torch.bfloat16, device="cuda")
+    ops.linear(xw.cuda()[:, 64:], w.cuda(), out=out[:, 8:])
+    assert torch.equal(out[:, 8:].cpu(), y_plain.cpu()) and float(out[:, :8].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("B,D,R,mode", [(512, 11008, 1536, 0), (130, 200, 64, 1), (256, 1376, 256, 1)])
+def test_swiglu_prefill_rows_tiled_kernel(ops, B, D, R, mode):
+    p = rand_bf16(B, 2 * R, seed=1)
+    gu, uu = rand_bf16(D, R, std=0.05, seed=2), rand_bf16(D, R, std=0.05, seed=3)
+    h = ops.swiglu_linear(p.cuda(), gu.cuda(), uu.cuda(), up_off=R, mode=mode)
+    g, u = p[:, :R].float() @ gu.float().t(), p[:, R:].float() @ uu.float().t()
+    if mode == 0:
+        ref = torch.nn.functional.silu(g.to(torch.bfloat16)) * u.to(torch.bfloat16)
+    else:
+        ref = ((g * torch.sigmoid(g)) * u).to(torch.bfloat16)
+    assert_close_bf16(h, ref, f"tiled swiglu mode {mode}", **bounds(ref))
