@@ -131,6 +131,8 @@ struct PrefillAttnArgs {
   float scale;
 };
 int launch_expand(const ExpandArgs& a, hipStream_t st);
+bool expand_tiles_apply(const ExpandArgs& a);                               // mfma_gemm.hip
+int launch_expand_tiles(const ExpandArgs& a, hipStream_t st);
 int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st);
 
 // matrix-core projections: y = epilogue(x . W^T) with the rounding points of the vector kernels

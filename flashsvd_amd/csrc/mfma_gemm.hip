@@ -20,8 +20,21 @@ constexpr int kGLd = kGBK + 8;      // LDS row stride in elements (144 bytes)
 
 // WT: 16 x 16 accumulator tiles per wave and dimension: 4 -> 128 x 128 per workgroup, 2 -> 64 x 64 (problems with
 // few output tiles, where more workgroups matter more than reuse)
-template <bool DUAL, int WT, int PF>
-__global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a) {
+// EXPAND: the head-expansion form of the prefill (y = P . u^T per head, then rotate-half RoPE at the token's position
+// and a store into the query buffer or the cache rows): a column tile is one 128-wide head, and a wave takes columns
+// [32 wn, 32 wn + 32) and [64 + 32 wn, 64 + 32 wn + 32) of it so that d and d + 64 of a rotation pair sit in one lane
+struct ExpandEpi {
+  const uint16_t* cos; const uint16_t* sin; int rope_len;
+  const int32_t* positions;
+  int M;                                   // tokens per batch row (x row r = batch r / M, token r % M)
+  int64_t sp_b, sp_m;                      // strides of the coefficient rows
+  int64_t sy_b, sy_m, sy_h;                // destination strides
+  int dst_by_position, dst_rows;
+};
+
+template <bool DUAL, int WT, int PF, bool EXPAND>
+__global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi ep) {
+  static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion uses the single 128 x 128 tile");
   constexpr int NM = DUAL ? 2 : 1;
   constexpr int kGBM = 32 * WT, kGBN = 32 * WT;
   extern __shared__ __align__(16) unsigned char gm_smem[];
@@ -41,7 +54,8 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a) {
 #pragma unroll
   for (int j = 0; j < WT; ++j) {
     const int64_t xr = min(m0 + ld_row + 32 * j, a.B - 1), wr = min(n0 + ld_row + 32 * j, a.N - 1);
-    gx[0][j] = a.x + xr * a.ldx + ld_chunk * 8;
+    if (EXPAND) gx[0][j] = a.x + (xr / ep.M) * ep.sp_b + (xr % ep.M) * ep.sp_m + ld_chunk * 8;
+    else gx[0][j] = a.x + xr * a.ldx + ld_chunk * 8;
     gw[0][j] = a.W + wr * a.ldw + ld_chunk * 8;
     if (DUAL) {
       gx[NM - 1][j] = a.x + xr * a.ldx + a.up_off + ld_chunk * 8;
@@ -100,7 +114,8 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a) {
 #pragma unroll
           for (int i = 0; i < WT; ++i) {
             fx[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + m * kTile + (wm * 16 * WT + i * 16 + lr) * kGLd + kk * 32 + lg * 8);
-            fw[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + (NM + m) * kTile + (wn * 16 * WT + i * 16 + lr) * kGLd + kk * 32 + lg * 8);
+            const int wrow = EXPAND ? (i < 2 ? wn * 32 + i * 16 : 64 + wn * 32 + (i - 2) * 16) : wn * 16 * WT + i * 16;
+            fw[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + (NM + m) * kTile + (wrow + lr) * kGLd + kk * 32 + lg * 8);
           }
 #pragma unroll
           for (int i = 0; i < WT; ++i)
@@ -125,6 +140,32 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a) {
     for (int e = 0; e < 4; ++e) {
       const int m = m0 + wm * 16 * WT + i * 16 + lg * 4 + e;
       if (m >= a.B) continue;
+      if (EXPAND) {
+        const int b = m / ep.M, t = m - b * ep.M;
+        const int pos = (ep.positions ? ep.positions[b] : 0) + t;
+        const int slot = ep.dst_by_position ? pos : t;
+        if (slot < 0 || slot >= ep.dst_rows) continue;   // outside the destination: dropped
+        const int head = blockIdx.x;
+        uint16_t* dst = a.y + (int64_t)b * ep.sy_b + (int64_t)slot * ep.sy_m + (int64_t)head * ep.sy_h;
+        const int tp = min(max(pos, 0), ep.rope_len - 1);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int d = wn * 32 + j * 16 + lr;
+          float x0 = acc[0][i][j][e], x1 = acc[0][i][j + 2][e];
+          if (a.bias) { x0 += bf16_bits_to_f32(a.bias[head * 128 + d]); x1 += bf16_bits_to_f32(a.bias[head * 128 + d + 64]); }
+          x0 = round_bf16(x0);                          // the projection's own rounding point
+          x1 = round_bf16(x1);
+          if (ep.cos) {                                 // eager bf16 arithmetic, one rounding per op
+            const float c = bf16_bits_to_f32(ep.cos[(int64_t)tp * 64 + d]), sn = bf16_bits_to_f32(ep.sin[(int64_t)tp * 64 + d]);
+            const float r0 = round_bf16(round_bf16(x0 * c) - round_bf16(x1 * sn));
+            const float r1 = round_bf16(round_bf16(x1 * c) + round_bf16(x0 * sn));
+            x0 = r0; x1 = r1;
+          }
+          dst[d] = (uint16_t)f32_to_bf16_bits(x0);
+          dst[d + 64] = (uint16_t)f32_to_bf16_bits(x1);
+        }
+        continue;
+      }
 #pragma unroll
       for (int j = 0; j < WT; ++j) {
         const int n = n0 + wn * 16 * WT + j * 16 + lr;
@@ -163,13 +204,13 @@ static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* wh
   constexpr int PF = (!DUAL && WT == 2) ? 4 : 2;
   const size_t lds = (size_t)2 * 2 * (DUAL ? 2 : 1) * BM * kGLd * 2;
   if (lds > 64 * 1024 && !granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, PF>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, PF, false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
   }
   const dim3 grid((a.N + BM - 1) / BM, (a.B + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, PF>), grid, dim3(kGT), lds, st, a);
+  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, PF, false>), grid, dim3(kGT), lds, st, a, ExpandEpi{});
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
@@ -180,6 +221,34 @@ int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* 
   const int64_t big = (int64_t)((a.N + 127) / 128) * ((a.B + 127) / 128);
   if (big >= 192) return dual ? launch_gemm_tiles_t<true, 4>(a, st, who) : launch_gemm_tiles_t<false, 4>(a, st, who);
   return dual ? launch_gemm_tiles_t<true, 2>(a, st, who) : launch_gemm_tiles_t<false, 2>(a, st, who);
+}
+
+// head expansion of the prefill on the tiled kernel: 128 token rows and more, head_dim 128, rank a multiple of 64,
+// coefficients shared by the heads
+bool expand_tiles_apply(const ExpandArgs& a) {
+  return a.Dh == 128 && (int64_t)a.B * a.M >= 128 && (a.R % kGBK) == 0 && a.sp_h == 0 && (a.sp_b % 8) == 0 && (a.sp_m % 8) == 0 &&
+         (a.ldu % 8) == 0;
+}
+
+int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
+  const char* who = "fsvd_lowrank_expand_heads";
+  static bool granted = false;
+  constexpr int PF = 2;
+  const size_t lds = (size_t)2 * 2 * 128 * kGLd * 2;
+  if (!granted) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<false, 4, PF, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
+    granted = true;
+  }
+  const int rows = a.B * a.M;
+  MfmaArgs g{a.p, 0, 0, a.u, nullptr, a.ldu, a.bias, nullptr, 0, a.y, 0, rows, a.heads * 128, a.R, 0};
+  ExpandEpi ep{a.cos, a.sin, a.rope_len, a.positions, a.M, a.sp_b, a.sp_m, a.sy_b, a.sy_m, a.sy_h, a.dst_by_position, a.dst_rows};
+  const dim3 grid(a.heads, (rows + 127) / 128);
+  hipLaunchKernelGGL((gemm_tiles_kernel<false, 4, PF, true>), grid, dim3(kGT), lds, st, g, ep);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
 }
 
 }  // namespace fsvd

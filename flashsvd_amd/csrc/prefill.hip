@@ -250,6 +250,7 @@ int launch_expand(const ExpandArgs& a, hipStream_t st) {
     set_last_error("%s: coefficient / factor pointers and strides must be 16-byte aligned", fn);
     return kErrBadAlign;
   }
+  if (expand_tiles_apply(a)) return launch_expand_tiles(a, st);   // long prompts: the LDS-tiled kernel
   const int T = a.B * a.M;
   hipLaunchKernelGGL(lowrank_expand_kernel, dim3((T + 127) / 128, a.heads), dim3(kPfThreads), 0, st, a);
   hipError_t e = hipGetLastError();

@@ -99,6 +99,36 @@ def test_expand_and_prefill_attention_primitives():
         assert_close_bf16(out[:, m], refm, f"row {m}", **bounds(refm))
 
 
+@pytest.mark.parametrize("B,M,R", [(1, 512, 1024), (2, 130, 64), (3, 50, 192)])
+def test_expand_long_prompts_tiled_kernel(B, M, R):
+    """128 token rows and more with a rank that is a multiple of 64: the LDS-tiled expansion; same result as the
+    oracle and as the per-wave kernel (rank 72 above takes that one)."""
+    from flashsvd_amd import hip_ops
+    H, dh, start = 3, 128, 7
+    S = start + M + 5
+    cos, sin = O.rope_tables(S, dh, dtype=BF16)
+    p = rand_bf16(B, M, R, seed=1)
+    u = rand_bf16(H * dh, R, std=R ** -0.5, seed=2)
+    bias = rand_bf16(H * dh, std=0.1, seed=3)
+    pos0 = torch.tensor([start + b for b in range(B)], dtype=torch.int32, device="cuda")
+    # rotated, by position, into cache rows
+    kc = torch.zeros(B, S, H, dh, dtype=BF16, device="cuda")
+    hip_ops.lowrank_expand_heads(p.cuda(), u.cuda(), num_heads=H, head_dim=dh, out=kc, cos=cos.cuda(), sin=sin.cuda(),
+                                 positions=pos0, dst_by_position=True)
+    for b in range(B):
+        s0 = start + b
+        ref = O.apply_rope(O.lin(p[b], u).reshape(M, H, dh), cos[s0:s0 + M][:, None], sin[s0:s0 + M][:, None])
+        assert_close_bf16(kc[b, s0:s0 + M], ref, f"rotated rows of batch {b}", **bounds(ref))
+        assert torch.all(kc[b, :s0] == 0) and torch.all(kc[b, s0 + M:] == 0)
+    # not rotated, with bias, by token index into a query-shaped buffer (strided coefficient rows)
+    wide = torch.zeros(B, M, R + 64, dtype=BF16)
+    wide[..., 64:] = p
+    q = torch.zeros(B, M, H, dh, dtype=BF16, device="cuda")
+    hip_ops.lowrank_expand_heads(wide.cuda()[..., 64:], u.cuda(), num_heads=H, head_dim=dh, out=q, bias=bias.cuda(), positions=pos0)
+    ref = O.lin(p, u, bias).reshape(B, M, H, dh)
+    assert_close_bf16(q, ref, "plain expansion with bias", **bounds(ref))
+
+
 def test_model_prefill_mfma_equals_decode_route():
     mw = O.make_model(d=512, n_heads=4, n_kv_heads=2, head_dim=128, ffn=1024, attn_rank=96, mlp_rank=128, n_layers=2,
                       vocab=300, dtype=BF16, seed=7, std=0.05)
