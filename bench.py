@@ -46,6 +46,8 @@ def _parse():
     ap.add_argument("--engine", choices=["persistent", "graph", "both"], default="both",
                     help="persistent: one resident kernel per token (fsvd_decode_step); graph: one HIP graph of the "
                          "per-operator kernels per token; both: time both, the headline value is the persistent step")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="only time the prompt pass (matrix-core kernels): W untimed and K timed passes over a 512-token prompt")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device copy 10 times (the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counters are scaled against) and exit")
@@ -165,6 +167,26 @@ def run_lowrank(args):
     t_prefill = time.perf_counter() - t0
     tok = out.logits[:, -1].float().argmax(-1, keepdim=True)
     res = dict(prefill_s=t_prefill)
+    # the first pass pays one-time set-up (weight packing, tables, kernel attributes): time warm passes as well
+    reps = args.steps if args.prefill_only else 2
+    scratch = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=torch.bfloat16)
+    for _ in range(args.warmup if args.prefill_only else 1):
+        model(prompt, past_key_values=scratch, cache_position=torch.arange(PROMPT_LEN), logits_to_keep=1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        model(prompt, past_key_values=scratch, cache_position=torch.arange(PROMPT_LEN), logits_to_keep=1)
+    torch.cuda.synchronize()
+    t_warm = (time.perf_counter() - t0) / reps
+    del scratch
+    d, D, Ra, Rm, H, Dh = (CFG[k] for k in ("hidden_size", "intermediate_size", "attn_rank", "mlp_rank", "num_heads", "head_dim"))
+    proj_flop = 2.0 * PROMPT_LEN * (8 * d * Ra + 3 * (d + D) * Rm)                    # every factor once per token
+    attn_flop = 2.0 * 2 * H * Dh * PROMPT_LEN * (PROMPT_LEN + 1) / 2                   # causal QK^T and PV
+    flop = args.layers * (proj_flop + attn_flop) + 2.0 * d * CFG["vocab_size"]
+    res["prefill"] = dict(prompt_len=PROMPT_LEN, warm_s=t_warm, tok_s=PROMPT_LEN / t_warm, flop=flop,
+                          TFLOPs=flop / t_warm / 1e12, frac_of_bf16_mfma_peak=flop / t_warm / 2.5e15, cold_s=t_prefill)
+    if args.prefill_only:
+        return res
     dec = GraphedDecoder(model, cache, B)
     dec.set_state(tok, PROMPT_LEN)
     if args.engine in ("graph", "both"):
@@ -381,6 +403,11 @@ def main():
     from flashsvd_amd import _lib
     _lib.load()
     lr = run_lowrank(args)
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tok/s, 7B-shape rank-0.5 bs1 prompt 512", "value": lr["prefill"]["tok_s"], "unit": "tok/s",
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16", "data": "synthetic",
+                          "prefill": lr["prefill"]}))
+        return
     line = {
         "metric": "decode tok/s, 7B-shape rank-0.5 bs1", "value": lr["tok_s"], "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": lr["ms_per_step"], "higher_is_better": True,
@@ -392,6 +419,7 @@ def main():
         "roofline": lr["roofline"],
         "step_hbm": {"bytes_per_token": lr["step_bytes"], "GB/s": lr["step_GBs"], "frac_of_peak": lr["step_GBs"] / HBM_PEAK_GBS},
         "prefill_s": lr["prefill_s"],
+        "prefill": lr["prefill"],
     }
     for k in ("persistent", "graph", "swiglu_roofline"):
         if k in lr:

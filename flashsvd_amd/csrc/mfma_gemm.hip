@@ -2,10 +2,12 @@
 //
 // Both operands are K-contiguous, which is the layout V_MFMA_F32_16X16X32_BF16 wants for its two inputs (each lane
 // holds 8 consecutive k of one row).  A workgroup of four waves owns a 128 x 128 output tile (a wave 64 x 64: 4 x 4
-// accumulator tiles), walks K in steps of 64 through a double-buffered LDS stage (rows padded to 72 elements so that
-// the 16-byte fragment reads of 16 consecutive rows fall on different banks) and overlaps the global loads of step
-// k + 1 with the products of step k.  Epilogue as in the vector kernels: bias, ONE rounding to bf16, residual — or,
-// for the gate / up pair, SwiGLU in either rounding mode.  Every weight is read once per 128 rows of x.
+// accumulator tiles) — or 64 x 64 when the problem has too few big tiles to give every compute unit work — and walks K
+// in steps of 64 or 128 through a double-buffered LDS stage (rows padded by 16 bytes so that the fragment reads of 16
+// consecutive rows fall on different banks).  Global loads run two to four steps ahead in registers and are written to
+// the idle LDS stage one step before their products.  Epilogue as in the vector kernels: bias, ONE rounding to bf16,
+// residual — or, for the gate / up pair, SwiGLU in either rounding mode — or the head expansion of the prompt pass
+// (RoPE, store into the query buffer or the cache rows).  Every weight is read once per 128 (64) rows of x.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -15,8 +17,7 @@ typedef __bf16 gm_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float gm_f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kGT = 256;            // threads: 2 x 2 waves
-constexpr int kGBK = 64;
-constexpr int kGLd = kGBK + 8;      // LDS row stride in elements (144 bytes)
+constexpr int kGBK = 64;            // K per step (the small tile takes 128 when K allows: half as many barriers)
 
 // WT: 16 x 16 accumulator tiles per wave and dimension: 4 -> 128 x 128 per workgroup, 2 -> 64 x 64 (problems with
 // few output tiles, where more workgroups matter more than reuse)
@@ -32,10 +33,13 @@ struct ExpandEpi {
   int dst_by_position, dst_rows;
 };
 
-template <bool DUAL, int WT, int PF, bool EXPAND>
+template <bool DUAL, int WT, int PF, bool EXPAND, int BK>
 __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi ep) {
   static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion uses the single 128 x 128 tile");
   constexpr int NM = DUAL ? 2 : 1;
+  constexpr int kGLd = BK + 8;            // LDS row stride in elements: 16 bytes of padding against bank conflicts
+  constexpr int CPR = BK / 8;             // 16-byte pieces per tile row
+  constexpr int NP = 32 * WT * CPR / kGT; // pieces per thread and operand
   constexpr int kGBM = 32 * WT, kGBN = 32 * WT;
   extern __shared__ __align__(16) unsigned char gm_smem[];
   // [stage][operand: x0, (x1), W0, (W1)][128 rows][kGLd]
@@ -45,15 +49,16 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.y * kGBM, n0 = blockIdx.x * kGBN;
-  const int ksteps = a.K / kGBK;
+  const int ksteps = a.K / BK;
 
-  // global -> register staging: a tile row is 128 bytes = 8 16-byte pieces; WT pieces per thread and operand
-  const int ld_row = tid >> 3, ld_chunk = tid & 7;   // rows ld_row + 32 * j, j = 0..WT-1
-  const uint16_t* gx[NM][WT];
-  const uint16_t* gw[NM][WT];
+  // global -> register staging: a tile row is CPR 16-byte pieces; NP pieces per thread and operand
+  constexpr int RPP = kGT / CPR;                      // rows covered by one pass of the workgroup
+  const int ld_row = tid / CPR, ld_chunk = tid % CPR; // rows ld_row + RPP * j, j = 0..NP-1
+  const uint16_t* gx[NM][NP];
+  const uint16_t* gw[NM][NP];
 #pragma unroll
-  for (int j = 0; j < WT; ++j) {
-    const int64_t xr = min(m0 + ld_row + 32 * j, a.B - 1), wr = min(n0 + ld_row + 32 * j, a.N - 1);
+  for (int j = 0; j < NP; ++j) {
+    const int64_t xr = min(m0 + ld_row + RPP * j, a.B - 1), wr = min(n0 + ld_row + RPP * j, a.N - 1);
     if (EXPAND) gx[0][j] = a.x + (xr / ep.M) * ep.sp_b + (xr % ep.M) * ep.sp_m + ld_chunk * 8;
     else gx[0][j] = a.x + xr * a.ldx + ld_chunk * 8;
     gw[0][j] = a.W + wr * a.ldw + ld_chunk * 8;
@@ -64,13 +69,13 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
   }
   // PF register sets hold the global loads of the next PF steps (set s % PF belongs to step s); a set is written
   // to the idle LDS stage one step before its products and refilled at once with the loads of step s + PF
-  u32x4_t rx[PF][NM][WT], rw[PF][NM][WT];
+  u32x4_t rx[PF][NM][NP], rw[PF][NM][NP];
   auto load_regs = [&](int set, int ks) {
-    const int k = min(ks, ksteps - 1) * kGBK;        // past the end: a valid address, never used
+    const int k = min(ks, ksteps - 1) * BK;          // past the end: a valid address, never used
 #pragma unroll
     for (int m = 0; m < NM; ++m)
 #pragma unroll
-      for (int j = 0; j < WT; ++j) {
+      for (int j = 0; j < NP; ++j) {
         rx[set][m][j] = *reinterpret_cast<const u32x4_t*>(gx[m][j] + k);
         rw[set][m][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(gw[m][j] + k));
       }
@@ -80,8 +85,8 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
 #pragma unroll
     for (int m = 0; m < NM; ++m)
 #pragma unroll
-      for (int j = 0; j < WT; ++j) {
-        const int off = (ld_row + 32 * j) * kGLd + ld_chunk * 8;
+      for (int j = 0; j < NP; ++j) {
+        const int off = (ld_row + RPP * j) * kGLd + ld_chunk * 8;
         *reinterpret_cast<u32x4_t*>(base + m * kTile + off) = rx[set][m][j];
         *reinterpret_cast<u32x4_t*>(base + (NM + m) * kTile + off) = rw[set][m][j];
       }
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
       if (ks >= ksteps) break;
       const uint16_t* base = lds + (ks & 1) * kStage;
 #pragma unroll
-      for (int kk = 0; kk < kGBK / 32; ++kk) {
+      for (int kk = 0; kk < BK / 32; ++kk) {
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
           gm_bf16x8_t fx[WT], fw[WT];
@@ -195,22 +200,23 @@ bool gemm_tiles_apply(const MfmaArgs& a) {
   return a.B >= 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0;
 }
 
-template <bool DUAL, int WT>
+template <bool DUAL, int WT, int BK>
 static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* who) {
   static bool granted = false;
   constexpr int BM = 32 * WT;
+  constexpr int kGLd = BK + 8;
   // register sets in flight: deep for the small single tile (few workgroups, latency-bound), two where a deeper
   // pipeline would cost a resident wave per SIMD
-  constexpr int PF = (!DUAL && WT == 2) ? 4 : 2;
+  constexpr int PF = (!DUAL && WT == 2 && BK == 64) ? 4 : 2;
   const size_t lds = (size_t)2 * 2 * (DUAL ? 2 : 1) * BM * kGLd * 2;
   if (lds > 64 * 1024 && !granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, PF, false>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, PF, false, BK>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
   }
   const dim3 grid((a.N + BM - 1) / BM, (a.B + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, PF, false>), grid, dim3(kGT), lds, st, a, ExpandEpi{});
+  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, PF, false, BK>), grid, dim3(kGT), lds, st, a, ExpandEpi{});
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
@@ -219,8 +225,9 @@ static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* wh
 int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
   // 128 x 128 tiles when they give every compute unit work, else 64 x 64
   const int64_t big = (int64_t)((a.N + 127) / 128) * ((a.B + 127) / 128);
-  if (big >= 192) return dual ? launch_gemm_tiles_t<true, 4>(a, st, who) : launch_gemm_tiles_t<false, 4>(a, st, who);
-  return dual ? launch_gemm_tiles_t<true, 2>(a, st, who) : launch_gemm_tiles_t<false, 2>(a, st, who);
+  if (big >= 192) return dual ? launch_gemm_tiles_t<true, 4, 64>(a, st, who) : launch_gemm_tiles_t<false, 4, 64>(a, st, who);
+  if (dual) return launch_gemm_tiles_t<true, 2, 64>(a, st, who);
+  return (a.K % 128) == 0 ? launch_gemm_tiles_t<false, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 2, 64>(a, st, who);
 }
 
 // head expansion of the prefill on the tiled kernel: 128 token rows and more, head_dim 128, rank a multiple of 64,
@@ -234,9 +241,10 @@ int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
   const char* who = "fsvd_lowrank_expand_heads";
   static bool granted = false;
   constexpr int PF = 2;
+  constexpr int kGLd = kGBK + 8;
   const size_t lds = (size_t)2 * 2 * 128 * kGLd * 2;
   if (!granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<false, 4, PF, true>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<false, 4, PF, true, kGBK>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
@@ -245,7 +253,7 @@ int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
   MfmaArgs g{a.p, 0, 0, a.u, nullptr, a.ldu, a.bias, nullptr, 0, a.y, 0, rows, a.heads * 128, a.R, 0};
   ExpandEpi ep{a.cos, a.sin, a.rope_len, a.positions, a.M, a.sp_b, a.sp_m, a.sy_b, a.sy_m, a.sy_h, a.dst_by_position, a.dst_rows};
   const dim3 grid(a.heads, (rows + 127) / 128);
-  hipLaunchKernelGGL((gemm_tiles_kernel<false, 4, PF, true>), grid, dim3(kGT), lds, st, g, ep);
+  hipLaunchKernelGGL((gemm_tiles_kernel<false, 4, PF, true, kGBK>), grid, dim3(kGT), lds, st, g, ep);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
