@@ -95,6 +95,37 @@ def per_layer_kernel_us(fn_per_layer, n_layers: int, reps: int = 10) -> float:
     return time_graph_ms(g, reps) * 1000.0 / n_layers
 
 
+def kernel_configs(model, cache, dec, n_layers: int) -> dict:
+    """The two kernel-level configurations of the benchmark contract, per CALL (all launches of the block replayed
+    from a graph over every layer's cold weights, launch gaps included): one low-rank attention block at the 7B shape
+    (rank projection, q/k/v expansion + RoPE + cache append, attention over the cached context, output projection) and
+    one low-rank SwiGLU MLP for 1, 8 and 32 rows."""
+    import torch
+    L = model.model.layers
+    d = CFG["hidden_size"]
+    out = {}
+    x = torch.randn(1, d, device="cuda").to(torch.bfloat16)
+    pos = torch.full((1,), PROMPT_LEN, dtype=torch.int32, device="cuda")
+
+    def attn(i):
+        n1 = L[i].input_layernorm
+        return L[i].self_attn.decode_token(x, cache, pos, norm_weight=n1.weight, eps=n1.variance_epsilon, residual=x,
+                                           rope=dec.rope, attn_ws=dec.attn_ws, nsplit=dec.nsplit)
+    us = per_layer_kernel_us(attn, n_layers)
+    nb = 8 * d * CFG["attn_rank"] * 2 + 2 * PROMPT_LEN * CFG["num_heads"] * CFG["head_dim"] * 2 + 2 * d * 2 * 2
+    out["attention_block_bs1_ctx512"] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3, "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS}
+    for B in (1, 8, 32):
+        xb = torch.randn(B, d, device="cuda").to(torch.bfloat16)
+
+        def mlp(i, xb=xb):
+            n2 = L[i].post_attention_layernorm
+            return L[i].mlp.run(xb, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=xb)
+        us = per_layer_kernel_us(mlp, n_layers)
+        nb = 3 * (d + CFG["intermediate_size"]) * CFG["mlp_rank"] * 2 + B * 2 * d * 2
+        out[f"swiglu_mlp_bs{B}"] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3, "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS}
+    return out
+
+
 def kernel_legs(model, cache, dec):
     """name -> (launch closure over layer index, algorithmic bytes per launch)."""
     import torch
@@ -222,6 +253,7 @@ def run_lowrank(args):
         del pdec
     best = res.get("persistent") or res["graph"]
     res["tok_s"], res["ms_per_step"] = best["tok_s"], best["ms_per_step"]
+    res["kernel_configs"] = kernel_configs(model, cache, dec, args.layers)
     legs = kernel_legs(model, cache, dec)
     name = "mlp_gate_up_u+swiglu"
     fn, nbytes = legs[name]
@@ -420,6 +452,7 @@ def main():
         "step_hbm": {"bytes_per_token": lr["step_bytes"], "GB/s": lr["step_GBs"], "frac_of_peak": lr["step_GBs"] / HBM_PEAK_GBS},
         "prefill_s": lr["prefill_s"],
         "prefill": lr["prefill"],
+        "kernel_configs": lr["kernel_configs"],
     }
     for k in ("persistent", "graph", "swiglu_roofline"):
         if k in lr:
