@@ -240,6 +240,182 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// 2b. the same attention for long prompts: 128 queries per workgroup (32 per wave), K and V tiles shared
+//     through LDS.  With 64 queries per workgroup and every wave fetching its own K fragments, a 64-key tile
+//     costs 80 KB of L2 traffic per 64 queries and the kernel is bound by L2 requests; here a tile is read ONCE
+//     per workgroup (32 KB per 128 queries), coalesced, one tile ahead into registers, and written to LDS
+//     (K row-major with a padded stride, V transposed: four adjacent keys per 8-byte write, key column XOR-ed
+//     with 8 * (d / 8 % 8) to spread the 16 dimension blocks over the banks).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(PrefillAttnArgs a) {
+  constexpr int DH = 128, BN = 64, QW = 32, KSTR = DH + 8, PSTR = BN + 8, VSTR = BN + 8;
+  extern __shared__ __align__(16) unsigned char pw_smem[];
+  uint16_t (*Ks)[KSTR] = reinterpret_cast<uint16_t (*)[KSTR]>(pw_smem);                              // [BN][KSTR]
+  uint16_t (*Vt)[VSTR] = reinterpret_cast<uint16_t (*)[VSTR]>(pw_smem + (size_t)BN * KSTR * 2);       // [DH][VSTR]
+  uint16_t (*Ps)[QW][PSTR] = reinterpret_cast<uint16_t (*)[QW][PSTR]>(pw_smem + (size_t)BN * KSTR * 2 + (size_t)DH * VSTR * 2);
+  uint16_t (*Pl)[QW][PSTR] = Ps + 4;
+
+  const int mt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int hk = h / (a.H / a.Hk);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int q0 = a.q_pos0 ? a.q_pos0[b] : 0;
+  const int m_base = mt * 128 + wave * QW;
+  const int n_keys_all = max(1, min(q0 + a.M, a.S));
+
+  bf16x8_t qf[2][4];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+    const int m = min(m_base + mi * 16 + lr, a.M - 1);
+    const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)m * a.sq_m + (int64_t)h * a.sq_h + lg * 8;
+#pragma unroll
+    for (int st = 0; st < 4; ++st) qf[mi][st] = pf_ld(qp + st * 32);
+  }
+  float m_run[2][4], l_run[2][4];
+  f32x4_t o[2][8];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { m_run[mi][i] = -INFINITY; l_run[mi][i] = 0.f; }
+#pragma unroll
+    for (int t = 0; t < 8; ++t) o[mi][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int last_m = min(mt * 128 + 127, a.M - 1);
+  const int k_end = a.causal ? min(n_keys_all, q0 + last_m + 1) : n_keys_all;
+  // last key this wave's rows may see: tiles past it are skipped by the wave (it still takes part in the staging)
+  const int wave_end = a.causal ? min(n_keys_all, q0 + min(m_base + QW - 1, a.M - 1) + 1) : n_keys_all;
+  const uint16_t* kb = a.k + (int64_t)b * a.sk_b + (int64_t)hk * a.sk_h;
+  const uint16_t* vb = a.v + (int64_t)b * a.sk_b + (int64_t)hk * a.sk_h;
+
+  // staging roles: 16 lanes cover one 256-byte row; K: rows tid/16 + 16 j; V: the four adjacent keys 4 (tid/16) + j
+  const int srow = tid >> 4, d0 = (tid & 15) * 8;
+  u32x4_t kreg[4], vreg[4];
+  auto request = [&](int n0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int kkey = min(n0 + srow + 16 * j, n_keys_all - 1), vkey = min(n0 + srow * 4 + j, n_keys_all - 1);
+      kreg[j] = *reinterpret_cast<const u32x4_t*>(kb + (int64_t)kkey * a.sk_s + d0);
+      vreg[j] = *reinterpret_cast<const u32x4_t*>(vb + (int64_t)vkey * a.sk_s + d0);
+    }
+  };
+  if (k_end > 0) request(0);
+
+  for (int n0 = 0; n0 < k_end; n0 += BN) {
+    __syncthreads();   // the previous tile's Ks / Vt are consumed
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(&Ks[srow + 16 * j][d0]) = kreg[j];
+    {
+      const int col = (srow * 4) ^ (8 * ((tid & 15) & 7));
+      const uint32_t w[4][4] = {{vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w}, {vreg[1].x, vreg[1].y, vreg[1].z, vreg[1].w},
+                                {vreg[2].x, vreg[2].y, vreg[2].z, vreg[2].w}, {vreg[3].x, vreg[3].y, vreg[3].z, vreg[3].w}};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        u32x2_t lo, hi;   // dimensions d0 + 2c (low halves) and d0 + 2c + 1 (high halves) of the four keys
+        lo.x = (w[0][c] & 0xffffu) | (w[1][c] << 16);
+        lo.y = (w[2][c] & 0xffffu) | (w[3][c] << 16);
+        hi.x = (w[0][c] >> 16) | (w[1][c] & 0xffff0000u);
+        hi.y = (w[2][c] >> 16) | (w[3][c] & 0xffff0000u);
+        *reinterpret_cast<u32x2_t*>(&Vt[d0 + 2 * c][col]) = lo;
+        *reinterpret_cast<u32x2_t*>(&Vt[d0 + 2 * c + 1][col]) = hi;
+      }
+    }
+    __syncthreads();   // tile visible
+    if (n0 + BN < k_end) request(n0 + BN);
+    if (n0 >= wave_end) continue;   // nothing this wave's rows may see (wave-uniform)
+
+    // ---- S = Q K^T for 32 rows x 64 keys
+    f32x4_t sacc[2][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      bf16x8_t kf[4];
+#pragma unroll
+      for (int st = 0; st < 4; ++st) kf[st] = pf_ld(&Ks[j * 16 + lr][st * 32 + lg * 8]);
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) {
+        sacc[mi][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int st = 0; st < 4; ++st) sacc[mi][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[mi][st], kf[st], sacc[mi][j], 0, 0, 0);
+      }
+    }
+    // ---- masks + online softmax on the accumulator layout (rows lg*4+i, key column j*16+lr), P to LDS
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m_base + mi * 16 + lg * 4 + i;
+        const int qpos = q0 + m;
+        float pv[4];
+        float rmax = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int key = n0 + j * 16 + lr;
+          float v = sacc[mi][j][i];
+          bool ok = key < n_keys_all && m < a.M;
+          if (a.causal) ok = ok && key <= qpos;
+          v = ok ? v * a.scale : -INFINITY;            // mask first, then scale, as the reference kernel
+          if (ok && a.pad_mask) ok = a.pad_mask[(int64_t)b * a.spm_b + key] != 0;
+          if (!ok) v = -INFINITY;
+          if (ok && a.add_mask) v += a.add_mask[(int64_t)b * a.sam_b + (int64_t)m * a.sam_q + key];
+          pv[j] = v;
+          rmax = fmaxf(rmax, v);
+        }
+        rmax = row16_max(rmax);
+        const float m_new = fmaxf(m_run[mi][i], rmax);
+        const float alpha = (m_run[mi][i] == -INFINITY) ? 0.f : __expf(m_run[mi][i] - m_new);
+        float rsum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float e = (pv[j] == -INFINITY || m_new == -INFINITY) ? 0.f : __expf(pv[j] - m_new);
+          rsum += e;
+          const uint32_t hi = f32_to_bf16_bits(e);
+          Ps[wave][mi * 16 + lg * 4 + i][j * 16 + lr] = (uint16_t)hi;
+          Pl[wave][mi * 16 + lg * 4 + i][j * 16 + lr] = (uint16_t)f32_to_bf16_bits(e - bf16_bits_to_f32(hi));
+        }
+        rsum = row16_sum(rsum);
+        l_run[mi][i] = l_run[mi][i] * alpha + rsum;
+        m_run[mi][i] = m_new;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o[mi][t][i] *= alpha;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();   // P is written and read by this wave only; LDS keeps a wave's accesses in order
+    // ---- O += P V : A = P rows (keys contiguous), B = Vt rows (keys contiguous, swizzled)
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      bf16x8_t pa[2], pb[2];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) {
+        pa[mi] = pf_ld(&Ps[wave][mi * 16 + lr][st * 32 + lg * 8]);
+        pb[mi] = pf_ld(&Pl[wave][mi * 16 + lr][st * 32 + lg * 8]);
+      }
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const bf16x8_t vf = pf_ld(&Vt[t * 16 + lr][(st * 32 + lg * 8) ^ (8 * ((2 * t + (lr >> 3)) & 7))]);
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) {
+          o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[mi], vf, o[mi][t], 0, 0, 0);
+          o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pb[mi], vf, o[mi][t], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- normalise and store; rows with no visible key give 0
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m_base + mi * 16 + lg * 4 + i;
+      if (m >= a.M) continue;
+      const float inv = l_run[mi][i] > 0.f ? 1.0f / l_run[mi][i] : 0.f;
+      uint16_t* op = a.out + (int64_t)b * a.so_b + (int64_t)m * a.so_m + (int64_t)h * a.so_h;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) op[t * 16 + lr] = (uint16_t)f32_to_bf16_bits(o[mi][t][i] * inv);
+    }
+}
+
 int launch_expand(const ExpandArgs& a, hipStream_t st) {
   const char* fn = "fsvd_lowrank_expand_heads";
   if (a.B <= 0 || a.M <= 0 || a.heads <= 0 || a.R <= 0) { set_last_error("%s: empty shape", fn); return kErrBadShape; }
@@ -267,7 +443,19 @@ int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
     set_last_error("%s: q / k / v pointers and strides must be 16-byte aligned", fn);
     return kErrBadAlign;
   }
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), 0, st, a);
+  if (a.M >= 128) {   // long prompts: 128 queries per workgroup, K / V tiles shared through LDS
+    constexpr size_t lds = (size_t)64 * 136 * 2 + (size_t)128 * 72 * 2 + (size_t)2 * 4 * 32 * 72 * 2;
+    static bool granted = false;
+    if (!granted) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_wide_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", fn, lds, hipGetErrorString(e)); return kErrLaunch; }
+      granted = true;
+    }
+    hipLaunchKernelGGL(attn_prefill_wide_kernel, dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
+  } else {
+    hipLaunchKernelGGL(attn_prefill_kernel, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), 0, st, a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;

@@ -44,9 +44,10 @@ def test_rope_attention_module_vs_oracle(B, H, Hk, M, R, shared):
     assert_close_bf16(out, ref, "prefill", **bounds(ref))
 
 
-def test_rope_attention_masks_biases_positions():
+@pytest.mark.parametrize("M", [70, 150])     # 64-query kernel / 128-query kernel with LDS-shared tiles
+def test_rope_attention_masks_biases_positions(M):
     from flashsvd_amd.kernels.rope_attn import FlashSVDRoPEAttention, QKVFactors
-    B, H, Hk, M, R, dh = 2, 4, 4, 70, 48, 128
+    B, H, Hk, R, dh = 2, 4, 4, 48, 128
     Pq, Pk, Pv, Vq, Vk, Vv = _factors(B, H, Hk, M, R, dh, False, seed=10)
     bq, bk, bv = rand_bf16(H * dh, std=0.1, seed=20), rand_bf16(H * dh, std=0.1, seed=21), rand_bf16(H * dh, std=0.1, seed=22)
     # left-padded second row, per-row positions
