@@ -5,7 +5,9 @@
 // weights are applied to Pv in rank space, t = sum_n p_n Pv_n, and one product t @ v_u[h]^T per
 // head finishes the job (the Acc[B,H,S,R] workspace idea of the reference's split-K design).
 //
-// Stage 1, grid (nsplit, Hk*groups, B), 4 waves: each wave owns 16 keys of a 64-key tile.
+// Stage 1, grid (nsplit, Hk*groups, B), 4 waves: each wave owns 16 keys of a 64-key tile, and takes KS such
+//   tiles per pass over R when the split is long, so that every k_u fragment it loads serves 16*KS keys
+//   (the pass is bound by the L2 traffic of k_u, which every wave re-reads).
 //   MFMA 16x16x32 bf16: A = Pk[16 keys x 32 r] and B = k_u[16 d x 32 r] are both contiguous along
 //   r, so both operands are plain 16-byte global loads in the instruction's native lane layout.
 //   The 8 accumulator tiles of a wave hold K[16 keys x 128 d]; d and d+64 sit in the same lane,
@@ -28,8 +30,8 @@ __device__ __forceinline__ bf16x8_t ld_frag(const uint16_t* p) {
 }
 __device__ __forceinline__ bf16x8_t zero_frag() { return __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u}); }
 
-template <int REP>
-__global__ __launch_bounds__(kRdThreads) void rank_decode_partial_kernel(RankDecodeArgs a) {
+template <int REP, int KS>
+__global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(RankDecodeArgs a) {
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
   __shared__ float qs[REP][DH];
   __shared__ float wm[4][REP], wl[4][REP];
@@ -85,26 +87,39 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_partial_kernel(RankDec
   const uint16_t* pv_b = a.pv + (int64_t)b * a.spv_b + (int64_t)hk * a.spv_h;
   const uint16_t* ku_h = a.k_u + (int64_t)hk * DH * a.ldku;
 
-  for (int kt = k0; kt < k1; kt += kRdTileKeys) {
-    const int wkey0 = kt + wave * 16;              // first key of this wave
-    if (wkey0 >= k1) continue;                     // whole wave past the end (no block barrier in the loop)
-    // ---- K tile = Pk[16 keys, R] @ k_u[h]^T on the matrix cores
-    f32x4_t acc[NT];
+  for (int kt = k0; kt < k1; kt += kRdTileKeys * KS) {
+    // KS key sub-tiles per pass share every k_u fragment: sub-tile j of this wave starts at kt + (4j + wave) * 16
+    if (kt + wave * 16 >= k1) continue;            // whole wave past the end (no block barrier in the loop)
+    // ---- K tiles = Pk[16 keys, R] @ k_u[h]^T on the matrix cores
+    f32x4_t accs[KS][NT];
+    const uint16_t* arow[KS];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    const int akey = min(wkey0 + lr, k1 - 1);
-    const uint16_t* arow = pk_b + (int64_t)akey * a.spk_s + lg * 8;
+    for (int j = 0; j < KS; ++j) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) accs[j][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const int akey = min(kt + (4 * j + wave) * 16 + lr, k1 - 1);
+      arow[j] = pk_b + (int64_t)akey * a.spk_s + lg * 8;
+    }
     const uint16_t* brow = ku_h + (int64_t)lr * a.ldku + lg * 8;
 #pragma unroll 2
     for (int r0 = 0; r0 < a.Rk; r0 += 32) {
       const bool in = r0 + lg * 8 < a.Rk;
-      const bf16x8_t af = in ? ld_frag(arow + r0) : zero_frag();
+      bf16x8_t af[KS];
+#pragma unroll
+      for (int j = 0; j < KS; ++j) af[j] = in ? ld_frag(arow[j] + r0) : zero_frag();
       bf16x8_t bf[NT];
 #pragma unroll
       for (int t = 0; t < NT; ++t) bf[t] = in ? ld_frag(brow + (int64_t)t * 16 * a.ldku + r0) : zero_frag();
 #pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bf[t], acc[t], 0, 0, 0);
+      for (int j = 0; j < KS; ++j)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j], bf[t], accs[j][t], 0, 0, 0);
     }
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+    const int wkey0 = kt + (4 * j + wave) * 16;    // first key of this sub-tile
+    if (wkey0 >= k1) break;
+    f32x4_t (&acc)[NT] = accs[j];
     // ---- rotate-half RoPE at absolute key positions (register-local: tiles t and t+4 pair up)
     if (a.cos) {
 #pragma unroll
@@ -169,6 +184,7 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_partial_kernel(RankDec
           }
         }
       }
+    }
     }
   }
 
@@ -258,9 +274,19 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   }
   const int rep = a.H / a.Hk;
   dim3 block(kRdThreads);
-  if (rep % 4 == 0) hipLaunchKernelGGL(rank_decode_partial_kernel<4>, dim3(a.nsplit, a.Hk * (rep / 4), a.B), block, 0, st, a);
-  else if (rep % 2 == 0) hipLaunchKernelGGL(rank_decode_partial_kernel<2>, dim3(a.nsplit, a.Hk * (rep / 2), a.B), block, 0, st, a);
-  else hipLaunchKernelGGL(rank_decode_partial_kernel<1>, dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
+  // key sub-tiles per pass: long splits amortise every k_u fragment over more keys (any value is correct for any
+  // length; short splits would only rebuild clamped keys)
+  const int per = (a.S + a.nsplit - 1) / a.nsplit;
+  const int ks = per >= 512 ? 4 : (per >= 128 ? 2 : 1);
+  if (rep % 4 == 0) hipLaunchKernelGGL((rank_decode_partial_kernel<4, 1>), dim3(a.nsplit, a.Hk * (rep / 4), a.B), block, 0, st, a);
+  else if (rep % 2 == 0) {
+    if (ks >= 2) hipLaunchKernelGGL((rank_decode_partial_kernel<2, 2>), dim3(a.nsplit, a.Hk * (rep / 2), a.B), block, 0, st, a);
+    else hipLaunchKernelGGL((rank_decode_partial_kernel<2, 1>), dim3(a.nsplit, a.Hk * (rep / 2), a.B), block, 0, st, a);
+  } else {
+    if (ks == 4) hipLaunchKernelGGL((rank_decode_partial_kernel<1, 4>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
+    else if (ks == 2) hipLaunchKernelGGL((rank_decode_partial_kernel<1, 2>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
+    else hipLaunchKernelGGL((rank_decode_partial_kernel<1, 1>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: stage 1 launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
   hipLaunchKernelGGL(rank_decode_merge_kernel, dim3(a.H, a.B), block, 0, st, a);

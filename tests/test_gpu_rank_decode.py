@@ -23,7 +23,9 @@ def _lin_layout(V):   # [heads,R,Dh] -> nn.Linear weight [heads*Dh, R]
 
 
 CASES = [(1, 32, 32, 512, 560, 1024, 1024, None), (1, 32, 32, 512, 560, 1024, 1024, 1), (2, 8, 2, 100, 128, 72, 40, 3),
-         (3, 4, 4, 1, 64, 64, 64, 2), (2, 16, 4, 333, 400, 1664, 1664, 4), (1, 2, 2, 65, 80, 8, 2048, None)]
+         (3, 4, 4, 1, 64, 64, 64, 2), (2, 16, 4, 333, 400, 1664, 1664, 4), (1, 2, 2, 65, 80, 8, 2048, None),
+         # long splits take the 2- and 4-sub-tile variants of stage 1 (ragged tails, MHA and 2 query heads per kv head)
+         (2, 8, 4, 700, 720, 136, 264, 2), (2, 4, 4, 450, 500, 200, 72, 2), (1, 4, 4, 1500, 1536, 64, 64, 1)]
 
 
 @pytest.mark.parametrize("B,H,Hk,L,S,Rk,Rv,nsplit", CASES)
