@@ -35,10 +35,16 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
   __shared__ float qs[REP][DH];
   __shared__ float wm[4][REP], wl[4][REP];
-  __shared__ float tbuf[4][kRdMaxChunks * 512];
+  // one LDS block, used twice: k_u chunks [2][128 d][64 r + 8 pad] bf16 while the keys stream, the four waves'
+  // rank-space partials [4][kRdMaxChunks*512] fp32 for the merge at the end
+  constexpr int KROW = 72;                         // 144-byte rows keep the 16-byte fragment reads off each other's banks
+  constexpr int KU_BYTES = 2 * DH * KROW * 2, TB_BYTES = 4 * kRdMaxChunks * 512 * 4;
+  __shared__ __align__(16) unsigned char smem[KU_BYTES > TB_BYTES ? KU_BYTES : TB_BYTES];
+  uint16_t (*kus)[DH][KROW] = reinterpret_cast<uint16_t (*)[DH][KROW]>(smem);
+  float (*tbuf)[kRdMaxChunks * 512] = reinterpret_cast<float (*)[kRdMaxChunks * 512]>(smem);
 
-  const int s = blockIdx.x, b = blockIdx.z;
   const int groups = a.H / a.Hk / REP;             // q-head groups per kv head handled by separate blocks
+  const int s = blockIdx.x, b = blockIdx.z;
   const int hk = blockIdx.y / groups, grp = blockIdx.y % groups;
   const int h0 = hk * (a.H / a.Hk) + grp * REP;    // first q head of this block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -69,7 +75,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
 #pragma unroll
   for (int g = 0; g < REP; ++g)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) qv[g][t] = qs[g][t * 16 + lr];
+    for (int t = 0; t < NT; ++t) qv[g][t] = qs[g][(t / 4) * HALF + lr * 4 + (t % 4)];
 
   const int nchunk = (a.Rv + 511) / 512;
   float m_run[REP], l_run[REP];
@@ -89,8 +95,10 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
 
   for (int kt = k0; kt < k1; kt += kRdTileKeys * KS) {
     // KS key sub-tiles per pass share every k_u fragment: sub-tile j of this wave starts at kt + (4j + wave) * 16
-    if (kt + wave * 16 >= k1) continue;            // whole wave past the end (no block barrier in the loop)
-    // ---- K tiles = Pk[16 keys, R] @ k_u[h]^T on the matrix cores
+    // ---- K tiles = Pk[16 keys, R] @ k_u[h]^T on the matrix cores.  k_u streams through LDS in 64-wide chunks of r,
+    // loaded once per workgroup (thread -> row tid/2, 32 r) and double-buffered; Pk fragments come straight from
+    // global memory in the instruction's lane layout.  Waves past the end of the split keep pace (clamped keys)
+    // because the chunk hand-over is a block barrier.
     f32x4_t accs[KS][NT];
     const uint16_t* arow[KS];
 #pragma unroll
@@ -100,38 +108,72 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
       const int akey = min(kt + (4 * j + wave) * 16 + lr, k1 - 1);
       arow[j] = pk_b + (int64_t)akey * a.spk_s + lg * 8;
     }
-    const uint16_t* brow = ku_h + (int64_t)lr * a.ldku + lg * 8;
-#pragma unroll 2
-    for (int r0 = 0; r0 < a.Rk; r0 += 32) {
-      const bool in = r0 + lg * 8 < a.Rk;
-      bf16x8_t af[KS];
+    // LDS row t*16 + lr holds head dimension d = (t/4)*64 + lr*4 + t%4: a lane's accumulator tiles t = 0..3 then
+    // cover four consecutive d (one 8-byte read of the rotation tables per key), tiles t and t+4 the rotate-half pair
+    const int krow = tid >> 1, kcol = (tid & 1) * 32;
+    const int kd = ((krow >> 4) / 4) * HALF + (krow & 15) * 4 + ((krow >> 4) % 4);
+    const uint16_t* kug = ku_h + (int64_t)kd * a.ldku + kcol;
+    const int nstep = (a.Rk + 63) / 64;
+    u32x4_t kreg[4];
+    bf16x8_t af[KS][2];
+    const auto load_ku = [&](int r0) {
 #pragma unroll
-      for (int j = 0; j < KS; ++j) af[j] = in ? ld_frag(arow[j] + r0) : zero_frag();
-      bf16x8_t bf[NT];
+      for (int i = 0; i < 4; ++i)
+        kreg[i] = (r0 + kcol + i * 8 < a.Rk) ? *reinterpret_cast<const u32x4_t*>(kug + r0 + i * 8) : u32x4_t{0u, 0u, 0u, 0u};
+    };
+    const auto store_ku = [&](int buf) {
 #pragma unroll
-      for (int t = 0; t < NT; ++t) bf[t] = in ? ld_frag(brow + (int64_t)t * 16 * a.ldku + r0) : zero_frag();
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t*>(&kus[buf][krow][kcol + i * 8]) = kreg[i];
+    };
+    const auto load_pk = [&](int r0) {
 #pragma unroll
       for (int j = 0; j < KS; ++j)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j], bf[t], accs[j][t], 0, 0, 0);
+        for (int k = 0; k < 2; ++k) af[j][k] = (r0 + k * 32 + lg * 8 < a.Rk) ? ld_frag(arow[j] + r0 + k * 32) : zero_frag();
+    };
+    // (the barrier that ended the previous tile's last chunk also freed both buffers)
+    load_ku(0);
+    load_pk(0);
+    store_ku(0);
+    __syncthreads();
+    for (int st = 0; st < nstep; ++st) {
+      const int cur = st & 1;
+      if (st + 1 < nstep) load_ku((st + 1) * 64);
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        bf16x8_t bf[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][k * 32 + lg * 8]));
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+          for (int t = 0; t < NT; ++t) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][k], bf[t], accs[j][t], 0, 0, 0);
+      }
+      if (st + 1 < nstep) {
+        load_pk((st + 1) * 64);                    // lands while the chunk is handed over
+        store_ku(cur ^ 1);
+      }
+      __syncthreads();
     }
 #pragma unroll
     for (int j = 0; j < KS; ++j) {
     const int wkey0 = kt + (4 * j + wave) * 16;    // first key of this sub-tile
-    if (wkey0 >= k1) break;
+    if (wkey0 >= k1) break;                        // wave-uniform; later sub-tiles start even further out
     f32x4_t (&acc)[NT] = accs[j];
     // ---- rotate-half RoPE at absolute key positions (register-local: tiles t and t+4 pair up)
     if (a.cos) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int pos = min(wkey0 + lg * 4 + i, a.rope_len - 1);
+        const uint2 cw = *reinterpret_cast<const uint2*>(a.cos + (int64_t)pos * HALF + lr * 4);
+        const uint2 sw = *reinterpret_cast<const uint2*>(a.sin + (int64_t)pos * HALF + lr * 4);
+        const float cv[4] = {bf16_lo(cw.x), bf16_hi(cw.x), bf16_lo(cw.y), bf16_hi(cw.y)};
+        const float sv[4] = {bf16_lo(sw.x), bf16_hi(sw.x), bf16_lo(sw.y), bf16_hi(sw.y)};
 #pragma unroll
         for (int t = 0; t < NT / 2; ++t) {
-          const int idx = t * 16 + lr;
-          const float c = bf16_bits_to_f32(a.cos[(int64_t)pos * HALF + idx]), sn = bf16_bits_to_f32(a.sin[(int64_t)pos * HALF + idx]);
           const float x0 = acc[t][i], x1 = acc[t + NT / 2][i];
-          acc[t][i] = x0 * c - x1 * sn;
-          acc[t + NT / 2][i] = x0 * sn + x1 * c;
+          acc[t][i] = x0 * cv[t] - x1 * sv[t];
+          acc[t + NT / 2][i] = x0 * sv[t] + x1 * cv[t];
         }
       }
     }
@@ -272,19 +314,22 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     set_last_error("%s: cache / factor pointers and strides must be 16-byte aligned", fn);
     return kErrBadAlign;
   }
+  if (a.cos && (((reinterpret_cast<uintptr_t>(a.cos) | reinterpret_cast<uintptr_t>(a.sin)) & 7) != 0)) {
+    set_last_error("%s: rotation tables must be 8-byte aligned", fn);
+    return kErrBadAlign;
+  }
   const int rep = a.H / a.Hk;
   dim3 block(kRdThreads);
   // key sub-tiles per pass: long splits amortise every k_u fragment over more keys (any value is correct for any
   // length; short splits would only rebuild clamped keys)
   const int per = (a.S + a.nsplit - 1) / a.nsplit;
-  const int ks = per >= 512 ? 4 : (per >= 128 ? 2 : 1);
+  const int ks = per >= 128 ? 2 : 1;
   if (rep % 4 == 0) hipLaunchKernelGGL((rank_decode_partial_kernel<4, 1>), dim3(a.nsplit, a.Hk * (rep / 4), a.B), block, 0, st, a);
   else if (rep % 2 == 0) {
     if (ks >= 2) hipLaunchKernelGGL((rank_decode_partial_kernel<2, 2>), dim3(a.nsplit, a.Hk * (rep / 2), a.B), block, 0, st, a);
     else hipLaunchKernelGGL((rank_decode_partial_kernel<2, 1>), dim3(a.nsplit, a.Hk * (rep / 2), a.B), block, 0, st, a);
   } else {
-    if (ks == 4) hipLaunchKernelGGL((rank_decode_partial_kernel<1, 4>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
-    else if (ks == 2) hipLaunchKernelGGL((rank_decode_partial_kernel<1, 2>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
+    if (ks >= 2) hipLaunchKernelGGL((rank_decode_partial_kernel<1, 2>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
     else hipLaunchKernelGGL((rank_decode_partial_kernel<1, 1>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
   }
   hipError_t e = hipGetLastError();
