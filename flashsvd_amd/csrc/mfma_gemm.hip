@@ -16,7 +16,7 @@ namespace fsvd {
 typedef __bf16 gm_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float gm_f32x4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kGT = 256;            // threads: 2 x 2 waves
+constexpr int kGT4 = 256;           // threads of the four-wave form: 2 x 2 waves
 constexpr int kGBK = 64;            // K per step (the small tile takes 128 when K allows: half as many barriers)
 
 // WT: 16 x 16 accumulator tiles per wave and dimension: 4 -> 128 x 128 per workgroup, 2 -> 64 x 64 (problems with
@@ -33,10 +33,18 @@ struct ExpandEpi {
   int dst_by_position, dst_rows;
 };
 
-template <bool DUAL, int WT, int PF, bool EXPAND, int BK>
-__global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi ep) {
+// NW: waves per workgroup.  4: a wave owns a 16 WT x 16 WT block of the output tile (both matrices of the gate / up
+// pair).  8 (pair, 128 x 128 only): waves 0-3 accumulate the gate matrix and waves 4-7 the up matrix of the same
+// blocks, which halves the accumulators per wave (two waves per SIMD instead of one); the up halves cross to their
+// gate partners through LDS once, before the SwiGLU epilogue.
+template <bool DUAL, int WT, int PF, bool EXPAND, int BK, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi ep) {
   static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion uses the single 128 x 128 tile");
+  static_assert(NW == 4 || (NW == 8 && DUAL && WT == 4), "eight waves are the split form of the 128 x 128 pair tile");
+  constexpr int kGT = NW * 64;
+  constexpr bool SPLIT = NW == 8;
   constexpr int NM = DUAL ? 2 : 1;
+  constexpr int NMA = SPLIT ? 1 : NM;     // accumulator sets per wave
   constexpr int kGLd = BK + 8;            // LDS row stride in elements: 16 bytes of padding against bank conflicts
   constexpr int CPR = BK / 8;             // 16-byte pieces per tile row
   constexpr int NP = 32 * WT * CPR / kGT; // pieces per thread and operand
@@ -46,7 +54,8 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
   uint16_t* lds = reinterpret_cast<uint16_t*>(gm_smem);
   constexpr int kTile = kGBM * kGLd;                 // elements per operand tile
   constexpr int kStage = 2 * NM * kTile;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
+  const int tid = threadIdx.x, wave = (tid >> 6) & 3, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
+  const int mat = SPLIT ? (tid >> 8) : 0;  // split form: which matrix of the pair this wave accumulates
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.y * kGBM, n0 = blockIdx.x * kGBN;
   const int ksteps = a.K / BK;
@@ -92,9 +101,9 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
       }
   };
 
-  gm_f32x4_t acc[NM][WT][WT];
+  gm_f32x4_t acc[NMA][WT][WT];
 #pragma unroll
-  for (int m = 0; m < NM; ++m)
+  for (int m = 0; m < NMA; ++m)
 #pragma unroll
     for (int i = 0; i < WT; ++i)
 #pragma unroll
@@ -114,7 +123,8 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
 #pragma unroll
       for (int kk = 0; kk < BK / 32; ++kk) {
 #pragma unroll
-        for (int m = 0; m < NM; ++m) {
+        for (int ma = 0; ma < NMA; ++ma) {
+          const int m = SPLIT ? mat : ma;
           gm_bf16x8_t fx[WT], fw[WT];
 #pragma unroll
           for (int i = 0; i < WT; ++i) {
@@ -126,7 +136,7 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
           for (int i = 0; i < WT; ++i)
 #pragma unroll
             for (int j = 0; j < WT; ++j)
-              acc[m][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fx[i], fw[j], acc[m][i][j], 0, 0, 0);
+              acc[ma][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fx[i], fw[j], acc[ma][i][j], 0, 0, 0);
         }
       }
       if (ks + 1 < ksteps) {
@@ -138,6 +148,24 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
     }
   }
 
+  // split pair: the up accumulators travel to the gate wave of the same block (same lane, same tile indices)
+  gm_f32x4_t upv[SPLIT ? WT : 1][SPLIT ? WT : 1];
+  if (SPLIT) {
+    gm_f32x4_t* ex = reinterpret_cast<gm_f32x4_t*>(gm_smem);     // [WT*WT][256] 16-byte words = 64 KB of the stages
+    __syncthreads();                                             // every wave has finished reading the last stage
+    if (mat == 1) {
+#pragma unroll
+      for (int i = 0; i < WT; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) ex[(i * WT + j) * 256 + (tid & 255)] = acc[0][i][j];
+    }
+    __syncthreads();
+    if (mat == 1) return;
+#pragma unroll
+    for (int i = 0; i < WT; ++i)
+#pragma unroll
+      for (int j = 0; j < WT; ++j) upv[i][j] = ex[(i * WT + j) * 256 + (tid & 255)];
+  }
   // element e of lane l of tile (i, j): row m = i*16 + (l/16)*4 + e of x, column n = j*16 + l%16 of W
 #pragma unroll
   for (int i = 0; i < WT; ++i)
@@ -178,7 +206,7 @@ __global__ __launch_bounds__(kGT) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi e
         float v0 = acc[0][i][j][e];
         float v;
         if (DUAL) {
-          float v1 = acc[NM - 1][i][j][e];
+          float v1 = SPLIT ? upv[SPLIT ? i : 0][SPLIT ? j : 0][e] : acc[NMA - 1][i][j][e];
           if (a.mode == 0) {
             v0 = round_bf16(v0);
             v1 = round_bf16(v1);
@@ -200,7 +228,7 @@ bool gemm_tiles_apply(const MfmaArgs& a) {
   return a.B >= 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0;
 }
 
-template <bool DUAL, int WT, int BK>
+template <bool DUAL, int WT, int BK, int NW = 4>
 static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* who) {
   static bool granted = false;
   constexpr int BM = 32 * WT;
@@ -210,13 +238,13 @@ static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* wh
   constexpr int PF = (!DUAL && WT == 2 && BK == 64) ? 4 : 2;
   const size_t lds = (size_t)2 * 2 * (DUAL ? 2 : 1) * BM * kGLd * 2;
   if (lds > 64 * 1024 && !granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, PF, false, BK>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, PF, false, BK, NW>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
   }
   const dim3 grid((a.N + BM - 1) / BM, (a.B + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, PF, false, BK>), grid, dim3(kGT), lds, st, a, ExpandEpi{});
+  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, PF, false, BK, NW>), grid, dim3(NW * 64), lds, st, a, ExpandEpi{});
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
@@ -225,7 +253,7 @@ static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* wh
 int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
   // 128 x 128 tiles when they give every compute unit work, else 64 x 64
   const int64_t big = (int64_t)((a.N + 127) / 128) * ((a.B + 127) / 128);
-  if (big >= 192) return dual ? launch_gemm_tiles_t<true, 4, 64>(a, st, who) : launch_gemm_tiles_t<false, 4, 64>(a, st, who);
+  if (big >= 192) return dual ? launch_gemm_tiles_t<true, 4, 64, 8>(a, st, who) : launch_gemm_tiles_t<false, 4, 64>(a, st, who);
   if (dual) return launch_gemm_tiles_t<true, 2, 64>(a, st, who);
   return (a.K % 128) == 0 ? launch_gemm_tiles_t<false, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 2, 64>(a, st, who);
 }
@@ -244,7 +272,7 @@ int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
   constexpr int kGLd = kGBK + 8;
   const size_t lds = (size_t)2 * 2 * 128 * kGLd * 2;
   if (!granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<false, 4, PF, true, kGBK>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<false, 4, PF, true, kGBK, 4>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
@@ -253,7 +281,7 @@ int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
   MfmaArgs g{a.p, 0, 0, a.u, nullptr, a.ldu, a.bias, nullptr, 0, a.y, 0, rows, a.heads * 128, a.R, 0};
   ExpandEpi ep{a.cos, a.sin, a.rope_len, a.positions, a.M, a.sp_b, a.sp_m, a.sy_b, a.sy_m, a.sy_h, a.dst_by_position, a.dst_rows};
   const dim3 grid(a.heads, (rows + 127) / 128);
-  hipLaunchKernelGGL((gemm_tiles_kernel<false, 4, PF, true, kGBK>), grid, dim3(kGT), lds, st, g, ep);
+  hipLaunchKernelGGL((gemm_tiles_kernel<false, 4, PF, true, kGBK, 4>), grid, dim3(kGT4), lds, st, g, ep);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
