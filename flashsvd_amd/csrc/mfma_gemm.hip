@@ -37,23 +37,24 @@ struct ExpandEpi {
 // pair).  8 (pair, 128 x 128 only): waves 0-3 accumulate the gate matrix and waves 4-7 the up matrix of the same
 // blocks, which halves the accumulators per wave (two waves per SIMD instead of one); the up halves cross to their
 // gate partners through LDS once, before the SwiGLU epilogue.
-template <bool DUAL, int WT, int PF, bool EXPAND, int BK, int NW>
+template <bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi ep) {
-  static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion uses the single 128 x 128 tile");
-  static_assert(NW == 4 || (NW == 8 && DUAL && WT == 4), "eight waves are the split form of the 128 x 128 pair tile");
+  static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion takes whole 128-wide heads");
+  static_assert(NW == 4 || (NW == 8 && DUAL && WT == 4 && WTM == 4), "eight waves are the split form of the 128 x 128 pair tile");
   constexpr int kGT = NW * 64;
   constexpr bool SPLIT = NW == 8;
   constexpr int NM = DUAL ? 2 : 1;
   constexpr int NMA = SPLIT ? 1 : NM;     // accumulator sets per wave
   constexpr int kGLd = BK + 8;            // LDS row stride in elements: 16 bytes of padding against bank conflicts
   constexpr int CPR = BK / 8;             // 16-byte pieces per tile row
-  constexpr int NP = 32 * WT * CPR / kGT; // pieces per thread and operand
-  constexpr int kGBM = 32 * WT, kGBN = 32 * WT;
+  constexpr int NPX = 32 * WTM * CPR / kGT; // pieces per thread of an x tile
+  constexpr int NP = 32 * WT * CPR / kGT;   // ... of a W tile
+  constexpr int kGBM = 32 * WTM, kGBN = 32 * WT;
   extern __shared__ __align__(16) unsigned char gm_smem[];
   // [stage][operand: x0, (x1), W0, (W1)][128 rows][kGLd]
   uint16_t* lds = reinterpret_cast<uint16_t*>(gm_smem);
-  constexpr int kTile = kGBM * kGLd;                 // elements per operand tile
-  constexpr int kStage = 2 * NM * kTile;
+  constexpr int kTileX = kGBM * kGLd, kTileW = kGBN * kGLd;   // elements per operand tile
+  constexpr int kStage = NM * (kTileX + kTileW);
   const int tid = threadIdx.x, wave = (tid >> 6) & 3, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
   const int mat = SPLIT ? (tid >> 8) : 0;  // split form: which matrix of the pair this wave accumulates
   const int wm = wave >> 1, wn = wave & 1;
@@ -63,49 +64,51 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   // global -> register staging: a tile row is CPR 16-byte pieces; NP pieces per thread and operand
   constexpr int RPP = kGT / CPR;                      // rows covered by one pass of the workgroup
   const int ld_row = tid / CPR, ld_chunk = tid % CPR; // rows ld_row + RPP * j, j = 0..NP-1
-  const uint16_t* gx[NM][NP];
+  const uint16_t* gx[NM][NPX];
   const uint16_t* gw[NM][NP];
 #pragma unroll
-  for (int j = 0; j < NP; ++j) {
-    const int64_t xr = min(m0 + ld_row + RPP * j, a.B - 1), wr = min(n0 + ld_row + RPP * j, a.N - 1);
+  for (int j = 0; j < NPX; ++j) {
+    const int64_t xr = min(m0 + ld_row + RPP * j, a.B - 1);
     if (EXPAND) gx[0][j] = a.x + (xr / ep.M) * ep.sp_b + (xr % ep.M) * ep.sp_m + ld_chunk * 8;
     else gx[0][j] = a.x + xr * a.ldx + ld_chunk * 8;
+    if (DUAL) gx[NM - 1][j] = a.x + xr * a.ldx + a.up_off + ld_chunk * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < NP; ++j) {
+    const int64_t wr = min(n0 + ld_row + RPP * j, a.N - 1);
     gw[0][j] = a.W + wr * a.ldw + ld_chunk * 8;
-    if (DUAL) {
-      gx[NM - 1][j] = a.x + xr * a.ldx + a.up_off + ld_chunk * 8;
-      gw[NM - 1][j] = a.W2 + wr * a.ldw + ld_chunk * 8;
-    }
+    if (DUAL) gw[NM - 1][j] = a.W2 + wr * a.ldw + ld_chunk * 8;
   }
   // PF register sets hold the global loads of the next PF steps (set s % PF belongs to step s); a set is written
   // to the idle LDS stage one step before its products and refilled at once with the loads of step s + PF
-  u32x4_t rx[PF][NM][NP], rw[PF][NM][NP];
+  u32x4_t rx[PF][NM][NPX], rw[PF][NM][NP];
   auto load_regs = [&](int set, int ks) {
     const int k = min(ks, ksteps - 1) * BK;          // past the end: a valid address, never used
 #pragma unroll
-    for (int m = 0; m < NM; ++m)
+    for (int m = 0; m < NM; ++m) {
 #pragma unroll
-      for (int j = 0; j < NP; ++j) {
-        rx[set][m][j] = *reinterpret_cast<const u32x4_t*>(gx[m][j] + k);
-        rw[set][m][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(gw[m][j] + k));
-      }
+      for (int j = 0; j < NPX; ++j) rx[set][m][j] = *reinterpret_cast<const u32x4_t*>(gx[m][j] + k);
+#pragma unroll
+      for (int j = 0; j < NP; ++j) rw[set][m][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(gw[m][j] + k));
+    }
   };
   auto store_lds = [&](int set, int stage) {
     uint16_t* base = lds + stage * kStage;
 #pragma unroll
-    for (int m = 0; m < NM; ++m)
+    for (int m = 0; m < NM; ++m) {
 #pragma unroll
-      for (int j = 0; j < NP; ++j) {
-        const int off = (ld_row + RPP * j) * kGLd + ld_chunk * 8;
-        *reinterpret_cast<u32x4_t*>(base + m * kTile + off) = rx[set][m][j];
-        *reinterpret_cast<u32x4_t*>(base + (NM + m) * kTile + off) = rw[set][m][j];
-      }
+      for (int j = 0; j < NPX; ++j) *reinterpret_cast<u32x4_t*>(base + m * kTileX + (ld_row + RPP * j) * kGLd + ld_chunk * 8) = rx[set][m][j];
+#pragma unroll
+      for (int j = 0; j < NP; ++j)
+        *reinterpret_cast<u32x4_t*>(base + NM * kTileX + m * kTileW + (ld_row + RPP * j) * kGLd + ld_chunk * 8) = rw[set][m][j];
+    }
   };
 
-  gm_f32x4_t acc[NMA][WT][WT];
+  gm_f32x4_t acc[NMA][WTM][WT];
 #pragma unroll
   for (int m = 0; m < NMA; ++m)
 #pragma unroll
-    for (int i = 0; i < WT; ++i)
+    for (int i = 0; i < WTM; ++i)
 #pragma unroll
       for (int j = 0; j < WT; ++j) acc[m][i][j] = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
 
@@ -125,15 +128,17 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
 #pragma unroll
         for (int ma = 0; ma < NMA; ++ma) {
           const int m = SPLIT ? mat : ma;
-          gm_bf16x8_t fx[WT], fw[WT];
+          gm_bf16x8_t fx[WTM], fw[WT];
+#pragma unroll
+          for (int i = 0; i < WTM; ++i)
+            fx[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + m * kTileX + (wm * 16 * WTM + i * 16 + lr) * kGLd + kk * 32 + lg * 8);
 #pragma unroll
           for (int i = 0; i < WT; ++i) {
-            fx[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + m * kTile + (wm * 16 * WT + i * 16 + lr) * kGLd + kk * 32 + lg * 8);
             const int wrow = EXPAND ? (i < 2 ? wn * 32 + i * 16 : 64 + wn * 32 + (i - 2) * 16) : wn * 16 * WT + i * 16;
-            fw[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + (NM + m) * kTile + (wrow + lr) * kGLd + kk * 32 + lg * 8);
+            fw[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + NM * kTileX + m * kTileW + (wrow + lr) * kGLd + kk * 32 + lg * 8);
           }
 #pragma unroll
-          for (int i = 0; i < WT; ++i)
+          for (int i = 0; i < WTM; ++i)
 #pragma unroll
             for (int j = 0; j < WT; ++j)
               acc[ma][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fx[i], fw[j], acc[ma][i][j], 0, 0, 0);
@@ -168,10 +173,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   }
   // element e of lane l of tile (i, j): row m = i*16 + (l/16)*4 + e of x, column n = j*16 + l%16 of W
 #pragma unroll
-  for (int i = 0; i < WT; ++i)
+  for (int i = 0; i < WTM; ++i)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int m = m0 + wm * 16 * WT + i * 16 + lg * 4 + e;
+      const int m = m0 + wm * 16 * WTM + i * 16 + lg * 4 + e;
       if (m >= a.B) continue;
       if (EXPAND) {
         const int b = m / ep.M, t = m - b * ep.M;
@@ -238,13 +243,13 @@ static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* wh
   constexpr int PF = (!DUAL && WT == 2 && BK == 64) ? 4 : 2;
   const size_t lds = (size_t)2 * 2 * (DUAL ? 2 : 1) * BM * kGLd * 2;
   if (lds > 64 * 1024 && !granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, PF, false, BK, NW>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, WT, PF, false, BK, NW>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
   }
   const dim3 grid((a.N + BM - 1) / BM, (a.B + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, PF, false, BK, NW>), grid, dim3(NW * 64), lds, st, a, ExpandEpi{});
+  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, WT, PF, false, BK, NW>), grid, dim3(NW * 64), lds, st, a, ExpandEpi{});
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
@@ -265,14 +270,16 @@ bool expand_tiles_apply(const ExpandArgs& a) {
          (a.ldu % 8) == 0;
 }
 
-int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
+template <int WTM>
+static int launch_expand_tiles_t(const ExpandArgs& a, hipStream_t st) {
   const char* who = "fsvd_lowrank_expand_heads";
   static bool granted = false;
   constexpr int PF = 2;
   constexpr int kGLd = kGBK + 8;
-  const size_t lds = (size_t)2 * 2 * 128 * kGLd * 2;
+  constexpr int BM = 32 * WTM;
+  const size_t lds = (size_t)2 * (BM + 128) * kGLd * 2;
   if (!granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<false, 4, PF, true, kGBK, 4>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<false, WTM, 4, PF, true, kGBK, 4>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
@@ -280,11 +287,17 @@ int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
   const int rows = a.B * a.M;
   MfmaArgs g{a.p, 0, 0, a.u, nullptr, a.ldu, a.bias, nullptr, 0, a.y, 0, rows, a.heads * 128, a.R, 0};
   ExpandEpi ep{a.cos, a.sin, a.rope_len, a.positions, a.M, a.sp_b, a.sp_m, a.sy_b, a.sy_m, a.sy_h, a.dst_by_position, a.dst_rows};
-  const dim3 grid(a.heads, (rows + 127) / 128);
-  hipLaunchKernelGGL((gemm_tiles_kernel<false, 4, PF, true, kGBK, 4>), grid, dim3(kGT4), lds, st, g, ep);
+  const dim3 grid(a.heads, (rows + BM - 1) / BM);
+  hipLaunchKernelGGL((gemm_tiles_kernel<false, WTM, 4, PF, true, kGBK, 4>), grid, dim3(kGT4), lds, st, g, ep);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
+}
+
+int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
+  // a column tile is always one head; 128 token rows per workgroup when that gives every compute unit two tiles, else 64
+  const int64_t big = (int64_t)a.heads * (((int64_t)a.B * a.M + 127) / 128);
+  return big >= 384 ? launch_expand_tiles_t<4>(a, st) : launch_expand_tiles_t<2>(a, st);
 }
 
 }  // namespace fsvd
