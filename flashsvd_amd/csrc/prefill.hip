@@ -248,8 +248,9 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
 //     (K row-major with a padded stride, V transposed: four adjacent keys per 8-byte write, key column XOR-ed
 //     with 8 * (d / 8 % 8) to spread the 16 dimension blocks over the banks).
 // ---------------------------------------------------------------------------------------------
+template <int MI>
 __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(PrefillAttnArgs a) {
-  constexpr int DH = 128, BN = 64, QW = 32, KSTR = DH + 8, PSTR = BN + 8, VSTR = BN + 8;
+  constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, KSTR = DH + 8, PSTR = BN + 8, VSTR = BN + 8;
   extern __shared__ __align__(16) unsigned char pw_smem[];
   uint16_t (*Ks)[KSTR] = reinterpret_cast<uint16_t (*)[KSTR]>(pw_smem);                              // [BN][KSTR]
   uint16_t (*Vt)[VSTR] = reinterpret_cast<uint16_t (*)[VSTR]>(pw_smem + (size_t)BN * KSTR * 2);       // [DH][VSTR]
@@ -261,28 +262,28 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, lg = lane >> 4;
   const int q0 = a.q_pos0 ? a.q_pos0[b] : 0;
-  const int m_base = mt * 128 + wave * QW;
+  const int m_base = mt * BM + wave * QW;
   const int n_keys_all = max(1, min(q0 + a.M, a.S));
 
-  bf16x8_t qf[2][4];
+  bf16x8_t qf[MI][4];
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi) {
+  for (int mi = 0; mi < MI; ++mi) {
     const int m = min(m_base + mi * 16 + lr, a.M - 1);
     const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)m * a.sq_m + (int64_t)h * a.sq_h + lg * 8;
 #pragma unroll
     for (int st = 0; st < 4; ++st) qf[mi][st] = pf_ld(qp + st * 32);
   }
-  float m_run[2][4], l_run[2][4];
-  f32x4_t o[2][8];
+  float m_run[MI][4], l_run[MI][4];
+  f32x4_t o[MI][8];
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi) {
+  for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) { m_run[mi][i] = -INFINITY; l_run[mi][i] = 0.f; }
 #pragma unroll
     for (int t = 0; t < 8; ++t) o[mi][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  const int last_m = min(mt * 128 + 127, a.M - 1);
+  const int last_m = min(mt * BM + BM - 1, a.M - 1);
   const int k_end = a.causal ? min(n_keys_all, q0 + last_m + 1) : n_keys_all;
   // last key this wave's rows may see: tiles past it are skipped by the wave (it still takes part in the staging)
   const int wave_end = a.causal ? min(n_keys_all, q0 + min(m_base + QW - 1, a.M - 1) + 1) : n_keys_all;
@@ -325,15 +326,15 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
     if (n0 + BN < k_end) request(n0 + BN);
     if (n0 >= wave_end) continue;   // nothing this wave's rows may see (wave-uniform)
 
-    // ---- S = Q K^T for 32 rows x 64 keys
-    f32x4_t sacc[2][4];
+    // ---- S = Q K^T for 16 MI rows x 64 keys
+    f32x4_t sacc[MI][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       bf16x8_t kf[4];
 #pragma unroll
       for (int st = 0; st < 4; ++st) kf[st] = pf_ld(&Ks[j * 16 + lr][st * 32 + lg * 8]);
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) {
+      for (int mi = 0; mi < MI; ++mi) {
         sacc[mi][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int st = 0; st < 4; ++st) sacc[mi][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[mi][st], kf[st], sacc[mi][j], 0, 0, 0);
@@ -341,7 +342,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
     }
     // ---- masks + online softmax on the accumulator layout (rows lg*4+i, key column j*16+lr), P to LDS
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int m = m_base + mi * 16 + lg * 4 + i;
@@ -384,9 +385,9 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
     // ---- O += P V : A = P rows (keys contiguous), B = Vt rows (keys contiguous, swizzled)
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
-      bf16x8_t pa[2], pb[2];
+      bf16x8_t pa[MI], pb[MI];
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) {
+      for (int mi = 0; mi < MI; ++mi) {
         pa[mi] = pf_ld(&Ps[wave][mi * 16 + lr][st * 32 + lg * 8]);
         pb[mi] = pf_ld(&Pl[wave][mi * 16 + lr][st * 32 + lg * 8]);
       }
@@ -394,7 +395,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
       for (int t = 0; t < 8; ++t) {
         const bf16x8_t vf = pf_ld(&Vt[t * 16 + lr][(st * 32 + lg * 8) ^ (8 * ((2 * t + (lr >> 3)) & 7))]);
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi) {
+        for (int mi = 0; mi < MI; ++mi) {
           o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[mi], vf, o[mi][t], 0, 0, 0);
           o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pb[mi], vf, o[mi][t], 0, 0, 0);
         }
@@ -404,7 +405,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
 
   // ---- normalise and store; rows with no visible key give 0
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi)
+  for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = m_base + mi * 16 + lg * 4 + i;
@@ -444,15 +445,18 @@ int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
     return kErrBadAlign;
   }
   if (a.M >= 128) {   // long prompts: 128 queries per workgroup, K / V tiles shared through LDS
-    constexpr size_t lds = (size_t)64 * 136 * 2 + (size_t)128 * 72 * 2 + (size_t)2 * 4 * 32 * 72 * 2;
+    // 128 query rows per workgroup when that gives every compute unit work, else 64 (half the rows per wave)
+    const bool wide = (int64_t)((a.M + 127) / 128) * a.H * a.B >= 384;
+    const size_t lds = (size_t)64 * 136 * 2 + (size_t)128 * 72 * 2 + (size_t)2 * 4 * (wide ? 32 : 16) * 72 * 2;
     static bool granted = false;
     if (!granted) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_wide_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<2>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)64 * 136 * 2 + (size_t)128 * 72 * 2 + (size_t)2 * 4 * 32 * 72 * 2));
       if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", fn, lds, hipGetErrorString(e)); return kErrLaunch; }
       granted = true;
     }
-    hipLaunchKernelGGL(attn_prefill_wide_kernel, dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
+    if (wide) hipLaunchKernelGGL(attn_prefill_wide_kernel<2>, dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
+    else hipLaunchKernelGGL(attn_prefill_wide_kernel<1>, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), lds, st, a);
   } else {
     hipLaunchKernelGGL(attn_prefill_kernel, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), 0, st, a);
   }

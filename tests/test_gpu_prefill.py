@@ -100,6 +100,21 @@ def test_expand_and_prefill_attention_primitives():
         assert_close_bf16(out[:, m], refm, f"row {m}", **bounds(refm))
 
 
+def test_prefill_attention_128_row_tiles():
+    """Enough (row tile, head, batch) triples for the 128-row form of the prompt attention (two 16-row blocks per wave);
+    grouped heads, a prefix already in the cache, a ragged last tile."""
+    from flashsvd_amd import hip_ops
+    B, M, H, Hk, dh, S, start = 3, 520, 32, 8, 128, 560, 29
+    kfull, vfull = rand_bf16(B, S, Hk, dh, seed=31), rand_bf16(B, S, Hk, dh, seed=32)
+    q = rand_bf16(B, M, H, dh, seed=33)
+    pos0 = torch.full((B,), start, dtype=torch.int32, device="cuda")
+    out = hip_ops.attn_prefill(q.cuda(), kfull.cuda(), vfull.cuda(), q_pos0=pos0, causal=True)
+    for m in (0, 15, 16, 127, 128, 300, 511, 512, M - 1):
+        n = start + m + 1
+        refm = O.dense_decode_attn(q[:, m], kfull[:, :n], vfull[:, :n])
+        assert_close_bf16(out[:, m], refm, f"row {m}", **bounds(refm))
+
+
 @pytest.mark.parametrize("B,M,R", [(1, 512, 1024), (2, 130, 64), (3, 50, 192)])
 def test_expand_long_prompts_tiled_kernel(B, M, R):
     """128 token rows and more with a rank that is a multiple of 64: the LDS-tiled expansion; same result as the
