@@ -48,6 +48,9 @@ def _parse():
                          "per-operator kernels per token; both: time both, the headline value is the persistent step")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only time the prompt pass (matrix-core kernels): W untimed and K timed passes over a 512-token prompt")
+    ap.add_argument("--stress", action="store_true",
+                    help="time the attention kernels of the stress configuration per layer (attention rank 1664: rank-space decode "
+                         "at batch 16 x context 4096, prompt attention path at 8 x 2048) and print their own JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device copy 10 times (the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counters are scaled against) and exit")
@@ -377,6 +380,70 @@ def run_dense(args):
     return dict(tok_s=args.steps / dt, ms_per_step=dt * 1000.0 / args.steps)
 
 
+def run_stress():
+    """Stress configuration of the 7B shape at parameter ratio ~0.8 (attention rank 1664), one layer's attention kernels:
+    decode at batch 16 over a 4096-token rank-space cache (K rebuilt in-kernel), and the prompt path at 8 x 2048 tokens
+    (q / k / v head expansion + RoPE + causal attention).  Matrix-core bound: flop / time against the bf16 peak."""
+    import torch
+    from flashsvd_amd import hip_ops
+    from flashsvd_amd.kernels.rank_decode import rank_decode
+
+    def timed(fn, reps=5, warm=2):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e-3 / reps
+
+    g = torch.Generator(device="cuda").manual_seed(0)
+    rnd = lambda *shape, std=1.0: (torch.randn(*shape, device="cuda", generator=g) * std).to(torch.bfloat16)
+    B, H, Hk, Dh, R, ctx = 16, 32, 32, 128, 1664, 4096
+    S = ctx + 4
+    q, pk, pv = rnd(B, H, Dh), rnd(B, S, R, std=0.5), rnd(B, S, R, std=0.5)
+    ku, vu = rnd(Hk * Dh, R, std=R ** -0.5), rnd(Hk * Dh, R, std=R ** -0.5)
+    ang = torch.arange(S, device="cuda", dtype=torch.float32)[:, None] * (1.0 / 10000.0 ** (torch.arange(0, Dh // 2, device="cuda").float() / (Dh // 2)))
+    cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)     # half tables [S, Dh/2]
+    lens = torch.full((B,), ctx, dtype=torch.int32, device="cuda")
+    out = torch.empty(B, H, Dh, device="cuda", dtype=torch.bfloat16)
+    t_dec = timed(lambda: rank_decode(q, pk, pv, ku, vu, cos, sin, lens, num_kv_heads=Hk, rotate_q=True, out=out))
+    flop_dec = 2.0 * B * ctx * R * Hk * Dh + 2.0 * B * H * ctx * R
+    cache_bytes = 2 * B * ctx * R * 2
+    del pk, pv
+    Bp, T = 8, 2048
+    p = rnd(Bp, T, 3 * R, std=0.5)
+    qu = rnd(H * Dh, R, std=R ** -0.5)
+    kc = torch.zeros(Bp, T, Hk, Dh, device="cuda", dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    qb = torch.empty(Bp, T, H, Dh, device="cuda", dtype=torch.bfloat16)
+    ob = torch.empty_like(qb)
+    pos0 = torch.zeros(Bp, dtype=torch.int32, device="cuda")
+
+    def expand():
+        hip_ops.lowrank_expand_heads(p[..., :R], qu, num_heads=H, head_dim=Dh, out=qb, cos=cos, sin=sin, positions=pos0)
+        hip_ops.lowrank_expand_heads(p[..., R:2 * R], ku, num_heads=Hk, head_dim=Dh, out=kc, cos=cos, sin=sin, positions=pos0, dst_by_position=True)
+        hip_ops.lowrank_expand_heads(p[..., 2 * R:], vu, num_heads=Hk, head_dim=Dh, out=vc, positions=pos0, dst_by_position=True)
+
+    t_exp = timed(expand, reps=3, warm=1)
+    t_att = timed(lambda: hip_ops.attn_prefill(qb, kc, vc, q_pos0=pos0, causal=True, out=ob), reps=3, warm=1)
+    flop_exp = 3 * 2.0 * Bp * T * R * H * Dh
+    flop_att = 2 * 2.0 * Bp * H * Dh * T * (T + 1) / 2
+    peak = 2500e12
+    return {
+        "rank_space_decode_attention_b16_ctx4096_r1664": {
+            "ms_per_layer": t_dec * 1e3, "flop": flop_dec, "TFLOPs": flop_dec / t_dec / 1e12, "frac_of_bf16_mfma_peak": flop_dec / t_dec / peak,
+            "cache_bytes": cache_bytes, "cache_GB/s": cache_bytes / t_dec / 1e9},
+        "prompt_attention_path_8x2048_r1664": {
+            "expand_qkv_ms": t_exp * 1e3, "expand_TFLOPs": flop_exp / t_exp / 1e12, "attention_ms": t_att * 1e3,
+            "attention_TFLOPs": flop_att / t_att / 1e12, "ms_per_layer": (t_exp + t_att) * 1e3,
+            "frac_of_bf16_mfma_peak": (flop_exp + flop_att) / (t_exp + t_att) / peak},
+    }
+
+
 def run_cpu_baseline():
     """The CPU oracle in fp32 (the precision of the reference's CPU path) on a bounded sample:
     2 of the 32 layers + final norm + lm_head, prompt 16, 6 greedy tokens; per-token decode time is
@@ -434,6 +501,10 @@ def main():
         return
     from flashsvd_amd import _lib
     _lib.load()
+    if args.stress:
+        print(json.dumps({"metric": "stress attention kernels, 7B-shape rank-0.8, per layer", "n_gpus": 1, "dtype": "bf16", "data": "synthetic",
+                          "stress": run_stress()}))
+        return
     lr = run_lowrank(args)
     if args.prefill_only:
         print(json.dumps({"metric": "prefill tok/s, 7B-shape rank-0.5 bs1 prompt 512", "value": lr["prefill"]["tok_s"], "unit": "tok/s",
