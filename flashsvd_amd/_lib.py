@@ -88,6 +88,7 @@ SIGNATURES = {
     "fsvd_decode_step_workgroups": (c_int, []),
     "fsvd_decode_step_prepare": (c_int, [c_void_p, c_int, c_int]),
     "fsvd_decode_step_validate": (c_int, [c_void_p, c_int, c_int]),
+    "fsvd_set_workspace": (c_int, [c_void_p, c_size_t, c_void_p]),
     "fsvd_decode_step": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
     "fsvd_decode_step_trace": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "fsvd_mlp_dual_split": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,

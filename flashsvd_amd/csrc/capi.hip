@@ -18,6 +18,22 @@ void set_last_error(const char* fmt, ...) {
 }
 }  // namespace fsvd
 
+namespace fsvd {
+// scratch registered by the caller for the K-split projections, one per device
+constexpr int kMaxDevices = 16;
+constexpr size_t kWsCounterBytes = 64 * 1024;
+static SplitWorkspace g_split_ws[kMaxDevices] = {};
+SplitWorkspace split_workspace() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SplitWorkspace{nullptr, 0, nullptr, 0};
+  return g_split_ws[dev];
+}
+__global__ void ws_clear_kernel(int32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+}  // namespace fsvd
+
 using namespace fsvd;
 
 #define FSVD_REQUIRE_PTR(p, fn)                             \
@@ -33,6 +49,22 @@ extern "C" {
 
 int fsvd_version(void) { return 100; }
 const char* fsvd_last_error(void) { return g_last_error; }
+
+int fsvd_set_workspace(void* ws, size_t bytes, void* stream) {
+  const char* fn = "fsvd_set_workspace";
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) { set_last_error("%s: no current device", fn); return kErrLaunch; }
+  if (ws == nullptr) { g_split_ws[dev] = SplitWorkspace{nullptr, 0, nullptr, 0}; return kOk; }
+  if ((reinterpret_cast<uintptr_t>(ws) & 255) != 0) { set_last_error("%s: buffer must be 256-byte aligned", fn); return kErrBadAlign; }
+  if (bytes < (size_t)1 << 20) { set_last_error("%s: %zu bytes is too small (1 MiB at least)", fn, bytes); return kErrBadShape; }
+  const int ncount = (int)(kWsCounterBytes / sizeof(int32_t));
+  hipLaunchKernelGGL(ws_clear_kernel, dim3((ncount + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<int32_t*>(ws), ncount);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+  g_split_ws[dev] = SplitWorkspace{reinterpret_cast<float*>(static_cast<char*>(ws) + kWsCounterBytes), (bytes - kWsCounterBytes) / sizeof(float),
+                                   static_cast<int32_t*>(ws), ncount};
+  return kOk;
+}
 
 int fsvd_linear(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* bias, const void* norm_w, float eps,
                 const void* res, int64_t ldres, void* y, int64_t ldy, int B, int N, int K, int cfg, void* stream) {

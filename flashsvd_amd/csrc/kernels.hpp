@@ -143,9 +143,17 @@ struct MfmaArgs {
   const uint16_t* bias; const uint16_t* res; int64_t ldres;
   uint16_t* y; int64_t ldy;
   int B, N, K, mode;
+  // K split over gridDim.z workgroups per output tile (filled by the launcher when a workspace is registered):
+  // fp32 partial tiles and one arrival counter per tile; the last workgroup to arrive adds the partials in order
+  int ksplit; float* ws_part; int32_t* ws_count;
 };
+// caller-owned scratch of the current device for the K-split projections (null when none is registered)
+struct SplitWorkspace { float* part; size_t part_floats; int32_t* count; int ncount; };
+SplitWorkspace split_workspace();                                            // capi.hip
 bool gemm_tiles_apply(const MfmaArgs& a);                                   // mfma_gemm.hip: 128 rows and more
 int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* who);
+bool gemm_rows_apply(const MfmaArgs& a);                                    // mfma_gemm.hip: 5..127 rows, K split
+int launch_gemm_rows(const MfmaArgs& a, bool dual, hipStream_t st, const char* who);
 
 int launch_linear(const LinearArgs& a, int cfg, hipStream_t st);
 // matrix-core path for 5+ rows (mfma_gemv.hip); launch_linear / launch_swiglu route to it when cfg == 0

@@ -8,6 +8,8 @@
 // the idle LDS stage one step before their products.  Epilogue as in the vector kernels: bias, ONE rounding to bf16,
 // residual — or, for the gate / up pair, SwiGLU in either rounding mode — or the head expansion of the prompt pass
 // (RoPE, store into the query buffer or the cache rows).  Every weight is read once per 128 (64) rows of x.
+#include <algorithm>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -59,7 +61,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   const int mat = SPLIT ? (tid >> 8) : 0;  // split form: which matrix of the pair this wave accumulates
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.y * kGBM, n0 = blockIdx.x * kGBN;
-  const int ksteps = a.K / BK;
+  // this workgroup's share of the K steps (all of them unless K is split over gridDim.z)
+  const int ksteps_all = a.K / BK;
+  const int kper = (ksteps_all + (int)gridDim.z - 1) / (int)gridDim.z;
+  const int kbeg = min((int)blockIdx.z * kper, ksteps_all);
+  const int ksteps = max(1, min(kper, ksteps_all - kbeg));   // a share past the end re-reads the last step and adds zero
+  const bool kdead = kbeg >= ksteps_all;
 
   // global -> register staging: a tile row is CPR 16-byte pieces; NP pieces per thread and operand
   constexpr int RPP = kGT / CPR;                      // rows covered by one pass of the workgroup
@@ -83,7 +90,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   // to the idle LDS stage one step before its products and refilled at once with the loads of step s + PF
   u32x4_t rx[PF][NM][NPX], rw[PF][NM][NP];
   auto load_regs = [&](int set, int ks) {
-    const int k = min(ks, ksteps - 1) * BK;          // past the end: a valid address, never used
+    const int k = min(kbeg + min(ks, ksteps - 1), ksteps_all - 1) * BK;   // past the end: a valid address, never used
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
 #pragma unroll
@@ -153,6 +160,55 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
     }
   }
 
+  // K split: park the partial tile (thread-major 16-byte words, coalesced), count arrivals; the last workgroup of a
+  // tile adds all partials in split order (its own included, so the sum does not depend on who came last)
+  if (gridDim.z > 1) {
+    constexpr int WPT = NMA * WTM * WT;                          // 16-byte words per thread
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    gm_f32x4_t* part = reinterpret_cast<gm_f32x4_t*>(a.ws_part) + (size_t)tile * gridDim.z * WPT * kGT;
+    gm_f32x4_t* mine = part + (size_t)blockIdx.z * WPT * kGT;
+    // write-through agent-scope stores (they do not stay dirty in this XCD's L2), all of them acknowledged before the
+    // arrival is counted; the reader below uses agent-scope loads, which do not look into its own L2.  No fence: a
+    // release or acquire fence per workgroup writes back / empties a whole L2 under the weight stream of the others
+#pragma unroll
+    for (int m = 0; m < NMA; ++m)
+#pragma unroll
+      for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) {
+          const gm_f32x4_t v = kdead ? gm_f32x4_t{0.f, 0.f, 0.f, 0.f} : acc[m][i][j];
+          unsigned long long* dst = reinterpret_cast<unsigned long long*>(mine + ((m * WTM + i) * WT + j) * kGT + tid);
+          __hip_atomic_store(dst, ((unsigned long long)__float_as_uint(v[1]) << 32) | __float_as_uint(v[0]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(dst + 1, ((unsigned long long)__float_as_uint(v[3]) << 32) | __float_as_uint(v[2]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    int* flag = reinterpret_cast<int*>(gm_smem);
+    if (tid == 0) {
+      const int prev = atomicAdd(a.ws_count + tile, 1);
+      const int last = prev == (int)gridDim.z - 1;
+      if (last) a.ws_count[tile] = 0;                            // ready for the next launch
+      *flag = last;
+    }
+    __syncthreads();
+    if (*flag == 0) return;
+#pragma unroll
+    for (int m = 0; m < NMA; ++m)
+#pragma unroll
+      for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) {
+          gm_f32x4_t sum = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
+          for (int z = 0; z < (int)gridDim.z; ++z) {
+            const unsigned long long* src = reinterpret_cast<const unsigned long long*>(part + (size_t)z * WPT * kGT + ((m * WTM + i) * WT + j) * kGT + tid);
+            const unsigned long long lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned long long hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            sum += gm_f32x4_t{__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)), __uint_as_float((uint32_t)hi),
+                              __uint_as_float((uint32_t)(hi >> 32))};
+          }
+          acc[m][i][j] = sum;
+        }
+  }
   // split pair: the up accumulators travel to the gate wave of the same block (same lane, same tile indices)
   gm_f32x4_t upv[SPLIT ? WT : 1][SPLIT ? WT : 1];
   if (SPLIT) {
@@ -233,23 +289,42 @@ bool gemm_tiles_apply(const MfmaArgs& a) {
   return a.B >= 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0;
 }
 
-template <bool DUAL, int WT, int BK, int NW = 4>
-static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* who) {
+// K split for a grid of `tiles` workgroups: enough shares to give every compute unit two workgroups, at least four
+// K steps per share, and only as many as the registered workspace holds (1 = no split)
+static int pick_ksplit(int64_t tiles, int ksteps, size_t floats_per_share, const SplitWorkspace& ws) {
+  if (ws.part == nullptr || tiles >= 512 || tiles > ws.ncount) return 1;
+  int z = (int)((512 + tiles - 1) / tiles);
+  z = std::min(z, std::min(16, ksteps / 4));
+  while (z > 1 && (size_t)tiles * z * floats_per_share > ws.part_floats) --z;
+  return std::max(z, 1);
+}
+
+template <bool DUAL, int WTM, int WT, int BK, int NW = 4>
+static int launch_gemm_tiles_t(const MfmaArgs& a0, hipStream_t st, const char* who) {
   static bool granted = false;
-  constexpr int BM = 32 * WT;
+  constexpr int BM = 32 * WTM, BN = 32 * WT;
   constexpr int kGLd = BK + 8;
   // register sets in flight: deep for the small single tile (few workgroups, latency-bound), two where a deeper
   // pipeline would cost a resident wave per SIMD
-  constexpr int PF = (!DUAL && WT == 2 && BK == 64) ? 4 : 2;
-  const size_t lds = (size_t)2 * 2 * (DUAL ? 2 : 1) * BM * kGLd * 2;
+  constexpr int PF = (!DUAL && WT == 2 && WTM == 2 && BK == 64) ? 4 : 2;
+  const size_t lds = (size_t)2 * (DUAL ? 2 : 1) * (BM + BN) * kGLd * 2;
   if (lds > 64 * 1024 && !granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WT, WT, PF, false, BK, NW>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WTM, WT, PF, false, BK, NW>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
   }
-  const dim3 grid((a.N + BM - 1) / BM, (a.B + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WT, WT, PF, false, BK, NW>), grid, dim3(NW * 64), lds, st, a, ExpandEpi{});
+  MfmaArgs a = a0;
+  dim3 grid((a.N + BN - 1) / BN, (a.B + BM - 1) / BM, 1);
+  const SplitWorkspace ws = split_workspace();
+  constexpr size_t share = (size_t)(DUAL && NW == 4 ? 2 : 1) * WTM * WT * 4 * NW * 64;   // floats one workgroup parks
+  // only the 32-row tiles split K: from 128 rows on a projection has enough tiles that parking and re-reading the
+  // partial tiles costs what the extra workgroups gain (measured at 512 rows: 42 -> 45 us, 25 -> 23 us, 64 -> 64 us)
+  a.ksplit = WTM == 1 ? pick_ksplit((int64_t)grid.x * grid.y, a.K / BK, share, ws) : 1;
+  a.ws_part = ws.part;
+  a.ws_count = ws.count;
+  grid.z = a.ksplit;
+  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WTM, WT, PF, false, BK, NW>), grid, dim3(NW * 64), lds, st, a, ExpandEpi{});
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
@@ -258,9 +333,21 @@ static int launch_gemm_tiles_t(const MfmaArgs& a, hipStream_t st, const char* wh
 int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
   // 128 x 128 tiles when they give every compute unit work, else 64 x 64
   const int64_t big = (int64_t)((a.N + 127) / 128) * ((a.B + 127) / 128);
-  if (big >= 192) return dual ? launch_gemm_tiles_t<true, 4, 64, 8>(a, st, who) : launch_gemm_tiles_t<false, 4, 64>(a, st, who);
-  if (dual) return launch_gemm_tiles_t<true, 2, 64>(a, st, who);
-  return (a.K % 128) == 0 ? launch_gemm_tiles_t<false, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 2, 64>(a, st, who);
+  if (big >= 192) return dual ? launch_gemm_tiles_t<true, 4, 4, 64, 8>(a, st, who) : launch_gemm_tiles_t<false, 4, 4, 64>(a, st, who);
+  if (dual) return launch_gemm_tiles_t<true, 2, 2, 64>(a, st, who);
+  return (a.K % 128) == 0 ? launch_gemm_tiles_t<false, 2, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 2, 2, 64>(a, st, who);
+}
+
+// 17..127 rows (batched decoding): 32-row tiles, 64 columns wide, K split over workgroups.  Needs the registered
+// workspace (without the split a narrow projection would occupy a fraction of the compute units).  Up to 16 rows the
+// wave-per-16-weight-rows kernel is as fast or faster (MLP of the 7B shape, 8 rows: 73 vs 79 us; 32 rows: 117 vs 81 us).
+bool gemm_rows_apply(const MfmaArgs& a) {
+  return a.B >= 17 && a.B < 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0 &&
+         split_workspace().part != nullptr;
+}
+int launch_gemm_rows(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
+  if (dual) return launch_gemm_tiles_t<true, 1, 2, 64>(a, st, who);
+  return (a.K % 128) == 0 ? launch_gemm_tiles_t<false, 1, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 1, 2, 64>(a, st, who);
 }
 
 // head expansion of the prefill on the tiled kernel: 128 token rows and more, head_dim 128, rank a multiple of 64,

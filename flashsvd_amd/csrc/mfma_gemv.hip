@@ -137,6 +137,8 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
     if ((tiles * c + 7) / 8 >= 256 && ksteps / c >= 4) { ks = c; break; }
   // many rows (prefill): the tiled kernel reads every weight once per 128 rows instead of once per 64
   if (gemm_tiles_apply(a0)) return launch_gemm_tiles(a0, DUAL, st, who);
+  // a batch of rows: 32-row tiles with K split over workgroups, when the caller has registered a workspace
+  if (gemm_rows_apply(a0)) return launch_gemm_rows(a0, DUAL, st, who);
   // batches above 64 rows go in slices of 64
   for (int b0 = 0; b0 < a0.B; b0 += 64) {
     MfmaArgs a = a0;

@@ -4,6 +4,7 @@ streams here; every arithmetic step runs in the HIP library."""
 from __future__ import annotations
 
 import math
+import os
 from typing import Optional
 
 import torch
@@ -42,6 +43,38 @@ def _rows(t: torch.Tensor, name: str) -> torch.Tensor:
         return t.reshape(-1, t.shape[-1])
 
 
+_SPLIT_WS: dict = {}                      # device index -> scratch tensor registered with the library (kept alive here)
+_SPLIT_WS_BYTES = (64 << 20) + (64 << 10)
+
+
+def ensure_split_workspace(device: torch.device) -> bool:
+    """Register, once per device, the scratch the library's K-split projections (17..127 rows) work in.  The library
+    allocates nothing itself; this hands it 64 MiB of torch memory.  ``FLASHSVD_AMD_SPLITK=0`` keeps the projections
+    unsplit; so does a first call made under stream capture (an allocation there would belong to the graph's pool).
+    Launches that use the scratch must be ordered on one stream per device."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx in _SPLIT_WS:
+        return _SPLIT_WS[idx] is not None
+    if os.environ.get("FLASHSVD_AMD_SPLITK", "1") == "0" or torch.cuda.is_current_stream_capturing():
+        return False
+    with torch.cuda.device(idx):
+        ws = torch.empty(_SPLIT_WS_BYTES, dtype=torch.uint8, device=f"cuda:{idx}")
+        rc = _lib.load().fsvd_set_workspace(ws.data_ptr(), ws.numel(), _stream())
+        _lib.check("fsvd_set_workspace", rc)
+        torch.cuda.current_stream().synchronize()      # cleared before any other stream can use it
+    _SPLIT_WS[idx] = ws
+    return True
+
+
+def release_split_workspace(device: Optional[torch.device] = None) -> None:
+    """Unregister (and free) the scratch of ``device``; projections run unsplit until it is registered again."""
+    idx = torch.cuda.current_device() if device is None or device.index is None else device.index
+    if _SPLIT_WS.pop(idx, None) is not None:
+        with torch.cuda.device(idx):
+            torch.cuda.synchronize()
+            _lib.check("fsvd_set_workspace", _lib.load().fsvd_set_workspace(None, 0, None))
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
            norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
            residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:
@@ -71,6 +104,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             if t.shape != (n,) or not t.is_contiguous():
                 raise ValueError(f"{nm} must be a contiguous [{n}] tensor")
     lib = _lib.load()
+    if 17 <= B < 128:
+        ensure_split_workspace(x.device)
     if norm_weight is not None and B >= 5 and cfg == 0 and K % 32 == 0:
         # five rows and more run on the matrix cores, which take the activations as they are: normalise once
         # up front (same rounding points as the fused prologue)
@@ -98,6 +133,8 @@ def swiglu_linear(p: torch.Tensor, gate_u: torch.Tensor, up_u: torch.Tensor, *, 
         out = torch.empty(*p.shape[:-1], D, device=p.device, dtype=_BF16)
     o2 = _rows(out, "out")
     lib = _lib.load()
+    if 17 <= B < 128:
+        ensure_split_workspace(p.device)
     rc = lib.fsvd_swiglu_linear(p2.data_ptr(), p2.stride(0), int(up_off), gate_u.data_ptr(), up_u.data_ptr(),
                                 gate_u.stride(0), o2.data_ptr(), o2.stride(0), B, D, R, int(mode), int(cfg), _stream())
     _lib.check("fsvd_swiglu_linear", rc)

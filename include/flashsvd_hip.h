@@ -39,6 +39,17 @@ extern "C" {
 int fsvd_version(void);
 const char* fsvd_last_error(void);
 
+/* Optional scratch for the projections of 17..127 rows (fsvd_linear, fsvd_swiglu_linear): with it they run on 32-row
+ * tiles and split K over several workgroups per tile (fp32 partial tiles and arrival counters live in this buffer; the
+ * sum is taken in a fixed order, so results do not depend on timing).
+ * The library never allocates device memory: the caller owns `ws` (device memory of the current device, 256-byte
+ * aligned, `bytes` >= 1 MiB to be of use, 64 MiB covers every shape of a 7B model) and keeps it alive until it
+ * registers another buffer or NULL.  The first 64 KiB are cleared here, on `stream`.  One buffer per device; launches
+ * that use it must be ordered on one stream (two concurrent projections would share the counters).  Without a
+ * registered buffer the same entry points run unsplit.  No counterpart in the reference (torch.matmul picks its own
+ * split-K workspace inside hipBLASLt). */
+int fsvd_set_workspace(void* ws, size_t bytes, void* stream);
+
 /* y[b,n] = (res[b,n] +) bf16( W[n,:] . norm(x[b,:]) (+ bias[n]) ),  W is an nn.Linear weight [N,K].
  * norm_w != NULL fuses the RMSNorm of x (w * bf16(x * rsqrt(mean(x^2)+eps))) in front.
  * Replaces the factor GEMVs the reference issues through torch: rank projection

@@ -120,7 +120,9 @@ def test_7b_width_two_layers_greedy_32_tie_aware():
             continue
         for lg, nm in ((ref_logits[0, s], "oracle"), (logits[0, s], "gpu")):
             gap = abs(float(lg[o] - lg[g])) / max(abs(float(lg[o])), 1e-6)
-            assert gap <= 1e-2, f"step {s}: gpu token {g} vs oracle {o} with a {nm} logit gap of {gap:.3%} (not a near-tie)"
+            # hidden states may differ by 1e-2 relative (the stated tolerance), so two logits closer than twice that can
+            # legitimately change places between two correct fp32 summation orders
+            assert gap <= 2e-2, f"step {s}: gpu token {g} vs oracle {o} with a {nm} logit gap of {gap:.3%} (not a near-tie)"
     assert n_equal >= 24, f"only {n_equal}/32 teacher-forced greedy tokens identical"
 
 

@@ -2,6 +2,7 @@
 the C ABI (flashsvd_amd.hip_ops -> libflashsvd_hip.so).  Tolerance: bf16 outputs within
 max-abs 2e-2 and max-rel 1e-2 of the oracle on the same seeded inputs."""
 import math
+import os
 
 import pytest
 import torch
@@ -175,7 +176,8 @@ def test_linear_batched_with_norm(ops):
     assert_close_bf16(y, O.lin(O.rms_norm(x, nw, 1e-6), w), "batched norm + linear")
 
 
-@pytest.mark.parametrize("B,D,R,mode", [(8, 11008, 1536, 0), (32, 1376, 256, 1), (5, 100, 64, 0), (33, 64, 96, 1)])
+@pytest.mark.parametrize("B,D,R,mode", [(8, 11008, 1536, 0), (32, 1376, 256, 1), (5, 100, 64, 0), (33, 64, 96, 1), (32, 11008, 1536, 0),
+                                        (100, 1376, 256, 1), (20, 200, 192, 0)])
 def test_swiglu_batched_matrix_cores(ops, B, D, R, mode):
     p = rand_bf16(B, 2 * R, seed=1)
     gu, uu = rand_bf16(D, R, std=0.05, seed=2), rand_bf16(D, R, std=0.05, seed=3)
@@ -185,7 +187,7 @@ def test_swiglu_batched_matrix_cores(ops, B, D, R, mode):
         ref = torch.nn.functional.silu(g.to(torch.bfloat16)) * u.to(torch.bfloat16)
     else:
         ref = ((g * torch.sigmoid(g)) * u).to(torch.bfloat16)
-    assert_close_bf16(h, ref, f"batched swiglu mode {mode}")
+    assert_close_bf16(h, ref, f"batched swiglu mode {mode}", **bounds(ref))
 
 
 # ---- 128 rows and more (prefill): the tiled matrix-core kernel (csrc/mfma_gemm.hip) behind the same entry points
@@ -219,3 +221,36 @@ def test_swiglu_prefill_rows_tiled_kernel(ops, B, D, R, mode):
     else:
         ref = ((g * torch.sigmoid(g)) * u).to(torch.bfloat16)
     assert_close_bf16(h, ref, f"tiled swiglu mode {mode}", **bounds(ref))
+
+
+# ---- K split over workgroups (registered scratch): same entry points, 17..127 rows
+@pytest.mark.parametrize("B,N,K", [(17, 1536, 11008), (32, 1024, 4096), (100, 200, 1536), (127, 4096, 1536), (64, 3072, 4096)])
+def test_linear_k_split_matches_unsplit_and_repeats(ops, B, N, K):
+    x, w = rand_bf16(B, K, seed=1).cuda(), rand_bf16(N, K, std=0.02, seed=2).cuda()
+    bias, res = rand_bf16(N, std=0.1, seed=4).cuda(), rand_bf16(B, N, seed=5).cuda()
+    dev = x.device
+    assert ops.ensure_split_workspace(dev)
+    y1 = ops.linear(x, w, bias, residual=res)
+    y2 = ops.linear(x, w, bias, residual=res)           # arrival counters are back at zero; partial sums in a fixed order
+    assert torch.equal(y1, y2)
+    ref = res.cpu() + O.lin(x.cpu(), w.cpu(), bias.cpu())
+    assert_close_bf16(y1, ref, f"k-split linear {B}x{N}x{K}", **bounds(ref))
+    os.environ["FLASHSVD_AMD_SPLITK"] = "0"             # keeps the wrapper from registering again
+    ops.release_split_workspace(dev)
+    try:
+        y0 = ops.linear(x, w, bias, residual=res)
+        assert_close_bf16(y0, ref, f"unsplit linear {B}x{N}x{K}", **bounds(ref))
+    finally:
+        del os.environ["FLASHSVD_AMD_SPLITK"]
+        assert ops.ensure_split_workspace(dev)
+
+
+def test_set_workspace_rejects_bad_buffers(ops, lib):
+    buf = torch.empty(2 << 20, dtype=torch.uint8, device="cuda")
+    assert lib.fsvd_set_workspace(buf.data_ptr() + 16, 1 << 20, None) != 0
+    assert b"aligned" in lib.fsvd_last_error()
+    assert lib.fsvd_set_workspace(buf.data_ptr(), 4096, None) != 0
+    assert b"too small" in lib.fsvd_last_error()
+    # the registered scratch of the wrapper is untouched by the refused calls
+    x, w = rand_bf16(8, 1024, seed=1).cuda(), rand_bf16(64, 1024, std=0.02, seed=2).cuda()
+    assert_close_bf16(ops.linear(x, w), O.lin(x.cpu(), w.cpu()), "after refused registrations")

@@ -38,7 +38,9 @@ def _tie_aware(g, o, ref_logits_row, what):
         return True
     rl = ref_logits_row.float()
     gap = float(rl[o] - rl[g])
-    assert gap <= 1e-2 * float(rl.abs().max()), f"{what}: token {g} vs oracle {o}, oracle logit gap {gap}"
+    # two logits a few bf16 steps apart (hidden states are only held to 1e-2 relative) may change places between two
+    # correct fp32 summation orders
+    assert gap <= 2e-2 * float(rl.abs().max()), f"{what}: token {g} vs oracle {o}, oracle logit gap {gap}"
     return False
 
 
