@@ -18,6 +18,7 @@
 // reciprocals are precomputed on the host, per-piece address arithmetic is incremental, and waves that
 // own no output rows skip the epilogue.
 #include <cstddef>
+#include <type_traits>
 #include <vector>
 
 #include "../../include/flashsvd_hip.h"
@@ -178,7 +179,11 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
   const int dq = (int)__umulhi((uint32_t)kT, m_kp);   // rows a lane advances per step (plus the carry of kofs)
   const int cps = c.pps >> 4;                   // chunks per matrix
   const bool lead = (tid & 15) == 0;
-  for (int s0 = 0; s0 < c.nsteps; s0 += SPB) {
+  // one batch of the window: products, DPP folds and (REFILL) the loads of the next batch.  The last batch is a copy
+  // of the loop body without refills: loads past the slab would sit in the memory pipeline in front of the stores
+  // that publish this phase's outputs
+  auto batch = [&](int s0, auto refill) {
+    constexpr bool REFILL = decltype(refill)::value;
     float d[kU];
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
@@ -188,8 +193,10 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
       if (GROUPED) xo += ((row >= g1 ? 1 : 0) + (row >= g2 ? 1 : 0)) * c.K;
       const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xs + xo);
       d[u] = dot8_bf16(R[u], xv, 0.f);
-      const uint32_t in = min((uint32_t)((s0 + u / NMAT + SPB) * kT) + tid, last);
-      R[u] = ld_stream(mat ? c.base1 : c.base0, in << 4);
+      if (REFILL) {
+        const uint32_t in = min((uint32_t)((s0 + u / NMAT + SPB) * kT) + tid, last);
+        R[u] = ld_stream(mat ? c.base1 : c.base0, in << 4);
+      }
       d[u] = row16_sum(d[u]);
       if (mat == NMAT - 1) {
         kofs += c.dk;
@@ -206,7 +213,10 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
         if (i < c.pps) cp[(u % NMAT) * cps + (i >> 4)] = d[u];
       }
     }
-  }
+  };
+  int s0 = 0;
+  for (; s0 + SPB < c.nsteps; s0 += SPB) batch(s0, std::true_type{});
+  if (s0 < c.nsteps) batch(s0, std::false_type{});
 }
 // sum of the chunk partials of one row, computed by an aligned group of 8 lanes (each lane adds every
 // eighth chunk, then a three-step DPP butterfly); every lane of the group gets the sum
