@@ -28,7 +28,9 @@
 namespace fsvd {
 
 constexpr int kT = 512;                 // threads per workgroup
-constexpr int kU = 10;                  // 16-byte weight pieces in flight per lane (rolling register window)
+constexpr int kU = 4;                   // 16-byte weight pieces in flight per lane (rolling register window).  Measured 2 / 4 / 6 / 8 /
+                                        // 10 / 12: 451 / 489 / 478 / 471 / 469 / 452 tok/s on the 7B shape: the polls for a phase's
+                                        // input queue behind the window requested just before them, so a deep window delays them
 constexpr int kUA = kU / 2;             // attention: keys (and values) in flight per 16-lane slot
 constexpr int kMaxIn = 16384;           // staged input elements (bf16) per phase
 constexpr int kMaxChunks = 8192;        // chunk partials per workgroup per phase
@@ -416,6 +418,10 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     GemvCtx gc;
     AttnWork aw;
     uint32_t resid = 0;
+    // addresses of the next phase's first window, worked out now (behind the wait for this phase's input) so that the
+    // request after publication is nothing but the loads
+    uint64_t nxt[kU];
+    window_addresses(dvB, w, pos, reinterpret_cast<uint64_t>(phases), nxt);
 
     // ------------------------------------------------------------------ stage + stream
     if (type == FSVD_PH_GEMV) {
@@ -602,12 +608,8 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     // ------------------------------------------------------------------ first window of the next phase
     // (the only place window loads are issued outside the streaming loops; phases without weights read a
     // dummy line so that the registers are always written here)
-    {
-      uint64_t addr[kU];
-      window_addresses(dvB, w, pos, reinterpret_cast<uint64_t>(phases), addr);
 #pragma unroll
-      for (int u = 0; u < kU; ++u) R[u] = ld_stream(addr[u], 0);
-    }
+    for (int u = 0; u < kU; ++u) R[u] = ld_stream(nxt[u], 0);
 
     // ------------------------------------------------------------------ phases that poll after the request
     if (type == FSVD_PH_EMBED) {
