@@ -241,21 +241,25 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
 }
 
 // ---------------------------------------------------------------------------------------------
-// 2b. the same attention for long prompts: 128 queries per workgroup (32 per wave), K and V tiles shared
-//     through LDS.  With 64 queries per workgroup and every wave fetching its own K fragments, a 64-key tile
-//     costs 80 KB of L2 traffic per 64 queries and the kernel is bound by L2 requests; here a tile is read ONCE
-//     per workgroup (32 KB per 128 queries), coalesced, one tile ahead into registers, and written to LDS
-//     (K row-major with a padded stride, V transposed: four adjacent keys per 8-byte write, key column XOR-ed
-//     with 8 * (d / 8 % 8) to spread the 16 dimension blocks over the banks).
+// 2b. the same attention for long prompts: 64 or 128 queries per workgroup (16 MI per wave), K and V tiles shared
+//     through LDS.  With every wave fetching its own K fragments a 64-key tile costs 80 KB of L2 traffic per 64
+//     queries and the kernel is bound by L2 requests; here a tile is read ONCE per workgroup, coalesced, one tile
+//     ahead into registers, and written to LDS (K row-major with a padded stride, V transposed: four adjacent keys
+//     per 8-byte write, key column XOR-ed with 8 * (d / 8 % 8) to spread the 16 dimension blocks over the banks).
+//
+//     Scores are computed TRANSPOSED, S^T = K Q^T: an accumulator lane then holds four consecutive keys of ONE query
+//     (column lr), so the softmax statistics are one value per lane and query block, and the eight softmax weights a
+//     lane owns in two 16-key blocks are exactly one B-operand fragment of O^T = V^T P^T — P never goes through LDS.
+//     The price is a key order inside every 32 keys that the V tile has to follow: MFMA k-slot (lg, e) holds key
+//     16 (e / 4) + 4 lg + e % 4, so V^T is stored with key offset ko at column 8 (ko % 16 / 4) + 4 (ko / 16) + ko % 4.
+//     P is a bf16 high part plus a bf16 residual (two products per fragment) so that it carries ~16 mantissa bits.
 // ---------------------------------------------------------------------------------------------
 template <int MI>
 __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(PrefillAttnArgs a) {
-  constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, KSTR = DH + 8, PSTR = BN + 8, VSTR = BN + 8;
+  constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, KSTR = DH + 8, VSTR = BN + 8;
   extern __shared__ __align__(16) unsigned char pw_smem[];
   uint16_t (*Ks)[KSTR] = reinterpret_cast<uint16_t (*)[KSTR]>(pw_smem);                              // [BN][KSTR]
   uint16_t (*Vt)[VSTR] = reinterpret_cast<uint16_t (*)[VSTR]>(pw_smem + (size_t)BN * KSTR * 2);       // [DH][VSTR]
-  uint16_t (*Ps)[QW][PSTR] = reinterpret_cast<uint16_t (*)[QW][PSTR]>(pw_smem + (size_t)BN * KSTR * 2 + (size_t)DH * VSTR * 2);
-  uint16_t (*Pl)[QW][PSTR] = Ps + 4;
 
   const int mt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int hk = h / (a.H / a.Hk);
@@ -273,12 +277,11 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
 #pragma unroll
     for (int st = 0; st < 4; ++st) qf[mi][st] = pf_ld(qp + st * 32);
   }
-  float m_run[MI][4], l_run[MI][4];
-  f32x4_t o[MI][8];
+  float m_run[MI], l_run[MI];          // statistics of query m_base + 16 mi + lr (the same in the four lanes lg of a column)
+  f32x4_t o[MI][8];                    // O^T: tile t, element i = dimension 16 t + 4 lg + i of that query
 #pragma unroll
   for (int mi = 0; mi < MI; ++mi) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { m_run[mi][i] = -INFINITY; l_run[mi][i] = 0.f; }
+    m_run[mi] = -INFINITY; l_run[mi] = 0.f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) o[mi][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
@@ -287,11 +290,15 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
   const int k_end = a.causal ? min(n_keys_all, q0 + last_m + 1) : n_keys_all;
   // last key this wave's rows may see: tiles past it are skipped by the wave (it still takes part in the staging)
   const int wave_end = a.causal ? min(n_keys_all, q0 + min(m_base + QW - 1, a.M - 1) + 1) : n_keys_all;
+  const bool rows_ragged = m_base + QW > a.M;
   const uint16_t* kb = a.k + (int64_t)b * a.sk_b + (int64_t)hk * a.sk_h;
   const uint16_t* vb = a.v + (int64_t)b * a.sk_b + (int64_t)hk * a.sk_h;
 
   // staging roles: 16 lanes cover one 256-byte row; K: rows tid/16 + 16 j; V: the four adjacent keys 4 (tid/16) + j
   const int srow = tid >> 4, d0 = (tid & 15) * 8;
+  // column of this thread's four keys in the permuted order of V^T (see above), before the bank swizzle
+  const int vko = (srow * 4) & 31;
+  const int vcol = ((srow * 4) & 32) + 8 * ((vko & 15) >> 2) + 4 * (vko >> 4);
   u32x4_t kreg[4], vreg[4];
   auto request = [&](int n0) {
 #pragma unroll
@@ -308,7 +315,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(&Ks[srow + 16 * j][d0]) = kreg[j];
     {
-      const int col = (srow * 4) ^ (8 * ((tid & 15) & 7));
+      const int col = vcol ^ (8 * ((tid & 15) & 7));
       const uint32_t w[4][4] = {{vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w}, {vreg[1].x, vreg[1].y, vreg[1].z, vreg[1].w},
                                 {vreg[2].x, vreg[2].y, vreg[2].z, vreg[2].w}, {vreg[3].x, vreg[3].y, vreg[3].z, vreg[3].w}};
 #pragma unroll
@@ -326,7 +333,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
     if (n0 + BN < k_end) request(n0 + BN);
     if (n0 >= wave_end) continue;   // nothing this wave's rows may see (wave-uniform)
 
-    // ---- S = Q K^T for 16 MI rows x 64 keys
+    // ---- S^T = K Q^T for 64 keys x 16 MI queries: block j, element i = key n0 + 16 j + 4 lg + i, query column lr
     f32x4_t sacc[MI][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -337,84 +344,98 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
       for (int mi = 0; mi < MI; ++mi) {
         sacc[mi][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int st = 0; st < 4; ++st) sacc[mi][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[mi][st], kf[st], sacc[mi][j], 0, 0, 0);
+        for (int st = 0; st < 4; ++st) sacc[mi][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[st], qf[mi][st], sacc[mi][j], 0, 0, 0);
       }
     }
-    // ---- masks + online softmax on the accumulator layout (rows lg*4+i, key column j*16+lr), P to LDS
+    // ---- masks + online softmax, one query per lane and block; tiles that need no mask take the short way
+    const bool plain = !a.pad_mask && !a.add_mask && !rows_ragged && n0 + BN <= n_keys_all &&
+                       (!a.causal || n0 + BN - 1 <= q0 + m_base);
+    bf16x8_t ph[MI][2], pl[MI][2];     // P^T fragments (high part, residual) of the two 32-key steps
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi) {
+      const int m = m_base + mi * 16 + lr;
+      const int qpos = q0 + m;
+      float mx = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int m = m_base + mi * 16 + lg * 4 + i;
-        const int qpos = q0 + m;
-        float pv[4];
-        float rmax = -INFINITY;
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int key = n0 + j * 16 + lr;
-          float v = sacc[mi][j][i];
-          bool ok = key < n_keys_all && m < a.M;
-          if (a.causal) ok = ok && key <= qpos;
-          v = ok ? v * a.scale : -INFINITY;            // mask first, then scale, as the reference kernel
-          if (ok && a.pad_mask) ok = a.pad_mask[(int64_t)b * a.spm_b + key] != 0;
-          if (!ok) v = -INFINITY;
-          if (ok && a.add_mask) v += a.add_mask[(int64_t)b * a.sam_b + (int64_t)m * a.sam_q + key];
-          pv[j] = v;
-          rmax = fmaxf(rmax, v);
+        for (int i = 0; i < 4; ++i) {
+          float v = sacc[mi][j][i] * a.scale;
+          if (!plain) {
+            const int key = n0 + j * 16 + lg * 4 + i;
+            bool ok = key < n_keys_all && m < a.M;
+            if (a.causal) ok = ok && key <= qpos;
+            if (ok && a.pad_mask) ok = a.pad_mask[(int64_t)b * a.spm_b + key] != 0;
+            if (!ok) v = -INFINITY;                    // mask first, then the additive term, as the reference kernel
+            else if (a.add_mask) v += a.add_mask[(int64_t)b * a.sam_b + (int64_t)m * a.sam_q + key];
+          }
+          sacc[mi][j][i] = v;
+          mx = fmaxf(mx, v);
         }
-        rmax = row16_max(rmax);
-        const float m_new = fmaxf(m_run[mi][i], rmax);
-        const float alpha = (m_run[mi][i] == -INFINITY) ? 0.f : __expf(m_run[mi][i] - m_new);
-        float rsum = 0.f;
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run[mi], mx);
+      const float alpha = (m_run[mi] == -INFINITY) ? 0.f : __expf(m_run[mi] - m_new);
+      float rsum = 0.f;
+      float e[4][4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float e = (pv[j] == -INFINITY || m_new == -INFINITY) ? 0.f : __expf(pv[j] - m_new);
-          rsum += e;
-          const uint32_t hi = f32_to_bf16_bits(e);
-          Ps[wave][mi * 16 + lg * 4 + i][j * 16 + lr] = (uint16_t)hi;
-          Pl[wave][mi * 16 + lg * 4 + i][j * 16 + lr] = (uint16_t)f32_to_bf16_bits(e - bf16_bits_to_f32(hi));
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = sacc[mi][j][i];
+          e[j][i] = (v == -INFINITY || m_new == -INFINITY) ? 0.f : __expf(v - m_new);
+          rsum += e[j][i];
         }
-        rsum = row16_sum(rsum);
-        l_run[mi][i] = l_run[mi][i] * alpha + rsum;
-        m_run[mi][i] = m_new;
+      rsum += __shfl_xor(rsum, 16);
+      rsum += __shfl_xor(rsum, 32);
+      l_run[mi] = l_run[mi] * alpha + rsum;
+      m_run[mi] = m_new;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) o[mi][t][i] *= alpha;
+      for (int t = 0; t < 8; ++t) o[mi][t] *= alpha;
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        uint32_t hw[4], lw[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {                  // k-slots 2c, 2c + 1: block 2 st + c / 2, elements 2 (c % 2), + 1
+          const float x0 = e[2 * st + (c >> 1)][2 * (c & 1)], x1 = e[2 * st + (c >> 1)][2 * (c & 1) + 1];
+          const uint32_t h0 = f32_to_bf16_bits(x0), h1 = f32_to_bf16_bits(x1);
+          hw[c] = h0 | (h1 << 16);
+          lw[c] = f32_to_bf16_bits(x0 - bf16_bits_to_f32(h0)) | (f32_to_bf16_bits(x1 - bf16_bits_to_f32(h1)) << 16);
+        }
+        ph[mi][st] = __builtin_bit_cast(bf16x8_t, u32x4_t{hw[0], hw[1], hw[2], hw[3]});
+        pl[mi][st] = __builtin_bit_cast(bf16x8_t, u32x4_t{lw[0], lw[1], lw[2], lw[3]});
       }
     }
-    __builtin_amdgcn_wave_barrier();   // P is written and read by this wave only; LDS keeps a wave's accesses in order
-    // ---- O += P V : A = P rows (keys contiguous), B = Vt rows (keys contiguous, swizzled)
+    // ---- O^T += V^T P^T : A = Vt rows (dimension 16 t + lr; keys in the permuted order), B = P^T fragments
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
-      bf16x8_t pa[MI], pb[MI];
-#pragma unroll
-      for (int mi = 0; mi < MI; ++mi) {
-        pa[mi] = pf_ld(&Ps[wave][mi * 16 + lr][st * 32 + lg * 8]);
-        pb[mi] = pf_ld(&Pl[wave][mi * 16 + lr][st * 32 + lg * 8]);
-      }
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const bf16x8_t vf = pf_ld(&Vt[t * 16 + lr][(st * 32 + lg * 8) ^ (8 * ((2 * t + (lr >> 3)) & 7))]);
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
-          o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[mi], vf, o[mi][t], 0, 0, 0);
-          o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pb[mi], vf, o[mi][t], 0, 0, 0);
+          o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph[mi][st], o[mi][t], 0, 0, 0);
+          o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[mi][st], o[mi][t], 0, 0, 0);
         }
       }
     }
   }
 
-  // ---- normalise and store; rows with no visible key give 0
+  // ---- normalise and store (four consecutive dimensions per lane and tile); rows with no visible key give 0
 #pragma unroll
-  for (int mi = 0; mi < MI; ++mi)
+  for (int mi = 0; mi < MI; ++mi) {
+    const int m = m_base + mi * 16 + lr;
+    if (m >= a.M) continue;
+    const float inv = l_run[mi] > 0.f ? 1.0f / l_run[mi] : 0.f;
+    uint16_t* op = a.out + (int64_t)b * a.so_b + (int64_t)m * a.so_m + (int64_t)h * a.so_h + lg * 4;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = m_base + mi * 16 + lg * 4 + i;
-      if (m >= a.M) continue;
-      const float inv = l_run[mi][i] > 0.f ? 1.0f / l_run[mi][i] : 0.f;
-      uint16_t* op = a.out + (int64_t)b * a.so_b + (int64_t)m * a.so_m + (int64_t)h * a.so_h;
-#pragma unroll
-      for (int t = 0; t < 8; ++t) op[t * 16 + lr] = (uint16_t)f32_to_bf16_bits(o[mi][t][i] * inv);
+    for (int t = 0; t < 8; ++t) {
+      u32x2_t w;
+      w.x = f32_to_bf16_bits(o[mi][t][0] * inv) | (f32_to_bf16_bits(o[mi][t][1] * inv) << 16);
+      w.y = f32_to_bf16_bits(o[mi][t][2] * inv) | (f32_to_bf16_bits(o[mi][t][3] * inv) << 16);
+      *reinterpret_cast<u32x2_t*>(op + t * 16) = w;
     }
+  }
 }
 
 int launch_expand(const ExpandArgs& a, hipStream_t st) {
@@ -444,17 +465,12 @@ int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
     set_last_error("%s: q / k / v pointers and strides must be 16-byte aligned", fn);
     return kErrBadAlign;
   }
-  if (a.M >= 128) {   // long prompts: 128 queries per workgroup, K / V tiles shared through LDS
+  // the LDS-shared kernel stores four dimensions of a row with one 8-byte write
+  const bool out8 = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.so_b % 4) == 0 && (a.so_m % 4) == 0 && (a.so_h % 4) == 0;
+  if (a.M >= 128 && out8) {   // long prompts: 64 or 128 queries per workgroup, K / V tiles shared through LDS
     // 128 query rows per workgroup when that gives every compute unit work, else 64 (half the rows per wave)
     const bool wide = (int64_t)((a.M + 127) / 128) * a.H * a.B >= 384;
-    const size_t lds = (size_t)64 * 136 * 2 + (size_t)128 * 72 * 2 + (size_t)2 * 4 * (wide ? 32 : 16) * 72 * 2;
-    static bool granted = false;
-    if (!granted) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<2>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)64 * 136 * 2 + (size_t)128 * 72 * 2 + (size_t)2 * 4 * 32 * 72 * 2));
-      if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", fn, lds, hipGetErrorString(e)); return kErrLaunch; }
-      granted = true;
-    }
+    const size_t lds = (size_t)64 * 136 * 2 + (size_t)128 * 72 * 2;
     if (wide) hipLaunchKernelGGL(attn_prefill_wide_kernel<2>, dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
     else hipLaunchKernelGGL(attn_prefill_wide_kernel<1>, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), lds, st, a);
   } else {
