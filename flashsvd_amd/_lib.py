@@ -31,7 +31,9 @@ class Phase(ctypes.Structure):
                 ("W", c_void_p * 3), ("norm_w", c_void_p), ("cos", c_void_p), ("sin", c_void_p),
                 ("k_cache", c_void_p), ("v_cache", c_void_p), ("sc_s", c_int64), ("sc_h", c_int64),
                 ("plain_out", c_void_p),
-                ("inp", TagBuf), ("aux0", TagBuf), ("aux1", TagBuf), ("out0", TagBuf), ("out1", TagBuf), ("out2", TagBuf),
+                ("inp", TagBuf), ("aux0", TagBuf), ("aux1", TagBuf), ("out0", TagBuf),
+                ("qsz", c_void_p * 2), ("ldg", ctypes.c_int32), ("gshift", ctypes.c_int32), ("wbits", ctypes.c_int32),
+                ("rsv0", ctypes.c_int32),
                 ("share_q", ctypes.c_int32), ("share_r", ctypes.c_int32), ("m_kp", ctypes.c_uint32), ("dk", ctypes.c_int32)]
 
 
@@ -90,7 +92,7 @@ SIGNATURES = {
     "fsvd_decode_step_validate": (c_int, [c_void_p, c_int, c_int]),
     "fsvd_set_workspace": (c_int, [c_void_p, c_size_t, c_void_p]),
     "fsvd_decode_step": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
-    "fsvd_decode_step_trace": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "fsvd_decode_step_trace": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "fsvd_mlp_dual_split": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                     c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -494,11 +494,11 @@ int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host
     const int rc = validate_decode_step(phases_host, nphase, nwg);
     if (rc != kOk) return rc;
   }
-  return launch_decode_step(phases_dev, nphase, state, nullptr, 1, static_cast<hipStream_t>(stream));
+  return launch_decode_step(phases_dev, nphase, state, nullptr, 1, decode_step_has_q4(phases_host, nphase), static_cast<hipStream_t>(stream));
 }
 
-int fsvd_decode_step_trace(const fsvd_phase* phases_dev, int nphase, fsvd_step_state* state, uint64_t* trace,
-                           size_t trace_words, int wg_stride, void* stream) {
+int fsvd_decode_step_trace(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase, fsvd_step_state* state,
+                           uint64_t* trace, size_t trace_words, int wg_stride, void* stream) {
   const char* fn = "fsvd_decode_step_trace";
   FSVD_REQUIRE_PTR(phases_dev, fn); FSVD_REQUIRE_PTR(state, fn); FSVD_REQUIRE_PTR(trace, fn);
   const int nwg = decode_step_workgroups();
@@ -507,7 +507,7 @@ int fsvd_decode_step_trace(const fsvd_phase* phases_dev, int nphase, fsvd_step_s
   const size_t need = (size_t)((nwg + wg_stride - 1) / wg_stride) * nphase * 4;
   if (trace_words < need) { set_last_error("%s: trace buffer holds %zu words, %zu needed", fn, trace_words, need); return kErrWorkspace; }
   return launch_decode_step(phases_dev, nphase, state, reinterpret_cast<unsigned long long*>(trace), wg_stride,
-                            static_cast<hipStream_t>(stream));
+                            decode_step_has_q4(phases_host, nphase), static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -36,7 +36,8 @@ constexpr int kMaxIn = 16384;           // staged input elements (bf16) per phas
 constexpr int kMaxChunks = 8192;        // chunk partials per workgroup per phase
 constexpr int kSpinLimit = 1 << 20;     // polls before a workgroup gives up
 constexpr int kSlots = kT / 16;         // 16-lane groups = keys in flight per load in the attention phase
-constexpr size_t kSmemBytes = (size_t)kMaxIn * 2 + (size_t)kMaxChunks * 4 + 256;
+constexpr int kMaxPieces = kMaxIn / 32;    // 32-column pieces of a staged input (int4 phases keep their sums)
+constexpr size_t kSmemBytes = (size_t)kMaxIn * 2 + (size_t)kMaxChunks * 4 + 256 + (size_t)kMaxPieces * 4;
 
 // ---------------------------------------------------------------------------------------------
 // tagged words
@@ -140,10 +141,14 @@ __device__ __forceinline__ uint64_t desc_u64(uint32_t dv, int word) {
 struct GemvCtx {
   int K, kp, nmat, r0, srows, pps, nsteps, dk;
   uint64_t base0, base1;     // byte addresses of the slab in matrix 0 / 1
+  int q4, ldg, gshift;       // int4 weights: a piece is 32 columns; scale | zero words [N, ldg], group = 32 << gshift columns
+  uint64_t sz0, sz1;         // byte addresses of the slab's scale | zero rows
 };
+template <bool Q4>
 __device__ __forceinline__ void gemv_ctx(uint32_t dv, int w, GemvCtx& c) {
   c.K = DF_I(dv, K);
-  c.kp = c.K >> 3;
+  c.q4 = Q4 && DF_I(dv, wbits) == 4;
+  c.kp = c.q4 ? c.K >> 5 : c.K >> 3;
   c.nmat = DF_I(dv, nmat);
   const int q = DF_I(dv, share_q), r = DF_I(dv, share_r);
   c.r0 = w * q + min(w, r);
@@ -151,10 +156,27 @@ __device__ __forceinline__ void gemv_ctx(uint32_t dv, int w, GemvCtx& c) {
   c.pps = c.srows * c.kp;                       // 16-byte pieces per matrix
   c.nsteps = (c.pps + kT - 1) / kT;             // lane steps per matrix
   c.dk = DF_I(dv, dk);                          // kT % kp
-  const uint64_t off = (uint64_t)(uint32_t)c.r0 * (uint32_t)c.K * 2u;
+  const uint64_t off = c.q4 ? (uint64_t)(uint32_t)c.r0 * (uint32_t)(c.K >> 1) : (uint64_t)(uint32_t)c.r0 * (uint32_t)c.K * 2u;
   c.base0 = desc_u64(dv, FSVD_DW(W)) + off;
   c.base1 = c.nmat > 1 ? desc_u64(dv, FSVD_DW(W) + 2) + off : c.base0;
+  c.ldg = c.gshift = 0;
+  c.sz0 = c.sz1 = 0;
+  if (c.q4) {
+    c.ldg = DF_I(dv, ldg);
+    c.gshift = DF_I(dv, gshift);
+    const uint64_t so = (uint64_t)(uint32_t)c.r0 * (uint32_t)c.ldg * 4u;
+    c.sz0 = desc_u64(dv, FSVD_DW(qsz)) + so;
+    c.sz1 = c.nmat > 1 ? desc_u64(dv, FSVD_DW(qsz) + 2) + so : c.sz0;
+  }
 }
+// byte offset, inside the slab's scale | zero rows, of the word that belongs to piece i (row i / kp, group (i % kp) >> gshift)
+__device__ __forceinline__ uint32_t q4_sz_off(const GemvCtx& c, uint32_t i, uint32_t m_kp) {
+  const uint32_t row = __umulhi(i, m_kp);
+  const uint32_t kofs = i - row * (uint32_t)c.kp;
+  return (row * (uint32_t)c.ldg + (kofs >> c.gshift)) << 2;
+}
+typedef const __attribute__((address_space(1))) uint32_t* gptr32_t;
+__device__ __forceinline__ uint32_t ld_stream32(uint64_t addr) { return __builtin_nontemporal_load((gptr32_t)addr); }
 // first window: slot u holds the piece of step u / NMAT in matrix u % NMAT
 template <int NMAT>
 __device__ __forceinline__ void gemv_window_addr(const GemvCtx& c, uint64_t (&addr)[kU]) {
@@ -163,6 +185,15 @@ __device__ __forceinline__ void gemv_window_addr(const GemvCtx& c, uint64_t (&ad
   for (int u = 0; u < kU; ++u) {
     const uint32_t i = min((uint32_t)((u / NMAT) * kT) + threadIdx.x, last);
     addr[u] = ((u % NMAT) ? c.base1 : c.base0) + (i << 4);
+  }
+}
+template <int NMAT>
+__device__ __forceinline__ void gemv_window_addr_sz(const GemvCtx& c, uint32_t m_kp, uint64_t (&addr)[kU]) {
+  const uint32_t last = (uint32_t)(c.pps - 1);
+#pragma unroll
+  for (int u = 0; u < kU; ++u) {
+    const uint32_t i = min((uint32_t)((u / NMAT) * kT) + threadIdx.x, last);
+    addr[u] = ((u % NMAT) ? c.sz1 : c.sz0) + q4_sz_off(c, i, m_kp);
   }
 }
 // consume the window batch by batch; every consumed slot is refilled at once with the piece kU / NMAT
@@ -213,6 +244,106 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
         if (s0 + u / NMAT >= c.nsteps) break;
         const int i = (s0 + u / NMAT) * kT + (int)tid;
         if (i < c.pps) cp[(u % NMAT) * cps + (i >> 4)] = d[u];
+      }
+    }
+  };
+  int s0 = 0;
+  for (; s0 + SPB < c.nsteps; s0 += SPB) batch(s0, std::true_type{});
+  if (s0 < c.nsteps) batch(s0, std::false_type{});
+}
+// ---------------------------------------------------------------------------------------------
+// the same walk over group-wise int4 weights: a 16-byte piece is 32 columns, 8 consecutive lanes form a chunk of
+// 256 columns of one row (K % 256 == 0).  No weight becomes a float: OR-ing 0x4300 over a nibble n gives the bf16
+// pattern of 128 + n, V_DOT2_F32_BF16 multiplies two of them with two activations, and with X_p = sum of the piece's
+// activations the piece contributes s * (D_p - (z + 128) * X_p).  The activations sit in LDS in the order the masks
+// deliver the nibbles (columns 0,4 | 1,5 | 2,6 | 3,7 of every eight), X_p beside them (q4_prepare_input).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float row8_sum(float v) {
+  v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f32<0x141>(v);  // row_half_mirror
+  return v;
+}
+__device__ __forceinline__ float dot32_q4(const u32x4_t& q, const u32x4_t* xs) {
+  float acc = 0.f;
+  const uint32_t qd[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const u32x4_t xv = xs[j];
+    const uint32_t d = qd[j];
+    acc = dot2_bf16((d & 0x000f000fu) | 0x43004300u, xv.x, acc);
+    acc = dot2_bf16(((d >> 4) & 0x000f000fu) | 0x43004300u, xv.y, acc);
+    acc = dot2_bf16(((d >> 8) & 0x000f000fu) | 0x43004300u, xv.z, acc);
+    acc = dot2_bf16(((d >> 12) & 0x000f000fu) | 0x43004300u, xv.w, acc);
+  }
+  return acc;
+}
+// permute the staged input in place and leave the sum of every 32-column piece in xsum (all threads; barriers by the caller)
+__device__ __forceinline__ void q4_prepare_input(uint16_t* xs, float* xsum, int in_len) {
+  const int n8 = in_len >> 3;
+  for (int e = threadIdx.x; e < n8; e += kT) {
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(xs + e * 8);
+    u32x4_t o;   // columns (0,1)(2,3)(4,5)(6,7) -> (0,4)(1,5)(2,6)(3,7)
+    o.x = (v.x & 0xffffu) | (v.z << 16);
+    o.y = (v.x >> 16) | (v.z & 0xffff0000u);
+    o.z = (v.y & 0xffffu) | (v.w << 16);
+    o.w = (v.y >> 16) | (v.w & 0xffff0000u);
+    *reinterpret_cast<u32x4_t*>(xs + e * 8) = o;
+    float t = 0.f;
+    t = dot2_bf16(0x3f803f80u, o.x, t);
+    t = dot2_bf16(0x3f803f80u, o.y, t);
+    t = dot2_bf16(0x3f803f80u, o.z, t);
+    t = dot2_bf16(0x3f803f80u, o.w, t);
+    t += dpp_f32<0xB1>(t);   // the four lanes of a quad hold the four eights of one piece (in_len % 32 == 0)
+    t += dpp_f32<0x4E>(t);
+    if ((threadIdx.x & 3) == 0) xsum[e >> 2] = t;
+  }
+}
+template <int NMAT, bool GROUPED>
+__device__ __forceinline__ void gemv_stream_q4(const GemvCtx& c, uint32_t m_kp, int g1, int g2, u32x4_t (&R)[kU], uint32_t (&SZ)[kU],
+                                               const uint16_t* xs, const float* xsum, float* cp) {
+  constexpr int SPB = kU / NMAT;                // steps per batch
+  const uint32_t tid = threadIdx.x;
+  const uint32_t last = (uint32_t)(c.pps - 1);
+  int row = (int)__umulhi(tid, m_kp);           // tid / kp
+  int kofs = (int)tid - row * c.kp;             // tid % kp: this lane's piece inside its row
+  row += c.r0;
+  const int dq = (int)__umulhi((uint32_t)kT, m_kp);
+  const int cps = c.pps >> 3;                   // chunks per matrix
+  const bool lead = (tid & 7) == 0;
+  auto batch = [&](int s0, auto refill) {
+    constexpr bool REFILL = decltype(refill)::value;
+    float d[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      if (s0 + u / NMAT >= c.nsteps) break;     // the rest of the window lies past the slab (uniform)
+      const int mat = u % NMAT;
+      int sel = mat;
+      if (GROUPED) sel += (row >= g1 ? 1 : 0) + (row >= g2 ? 1 : 0);
+      const float dp = dot32_q4(R[u], reinterpret_cast<const u32x4_t*>(xs + sel * c.K + kofs * 32));
+      const uint32_t sz = SZ[u];
+      const float sc = (float)__builtin_bit_cast(_Float16, (unsigned short)(sz & 0xffffu));
+      const float zz = (float)(int)(sz >> 16);
+      d[u] = sc * (dp - zz * xsum[sel * c.kp + kofs]);
+      if (REFILL) {
+        const uint32_t in = min((uint32_t)((s0 + u / NMAT + SPB) * kT) + tid, last);
+        R[u] = ld_stream(mat ? c.base1 : c.base0, in << 4);
+        SZ[u] = ld_stream32((mat ? c.sz1 : c.sz0) + q4_sz_off(c, in, m_kp));
+      }
+      d[u] = row8_sum(d[u]);
+      if (mat == NMAT - 1) {
+        kofs += c.dk;
+        const bool carry = kofs >= c.kp;
+        kofs = carry ? kofs - c.kp : kofs;
+        if (GROUPED) row += dq + (carry ? 1 : 0);
+      }
+    }
+    if (lead) {
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        if (s0 + u / NMAT >= c.nsteps) break;
+        const int i = (s0 + u / NMAT) * kT + (int)tid;
+        if (i < c.pps) cp[(u % NMAT) * cps + (i >> 3)] = d[u];
       }
     }
   };
@@ -361,15 +492,21 @@ __device__ __forceinline__ void softmax_step(float sc, const u32x4_t& v, float& 
 // Addresses of the first window of the phase described by dv.  The loads themselves are issued at ONE
 // place in the kernel, straight into the window registers: a second issue site would make the compiler
 // merge two register sets, which it does by waiting for every load and copying.
-__device__ __forceinline__ void window_addresses(uint32_t dv, int w, int pos, uint64_t dummy, uint64_t (&addr)[kU]) {
+template <bool Q4>
+__device__ __forceinline__ void window_addresses(uint32_t dv, int w, int pos, uint64_t dummy, uint64_t (&addr)[kU], uint64_t (&addr_sz)[kU]) {
   const int type = DF_I(dv, type);
 #pragma unroll
-  for (int u = 0; u < kU; ++u) addr[u] = dummy;
+  for (int u = 0; u < kU; ++u) addr[u] = addr_sz[u] = dummy;
   if (type == FSVD_PH_GEMV) {
     GemvCtx c;
-    gemv_ctx(dv, w, c);
+    gemv_ctx<Q4>(dv, w, c);
     if (c.nmat == 1) gemv_window_addr<1>(c, addr);
     else gemv_window_addr<2>(c, addr);
+    if (Q4 && c.q4) {
+      const uint32_t m_kp = desc_u32(dv, FSVD_DW(m_kp));
+      if (c.nmat == 1) gemv_window_addr_sz<1>(c, m_kp, addr_sz);
+      else gemv_window_addr_sz<2>(c, m_kp, addr_sz);
+    }
   } else if (type == FSVD_PH_ATTN) {
     AttnWork aw;
     attn_setup(dv, w, pos, aw);
@@ -386,7 +523,8 @@ __device__ __forceinline__ void raise_error(fsvd_step_state* st, int p, int w) {
 
 // TRACE: workgroups 0, stride, 2*stride, ... record wall-clock ticks (100 MHz) per phase:
 // [0] phase entered, [1] input staged, [2] weights consumed, [3] epilogue done
-template <bool TRACE>
+// Q4: the list may hold int4 GEMV phases (wbits == 4); the build without them keeps the bf16 walk free of their code
+template <bool TRACE, bool Q4>
 __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __restrict__ phases, int nph, fsvd_step_state* st,
                                                          unsigned long long* trace, int trace_stride) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -394,6 +532,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
   float* cp = reinterpret_cast<float*>(smem_raw + (size_t)kMaxIn * 2);
   float* red = cp + kMaxChunks;            // 32 floats
   int* ired = reinterpret_cast<int*>(red + 32);
+  float* xsum = reinterpret_cast<float*>(smem_raw + (size_t)kMaxIn * 2 + (size_t)kMaxChunks * 4 + 256);   // [kMaxPieces]
 
   const int tid = threadIdx.x, w = blockIdx.x, nwg = gridDim.x;
   if (st->err != 0) return;
@@ -402,6 +541,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
   const int limit = st->spin_limit > 0 ? st->spin_limit : kSpinLimit;
 
   u32x4_t R[kU];
+  uint32_t SZ[kU];                         // int4 phases: scale | zero word of the piece in the same slot
   uint32_t dvA = desc_fetch(phases, 0, nph), dvB = dvA;   // descriptors of phase p and p+1
 
   // Iteration p: finish phase p (its first weights were requested one iteration earlier), publish its
@@ -420,12 +560,12 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     uint32_t resid = 0;
     // addresses of the next phase's first window, worked out now (behind the wait for this phase's input) so that the
     // request after publication is nothing but the loads
-    uint64_t nxt[kU];
-    window_addresses(dvB, w, pos, reinterpret_cast<uint64_t>(phases), nxt);
+    uint64_t nxt[kU], nxt_sz[kU];
+    window_addresses<Q4>(dvB, w, pos, reinterpret_cast<uint64_t>(phases), nxt, nxt_sz);
 
     // ------------------------------------------------------------------ stage + stream
     if (type == FSVD_PH_GEMV) {
-      gemv_ctx(dv, w, gc);
+      gemv_ctx<Q4>(dv, w, gc);
       const int epi = DF_I(dv, epilogue);
       if (epi == FSVD_EP_RESID && (tid >> 3) < gc.srows) resid = ld_coh32(DF_P(dv, aux0), gc.r0 + (tid >> 3));
       const int gH = DF_I(dv, H);                 // > 0: rows are q | k | v groups with their own inputs
@@ -435,15 +575,29 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       bool ok;
       if (in_len <= 4 * kT * 2) ok = stage_input<4>(DF_P(dv, in), in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red);
       else ok = stage_input<12>(DF_P(dv, in), in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red);
-      if (__syncthreads_or(ok ? 0 : 1)) { raise_error(st, p, w); return; }
+      if (__syncthreads_or((ok && (Q4 || DF_I(dv, wbits) != 4)) ? 0 : 1)) { raise_error(st, p, w); return; }   // int4 phase in the bf16 build
+      if (Q4 && gc.q4) {
+        q4_prepare_input(xs, xsum, in_len);
+        __syncthreads();
+      }
       if (TRACE && tr) tr[1] = wall_clock64();
-      if (gH > 0) {
+      const uint32_t m_kp = desc_u32(dv, FSVD_DW(m_kp));
+      if (Q4 && gc.q4) {
+        if (gH > 0) {
+          const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
+          gemv_stream_q4<1, true>(gc, m_kp, g1, g2, R, SZ, xs, xsum, cp);
+        } else if (gc.nmat == 1) {
+          gemv_stream_q4<1, false>(gc, m_kp, 0, 0, R, SZ, xs, xsum, cp);
+        } else {
+          gemv_stream_q4<2, false>(gc, m_kp, 0, 0, R, SZ, xs, xsum, cp);
+        }
+      } else if (gH > 0) {
         const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
-        gemv_stream<1, true>(gc, desc_u32(dv, FSVD_DW(m_kp)), g1, g2, R, xs, cp);
+        gemv_stream<1, true>(gc, m_kp, g1, g2, R, xs, cp);
       } else if (gc.nmat == 1) {
-        gemv_stream<1, false>(gc, desc_u32(dv, FSVD_DW(m_kp)), 0, 0, R, xs, cp);
+        gemv_stream<1, false>(gc, m_kp, 0, 0, R, xs, cp);
       } else {
-        gemv_stream<2, false>(gc, desc_u32(dv, FSVD_DW(m_kp)), 0, 0, R, xs, cp);
+        gemv_stream<2, false>(gc, m_kp, 0, 0, R, xs, cp);
       }
       __syncthreads();
     } else if (type == FSVD_PH_ATTN) {
@@ -522,7 +676,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     // ------------------------------------------------------------------ publish (GEMV, attention)
     if (type == FSVD_PH_GEMV) {
       const int epi = DF_I(dv, epilogue);
-      const int cpr = gc.kp >> 4;
+      const int cpr = gc.q4 ? gc.kp >> 3 : gc.kp >> 4;   // chunks per row: 256 columns (int4) or 128
       const uint32_t tout = DF_TAG16(dv, out0, epoch);
       void* out = DF_P(dv, out0);
       const int grp = tid >> 3;
@@ -609,7 +763,10 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     // (the only place window loads are issued outside the streaming loops; phases without weights read a
     // dummy line so that the registers are always written here)
 #pragma unroll
-    for (int u = 0; u < kU; ++u) R[u] = ld_stream(nxt[u], 0);
+    for (int u = 0; u < kU; ++u) {
+      R[u] = ld_stream(nxt[u], 0);
+      if (Q4) SZ[u] = ld_stream32(nxt_sz[u]);
+    }
 
     // ------------------------------------------------------------------ phases that poll after the request
     if (type == FSVD_PH_EMBED) {
@@ -711,9 +868,13 @@ int decode_step_workgroups() {
   if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<false, false>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)kSmemBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<true, false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)kSmemBytes) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<false, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)kSmemBytes) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<true, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)kSmemBytes) != hipSuccess)
       return 0;
     attr_set = true;
@@ -732,9 +893,10 @@ int prepare_decode_step(fsvd_phase* ph, int nph, int nwg) {
     d.share_r = items % nwg;
     d.m_kp = 0;
     d.dk = 0;
-    if (d.type == FSVD_PH_GEMV && d.K >= 8) {
-      d.m_kp = 0xffffffffu / (uint32_t)(d.K / 8) + 1u;
-      d.dk = kT % (d.K / 8);
+    const int pc = d.wbits == 4 ? 32 : 8;       // columns per 16-byte piece
+    if (d.type == FSVD_PH_GEMV && d.K >= pc) {
+      d.m_kp = 0xffffffffu / (uint32_t)(d.K / pc) + 1u;
+      d.dk = kT % (d.K / pc);
     }
   }
   return kOk;
@@ -758,8 +920,9 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
       if (d.type == FSVD_PH_EMBED || d.type == FSVD_PH_GEMV) items = d.N;
       else if (d.type == FSVD_PH_MERGE) items = d.H * d.Dh;
       bool ok = d.share_q == items / nwg && d.share_r == items % nwg;
-      if (d.type == FSVD_PH_GEMV && d.K >= 8)
-        ok = ok && d.m_kp == 0xffffffffu / (uint32_t)(d.K / 8) + 1u && d.dk == kT % (d.K / 8);
+      const int pc = d.wbits == 4 ? 32 : 8;
+      if (d.type == FSVD_PH_GEMV && d.K >= pc)
+        ok = ok && d.m_kp == 0xffffffffu / (uint32_t)(d.K / pc) + 1u && d.dk == kT % (d.K / pc);
       if (!ok) return bad("derived fields missing: call fsvd_decode_step_prepare", p);
     }
     switch (d.type) {
@@ -769,7 +932,16 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         break;
       case FSVD_PH_GEMV: {
         if (d.nmat < 1 || d.nmat > 2 || !d.W[0] || (d.nmat == 2 && !d.W[1])) return bad("GEMV needs 1 or 2 matrices", p);
-        if (d.K <= 0 || d.K % 128 != 0) return bad("K must be a positive multiple of 128", p);
+        if (d.wbits != 0 && d.wbits != 16 && d.wbits != 4) return bad("wbits must be 0 / 16 (bf16) or 4", p);
+        const bool q4 = d.wbits == 4;
+        if (d.K <= 0 || d.K % (q4 ? 256 : 128) != 0) return bad(q4 ? "K must be a positive multiple of 256 for int4 weights" : "K must be a positive multiple of 128", p);
+        if (q4) {
+          if (!d.qsz[0] || (d.nmat == 2 && !d.qsz[1])) return bad("int4 GEMV needs the scale | zero words of every matrix", p);
+          if (d.gshift < 0 || d.gshift > 20) return bad("bad group shift", p);
+          if (d.ldg < (((d.K / 32) - 1) >> d.gshift) + 1) return bad("scale | zero rows shorter than the number of groups", p);
+          for (int m = 0; m < d.nmat; ++m)
+            if (reinterpret_cast<uintptr_t>(d.qsz[m]) & 3) return bad("scale | zero words must be 4-byte aligned", p);
+        }
         if (d.N < nwg) return bad("fewer rows than workgroups", p);
         if (d.H > 0) {   // q | k | v row groups reading [Pq | Pk | Pv]
           if (d.nmat != 1 || d.epilogue != FSVD_EP_STORE || d.norm_w) return bad("grouped GEMV is a plain single-matrix store", p);
@@ -779,11 +951,11 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         if (d.nmat * d.K > kMaxIn) return bad("input vector longer than the staging buffer", p);
         if (d.norm_w && d.nmat * d.K > kT * 12 * 2) return bad("normalised input too long for one staging round", p);
         const int64_t rows = ((int64_t)d.N + nwg - 1) / nwg;
-        if (rows * d.nmat * (d.K / 128) > kMaxChunks) return bad("too many rows per workgroup for the partial buffer", p);
+        if (rows * d.nmat * (d.K / (q4 ? 256 : 128)) > kMaxChunks) return bad("too many rows per workgroup for the partial buffer", p);
         if ((d.epilogue == FSVD_EP_SWIGLU) != (d.nmat == 2)) return bad("SwiGLU epilogue needs exactly two matrices", p);
         if (d.epilogue == FSVD_EP_RESID && !d.aux0.ptr) return bad("residual epilogue needs aux0", p);
         if (d.epilogue == FSVD_EP_RESID && rows > kT / 8) return bad("residual epilogue handles at most kT/8 rows per workgroup", p);
-        if (rows * d.nmat * (d.K / 8) * (int64_t)(d.K / 8) >= (1ll << 32)) return bad("slab too large for the index arithmetic", p);
+        if ((rows + kU) * d.nmat * (d.K / (q4 ? 32 : 8)) * (int64_t)(d.K / (q4 ? 32 : 8)) >= (1ll << 32)) return bad("slab too large for the index arithmetic", p);
         if (d.epilogue == FSVD_EP_LOGITS && !d.plain_out) return bad("logits epilogue needs plain_out", p);
         if (d.epilogue < 0 || d.epilogue > FSVD_EP_LOGITS) return bad("unknown epilogue", p);
         if (!d.in.ptr || !d.out0.ptr) return bad("GEMV needs in and out0", p);
@@ -863,12 +1035,26 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
   return kOk;
 }
 
-int launch_decode_step(const fsvd_phase* dev, int nph, fsvd_step_state* st, unsigned long long* trace, int trace_stride,
+bool decode_step_has_q4(const fsvd_phase* host, int nph) {
+  if (!host) return false;
+  for (int p = 0; p < nph; ++p)
+    if (host[p].type == FSVD_PH_GEMV && host[p].wbits == 4) return true;
+  return false;
+}
+
+// q4: the list holds int4 GEMV phases (the build without their code is ~5 % faster on a bf16 list; it raises the
+// step's error flag if it meets one)
+int launch_decode_step(const fsvd_phase* dev, int nph, fsvd_step_state* st, unsigned long long* trace, int trace_stride, bool q4,
                        hipStream_t stream) {
   const int nwg = decode_step_workgroups();
   if (nwg <= 0) { set_last_error("fsvd_decode_step: cannot query the device"); return kErrLaunch; }
-  if (trace) hipLaunchKernelGGL(decode_step_kernel<true>, dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, trace, trace_stride);
-  else hipLaunchKernelGGL(decode_step_kernel<false>, dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, nullptr, 1);
+  if (trace) {
+    if (q4) hipLaunchKernelGGL((decode_step_kernel<true, true>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, trace, trace_stride);
+    else hipLaunchKernelGGL((decode_step_kernel<true, false>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, trace, trace_stride);
+  } else {
+    if (q4) hipLaunchKernelGGL((decode_step_kernel<false, true>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, nullptr, 1);
+    else hipLaunchKernelGGL((decode_step_kernel<false, false>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, nullptr, 1);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("fsvd_decode_step: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
   return kOk;

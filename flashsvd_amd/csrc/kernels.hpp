@@ -193,7 +193,8 @@ namespace fsvd {
 int decode_step_workgroups();
 int prepare_decode_step(fsvd_phase* host_phases, int nph, int nwg);
 int validate_decode_step(const fsvd_phase* host_phases, int nph, int nwg);
+bool decode_step_has_q4(const fsvd_phase* host_phases, int nph);
 int launch_decode_step(const fsvd_phase* dev_phases, int nph, fsvd_step_state* state, unsigned long long* trace,
-                       int trace_stride, hipStream_t stream);
+                       int trace_stride, bool q4, hipStream_t stream);
 }  // namespace fsvd
 

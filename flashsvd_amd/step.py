@@ -73,10 +73,22 @@ class PersistentDecoder:
         def tagged64(n):
             return torch.zeros(n, dtype=torch.int64, device=dev)
 
-        from .quant import is_quantized
+        from .quant import PackedQuantLinear, is_quantized, pack_quant_rows
+        # a layer is either all bf16 factors or all group-wise int4 factors (PackedQuantLinear, no bias, K % 256 == 0)
+        layer_q4 = []
         for li, layer in enumerate(inner.layers):
-            if is_quantized(*layer.self_attn._factor_modules(), *layer.mlp._factor_modules()):
-                raise ValueError(f"PersistentDecoder streams bf16 factors; layer {li} holds int4 modules")
+            mods = [*layer.self_attn._factor_modules(), *layer.mlp._factor_modules()]
+            if not is_quantized(*mods):
+                layer_q4.append(False)
+                continue
+            for m in mods:
+                if not isinstance(m, PackedQuantLinear) or m.bits != 4 or m.bias is not None or m.in_features % 256 != 0:
+                    raise ValueError(f"PersistentDecoder: layer {li} mixes int4 and other factors, or holds an int4 factor "
+                                     "with a bias or a row length that is not a multiple of 256")
+                gs = int(m.group_size)
+                if gs < m.in_features and (gs < 32 or gs & (gs - 1)):
+                    raise ValueError(f"PersistentDecoder: int4 group size {gs} is not a power of two >= 32")
+            layer_q4.append(True)
         # ranks may differ from layer to layer (buffers take the largest); within a layer q, k and v share
         # one rank because their head expansion is a single grouped product
         ranks = []
@@ -108,11 +120,28 @@ class PersistentDecoder:
 
         ph: list[Phase] = []
 
-        def gemv(W, N, K, inp, out, *, nmat=1, norm=None, eps=0.0, epi=EP_STORE, aux=None, plain=None, groups=None):
+        def sz_words(scales, zeros):
+            """uint32 [N, G]: fp16 scale bits in the low half, zero point + 128 in the high half (what a piece needs in one load)."""
+            lo = scales.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
+            hi = (zeros.to(torch.int32) + 128) << 16
+            return (lo | hi).contiguous()
+
+        def gemv(W, N, K, inp, out, *, nmat=1, norm=None, eps=0.0, epi=EP_STORE, aux=None, plain=None, groups=None, q4=None):
             p = Phase()
             p.type, p.epilogue, p.N, p.K, p.nmat, p.mode = PH_GEMV, epi, N, K, nmat, mode
             if groups is not None:          # rows are q | k | v heads, each group reads its own K-long input
                 p.H, p.Hk, p.Dh = groups
+            if q4 is not None:              # W holds (qweight, scales, zeros) triples; q4 = group size
+                gs = min(int(q4), K)
+                p.wbits, p.gshift = 4, int(math.log2(gs // 32))
+                for i, (qw, sc, zr) in enumerate(W):
+                    G = (K + gs - 1) // gs
+                    if tuple(qw.shape) != (N, K // 2) or not qw.is_contiguous() or tuple(sc.shape) != (N, G) or tuple(zr.shape) != (N, G):
+                        raise ValueError(f"int4 factor {tuple(qw.shape)} / {tuple(sc.shape)} does not match [{N},{K}] in groups of {gs}")
+                    sz = sz_words(sc, zr)
+                    p.W[i], p.qsz[i], p.ldg = qw.data_ptr(), sz.data_ptr(), G
+                    self._keep += [qw, sz]
+                W = ()
             for i, w in enumerate(W):
                 if tuple(w.shape) != (N, K) or not w.is_contiguous():
                     raise ValueError(f"weight {tuple(w.shape)} is not a contiguous [{N},{K}] matrix")
@@ -145,12 +174,30 @@ class PersistentDecoder:
             kc, vc = cache.key_cache[l][0], cache.value_cache[l][0]      # [S, Hk, Dh]
             n1, n2 = layer.input_layernorm, layer.post_attention_layernorm
             xin, xmid, xout = _tb(self.XA, L + 1, l), _tb(self.XB, L, l), _tb(self.XA, L + 1, l + 1)
-            gemv([at._packed_qkv_v], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
-            # q, k, v head expansion as one GEMV over the row-packed [q_u; k_u; v_u] (the three module
-            # weights become views of one buffer); RoPE and the cache append happen in the attention phase
-            qkv_u = _packed_rows([at.q_u_proj, at.k_u_proj, at.v_u_proj])
-            self._keep.append(qkv_u)
-            gemv([qkv_u], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
+            q4 = layer_q4[l]
+
+            def triple(*mods):
+                """(qweight, scales, zeros) of one int4 module, or of several stacked row-wise into one stream."""
+                if len(mods) == 1:
+                    m = mods[0]
+                    return (m.qweight, m.scales, m.zeros), int(m.group_size)
+                pk = pack_quant_rows(mods)
+                if pk is None:
+                    raise ValueError(f"PersistentDecoder: int4 factors of layer {l} cannot share a stream (group sizes differ)")
+                return pk, int(mods[0].group_size)
+
+            if q4:
+                w, gs = triple(at.q_v_proj, at.k_v_proj, at.v_v_proj)
+                gemv([w], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon, q4=gs)
+                w, gs = triple(at.q_u_proj, at.k_u_proj, at.v_u_proj)
+                gemv([w], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh), q4=gs)
+            else:
+                gemv([at._packed_qkv_v], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
+                # q, k, v head expansion as one GEMV over the row-packed [q_u; k_u; v_u] (the three module
+                # weights become views of one buffer); RoPE and the cache append happen in the attention phase
+                qkv_u = _packed_rows([at.q_u_proj, at.k_u_proj, at.v_u_proj])
+                self._keep.append(qkv_u)
+                gemv([qkv_u], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
             a = Phase()
             a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
             a.fparam = 1.0 / math.sqrt(Dh)
@@ -162,13 +209,29 @@ class PersistentDecoder:
             m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
             m.inp, m.out0 = _tb(self.PART, L, l), _tb(self.A, L, l)
             ph.append(m)
-            gemv([at.o_v_proj.weight], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
-            gemv([at.o_u_proj.weight], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
-            gemv([mlp._packed_gu_v], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
-            gemv([mlp.gate_u_proj.weight, mlp.up_u_proj.weight], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2,
-                 epi=EP_SWIGLU)
-            gemv([mlp.down_v_proj.weight], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
-            gemv([mlp.down_u_proj.weight], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
+            if q4:
+                w, gs = triple(at.o_v_proj)
+                gemv([w], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l), q4=gs)
+                w, gs = triple(at.o_u_proj)
+                gemv([w], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin, q4=gs)
+                w, gs = triple(mlp.gate_v_proj, mlp.up_v_proj)
+                gemv([w], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon, q4=gs)
+                (wg, gs), (wu, gs2) = triple(mlp.gate_u_proj), triple(mlp.up_u_proj)
+                if gs != gs2:
+                    raise ValueError(f"PersistentDecoder: gate_u / up_u of layer {l} use different int4 group sizes")
+                gemv([wg, wu], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2, epi=EP_SWIGLU, q4=gs)
+                w, gs = triple(mlp.down_v_proj)
+                gemv([w], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l), q4=gs)
+                w, gs = triple(mlp.down_u_proj)
+                gemv([w], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid, q4=gs)
+            else:
+                gemv([at.o_v_proj.weight], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
+                gemv([at.o_u_proj.weight], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
+                gemv([mlp._packed_gu_v], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
+                gemv([mlp.gate_u_proj.weight, mlp.up_u_proj.weight], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2,
+                     epi=EP_SWIGLU)
+                gemv([mlp.down_v_proj.weight], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
+                gemv([mlp.down_u_proj.weight], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
             cache._layer_initialized[l] = True
         fn = inner.norm
         gemv([model.lm_head.weight], V, d, _tb(self.XA, L + 1, L), _tb(self.CAND, 1, 0), norm=fn.weight,
@@ -232,7 +295,8 @@ class PersistentDecoder:
             raise IndexError("no room for another step")
         nt = (self.nwg + wg_stride - 1) // wg_stride
         buf = torch.zeros(nt * self.nph * 4, dtype=torch.int64, device=self.state.device)
-        rc = self.lib.fsvd_decode_step_trace(self.dev_phases.data_ptr(), self.nph, self.state.data_ptr(), buf.data_ptr(),
+        rc = self.lib.fsvd_decode_step_trace(self.dev_phases.data_ptr(), ctypes.addressof(self.host_phases), self.nph,
+                                             self.state.data_ptr(), buf.data_ptr(),
                                              buf.numel(), int(wg_stride), torch.cuda.current_stream().cuda_stream)
         _lib.check("fsvd_decode_step_trace", rc)
         self._host_pos += 1

@@ -247,7 +247,7 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
  * every workgroup leaves; later launches return immediately until the caller clears err.
  * ------------------------------------------------------------------------------------------- */
 #define FSVD_PH_EMBED 0   /* out0[n] = W[0][token, n]                                   (N = hidden)        */
-#define FSVD_PH_GEMV 1    /* out0 = epilogue(W[m] . norm(in)), m < nmat                                      */
+#define FSVD_PH_GEMV 1    /* out0 = epilogue(W[m] . norm(in)), m < nmat; bf16 weights, or int4 when wbits == 4  */
 #define FSVD_PH_ATTN 3    /* in = un-rotated [q | k | v] of the current token ((H + 2*Hk) * Dh values, the   */
                           /* output of a GEMV over the row-packed [q_u; k_u; v_u]): rotate-half RoPE on q, k */
                           /* at state->pos, append k, v to the cache, split-KV attention; out0 = partials    */
@@ -278,7 +278,13 @@ typedef struct fsvd_phase {
   void* k_cache; void* v_cache; /* batch row of the dense cache, [S, Hk, Dh] with strides sc_s, sc_h          */
   int64_t sc_s, sc_h;
   void* plain_out;              /* EP_LOGITS: bf16 logits [N]; ARGMAX: int64 token log indexed by state->step */
-  fsvd_tagbuf in, aux0, aux1, out0, out1, out2;   /* aux0: residual of EP_RESID; aux1, out1, out2 reserved */
+  fsvd_tagbuf in, aux0, aux1, out0;   /* aux0: residual of EP_RESID; aux1 reserved                            */
+  /* GEMV over group-wise int4 weights (wbits == 4; 0 or 16 = bf16): W[m] is the packed matrix [N, K/2] bytes (two
+   * columns per byte, even column in the low nibble, as PackedQuantLinear.qweight); qsz[m] is uint32 [N, ldg] with
+   * the fp16 scale bits of a group in the low half and (zero point + 128) in the high half; a group is
+   * 32 << gshift columns.  K % 256 == 0.  Arithmetic as fsvd_linear_q4: y = sum_g s_g * sum_k x_k (q_k - z_g), fp32. */
+  const void* qsz[2];
+  int32_t ldg, gshift, wbits, rsv0;
   /* derived by fsvd_decode_step_prepare (do not fill by hand): work items (rows, merge outputs) are
    * dealt as share_q per workgroup plus one more for the first share_r workgroups; m_kp is the 32-bit
    * reciprocal of K/8 and dk = (threads per workgroup) mod (K/8) */
@@ -304,7 +310,9 @@ int fsvd_decode_step_prepare(fsvd_phase* phases_host, int nphase, int workgroups
 /* The host-side check of fsvd_decode_step alone (no launch): 0, or a negative status with fsvd_last_error(). */
 int fsvd_decode_step_validate(const fsvd_phase* phases_host, int nphase, int workgroups);
 /* phases_dev: the list in device memory; phases_host: the same list in host memory (validated on every
- * call unless validate == 0); state: device.  Launch is asynchronous on `stream`. */
+ * call unless validate == 0; it also tells the launcher whether the list holds int4 phases, so it may be NULL
+ * only for lists without them — the kernel build without int4 code raises state->err on such a phase);
+ * state: device.  Launch is asynchronous on `stream`. */
 int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase,
                      fsvd_step_state* state, int validate, void* stream);
 /* The same step with per-phase time stamps (the hipEvent-per-module decode profiler of the reference,
@@ -312,8 +320,8 @@ int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host
  * write trace[(wg / wg_stride) * nphase * 4 + phase * 4 + k], k = 0 phase entered, 1 input staged,
  * 2 weights consumed, 3 epilogue done, in ticks of the 100 MHz device wall clock.  The list must have
  * passed fsvd_decode_step's validation before. */
-int fsvd_decode_step_trace(const fsvd_phase* phases_dev, int nphase, fsvd_step_state* state, uint64_t* trace,
-                           size_t trace_words, int wg_stride, void* stream);
+int fsvd_decode_step_trace(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase, fsvd_step_state* state,
+                           uint64_t* trace, size_t trace_words, int wg_stride, void* stream);
 
 #ifdef __cplusplus
 }

@@ -108,7 +108,7 @@ def test_q4_argument_checks():
 
 def test_quantized_model_decodes_like_the_oracle_on_dequantized_weights(monkeypatch):
     """Every factor linear of a small model quantised to int4: prefill + teacher-forced decode through the per-kernel
-    path against the oracle run on the dequantised (bf16) weights; the persistent step refuses the model."""
+    path and through the persistent step against the oracle run on the dequantised (bf16) weights."""
     from flashsvd_amd import quant as Q
     from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
     from flashsvd_amd.step import PersistentDecoder, make_persistent_decoder
@@ -137,7 +137,35 @@ def test_quantized_model_decodes_like_the_oracle_on_dequantized_weights(monkeypa
         _, h = model.decode_step(ref_tok[:, s - 1:s].cuda(), cache, pos, return_hidden=True)
         r = ref_hid[:, s].float()
         assert_close_bf16(h, r, f"decode hidden state {s}", abs_tol=3 * bounds(r)["abs_tol"], rel_tol=3e-2)
-    with pytest.raises(ValueError, match="int4 modules"):
-        PersistentDecoder(model, cache)
+    # the persistent step streams the same int4 factors (phases with wbits == 4): teacher-forced against the same oracle,
+    # and against the per-kernel path on the hidden state of every step
     monkeypatch.setenv("FLASHSVD_AMD_DECODE_ENGINE", "auto")
-    assert make_persistent_decoder(model, cache, 1) is None
+    cache2 = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=Lp + n_new + 4, device="cuda", dtype=BF16)
+    model(prompt.cuda(), past_key_values=cache2, cache_position=torch.arange(Lp))
+    dec = make_persistent_decoder(model, cache2, 1)
+    assert isinstance(dec, PersistentDecoder)
+    assert any(int(ph.wbits) == 4 for ph in dec.host_phases)
+    for s in range(1, n_new):
+        dec.set_state(ref_tok[:, s - 1], Lp + s - 1)
+        dec.step(1)
+        dec.check()
+        r = ref_hid[:, s].float()
+        assert_close_bf16(dec.hidden()[None].cpu(), r, f"persistent step, hidden state {s}", abs_tol=3 * bounds(r)["abs_tol"], rel_tol=3e-2)
+    assert_close_bf16(cache2.key_cache[1][:, :Lp + n_new - 1], cache.key_cache[1][:, :Lp + n_new - 1].cpu(), "K rows of layer 1 vs the per-kernel path",
+                      abs_tol=3 * bounds(cache.key_cache[1].float().cpu())["abs_tol"], rel_tol=3e-2)
+
+
+def test_persistent_step_rejects_int4_layers_it_cannot_stream():
+    """A layer that mixes int4 and bf16 factors is refused at construction (the driver then takes the per-kernel engine)."""
+    from flashsvd_amd import quant as Q
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    from flashsvd_amd.step import PersistentDecoder
+    from tests.util import model_from_oracle
+    mw = O.make_model(d=1024, n_heads=8, n_kv_heads=4, head_dim=128, ffn=2048, attn_rank=256, mlp_rank=512,
+                      n_layers=1, vocab=2048, dtype=BF16, seed=7)
+    model = model_from_oracle(mw)
+    names = [n for n in Q.factor_linear_names(model) if "down_u_proj" not in n]
+    Q.replace_linears_with_packed_quant_inplace(model, module_names=names, bits=4, group_size=128, sym=False)
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=32, device="cuda", dtype=BF16)
+    with pytest.raises(ValueError, match="mixes int4"):
+        PersistentDecoder(model, cache)
