@@ -176,7 +176,8 @@ __device__ __forceinline__ uint32_t q4_sz_off(const GemvCtx& c, uint32_t i, uint
   return (row * (uint32_t)c.ldg + (kofs >> c.gshift)) << 2;
 }
 typedef const __attribute__((address_space(1))) uint32_t* gptr32_t;
-__device__ __forceinline__ uint32_t ld_stream32(uint64_t addr) { return __builtin_nontemporal_load((gptr32_t)addr); }
+// plain (cacheable) loads: the scale / zero words are a sixteenth of the weight bytes and are read again every token
+__device__ __forceinline__ uint32_t ld_stream32(uint64_t addr) { return *(gptr32_t)addr; }
 // first window: slot u holds the piece of step u / NMAT in matrix u % NMAT
 template <int NMAT>
 __device__ __forceinline__ void gemv_window_addr(const GemvCtx& c, uint64_t (&addr)[kU]) {
@@ -256,7 +257,7 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
 // 256 columns of one row (K % 256 == 0).  No weight becomes a float: OR-ing 0x4300 over a nibble n gives the bf16
 // pattern of 128 + n, V_DOT2_F32_BF16 multiplies two of them with two activations, and with X_p = sum of the piece's
 // activations the piece contributes s * (D_p - (z + 128) * X_p).  The activations sit in LDS in the order the masks
-// deliver the nibbles (columns 0,4 | 1,5 | 2,6 | 3,7 of every eight), X_p beside them (q4_prepare_input).
+// deliver the nibbles (columns 0,4 | 1,5 | 2,6 | 3,7 of every eight), X_p beside them (stage_store).
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ float row8_sum(float v) {
   v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
@@ -277,27 +278,6 @@ __device__ __forceinline__ float dot32_q4(const u32x4_t& q, const u32x4_t* xs) {
     acc = dot2_bf16(((d >> 12) & 0x000f000fu) | 0x43004300u, xv.w, acc);
   }
   return acc;
-}
-// permute the staged input in place and leave the sum of every 32-column piece in xsum (all threads; barriers by the caller)
-__device__ __forceinline__ void q4_prepare_input(uint16_t* xs, float* xsum, int in_len) {
-  const int n8 = in_len >> 3;
-  for (int e = threadIdx.x; e < n8; e += kT) {
-    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(xs + e * 8);
-    u32x4_t o;   // columns (0,1)(2,3)(4,5)(6,7) -> (0,4)(1,5)(2,6)(3,7)
-    o.x = (v.x & 0xffffu) | (v.z << 16);
-    o.y = (v.x >> 16) | (v.z & 0xffff0000u);
-    o.z = (v.y & 0xffffu) | (v.w << 16);
-    o.w = (v.y >> 16) | (v.w & 0xffff0000u);
-    *reinterpret_cast<u32x4_t*>(xs + e * 8) = o;
-    float t = 0.f;
-    t = dot2_bf16(0x3f803f80u, o.x, t);
-    t = dot2_bf16(0x3f803f80u, o.y, t);
-    t = dot2_bf16(0x3f803f80u, o.z, t);
-    t = dot2_bf16(0x3f803f80u, o.w, t);
-    t += dpp_f32<0xB1>(t);   // the four lanes of a quad hold the four eights of one piece (in_len % 32 == 0)
-    t += dpp_f32<0x4E>(t);
-    if ((threadIdx.x & 3) == 0) xsum[e >> 2] = t;
-  }
 }
 template <int NMAT, bool GROUPED>
 __device__ __forceinline__ void gemv_stream_q4(const GemvCtx& c, uint32_t m_kp, int g1, int g2, u32x4_t (&R)[kU], uint32_t (&SZ)[kU],
@@ -365,9 +345,22 @@ __device__ __forceinline__ float row_sum8(const float* cp, int row, int cpr) {
 
 // poll the tagged input of a GEMV phase into LDS as packed bf16, RMS-normalised when asked.
 // NS 64-bit words per lane per round; a normalised input fits one round (checked on the host).
+// one packed pair of staged values (elements 2q, 2q + 1) into LDS.  For an int4 phase the eight values of four
+// neighbouring lanes are stored in the order the nibble masks deliver the weights (columns 0,4 | 1,5 | 2,6 | 3,7) and the
+// sum of every 32-column piece (16 lanes) is left in xsum.
+__device__ __forceinline__ void stage_store(uint16_t* xs, float* xsum, int q, uint32_t word, bool q4) {
+  uint32_t* xs32 = reinterpret_cast<uint32_t*>(xs);
+  if (!q4) { xs32[q] = word; return; }
+  const uint32_t partner = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)word, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+  const int pos = threadIdx.x & 3;
+  const uint32_t out = (pos & 2) ? (partner >> 16) | (word & 0xffff0000u) : (word & 0xffffu) | (partner << 16);
+  xs32[(q & ~3) + ((pos & 1) * 2 + (pos >> 1))] = out;
+  const float s = row16_sum(bf16_lo(word) + bf16_hi(word));
+  if ((threadIdx.x & 15) == 0) xsum[q >> 4] = s;
+}
 template <int NS>
 __device__ __forceinline__ bool stage_input(const void* in, int in_len, uint32_t tin, const uint32_t* norm_w, float eps,
-                                            const fsvd_step_state* st, int limit, uint16_t* xs, float* red) {
+                                            const fsvd_step_state* st, int limit, uint16_t* xs, float* red, bool q4, float* xsum) {
   const int tid = threadIdx.x;
   const int nw64 = in_len >> 1;
   const bool norm = norm_w != nullptr;
@@ -406,7 +399,7 @@ __device__ __forceinline__ bool stage_input(const void* in, int in_len, uint32_t
           ss += a * a + b * b;
           v[j] = ((uint64_t)hi << 32) | lo;   // raw values; scaled once the sum is known
         } else {
-          reinterpret_cast<uint32_t*>(xs)[q] = lo | (hi << 16);
+          stage_store(xs, xsum, q, lo | (hi << 16), q4);
         }
       }
     }
@@ -424,8 +417,7 @@ __device__ __forceinline__ bool stage_input(const void* in, int in_len, uint32_t
         const int q = base + j * kT + tid;
         if (q < nw64) {
           const float a = bf16_bits_to_f32((uint32_t)v[j]), b = bf16_bits_to_f32((uint32_t)(v[j] >> 32));
-          reinterpret_cast<uint32_t*>(xs)[q] =
-              pack_bf16x2(bf16_lo(nwt[j]) * round_bf16(a * rs), bf16_hi(nwt[j]) * round_bf16(b * rs));
+          stage_store(xs, xsum, q, pack_bf16x2(bf16_lo(nwt[j]) * round_bf16(a * rs), bf16_hi(nwt[j]) * round_bf16(b * rs)), q4);
         }
       }
     }
@@ -573,13 +565,9 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       const uint32_t tin = DF_TAG16(dv, in, epoch);
       const uint32_t* nw = static_cast<const uint32_t*>(DF_P(dv, norm_w));
       bool ok;
-      if (in_len <= 4 * kT * 2) ok = stage_input<4>(DF_P(dv, in), in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red);
-      else ok = stage_input<12>(DF_P(dv, in), in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red);
+      if (in_len <= 4 * kT * 2) ok = stage_input<4>(DF_P(dv, in), in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+      else ok = stage_input<12>(DF_P(dv, in), in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
       if (__syncthreads_or((ok && (Q4 || DF_I(dv, wbits) != 4)) ? 0 : 1)) { raise_error(st, p, w); return; }   // int4 phase in the bf16 build
-      if (Q4 && gc.q4) {
-        q4_prepare_input(xs, xsum, in_len);
-        __syncthreads();
-      }
       if (TRACE && tr) tr[1] = wall_clock64();
       const uint32_t m_kp = desc_u32(dv, FSVD_DW(m_kp));
       if (Q4 && gc.q4) {
