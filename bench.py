@@ -51,6 +51,9 @@ def _parse():
     ap.add_argument("--stress", action="store_true",
                     help="time the attention kernels of the stress configuration per layer (attention rank 1664: rank-space decode "
                          "at batch 16 x context 4096, prompt attention path at 8 x 2048) and print their own JSON line")
+    ap.add_argument("--quant", action="store_true",
+                    help="the same model with every factor quantised to group-wise int4 (group 128): decode tok/s of both engines "
+                         "and the bytes that cross HBM per token, as its own JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device copy 10 times (the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counters are scaled against) and exit")
@@ -444,6 +447,40 @@ def run_stress():
     }
 
 
+def run_quant(args):
+    """Config 4 with every factor linear as group-wise int4 (PackedQuantLinear, group 128, asymmetric): the persistent step
+    streams the packed nibbles (phases with wbits == 4), the per-operator graph uses fsvd_linear_q4 / fsvd_swiglu_linear_q4."""
+    import os
+    import torch
+    from flashsvd_amd import api, llama, quant as Q
+    cfg = dict(CFG, num_layers=args.layers)
+    model = llama.materialize(llama.build_model(**cfg), "cuda", torch.bfloat16, seed=0)
+    n = Q.replace_linears_with_packed_quant_inplace(model, module_names=Q.factor_linear_names(model), bits=4, group_size=128, sym=False)
+    torch.cuda.empty_cache()
+    wbytes = 0
+    for m in model.modules():
+        if isinstance(m, Q.PackedQuantLinear):
+            wbytes += m.qweight.numel() + 2 * m.scales.numel() + 2 * m.zeros.numel()
+    head = model.lm_head.weight.numel() * 2
+    mid = PROMPT_LEN + args.warmup + args.steps // 2
+    kv = 2 * args.layers * mid * cfg["num_kv_heads"] * cfg["head_dim"] * 2
+    step_bytes = wbytes + head + kv
+    res = {"modules": n, "resident_GB": torch.cuda.memory_allocated() / 1e9, "bytes_per_token": step_bytes}
+    keep = os.environ.get("FLASHSVD_AMD_DECODE_ENGINE")
+    try:
+        for eng in ("persistent", "graph"):
+            os.environ["FLASHSVD_AMD_DECODE_ENGINE"] = eng
+            r = api.decode_kvcache_eval(model, prompt_len=PROMPT_LEN, new_tokens=args.steps, warmup=args.warmup)
+            res[eng] = {"tok_s": r["decode_tok_s"], "ms_per_step": 1e3 / r["decode_tok_s"],
+                        "GB/s": step_bytes * r["decode_tok_s"] / 1e9, "frac_of_peak": step_bytes * r["decode_tok_s"] / 1e9 / HBM_PEAK_GBS}
+    finally:
+        if keep is None:
+            os.environ.pop("FLASHSVD_AMD_DECODE_ENGINE", None)
+        else:
+            os.environ["FLASHSVD_AMD_DECODE_ENGINE"] = keep
+    return res
+
+
 def run_cpu_baseline():
     """The CPU oracle in fp32 (the precision of the reference's CPU path) on a bounded sample:
     2 of the 32 layers + final norm + lm_head, prompt 16, 6 greedy tokens; per-token decode time is
@@ -501,6 +538,12 @@ def main():
         return
     from flashsvd_amd import _lib
     _lib.load()
+    if args.quant:
+        q = run_quant(args)
+        print(json.dumps({"metric": "decode tok/s, 7B-shape rank-0.5 bs1, int4 factors (group 128)", "value": q["persistent"]["tok_s"], "unit": "tok/s",
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "int4 weights, bf16 activations, fp32 sums",
+                          "data": "synthetic", "quant": q}))
+        return
     if args.stress:
         print(json.dumps({"metric": "stress attention kernels, 7B-shape rank-0.8, per layer", "n_gpus": 1, "dtype": "bf16", "data": "synthetic",
                           "stress": run_stress()}))
