@@ -37,7 +37,9 @@ constexpr int kMaxChunks = 8192;        // chunk partials per workgroup per phas
 constexpr int kSpinLimit = 1 << 20;     // polls before a workgroup gives up
 constexpr int kSlots = kT / 16;         // 16-lane groups = keys in flight per load in the attention phase
 constexpr int kMaxPieces = kMaxIn / 32;    // 32-column pieces of a staged input (int4 phases keep their sums)
-constexpr size_t kSmemBytes = (size_t)kMaxIn * 2 + (size_t)kMaxChunks * 4 + 256 + (size_t)kMaxPieces * 4;
+constexpr int kSzLoads = 3;                // 4-byte loads per lane that bring a slab's scale | zero table (int4 phases)
+constexpr int kMaxSz = kSzLoads * kT;      // words of that table: rows x groups x matrices of a workgroup's slab
+constexpr size_t kSmemBytes = (size_t)kMaxIn * 2 + (size_t)kMaxChunks * 4 + 256 + (size_t)kMaxPieces * 4 + (size_t)kMaxSz * 4;
 
 // ---------------------------------------------------------------------------------------------
 // tagged words
@@ -169,12 +171,6 @@ __device__ __forceinline__ void gemv_ctx(uint32_t dv, int w, GemvCtx& c) {
     c.sz1 = c.nmat > 1 ? desc_u64(dv, FSVD_DW(qsz) + 2) + so : c.sz0;
   }
 }
-// byte offset, inside the slab's scale | zero rows, of the word that belongs to piece i (row i / kp, group (i % kp) >> gshift)
-__device__ __forceinline__ uint32_t q4_sz_off(const GemvCtx& c, uint32_t i, uint32_t m_kp) {
-  const uint32_t row = __umulhi(i, m_kp);
-  const uint32_t kofs = i - row * (uint32_t)c.kp;
-  return (row * (uint32_t)c.ldg + (kofs >> c.gshift)) << 2;
-}
 typedef const __attribute__((address_space(1))) uint32_t* gptr32_t;
 // plain (cacheable) loads: the scale / zero words are a sixteenth of the weight bytes and are read again every token
 __device__ __forceinline__ uint32_t ld_stream32(uint64_t addr) { return *(gptr32_t)addr; }
@@ -188,13 +184,14 @@ __device__ __forceinline__ void gemv_window_addr(const GemvCtx& c, uint64_t (&ad
     addr[u] = ((u % NMAT) ? c.base1 : c.base0) + (i << 4);
   }
 }
-template <int NMAT>
-__device__ __forceinline__ void gemv_window_addr_sz(const GemvCtx& c, uint32_t m_kp, uint64_t (&addr)[kU]) {
-  const uint32_t last = (uint32_t)(c.pps - 1);
+// the scale | zero words of a slab are contiguous in memory (rows of ldg words, ldg = groups per row): word i of the
+// table [matrix][row][group] for lane tid is i = j * kT + tid, j < kSzLoads
+__device__ __forceinline__ void gemv_sz_table_addr(const GemvCtx& c, uint64_t (&addr)[kSzLoads]) {
+  const uint32_t per = (uint32_t)(c.srows * c.ldg), total = per * (uint32_t)c.nmat;
 #pragma unroll
-  for (int u = 0; u < kU; ++u) {
-    const uint32_t i = min((uint32_t)((u / NMAT) * kT) + threadIdx.x, last);
-    addr[u] = ((u % NMAT) ? c.sz1 : c.sz0) + q4_sz_off(c, i, m_kp);
+  for (int j = 0; j < kSzLoads; ++j) {
+    const uint32_t i = min((uint32_t)(j * kT) + threadIdx.x, total - 1);
+    addr[j] = (i >= per ? c.sz1 + ((uint64_t)(i - per) << 2) : c.sz0 + ((uint64_t)i << 2));
   }
 }
 // consume the window batch by batch; every consumed slot is refilled at once with the piece kU / NMAT
@@ -280,16 +277,16 @@ __device__ __forceinline__ float dot32_q4(const u32x4_t& q, const u32x4_t* xs) {
   return acc;
 }
 template <int NMAT, bool GROUPED>
-__device__ __forceinline__ void gemv_stream_q4(const GemvCtx& c, uint32_t m_kp, int g1, int g2, u32x4_t (&R)[kU], uint32_t (&SZ)[kU],
+__device__ __forceinline__ void gemv_stream_q4(const GemvCtx& c, uint32_t m_kp, int g1, int g2, u32x4_t (&R)[kU], const uint32_t* sztab,
                                                const uint16_t* xs, const float* xsum, float* cp) {
   constexpr int SPB = kU / NMAT;                // steps per batch
   const uint32_t tid = threadIdx.x;
   const uint32_t last = (uint32_t)(c.pps - 1);
-  int row = (int)__umulhi(tid, m_kp);           // tid / kp
-  int kofs = (int)tid - row * c.kp;             // tid % kp: this lane's piece inside its row
-  row += c.r0;
+  int lrow = (int)__umulhi(tid, m_kp);          // tid / kp: row inside the slab
+  int kofs = (int)tid - lrow * c.kp;            // tid % kp: this lane's piece inside its row
   const int dq = (int)__umulhi((uint32_t)kT, m_kp);
   const int cps = c.pps >> 3;                   // chunks per matrix
+  const int szper = c.srows * c.ldg;            // table words per matrix
   const bool lead = (tid & 7) == 0;
   auto batch = [&](int s0, auto refill) {
     constexpr bool REFILL = decltype(refill)::value;
@@ -299,23 +296,22 @@ __device__ __forceinline__ void gemv_stream_q4(const GemvCtx& c, uint32_t m_kp, 
       if (s0 + u / NMAT >= c.nsteps) break;     // the rest of the window lies past the slab (uniform)
       const int mat = u % NMAT;
       int sel = mat;
-      if (GROUPED) sel += (row >= g1 ? 1 : 0) + (row >= g2 ? 1 : 0);
+      if (GROUPED) sel += (c.r0 + lrow >= g1 ? 1 : 0) + (c.r0 + lrow >= g2 ? 1 : 0);
       const float dp = dot32_q4(R[u], reinterpret_cast<const u32x4_t*>(xs + sel * c.K + kofs * 32));
-      const uint32_t sz = SZ[u];
+      const uint32_t sz = sztab[mat * szper + min(lrow, c.srows - 1) * c.ldg + (kofs >> c.gshift)];
       const float sc = (float)__builtin_bit_cast(_Float16, (unsigned short)(sz & 0xffffu));
       const float zz = (float)(int)(sz >> 16);
       d[u] = sc * (dp - zz * xsum[sel * c.kp + kofs]);
       if (REFILL) {
         const uint32_t in = min((uint32_t)((s0 + u / NMAT + SPB) * kT) + tid, last);
         R[u] = ld_stream(mat ? c.base1 : c.base0, in << 4);
-        SZ[u] = ld_stream32((mat ? c.sz1 : c.sz0) + q4_sz_off(c, in, m_kp));
       }
       d[u] = row8_sum(d[u]);
       if (mat == NMAT - 1) {
         kofs += c.dk;
         const bool carry = kofs >= c.kp;
         kofs = carry ? kofs - c.kp : kofs;
-        if (GROUPED) row += dq + (carry ? 1 : 0);
+        lrow += dq + (carry ? 1 : 0);
       }
     }
     if (lead) {
@@ -485,20 +481,18 @@ __device__ __forceinline__ void softmax_step(float sc, const u32x4_t& v, float& 
 // place in the kernel, straight into the window registers: a second issue site would make the compiler
 // merge two register sets, which it does by waiting for every load and copying.
 template <bool Q4>
-__device__ __forceinline__ void window_addresses(uint32_t dv, int w, int pos, uint64_t dummy, uint64_t (&addr)[kU], uint64_t (&addr_sz)[kU]) {
+__device__ __forceinline__ void window_addresses(uint32_t dv, int w, int pos, uint64_t dummy, uint64_t (&addr)[kU], uint64_t (&addr_sz)[kSzLoads]) {
   const int type = DF_I(dv, type);
 #pragma unroll
-  for (int u = 0; u < kU; ++u) addr[u] = addr_sz[u] = dummy;
+  for (int u = 0; u < kU; ++u) addr[u] = dummy;
+#pragma unroll
+  for (int j = 0; j < kSzLoads; ++j) addr_sz[j] = dummy;
   if (type == FSVD_PH_GEMV) {
     GemvCtx c;
     gemv_ctx<Q4>(dv, w, c);
     if (c.nmat == 1) gemv_window_addr<1>(c, addr);
     else gemv_window_addr<2>(c, addr);
-    if (Q4 && c.q4) {
-      const uint32_t m_kp = desc_u32(dv, FSVD_DW(m_kp));
-      if (c.nmat == 1) gemv_window_addr_sz<1>(c, m_kp, addr_sz);
-      else gemv_window_addr_sz<2>(c, m_kp, addr_sz);
-    }
+    if (Q4 && c.q4) gemv_sz_table_addr(c, addr_sz);
   } else if (type == FSVD_PH_ATTN) {
     AttnWork aw;
     attn_setup(dv, w, pos, aw);
@@ -525,6 +519,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
   float* red = cp + kMaxChunks;            // 32 floats
   int* ired = reinterpret_cast<int*>(red + 32);
   float* xsum = reinterpret_cast<float*>(smem_raw + (size_t)kMaxIn * 2 + (size_t)kMaxChunks * 4 + 256);   // [kMaxPieces]
+  uint32_t* sztab = reinterpret_cast<uint32_t*>(xsum + kMaxPieces);                                        // [kMaxSz]
 
   const int tid = threadIdx.x, w = blockIdx.x, nwg = gridDim.x;
   if (st->err != 0) return;
@@ -533,7 +528,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
   const int limit = st->spin_limit > 0 ? st->spin_limit : kSpinLimit;
 
   u32x4_t R[kU];
-  uint32_t SZ[kU];                         // int4 phases: scale | zero word of the piece in the same slot
+  uint32_t SZ[kSzLoads];                   // int4 phases: this lane's words of the slab's scale | zero table, on their way to LDS
   uint32_t dvA = desc_fetch(phases, 0, nph), dvB = dvA;   // descriptors of phase p and p+1
 
   // Iteration p: finish phase p (its first weights were requested one iteration earlier), publish its
@@ -552,7 +547,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     uint32_t resid = 0;
     // addresses of the next phase's first window, worked out now (behind the wait for this phase's input) so that the
     // request after publication is nothing but the loads
-    uint64_t nxt[kU], nxt_sz[kU];
+    uint64_t nxt[kU], nxt_sz[kSzLoads];
     window_addresses<Q4>(dvB, w, pos, reinterpret_cast<uint64_t>(phases), nxt, nxt_sz);
 
     // ------------------------------------------------------------------ stage + stream
@@ -567,17 +562,21 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       bool ok;
       if (in_len <= 4 * kT * 2) ok = stage_input<4>(DF_P(dv, in), in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
       else ok = stage_input<12>(DF_P(dv, in), in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+      if (Q4 && gc.q4) {   // the slab's scale | zero table came with the window, ahead of the polls; the barrier publishes it
+#pragma unroll
+        for (int j = 0; j < kSzLoads; ++j) sztab[j * kT + tid] = SZ[j];
+      }
       if (__syncthreads_or((ok && (Q4 || DF_I(dv, wbits) != 4)) ? 0 : 1)) { raise_error(st, p, w); return; }   // int4 phase in the bf16 build
       if (TRACE && tr) tr[1] = wall_clock64();
       const uint32_t m_kp = desc_u32(dv, FSVD_DW(m_kp));
       if (Q4 && gc.q4) {
         if (gH > 0) {
           const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
-          gemv_stream_q4<1, true>(gc, m_kp, g1, g2, R, SZ, xs, xsum, cp);
+          gemv_stream_q4<1, true>(gc, m_kp, g1, g2, R, sztab, xs, xsum, cp);
         } else if (gc.nmat == 1) {
-          gemv_stream_q4<1, false>(gc, m_kp, 0, 0, R, SZ, xs, xsum, cp);
+          gemv_stream_q4<1, false>(gc, m_kp, 0, 0, R, sztab, xs, xsum, cp);
         } else {
-          gemv_stream_q4<2, false>(gc, m_kp, 0, 0, R, SZ, xs, xsum, cp);
+          gemv_stream_q4<2, false>(gc, m_kp, 0, 0, R, sztab, xs, xsum, cp);
         }
       } else if (gH > 0) {
         const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
@@ -751,9 +750,10 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     // (the only place window loads are issued outside the streaming loops; phases without weights read a
     // dummy line so that the registers are always written here)
 #pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      R[u] = ld_stream(nxt[u], 0);
-      if (Q4) SZ[u] = ld_stream32(nxt_sz[u]);
+    for (int u = 0; u < kU; ++u) R[u] = ld_stream(nxt[u], 0);
+    if (Q4) {
+#pragma unroll
+      for (int j = 0; j < kSzLoads; ++j) SZ[j] = ld_stream32(nxt_sz[j]);
     }
 
     // ------------------------------------------------------------------ phases that poll after the request
@@ -897,6 +897,7 @@ static int bad(const char* what, int p) {
 
 int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
   if (nph < 2) return bad("a step needs at least two phases", 0);
+
   // last phase index that wrote each buffer and whether a "closing" GEMV consumed a fully-shared vector since
   struct Seen { const void* ptr; int last_write; fsvd_tagbuf tb; };
   std::vector<Seen> seen;
@@ -927,6 +928,7 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
           if (!d.qsz[0] || (d.nmat == 2 && !d.qsz[1])) return bad("int4 GEMV needs the scale | zero words of every matrix", p);
           if (d.gshift < 0 || d.gshift > 20) return bad("bad group shift", p);
           if (d.ldg < (((d.K / 32) - 1) >> d.gshift) + 1) return bad("scale | zero rows shorter than the number of groups", p);
+          if ((((int64_t)d.N + nwg - 1) / nwg) * d.ldg * d.nmat > kMaxSz) return bad("scale | zero table of a workgroup's rows does not fit its LDS buffer", p);
           for (int m = 0; m < d.nmat; ++m)
             if (reinterpret_cast<uintptr_t>(d.qsz[m]) & 3) return bad("scale | zero words must be 4-byte aligned", p);
         }
