@@ -1,4 +1,4 @@
-// Decode projections for 5..64 rows at once (batched decoding, token-tiled MLP) on the matrix cores.
+// Decode projections for 3..64 rows at once (batched decoding, token-tiled MLP) on the matrix cores.
 //
 // At batch 1 a projection is a row-dot GEMV on the vector ALU; from a handful of rows on, the vector
 // path has to re-read the activations from LDS once per weight row and row of the batch and runs out of
@@ -161,14 +161,14 @@ static inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) 
 
 // true when the matrix-core path applies (the caller then skips the vector kernel)
 bool mfma_linear_applies(const LinearArgs& a) {
-  return a.B >= 5 && a.norm_w == nullptr && (a.K % 32) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && al16(a.W) && al16(a.x);
+  return a.B >= 3 && a.norm_w == nullptr && (a.K % 32) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && al16(a.W) && al16(a.x);
 }
 int launch_linear_mfma(const LinearArgs& a, hipStream_t st) {
   MfmaArgs m{a.x, a.ldx, 0, a.W, nullptr, a.ldw, a.bias, a.res, a.ldres, a.y, a.ldy, a.B, a.N, a.K, 0};
   return launch_mfma<false>(m, st, "fsvd_linear");
 }
 bool mfma_swiglu_applies(const SwigluArgs& a) {
-  return a.B >= 5 && (a.R % 32) == 0 && (a.ldw % 8) == 0 && (a.ldp % 8) == 0 && (a.up_off % 8) == 0 && al16(a.gate_u) &&
+  return a.B >= 3 && (a.R % 32) == 0 && (a.ldw % 8) == 0 && (a.ldp % 8) == 0 && (a.up_off % 8) == 0 && al16(a.gate_u) &&
          al16(a.up_u) && al16(a.p);
 }
 int launch_swiglu_mfma(const SwigluArgs& a, hipStream_t st) {

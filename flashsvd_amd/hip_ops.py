@@ -106,8 +106,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     lib = _lib.load()
     if 17 <= B < 128:
         ensure_split_workspace(x.device)
-    if norm_weight is not None and B >= 5 and cfg == 0 and K % 32 == 0:
-        # five rows and more run on the matrix cores, which take the activations as they are: normalise once
+    if norm_weight is not None and B >= 3 and cfg == 0 and K % 32 == 0:
+        # three rows and more run on the matrix cores, which take the activations as they are: normalise once
         # up front (same rounding points as the fused prologue)
         x2 = rmsnorm(x2, norm_weight, eps)
         norm_weight = None

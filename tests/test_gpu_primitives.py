@@ -155,8 +155,8 @@ def test_errors_are_python_exceptions(ops):
         ops.attn_decode_densekv(q, kc, kc.clone(), torch.tensor([4], dtype=torch.int32).cuda(), nsplit=1)
 
 
-# ---- five rows and more: the matrix-core path (csrc/mfma_gemv.hip) behind the same entry points
-@pytest.mark.parametrize("B,N,K", [(5, 48, 1024), (8, 3072, 4096), (16, 1536, 11008), (17, 100, 2048), (32, 4096, 1536),
+# ---- three rows and more: the matrix-core path (csrc/mfma_gemv.hip) behind the same entry points
+@pytest.mark.parametrize("B,N,K", [(3, 512, 4096), (4, 1536, 11008), (5, 48, 1024), (8, 3072, 4096), (16, 1536, 11008), (17, 100, 2048), (32, 4096, 1536),
                                    (64, 256, 512), (70, 33, 256), (8, 40, 96)])
 def test_linear_batched_matrix_cores(ops, B, N, K):
     x, w = rand_bf16(B, K, seed=1), rand_bf16(N, K, std=0.02, seed=2)
@@ -176,7 +176,7 @@ def test_linear_batched_with_norm(ops):
     assert_close_bf16(y, O.lin(O.rms_norm(x, nw, 1e-6), w), "batched norm + linear")
 
 
-@pytest.mark.parametrize("B,D,R,mode", [(8, 11008, 1536, 0), (32, 1376, 256, 1), (5, 100, 64, 0), (33, 64, 96, 1), (32, 11008, 1536, 0),
+@pytest.mark.parametrize("B,D,R,mode", [(3, 11008, 1536, 0), (4, 1376, 256, 1), (8, 11008, 1536, 0), (32, 1376, 256, 1), (5, 100, 64, 0), (33, 64, 96, 1), (32, 11008, 1536, 0),
                                         (100, 1376, 256, 1), (20, 200, 192, 0)])
 def test_swiglu_batched_matrix_cores(ops, B, D, R, mode):
     p = rand_bf16(B, 2 * R, seed=1)
