@@ -39,8 +39,9 @@ __global__ __launch_bounds__(kMfThreads) void mfma_linear_kernel(MfmaArgs a) {
   const int rt = wave / KS, ks = wave % KS;
   const int n0 = (blockIdx.x * RT + rt) * 16;
   const int ksteps = a.K >> 5;
-  const int per = (ksteps + KS - 1) / KS;
-  const int s0 = ks * per, s1 = min(ksteps, s0 + per);
+  // the KS waves of a weight tile take the k-steps in turn (wave ks: steps ks, ks + KS, ...), so that together they read
+  // KS * 64 contiguous bytes of every row at a time; s counts this wave's own steps
+  const int s0 = 0, s1 = (ksteps - ks + KS - 1) / KS;
   const int64_t wo = (int64_t)min(n0 + lr, a.N - 1) * a.ldw + lg * 8;
   const uint16_t* w0 = a.W + wo;
   const uint16_t* w1 = DUAL ? a.W2 + wo : nullptr;
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(kMfThreads) void mfma_linear_kernel(MfmaArgs a) {
     bf16x8_t fa0[UN], fa1[UN], fb0[UN][NB], fb1[UN][NB];
 #pragma unroll
     for (int j = 0; j < UN; ++j) {
-      const int k = min(s + j, s1 - 1) << 5;
+      const int k = (min(s + j, s1 - 1) * KS + ks) << 5;
       fa0[j] = ldw_frag(w0 + k);
       if (DUAL) fa1[j] = ldw_frag(w1 + k);
 #pragma unroll
