@@ -154,34 +154,58 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
       const int ks = ks0 + u;
       if (ks >= ksteps) break;
       const uint16_t* base = lds + (ks & 1) * kStage;
+      // The step as Q blocks of WTM x WT products (k slice kk of matrix ma).  The fragments of block q + 1 are read
+      // while block q multiplies, and the last block, which has nothing left to read, carries the LDS writes of the
+      // next stage and the global loads that refill their registers: the other stage was last read before the
+      // barrier that ended step ks - 1, and past the last step both are harmless (clamped addresses, a dead stage).
+      constexpr int Q = (BK / 32) * NMA;
+      gm_bf16x8_t fx[2][WTM], fw[2][WT];
+      const auto load_frags = [&](int q, int set) {
+        const int kk = q / NMA, m = SPLIT ? mat : q % NMA;
+        const int fcol = (((kk * 4) ^ fr_hi) + fr_lo) * 8;
 #pragma unroll
-      for (int kk = 0; kk < BK / 32; ++kk) {
+        for (int i = 0; i < WTM; ++i)
+          fx[set][i] = *reinterpret_cast<const gm_bf16x8_t*>(base + m * kTileX + (wm * 16 * WTM + i * 16 + lr) * kGLd + fcol);
 #pragma unroll
-        for (int ma = 0; ma < NMA; ++ma) {
-          const int m = SPLIT ? mat : ma;
-          gm_bf16x8_t fx[WTM], fw[WT];
-          const int fcol = (((kk * 4) ^ fr_hi) + fr_lo) * 8;
+        for (int i = 0; i < WT; ++i) {
+          const int wrow = EXPAND ? (i < 2 ? wn * 32 + i * 16 : 64 + wn * 32 + (i - 2) * 16) : wn * 16 * WT + i * 16;
+          fw[set][i] = *reinterpret_cast<const gm_bf16x8_t*>(base + NM * kTileX + m * kTileW + (wrow + lr) * kGLd + fcol);
+        }
+      };
+      load_frags(0, 0);
 #pragma unroll
-          for (int i = 0; i < WTM; ++i)
-            fx[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + m * kTileX + (wm * 16 * WTM + i * 16 + lr) * kGLd + fcol);
+      for (int q = 0; q < Q; ++q) {
+        if (q + 1 < Q) {
+          load_frags(q + 1, (q + 1) & 1);
+        } else {
+          store_lds((u + 1) % PF, (ks + 1) & 1);
+          load_regs((u + 1) % PF, ks + 1 + PF);
+        }
 #pragma unroll
-          for (int i = 0; i < WT; ++i) {
-            const int wrow = EXPAND ? (i < 2 ? wn * 32 + i * 16 : 64 + wn * 32 + (i - 2) * 16) : wn * 16 * WT + i * 16;
-            fw[i] = *reinterpret_cast<const gm_bf16x8_t*>(base + NM * kTileX + m * kTileW + (wrow + lr) * kGLd + fcol);
+        for (int i = 0; i < WTM; ++i)
+#pragma unroll
+          for (int j = 0; j < WT; ++j)
+            acc[q % NMA][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fx[q & 1][i], fw[q & 1][j], acc[q % NMA][i][j], 0, 0, 0);
+        // issue order: memory instructions spread between the products instead of ahead of them
+        constexpr int kMf = WTM * WT;
+        if (q + 1 < Q) {
+          constexpr int kRd = WTM + WT, kPer = kMf / kRd > 0 ? kMf / kRd : 1;
+#pragma unroll
+          for (int n = 0; n < kRd; ++n) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // one LDS read
+            __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);  // products
           }
+        } else {
+          constexpr int kWr = NM * (NPX + NP), kPer = kMf / kWr > 0 ? kMf / kWr : 1;
 #pragma unroll
-          for (int i = 0; i < WTM; ++i)
-#pragma unroll
-            for (int j = 0; j < WT; ++j)
-              acc[ma][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fx[i], fw[j], acc[ma][i][j], 0, 0, 0);
+          for (int n = 0; n < kWr; ++n) {
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);     // one LDS write
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);     // one global load
+            __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
+          }
         }
       }
-      if (ks + 1 < ksteps) {
-        // the other stage was last read before the barrier that ended step ks - 1
-        store_lds((u + 1) % PF, (ks + 1) & 1);
-        load_regs((u + 1) % PF, ks + 1 + PF);
-        __syncthreads();
-      }
+      __syncthreads();
     }
   }
 
