@@ -98,6 +98,14 @@ __device__ __forceinline__ void wait_stores_acked() {
   __builtin_amdgcn_s_waitcnt(0);   // vmcnt(0) expcnt(0) lgkmcnt(0)
 }
 
+// Workgroups are handed to the eight XCDs in turn (linear id % 8) and every XCD has an L2 of its own.  Position of
+// workgroup `linear` of `total` in an order that gives each XCD one contiguous run: workgroups that read the same
+// operands sit next to each other in that order and so share an L2.
+__device__ __forceinline__ int xcd_run_index(int linear, int total) {
+  const int xcd = linear & 7, q = total >> 3, rem = total & 7;
+  return xcd * q + min(xcd, rem) + (linear >> 3);
+}
+
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
 }  // namespace fsvd

@@ -4,8 +4,10 @@
 // holds 8 consecutive k of one row).  A workgroup of four waves owns a 128 x 128 output tile (a wave 64 x 64: 4 x 4
 // accumulator tiles) — or 64 x 64 when the problem has too few big tiles to give every compute unit work — and walks K
 // in steps of 64 or 128 through a double-buffered LDS stage (the 16-byte pieces of a row swizzled so that the fragment
-// reads of 16 consecutive rows fall on different banks).  Global loads run two to four steps ahead in registers and are written to
-// the idle LDS stage one step before their products.  Epilogue as in the vector kernels: bias, ONE rounding to bf16,
+// reads of 16 consecutive rows fall on different banks).  Two ways to fill a stage: global loads that run two to four
+// steps ahead in registers and are written to the idle stage one step before their products (few workgroups per compute
+// unit, long K: latency-bound), or loads that write LDS themselves one step ahead (no staging registers, no LDS write
+// instructions; pays when two or three workgroups share a compute unit).  Epilogue as in the vector kernels: bias, ONE rounding to bf16,
 // residual — or, for the gate / up pair, SwiGLU in either rounding mode — or the head expansion of the prompt pass
 // (RoPE, store into the query buffer or the cache rows).  Every weight is read once per 128 (64) rows of x.
 #include <algorithm>
@@ -45,6 +47,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   static_assert(NW == 4 || (NW == 8 && DUAL && WT == 4 && WTM == 4), "eight waves are the split form of the 128 x 128 pair tile");
   constexpr int kGT = NW * 64;
   constexpr bool SPLIT = NW == 8;
+  constexpr bool DTL = PF < 0;            // global loads write the LDS stages themselves (no register sets), -PF stages
+  constexpr int PFR = DTL ? 1 : PF;
+  constexpr int NS = DTL ? -PF : 2;       // LDS stages
   constexpr int NM = DUAL ? 2 : 1;
   constexpr int NMA = SPLIT ? 1 : NM;     // accumulator sets per wave
   constexpr int kGLd = BK;                // LDS row stride in elements: no padding, the 16-byte pieces of a row are swizzled
@@ -60,15 +65,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   const int tid = threadIdx.x, wave = (tid >> 6) & 3, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
   const int mat = SPLIT ? (tid >> 8) : 0;  // split form: which matrix of the pair this wave accumulates
   const int wm = wave >> 1, wn = wave & 1;
-  // Workgroups are handed to the eight XCDs in turn (linear id % 8), and each XCD has an L2 of its own: give every
-  // XCD one contiguous run of tiles, ordered in bands of eight row tiles walked column by column, so that the
-  // workgroups resident on an XCD at one time share a few x tiles and a few W tiles
+  // every XCD takes one contiguous run of tiles, ordered in bands of eight row tiles walked column by column, so that
+  // the workgroups resident on an XCD at one time share a few x tiles and a few W tiles in its L2
   int tile_m, tile_n;
   {
-    const int NT = gridDim.x, MT = gridDim.y, T = NT * MT;
-    const int L = blockIdx.y * NT + blockIdx.x;
-    const int xcd = L & 7, q = T >> 3, rem = T & 7;
-    const int t = xcd * q + min(xcd, rem) + (L >> 3);
+    const int NT = gridDim.x, MT = gridDim.y;
+    const int t = xcd_run_index(blockIdx.y * NT + blockIdx.x, NT * MT);
     const int band = t / (8 * NT), tb = t - band * 8 * NT;
     const int bh = min(8, MT - band * 8);
     tile_n = tb / bh;
@@ -92,25 +94,28 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   // swizzle term of a thread never changes.
   static_assert(RPP % CPR == 0 && CPR <= 16, "swizzle term must be constant per thread");
   const int st_chunk = ld_chunk ^ (ld_row % CPR);
+  // direct form: lane i of a load instruction lands at 16 i bytes past the instruction's LDS base, i.e. at piece
+  // ld_chunk of its row, so it fetches the piece that belongs there
+  const int g_chunk = DTL ? st_chunk : ld_chunk;
   const int fr_hi = (lr % CPR) & ~3, fr_lo = lg ^ (lr & 3);   // fragment piece kk*4 + lg -> ((kk*4) ^ fr_hi) + fr_lo
   const uint16_t* gx[NM][NPX];
   const uint16_t* gw[NM][NP];
 #pragma unroll
   for (int j = 0; j < NPX; ++j) {
     const int64_t xr = min(m0 + ld_row + RPP * j, a.B - 1);
-    if (EXPAND) gx[0][j] = a.x + (xr / ep.M) * ep.sp_b + (xr % ep.M) * ep.sp_m + ld_chunk * 8;
-    else gx[0][j] = a.x + xr * a.ldx + ld_chunk * 8;
-    if (DUAL) gx[NM - 1][j] = a.x + xr * a.ldx + a.up_off + ld_chunk * 8;
+    if (EXPAND) gx[0][j] = a.x + (xr / ep.M) * ep.sp_b + (xr % ep.M) * ep.sp_m + g_chunk * 8;
+    else gx[0][j] = a.x + xr * a.ldx + g_chunk * 8;
+    if (DUAL) gx[NM - 1][j] = a.x + xr * a.ldx + a.up_off + g_chunk * 8;
   }
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
     const int64_t wr = min(n0 + ld_row + RPP * j, a.N - 1);
-    gw[0][j] = a.W + wr * a.ldw + ld_chunk * 8;
-    if (DUAL) gw[NM - 1][j] = a.W2 + wr * a.ldw + ld_chunk * 8;
+    gw[0][j] = a.W + wr * a.ldw + g_chunk * 8;
+    if (DUAL) gw[NM - 1][j] = a.W2 + wr * a.ldw + g_chunk * 8;
   }
   // PF register sets hold the global loads of the next PF steps (set s % PF belongs to step s); a set is written
   // to the idle LDS stage one step before its products and refilled at once with the loads of step s + PF
-  u32x4_t rx[PF][NM][NPX], rw[PF][NM][NP];
+  u32x4_t rx[PFR][NM][NPX], rw[PFR][NM][NP];
   auto load_regs = [&](int set, int ks) {
     const int k = min(kbeg + min(ks, ksteps - 1), ksteps_all - 1) * BK;   // past the end: a valid address, never used
 #pragma unroll
@@ -135,6 +140,22 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
     }
   };
 
+  typedef const __attribute__((address_space(1))) void* gm_gptr_t;
+  typedef __attribute__((address_space(3))) void* gm_lptr_t;
+  const auto issue_direct = [&](int stage, int ks) {
+    const int k = min(kbeg + min(ks, ksteps - 1), ksteps_all - 1) * BK;
+    uint16_t* sb = lds + stage * kStage + ((tid >> 6) * (64 / CPR)) * kGLd;   // this wave's rows of a pass
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+#pragma unroll
+      for (int j = 0; j < NPX; ++j)
+        __builtin_amdgcn_global_load_lds((gm_gptr_t)(gx[m][j] + k), (gm_lptr_t)(sb + m * kTileX + RPP * j * kGLd), 16, 0, 0);
+#pragma unroll
+      for (int j = 0; j < NP; ++j)
+        __builtin_amdgcn_global_load_lds((gm_gptr_t)(gw[m][j] + k), (gm_lptr_t)(sb + NM * kTileX + m * kTileW + RPP * j * kGLd), 16, 0, 0);
+    }
+  };
+
   gm_f32x4_t acc[NMA][WTM][WT];
 #pragma unroll
   for (int m = 0; m < NMA; ++m)
@@ -143,17 +164,28 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
 #pragma unroll
       for (int j = 0; j < WT; ++j) acc[m][i][j] = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
 
+  // direct form: the loads of step s + NS - 1 are issued during step s; all but the newest NS - 2 groups of kLd loads
+  // have to be complete before the barrier that opens the next stage
+  constexpr int kLd = NM * (NPX + NP), kOpen = (NS - 2) * kLd;
+  static_assert(kOpen < 64, "vmcnt holds six bits");
+  constexpr int kWaitOpen = (kOpen & 15) | (7 << 4) | (15 << 8) | ((kOpen >> 4) << 14);
+  if (DTL) {
 #pragma unroll
-  for (int u = 0; u < PF; ++u) load_regs(u, u);
-  store_lds(0, 0);
-  load_regs(0, PF);
+    for (int s0 = 0; s0 < NS - 1; ++s0) issue_direct(s0, s0);
+    __builtin_amdgcn_s_waitcnt(kWaitOpen);
+  } else {
+#pragma unroll
+    for (int u = 0; u < PFR; ++u) load_regs(u, u);
+    store_lds(0, 0);
+    load_regs(0, PFR);
+  }
   __syncthreads();
-  for (int ks0 = 0; ks0 < ksteps; ks0 += PF) {
+  for (int ks0 = 0; ks0 < ksteps; ks0 += PFR) {
 #pragma unroll
-    for (int u = 0; u < PF; ++u) {
+    for (int u = 0; u < PFR; ++u) {
       const int ks = ks0 + u;
       if (ks >= ksteps) break;
-      const uint16_t* base = lds + (ks & 1) * kStage;
+      const uint16_t* base = lds + (ks % NS) * kStage;
       // The step as Q blocks of WTM x WT products (k slice kk of matrix ma).  The fragments of block q + 1 are read
       // while block q multiplies, and the last block, which has nothing left to read, carries the LDS writes of the
       // next stage and the global loads that refill their registers: the other stage was last read before the
@@ -175,11 +207,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
       load_frags(0, 0);
 #pragma unroll
       for (int q = 0; q < Q; ++q) {
+        if (DTL && q == 0) issue_direct((ks + NS - 1) % NS, ks + NS - 1);
         if (q + 1 < Q) {
           load_frags(q + 1, (q + 1) & 1);
-        } else {
-          store_lds((u + 1) % PF, (ks + 1) & 1);
-          load_regs((u + 1) % PF, ks + 1 + PF);
+        } else if (!DTL) {
+          store_lds((u + 1) % PFR, (ks + 1) & 1);
+          load_regs((u + 1) % PFR, ks + 1 + PFR);
         }
 #pragma unroll
         for (int i = 0; i < WTM; ++i)
@@ -195,7 +228,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // one LDS read
             __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);  // products
           }
-        } else {
+        } else if (!DTL) {
           constexpr int kWr = NM * (NPX + NP), kPer = kMf / kWr > 0 ? kMf / kWr : 1;
 #pragma unroll
           for (int n = 0; n < kWr; ++n) {
@@ -205,6 +238,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
           }
         }
       }
+      if (DTL) __builtin_amdgcn_s_waitcnt(kWaitOpen);   // this wave's pieces of the next stage have landed
       __syncthreads();
     }
   }
@@ -348,15 +382,15 @@ static int pick_ksplit(int64_t tiles, int ksteps, size_t floats_per_share, const
   return std::max(z, 1);
 }
 
-template <bool DUAL, int WTM, int WT, int BK, int NW = 4>
+template <bool DUAL, int WTM, int WT, int BK, int NW = 4, int PFSEL = 99>
 static int launch_gemm_tiles_t(const MfmaArgs& a0, hipStream_t st, const char* who) {
   static bool granted = false;
   constexpr int BM = 32 * WTM, BN = 32 * WT;
   constexpr int kGLd = BK;
   // register sets in flight: deep for the small single tile (few workgroups, latency-bound), two where a deeper
   // pipeline would cost a resident wave per SIMD
-  constexpr int PF = (!DUAL && WT == 2 && WTM == 2 && BK == 64) ? 4 : 2;
-  const size_t lds = (size_t)2 * (DUAL ? 2 : 1) * (BM + BN) * kGLd * 2;
+  constexpr int PF = PFSEL != 99 ? PFSEL : (!DUAL && WT == 2 && WTM == 2 && BK == 64) ? 4 : 2;
+  const size_t lds = (size_t)(PF < 0 ? -PF : 2) * (DUAL ? 2 : 1) * (BM + BN) * kGLd * 2;
   if (lds > 64 * 1024 && !granted) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WTM, WT, PF, false, BK, NW>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -384,11 +418,16 @@ int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* 
   // Forms by tile count (measured on the projections of the 7B shape at 128..4096 rows).  The pair kernel: the
   // eight-wave 128 x 128 form from two big tiles per compute unit on, else 64 x 64.  A single matrix: 128 x 128 from
   // 448 big tiles on, 128 x 64 from 256 on, else 64 x 64 — in K steps of 64 with a deep register pipeline when there
-  // are more of those than the chip holds at once (320), in steps of 128 (half as many barriers) when there are fewer.
+  // are more of those than the chip holds at once (320), in steps of 128 (half as many barriers) when there are fewer:
+  // with one workgroup or less per compute unit and a long K only loads issued several steps ahead hide the latency.
   if (dual) return big >= 512 ? launch_gemm_tiles_t<true, 4, 4, 64, 8>(a, st, who) : launch_gemm_tiles_t<true, 2, 2, 64>(a, st, who);
-  if (big >= 448) return launch_gemm_tiles_t<false, 4, 4, 64>(a, st, who);
-  if (big >= 256) return launch_gemm_tiles_t<false, 4, 2, 64>(a, st, who);
+  // a single matrix with at least one big tile per compute unit: loads straight into LDS, two stages (the second and
+  // third workgroup of a compute unit cover the one-step load distance; 4..12 % faster than the register pipeline)
+  if (big >= 448) return launch_gemm_tiles_t<false, 4, 4, 64, 4, -2>(a, st, who);
+  if (big >= 256) return launch_gemm_tiles_t<false, 4, 2, 64, 4, -2>(a, st, who);
   const int64_t small = (int64_t)((a.N + 63) / 64) * ((a.B + 63) / 64);
+  // short K and two small tiles per compute unit: the same, in steps of 128 (q_u / down_u at 512 rows: 12 -> 10 us)
+  if (small >= 512 && a.K <= 2048 && (a.K % 128) == 0) return launch_gemm_tiles_t<false, 2, 2, 128, 4, -2>(a, st, who);
   return (small < 320 && (a.K % 128) == 0) ? launch_gemm_tiles_t<false, 2, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 2, 2, 64>(a, st, who);
 }
 
@@ -415,7 +454,7 @@ template <int WTM>
 static int launch_expand_tiles_t(const ExpandArgs& a, hipStream_t st) {
   const char* who = "fsvd_lowrank_expand_heads";
   static bool granted = false;
-  constexpr int PF = 2;
+  constexpr int PF = 2;   // register pipeline (loads straight into LDS were slower here: 0.92 -> 1.03 ms at 8 x 2048 rows)
   constexpr int kGLd = kGBK;
   constexpr int BM = 32 * WTM;
   const size_t lds = (size_t)2 * (BM + 128) * kGLd * 2;

@@ -256,12 +256,19 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
 // ---------------------------------------------------------------------------------------------
 template <int MI>
 __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(PrefillAttnArgs a) {
-  constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, KSTR = DH + 8, VSTR = BN + 8;
+  constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, VSTR = BN + 8;
+  // K rows of 288 bytes: a 16-byte LDS read is served 16 lanes a cycle (lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of a
+  // half wave); rows 16 r apart with r odd multiples of 32 bytes give those lanes 16 different bank groups
+  constexpr int KSTR = DH + 16;
   extern __shared__ __align__(16) unsigned char pw_smem[];
   uint16_t (*Ks)[KSTR] = reinterpret_cast<uint16_t (*)[KSTR]>(pw_smem);                              // [BN][KSTR]
   uint16_t (*Vt)[VSTR] = reinterpret_cast<uint16_t (*)[VSTR]>(pw_smem + (size_t)BN * KSTR * 2);       // [DH][VSTR]
 
-  const int mt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // the query tiles of a head (and the heads of a kv head) run on one XCD, so its K and V come out of one L2; under
+  // a causal mask the last tiles, which see the most keys, start first
+  const int MT = gridDim.x;
+  const int t = xcd_run_index(blockIdx.x + MT * (blockIdx.y + gridDim.y * blockIdx.z), MT * gridDim.y * gridDim.z);
+  const int mt = a.causal ? MT - 1 - t % MT : t % MT, h = (t / MT) % (int)gridDim.y, b = t / (MT * (int)gridDim.y);
   const int hk = h / (a.H / a.Hk);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, lg = lane >> 4;
@@ -470,7 +477,7 @@ int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
   if (a.M >= 128 && out8) {   // long prompts: 64 or 128 queries per workgroup, K / V tiles shared through LDS
     // 128 query rows per workgroup when that gives every compute unit work, else 64 (half the rows per wave)
     const bool wide = (int64_t)((a.M + 127) / 128) * a.H * a.B >= 384;
-    const size_t lds = (size_t)64 * 136 * 2 + (size_t)128 * 72 * 2;
+    const size_t lds = (size_t)64 * 144 * 2 + (size_t)128 * 72 * 2;
     if (wide) hipLaunchKernelGGL(attn_prefill_wide_kernel<2>, dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
     else hipLaunchKernelGGL(attn_prefill_wide_kernel<1>, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), lds, st, a);
   } else {

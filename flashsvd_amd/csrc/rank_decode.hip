@@ -35,17 +35,23 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
   __shared__ float qs[REP][DH];
   __shared__ float wm[4][REP], wl[4][REP];
-  // one LDS block, used twice: k_u chunks [2][128 d][64 r + 8 pad] bf16 while the keys stream, the four waves'
+  // one LDS block, used twice: k_u chunks [2][128 d][64 r] bf16 while the keys stream, the four waves'
   // rank-space partials [4][kRdMaxChunks*512] fp32 for the merge at the end
-  constexpr int KROW = 72;                         // 144-byte rows keep the 16-byte fragment reads off each other's banks
+  // 128-byte rows, 16-byte piece c of row d stored at piece c ^ (d % 8): a 16-byte LDS read is served 16 lanes a cycle
+  // (lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of a half wave), and with this placement the fragment reads (lane =
+  // row % 16 + 16 * piece) touch every bank once per group (rows padded to 144 bytes put two lanes on a bank)
+  constexpr int KROW = 64;
   constexpr int KU_BYTES = 2 * DH * KROW * 2, TB_BYTES = 4 * kRdMaxChunks * 512 * 4;
   __shared__ __align__(16) unsigned char smem[KU_BYTES > TB_BYTES ? KU_BYTES : TB_BYTES];
   uint16_t (*kus)[DH][KROW] = reinterpret_cast<uint16_t (*)[DH][KROW]>(smem);
   float (*tbuf)[kRdMaxChunks * 512] = reinterpret_cast<float (*)[kRdMaxChunks * 512]>(smem);
 
   const int groups = a.H / a.Hk / REP;             // q-head groups per kv head handled by separate blocks
-  const int s = blockIdx.x, b = blockIdx.z;
-  const int hk = blockIdx.y / groups, grp = blockIdx.y % groups;
+  // the head groups of one key range (they read the same cache rows) are neighbours on one XCD
+  const int GY = gridDim.y;
+  const int t = xcd_run_index(blockIdx.x + (int)gridDim.x * (blockIdx.y + GY * blockIdx.z), (int)gridDim.x * GY * gridDim.z);
+  const int gy = t % GY, s = (t / GY) % (int)gridDim.x, b = t / (GY * (int)gridDim.x);
+  const int hk = gy / groups, grp = gy % groups;
   const int h0 = hk * (a.H / a.Hk) + grp * REP;    // first q head of this block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, lg = lane >> 4;        // column-in-tile / row group
@@ -123,7 +129,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
     };
     const auto store_ku = [&](int buf) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t*>(&kus[buf][krow][kcol + i * 8]) = kreg[i];
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t*>(&kus[buf][krow][(((kcol >> 3) + i) ^ (krow & 7)) * 8]) = kreg[i];
     };
     const auto load_pk = [&](int r0) {
 #pragma unroll
@@ -143,7 +149,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
       for (int k = 0; k < 2; ++k) {
         bf16x8_t bf[NT];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][k * 32 + lg * 8]));
+        for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
 #pragma unroll
         for (int j = 0; j < KS; ++j)
 #pragma unroll
