@@ -92,12 +92,14 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   // below (lane = row % 16 + 16 * piece) touch every bank once per group, which row padding of 16 bytes does not
   // achieve (two lanes per bank, half the read rate).  RPP and the fragment row bases are multiples of CPR, so the
   // swizzle term of a thread never changes.
-  static_assert(RPP % CPR == 0 && CPR <= 16, "swizzle term must be constant per thread");
-  const int st_chunk = ld_chunk ^ (ld_row % CPR);
+  // (Rows of 64 bytes, K steps of 32: four rows span the banks once, and the term is (-(r / 4)) % 4 instead.)
+  static_assert(RPP % 16 == 0 && CPR >= 4 && CPR <= 16, "swizzle term must be constant per thread");
+  const auto swz = [](int r) { return CPR == 4 ? ((-(r >> 2)) & 3) : r % CPR; };
+  const int st_chunk = ld_chunk ^ swz(ld_row);
   // direct form: lane i of a load instruction lands at 16 i bytes past the instruction's LDS base, i.e. at piece
   // ld_chunk of its row, so it fetches the piece that belongs there
   const int g_chunk = DTL ? st_chunk : ld_chunk;
-  const int fr_hi = (lr % CPR) & ~3, fr_lo = lg ^ (lr & 3);   // fragment piece kk*4 + lg -> ((kk*4) ^ fr_hi) + fr_lo
+  const int fr_hi = swz(lr) & ~3, fr_lo = lg ^ (swz(lr) & 3);   // fragment piece kk*4 + lg -> ((kk*4) ^ fr_hi) + fr_lo
   const uint16_t* gx[NM][NPX];
   const uint16_t* gw[NM][NP];
 #pragma unroll
@@ -420,6 +422,9 @@ int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* 
   // 448 big tiles on, 128 x 64 from 256 on, else 64 x 64 — in K steps of 64 with a deep register pipeline when there
   // are more of those than the chip holds at once (320), in steps of 128 (half as many barriers) when there are fewer:
   // with one workgroup or less per compute unit and a long K only loads issued several steps ahead hide the latency.
+  // the pair at four big tiles per compute unit and more: four waves with both accumulator sets, K steps of 32
+  // loaded straight into LDS (two workgroups per compute unit; 221 -> 197 us at 2048 rows of the 7B MLP)
+  if (dual && big >= 1024) return launch_gemm_tiles_t<true, 4, 4, 32, 4, -2>(a, st, who);
   if (dual) return big >= 512 ? launch_gemm_tiles_t<true, 4, 4, 64, 8>(a, st, who) : launch_gemm_tiles_t<true, 2, 2, 64>(a, st, who);
   // a single matrix with at least one big tile per compute unit: loads straight into LDS, two stages (the second and
   // third workgroup of a compute unit cover the one-step load distance; 4..12 % faster than the register pipeline)
