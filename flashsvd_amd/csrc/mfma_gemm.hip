@@ -422,17 +422,17 @@ int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* 
   // 448 big tiles on, 128 x 64 from 256 on, else 64 x 64 — in K steps of 64 with a deep register pipeline when there
   // are more of those than the chip holds at once (320), in steps of 128 (half as many barriers) when there are fewer:
   // with one workgroup or less per compute unit and a long K only loads issued several steps ahead hide the latency.
-  // the pair at four big tiles per compute unit and more: four waves with both accumulator sets, K steps of 32
-  // loaded straight into LDS (two workgroups per compute unit; 221 -> 197 us at 2048 rows of the 7B MLP)
+  // The pair at four big tiles per compute unit and more: four waves with both accumulator sets, K steps of 32
+  // loaded straight into LDS (two workgroups per compute unit; 243 -> 214 us at 2048 rows of the 7B MLP)
   if (dual && big >= 1024) return launch_gemm_tiles_t<true, 4, 4, 32, 4, -2>(a, st, who);
   if (dual) return big >= 512 ? launch_gemm_tiles_t<true, 4, 4, 64, 8>(a, st, who) : launch_gemm_tiles_t<true, 2, 2, 64>(a, st, who);
-  // a single matrix with at least one big tile per compute unit: loads straight into LDS, two stages (the second and
-  // third workgroup of a compute unit cover the one-step load distance; 4..12 % faster than the register pipeline)
+  // a single matrix with more than one big tile per compute unit: loads straight into LDS, two stages (the second and
+  // third workgroup of a compute unit cover the one-step load distance; 5..8 % faster than the register pipeline with
+  // weights that come from HBM, and slower than it below these tile counts)
   if (big >= 448) return launch_gemm_tiles_t<false, 4, 4, 64, 4, -2>(a, st, who);
-  if (big >= 256) return launch_gemm_tiles_t<false, 4, 2, 64, 4, -2>(a, st, who);
+  if (big >= 320) return launch_gemm_tiles_t<false, 4, 2, 64, 4, -2>(a, st, who);
+  if (big >= 256) return launch_gemm_tiles_t<false, 4, 2, 64>(a, st, who);
   const int64_t small = (int64_t)((a.N + 63) / 64) * ((a.B + 63) / 64);
-  // short K and two small tiles per compute unit: the same, in steps of 128 (q_u / down_u at 512 rows: 12 -> 10 us)
-  if (small >= 512 && a.K <= 2048 && (a.K % 128) == 0) return launch_gemm_tiles_t<false, 2, 2, 128, 4, -2>(a, st, who);
   return (small < 320 && (a.K % 128) == 0) ? launch_gemm_tiles_t<false, 2, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 2, 2, 64>(a, st, who);
 }
 
