@@ -247,7 +247,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
 
   // K split: park the partial tile (thread-major 16-byte words, coalesced), count arrivals; the last workgroup of a
   // tile adds all partials in split order (its own included, so the sum does not depend on who came last)
-  if (gridDim.z > 1) {
+  if (WTM == 1 && gridDim.z > 1) {         // only the 32-row tiles are ever launched with a split
     constexpr int WPT = NMA * WTM * WT;                          // 16-byte words per thread
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     gm_f32x4_t* part = reinterpret_cast<gm_f32x4_t*>(a.ws_part) + (size_t)tile * gridDim.z * WPT * kGT;
@@ -277,22 +277,42 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
     }
     __syncthreads();
     if (*flag == 0) return;
+    // the shares are added in split order; the loads of several shares are in flight at once (each comes from beyond
+    // this XCD's L2, and one share per round trip made the reduction the longest part of a narrow projection)
+    constexpr int ZC = WPT <= 2 ? 8 : (WPT <= 4 ? 4 : 2);
 #pragma unroll
     for (int m = 0; m < NMA; ++m)
 #pragma unroll
       for (int i = 0; i < WTM; ++i)
 #pragma unroll
-        for (int j = 0; j < WT; ++j) {
-          gm_f32x4_t sum = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
-          for (int z = 0; z < (int)gridDim.z; ++z) {
-            const unsigned long long* src = reinterpret_cast<const unsigned long long*>(part + (size_t)z * WPT * kGT + ((m * WTM + i) * WT + j) * kGT + tid);
-            const unsigned long long lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const unsigned long long hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            sum += gm_f32x4_t{__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)), __uint_as_float((uint32_t)hi),
-                              __uint_as_float((uint32_t)(hi >> 32))};
-          }
-          acc[m][i][j] = sum;
+        for (int j = 0; j < WT; ++j) acc[m][i][j] = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int z0 = 0; z0 < (int)gridDim.z; z0 += ZC) {
+      unsigned long long lo[ZC][WPT], hi[ZC][WPT];
+#pragma unroll
+      for (int u = 0; u < ZC; ++u) {
+        const int z = min(z0 + u, (int)gridDim.z - 1);
+#pragma unroll
+        for (int w = 0; w < WPT; ++w) {
+          const unsigned long long* src = reinterpret_cast<const unsigned long long*>(part + (size_t)z * WPT * kGT + w * kGT + tid);
+          lo[u][w] = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          hi[u][w] = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+      }
+#pragma unroll
+      for (int u = 0; u < ZC; ++u) {
+        if (z0 + u >= (int)gridDim.z) break;
+#pragma unroll
+        for (int m = 0; m < NMA; ++m)
+#pragma unroll
+          for (int i = 0; i < WTM; ++i)
+#pragma unroll
+            for (int j = 0; j < WT; ++j) {
+              const int w = (m * WTM + i) * WT + j;
+              acc[m][i][j] += gm_f32x4_t{__uint_as_float((uint32_t)lo[u][w]), __uint_as_float((uint32_t)(lo[u][w] >> 32)),
+                                         __uint_as_float((uint32_t)hi[u][w]), __uint_as_float((uint32_t)(hi[u][w] >> 32))};
+            }
+      }
+    }
   }
   // split pair: the up accumulators travel to the gate wave of the same block (same lane, same tile indices)
   gm_f32x4_t upv[SPLIT ? WT : 1][SPLIT ? WT : 1];
@@ -438,9 +458,12 @@ int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* 
 
 // 17..127 rows (batched decoding): 32-row tiles, 64 columns wide, K split over workgroups.  Needs the registered
 // workspace (without the split a narrow projection would occupy a fraction of the compute units).  Up to 16 rows the
-// wave-per-16-weight-rows kernel is as fast or faster (MLP of the 7B shape, 8 rows: 73 vs 79 us; 32 rows: 117 vs 81 us).
+// wave-per-16-weight-rows kernel is as fast or faster (MLP of the 7B shape, 8 rows: 73 vs 79 us; 32 rows: 117 vs 75 us)
+// unless the matrix has fewer than 128 of its 16-row tiles, one workgroup each (down_v of the 7B MLP, 1536 x 11008, at
+// 8 rows: 22.6 us there, 17 us here).
 bool gemm_rows_apply(const MfmaArgs& a) {
-  return a.B >= 17 && a.B < 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0 &&
+  const bool rows = a.B >= 17 || (a.B >= 3 && (a.N + 15) / 16 < 128);
+  return rows && a.B < 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0 &&
          split_workspace().part != nullptr;
 }
 int launch_gemm_rows(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {

@@ -48,7 +48,7 @@ _SPLIT_WS_BYTES = (64 << 20) + (64 << 10)
 
 
 def ensure_split_workspace(device: torch.device) -> bool:
-    """Register, once per device, the scratch the library's K-split projections (17..127 rows) work in.  The library
+    """Register, once per device, the scratch the library's K-split projections (3..127 rows) work in.  The library
     allocates nothing itself; this hands it 64 MiB of torch memory.  ``FLASHSVD_AMD_SPLITK=0`` keeps the projections
     unsplit; so does a first call made under stream capture (an allocation there would belong to the graph's pool).
     Launches that use the scratch must be ordered on one stream per device."""
@@ -104,7 +104,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             if t.shape != (n,) or not t.is_contiguous():
                 raise ValueError(f"{nm} must be a contiguous [{n}] tensor")
     lib = _lib.load()
-    if 17 <= B < 128:
+    if 3 <= B < 128:
         ensure_split_workspace(x.device)
     if norm_weight is not None and B >= 3 and cfg == 0 and K % 32 == 0:
         # three rows and more run on the matrix cores, which take the activations as they are: normalise once
@@ -133,7 +133,7 @@ def swiglu_linear(p: torch.Tensor, gate_u: torch.Tensor, up_u: torch.Tensor, *, 
         out = torch.empty(*p.shape[:-1], D, device=p.device, dtype=_BF16)
     o2 = _rows(out, "out")
     lib = _lib.load()
-    if 17 <= B < 128:
+    if 3 <= B < 128:
         ensure_split_workspace(p.device)
     rc = lib.fsvd_swiglu_linear(p2.data_ptr(), p2.stride(0), int(up_off), gate_u.data_ptr(), up_u.data_ptr(),
                                 gate_u.stride(0), o2.data_ptr(), o2.stride(0), B, D, R, int(mode), int(cfg), _stream())

@@ -39,9 +39,10 @@ extern "C" {
 int fsvd_version(void);
 const char* fsvd_last_error(void);
 
-/* Optional scratch for the projections of 17..127 rows (fsvd_linear, fsvd_swiglu_linear): with it they run on 32-row
- * tiles and split K over several workgroups per tile (fp32 partial tiles and arrival counters live in this buffer; the
- * sum is taken in a fixed order, so results do not depend on timing).
+/* Optional scratch for the projections of 17..127 rows, and of 3..16 rows when the matrix has fewer than 2048 rows
+ * (fsvd_linear, fsvd_swiglu_linear): with it they run on 32-row tiles and split K over several workgroups per tile
+ * (fp32 partial tiles and arrival counters live in this buffer; the sum is taken in a fixed order, so results do not
+ * depend on timing).
  * The library never allocates device memory: the caller owns `ws` (device memory of the current device, 256-byte
  * aligned, `bytes` >= 1 MiB to be of use, 64 MiB covers every shape of a 7B model) and keeps it alive until it
  * registers another buffer or NULL.  The first 64 KiB are cleared here, on `stream`.  One buffer per device; launches
