@@ -247,7 +247,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
 
   // K split: park the partial tile (thread-major 16-byte words, coalesced), count arrivals; the last workgroup of a
   // tile adds all partials in split order (its own included, so the sum does not depend on who came last)
-  if (WTM == 1 && gridDim.z > 1) {         // only the 32-row tiles are ever launched with a split
+  if (WTM <= 2 && gridDim.z > 1) {         // only the 32- and 64-row tiles are ever launched with a split
     constexpr int WPT = NMA * WTM * WT;                          // 16-byte words per thread
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     gm_f32x4_t* part = reinterpret_cast<gm_f32x4_t*>(a.ws_part) + (size_t)tile * gridDim.z * WPT * kGT;
@@ -396,12 +396,26 @@ bool gemm_tiles_apply(const MfmaArgs& a) {
 
 // K split for a grid of `tiles` workgroups: enough shares to give every compute unit two workgroups, at least four
 // K steps per share, and only as many as the registered workspace holds (1 = no split)
-static int pick_ksplit(int64_t tiles, int ksteps, size_t floats_per_share, const SplitWorkspace& ws) {
-  if (ws.part == nullptr || tiles >= 512 || tiles > ws.ncount) return 1;
-  int z = (int)((512 + tiles - 1) / tiles);
-  z = std::min(z, std::min(16, ksteps / 4));
+static int fit_ksplit(int z, int64_t tiles, int ksteps, size_t floats_per_share, const SplitWorkspace& ws, int cap) {
+  if (ws.part == nullptr || tiles > ws.ncount) return 1;
+  z = std::min(z, std::min(cap, ksteps / 4));
   while (z > 1 && (size_t)tiles * z * floats_per_share > ws.part_floats) --z;
   return std::max(z, 1);
+}
+static int pick_ksplit(int64_t tiles, int ksteps, size_t floats_per_share, const SplitWorkspace& ws) {
+  if (tiles >= 512) return 1;
+  return fit_ksplit((int)((512 + tiles - 1) / tiles), tiles, ksteps, floats_per_share, ws, 16);
+}
+// 64 x 64 tiles of a prompt projection (128 rows and more): a split pays only where the unsplit launch leaves compute
+// units idle (up to 128 tiles: two workgroups per tile-starved pair of compute units) or walks a very long K with at
+// most two workgroups per compute unit (down_v of the 7B MLP, K = 11008).  Measured at 128..1024 rows with weights from
+// HBM: o_v 18 -> 12..15 us, down_v 51 -> 25 (128 rows), 32 (256), 46 (512), 92 -> 76 (1024); everything else is as fast
+// or faster unsplit.
+static int pick_ksplit_prompt(int64_t tiles, int ksteps, int K, size_t floats_per_share, const SplitWorkspace& ws) {
+  int z = 1;
+  if (tiles <= 128) z = (int)((256 + tiles - 1) / tiles);
+  if (K >= 8192 && tiles < 512) z = std::max(z, (int)((768 + tiles - 1) / tiles));
+  return z > 1 ? fit_ksplit(z, tiles, ksteps, floats_per_share, ws, 8) : 1;
 }
 
 template <bool DUAL, int WTM, int WT, int BK, int NW = 4, int PFSEL = 99>
@@ -423,9 +437,11 @@ static int launch_gemm_tiles_t(const MfmaArgs& a0, hipStream_t st, const char* w
   dim3 grid((a.N + BN - 1) / BN, (a.B + BM - 1) / BM, 1);
   const SplitWorkspace ws = split_workspace();
   constexpr size_t share = (size_t)(DUAL && NW == 4 ? 2 : 1) * WTM * WT * 4 * NW * 64;   // floats one workgroup parks
-  // only the 32-row tiles split K: from 128 rows on a projection has enough tiles that parking and re-reading the
-  // partial tiles costs what the extra workgroups gain (measured at 512 rows: 42 -> 45 us, 25 -> 23 us, 64 -> 64 us)
-  a.ksplit = WTM == 1 ? pick_ksplit((int64_t)grid.x * grid.y, a.K / BK, share, ws) : 1;
+  // the 32-row tiles split K whenever that fills the chip; 64 x 64 prompt tiles only where measured to pay; larger
+  // tiles never (parking and re-reading the partial tiles costs what the extra workgroups gain)
+  if (WTM == 1) a.ksplit = pick_ksplit((int64_t)grid.x * grid.y, a.K / BK, share, ws);
+  else if (WTM == 2 && !DUAL) a.ksplit = pick_ksplit_prompt((int64_t)grid.x * grid.y, a.K / BK, a.K, share, ws);
+  else a.ksplit = 1;
   a.ws_part = ws.part;
   a.ws_count = ws.count;
   grid.z = a.ksplit;

@@ -104,7 +104,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             if t.shape != (n,) or not t.is_contiguous():
                 raise ValueError(f"{nm} must be a contiguous [{n}] tensor")
     lib = _lib.load()
-    if 3 <= B < 128:
+    if B >= 3:
         ensure_split_workspace(x.device)
     if norm_weight is not None and B >= 3 and cfg == 0 and K % 32 == 0:
         # three rows and more run on the matrix cores, which take the activations as they are: normalise once

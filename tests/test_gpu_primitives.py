@@ -224,9 +224,10 @@ def test_swiglu_prefill_rows_tiled_kernel(ops, B, D, R, mode):
 
 
 # ---- K split over workgroups (registered scratch): same entry points, 17..127 rows, and 3..16 rows of a matrix with
-#      fewer than 128 sixteen-row tiles
+#      fewer than 128 sixteen-row tiles, and prompt rows of projections with few 64 x 64 tiles or a very long K
 @pytest.mark.parametrize("B,N,K", [(17, 1536, 11008), (32, 1024, 4096), (100, 200, 1536), (127, 4096, 1536), (64, 3072, 4096),
-                                   (8, 1536, 11008), (3, 200, 1536), (16, 2032, 4096)])
+                                   (8, 1536, 11008), (3, 200, 1536), (16, 2032, 4096),
+                                   (128, 1024, 4096), (300, 1536, 11008), (512, 1000, 4096), (1024, 1536, 11008)])
 def test_linear_k_split_matches_unsplit_and_repeats(ops, B, N, K):
     x, w = rand_bf16(B, K, seed=1).cuda(), rand_bf16(N, K, std=0.02, seed=2).cuda()
     bias, res = rand_bf16(N, std=0.1, seed=4).cuda(), rand_bf16(B, N, seed=5).cuda()
