@@ -463,6 +463,53 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_kernel(const uint16_t* __res
   }
 }
 
+// the same with 16-byte accesses and the row kept in registers between the two passes (K a multiple of 8, at most
+// 8 * NC * kThreads, rows 16-byte aligned): a prompt of 512 rows x 4096 took 9.9 us with 2-byte accesses
+template <int NC>
+__global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                              const uint16_t* __restrict__ w, float eps,
+                                                              uint16_t* __restrict__ y, int64_t ldy, int K) {
+  __shared__ float red[kWaves];
+  const uint16_t* src = x + (int64_t)blockIdx.x * ldx;
+  uint16_t* dst = y + (int64_t)blockIdx.x * ldy;
+  const int nchunk = K >> 3;
+  u32x4_t v[NC];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int ch = threadIdx.x + c * kThreads;
+    v[c] = ch < nchunk ? *reinterpret_cast<const u32x4_t*>(src + ch * 8) : u32x4_t{0u, 0u, 0u, 0u};
+    const uint32_t e[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a = bf16_lo(e[i]), b = bf16_hi(e[i]);
+      ss += a * a;
+      ss += b * b;
+    }
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int i = 0; i < kWaves; ++i) tot += red[i];
+  const float rs = rsqrtf(tot / (float)K + eps);
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int ch = threadIdx.x + c * kThreads;
+    if (ch >= nchunk) break;
+    const u32x4_t wv = *reinterpret_cast<const u32x4_t*>(w + ch * 8);
+    const uint32_t e[4] = {v[c].x, v[c].y, v[c].z, v[c].w}, g[4] = {wv.x, wv.y, wv.z, wv.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a = round_bf16(bf16_lo(e[i]) * rs), b = round_bf16(bf16_hi(e[i]) * rs);
+      o[i] = f32_to_bf16_bits(bf16_lo(g[i]) * a) | (f32_to_bf16_bits(bf16_hi(g[i]) * b) << 16);
+    }
+    *reinterpret_cast<u32x4_t*>(dst + ch * 8) = u32x4_t{o[0], o[1], o[2], o[3]};
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // host-side launchers
 // ---------------------------------------------------------------------------------------
@@ -599,7 +646,11 @@ int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st) {
 int launch_rmsnorm(const uint16_t* x, int64_t ldx, const uint16_t* w, float eps, uint16_t* y, int64_t ldy, int rows,
                    int K, hipStream_t st) {
   if (rows <= 0 || K <= 0) { set_last_error("fsvd_rmsnorm: empty shape"); return kErrBadShape; }
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
+  const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool vec = (K % 8) == 0 && al(x) && al(w) && al(y) && (ldx % 8) == 0 && (ldy % 8) == 0;
+  if (vec && K <= 8 * 2 * kThreads) hipLaunchKernelGGL(rmsnorm_vec_kernel<2>, dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
+  else if (vec && K <= 8 * 8 * kThreads) hipLaunchKernelGGL(rmsnorm_vec_kernel<8>, dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
+  else hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
   FSVD_CHECK_LAUNCH("fsvd_rmsnorm");
   return kOk;
 }
