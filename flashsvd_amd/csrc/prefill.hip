@@ -245,7 +245,9 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
 //     through LDS.  With every wave fetching its own K fragments a 64-key tile costs 80 KB of L2 traffic per 64
 //     queries and the kernel is bound by L2 requests; here a tile is read ONCE per workgroup, coalesced, one tile
 //     ahead into registers, and written to LDS (K row-major with a padded stride, V transposed: four adjacent keys
-//     per 8-byte write, key column XOR-ed with 8 * (d / 8 % 8) to spread the 16 dimension blocks over the banks).
+//     per 8-byte write, rows of 128 bytes whose 16-byte pieces are XOR-ed with (d / 2 % 8) ^ (d / 8 % 8): the 16-byte
+//     fragment reads — served 16 lanes a cycle, lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of a half wave — and the
+//     8-byte transposing writes, 8 lanes a cycle, then both touch every bank once; found by enumeration).
 //
 //     Scores are computed TRANSPOSED, S^T = K Q^T: an accumulator lane then holds four consecutive keys of ONE query
 //     (column lr), so the softmax statistics are one value per lane and query block, and the eight softmax weights a
@@ -256,7 +258,7 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
 // ---------------------------------------------------------------------------------------------
 template <int MI>
 __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(PrefillAttnArgs a) {
-  constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, VSTR = BN + 8;
+  constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, VSTR = BN;
   // K rows of 288 bytes: a 16-byte LDS read is served 16 lanes a cycle (lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of a
   // half wave); rows 16 r apart with r odd multiples of 32 bytes give those lanes 16 different bank groups
   constexpr int KSTR = DH + 16;
@@ -322,7 +324,6 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(&Ks[srow + 16 * j][d0]) = kreg[j];
     {
-      const int col = vcol ^ (8 * ((tid & 15) & 7));
       const uint32_t w[4][4] = {{vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w}, {vreg[1].x, vreg[1].y, vreg[1].z, vreg[1].w},
                                 {vreg[2].x, vreg[2].y, vreg[2].z, vreg[2].w}, {vreg[3].x, vreg[3].y, vreg[3].z, vreg[3].w}};
 #pragma unroll
@@ -332,6 +333,8 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
         lo.y = (w[2][c] & 0xffffu) | (w[3][c] << 16);
         hi.x = (w[0][c] >> 16) | (w[1][c] & 0xffff0000u);
         hi.y = (w[2][c] >> 16) | (w[3][c] & 0xffff0000u);
+        // rows d0 + 2c and d0 + 2c + 1 share the swizzle term (row / 2 % 8) ^ (row / 8 % 8)
+        const int col = vcol ^ (8 * (((((tid & 1) << 2) + c) ^ (tid & 7))));
         *reinterpret_cast<u32x2_t*>(&Vt[d0 + 2 * c][col]) = lo;
         *reinterpret_cast<u32x2_t*>(&Vt[d0 + 2 * c + 1][col]) = hi;
       }
@@ -418,7 +421,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
     for (int st = 0; st < 2; ++st) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
-        const bf16x8_t vf = pf_ld(&Vt[t * 16 + lr][(st * 32 + lg * 8) ^ (8 * ((2 * t + (lr >> 3)) & 7))]);
+        const bf16x8_t vf = pf_ld(&Vt[t * 16 + lr][(st * 32 + lg * 8) ^ (8 * ((lr >> 1) ^ ((2 * t + (lr >> 3)) & 7)))]);
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
           o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph[mi][st], o[mi][t], 0, 0, 0);
@@ -477,7 +480,7 @@ int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
   if (a.M >= 128 && out8) {   // long prompts: 64 or 128 queries per workgroup, K / V tiles shared through LDS
     // 128 query rows per workgroup when that gives every compute unit work, else 64 (half the rows per wave)
     const bool wide = (int64_t)((a.M + 127) / 128) * a.H * a.B >= 384;
-    const size_t lds = (size_t)64 * 144 * 2 + (size_t)128 * 72 * 2;
+    const size_t lds = (size_t)64 * 144 * 2 + (size_t)128 * 64 * 2;
     if (wide) hipLaunchKernelGGL(attn_prefill_wide_kernel<2>, dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
     else hipLaunchKernelGGL(attn_prefill_wide_kernel<1>, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), lds, st, a);
   } else {
