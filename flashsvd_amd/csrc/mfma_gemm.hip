@@ -220,7 +220,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
         for (int i = 0; i < WTM; ++i)
 #pragma unroll
           for (int j = 0; j < WT; ++j)
-            acc[q % NMA][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fx[q & 1][i], fw[q & 1][j], acc[q % NMA][i][j], 0, 0, 0);
+            acc[q % NMA][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[q & 1][j], fx[q & 1][i], acc[q % NMA][i][j], 0, 0, 0);
         // issue order: memory instructions spread between the products instead of ahead of them
         constexpr int kMf = WTM * WT;
         if (q + 1 < Q) {
@@ -332,43 +332,89 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
 #pragma unroll
       for (int j = 0; j < WT; ++j) upv[i][j] = ex[(i * WT + j) * 256 + (tid & 255)];
   }
-  // element e of lane l of tile (i, j): row m = i*16 + (l/16)*4 + e of x, column n = j*16 + l%16 of W
+  // The products are taken as W . x^T (W fragment as the first operand), so element e of lane l of tile (i, j) is row
+  // m = i*16 + l%16 of x and column n = j*16 + (l/16)*4 + e of W: a lane owns four consecutive columns of one row and
+  // stores them with one 8-byte write (one 2-byte write each when the destination is not 8-byte aligned)
+  const auto al8 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7) == 0; };
 #pragma unroll
-  for (int i = 0; i < WTM; ++i)
+  for (int i = 0; i < WTM; ++i) {
+    const int m = m0 + wm * 16 * WTM + i * 16 + lr;
+    if (m >= a.B) continue;
+    if (EXPAND) {
+      const int b = m / ep.M, t = m - b * ep.M;
+      const int pos = (ep.positions ? ep.positions[b] : 0) + t;
+      const int slot = ep.dst_by_position ? pos : t;
+      if (slot < 0 || slot >= ep.dst_rows) continue;   // outside the destination: dropped
+      const int head = tile_n;
+      uint16_t* dst = a.y + (int64_t)b * ep.sy_b + (int64_t)slot * ep.sy_m + (int64_t)head * ep.sy_h;
+      const int tp = min(max(pos, 0), ep.rope_len - 1);
+      const bool dst8 = al8(dst), tab8 = ep.cos && al8(ep.cos) && al8(ep.sin);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int m = m0 + wm * 16 * WTM + i * 16 + lg * 4 + e;
-      if (m >= a.B) continue;
-      if (EXPAND) {
-        const int b = m / ep.M, t = m - b * ep.M;
-        const int pos = (ep.positions ? ep.positions[b] : 0) + t;
-        const int slot = ep.dst_by_position ? pos : t;
-        if (slot < 0 || slot >= ep.dst_rows) continue;   // outside the destination: dropped
-        const int head = tile_n;
-        uint16_t* dst = a.y + (int64_t)b * ep.sy_b + (int64_t)slot * ep.sy_m + (int64_t)head * ep.sy_h;
-        const int tp = min(max(pos, 0), ep.rope_len - 1);
+      for (int j = 0; j < 2; ++j) {
+        const int d0 = wn * 32 + j * 16 + lg * 4;
+        float c[4], sn[4];
+        if (ep.cos) {
+          if (tab8) {
+            const u32x2_t cw = *reinterpret_cast<const u32x2_t*>(ep.cos + (int64_t)tp * 64 + d0);
+            const u32x2_t sw = *reinterpret_cast<const u32x2_t*>(ep.sin + (int64_t)tp * 64 + d0);
+            c[0] = bf16_lo(cw.x); c[1] = bf16_hi(cw.x); c[2] = bf16_lo(cw.y); c[3] = bf16_hi(cw.y);
+            sn[0] = bf16_lo(sw.x); sn[1] = bf16_hi(sw.x); sn[2] = bf16_lo(sw.y); sn[3] = bf16_hi(sw.y);
+          } else {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int d = wn * 32 + j * 16 + lr;
+            for (int e = 0; e < 4; ++e) {
+              c[e] = bf16_bits_to_f32(ep.cos[(int64_t)tp * 64 + d0 + e]);
+              sn[e] = bf16_bits_to_f32(ep.sin[(int64_t)tp * 64 + d0 + e]);
+            }
+          }
+        }
+        uint32_t o0[4], o1[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int d = d0 + e;
           float x0 = acc[0][i][j][e], x1 = acc[0][i][j + 2][e];
           if (a.bias) { x0 += bf16_bits_to_f32(a.bias[head * 128 + d]); x1 += bf16_bits_to_f32(a.bias[head * 128 + d + 64]); }
           x0 = round_bf16(x0);                          // the projection's own rounding point
           x1 = round_bf16(x1);
           if (ep.cos) {                                 // eager bf16 arithmetic, one rounding per op
-            const float c = bf16_bits_to_f32(ep.cos[(int64_t)tp * 64 + d]), sn = bf16_bits_to_f32(ep.sin[(int64_t)tp * 64 + d]);
-            const float r0 = round_bf16(round_bf16(x0 * c) - round_bf16(x1 * sn));
-            const float r1 = round_bf16(round_bf16(x1 * c) + round_bf16(x0 * sn));
+            const float r0 = round_bf16(round_bf16(x0 * c[e]) - round_bf16(x1 * sn[e]));
+            const float r1 = round_bf16(round_bf16(x1 * c[e]) + round_bf16(x0 * sn[e]));
             x0 = r0; x1 = r1;
           }
-          dst[d] = (uint16_t)f32_to_bf16_bits(x0);
-          dst[d + 64] = (uint16_t)f32_to_bf16_bits(x1);
+          o0[e] = f32_to_bf16_bits(x0);
+          o1[e] = f32_to_bf16_bits(x1);
         }
-        continue;
-      }
+        if (dst8) {
+          *reinterpret_cast<u32x2_t*>(dst + d0) = u32x2_t{o0[0] | (o0[1] << 16), o0[2] | (o0[3] << 16)};
+          *reinterpret_cast<u32x2_t*>(dst + d0 + 64) = u32x2_t{o1[0] | (o1[1] << 16), o1[2] | (o1[3] << 16)};
+        } else {
 #pragma unroll
-      for (int j = 0; j < WT; ++j) {
-        const int n = n0 + wn * 16 * WT + j * 16 + lr;
-        if (n >= a.N) continue;
+          for (int e = 0; e < 4; ++e) { dst[d0 + e] = (uint16_t)o0[e]; dst[d0 + 64 + e] = (uint16_t)o1[e]; }
+        }
+      }
+      continue;
+    }
+    uint16_t* yrow = a.y + (int64_t)m * a.ldy;
+    const uint16_t* rrow = a.res ? a.res + (int64_t)m * a.ldres : nullptr;
+    const bool y8 = al8(yrow), r8 = rrow && al8(rrow);
+#pragma unroll
+    for (int j = 0; j < WT; ++j) {
+      const int nb = n0 + wn * 16 * WT + j * 16 + lg * 4;
+      if (nb >= a.N) continue;
+      const bool whole = nb + 3 < a.N;
+      float r[4] = {0.f, 0.f, 0.f, 0.f};
+      if (!DUAL && rrow) {
+        if (whole && r8) {
+          const u32x2_t rw = *reinterpret_cast<const u32x2_t*>(rrow + nb);
+          r[0] = bf16_lo(rw.x); r[1] = bf16_hi(rw.x); r[2] = bf16_lo(rw.y); r[3] = bf16_hi(rw.y);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (nb + e < a.N) r[e] = bf16_bits_to_f32(rrow[nb + e]);
+        }
+      }
+      uint32_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
         float v0 = acc[0][i][j][e];
         float v;
         if (DUAL) {
@@ -381,13 +427,21 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
             v = round_bf16((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
           }
         } else {
-          if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
+          if (a.bias && nb + e < a.N) v0 += bf16_bits_to_f32(a.bias[nb + e]);
           v = round_bf16(v0);
-          if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)m * a.ldres + n]) + v);
+          if (rrow) v = round_bf16(r[e] + v);
         }
-        a.y[(int64_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+        o[e] = f32_to_bf16_bits(v);
+      }
+      if (whole && y8) {
+        *reinterpret_cast<u32x2_t*>(yrow + nb) = u32x2_t{o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (nb + e < a.N) yrow[nb + e] = (uint16_t)o[e];
       }
     }
+  }
 }
 
 bool gemm_tiles_apply(const MfmaArgs& a) {
