@@ -16,6 +16,15 @@ _lib = None
 _i32p = ctypes.POINTER(ctypes.c_int32)
 
 
+class ExpandDesc(ctypes.Structure):
+    """fsvd_expand_desc: one head expansion of a batched call (fsvd_lowrank_expand_heads_multi)."""
+    _fields_ = [("p", c_void_p), ("sp_b", c_int64), ("sp_m", c_int64), ("sp_h", c_int64),
+                ("u", c_void_p), ("ldu", c_int64), ("bias", c_void_p),
+                ("y", c_void_p), ("sy_b", c_int64), ("sy_m", c_int64), ("sy_h", c_int64),
+                ("heads", ctypes.c_int32), ("R", ctypes.c_int32), ("rotate", ctypes.c_int32),
+                ("dst_by_position", ctypes.c_int32), ("dst_rows", ctypes.c_int32), ("rsv0", ctypes.c_int32)]
+
+
 class TagBuf(ctypes.Structure):
     """fsvd_tagbuf: a tagged hand-off vector and which of its per-step uses a phase touches."""
     _fields_ = [("ptr", c_void_p), ("uses_per_step", ctypes.c_int32), ("use", ctypes.c_int32)]
@@ -76,6 +85,8 @@ SIGNATURES = {
     "fsvd_lowrank_expand_heads": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
                                           c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
                                           c_int, c_void_p]),
+    "fsvd_lowrank_expand_heads_multi": (c_int, [ctypes.POINTER(ExpandDesc), c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                                c_void_p]),
     "fsvd_attn_prefill": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p,
                                   c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),

@@ -454,6 +454,40 @@ int fsvd_lowrank_expand_heads(const void* p, int64_t sp_b, int64_t sp_m, int64_t
   return launch_expand(a, static_cast<hipStream_t>(stream));
 }
 
+int fsvd_lowrank_expand_heads_multi(const fsvd_expand_desc* desc, int n, const void* cos, const void* sin, int rope_len,
+                                    const int32_t* positions, int B, int M, int Dh, void* stream) {
+  const char* fn = "fsvd_lowrank_expand_heads_multi";
+  FSVD_REQUIRE_PTR(desc, fn);
+  if (n < 1 || n > 3) { set_last_error("%s: %d descriptors (1..3)", fn, n); return kErrBadShape; }
+  if ((cos == nullptr) != (sin == nullptr) || (cos && rope_len <= 0)) { set_last_error("%s: cos/sin must both be set with rope_len > 0", fn); return kErrBadShape; }
+  ExpandArgs a[3];
+  for (int k = 0; k < n; ++k) {
+    const fsvd_expand_desc& d = desc[k];
+    FSVD_REQUIRE_PTR(d.p, fn); FSVD_REQUIRE_PTR(d.u, fn); FSVD_REQUIRE_PTR(d.y, fn);
+    if (d.rotate && !cos) { set_last_error("%s: descriptor %d asks for the rotation but no tables were given", fn, k); return kErrBadShape; }
+    if (d.ldu < d.R || d.sy_h < Dh || d.dst_rows <= 0) {
+      set_last_error("%s: descriptor %d: inconsistent strides (ldu=%lld R=%d sy_h=%lld dst_rows=%d)", fn, k, (long long)d.ldu, d.R, (long long)d.sy_h, d.dst_rows);
+      return kErrBadShape;
+    }
+    a[k] = ExpandArgs{cu16(d.p), d.sp_b, d.sp_m, d.sp_h, cu16(d.u), d.ldu, cu16(d.bias), d.rotate ? cu16(cos) : nullptr,
+                      d.rotate ? cu16(sin) : nullptr, rope_len, positions, u16(d.y), d.sy_b, d.sy_m, d.sy_h, d.dst_by_position,
+                      d.dst_rows, B, M, d.heads, Dh, d.R};
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (expand_multi_apply(a, n)) {
+    // the single-expansion checks (head_dim, alignment) hold for every descriptor: expand_tiles_apply covers strides
+    // and rank, the pointers are checked here
+    bool ok = true;
+    for (int k = 0; k < n; ++k) ok = ok && ((reinterpret_cast<uintptr_t>(a[k].p) | reinterpret_cast<uintptr_t>(a[k].u)) & 15) == 0 && (a[k].sp_h % 8) == 0;
+    if (ok) return launch_expand_multi(a, n, st);
+  }
+  for (int k = 0; k < n; ++k) {
+    const int rc = launch_expand(a[k], st);
+    if (rc != kOk) return rc;
+  }
+  return kOk;
+}
+
 int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h, const void* k, const void* v, int64_t sk_b,
                       int64_t sk_s, int64_t sk_h, const int32_t* q_pos0, const uint8_t* pad_mask, int64_t spm_b,
                       const float* add_mask, int64_t sam_b, int64_t sam_q, void* out, int64_t so_b, int64_t so_m, int64_t so_h,

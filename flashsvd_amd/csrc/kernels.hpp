@@ -133,6 +133,8 @@ struct PrefillAttnArgs {
 int launch_expand(const ExpandArgs& a, hipStream_t st);
 bool expand_tiles_apply(const ExpandArgs& a);                               // mfma_gemm.hip
 int launch_expand_tiles(const ExpandArgs& a, hipStream_t st);
+bool expand_multi_apply(const ExpandArgs* d, int n);                        // two or three expansions in one launch
+int launch_expand_multi(const ExpandArgs* d, int n, hipStream_t st);
 int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st);
 
 // matrix-core projections: y = epilogue(x . W^T) with the rounding points of the vector kernels

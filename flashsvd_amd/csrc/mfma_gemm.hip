@@ -42,7 +42,7 @@ struct ExpandEpi {
 // blocks, which halves the accumulators per wave (two waves per SIMD instead of one); the up halves cross to their
 // gate partners through LDS once, before the SwiGLU epilogue.
 template <bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
-__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi ep) {
+__device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandEpi& ep, const int tile_m, const int tile_n) {
   static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion takes whole 128-wide heads");
   static_assert(NW == 4 || (NW == 8 && DUAL && WT == 4 && WTM == 4), "eight waves are the split form of the 128 x 128 pair tile");
   constexpr int kGT = NW * 64;
@@ -65,17 +65,6 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   const int tid = threadIdx.x, wave = (tid >> 6) & 3, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
   const int mat = SPLIT ? (tid >> 8) : 0;  // split form: which matrix of the pair this wave accumulates
   const int wm = wave >> 1, wn = wave & 1;
-  // every XCD takes one contiguous run of tiles, ordered in bands of eight row tiles walked column by column, so that
-  // the workgroups resident on an XCD at one time share a few x tiles and a few W tiles in its L2
-  int tile_m, tile_n;
-  {
-    const int NT = gridDim.x, MT = gridDim.y;
-    const int t = xcd_run_index(blockIdx.y * NT + blockIdx.x, NT * MT);
-    const int band = t / (8 * NT), tb = t - band * 8 * NT;
-    const int bh = min(8, MT - band * 8);
-    tile_n = tb / bh;
-    tile_m = band * 8 + tb - tile_n * bh;
-  }
   const int m0 = tile_m * kGBM, n0 = tile_n * kGBN;
   // this workgroup's share of the K steps (all of them unless K is split over gridDim.z)
   const int ksteps_all = a.K / BK;
@@ -444,6 +433,35 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(Mf
   }
 }
 
+// every XCD takes one contiguous run of tiles, ordered in bands of eight row tiles walked column by column, so that
+// the workgroups resident on an XCD at one time share a few x tiles and a few W tiles in its L2
+__device__ __forceinline__ void tile_of_workgroup(int NT, int MT, int& tile_m, int& tile_n) {
+  const int t = xcd_run_index(blockIdx.y * NT + blockIdx.x, NT * MT);
+  const int band = t / (8 * NT), tb = t - band * 8 * NT;
+  const int bh = min(8, MT - band * 8);
+  tile_n = tb / bh;
+  tile_m = band * 8 + tb - tile_n * bh;
+}
+
+template <bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi ep) {
+  int tile_m, tile_n;
+  tile_of_workgroup(gridDim.x, gridDim.y, tile_m, tile_n);
+  gemm_tiles_body<DUAL, WTM, WT, PF, EXPAND, BK, NW>(a, ep, tile_m, tile_n);
+}
+
+// up to three head expansions of the same token rows (q, k, v of a prompt pass) in one launch: column tile = one head
+// of one of them.  At 512 rows a single expansion has one workgroup per compute unit and waits on its own loads; the
+// three together give every compute unit three.
+struct ExpandBatch { MfmaArgs a[3]; ExpandEpi ep[3]; int first_head[4]; };
+template <int WTM>
+__global__ __launch_bounds__(kGT4, 2) void expand_multi_kernel(ExpandBatch eb) {
+  int tile_m, tile_n;
+  tile_of_workgroup(gridDim.x, gridDim.y, tile_m, tile_n);
+  const int k = tile_n >= eb.first_head[2] ? 2 : (tile_n >= eb.first_head[1] ? 1 : 0);
+  gemm_tiles_body<false, WTM, 4, 2, true, kGBK, 4>(eb.a[k], eb.ep[k], tile_m, tile_n - eb.first_head[k]);
+}
+
 bool gemm_tiles_apply(const MfmaArgs& a) {
   return a.B >= 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0;
 }
@@ -570,6 +588,50 @@ static int launch_expand_tiles_t(const ExpandArgs& a, hipStream_t st) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
+}
+
+template <int WTM>
+static int launch_expand_multi_t(const ExpandArgs* d, int n, hipStream_t st) {
+  const char* who = "fsvd_lowrank_expand_heads_multi";
+  static bool granted = false;
+  constexpr int BM = 32 * WTM;
+  const size_t lds = (size_t)2 * (BM + 128) * kGBK * 2;
+  if (!granted) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&expand_multi_kernel<WTM>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
+    granted = true;
+  }
+  const int rows = d[0].B * d[0].M;
+  ExpandBatch eb{};
+  int heads = 0;
+  for (int k = 0; k < 3; ++k) {
+    const ExpandArgs& a = d[k < n ? k : n - 1];
+    eb.a[k] = MfmaArgs{a.p, 0, 0, a.u, nullptr, a.ldu, a.bias, nullptr, 0, a.y, 0, rows, a.heads * 128, a.R, 0};
+    eb.ep[k] = ExpandEpi{a.cos, a.sin, a.rope_len, a.positions, a.M, a.sp_b, a.sp_m, a.sy_b, a.sy_m, a.sy_h, a.dst_by_position, a.dst_rows};
+    eb.first_head[k] = heads;
+    if (k < n) heads += a.heads;
+  }
+  eb.first_head[3] = heads;
+  for (int k = n; k < 3; ++k) eb.first_head[k] = heads;    // unused sets start past the last head
+  const dim3 grid(heads, (rows + BM - 1) / BM);
+  hipLaunchKernelGGL(expand_multi_kernel<WTM>, grid, dim3(kGT4), lds, st, eb);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
+// the batched form applies when every expansion would take the tiled kernel and they cover the same token rows
+bool expand_multi_apply(const ExpandArgs* d, int n) {
+  if (n < 2 || n > 3) return false;
+  for (int k = 0; k < n; ++k)
+    if (!expand_tiles_apply(d[k]) || d[k].B != d[0].B || d[k].M != d[0].M) return false;
+  return true;
+}
+int launch_expand_multi(const ExpandArgs* d, int n, hipStream_t st) {
+  int heads = 0;
+  for (int k = 0; k < n; ++k) heads += d[k].heads;
+  const int64_t big = (int64_t)heads * (((int64_t)d[0].B * d[0].M + 127) / 128);
+  return big >= 384 ? launch_expand_multi_t<4>(d, n, st) : launch_expand_multi_t<2>(d, n, st);
 }
 
 int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {

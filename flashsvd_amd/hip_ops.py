@@ -358,14 +358,9 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, out: Optio
     return out
 
 
-def lowrank_expand_heads(p: torch.Tensor, u: torch.Tensor, *, num_heads: int, head_dim: int, out: torch.Tensor,
-                         cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
-                         positions: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
-                         dst_by_position: bool = False, head_stride: Optional[int] = None) -> torch.Tensor:
-    """out[b, row, h, :] = rope(p[b, m, (h), :] @ u[h*Dh:(h+1)*Dh].T + bias); see fsvd_lowrank_expand_heads.
-    p is [B, M, R] (shared by all heads) or [B, M, heads, R]; out is [B, rows, heads, Dh]."""
+def _expand_operands(p, u, heads, Dh, out, bias, head_stride):
+    """Checks of one head expansion; returns (B, M, R, coefficient strides)."""
     _need(p, "p"); _need(u, "u"); _need(out, "out")
-    heads, Dh = int(num_heads), int(head_dim)
     if p.dim() == 3:
         B, M, R = p.shape
         sp = (p.stride(0), p.stride(1), 0 if head_stride is None else int(head_stride))
@@ -382,26 +377,77 @@ def lowrank_expand_heads(p: torch.Tensor, u: torch.Tensor, *, num_heads: int, he
         raise ValueError(f"u must be [{heads * Dh}, {R}], got {tuple(u.shape)}")
     if out.dim() != 4 or out.shape[0] < B or out.shape[2] != heads or out.shape[3] != Dh:
         raise ValueError(f"out must be [B>={B}, rows, {heads}, {Dh}], got {tuple(out.shape)}")
-    rope_len = 0
-    if cos is not None:
-        _need(cos, "cos"); _need(sin, "sin")
-        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2 or not cos.is_contiguous() or not sin.is_contiguous():
-            raise ValueError(f"cos/sin must be contiguous [len, {Dh // 2}] tables")
-        rope_len = cos.shape[0]
-    if positions is not None:
-        _need(positions, "positions", dtype=torch.int32)
-        if positions.numel() != B:
-            raise ValueError(f"positions must be int32 [{B}]")
     if bias is not None:
         _need(bias, "bias")
         if bias.numel() != heads * Dh or not bias.is_contiguous():
             raise ValueError(f"bias must be contiguous [{heads * Dh}]")
+    return B, M, R, sp
+
+
+def _rope_tables(cos, sin, Dh):
+    if cos is None:
+        return 0
+    _need(cos, "cos"); _need(sin, "sin")
+    if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2 or not cos.is_contiguous() or not sin.is_contiguous():
+        raise ValueError(f"cos/sin must be contiguous [len, {Dh // 2}] tables")
+    return cos.shape[0]
+
+
+def lowrank_expand_heads(p: torch.Tensor, u: torch.Tensor, *, num_heads: int, head_dim: int, out: torch.Tensor,
+                         cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                         positions: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+                         dst_by_position: bool = False, head_stride: Optional[int] = None) -> torch.Tensor:
+    """out[b, row, h, :] = rope(p[b, m, (h), :] @ u[h*Dh:(h+1)*Dh].T + bias); see fsvd_lowrank_expand_heads.
+    p is [B, M, R] (shared by all heads) or [B, M, heads, R]; out is [B, rows, heads, Dh]."""
+    heads, Dh = int(num_heads), int(head_dim)
+    B, M, R, sp = _expand_operands(p, u, heads, Dh, out, bias, head_stride)
+    rope_len = _rope_tables(cos, sin, Dh)
+    if positions is not None:
+        _need(positions, "positions", dtype=torch.int32)
+        if positions.numel() != B:
+            raise ValueError(f"positions must be int32 [{B}]")
     lib = _lib.load()
     rc = lib.fsvd_lowrank_expand_heads(p.data_ptr(), sp[0], sp[1], sp[2], u.data_ptr(), u.stride(0), _ptr(bias), _ptr(cos), _ptr(sin),
                                        rope_len, _ptr(positions), out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
                                        int(bool(dst_by_position)), out.shape[1], B, M, heads, Dh, R, _stream())
     _lib.check("fsvd_lowrank_expand_heads", rc)
     return out
+
+
+def lowrank_expand_heads_multi(items, *, head_dim: int, cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                               positions: Optional[torch.Tensor] = None) -> None:
+    """The q / k / v expansions of one prompt pass in one call (fsvd_lowrank_expand_heads_multi): ``items`` is a list of one
+    to three dicts with the keyword arguments of :func:`lowrank_expand_heads` for one expansion (``p``, ``u``,
+    ``num_heads``, ``out``, optional ``bias``, ``dst_by_position``, ``head_stride``) plus ``rotate`` (apply cos / sin).
+    The same results as separate calls; a single launch when every expansion takes the tiled kernel."""
+    Dh = int(head_dim)
+    if not 1 <= len(items) <= 3:
+        raise ValueError(f"{len(items)} expansions (1..3)")
+    rope_len = _rope_tables(cos, sin, Dh)
+    descs = (_lib.ExpandDesc * len(items))()
+    shape = None
+    for d, it in zip(descs, items):
+        heads, out, bias = int(it["num_heads"]), it["out"], it.get("bias")
+        B, M, R, sp = _expand_operands(it["p"], it["u"], heads, Dh, out, bias, it.get("head_stride"))
+        if shape is None:
+            shape = (B, M)
+        elif shape != (B, M):
+            raise ValueError(f"expansions of one call cover the same token rows: {shape} vs {(B, M)}")
+        if it.get("rotate") and cos is None:
+            raise ValueError("rotate asked for without cos / sin")
+        d.p, d.sp_b, d.sp_m, d.sp_h = it["p"].data_ptr(), sp[0], sp[1], sp[2]
+        d.u, d.ldu, d.bias = it["u"].data_ptr(), it["u"].stride(0), _ptr(bias)
+        d.y, d.sy_b, d.sy_m, d.sy_h = out.data_ptr(), out.stride(0), out.stride(1), out.stride(2)
+        d.heads, d.R, d.rotate = heads, R, int(bool(it.get("rotate")))
+        d.dst_by_position, d.dst_rows, d.rsv0 = int(bool(it.get("dst_by_position"))), out.shape[1], 0
+    B, M = shape
+    if positions is not None:
+        _need(positions, "positions", dtype=torch.int32)
+        if positions.numel() != B:
+            raise ValueError(f"positions must be int32 [{B}]")
+    lib = _lib.load()
+    rc = lib.fsvd_lowrank_expand_heads_multi(descs, len(items), _ptr(cos), _ptr(sin), rope_len, _ptr(positions), B, M, Dh, _stream())
+    _lib.check("fsvd_lowrank_expand_heads_multi", rc)
 
 
 def attn_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, q_pos0: Optional[torch.Tensor] = None, causal: bool = True,

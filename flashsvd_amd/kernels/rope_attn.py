@@ -113,11 +113,11 @@ class FlashSVDRoPEAttention(nn.Module):
         q = torch.empty(B, M, H, dh, device=dev, dtype=dt)
         k = torch.empty(B, M, Hk, dh, device=dev, dtype=dt)
         v = torch.empty(B, M, Hk, dh, device=dev, dtype=dt)
-        hip_ops.lowrank_expand_heads(coeff(f.Pq), _as_linear_layout(f.Vq), num_heads=H, head_dim=dh, out=q, cos=cos, sin=sin,
-                                     positions=offs, bias=bias(f.bq, H))
-        hip_ops.lowrank_expand_heads(coeff(f.Pk), _as_linear_layout(f.Vk), num_heads=Hk, head_dim=dh, out=k, cos=cos, sin=sin,
-                                     positions=offs, bias=bias(f.bk, Hk))
-        hip_ops.lowrank_expand_heads(coeff(f.Pv), _as_linear_layout(f.Vv), num_heads=Hk, head_dim=dh, out=v, bias=bias(f.bv, Hk))
+        hip_ops.lowrank_expand_heads_multi(
+            [dict(p=coeff(f.Pq), u=_as_linear_layout(f.Vq), num_heads=H, out=q, rotate=True, bias=bias(f.bq, H)),
+             dict(p=coeff(f.Pk), u=_as_linear_layout(f.Vk), num_heads=Hk, out=k, rotate=True, bias=bias(f.bk, Hk)),
+             dict(p=coeff(f.Pv), u=_as_linear_layout(f.Vv), num_heads=Hk, out=v, bias=bias(f.bv, Hk))],
+            head_dim=dh, cos=cos, sin=sin, positions=offs)
 
         pad = add = None
         if attention_mask is not None:

@@ -413,12 +413,11 @@ class SVD_LlamaAttention(nn.Module):
             # cache rows start..start+T-1), then causal flash attention over the cache
             pos0 = torch.full((B,), start, device=x.device, dtype=torch.int32)
             q = torch.empty(B, T, H, Dh, device=x.device, dtype=x.dtype)
-            hip_ops.lowrank_expand_heads(p[..., :rq], wq, num_heads=H, head_dim=Dh, out=q,
-                                         cos=rope[0], sin=rope[1], positions=pos0)
-            hip_ops.lowrank_expand_heads(p[..., rq:rq + rk], wk, num_heads=Hk, head_dim=Dh, out=kc[:B],
-                                         cos=rope[0], sin=rope[1], positions=pos0, dst_by_position=True)
-            hip_ops.lowrank_expand_heads(p[..., rq + rk:], wv, num_heads=Hk, head_dim=Dh, out=vc[:B],
-                                         positions=pos0, dst_by_position=True)
+            hip_ops.lowrank_expand_heads_multi(
+                [dict(p=p[..., :rq], u=wq, num_heads=H, out=q, rotate=True),
+                 dict(p=p[..., rq:rq + rk], u=wk, num_heads=Hk, out=kc[:B], rotate=True, dst_by_position=True),
+                 dict(p=p[..., rq + rk:], u=wv, num_heads=Hk, out=vc[:B], dst_by_position=True)],
+                head_dim=Dh, cos=rope[0], sin=rope[1], positions=pos0)
             hip_ops.attn_prefill(q, kc[:B], vc[:B], q_pos0=pos0, causal=True, out=a.view(B, T, H, Dh))
         else:
             positions = torch.arange(start, start + T, device=x.device, dtype=torch.int32)

@@ -219,6 +219,22 @@ int fsvd_lowrank_expand_heads(const void* p, int64_t sp_b, int64_t sp_m, int64_t
                               const void* bias, const void* cos, const void* sin, int rope_len, const int32_t* positions,
                               void* y, int64_t sy_b, int64_t sy_m, int64_t sy_h, int dst_by_position, int dst_rows,
                               int B, int M, int heads, int Dh, int R, void* stream);
+/* The q, k and v expansions of one prompt pass in one call: the same results as `n` calls of
+ * fsvd_lowrank_expand_heads on the same token rows (one per descriptor; `rotate` selects whether that one gets the
+ * rotation), and a single launch when every one of them takes the tiled kernel (128 token rows and more, rank a
+ * multiple of 64, coefficients shared by the heads).  The reference computes all three inside one kernel as well
+ * (rope_sdpa.py:67-248 takes Pq/Vq, Pk/Vk, Pv/Vv together).  n = 1..3. */
+typedef struct fsvd_expand_desc {
+  const void* p; int64_t sp_b, sp_m, sp_h;   /* rank coefficients [B,M,(heads),R] */
+  const void* u; int64_t ldu;                /* [heads*Dh, R] */
+  const void* bias;                          /* [heads*Dh] or NULL */
+  void* y; int64_t sy_b, sy_m, sy_h;         /* destination [B, rows, heads, Dh] */
+  int32_t heads, R;
+  int32_t rotate;                            /* 1: rotate-half RoPE with the call's cos / sin */
+  int32_t dst_by_position, dst_rows, rsv0;
+} fsvd_expand_desc;
+int fsvd_lowrank_expand_heads_multi(const fsvd_expand_desc* desc, int n, const void* cos, const void* sin, int rope_len,
+                                    const int32_t* positions, int B, int M, int Dh, void* stream);
 int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
                       const void* k, const void* v, int64_t sk_b, int64_t sk_s, int64_t sk_h,
                       const int32_t* q_pos0, const uint8_t* pad_mask, int64_t spm_b,

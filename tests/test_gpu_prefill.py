@@ -145,6 +145,48 @@ def test_expand_long_prompts_tiled_kernel(B, M, R):
     assert_close_bf16(q, ref, "plain expansion with bias", **bounds(ref))
 
 
+@pytest.mark.parametrize("B,M,Rq,Rk,Rv", [(1, 512, 1024, 1024, 1024), (2, 130, 128, 64, 192), (2, 40, 64, 64, 64), (1, 256, 128, 72, 64)])
+def test_expand_multi_equals_separate_calls(B, M, Rq, Rk, Rv):
+    """q / k / v expansions in one call: bit-identical to three separate calls, whether the call becomes one launch
+    (128 rows and more, ranks multiples of 64) or falls back to one launch per expansion (short prompt, rank 72)."""
+    from flashsvd_amd import hip_ops
+    H, Hk, dh, start = 4, 2, 128, 5
+    S = start + M + 3
+    cos, sin = (t.cuda() for t in O.rope_tables(S, dh, dtype=BF16))
+    packed = rand_bf16(B, M, Rq + Rk + Rv, seed=1).cuda()        # the rank coefficients as the model holds them: one row
+    pq, pk, pv = packed[..., :Rq], packed[..., Rq:Rq + Rk], packed[..., Rq + Rk:]
+    uq, uk, uv = (rand_bf16(h * dh, r, std=r ** -0.5, seed=s).cuda() for h, r, s in ((H, Rq, 2), (Hk, Rk, 3), (Hk, Rv, 4)))
+    bq = rand_bf16(H * dh, std=0.1, seed=5).cuda()
+    pos0 = torch.tensor([start + b for b in range(B)], dtype=torch.int32, device="cuda")
+
+    def buffers():
+        return (torch.zeros(B, M, H, dh, dtype=BF16, device="cuda"), torch.zeros(B, S, Hk, dh, dtype=BF16, device="cuda"),
+                torch.zeros(B, S, Hk, dh, dtype=BF16, device="cuda"))
+
+    q1, k1, v1 = buffers()
+    hip_ops.lowrank_expand_heads(pq, uq, num_heads=H, head_dim=dh, out=q1, cos=cos, sin=sin, positions=pos0, bias=bq)
+    hip_ops.lowrank_expand_heads(pk, uk, num_heads=Hk, head_dim=dh, out=k1, cos=cos, sin=sin, positions=pos0, dst_by_position=True)
+    hip_ops.lowrank_expand_heads(pv, uv, num_heads=Hk, head_dim=dh, out=v1, positions=pos0, dst_by_position=True)
+    q2, k2, v2 = buffers()
+    hip_ops.lowrank_expand_heads_multi(
+        [dict(p=pq, u=uq, num_heads=H, out=q2, rotate=True, bias=bq),
+         dict(p=pk, u=uk, num_heads=Hk, out=k2, rotate=True, dst_by_position=True),
+         dict(p=pv, u=uv, num_heads=Hk, out=v2, dst_by_position=True)],
+        head_dim=dh, cos=cos, sin=sin, positions=pos0)
+    assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    ref = O.lin(pv.cpu(), uv.cpu()).reshape(B, M, Hk, dh)
+    for b in range(B):
+        assert_close_bf16(v2[b, start + b:start + b + M], ref[b], f"v rows of batch {b}", **bounds(ref[b]))
+    # two expansions, and token rows that do not match
+    k3, v3 = buffers()[1:]
+    hip_ops.lowrank_expand_heads_multi([dict(p=pk, u=uk, num_heads=Hk, out=k3, rotate=True, dst_by_position=True),
+                                        dict(p=pv, u=uv, num_heads=Hk, out=v3, dst_by_position=True)],
+                                       head_dim=dh, cos=cos, sin=sin, positions=pos0)
+    assert torch.equal(k1, k3) and torch.equal(v1, v3)
+    with pytest.raises(ValueError, match="same token rows"):
+        hip_ops.lowrank_expand_heads_multi([dict(p=pk, u=uk, num_heads=Hk, out=k3), dict(p=pv[:, :M - 1], u=uv, num_heads=Hk, out=v3)], head_dim=dh)
+
+
 def test_model_prefill_mfma_equals_decode_route():
     mw = O.make_model(d=512, n_heads=4, n_kv_heads=2, head_dim=128, ffn=1024, attn_rank=96, mlp_rank=128, n_layers=2,
                       vocab=300, dtype=BF16, seed=7, std=0.05)
