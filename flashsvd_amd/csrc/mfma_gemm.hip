@@ -44,9 +44,13 @@ struct ExpandEpi {
 template <bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
 __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandEpi& ep, const int tile_m, const int tile_n) {
   static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion takes whole 128-wide heads");
-  static_assert(NW == 4 || (NW == 8 && DUAL && WT == 4 && WTM == 4), "eight waves are the split form of the 128 x 128 pair tile");
+  static_assert(NW == 4 || (NW == 8 && DUAL && WT == 4 && WTM == 4) || (NW == 8 && !DUAL && !EXPAND && BK >= 64),
+                "eight waves: the split form of the 128 x 128 pair tile, or two halves of every K step of a single matrix");
   constexpr int kGT = NW * 64;
-  constexpr bool SPLIT = NW == 8;
+  constexpr bool SPLIT = NW == 8 && DUAL;
+  // single matrix, eight waves: waves 4-7 take the second half of the k slices of every step and hand their sums to
+  // waves 0-3 at the end (a tile that has a compute unit to itself then still runs two waves per SIMD)
+  constexpr bool KHALF = NW == 8 && !DUAL;
   constexpr bool DTL = PF < 0;            // global loads write the LDS stages themselves (no register sets), -PF stages
   constexpr int PFR = DTL ? 1 : PF;
   constexpr int NS = DTL ? -PF : 2;       // LDS stages
@@ -63,7 +67,7 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
   constexpr int kTileX = kGBM * kGLd, kTileW = kGBN * kGLd;   // elements per operand tile
   constexpr int kStage = NM * (kTileX + kTileW);
   const int tid = threadIdx.x, wave = (tid >> 6) & 3, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
-  const int mat = SPLIT ? (tid >> 8) : 0;  // split form: which matrix of the pair this wave accumulates
+  const int mat = NW == 8 ? (tid >> 8) : 0;   // eight waves: which matrix of the pair / which half of the k slices
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = tile_m * kGBM, n0 = tile_n * kGBN;
   // this workgroup's share of the K steps (all of them unless K is split over gridDim.z)
@@ -181,10 +185,10 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
       // while block q multiplies, and the last block, which has nothing left to read, carries the LDS writes of the
       // next stage and the global loads that refill their registers: the other stage was last read before the
       // barrier that ended step ks - 1, and past the last step both are harmless (clamped addresses, a dead stage).
-      constexpr int Q = (BK / 32) * NMA;
+      constexpr int Q = KHALF ? BK / 64 : (BK / 32) * NMA;
       gm_bf16x8_t fx[2][WTM], fw[2][WT];
       const auto load_frags = [&](int q, int set) {
-        const int kk = q / NMA, m = SPLIT ? mat : q % NMA;
+        const int kk = KHALF ? mat * (BK / 64) + q : q / NMA, m = SPLIT ? mat : (KHALF ? 0 : q % NMA);
         const int fcol = (((kk * 4) ^ fr_hi) + fr_lo) * 8;
 #pragma unroll
         for (int i = 0; i < WTM; ++i)
@@ -234,6 +238,24 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
     }
   }
 
+  if (KHALF) {
+    gm_f32x4_t* ex = reinterpret_cast<gm_f32x4_t*>(gm_smem);     // [WTM*WT][256] 16-byte words, inside the stages
+    __syncthreads();                                             // every wave has finished reading the last stage
+    if (mat == 1) {
+#pragma unroll
+      for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) ex[(i * WT + j) * 256 + (tid & 255)] = acc[0][i][j];
+    }
+    __syncthreads();
+    if (mat == 0) {
+#pragma unroll
+      for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) acc[0][i][j] += ex[(i * WT + j) * 256 + (tid & 255)];
+    }
+  }
+  const bool writer = !KHALF || mat == 0;   // waves 4-7 of the halved form keep the barriers below company and store nothing
   // K split: park the partial tile (thread-major 16-byte words, coalesced), count arrivals; the last workgroup of a
   // tile adds all partials in split order (its own included, so the sum does not depend on who came last)
   if (WTM <= 2 && gridDim.z > 1) {         // only the 32- and 64-row tiles are ever launched with a split
@@ -250,6 +272,7 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
       for (int i = 0; i < WTM; ++i)
 #pragma unroll
         for (int j = 0; j < WT; ++j) {
+          if (!writer) break;
           const gm_f32x4_t v = kdead ? gm_f32x4_t{0.f, 0.f, 0.f, 0.f} : acc[m][i][j];
           unsigned long long* dst = reinterpret_cast<unsigned long long*>(mine + ((m * WTM + i) * WT + j) * kGT + tid);
           __hip_atomic_store(dst, ((unsigned long long)__float_as_uint(v[1]) << 32) | __float_as_uint(v[0]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -265,7 +288,7 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
       *flag = last;
     }
     __syncthreads();
-    if (*flag == 0) return;
+    if (*flag == 0 || !writer) return;
     // the shares are added in split order; the loads of several shares are in flight at once (each comes from beyond
     // this XCD's L2, and one share per round trip made the reduction the longest part of a narrow projection)
     constexpr int ZC = WPT <= 2 ? 8 : (WPT <= 4 ? 4 : 2);
@@ -303,6 +326,7 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
       }
     }
   }
+  if (!writer) return;
   // split pair: the up accumulators travel to the gate wave of the same block (same lane, same tile indices)
   gm_f32x4_t upv[SPLIT ? WT : 1][SPLIT ? WT : 1];
   if (SPLIT) {
@@ -539,7 +563,14 @@ int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* 
   // weights that come from HBM, and slower than it below these tile counts)
   if (big >= 448) return launch_gemm_tiles_t<false, 4, 4, 64, 4, -2>(a, st, who);
   if (big >= 320) return launch_gemm_tiles_t<false, 4, 2, 64, 4, -2>(a, st, who);
+  // about one tile per compute unit: eight waves on a 128 x 128 or 128 x 64 tile, each half of them on half of the k
+  // slices of a step, so that a workgroup alone on its compute unit still runs two waves per SIMD (rank projections at
+  // 512 rows 36 -> 29 us, at 1024 rows 50 -> 43; down_v at 2048 rows 131 -> 109; with fewer tiles than ~0.6 per
+  // compute unit the 64 x 64 tiles below win, with more the four-wave forms that share a compute unit)
+  if (big >= 144 && big <= 256) return launch_gemm_tiles_t<false, 4, 4, 64, 8>(a, st, who);
   if (big >= 256) return launch_gemm_tiles_t<false, 4, 2, 64>(a, st, who);
+  const int64_t half = (int64_t)((a.N + 63) / 64) * ((a.B + 127) / 128);
+  if (half >= 160 && half <= 256 && (a.K % 128) == 0) return launch_gemm_tiles_t<false, 4, 2, 128, 8>(a, st, who);
   const int64_t small = (int64_t)((a.N + 63) / 64) * ((a.B + 63) / 64);
   return (small < 320 && (a.K % 128) == 0) ? launch_gemm_tiles_t<false, 2, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 2, 2, 64>(a, st, who);
 }
