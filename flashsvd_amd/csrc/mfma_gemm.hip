@@ -1,15 +1,17 @@
 // Prefill projections: y[M, N] = epilogue(x[M, K] . W[N, K]^T) for 128 rows and more, on the matrix cores.
 //
 // Both operands are K-contiguous, which is the layout V_MFMA_F32_16X16X32_BF16 wants for its two inputs (each lane
-// holds 8 consecutive k of one row).  A workgroup of four waves owns a 128 x 128 output tile (a wave 64 x 64: 4 x 4
-// accumulator tiles) — or 64 x 64 when the problem has too few big tiles to give every compute unit work — and walks K
-// in steps of 64 or 128 through a double-buffered LDS stage (the 16-byte pieces of a row swizzled so that the fragment
-// reads of 16 consecutive rows fall on different banks).  Two ways to fill a stage: global loads that run two to four
-// steps ahead in registers and are written to the idle stage one step before their products (few workgroups per compute
+// holds 8 consecutive k of one row).  A workgroup of four or eight waves owns a 128 x 128, 128 x 64 or 64 x 64 output
+// tile (32 x 64 below 128 rows) — the launcher picks by how many tiles the problem has for 256 compute units — and walks
+// K in steps of 32, 64 or 128 through two LDS stages (the 16-byte pieces of a row swizzled so that the fragment reads of
+// 16 consecutive rows fall on different banks).  Two ways to fill a stage: global loads that run two to four steps
+// ahead in registers and are written to the idle stage one step before their products (few workgroups per compute
 // unit, long K: latency-bound), or loads that write LDS themselves one step ahead (no staging registers, no LDS write
-// instructions; pays when two or three workgroups share a compute unit).  Epilogue as in the vector kernels: bias, ONE rounding to bf16,
-// residual — or, for the gate / up pair, SwiGLU in either rounding mode — or the head expansion of the prompt pass
-// (RoPE, store into the query buffer or the cache rows).  Every weight is read once per 128 (64) rows of x.
+// instructions; pays when two or three workgroups share a compute unit).  The products are W . x^T, so a lane of the
+// accumulator owns four consecutive output columns of one row (8-byte epilogue accesses).  Epilogue as in the vector
+// kernels: bias, ONE rounding to bf16, residual — or, for the gate / up pair, SwiGLU in either rounding mode — or the
+// head expansion of the prompt pass (RoPE, store into the query buffer or the cache rows).  Few tiles or a very long K:
+// K split over workgroups, partial tiles added in a fixed order by the last arrival.
 #include <algorithm>
 
 #include "common.hpp"
@@ -37,10 +39,12 @@ struct ExpandEpi {
   int dst_by_position, dst_rows;
 };
 
-// NW: waves per workgroup.  4: a wave owns a 16 WT x 16 WT block of the output tile (both matrices of the gate / up
-// pair).  8 (pair, 128 x 128 only): waves 0-3 accumulate the gate matrix and waves 4-7 the up matrix of the same
+// NW: waves per workgroup.  4: a wave owns a 16 WTM x 16 WT block of the output tile (both matrices of the gate / up
+// pair).  8, pair (128 x 128 only): waves 0-3 accumulate the gate matrix and waves 4-7 the up matrix of the same
 // blocks, which halves the accumulators per wave (two waves per SIMD instead of one); the up halves cross to their
-// gate partners through LDS once, before the SwiGLU epilogue.
+// gate partners through LDS once, before the SwiGLU epilogue.  8, single matrix: waves 4-7 take the second half of the
+// k slices of every step and hand their sums to waves 0-3 through LDS at the end.
+// PF > 0: register sets in flight; PF < 0: loads straight into LDS with -PF stages.
 template <bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
 __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandEpi& ep, const int tile_m, const int tile_n) {
   static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion takes whole 128-wide heads");
@@ -328,20 +332,20 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
   }
   if (!writer) return;
   // split pair: the up accumulators travel to the gate wave of the same block (same lane, same tile indices)
-  gm_f32x4_t upv[SPLIT ? WT : 1][SPLIT ? WT : 1];
+  gm_f32x4_t upv[SPLIT ? WTM : 1][SPLIT ? WT : 1];
   if (SPLIT) {
-    gm_f32x4_t* ex = reinterpret_cast<gm_f32x4_t*>(gm_smem);     // [WT*WT][256] 16-byte words = 64 KB of the stages
+    gm_f32x4_t* ex = reinterpret_cast<gm_f32x4_t*>(gm_smem);     // [WTM*WT][256] 16-byte words, at most half of the stages
     __syncthreads();                                             // every wave has finished reading the last stage
     if (mat == 1) {
 #pragma unroll
-      for (int i = 0; i < WT; ++i)
+      for (int i = 0; i < WTM; ++i)
 #pragma unroll
         for (int j = 0; j < WT; ++j) ex[(i * WT + j) * 256 + (tid & 255)] = acc[0][i][j];
     }
     __syncthreads();
     if (mat == 1) return;
 #pragma unroll
-    for (int i = 0; i < WT; ++i)
+    for (int i = 0; i < WTM; ++i)
 #pragma unroll
       for (int j = 0; j < WT; ++j) upv[i][j] = ex[(i * WT + j) * 256 + (tid & 255)];
   }
