@@ -561,7 +561,12 @@ int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* 
   // The pair at four big tiles per compute unit and more: four waves with both accumulator sets, K steps of 32
   // loaded straight into LDS (two workgroups per compute unit; 243 -> 214 us at 2048 rows of the 7B MLP)
   if (dual && big >= 1024) return launch_gemm_tiles_t<true, 4, 4, 32, 4, -2>(a, st, who);
-  if (dual) return big >= 512 ? launch_gemm_tiles_t<true, 4, 4, 64, 8>(a, st, who) : launch_gemm_tiles_t<true, 2, 2, 64>(a, st, who);
+  if (dual && big >= 512) return launch_gemm_tiles_t<true, 4, 4, 64, 8>(a, st, who);
+  // two and a half to four 64 x 128 tiles per compute unit: that tile, K steps of 32 straight into LDS, three
+  // workgroups per compute unit (7B MLP at 512 rows 83 -> 77 us, at 768 rows 114 -> 110; slower outside this range)
+  const int64_t wide = (int64_t)((a.N + 127) / 128) * ((a.B + 63) / 64);
+  if (dual && wide >= 640 && wide <= 1100) return launch_gemm_tiles_t<true, 2, 4, 32, 4, -2>(a, st, who);
+  if (dual) return launch_gemm_tiles_t<true, 2, 2, 64>(a, st, who);
   // a single matrix with more than one big tile per compute unit: loads straight into LDS, two stages (the second and
   // third workgroup of a compute unit cover the one-step load distance; 5..8 % faster than the register pipeline with
   // weights that come from HBM, and slower than it below these tile counts)
