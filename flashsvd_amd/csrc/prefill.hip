@@ -256,15 +256,22 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
 //     16 (e / 4) + 4 lg + e % 4, so V^T is stored with key offset ko at column 8 (ko % 16 / 4) + 4 (ko / 16) + ko % 4.
 //     P is a bf16 high part plus a bf16 residual (two products per fragment) so that it carries ~16 mantissa bits.
 // ---------------------------------------------------------------------------------------------
-template <int MI>
-__global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(PrefillAttnArgs a) {
+// NG = 2: eight waves; waves 4-7 are a second group with K / V tiles of its own that takes every other key tile, and the
+// two groups' running statistics and outputs are merged through LDS at the end — for prompts whose (query tile, head)
+// pairs number no more than the compute units, where a workgroup alone on its compute unit walks its key tiles with
+// one wave per SIMD and waits out every load and barrier.
+template <int MI, int NG>
+__global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill_wide_kernel(PrefillAttnArgs a) {
   constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, VSTR = BN;
   // K rows of 288 bytes: a 16-byte LDS read is served 16 lanes a cycle (lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of a
   // half wave); rows 16 r apart with r odd multiples of 32 bytes give those lanes 16 different bank groups
   constexpr int KSTR = DH + 16;
   extern __shared__ __align__(16) unsigned char pw_smem[];
-  uint16_t (*Ks)[KSTR] = reinterpret_cast<uint16_t (*)[KSTR]>(pw_smem);                              // [BN][KSTR]
-  uint16_t (*Vt)[VSTR] = reinterpret_cast<uint16_t (*)[VSTR]>(pw_smem + (size_t)BN * KSTR * 2);       // [DH][VSTR]
+  constexpr int kGroupBytes = BN * KSTR * 2 + DH * VSTR * 2;
+  const int grp = NG == 1 ? 0 : (int)(threadIdx.x >> 8);
+  unsigned char* gsm = pw_smem + (size_t)grp * kGroupBytes;
+  uint16_t (*Ks)[KSTR] = reinterpret_cast<uint16_t (*)[KSTR]>(gsm);                                   // [BN][KSTR]
+  uint16_t (*Vt)[VSTR] = reinterpret_cast<uint16_t (*)[VSTR]>(gsm + (size_t)BN * KSTR * 2);            // [DH][VSTR]
 
   // the query tiles of a head (and the heads of a kv head) run on one XCD, so its K and V come out of one L2; under
   // a causal mask the last tiles, which see the most keys, start first
@@ -272,7 +279,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
   const int t = xcd_run_index(blockIdx.x + MT * (blockIdx.y + gridDim.y * blockIdx.z), MT * gridDim.y * gridDim.z);
   const int mt = a.causal ? MT - 1 - t % MT : t % MT, h = (t / MT) % (int)gridDim.y, b = t / (MT * (int)gridDim.y);
   const int hk = h / (a.H / a.Hk);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;   // thread and wave within the group
   const int lr = lane & 15, lg = lane >> 4;
   const int q0 = a.q_pos0 ? a.q_pos0[b] : 0;
   const int m_base = mt * BM + wave * QW;
@@ -317,10 +324,13 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
       vreg[j] = *reinterpret_cast<const u32x4_t*>(vb + (int64_t)vkey * a.sk_s + d0);
     }
   };
-  if (k_end > 0) request(0);
+  if (grp * BN < k_end) request(grp * BN);
 
-  for (int n0 = 0; n0 < k_end; n0 += BN) {
+  for (int n00 = 0; n00 < k_end; n00 += NG * BN) {
+    const int n0 = n00 + grp * BN;
+    const bool live = n0 < k_end;       // the second group may have no tile in the last round; it still meets the barriers
     __syncthreads();   // the previous tile's Ks / Vt are consumed
+    if (live) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(&Ks[srow + 16 * j][d0]) = kreg[j];
     {
@@ -339,9 +349,10 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
         *reinterpret_cast<u32x2_t*>(&Vt[d0 + 2 * c + 1][col]) = hi;
       }
     }
+    }
     __syncthreads();   // tile visible
-    if (n0 + BN < k_end) request(n0 + BN);
-    if (n0 >= wave_end) continue;   // nothing this wave's rows may see (wave-uniform)
+    if (n0 + NG * BN < k_end) request(n0 + NG * BN);
+    if (!live || n0 >= wave_end) continue;   // nothing this wave's rows may see (wave-uniform)
 
     // ---- S^T = K Q^T for 64 keys x 16 MI queries: block j, element i = key n0 + 16 j + 4 lg + i, query column lr
     f32x4_t sacc[MI][4];
@@ -431,6 +442,31 @@ __global__ __launch_bounds__(kPfThreads, 2) void attn_prefill_wide_kernel(Prefil
     }
   }
 
+  if (NG == 2) {
+    // merge the two groups: (m, l, O) of group 1 through LDS (word-major, one 16-byte word per lane and slot)
+    f32x4_t* mb = reinterpret_cast<f32x4_t*>(pw_smem);
+    __syncthreads();                   // both groups are done with their K / V tiles
+    if (grp == 1) {
+#pragma unroll
+      for (int mi = 0; mi < MI; ++mi) {
+        mb[(mi * 9) * 256 + tid] = f32x4_t{m_run[mi], l_run[mi], 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) mb[(mi * 9 + 1 + t) * 256 + tid] = o[mi][t];
+      }
+    }
+    __syncthreads();
+    if (grp == 1) return;
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+      const f32x4_t st = mb[(mi * 9) * 256 + tid];
+      const float m1 = st[0], l1 = st[1];
+      const float m = fmaxf(m_run[mi], m1);
+      const float a0 = m_run[mi] == -INFINITY ? 0.f : __expf(m_run[mi] - m), a1 = m1 == -INFINITY ? 0.f : __expf(m1 - m);
+      l_run[mi] = l_run[mi] * a0 + l1 * a1;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) o[mi][t] = o[mi][t] * a0 + mb[(mi * 9 + 1 + t) * 256 + tid] * a1;
+    }
+  }
   // ---- normalise and store (four consecutive dimensions per lane and tile); rows with no visible key give 0
 #pragma unroll
   for (int mi = 0; mi < MI; ++mi) {
@@ -481,8 +517,18 @@ int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
     // 128 query rows per workgroup when that gives every compute unit work, else 64 (half the rows per wave)
     const bool wide = (int64_t)((a.M + 127) / 128) * a.H * a.B >= 384;
     const size_t lds = (size_t)64 * 144 * 2 + (size_t)128 * 64 * 2;
-    if (wide) hipLaunchKernelGGL(attn_prefill_wide_kernel<2>, dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
-    else hipLaunchKernelGGL(attn_prefill_wide_kernel<1>, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), lds, st, a);
+    // no more 64-row workgroups than ~1.25 per compute unit: two groups of waves share the key tiles of each
+    const bool pair = !wide && (int64_t)((a.M + 63) / 64) * a.H * a.B <= 320;
+    if (pair) {
+      static bool granted = false;
+      if (!granted) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * lds));
+        if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", fn, 2 * lds, hipGetErrorString(e)); return kErrLaunch; }
+        granted = true;
+      }
+      hipLaunchKernelGGL((attn_prefill_wide_kernel<1, 2>), dim3((a.M + 63) / 64, a.H, a.B), dim3(2 * kPfThreads), 2 * lds, st, a);
+    } else if (wide) hipLaunchKernelGGL((attn_prefill_wide_kernel<2, 1>), dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
+    else hipLaunchKernelGGL((attn_prefill_wide_kernel<1, 1>), dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), lds, st, a);
   } else {
     hipLaunchKernelGGL(attn_prefill_kernel, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), 0, st, a);
   }
