@@ -100,16 +100,20 @@ def test_expand_and_prefill_attention_primitives():
         assert_close_bf16(out[:, m], refm, f"row {m}", **bounds(refm))
 
 
-def test_prefill_attention_128_row_tiles():
-    """Enough (row tile, head, batch) triples for the 128-row form of the prompt attention (two 16-row blocks per wave);
-    grouped heads, a prefix already in the cache, a ragged last tile."""
+@pytest.mark.parametrize("B,M", [(3, 520), (2, 500), (1, 300)])
+def test_prefill_attention_row_tile_forms(B, M):
+    """The three forms of the LDS-shared prompt attention: 128 query rows per workgroup (B = 3: enough row tile / head /
+    batch triples), 64 rows with four waves (B = 2), 64 rows with a second group of waves on every other key tile (B = 1:
+    no more workgroups than compute units); grouped heads, a prefix already in the cache, a ragged last tile."""
     from flashsvd_amd import hip_ops
-    B, M, H, Hk, dh, S, start = 3, 520, 32, 8, 128, 560, 29
+    H, Hk, dh, S, start = 32, 8, 128, 560, 29
     kfull, vfull = rand_bf16(B, S, Hk, dh, seed=31), rand_bf16(B, S, Hk, dh, seed=32)
     q = rand_bf16(B, M, H, dh, seed=33)
     pos0 = torch.full((B,), start, dtype=torch.int32, device="cuda")
     out = hip_ops.attn_prefill(q.cuda(), kfull.cuda(), vfull.cuda(), q_pos0=pos0, causal=True)
-    for m in (0, 15, 16, 127, 128, 300, 511, 512, M - 1):
+    for m in (0, 15, 16, 63, 64, 127, 128, 299, 300, 511, 512, M - 1):
+        if m >= M:
+            continue
         n = start + m + 1
         refm = O.dense_decode_attn(q[:, m], kfull[:, :n], vfull[:, :n])
         assert_close_bf16(out[:, m], refm, f"row {m}", **bounds(refm))
