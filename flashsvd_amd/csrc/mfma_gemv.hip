@@ -28,6 +28,50 @@ __device__ __forceinline__ bf16x8_t ldx_frag(const uint16_t* p) {
 }
 
 
+// the waves' partial tiles through LDS, added in wave order, then the epilogue of the vector kernels
+template <int NB, bool DUAL, int KS>
+__device__ __forceinline__ void mfma_finish(const MfmaArgs& a, float (*red)[DUAL ? 2 : 1][NB][4][64], const f32x4_t (&acc)[DUAL ? 2 : 1][NB]) {
+  constexpr int NM = DUAL ? 2 : 1;
+  constexpr int RT = kMfWaves / KS;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+#pragma unroll
+  for (int m = 0; m < NM; ++m)
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][m][t][i][lane] = acc[m][t][i];
+  __syncthreads();
+  // one thread per output element of the RT tiles of 16 x (16 * NB): element i of lane l is row
+  // (l / 16) * 4 + i, batch column l % 16; the KS partial tiles are added in wave order
+  for (int o = tid; o < RT * NB * 256; o += kMfThreads) {
+    const int q = o / (NB * 256), oo = o - q * (NB * 256);
+    const int t = oo >> 8, r = oo & 255, i = r >> 6, l = r & 63;
+    const int n = (blockIdx.x * RT + q) * 16 + (l >> 4) * 4 + i, b = t * 16 + (l & 15);
+    float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+    for (int w = 0; w < KS; ++w) {
+      v0 += red[q * KS + w][0][t][i][l];
+      if (DUAL) v1 += red[q * KS + w][NM - 1][t][i][l];
+    }
+    if (n >= a.N || b >= a.B) continue;
+    float v;
+    if (DUAL) {
+      if (a.mode == 0) {
+        v0 = round_bf16(v0);
+        v1 = round_bf16(v1);
+        v = round_bf16(round_bf16(silu_f32(v0)) * v1);
+      } else {
+        v = round_bf16((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
+      }
+    } else {
+      if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
+      v = round_bf16(v0);
+      if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)b * a.ldres + n]) + v);
+    }
+    a.y[(int64_t)b * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+  }
+}
+
 // NB: 16-row batch tiles (B <= 16 * NB); KS: waves that split K for one 16-row weight tile, so a workgroup
 // of 8 waves covers 8 / KS weight tiles
 template <int NB, bool DUAL, int KS>
@@ -81,42 +125,105 @@ __global__ __launch_bounds__(kMfThreads) void mfma_linear_kernel(MfmaArgs a) {
       }
     }
   }
+  mfma_finish<NB, DUAL, KS>(a, red, acc);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Up to 16 rows: the same decomposition (a wave = 16 weight rows x a share of K, partial tiles added in wave order), but
+// the weights arrive the way the batch-1 kernels read them: whole 128- or 256-byte pieces of a row, loaded straight into
+// a ring of LDS stages that belongs to the wave (no barrier in the loop, only the wave's own load counter), and the
+// matrix-core fragments are read from there.  The fragment loads of the kernel above touch 16 rows x 64 bytes per
+// instruction; timing that kernel with 1 KB-contiguous loads of the same volume (wrong results, same traffic) showed the
+// access pattern to cost a third of its time.  LDS position p of a row holds piece p ^ (row % pieces): conflict-free
+// 16-byte fragment reads (see mfma_gemm.hip).
+// ---------------------------------------------------------------------------------------------
+template <bool DUAL> struct StreamShape {
+  static constexpr int CKB = DUAL ? 128 : 256;     // bytes of a weight row per chunk
+  static constexpr int NM = DUAL ? 2 : 1;
+  static constexpr int kStage = NM * 16 * CKB;     // 4 KB either way
+};
+
+// D: chunks in a wave's ring (D - 1 in flight while one multiplies)
+template <bool DUAL, int KS, int D>
+__global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
+  typedef StreamShape<DUAL> SS;
+  constexpr int NB = 1, NM = SS::NM, CKB = SS::CKB, kStage = SS::kStage;
+  constexpr int RT = kMfWaves / KS;
+  constexpr int PPR = CKB / 16;                    // 16-byte pieces per row and chunk
+  constexpr int KST = CKB / 64;                    // k-steps of 32 per chunk
+  constexpr int RPI = 64 / PPR;                    // rows one load instruction covers (64 lanes x 16 bytes)
+  constexpr int NI = 16 / RPI;                     // load instructions per matrix and chunk
+  constexpr int kGroup = NM * NI + NM * KST;       // loads per chunk: weight pieces into LDS, activation fragments into registers
+  static_assert((D - 1) * kGroup < 64 && D >= 2 && D <= 4, "vmcnt holds six bits; the waits below cover up to three groups in flight");
+  extern __shared__ __align__(16) unsigned char st_smem[];     // [8 waves][D][kStage]; the partial tiles at the end
+  float (*red)[NM][NB][4][64] = reinterpret_cast<float (*)[NM][NB][4][64]>(st_smem);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
+  const int rt = wave / KS, ks = wave % KS;
+  const int n0 = (blockIdx.x * RT + rt) * 16;
+  unsigned char* ring = st_smem + (size_t)wave * D * kStage;
+  const int nchunk = a.K / (CKB / 2);
+  const int cw = (nchunk - ks + KS - 1) / KS;      // this wave's chunks: ks, ks + KS, ... (the KS waves of a tile read adjacent pieces)
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  const int lrow = lane / PPR, lpc = lane % PPR;
+  const uint16_t* wsrc[NM][NI];
 #pragma unroll
-  for (int m = 0; m < NM; ++m)
-#pragma unroll
-    for (int t = 0; t < NB; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) red[wave][m][t][i][lane] = acc[m][t][i];
-  __syncthreads();
-  // one thread per output element of the RT tiles of 16 x (16 * NB): element i of lane l is row
-  // (l / 16) * 4 + i, batch column l % 16; the KS partial tiles are added in wave order
-  for (int o = tid; o < RT * NB * 256; o += kMfThreads) {
-    const int q = o / (NB * 256), oo = o - q * (NB * 256);
-    const int t = oo >> 8, r = oo & 255, i = r >> 6, l = r & 63;
-    const int n = (blockIdx.x * RT + q) * 16 + (l >> 4) * 4 + i, b = t * 16 + (l & 15);
-    float v0 = 0.f, v1 = 0.f;
-#pragma unroll
-    for (int w = 0; w < KS; ++w) {
-      v0 += red[q * KS + w][0][t][i][l];
-      if (DUAL) v1 += red[q * KS + w][NM - 1][t][i][l];
-    }
-    if (n >= a.N || b >= a.B) continue;
-    float v;
-    if (DUAL) {
-      if (a.mode == 0) {
-        v0 = round_bf16(v0);
-        v1 = round_bf16(v1);
-        v = round_bf16(round_bf16(silu_f32(v0)) * v1);
-      } else {
-        v = round_bf16((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
-      }
-    } else {
-      if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
-      v = round_bf16(v0);
-      if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)b * a.ldres + n]) + v);
-    }
-    a.y[(int64_t)b * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+  for (int q = 0; q < NI; ++q) {
+    const int row = q * RPI + lrow;
+    const int64_t off = (int64_t)min(n0 + row, a.N - 1) * a.ldw + ((lpc ^ (row % PPR)) * 8);
+    wsrc[0][q] = a.W + off;
+    if (DUAL) wsrc[NM - 1][q] = a.W2 + off;
   }
+  const uint16_t* xsrc = a.x + (int64_t)min(lr, a.B - 1) * a.ldx + lg * 8;
+  bf16x8_t xf[D][NM][KST];
+  // The wave's load counter is the only synchronisation: it counts weight pieces and activation fragments alike, in
+  // issue order, so the loads of one chunk must stay together in the instruction stream (scheduling fences around them).
+  const auto issue = [&](int c, int slot) {
+    const int k0 = (c * KS + ks) * (CKB / 2);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+#pragma unroll
+      for (int q = 0; q < NI; ++q)
+        __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[m][q] + k0), (lptr_t)(ring + slot * kStage + m * 16 * CKB + q * 1024), 16, 0, 0);
+#pragma unroll
+      for (int s = 0; s < KST; ++s) xf[slot][m][s] = ldx_frag(xsrc + (m ? a.up_off : 0) + k0 + s * 32);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  f32x4_t acc[NM][NB];
+#pragma unroll
+  for (int m = 0; m < NM; ++m) acc[m][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  // load counter values that leave the newest r groups in flight
+  constexpr int kW0 = (7 << 4) | (15 << 8);
+  const auto vm = [](int n) { return (n & 15) | ((n >> 4) << 14); };
+#pragma unroll
+  for (int c = 0; c < D - 1; ++c)
+    if (c < cw) issue(c, c);
+  for (int c0 = 0; c0 < cw; c0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int c = c0 + u;
+      if (c >= cw) break;
+      if (c + D - 1 < cw) issue(c + D - 1, (u + D - 1) % D);
+      // chunk c has landed once no more than the groups issued after it are outstanding
+      const int newer = min(D - 1, cw - 1 - c);
+      if (newer >= 3) __builtin_amdgcn_s_waitcnt(kW0 | vm(3 * kGroup));
+      else if (newer == 2) __builtin_amdgcn_s_waitcnt(kW0 | vm(2 * kGroup));
+      else if (newer == 1) __builtin_amdgcn_s_waitcnt(kW0 | vm(kGroup));
+      else __builtin_amdgcn_s_waitcnt(kW0 | vm(0));
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < KST; ++s)
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+          const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(ring + u * kStage + m * 16 * CKB + lr * CKB + (((s * 4 + lg) ^ (lr % PPR)) * 16));
+          acc[m][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[u][m][s], acc[m][0], 0, 0, 0);
+        }
+    }
+  }
+  __syncthreads();                                 // every wave is done with its ring: the partial tiles take its place
+  mfma_finish<NB, DUAL, KS>(a, red, acc);
 }
 
 template <int NB, bool DUAL>
@@ -126,6 +233,47 @@ static void launch_mfma_ks(const MfmaArgs& a, int ks, hipStream_t st) {
   if (ks == 2) hipLaunchKernelGGL((mfma_linear_kernel<NB, DUAL, 2>), dim3((tiles + 3) / 4), block, 0, st, a);
   else if (ks == 4) hipLaunchKernelGGL((mfma_linear_kernel<NB, DUAL, 4>), dim3((tiles + 1) / 2), block, 0, st, a);
   else hipLaunchKernelGGL((mfma_linear_kernel<NB, DUAL, 8>), dim3(tiles), block, 0, st, a);
+}
+
+// the streaming form: up to 16 rows, K a whole number of chunks with at least one chunk per wave of a tile
+template <bool DUAL>
+static bool stream_applies(const MfmaArgs& a, int ks) {
+  constexpr int ck = StreamShape<DUAL>::CKB / 2;
+  return a.B <= 16 && (a.K % ck) == 0 && a.K / ck >= ks;
+}
+template <bool DUAL, int D>
+static int launch_mfma_stream_d(const MfmaArgs& a, int ks, hipStream_t st, const char* who) {
+  static bool granted[3] = {false, false, false};
+  const int tiles = (a.N + 15) / 16;
+  const size_t lds = (size_t)kMfWaves * D * StreamShape<DUAL>::kStage;
+  const auto grant = [&](const void* f, int i) {
+    if (granted[i] || lds <= 64 * 1024) return true;
+    hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return false; }
+    return granted[i] = true;
+  };
+  const dim3 block(kMfThreads);
+  if (ks == 2) {
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 2, D>), 0)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 2, D>), dim3((tiles + 3) / 4), block, lds, st, a);
+  } else if (ks == 4) {
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 4, D>), 1)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 4, D>), dim3((tiles + 1) / 2), block, lds, st, a);
+  } else {
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 8, D>), 2)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 8, D>), dim3(tiles), block, lds, st, a);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+// Eight waves per weight tile whenever K has a chunk for each, and a ring of two chunks: 64 KB of LDS, so two
+// workgroups share a compute unit — measured better than deeper rings with one workgroup per compute unit or fewer waves
+// per tile (7B MLP at 8 rows, ring 4 / 2: rank projection 8.9 / 7.9 us, pair 19.7 / 15.9, down_u 4.9 / 4.9).
+template <bool DUAL>
+static int launch_mfma_stream(const MfmaArgs& a, int ks, hipStream_t st, const char* who) {
+  if (a.K / (StreamShape<DUAL>::CKB / 2) >= 8) ks = 8;
+  return launch_mfma_stream_d<DUAL, 2>(a, ks, st, who);
 }
 
 template <bool DUAL>
@@ -148,6 +296,11 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
     a.y = a0.y + (int64_t)b0 * a0.ldy;
     if (a0.res) a.res = a0.res + (int64_t)b0 * a0.ldres;
     const int nb = (a.B + 15) / 16;
+    if (nb == 1 && stream_applies<DUAL>(a, ks)) {
+      const int rc = launch_mfma_stream<DUAL>(a, ks, st, who);
+      if (rc != kOk) return rc;
+      continue;
+    }
     if (nb == 1) launch_mfma_ks<1, DUAL>(a, ks, st);
     else if (nb == 2) launch_mfma_ks<2, DUAL>(a, ks, st);
     else if (nb == 3) launch_mfma_ks<3, DUAL>(a, ks, st);

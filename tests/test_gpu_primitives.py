@@ -226,6 +226,45 @@ def test_swiglu_prefill_rows_tiled_kernel(ops, B, D, R, mode):
     assert_close_bf16(h, ref, f"tiled swiglu mode {mode}", **bounds(ref))
 
 
+# ---- 3..16 rows: weights streamed through a wave's own LDS ring (its load counter is the only synchronisation)
+@pytest.mark.parametrize("B", [3, 8, 16])
+def test_small_batch_streaming_projections_repeat_bit_identically(ops, B):
+    """Shapes of the 7B MLP and an attention projection; every call of 20 gives the same bits (a chunk read before it
+    has landed would show as a difference between calls) and they match the oracle."""
+    d, R, D = 4096, 1536, 11008
+    x, p, h = rand_bf16(B, d, seed=1).cuda(), rand_bf16(B, 2 * R, seed=2).cuda(), rand_bf16(B, D, seed=3).cuda()
+    w_rank = rand_bf16(2 * R, d, std=0.02, seed=4).cuda()
+    gu, uu = rand_bf16(D, R, std=0.03, seed=5).cuda(), rand_bf16(D, R, std=0.03, seed=6).cuda()
+    w_down = rand_bf16(d, R, std=0.03, seed=7).cuda()
+    w_long = rand_bf16(1000, D - 0, std=0.01, seed=8).cuda()          # long K, ragged last weight tile
+    res = rand_bf16(B, d, seed=9).cuda()
+    os.environ["FLASHSVD_AMD_SPLITK"] = "0"                          # keep the narrow matrix on this kernel too
+    ops.release_split_workspace(x.device)
+    try:
+        calls = {
+            "rank": lambda: ops.linear(x, w_rank),
+            "pair": lambda: ops.swiglu_linear(p, gu, uu, up_off=R, mode=0),
+            "down_u": lambda: ops.linear(p[:, :R], w_down, residual=res),
+            "long": lambda: ops.linear(h, w_long),
+        }
+        first = {k: f() for k, f in calls.items()}
+        for _ in range(20):
+            for k, f in calls.items():
+                assert torch.equal(f(), first[k]), k
+    finally:
+        del os.environ["FLASHSVD_AMD_SPLITK"]
+        assert ops.ensure_split_workspace(x.device)
+    ref = O.lin(x.cpu(), w_rank.cpu())
+    assert_close_bf16(first["rank"], ref, "rank projection", **bounds(ref))
+    g, u = p.cpu()[:, :R].float() @ gu.cpu().float().t(), p.cpu()[:, R:].float() @ uu.cpu().float().t()
+    ref = torch.nn.functional.silu(g.to(torch.bfloat16)) * u.to(torch.bfloat16)
+    assert_close_bf16(first["pair"], ref, "pair", **bounds(ref))
+    ref = res.cpu() + O.lin(p.cpu()[:, :R], w_down.cpu())
+    assert_close_bf16(first["down_u"], ref, "down_u", **bounds(ref))
+    ref = O.lin(h.cpu(), w_long.cpu())
+    assert_close_bf16(first["long"], ref, "long K", **bounds(ref))
+
+
 # ---- K split over workgroups (registered scratch): same entry points, 17..127 rows, and 3..16 rows of a matrix with
 #      fewer than 128 sixteen-row tiles, and prompt rows of projections with few 64 x 64 tiles or a very long K
 @pytest.mark.parametrize("B,N,K", [(17, 1536, 11008), (32, 1024, 4096), (100, 200, 1536), (127, 4096, 1536), (64, 3072, 4096),
