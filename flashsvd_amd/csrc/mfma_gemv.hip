@@ -8,6 +8,9 @@
 // from L2: the batch is tiny) to V_MFMA_F32_16X16X32_BF16 and accumulates a 16 x 16 fp32 tile per 16
 // batch rows; the waves' tiles are added in wave order through LDS (deterministic) and the epilogue
 // applies the rounding points of the vector kernels: bias, one bf16 rounding, residual, or SwiGLU.
+// Two forms of the weight stream: fragments loaded straight from global memory (16 rows x 64 bytes per instruction;
+// any K that is a multiple of 32, up to 64 rows), and, up to 32 rows with K a whole number of 128- / 256-byte pieces,
+// whole row pieces loaded into a wave-private LDS ring and fragments read from there (a third faster).
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -144,16 +147,16 @@ template <bool DUAL> struct StreamShape {
 };
 
 // D: chunks in a wave's ring (D - 1 in flight while one multiplies)
-template <bool DUAL, int KS, int D>
+template <bool DUAL, int KS, int D, int NB>
 __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
   typedef StreamShape<DUAL> SS;
-  constexpr int NB = 1, NM = SS::NM, CKB = SS::CKB, kStage = SS::kStage;
+  constexpr int NM = SS::NM, CKB = SS::CKB, kStage = SS::kStage;
   constexpr int RT = kMfWaves / KS;
   constexpr int PPR = CKB / 16;                    // 16-byte pieces per row and chunk
   constexpr int KST = CKB / 64;                    // k-steps of 32 per chunk
   constexpr int RPI = 64 / PPR;                    // rows one load instruction covers (64 lanes x 16 bytes)
   constexpr int NI = 16 / RPI;                     // load instructions per matrix and chunk
-  constexpr int kGroup = NM * NI + NM * KST;       // loads per chunk: weight pieces into LDS, activation fragments into registers
+  constexpr int kGroup = NM * NI + NM * KST * NB;  // loads per chunk: weight pieces into LDS, activation fragments into registers
   static_assert((D - 1) * kGroup < 64 && D >= 2 && D <= 4, "vmcnt holds six bits; the waits below cover up to three groups in flight");
   extern __shared__ __align__(16) unsigned char st_smem[];     // [8 waves][D][kStage]; the partial tiles at the end
   float (*red)[NM][NB][4][64] = reinterpret_cast<float (*)[NM][NB][4][64]>(st_smem);
@@ -174,8 +177,10 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
     wsrc[0][q] = a.W + off;
     if (DUAL) wsrc[NM - 1][q] = a.W2 + off;
   }
-  const uint16_t* xsrc = a.x + (int64_t)min(lr, a.B - 1) * a.ldx + lg * 8;
-  bf16x8_t xf[D][NM][KST];
+  const uint16_t* xsrc[NB];
+#pragma unroll
+  for (int t = 0; t < NB; ++t) xsrc[t] = a.x + (int64_t)min(t * 16 + lr, a.B - 1) * a.ldx + lg * 8;
+  bf16x8_t xf[D][NM][KST][NB];
   // The wave's load counter is the only synchronisation: it counts weight pieces and activation fragments alike, in
   // issue order, so the loads of one chunk must stay together in the instruction stream (scheduling fences around them).
   const auto issue = [&](int c, int slot) {
@@ -187,13 +192,17 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
       for (int q = 0; q < NI; ++q)
         __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[m][q] + k0), (lptr_t)(ring + slot * kStage + m * 16 * CKB + q * 1024), 16, 0, 0);
 #pragma unroll
-      for (int s = 0; s < KST; ++s) xf[slot][m][s] = ldx_frag(xsrc + (m ? a.up_off : 0) + k0 + s * 32);
+      for (int s = 0; s < KST; ++s)
+#pragma unroll
+        for (int t = 0; t < NB; ++t) xf[slot][m][s][t] = ldx_frag(xsrc[t] + (m ? a.up_off : 0) + k0 + s * 32);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
   f32x4_t acc[NM][NB];
 #pragma unroll
-  for (int m = 0; m < NM; ++m) acc[m][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int m = 0; m < NM; ++m)
+#pragma unroll
+    for (int t = 0; t < NB; ++t) acc[m][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   // load counter values that leave the newest r groups in flight
   constexpr int kW0 = (7 << 4) | (15 << 8);
   const auto vm = [](int n) { return (n & 15) | ((n >> 4) << 14); };
@@ -218,7 +227,8 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
           const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(ring + u * kStage + m * 16 * CKB + lr * CKB + (((s * 4 + lg) ^ (lr % PPR)) * 16));
-          acc[m][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[u][m][s], acc[m][0], 0, 0, 0);
+#pragma unroll
+          for (int t = 0; t < NB; ++t) acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[u][m][s][t], acc[m][t], 0, 0, 0);
         }
     }
   }
@@ -239,9 +249,9 @@ static void launch_mfma_ks(const MfmaArgs& a, int ks, hipStream_t st) {
 template <bool DUAL>
 static bool stream_applies(const MfmaArgs& a, int ks) {
   constexpr int ck = StreamShape<DUAL>::CKB / 2;
-  return a.B <= 16 && (a.K % ck) == 0 && a.K / ck >= ks;
+  return a.B <= 32 && (a.K % ck) == 0 && a.K / ck >= ks;
 }
-template <bool DUAL, int D>
+template <bool DUAL, int D, int NB>
 static int launch_mfma_stream_d(const MfmaArgs& a, int ks, hipStream_t st, const char* who) {
   static bool granted[3] = {false, false, false};
   const int tiles = (a.N + 15) / 16;
@@ -254,14 +264,14 @@ static int launch_mfma_stream_d(const MfmaArgs& a, int ks, hipStream_t st, const
   };
   const dim3 block(kMfThreads);
   if (ks == 2) {
-    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 2, D>), 0)) return kErrLaunch;
-    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 2, D>), dim3((tiles + 3) / 4), block, lds, st, a);
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 2, D, NB>), 0)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 2, D, NB>), dim3((tiles + 3) / 4), block, lds, st, a);
   } else if (ks == 4) {
-    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 4, D>), 1)) return kErrLaunch;
-    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 4, D>), dim3((tiles + 1) / 2), block, lds, st, a);
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 4, D, NB>), 1)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 4, D, NB>), dim3((tiles + 1) / 2), block, lds, st, a);
   } else {
-    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 8, D>), 2)) return kErrLaunch;
-    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 8, D>), dim3(tiles), block, lds, st, a);
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 8, D, NB>), 2)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 8, D, NB>), dim3(tiles), block, lds, st, a);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
@@ -273,7 +283,7 @@ static int launch_mfma_stream_d(const MfmaArgs& a, int ks, hipStream_t st, const
 template <bool DUAL>
 static int launch_mfma_stream(const MfmaArgs& a, int ks, hipStream_t st, const char* who) {
   if (a.K / (StreamShape<DUAL>::CKB / 2) >= 8) ks = 8;
-  return launch_mfma_stream_d<DUAL, 2>(a, ks, st, who);
+  return a.B <= 16 ? launch_mfma_stream_d<DUAL, 2, 1>(a, ks, st, who) : launch_mfma_stream_d<DUAL, 2, 2>(a, ks, st, who);
 }
 
 template <bool DUAL>
@@ -286,8 +296,12 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
     if ((tiles * c + 7) / 8 >= 256 && ksteps / c >= 4) { ks = c; break; }
   // many rows (prefill): the tiled kernel reads every weight once per 128 rows instead of once per 64
   if (gemm_tiles_apply(a0)) return launch_gemm_tiles(a0, DUAL, st, who);
-  // a batch of rows: 32-row tiles with K split over workgroups, when the caller has registered a workspace
-  if (gemm_rows_apply(a0)) return launch_gemm_rows(a0, DUAL, st, who);
+  // a batch of rows: 32-row tiles with K split over workgroups, when the caller has registered a workspace — from 33
+  // rows on, and below that for matrices with fewer than 128 weight tiles (the streaming form would leave compute units
+  // idle: down_v of the 7B MLP at 32 rows 26.7 us there, 17.3 us split; the wide ones 12.3 / 25.3 / 6.7 us streamed
+  // against 13.4 / 28.8 / 8.8 us split)
+  const bool streamed = a0.B <= 32 && tiles >= 128 && stream_applies<DUAL>(a0, ks);
+  if (gemm_rows_apply(a0) && !streamed) return launch_gemm_rows(a0, DUAL, st, who);
   // batches above 64 rows go in slices of 64
   for (int b0 = 0; b0 < a0.B; b0 += 64) {
     MfmaArgs a = a0;
@@ -296,7 +310,7 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
     a.y = a0.y + (int64_t)b0 * a0.ldy;
     if (a0.res) a.res = a0.res + (int64_t)b0 * a0.ldres;
     const int nb = (a.B + 15) / 16;
-    if (nb == 1 && stream_applies<DUAL>(a, ks)) {
+    if (nb <= 2 && stream_applies<DUAL>(a, ks)) {
       const int rc = launch_mfma_stream<DUAL>(a, ks, st, who);
       if (rc != kOk) return rc;
       continue;

@@ -226,8 +226,8 @@ def test_swiglu_prefill_rows_tiled_kernel(ops, B, D, R, mode):
     assert_close_bf16(h, ref, f"tiled swiglu mode {mode}", **bounds(ref))
 
 
-# ---- 3..16 rows: weights streamed through a wave's own LDS ring (its load counter is the only synchronisation)
-@pytest.mark.parametrize("B", [3, 8, 16])
+# ---- 3..32 rows: weights streamed through a wave's own LDS ring (its load counter is the only synchronisation)
+@pytest.mark.parametrize("B", [3, 8, 16, 17, 32])
 def test_small_batch_streaming_projections_repeat_bit_identically(ops, B):
     """Shapes of the 7B MLP and an attention projection; every call of 20 gives the same bits (a chunk read before it
     has landed would show as a difference between calls) and they match the oracle."""
