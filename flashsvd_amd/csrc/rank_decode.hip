@@ -30,7 +30,10 @@ __device__ __forceinline__ bf16x8_t ld_frag(const uint16_t* p) {
 }
 __device__ __forceinline__ bf16x8_t zero_frag() { return __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u}); }
 
-template <int REP, int KS>
+// PKL: the Pk rows of a chunk (16 keys x 128 bytes per key sub-tile) are loaded as whole 128-byte pieces straight into an
+// LDS slot of the wave and the fragments read from there, instead of 16 rows x 64 bytes per fragment load from global
+// memory (Rk a multiple of 64; 13 % of the kernel's time at 16 x 4096 keys of rank 1664 was that access pattern)
+template <int REP, int KS, bool PKL>
 __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(RankDecodeArgs a) {
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
   __shared__ float qs[REP][DH];
@@ -43,6 +46,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   constexpr int KROW = 64;
   constexpr int KU_BYTES = 2 * DH * KROW * 2, TB_BYTES = 4 * kRdMaxChunks * 512 * 4;
   __shared__ __align__(16) unsigned char smem[KU_BYTES > TB_BYTES ? KU_BYTES : TB_BYTES];
+  __shared__ __align__(16) unsigned char pkslot[PKL ? 4 * KS * 2048 : 16];   // [wave][sub-tile][16 keys][128 bytes]
   uint16_t (*kus)[DH][KROW] = reinterpret_cast<uint16_t (*)[DH][KROW]>(smem);
   float (*tbuf)[kRdMaxChunks * 512] = reinterpret_cast<float (*)[kRdMaxChunks * 512]>(smem);
 
@@ -137,13 +141,52 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
 #pragma unroll
         for (int k = 0; k < 2; ++k) af[j][k] = (r0 + k * 32 + lg * 8 < a.Rk) ? ld_frag(arow[j] + r0 + k * 32) : zero_frag();
     };
+    // PKL: lane -> key row lane / 8 (+ 8 per instruction) and the piece that belongs at LDS position lane % 8 of that row
+    // (position p of row r holds piece p ^ r % 8: conflict-free 16-byte fragment reads)
+    typedef const __attribute__((address_space(1))) void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    unsigned char* myslot = pkslot + (PKL ? wave * KS * 2048 : 0);
+    const uint16_t* prow[KS][2];
+    if (PKL) {
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int row = i * 8 + (lane >> 3);
+          const int pkey = min(kt + (4 * j + wave) * 16 + row, k1 - 1);
+          prow[j][i] = pk_b + (int64_t)pkey * a.spk_s + (((lane & 7) ^ (row & 7)) * 8);
+        }
+    }
+    const auto issue_pk = [&](int r0) {
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          __builtin_amdgcn_global_load_lds((gptr_t)(prow[j][i] + r0), (lptr_t)(myslot + j * 2048 + i * 1024), 16, 0, 0);
+    };
+    const auto read_pk = [&]() {
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+#pragma unroll
+        for (int k = 0; k < 2; ++k)
+          af[j][k] = *reinterpret_cast<const bf16x8_t*>(myslot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
+    };
     // (the barrier that ended the previous tile's last chunk also freed both buffers)
     load_ku(0);
-    load_pk(0);
+    if (PKL) issue_pk(0); else load_pk(0);
     store_ku(0);
     __syncthreads();
     for (int st = 0; st < nstep; ++st) {
       const int cur = st & 1;
+      if (PKL) {
+        // the chunk's pieces were requested a whole step ago: wait for them, take the fragments into registers, and
+        // hand the slot to the next chunk at once
+        __builtin_amdgcn_s_waitcnt(0);
+        read_pk();
+        __builtin_amdgcn_s_waitcnt(0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (st + 1 < nstep) issue_pk((st + 1) * 64);
+      }
       if (st + 1 < nstep) load_ku((st + 1) * 64);
 #pragma unroll
       for (int k = 0; k < 2; ++k) {
@@ -156,7 +199,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
           for (int t = 0; t < NT; ++t) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][k], bf[t], accs[j][t], 0, 0, 0);
       }
       if (st + 1 < nstep) {
-        load_pk((st + 1) * 64);                    // lands while the chunk is handed over
+        if (!PKL) load_pk((st + 1) * 64);          // lands while the chunk is handed over
         store_ku(cur ^ 1);
       }
       __syncthreads();
@@ -330,14 +373,21 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   // length; short splits would only rebuild clamped keys)
   const int per = (a.S + a.nsplit - 1) / a.nsplit;
   const int ks = per >= 128 ? 2 : 1;
-  if (rep % 4 == 0) hipLaunchKernelGGL((rank_decode_partial_kernel<4, 1>), dim3(a.nsplit, a.Hk * (rep / 4), a.B), block, 0, st, a);
+  const bool pkl = (a.Rk % 64) == 0;               // whole 128-byte pieces of every Pk row
+#define FSVD_RD_LAUNCH(REP_, KS_, GY_)                                                                                              \
+  do {                                                                                                                              \
+    if (pkl) hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, true>), dim3(a.nsplit, GY_, a.B), block, 0, st, a);          \
+    else hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, false>), dim3(a.nsplit, GY_, a.B), block, 0, st, a);             \
+  } while (0)
+  if (rep % 4 == 0) FSVD_RD_LAUNCH(4, 1, a.Hk * (rep / 4));
   else if (rep % 2 == 0) {
-    if (ks >= 2) hipLaunchKernelGGL((rank_decode_partial_kernel<2, 2>), dim3(a.nsplit, a.Hk * (rep / 2), a.B), block, 0, st, a);
-    else hipLaunchKernelGGL((rank_decode_partial_kernel<2, 1>), dim3(a.nsplit, a.Hk * (rep / 2), a.B), block, 0, st, a);
+    if (ks >= 2) FSVD_RD_LAUNCH(2, 2, a.Hk * (rep / 2));
+    else FSVD_RD_LAUNCH(2, 1, a.Hk * (rep / 2));
   } else {
-    if (ks >= 2) hipLaunchKernelGGL((rank_decode_partial_kernel<1, 2>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
-    else hipLaunchKernelGGL((rank_decode_partial_kernel<1, 1>), dim3(a.nsplit, a.Hk * rep, a.B), block, 0, st, a);
+    if (ks >= 2) FSVD_RD_LAUNCH(1, 2, a.Hk * rep);
+    else FSVD_RD_LAUNCH(1, 1, a.Hk * rep);
   }
+#undef FSVD_RD_LAUNCH
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: stage 1 launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
   hipLaunchKernelGGL(rank_decode_merge_kernel, dim3(a.H, a.B), block, 0, st, a);
