@@ -75,6 +75,62 @@ __device__ __forceinline__ void mfma_finish(const MfmaArgs& a, float (*red)[DUAL
   }
 }
 
+// K split over the gridDim.y workgroups of a weight tile (single matrix): the workgroup's sum of every output element is
+// parked in the caller's workspace with write-through agent-scope stores, the arrival is counted once all of them are
+// acknowledged, and the last workgroup to arrive adds the gridDim.y shares in split order (its own included, so the sum
+// does not depend on who came last) through agent-scope loads, all in flight at once, then applies the epilogue.  No
+// fence: a release or acquire fence writes back or empties a whole L2 under the weight streams of the other workgroups.
+template <int NB, int KS>
+__device__ __forceinline__ void mfma_finish_split(const MfmaArgs& a, float (*red)[1][NB][4][64], const f32x4_t (&acc)[1][NB]) {
+  constexpr int RT = kMfWaves / KS;
+  constexpr int E = RT * NB * 256;                 // output elements of this workgroup
+  constexpr int kMaxZ = 8;
+  __shared__ int last_flag;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int Z = gridDim.y;
+#pragma unroll
+  for (int t = 0; t < NB; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][0][t][i][lane] = acc[0][t][i];
+  __syncthreads();
+  uint32_t* part = reinterpret_cast<uint32_t*>(a.ws_part) + (size_t)blockIdx.x * Z * E;
+  for (int o = tid; o < E; o += kMfThreads) {
+    const int q = o / (NB * 256), oo = o - q * (NB * 256);
+    const int t = oo >> 8, r = oo & 255, i = r >> 6, l = r & 63;
+    float v0 = 0.f;
+#pragma unroll
+    for (int w = 0; w < KS; ++w) v0 += red[q * KS + w][0][t][i][l];
+    __hip_atomic_store(part + (size_t)blockIdx.y * E + o, __float_as_uint(v0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (tid == 0) {
+    const int prev = atomicAdd(a.ws_count + blockIdx.x, 1);
+    const int last = prev == Z - 1;
+    if (last) a.ws_count[blockIdx.x] = 0;          // ready for the next launch
+    last_flag = last;
+  }
+  __syncthreads();
+  if (last_flag == 0) return;
+  for (int o = tid; o < E; o += kMfThreads) {
+    const int q = o / (NB * 256), oo = o - q * (NB * 256);
+    const int t = oo >> 8, r = oo & 255, i = r >> 6, l = r & 63;
+    const int n = (blockIdx.x * RT + q) * 16 + (l >> 4) * 4 + i, b = t * 16 + (l & 15);
+    uint32_t sh[kMaxZ];
+#pragma unroll
+    for (int z = 0; z < kMaxZ; ++z) sh[z] = __hip_atomic_load(part + (size_t)min(z, Z - 1) * E + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float v0 = 0.f;
+#pragma unroll
+    for (int z = 0; z < kMaxZ; ++z)
+      if (z < Z) v0 += __uint_as_float(sh[z]);
+    if (n >= a.N || b >= a.B) continue;
+    if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
+    float v = round_bf16(v0);
+    if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)b * a.ldres + n]) + v);
+    a.y[(int64_t)b * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+  }
+}
+
 // NB: 16-row batch tiles (B <= 16 * NB); KS: waves that split K for one 16-row weight tile, so a workgroup
 // of 8 waves covers 8 / KS weight tiles
 template <int NB, bool DUAL, int KS>
@@ -147,8 +203,11 @@ template <bool DUAL> struct StreamShape {
 };
 
 // D: chunks in a wave's ring (D - 1 in flight while one multiplies)
-template <bool DUAL, int KS, int D, int NB>
+// ZS: K also split over the gridDim.y workgroups of a tile (single matrix; narrow projections that would otherwise
+// leave compute units idle): the KS waves of workgroup z act as waves z * KS .. z * KS + KS - 1 of KS * gridDim.y
+template <bool DUAL, int KS, int D, int NB, bool ZS = false>
 __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
+  static_assert(!ZS || !DUAL, "the split over workgroups is built for a single matrix");
   typedef StreamShape<DUAL> SS;
   constexpr int NM = SS::NM, CKB = SS::CKB, kStage = SS::kStage;
   constexpr int RT = kMfWaves / KS;
@@ -161,11 +220,12 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
   extern __shared__ __align__(16) unsigned char st_smem[];     // [8 waves][D][kStage]; the partial tiles at the end
   float (*red)[NM][NB][4][64] = reinterpret_cast<float (*)[NM][NB][4][64]>(st_smem);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
-  const int rt = wave / KS, ks = wave % KS;
+  const int rt = wave / KS, ks = ZS ? (int)blockIdx.y * KS + wave % KS : wave % KS;
+  const int KSV = ZS ? KS * (int)gridDim.y : KS;   // waves that share a weight tile
   const int n0 = (blockIdx.x * RT + rt) * 16;
   unsigned char* ring = st_smem + (size_t)wave * D * kStage;
   const int nchunk = a.K / (CKB / 2);
-  const int cw = (nchunk - ks + KS - 1) / KS;      // this wave's chunks: ks, ks + KS, ... (the KS waves of a tile read adjacent pieces)
+  const int cw = max(0, (nchunk - ks + KSV - 1) / KSV);   // this wave's chunks: ks, ks + KSV, ... (the waves of a tile read adjacent pieces)
   typedef const __attribute__((address_space(1))) void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
   const int lrow = lane / PPR, lpc = lane % PPR;
@@ -184,7 +244,7 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
   // The wave's load counter is the only synchronisation: it counts weight pieces and activation fragments alike, in
   // issue order, so the loads of one chunk must stay together in the instruction stream (scheduling fences around them).
   const auto issue = [&](int c, int slot) {
-    const int k0 = (c * KS + ks) * (CKB / 2);
+    const int k0 = (c * KSV + ks) * (CKB / 2);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
@@ -233,7 +293,8 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
     }
   }
   __syncthreads();                                 // every wave is done with its ring: the partial tiles take its place
-  mfma_finish<NB, DUAL, KS>(a, red, acc);
+  if constexpr (ZS) mfma_finish_split<NB, KS>(a, red, acc);
+  else mfma_finish<NB, DUAL, KS>(a, red, acc);
 }
 
 template <int NB, bool DUAL>
@@ -286,6 +347,45 @@ static int launch_mfma_stream(const MfmaArgs& a, int ks, hipStream_t st, const c
   return a.B <= 16 ? launch_mfma_stream_d<DUAL, 2, 1>(a, ks, st, who) : launch_mfma_stream_d<DUAL, 2, 2>(a, ks, st, who);
 }
 
+// Narrow projections (fewer than 128 weight tiles, e.g. down_v of the 7B MLP: 96) at 3..32 rows: the streaming form with
+// K split over up to eight workgroups per tile as well, enough to give every compute unit about two workgroups while
+// every wave keeps at least one chunk.  Needs the registered workspace.  Measured per call, 32-row tiles split over
+// workgroups -> this form: down_v (1536 x 11008, five shares) 16.4 -> 12.2 us at 8 rows, 17.4 -> 16.6 at 32 rows; o_v
+// (1024 x 4096, four shares) 8.7 -> 6.2 at 8 rows, 8.8 -> 7.5 at 32 rows.
+constexpr int kStreamSplitMax = 8;
+static int stream_split_shares(const MfmaArgs& a) {
+  constexpr int ck = StreamShape<false>::CKB / 2;
+  if (a.B > 32 || (a.K % ck) != 0) return 1;
+  const SplitWorkspace ws = split_workspace();
+  const int tiles = (a.N + 15) / 16, nchunk = a.K / ck;
+  if (ws.part == nullptr || tiles > ws.ncount || tiles >= 128) return 1;
+  const size_t share = (size_t)(a.B <= 16 ? 1 : 2) * 256;
+  int z = std::min(kStreamSplitMax, (480 + tiles - 1) / tiles);
+  while (z > 1 && (nchunk < kMfWaves * z || (size_t)tiles * z * share > ws.part_floats)) --z;
+  return z;
+}
+template <int NB>
+static int launch_mfma_stream_split(const MfmaArgs& a0, int z, hipStream_t st, const char* who) {
+  static bool granted = false;
+  constexpr int D = 2;
+  const size_t lds = (size_t)kMfWaves * D * StreamShape<false>::kStage;
+  const void* f = reinterpret_cast<const void*>(&mfma_stream_kernel<false, 8, D, NB, true>);
+  if (!granted && lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
+    granted = true;
+  }
+  MfmaArgs a = a0;
+  const SplitWorkspace ws = split_workspace();
+  a.ksplit = z;
+  a.ws_part = ws.part;
+  a.ws_count = ws.count;
+  hipLaunchKernelGGL((mfma_stream_kernel<false, 8, D, NB, true>), dim3((a.N + 15) / 16, z), dim3(kMfThreads), lds, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
 template <bool DUAL>
 static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
   // K is split over as few waves as still give every compute unit a workgroup: long slices amortise the
@@ -297,10 +397,14 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
   // many rows (prefill): the tiled kernel reads every weight once per 128 rows instead of once per 64
   if (gemm_tiles_apply(a0)) return launch_gemm_tiles(a0, DUAL, st, who);
   // a batch of rows: 32-row tiles with K split over workgroups, when the caller has registered a workspace — from 33
-  // rows on, and below that for matrices with fewer than 128 weight tiles (the streaming form would leave compute units
-  // idle: down_v of the 7B MLP at 32 rows 26.7 us there, 17.3 us split; the wide ones 12.3 / 25.3 / 6.7 us streamed
-  // against 13.4 / 28.8 / 8.8 us split)
+  // rows on (up to 32 rows the streaming form is faster: 12.3 / 25.3 / 6.7 us against 13.4 / 28.8 / 8.8 us on the wide
+  // matrices of the 7B MLP; matrices with fewer than 128 weight tiles take its split form above, or the 32-row tiles
+  // when their K does not divide into chunks)
   const bool streamed = a0.B <= 32 && tiles >= 128 && stream_applies<DUAL>(a0, ks);
+  if constexpr (!DUAL) {
+    const int z = stream_split_shares(a0);
+    if (z > 1) return a0.B <= 16 ? launch_mfma_stream_split<1>(a0, z, st, who) : launch_mfma_stream_split<2>(a0, z, st, who);
+  }
   if (gemm_rows_apply(a0) && !streamed) return launch_gemm_rows(a0, DUAL, st, who);
   // batches above 64 rows go in slices of 64
   for (int b0 = 0; b0 < a0.B; b0 += 64) {
