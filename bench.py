@@ -120,6 +120,23 @@ def kernel_configs(model, cache, dec, n_layers: int) -> dict:
     us = per_layer_kernel_us(attn, n_layers)
     nb = 8 * d * CFG["attn_rank"] * 2 + 2 * PROMPT_LEN * CFG["num_heads"] * CFG["head_dim"] * 2 + 2 * d * 2 * 2
     out["attention_block_bs1_ctx512"] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3, "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS}
+    # the same block over a rank-space cache (coefficients Pk / Pv of 512 tokens, K and V rebuilt in the kernel)
+    from flashsvd_amd.runtime.cache import FlashSVDLegacySparseKVCache
+    Ra = CFG["attn_rank"]
+    rcache = FlashSVDLegacySparseKVCache(model.config, max_batch_size=1, max_cache_len=PROMPT_LEN + 8, device="cuda", dtype=torch.bfloat16)
+    for i in range(n_layers):
+        rcache.ensure_layer_ranks(i, Ra, Ra)
+        rcache.key_cache[i][:, :PROMPT_LEN].normal_(0.0, 1.0)
+        rcache.value_cache[i][:, :PROMPT_LEN].normal_(0.0, 1.0)
+
+    def attn_rank(i):
+        n1 = L[i].input_layernorm
+        return L[i].self_attn.decode_token(x, rcache, pos, norm_weight=n1.weight, eps=n1.variance_epsilon, residual=x, rope=dec.rope)
+    us = per_layer_kernel_us(attn_rank, n_layers)
+    nb = 8 * d * Ra * 2 + 2 * PROMPT_LEN * Ra * 2 + 2 * Ra * 2 + 2 * d * 2 * 2
+    out["attention_block_bs1_ctx512_rank_kv"] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3, "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS,
+                                                 "rebuild_GFLOP": 2 * PROMPT_LEN * Ra * CFG["num_kv_heads"] * CFG["head_dim"] / 1e9}
+    del rcache
     for B in (1, 8, 32):
         xb = torch.randn(B, d, device="cuda").to(torch.bfloat16)
 

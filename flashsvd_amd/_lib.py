@@ -82,6 +82,8 @@ SIGNATURES = {
                                         c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                         c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                         c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
+    "fsvd_rankkv_append": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p,
+                                   c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_lowrank_expand_heads": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
                                           c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
                                           c_int, c_void_p]),

@@ -441,6 +441,23 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h, const voi
   return launch_rank_decode(a, static_cast<hipStream_t>(stream));
 }
 
+int fsvd_rankkv_append(const void* pk, int64_t ldpk, const void* pv, int64_t ldpv, void* pk_cache, int64_t spk_b, int64_t spk_s,
+                       void* pv_cache, int64_t spv_b, int64_t spv_s, const int32_t* positions, int B, int S, int Rk, int Rv, void* stream) {
+  const char* fn = "fsvd_rankkv_append";
+  FSVD_REQUIRE_PTR(pk, fn); FSVD_REQUIRE_PTR(pv, fn); FSVD_REQUIRE_PTR(pk_cache, fn); FSVD_REQUIRE_PTR(pv_cache, fn); FSVD_REQUIRE_PTR(positions, fn);
+  if (B <= 0 || S <= 0 || Rk <= 0 || Rv <= 0 || (Rk % 8) || (Rv % 8) || ldpk < Rk || ldpv < Rv || spk_s < Rk || spv_s < Rv) {
+    set_last_error("%s: bad shape B=%d S=%d Rk=%d Rv=%d (ranks are multiples of 8, row strides at least the rank)", fn, B, S, Rk, Rv);
+    return kErrBadShape;
+  }
+  const auto mis = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+  if (mis(pk) || mis(pv) || mis(pk_cache) || mis(pv_cache) || (ldpk % 8) || (ldpv % 8) || (spk_b % 8) || (spk_s % 8) || (spv_b % 8) || (spv_s % 8)) {
+    set_last_error("%s: pointers and strides must be 16-byte aligned", fn);
+    return kErrBadAlign;
+  }
+  return launch_rankkv_append(cu16(pk), ldpk, cu16(pv), ldpv, u16(pk_cache), spk_b, spk_s, u16(pv_cache), spv_b, spv_s, positions, B, S, Rk, Rv,
+                              static_cast<hipStream_t>(stream));
+}
+
 int fsvd_lowrank_expand_heads(const void* p, int64_t sp_b, int64_t sp_m, int64_t sp_h, const void* u, int64_t ldu, const void* bias,
                               const void* cos, const void* sin, int rope_len, const int32_t* positions, void* y, int64_t sy_b,
                               int64_t sy_m, int64_t sy_h, int dst_by_position, int dst_rows, int B, int M, int heads, int Dh, int R,

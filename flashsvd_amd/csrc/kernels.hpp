@@ -108,6 +108,8 @@ struct RankDecodeArgs {
   float scale;
 };
 int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st);
+int launch_rankkv_append(const uint16_t* pk, int64_t ldpk, const uint16_t* pv, int64_t ldpv, uint16_t* pkc, int64_t spk_b, int64_t spk_s,
+                         uint16_t* pvc, int64_t spv_b, int64_t spv_s, const int32_t* positions, int B, int S, int Rk, int Rv, hipStream_t st);
 
 struct ExpandArgs {
   const uint16_t* p; int64_t sp_b, sp_m, sp_h;      // rank coefficients [B,M,(heads),R]; sp_h = 0 when shared

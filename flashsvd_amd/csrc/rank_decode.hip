@@ -30,11 +30,26 @@ __device__ __forceinline__ bf16x8_t ld_frag(const uint16_t* p) {
 }
 __device__ __forceinline__ bf16x8_t zero_frag() { return __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u}); }
 
+// dynamic LDS of the partial kernel: k_u stages [stage][128 d][64 r] bf16 (two, or three in the deep form), reused for the
+// four waves' rank-space partials [4][kRdMaxChunks * 512] fp32 at the end; then the waves' Pk slots
+template <int KS, bool PKL, bool DEEP> struct RankDecodeLds {
+  static constexpr int kStages = DEEP ? 3 : 2;
+  static constexpr int kKu = kStages * 128 * 64 * 2, kTb = 4 * kRdMaxChunks * 512 * 4;
+  static constexpr int kMain = kKu > kTb ? kKu : kTb;
+  static constexpr int kPkSlots = DEEP ? 2 : 1;
+  static constexpr int kBytes = kMain + (PKL ? 4 * kPkSlots * KS * 2048 : 0);
+};
+
 // PKL: the Pk rows of a chunk (16 keys x 128 bytes per key sub-tile) are loaded as whole 128-byte pieces straight into an
 // LDS slot of the wave and the fragments read from there, instead of 16 rows x 64 bytes per fragment load from global
 // memory (Rk a multiple of 64; 13 % of the kernel's time at 16 x 4096 keys of rank 1664 was that access pattern)
-template <int REP, int KS, bool PKL>
+// DEEP (short splits: one key tile or a few per workgroup, so the pass over r is a chain of chunk latencies): k_u chunks
+// are loaded straight into a ring of three LDS stages as well, two chunks ahead, and the Pk pieces two chunks ahead into
+// two slots per wave; the wave's load counter and one barrier per chunk are the synchronisation.  Batch 1, 512 keys,
+// rank 1024: 24 us -> see the launcher.
+template <int REP, int KS, bool PKL, bool DEEP = false>
 __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(RankDecodeArgs a) {
+  static_assert(!DEEP || (PKL && KS == 1), "the deep form is built for single sub-tiles with Pk through LDS");
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
   __shared__ float qs[REP][DH];
   __shared__ float wm[4][REP], wl[4][REP];
@@ -44,9 +59,10 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   // (lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of a half wave), and with this placement the fragment reads (lane =
   // row % 16 + 16 * piece) touch every bank once per group (rows padded to 144 bytes put two lanes on a bank)
   constexpr int KROW = 64;
-  constexpr int KU_BYTES = 2 * DH * KROW * 2, TB_BYTES = 4 * kRdMaxChunks * 512 * 4;
-  __shared__ __align__(16) unsigned char smem[KU_BYTES > TB_BYTES ? KU_BYTES : TB_BYTES];
-  __shared__ __align__(16) unsigned char pkslot[PKL ? 4 * KS * 2048 : 16];   // [wave][sub-tile][16 keys][128 bytes]
+  typedef RankDecodeLds<KS, PKL, DEEP> Lds;
+  extern __shared__ __align__(16) unsigned char rd_smem[];
+  unsigned char* smem = rd_smem;                                 // k_u stages, then the waves' partials
+  unsigned char* pkslot = rd_smem + Lds::kMain;                  // [wave][slot][sub-tile][16 keys][128 bytes]
   uint16_t (*kus)[DH][KROW] = reinterpret_cast<uint16_t (*)[DH][KROW]>(smem);
   float (*tbuf)[kRdMaxChunks * 512] = reinterpret_cast<float (*)[kRdMaxChunks * 512]>(smem);
 
@@ -145,7 +161,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
     // (position p of row r holds piece p ^ r % 8: conflict-free 16-byte fragment reads)
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    unsigned char* myslot = pkslot + (PKL ? wave * KS * 2048 : 0);
+    unsigned char* myslot = pkslot + (PKL ? wave * Lds::kPkSlots * KS * 2048 : 0);
     const uint16_t* prow[KS][2];
     if (PKL) {
 #pragma unroll
@@ -171,6 +187,60 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         for (int k = 0; k < 2; ++k)
           af[j][k] = *reinterpret_cast<const bf16x8_t*>(myslot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
     };
+    if constexpr (DEEP) {
+      // lane -> LDS row wave * 32 + i * 8 + lane / 8 and position lane % 8 of a stage; the row holds head dimension kd(row)
+      // and its position p the piece p ^ row % 8 (the placement store_ku gives the register form)
+      const uint16_t* kusrc[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = wave * 32 + i * 8 + (lane >> 3);
+        const int rd = ((row >> 4) / 4) * HALF + (row & 15) * 4 + ((row >> 4) % 4);
+        kusrc[i] = ku_h + (int64_t)rd * a.ldku + (((lane & 7) ^ (row & 7)) * 8);
+      }
+      constexpr int kGroup = 6;                    // loads per chunk and wave: four of k_u, two of Pk
+      const auto issue_group = [&](int c) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          __builtin_amdgcn_global_load_lds((gptr_t)(kusrc[i] + c * 64), (lptr_t)(smem + (c % 3) * (DH * KROW * 2) + (wave * 32 + i * 8) * 128), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          __builtin_amdgcn_global_load_lds((gptr_t)(prow[0][i] + c * 64), (lptr_t)(myslot + (c & 1) * 2048 + i * 1024), 16, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      constexpr int kNoLgkm = (7 << 4) | (15 << 8);              // wait on the load counter only
+      constexpr int kNoVm = (7 << 4) | 15 | (3 << 14);           // wait on the LDS counter only
+      // (the barrier that ended the previous tile freed every stage and slot)
+      issue_group(0);
+      if (nstep > 1) issue_group(1);
+      for (int st = 0; st < nstep; ++st) {
+        // chunk st has landed once only the group issued after it is outstanding
+        if (st + 1 < nstep) __builtin_amdgcn_s_waitcnt(kNoLgkm | kGroup);
+        else __builtin_amdgcn_s_waitcnt(kNoLgkm | 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 2; ++k)
+          af[0][k] = *reinterpret_cast<const bf16x8_t*>(myslot + (st & 1) * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
+        __builtin_amdgcn_s_waitcnt(kNoVm | (0 << 8));            // fragments in registers: the slot is free again
+        // everyone's pieces of chunk st are in, and stage (st - 1) % 3 is read out (its fragments fed matrix products that
+        // precede this point).  The bare barrier instruction: __syncthreads() carries a fence that waits for ALL of the
+        // wave's loads, the chunks requested ahead included
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (st + 2 < nstep) issue_group(st + 2);
+        const int cur = st % 3;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          bf16x8_t bf[NT];
+#pragma unroll
+          for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+#pragma unroll
+          for (int t = 0; t < NT; ++t) accs[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[0][k], bf[t], accs[0][t], 0, 0, 0);
+        }
+      }
+      __syncthreads();                                           // the last stages are read out before the next tile refills them
+    } else {
     // (the barrier that ended the previous tile's last chunk also freed both buffers)
     load_ku(0);
     if (PKL) issue_pk(0); else load_pk(0);
@@ -203,6 +273,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         store_ku(cur ^ 1);
       }
       __syncthreads();
+    }
     }
 #pragma unroll
     for (int j = 0; j < KS; ++j) {
@@ -302,13 +373,28 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
 }
 
 // out[b,h,:] = (sum_s w_s Acc_s / max(sum_s w_s L_s, 1e-20)) @ v_u[h]^T (+ bv[h])
+// grid (H, B, head-dimension slices): every slice merges the splits for itself (a few KB from L2) and multiplies by its
+// 128 / gridDim.z rows of v_u[h]; a wave takes four rows at a time with all of their loads in flight.  With one workgroup
+// per head and one row per wave at a time, a batch-1 call spent 36 us here on 32 compute units (8 MB of v_u, one load
+// latency per row).
 __global__ __launch_bounds__(kRdThreads) void rank_decode_merge_kernel(RankDecodeArgs a) {
-  constexpr int DH = 128;
-  __shared__ float ts[kRdMaxChunks * 512];
-  __shared__ float wsc[64];
+  constexpr int DH = 128, RW = 4, NIT = kRdMaxChunks;
+  __shared__ __align__(16) float ts[kRdMaxChunks * 512];
   const int h = blockIdx.x, b = blockIdx.y;
+  const int rows = DH / (int)gridDim.z, d0 = (int)blockIdx.z * rows;   // gridDim.z divides 128 / (4 waves * RW) = 8
   const int hk = h / (a.H / a.Hk);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // the v_u rows of the first round are requested before the merge, which is a chain of dependent loads of its own
+  u32x4_t v[RW][NIT];
+  const auto load_rows = [&](int dd) {
+    const uint16_t* row = a.v_u + (int64_t)(hk * DH + d0 + dd) * a.ldvu + lane * 8;
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+      for (int j = 0; j < RW; ++j)
+        v[j][it] = (lane * 8 + it * 512 < a.Rv) ? *reinterpret_cast<const u32x4_t*>(row + (int64_t)j * a.ldvu + it * 512) : u32x4_t{0u, 0u, 0u, 0u};
+  };
+  load_rows(wave * RW);
   const int64_t slot0 = ((int64_t)b * a.H + h) * a.nsplit;
   float M = -INFINITY;
   for (int s = 0; s < a.nsplit; ++s) M = fmaxf(M, a.ws_m[slot0 + s]);
@@ -318,30 +404,52 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_merge_kernel(RankDecod
     den += ((m == -INFINITY) ? 0.f : __expf(m - M)) * a.ws_l[slot0 + s];
   }
   const float inv = 1.0f / fmaxf(den, 1e-20f);
-  for (int r = tid; r < a.Rv; r += kRdThreads) {
-    float t = 0.f;
-    for (int s = 0; s < a.nsplit; ++s) {
-      const float m = a.ws_m[slot0 + s];
-      const float w = (m == -INFINITY) ? 0.f : __expf(m - M);
-      t += w * a.ws_acc[(slot0 + s) * a.Rv + r];
-    }
-    ts[r] = t * inv;
+  // four consecutive r per thread, the loads of up to eight splits in flight at once (one split per round trip made this
+  // loop the longest part of the kernel); the splits are added in order
+  constexpr int SU = 8;
+  for (int r = tid * 4; r < kRdMaxChunks * 512; r += kRdThreads * 4) {
+    f32x4_t t = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (r < a.Rv)                                  // Rv is a multiple of 8: the four are all inside or all outside
+      for (int s0 = 0; s0 < a.nsplit; s0 += SU) {
+        f32x4_t x[SU];
+        float w[SU];
+#pragma unroll
+        for (int u = 0; u < SU; ++u) {
+          const int sidx = min(s0 + u, a.nsplit - 1);
+          x[u] = *reinterpret_cast<const f32x4_t*>(a.ws_acc + (slot0 + sidx) * a.Rv + r);
+          const float m = a.ws_m[slot0 + sidx];
+          w[u] = (s0 + u < a.nsplit && m != -INFINITY) ? __expf(m - M) : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < SU; ++u) t += w[u] * x[u];
+      }
+    *reinterpret_cast<f32x4_t*>(&ts[r]) = t * inv;  // zero past Rv: the products below run over whole chunks
   }
   __syncthreads();
-  (void)wsc;
   uint16_t* outp = a.out + (int64_t)b * a.so_b + (int64_t)h * a.so_h;
-  for (int d = wave; d < DH; d += kRdThreads / 64) {
-    const uint16_t* row = a.v_u + (int64_t)(hk * DH + d) * a.ldvu;
-    float acc = 0.f;
-    for (int r = lane * 8; r < a.Rv; r += 512) {
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(row + r);
-      acc += ts[r] * bf16_lo(v.x) + ts[r + 1] * bf16_hi(v.x) + ts[r + 2] * bf16_lo(v.y) + ts[r + 3] * bf16_hi(v.y) +
-             ts[r + 4] * bf16_lo(v.z) + ts[r + 5] * bf16_hi(v.z) + ts[r + 6] * bf16_lo(v.w) + ts[r + 7] * bf16_hi(v.w);
+  // wave w takes rows d0 + w * RW + j (+ 4 * RW per round); rows is a multiple of 4 * RW
+  for (int dd = wave * RW; dd < rows; dd += (kRdThreads / 64) * RW) {
+    if (dd != wave * RW) load_rows(dd);
+    float acc[RW];
+#pragma unroll
+    for (int j = 0; j < RW; ++j) acc[j] = 0.f;
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int r = lane * 8 + it * 512;
+      const f32x4_t t0 = *reinterpret_cast<const f32x4_t*>(&ts[r]), t1 = *reinterpret_cast<const f32x4_t*>(&ts[r + 4]);
+#pragma unroll
+      for (int j = 0; j < RW; ++j)
+        acc[j] += t0[0] * bf16_lo(v[j][it].x) + t0[1] * bf16_hi(v[j][it].x) + t0[2] * bf16_lo(v[j][it].y) + t0[3] * bf16_hi(v[j][it].y) +
+                  t1[0] * bf16_lo(v[j][it].z) + t1[1] * bf16_hi(v[j][it].z) + t1[2] * bf16_lo(v[j][it].w) + t1[3] * bf16_hi(v[j][it].w);
     }
-    acc = wave_sum(acc);
-    if (lane == 0) {
-      if (a.bv) acc += bf16_bits_to_f32(a.bv[hk * DH + d]);
-      outp[d] = (uint16_t)f32_to_bf16_bits(acc);
+#pragma unroll
+    for (int j = 0; j < RW; ++j) {
+      float o = wave_sum(acc[j]);
+      if (lane == 0) {
+        const int d = d0 + dd + j;
+        if (a.bv) o += bf16_bits_to_f32(a.bv[hk * DH + d]);
+        outp[d] = (uint16_t)f32_to_bf16_bits(o);
+      }
     }
   }
 }
@@ -358,6 +466,7 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     return kErrBadShape;
   }
   const auto mis = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+  if (mis(a.ws_acc)) { set_last_error("%s: the Acc workspace must be 16-byte aligned", fn); return kErrBadAlign; }
   if (mis(a.pk) || mis(a.pv) || mis(a.k_u) || mis(a.v_u) || (a.spk_s % 8) || (a.spv_s % 8) || (a.spk_b % 8) || (a.spv_b % 8) || (a.spk_h % 8) || (a.spv_h % 8) ||
       (a.ldku % 8) || (a.ldvu % 8)) {
     set_last_error("%s: cache / factor pointers and strides must be 16-byte aligned", fn);
@@ -374,10 +483,26 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   const int per = (a.S + a.nsplit - 1) / a.nsplit;
   const int ks = per >= 128 ? 2 : 1;
   const bool pkl = (a.Rk % 64) == 0;               // whole 128-byte pieces of every Pk row
+  // short splits (one sub-tile per wave and pass): the deep form, whose pass over r is not a chain of load latencies
+  // (batch 1, 512 keys, rank 1024, 32 heads: 24 us per launch with chunks requested one step ahead through registers)
+  const bool deep = pkl && ks == 1;
+#define FSVD_RD_LAUNCH_T(REP_, KS_, PKL_, DEEP_, GY_)                                                                               \
+  do {                                                                                                                              \
+    constexpr int lds = RankDecodeLds<KS_, PKL_, DEEP_>::kBytes;                                                                    \
+    static bool granted = false;                                                                                                    \
+    if (!granted && lds >= 48 * 1024) {                                                                                             \
+      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_decode_partial_kernel<REP_, KS_, PKL_, DEEP_>),       \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);                                         \
+      if (ea != hipSuccess) { set_last_error("%s: cannot reserve %d bytes of LDS: %s", fn, lds, hipGetErrorString(ea)); return kErrLaunch; } \
+      granted = true;                                                                                                               \
+    }                                                                                                                               \
+    hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, PKL_, DEEP_>), dim3(a.nsplit, GY_, a.B), block, lds, st, a);          \
+  } while (0)
 #define FSVD_RD_LAUNCH(REP_, KS_, GY_)                                                                                              \
   do {                                                                                                                              \
-    if (pkl) hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, true>), dim3(a.nsplit, GY_, a.B), block, 0, st, a);          \
-    else hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, false>), dim3(a.nsplit, GY_, a.B), block, 0, st, a);             \
+    if (KS_ == 1 && deep) FSVD_RD_LAUNCH_T(REP_, 1, true, true, GY_);                                                               \
+    else if (pkl) FSVD_RD_LAUNCH_T(REP_, KS_, true, false, GY_);                                                                    \
+    else FSVD_RD_LAUNCH_T(REP_, KS_, false, false, GY_);                                                                            \
   } while (0)
   if (rep % 4 == 0) FSVD_RD_LAUNCH(4, 1, a.Hk * (rep / 4));
   else if (rep % 2 == 0) {
@@ -387,12 +512,39 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     if (ks >= 2) FSVD_RD_LAUNCH(1, 2, a.Hk * rep);
     else FSVD_RD_LAUNCH(1, 1, a.Hk * rep);
   }
+#undef FSVD_RD_LAUNCH_T
 #undef FSVD_RD_LAUNCH
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: stage 1 launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
-  hipLaunchKernelGGL(rank_decode_merge_kernel, dim3(a.H, a.B), block, 0, st, a);
+  // head-dimension slices: enough workgroups for two per compute unit, at most eight per head (16 rows each)
+  int dz = 1;
+  while (dz < 8 && (int64_t)a.H * a.B * dz < 512) dz *= 2;
+  hipLaunchKernelGGL(rank_decode_merge_kernel, dim3(a.H, a.B, dz), block, 0, st, a);
   e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: stage 2 launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+
+// One token's rank coefficients into the caches: cache[b, positions[b], :] = row b (16-byte pieces; a row whose position
+// is outside [0, S) is dropped).  One launch instead of an index tensor and two scatters.
+__global__ __launch_bounds__(256) void rankkv_append_kernel(const uint16_t* pk, int64_t ldpk, const uint16_t* pv, int64_t ldpv,
+                                                            uint16_t* pkc, int64_t spk_b, int64_t spk_s, uint16_t* pvc, int64_t spv_b,
+                                                            int64_t spv_s, const int32_t* positions, int S, int Rk, int Rv) {
+  const int b = blockIdx.x, pos = positions[b];
+  if (pos < 0 || pos >= S) return;
+  const int nk = Rk / 8, nv = Rv / 8;
+  for (int i = threadIdx.x; i < nk + nv; i += blockDim.x) {
+    if (i < nk)
+      *reinterpret_cast<u32x4_t*>(pkc + (int64_t)b * spk_b + (int64_t)pos * spk_s + i * 8) = *reinterpret_cast<const u32x4_t*>(pk + (int64_t)b * ldpk + i * 8);
+    else
+      *reinterpret_cast<u32x4_t*>(pvc + (int64_t)b * spv_b + (int64_t)pos * spv_s + (i - nk) * 8) = *reinterpret_cast<const u32x4_t*>(pv + (int64_t)b * ldpv + (i - nk) * 8);
+  }
+}
+int launch_rankkv_append(const uint16_t* pk, int64_t ldpk, const uint16_t* pv, int64_t ldpv, uint16_t* pkc, int64_t spk_b, int64_t spk_s,
+                         uint16_t* pvc, int64_t spv_b, int64_t spv_s, const int32_t* positions, int B, int S, int Rk, int Rv, hipStream_t st) {
+  hipLaunchKernelGGL(rankkv_append_kernel, dim3(B), dim3(256), 0, st, pk, ldpk, pv, ldpv, pkc, spk_b, spk_s, pvc, spv_b, spv_s, positions, S, Rk, Rv);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("fsvd_rankkv_append: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
 }
 

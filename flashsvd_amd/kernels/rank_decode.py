@@ -108,6 +108,30 @@ def rank_decode(q: torch.Tensor, pk_cache: torch.Tensor, pv_cache: torch.Tensor,
     return out
 
 
+def rankkv_append(pk: torch.Tensor, pv: torch.Tensor, pk_cache: torch.Tensor, pv_cache: torch.Tensor, positions: torch.Tensor) -> None:
+    """pk_cache[b, positions[b]] = pk[b], pv_cache[b, positions[b]] = pv[b] in one launch: the one-token case of
+    FlashSVDLegacySparseKVCache.update (runtime/cache/attn_legacy_sparse_kv.py:113-169).  pk / pv [B,R] (row views of a
+    wider buffer are fine), caches [>=B,S,R] bf16, positions int32 [B] on the device; positions outside the cache are dropped."""
+    for t, nm in ((pk, "pk"), (pv, "pv"), (pk_cache, "pk_cache"), (pv_cache, "pv_cache")):
+        if not t.is_cuda or t.dtype != torch.bfloat16:
+            raise ValueError(f"{nm} must be a bfloat16 GPU tensor")
+        if t.stride(-1) != 1:
+            raise ValueError(f"{nm} needs unit stride on the last axis")
+    B, Rk = pk.shape
+    Rv = pv.shape[1]
+    if pv.shape[0] != B or pk_cache.dim() != 3 or pv_cache.dim() != 3 or pk_cache.shape[0] < B or pv_cache.shape[0] < B:
+        raise ValueError(f"shapes do not agree: pk {tuple(pk.shape)} pv {tuple(pv.shape)} caches {tuple(pk_cache.shape)} / {tuple(pv_cache.shape)}")
+    if pk_cache.shape[2] != Rk or pv_cache.shape[2] != Rv or pk_cache.shape[1] != pv_cache.shape[1]:
+        raise ValueError(f"cache ranks / lengths do not match the rows: {tuple(pk_cache.shape)} / {tuple(pv_cache.shape)} for ranks {Rk} / {Rv}")
+    if positions.dtype != torch.int32 or positions.numel() != B or not positions.is_cuda:
+        raise ValueError(f"positions must be int32 [{B}] on the device")
+    lib = _lib.load()
+    rc = lib.fsvd_rankkv_append(pk.data_ptr(), pk.stride(0), pv.data_ptr(), pv.stride(0), pk_cache.data_ptr(), pk_cache.stride(0),
+                                pk_cache.stride(1), pv_cache.data_ptr(), pv_cache.stride(0), pv_cache.stride(1), positions.data_ptr(),
+                                B, int(pk_cache.shape[1]), Rk, Rv, stream())
+    check("fsvd_rankkv_append", rc)
+
+
 def flashsvd_attn_decode_packed(factors: DecodePackedFactors, cos_half: Optional[torch.Tensor], sin_half: Optional[torch.Tensor], *,
                                 seqlen_k: Optional[int] = None, causal: bool = True, split_k: int = 512, bn: int = 64,
                                 br: int = 64, num_warps_stage1: int = 4, num_stages_stage1: int = 2, num_warps_stage2: int = 4,
@@ -143,4 +167,4 @@ def flashsvd_attn_decode_packed(factors: DecodePackedFactors, cos_half: Optional
 
 flashsvd_attn_decode_packed_v1 = flashsvd_attn_decode_packed
 
-__all__ = ["DecodePackedFactors", "flashsvd_attn_decode_packed", "flashsvd_attn_decode_packed_v1", "rank_decode"]
+__all__ = ["DecodePackedFactors", "flashsvd_attn_decode_packed", "flashsvd_attn_decode_packed_v1", "rank_decode", "rankkv_append"]

@@ -319,7 +319,7 @@ class SVD_LlamaAttention(nn.Module):
 
     def _decode_token_rank(self, x, cache, positions, *, norm_weight=None, eps=1e-6, residual=None, rope=None):
         """Rank-space cache: append Pk, Pv (pre-RoPE coefficients) and attend with in-kernel K rebuild."""
-        from .kernels.rank_decode import rank_decode
+        from .kernels.rank_decode import rank_decode, rankkv_append
         from .quant import is_quantized
         if is_quantized(*self._factor_modules()):
             raise NotImplementedError("the rank-space cache reads bf16 head bases; int4 factors decode through the dense cache")
@@ -331,10 +331,13 @@ class SVD_LlamaAttention(nn.Module):
         if rope is None:
             rope = cache.get_rope_tables(seqlen=cache.max_cache_len, head_dim=Dh, device=x.device, dtype=x.dtype)
         p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)       # [B, rq+rk+rv]
-        rows = torch.arange(B, device=x.device)
-        pos = positions.long()
-        pkc[rows, pos] = p[:, rq:rq + rk]        # device-side scatter of the new coefficients (data movement only)
-        pvc[rows, pos] = p[:, rq + rk:]
+        if rq % 8 == 0 and rk % 8 == 0 and rv % 8 == 0 and positions.dtype == torch.int32:
+            rankkv_append(p[:, rq:rq + rk], p[:, rq + rk:], pkc, pvc, positions)      # one launch
+        else:
+            rows = torch.arange(B, device=x.device)
+            pos = positions.long()
+            pkc[rows, pos] = p[:, rq:rq + rk]    # device-side scatter of the new coefficients (data movement only)
+            pvc[rows, pos] = p[:, rq + rk:]
         cache._layer_initialized[self.layer_idx] = True
         q = hip_ops.linear(p[:, :rq], self.q_u_proj.weight).view(B, H, Dh)
         a = rank_decode(q, pkc[:B], pvc[:B], self.k_u_proj.weight, self.v_u_proj.weight, rope[0], rope[1], positions,

@@ -201,6 +201,14 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,
                             void* out, int64_t so_b, int64_t so_h,
                             int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit, float scale, void* stream);
 
+/* One decoded token per batch row into a rank-space cache: pk_cache[b, positions[b], :] = pk[b, :] and the same for pv
+ * (FlashSVDLegacySparseKVCache.update with one position per row, runtime/cache/attn_legacy_sparse_kv.py:113-169: two
+ * index_copy_ calls there; one launch here).  Caches are [B,S,R] with strides (sp*_b, sp*_s, 1); a row whose position is
+ * outside [0, S) is dropped.  bf16; ranks multiples of 8; pointers and strides 16-byte aligned. */
+int fsvd_rankkv_append(const void* pk, int64_t ldpk, const void* pv, int64_t ldpv,
+                       void* pk_cache, int64_t spk_b, int64_t spk_s, void* pv_cache, int64_t spv_b, int64_t spv_s,
+                       const int32_t* positions, int B, int S, int Rk, int Rv, void* stream);
+
 /* Full-sequence low-rank RoPE attention = the role of the fused Triton kernel flashsvd_rope_sdpa
  * (kernels/attn/prefill/rope_sdpa.py:67-248, wrapper FlashSVDRoPEAttention :254-427), as two launches:
  *

@@ -80,6 +80,40 @@ def test_packed_api_shared_and_headwise(RD):
     assert_close_bf16(outh, refh, "packed headwise")
 
 
+@pytest.mark.parametrize("B,H,Hk,L,S,R", [(1, 32, 32, 512, 560, 1024), (2, 16, 4, 333, 400, 1664), (4, 8, 8, 130, 192, 192)])
+def test_short_splits_repeat_bit_identically(RD, B, H, Hk, L, S, R):
+    """Short splits stream k_u and Pk two chunks ahead into LDS rings guarded only by the wave's load counter and a bare
+    barrier: a chunk read before it has landed, or a stage refilled while still being read, would show as a difference
+    between calls."""
+    Dh = 128
+    cos, sin = O.rope_tables(S, Dh, dtype=BF16)
+    q = rand_bf16(B, H, Dh, seed=1).cuda()
+    Pk, Pv = rand_bf16(B, S, R, seed=2).cuda(), rand_bf16(B, S, R, seed=3).cuda()
+    ku, vu = rand_bf16(Hk * Dh, R, std=R ** -0.5, seed=4).cuda(), rand_bf16(Hk * Dh, R, std=R ** -0.5, seed=5).cuda()
+    lens = torch.tensor([max(1, L - 17 * b) for b in range(B)], dtype=torch.int32).cuda()
+    first = RD.rank_decode(q, Pk, Pv, ku, vu, cos.cuda(), sin.cuda(), lens, num_kv_heads=Hk)
+    for _ in range(20):
+        assert torch.equal(RD.rank_decode(q, Pk, Pv, ku, vu, cos.cuda(), sin.cuda(), lens, num_kv_heads=Hk), first)
+
+
+def test_rankkv_append_matches_index_copy(RD):
+    B, S, Rk, Rv = 3, 40, 72, 136
+    p = rand_bf16(B, 64 + Rk + Rv, seed=1).cuda()                       # coefficients as row slices of a wider buffer
+    pkc, pvc = rand_bf16(B + 1, S, Rk, seed=2).cuda(), rand_bf16(B + 1, S, Rv, seed=3).cuda()
+    ek, ev = pkc.clone(), pvc.clone()
+    pos = torch.tensor([0, 39, 40], dtype=torch.int32).cuda()           # the last row is outside the cache: dropped
+    RD.rankkv_append(p[:, 64:64 + Rk], p[:, 64 + Rk:], pkc, pvc, pos)
+    for b in range(2):
+        ek[b, int(pos[b])] = p[b, 64:64 + Rk]
+        ev[b, int(pos[b])] = p[b, 64 + Rk:]
+    assert torch.equal(pkc, ek) and torch.equal(pvc, ev)
+    with pytest.raises(ValueError, match="int32"):
+        RD.rankkv_append(p[:, 64:64 + Rk], p[:, 64 + Rk:], pkc, pvc, pos.long())
+    from flashsvd_amd._lib import FlashSVDHipError
+    with pytest.raises(FlashSVDHipError, match="aligned"):
+        RD.rankkv_append(p[:, 60:60 + Rk], p[:, 64 + Rk:], pkc, pvc, pos)
+
+
 def test_rank_decode_rejects_unsupported(RD):
     from flashsvd_amd._lib import FlashSVDHipError
     c = lambda *s: rand_bf16(*s).cuda()
