@@ -159,15 +159,33 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
   if (!last_flag) return;
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   if (tid < DH) {
+    // the loads of eight splits are in flight at once (each comes from beyond this XCD's L2; one split per round trip
+    // made this merge a third of the kernel at eight splits); the splits are added in order
+    constexpr int SU = 8;
     float M = -INFINITY;
-    for (int i = 0; i < a.nsplit; ++i) M = fmaxf(M, ld_agent(part_ws + (int64_t)i * (DH + 2) + DH));
+    for (int i0 = 0; i0 < a.nsplit; i0 += SU) {
+      float mi[SU];
+#pragma unroll
+      for (int u = 0; u < SU; ++u) mi[u] = ld_agent(part_ws + (int64_t)min(i0 + u, a.nsplit - 1) * (DH + 2) + DH);
+#pragma unroll
+      for (int u = 0; u < SU; ++u) M = fmaxf(M, mi[u]);
+    }
     float num = 0.f, den = 0.f;
-    for (int i = 0; i < a.nsplit; ++i) {
-      const float* pw = part_ws + (int64_t)i * (DH + 2);
-      const float mi = ld_agent(pw + DH);
-      const float w = (mi == -INFINITY) ? 0.f : __expf(mi - M);
-      num += w * ld_agent(pw + tid);
-      den += w * ld_agent(pw + DH + 1);
+    for (int i0 = 0; i0 < a.nsplit; i0 += SU) {
+      float mi[SU], oi[SU], li[SU];
+#pragma unroll
+      for (int u = 0; u < SU; ++u) {
+        const float* pw = part_ws + (int64_t)min(i0 + u, a.nsplit - 1) * (DH + 2);
+        mi[u] = ld_agent(pw + DH);
+        oi[u] = ld_agent(pw + tid);
+        li[u] = ld_agent(pw + DH + 1);
+      }
+#pragma unroll
+      for (int u = 0; u < SU; ++u) {
+        const float w = (i0 + u >= a.nsplit || mi[u] == -INFINITY) ? 0.f : __expf(mi[u] - M);
+        num += w * oi[u];
+        den += w * li[u];
+      }
     }
     outp[tid] = (uint16_t)f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
   }
