@@ -190,13 +190,26 @@ __global__ __launch_bounds__(kXwThreads) void xw_gemv_kernel(XwArgs a) {
 #pragma unroll
         for (int b = 0; b < BATCH; ++b)
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            float t = 0.f;
-            for (int s = 0; s < a.ksplit; ++s)
-              t += __hip_atomic_load(tile_ws + (int64_t)s * (NW * BATCH * TN) + (w * BATCH + b) * TN + tx * 8 + i,
-                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            tot[w][b][i] = t;
-          }
+          for (int i = 0; i < 8; ++i) tot[w][b][i] = 0.f;
+      // one share at a time, all of its words in flight together (every load comes from beyond this XCD's L2; with the
+      // shares as the inner loop each word cost a round trip of its own); the shares are added in split order
+      for (int s = 0; s < a.ksplit; ++s) {
+        float sh[NW][BATCH][8];
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+#pragma unroll
+          for (int b = 0; b < BATCH; ++b)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              sh[w][b][i] = __hip_atomic_load(tile_ws + (int64_t)s * (NW * BATCH * TN) + (w * BATCH + b) * TN + tx * 8 + i,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+#pragma unroll
+          for (int b = 0; b < BATCH; ++b)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tot[w][b][i] += sh[w][b][i];
+      }
     }
     if (tid == 0) __hip_atomic_store(&a.counters[tile_id], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
