@@ -396,12 +396,16 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_merge_kernel(RankDecod
   };
   load_rows(wave * RW);
   const int64_t slot0 = ((int64_t)b * a.H + h) * a.nsplit;
-  float M = -INFINITY;
-  for (int s = 0; s < a.nsplit; ++s) M = fmaxf(M, a.ws_m[slot0 + s]);
-  float den = 0.f;
-  for (int s = 0; s < a.nsplit; ++s) {
-    const float m = a.ws_m[slot0 + s];
-    den += ((m == -INFINITY) ? 0.f : __expf(m - M)) * a.ws_l[slot0 + s];
+  // running maxima and sums of the splits: lane i of every wave takes split i (one round trip for up to 64 splits)
+  float M = -INFINITY, den = 0.f;
+  for (int s0 = 0; s0 < a.nsplit; s0 += 64) {
+    const int sidx = s0 + lane;
+    const float m = sidx < a.nsplit ? a.ws_m[slot0 + sidx] : -INFINITY;
+    const float l = sidx < a.nsplit ? a.ws_l[slot0 + sidx] : 0.f;
+    const float Mn = fmaxf(M, wave_max(m));
+    const float part = wave_sum((m == -INFINITY) ? 0.f : __expf(m - Mn) * l);
+    den = ((M == -INFINITY) ? 0.f : den * __expf(M - Mn)) + part;
+    M = Mn;
   }
   const float inv = 1.0f / fmaxf(den, 1e-20f);
   // four consecutive r per thread, the loads of up to eight splits in flight at once (one split per round trip made this
