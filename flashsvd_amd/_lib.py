@@ -77,6 +77,11 @@ SIGNATURES = {
                                          c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int,
                                          c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
                                          c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
+    "fsvd_attn_decode_densekv_static_max_bytes": (c_size_t, []),
+    "fsvd_attn_decode_densekv_static": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                                c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int,
+                                                c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
+                                                c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "fsvd_rmsnorm": (c_int, [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "fsvd_attn_decode_rankkv": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
                                         c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,

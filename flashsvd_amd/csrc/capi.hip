@@ -3,6 +3,7 @@
 #include <cstdio>
 #include <cstring>
 #include <algorithm>
+#include <mutex>
 
 #include "../../include/flashsvd_hip.h"
 #include "common.hpp"
@@ -193,6 +194,60 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h, void* k_
                    cu16(cos), cu16(sin), rope_len, u16(out), so_b, so_h, ws_part, ws_count, B, H, Hk, Dh, S, nsplit,
                    scale > 0.f ? scale : 1.0f / sqrtf((float)Dh)};
   return launch_attn_decode(a, st);
+}
+
+// ---- the same attention with library-owned scratch: nothing is allocated and no workspace is passed in -------------
+// One array per GPU (each device holds its own copy of a __device__ variable at its own address); its address is
+// looked up once per device and only that address, never the array's name, is handed to kernels.
+static constexpr size_t kStaticScratchBytes = (size_t)4 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_static_scratch[kMaxDevices] = {};
+static std::mutex g_static_scratch_mu;
+
+static int static_scratch_ptr(void** out, const char* fn) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) { set_last_error("%s: no current device", fn); return kErrLaunch; }
+  std::lock_guard<std::mutex> lock(g_static_scratch_mu);
+  if (g_static_scratch[dev] == nullptr) {
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) { set_last_error("%s: hipGetSymbolAddress failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+    g_static_scratch[dev] = p;
+  }
+  *out = g_static_scratch[dev];
+  return kOk;
+}
+
+size_t fsvd_attn_decode_densekv_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int fsvd_attn_decode_densekv_static(const void* q, int64_t sq_b, int64_t sq_h, void* k_cache, void* v_cache, int64_t sc_b,
+                                    int64_t sc_s, int64_t sc_h, const void* k_new, int64_t sk_b, int64_t sk_h, const void* v_new,
+                                    int64_t sv_b, int64_t sv_h, const int32_t* cache_seqlens, int seqlen_add, const void* cos,
+                                    const void* sin, int rope_len, void* out, int64_t so_b, int64_t so_h, int B, int H, int Hk,
+                                    int Dh, int S, int nsplit, float scale, void* stream) {
+  const char* fn = "fsvd_attn_decode_densekv_static";
+  if (B <= 0 || H <= 0 || Dh <= 0 || nsplit <= 0) { set_last_error("%s: bad shape", fn); return kErrBadShape; }
+  void* ws = nullptr;
+  size_t need = 0;
+  if (nsplit > 1) {
+    need = fsvd_attn_decode_workspace_bytes(B, H, Dh, nsplit);
+    if (need > kStaticScratchBytes) {
+      set_last_error("%s: B=%d H=%d Dh=%d nsplit=%d needs %zu bytes of scratch, the built-in array holds %zu "
+                     "(use fsvd_attn_decode_densekv with a caller-owned workspace)", fn, B, H, Dh, nsplit, need, kStaticScratchBytes);
+      return kErrWorkspace;
+    }
+    if ((size_t)B * H * sizeof(int32_t) > kAttnCounterBytes) { set_last_error("%s: B*H = %d exceeds the arrival counters", fn, B * H); return kErrBadShape; }
+    int rc = static_scratch_ptr(&ws, fn);
+    if (rc != kOk) return rc;
+    // the array keeps what the previous call left; the arrival counters of this call start at zero whatever that was
+    // (a fill kernel, not a memset node: this entry point is meant for callers under stream capture)
+    const int ncount = B * H;
+    hipLaunchKernelGGL(ws_clear_kernel, dim3((ncount + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<int32_t*>(ws), ncount);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_last_error("%s: launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
+  }
+  return fsvd_attn_decode_densekv(q, sq_b, sq_h, k_cache, v_cache, sc_b, sc_s, sc_h, k_new, sk_b, sk_h, v_new, sv_b, sv_h, cache_seqlens,
+                                  seqlen_add, cos, sin, rope_len, out, so_b, so_h, ws, need, B, H, Hk, Dh, S, nsplit, scale, stream);
 }
 
 int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, void* stream) {

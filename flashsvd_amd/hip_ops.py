@@ -293,8 +293,10 @@ def attn_decode_densekv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
                         k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
                         cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, seqlen_add: int = 0,
                         nsplit: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
-                        out: Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None) -> torch.Tensor:
-    """q [B,H,Dh] over caches [B,S,Hk,Dh]; see fsvd_attn_decode_densekv in include/flashsvd_hip.h."""
+                        out: Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None,
+                        static_scratch: bool = False) -> torch.Tensor:
+    """q [B,H,Dh] over caches [B,S,Hk,Dh]; see fsvd_attn_decode_densekv in include/flashsvd_hip.h.
+    static_scratch=True takes fsvd_attn_decode_densekv_static (the library's own fixed scratch array)."""
     _need(q, "q"); _need(k_cache, "k_cache"); _need(v_cache, "v_cache")
     _need(cache_seqlens, "cache_seqlens", dtype=torch.int32)
     if q.dim() != 3 or q.stride(2) != 1:
@@ -327,6 +329,17 @@ def attn_decode_densekv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     elif out.shape != (B, H, Dh) or out.stride(2) != 1:
         raise ValueError("out must be [B,H,Dh] with unit inner stride")
     lib = _lib.load()
+    if static_scratch:
+        # library-owned scratch: no workspace tensor, nothing allocated inside the call (out must then be given too
+        # by a caller that may not allocate)
+        rc = lib.fsvd_attn_decode_densekv_static(q.data_ptr(), q.stride(0), q.stride(1), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                 k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+                                                 _ptr(k_new), sk_b, sk_h, _ptr(v_new), sv_b, sv_h, cache_seqlens.data_ptr(),
+                                                 int(seqlen_add), _ptr(cos), _ptr(sin), rope_len, out.data_ptr(), out.stride(0),
+                                                 out.stride(1), B, H, Hk, Dh, S, int(nsplit),
+                                                 float(softmax_scale) if softmax_scale else 0.0, _stream())
+        _lib.check("fsvd_attn_decode_densekv_static", rc)
+        return out
     ws_ptr, ws_bytes = None, 0
     if nsplit > 1:
         if workspace is None:

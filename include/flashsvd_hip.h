@@ -123,6 +123,23 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h,
                              void* workspace, size_t workspace_bytes,
                              int B, int H, int Hk, int Dh, int S, int nsplit, float scale, void* stream);
 
+/* fsvd_attn_decode_densekv with the split scratch held by the library itself: no workspace argument and no device
+ * allocation anywhere in the call.  No counterpart in the reference; it exists for callers that cannot allocate
+ * or size a workspace — code under HIP stream capture, tight serving loops, harnesses that forbid hipMalloc.  The
+ * scratch is one fixed array of fsvd_attn_decode_densekv_static_max_bytes() (4 MiB) per GPU, held until the process
+ * ends; a call whose fsvd_attn_decode_workspace_bytes(B, H, Dh, nsplit) exceeds it returns FSVD_ERR_WORKSPACE.  Every
+ * call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls ordered
+ * on one stream are safe, and each call clears the arrival counters it uses before its kernels run.  Results are
+ * bit-identical to fsvd_attn_decode_densekv on the same arguments. */
+size_t fsvd_attn_decode_densekv_static_max_bytes(void);
+int fsvd_attn_decode_densekv_static(const void* q, int64_t sq_b, int64_t sq_h,
+                                    void* k_cache, void* v_cache, int64_t sc_b, int64_t sc_s, int64_t sc_h,
+                                    const void* k_new, int64_t sk_b, int64_t sk_h, const void* v_new, int64_t sv_b, int64_t sv_h,
+                                    const int32_t* cache_seqlens, int seqlen_add,
+                                    const void* cos, const void* sin, int rope_len,
+                                    void* out, int64_t so_b, int64_t so_h,
+                                    int B, int H, int Hk, int Dh, int S, int nsplit, float scale, void* stream);
+
 /* y = w * bf16(x * rsqrt(mean(x^2)+eps)) over rows of length K.
  * benchmark/mlp/bench_svd_llama_decode_graph.py:78-83. */
 int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, void* stream);
