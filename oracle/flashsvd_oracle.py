@@ -32,6 +32,12 @@ Pinning status (see tests/test_oracle_pins.py):
   pack_int4 / quantize_weight / dequantize_weight / quant_linear
                              hand-worked vectors, pack/unpack round trip, |w - dequant| <= scale/2,
                              symmetric zero point, all-zero group, fp64 closed form of the linear
+  exact mode (act_dtype=fp64) same functions on fp64 activations: equals an independent float64 restatement with
+                             numpy loops on a small block; a bf16 run stays within the bf16 rounding budget of it
+Where this restatement is deliberately finer than the reference's own torch code: ``rank_decode_attn`` keeps the
+rebuilt K (and V) tiles in fp32, while the reference's streaming function rounds each einsum result to the input
+dtype first (benchmark/attn/decode_compare.py:718-721); the absent fused kernels keep them in registers, and the
+difference (one bf16 rounding of K before the scores) is inside the decode tolerance.
 parity unpinned (source absent from the reference checkout, behaviour defined here):
   the op order / rounding points of models/llama.py (SVD_LlamaAttention.forward,
   SVD_LlamaMLP.forward) and the bit-level behaviour of flash-attn 2.8.3.
@@ -49,15 +55,25 @@ import torch.nn.functional as F
 # ----------------------------------------------------------------------------
 # primitives
 # ----------------------------------------------------------------------------
+def _ct(x: torch.Tensor) -> torch.dtype:
+    """Accumulation type: fp32, or fp64 when the activations themselves are fp64 (the exact mode below)."""
+    return torch.float64 if x.dtype == torch.float64 else torch.float32
+
+
 def lin(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``nn.Linear``: y = x @ w.T (+ bias), w is [out, in]; fp32 accumulate, one rounding.
 
     Follows the chain-of-linears reference at
     benchmark/attn/bench_real_checkpoint_decode_reconstruct.py:116-123.
+
+    Exact mode: with fp32 or fp64 activations ``x`` and the same (bf16-valued) weights the final cast is
+    a no-op, so a forward pass fed fp64 activations carries no intermediate rounding at all — the ground
+    truth that two bf16 implementations with different fp32 summation orders are both measured against.
     """
-    y = x.float() @ w.float().t()
+    ct = _ct(x)
+    y = x.to(ct) @ w.to(ct).t()
     if bias is not None:
-        y = y + bias.float()
+        y = y + bias.to(ct)
     return y.to(x.dtype)
 
 
@@ -71,9 +87,9 @@ def lowrank_pair(x: torch.Tensor, v_w: torch.Tensor, u_w: torch.Tensor) -> torch
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
     """benchmark/mlp/bench_svd_llama_decode_graph.py:78-83 (cast to input dtype, then * w)."""
-    x32 = x.float()
+    x32 = x.to(_ct(x))
     var = x32.pow(2).mean(-1, keepdim=True)
-    return weight * (x32 * torch.rsqrt(var + float(eps))).to(x.dtype)
+    return weight.to(x.dtype) * (x32 * torch.rsqrt(var + float(eps))).to(x.dtype)
 
 
 def rope_tables(seqlen: int, head_dim: int, theta: float = 10000.0,
@@ -473,9 +489,10 @@ def _attend(q, k, v, q_pos0: int) -> torch.Tensor:
     B, T, H, Dh = q.shape
     Lk, Hk = k.shape[1], k.shape[2]
     rep = H // Hk
-    qf = q.float().permute(0, 2, 1, 3).reshape(B, Hk, rep, T, Dh)
-    kf = k.float().permute(0, 2, 1, 3)
-    vf = v.float().permute(0, 2, 1, 3)
+    ct = _ct(q)
+    qf = q.to(ct).permute(0, 2, 1, 3).reshape(B, Hk, rep, T, Dh)
+    kf = k.to(ct).permute(0, 2, 1, 3)
+    vf = v.to(ct).permute(0, 2, 1, 3)
     scores = torch.einsum("bkgtd,bkld->bkgtl", qf, kf) * (1.0 / math.sqrt(Dh))
     qpos = torch.arange(T)[:, None] + q_pos0
     kpos = torch.arange(Lk)[None, :]
@@ -539,14 +556,25 @@ def block_forward(mw: ModelWeights, li: int, x: torch.Tensor, pos0: int, cache, 
 
 
 def model_forward(mw: ModelWeights, ids: torch.Tensor, pos0: int = 0, cache=None,
-                  cos=None, sin=None, last_only: bool = True, return_hidden: bool = False):
-    """embed -> blocks -> final RMSNorm -> lm_head.  utils/evaluator.py:50-82."""
+                  cos=None, sin=None, last_only: bool = True, return_hidden: bool = False,
+                  act_dtype: Optional[torch.dtype] = None, layer_inputs: Optional[list] = None):
+    """embed -> blocks -> final RMSNorm -> lm_head.  utils/evaluator.py:50-82.
+
+    ``act_dtype`` (fp32 / fp64) runs the exact mode: the stored weights and rotation tables as they are,
+    activations and caches in ``act_dtype``, no rounding between operators.  ``layer_inputs``, if a list,
+    receives the input of every block and, last, the output of the final block."""
     dtype = mw.embed.dtype
     if cos is None:
         cos, sin = rope_tables(pos0 + ids.shape[1], mw.head_dim, mw.rope_theta, dtype)
     x = mw.embed[ids]
+    if act_dtype is not None:
+        x = x.to(act_dtype)
     for li in range(len(mw.blocks)):
+        if layer_inputs is not None:
+            layer_inputs.append(x)
         x = block_forward(mw, li, x, pos0, cache, cos, sin)
+    if layer_inputs is not None:
+        layer_inputs.append(x)
     hidden = x
     xn = rms_norm(x[:, -1:] if last_only else x, mw.norm, mw.eps)
     logits = lin(xn, mw.lm_head)
@@ -554,22 +582,34 @@ def model_forward(mw: ModelWeights, ids: torch.Tensor, pos0: int = 0, cache=None
 
 
 def greedy_decode(mw: ModelWeights, prompt: torch.Tensor, n_new: int, cache_kind: str = "dense",
-                  return_hidden: bool = False, return_logits: bool = False):
+                  return_hidden: bool = False, return_logits: bool = False,
+                  act_dtype: Optional[torch.dtype] = None, forced: Optional[torch.Tensor] = None,
+                  layer_trace: Optional[list] = None):
     """Prefill yields token 0; each later token is one decode forward at
     cache_position = prompt_len + step.  scripts/demo_support/api.py:285-312,
-    benchmark/decode/check_flashsvd_decode_correctness.py:277-322."""
+    benchmark/decode/check_flashsvd_decode_correctness.py:277-322.
+
+    ``act_dtype``: exact mode (see model_forward).  ``forced`` [B, n_new]: teacher forcing — the token fed
+    at step s is ``forced[:, s-1]`` instead of this run's own argmax (the teacher-forced protocol of
+    check_flashsvd_decode_correctness.py:220-265).  ``layer_trace``, if a list, receives per decode step the
+    list of block inputs (+ the last block's output) of that step."""
     dtype = mw.embed.dtype
     B, Lp = prompt.shape
     max_len = Lp + n_new + 4
-    cache = (RankCache if cache_kind == "rank" else DenseCache)(mw, B, max_len, dtype)
+    cache = (RankCache if cache_kind == "rank" else DenseCache)(mw, B, max_len, act_dtype or dtype)
     cos, sin = rope_tables(max_len, mw.head_dim, mw.rope_theta, dtype)
-    logits, hid = model_forward(mw, prompt, 0, cache, cos, sin, return_hidden=True)
+    logits, hid = model_forward(mw, prompt, 0, cache, cos, sin, return_hidden=True, act_dtype=act_dtype)
     hiddens = [hid[:, -1]]
     all_logits = [logits[:, -1]]
     tok = logits[:, -1].float().argmax(-1, keepdim=True)
     toks = [tok]
     for step in range(n_new - 1):
-        logits, hid = model_forward(mw, tok, Lp + step, cache, cos, sin, return_hidden=True)
+        feed = tok if forced is None else forced[:, step:step + 1]
+        li = [] if layer_trace is not None else None
+        logits, hid = model_forward(mw, feed, Lp + step, cache, cos, sin, return_hidden=True, act_dtype=act_dtype,
+                                    layer_inputs=li)
+        if layer_trace is not None:
+            layer_trace.append(li)
         hiddens.append(hid[:, -1])
         all_logits.append(logits[:, -1])
         tok = logits[:, -1].float().argmax(-1, keepdim=True)

@@ -366,3 +366,175 @@ def test_int4_round_trip_error_bound_and_linear_closed_form():
     yb = O.quant_linear(xb, qw, sc, zr, group_size=32)
     wb = O.dequantize_weight(qw, sc, zr, in_features=96, group_size=32, dtype=torch.bfloat16)
     assert yb.dtype == torch.bfloat16 and torch.equal(yb, (xb.float() @ wb.float().t()).to(torch.bfloat16))
+
+
+# ---------------------------------------------------------------- argument-level pins
+def test_rope_sdpa_prefill_biases_and_additive_mask_match_sdpa():
+    """bq / bk / bv and the additive mask against torch SDPA on explicitly biased, rotated q / k / v.  The kernel
+    indexes bk and bv with the QUERY head (kernels/attn/prefill/rope_sdpa.py:176-183,229-230): under GQA two query
+    heads that share a kv head then see different keys, which an index by kv head would not reproduce."""
+    B, H, Hk, M, R, dh = 2, 4, 2, 9, 5, 8
+    rep = H // Hk
+    cos, sin = O.rope_tables(M, dh)
+    Pq, Pk, Pv = _rand(B, H, M, R, seed=11), _rand(B, Hk, M, R, seed=12), _rand(B, Hk, M, R, seed=13)
+    Vq, Vk, Vv = _rand(H, R, dh, seed=14), _rand(Hk, R, dh, seed=15), _rand(Hk, R, dh, seed=16)
+    bq, bk, bv = _rand(H * dh, seed=17), _rand(H * dh, seed=18), _rand(H * dh, seed=19)
+    add = _rand(B, 1, M, M, seed=20)
+    out = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin, bq=bq, bk=bk, bv=bv, add_mask=add)
+
+    d64 = torch.float64
+    c, s = cos.to(d64), sin.to(d64)
+
+    def rot(x):   # [M, dh] rotate-half, written out per pair
+        y = torch.empty_like(x)
+        for i in range(dh // 2):
+            y[:, i] = x[:, i] * c[:, i] - x[:, i + dh // 2] * s[:, i]
+            y[:, i + dh // 2] = x[:, i] * s[:, i] + x[:, i + dh // 2] * c[:, i]
+        return y
+
+    ref = torch.empty(B, M, H, dh, dtype=d64)
+    causal = torch.full((M, M), -float("inf"), dtype=d64).triu(1)
+    for b in range(B):
+        for h in range(H):
+            hk = h // rep
+            q = rot(Pq[b, h].to(d64) @ Vq[h].to(d64) + bq[h * dh:(h + 1) * dh].to(d64))
+            k = rot(Pk[b, hk].to(d64) @ Vk[hk].to(d64) + bk[h * dh:(h + 1) * dh].to(d64))
+            v = Pv[b, hk].to(d64) @ Vv[hk].to(d64) + bv[h * dh:(h + 1) * dh].to(d64)
+            ref[b, :, h] = torch.nn.functional.scaled_dot_product_attention(
+                q[None], k[None], v[None], attn_mask=(causal + add[b, 0].to(d64))[None])[0]
+    assert torch.allclose(out.to(d64), ref, atol=2e-5)
+    # a bias indexed by kv head would make heads 0 and 1 (same kv head) share keys: they must not
+    bk2 = bk.clone()
+    bk2[dh:2 * dh] += 1.0          # query head 1 only
+    out2 = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin, bq=bq, bk=bk2, bv=bv, add_mask=add)
+    assert torch.allclose(out2[:, :, 0], out[:, :, 0], atol=1e-6) and torch.allclose(out2[:, :, 2:], out[:, :, 2:], atol=1e-6)
+    assert not torch.allclose(out2[:, :, 1], out[:, :, 1], atol=1e-3)
+    # the additive mask alone (no biases) against SDPA as well
+    out3 = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin, add_mask=add)
+    q = O.apply_rope_fp32(torch.einsum("bhmr,hrd->bhmd", Pq, Vq), cos[None, None], sin[None, None])
+    k = O.apply_rope_fp32(torch.einsum("bhmr,hrd->bhmd", Pk, Vk), cos[None, None], sin[None, None])
+    v = torch.einsum("bhmr,hrd->bhmd", Pv, Vv)
+    ref3 = torch.nn.functional.scaled_dot_product_attention(
+        q, k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1), attn_mask=causal.float()[None, None] + add)
+    assert torch.allclose(out3, ref3.permute(0, 2, 1, 3), atol=1e-5)
+
+
+def _bf(x):
+    """One rounding to bf16, result held in float64 (inputs far inside the fp32 range)."""
+    return x.to(torch.float32).to(torch.bfloat16).to(torch.float64)
+
+
+def test_dual_split_bf16_rounding_points_v1_workspace_and_v3():
+    """The bf16 rounding points of the v1 (workspace dtype) and v3 (per-tile s) variants against a float64 restatement
+    with every rounding written out.  Operands are small multiples of 1/8 so that every fp32 partial sum is exact and
+    a rounding applied at the wrong place (or left out) changes bits; only silu involves a transcendental."""
+    bf = torch.bfloat16
+    B, L, R, D, Hd, BD, BR2 = 2, 1, 8, 24, 6, 8, 4
+    g = torch.Generator().manual_seed(77)
+
+    def grid(*shape, span=8):
+        return (torch.randint(-span, span + 1, shape, generator=g).float() / 8).to(bf)
+
+    PUp, PGate = grid(B, L, R), grid(B, L, R)
+    GateU, UpU, DownV, DownU, b2 = grid(R, D), grid(R, D), grid(D, R), grid(R, Hd), grid(Hd)
+    d64 = torch.float64
+    gg = PGate.reshape(B, R).to(d64) @ GateU.to(d64)
+    uu = PUp.reshape(B, R).to(d64) @ UpU.to(d64)
+    h = _bf((gg / (1 + torch.exp(-gg))) * uu)                       # dual_split_triton.py:207
+    tiles = [h[:, d0:d0 + BD] @ DownV[d0:d0 + BD].to(d64) for d0 in range(0, D, BD)]
+    # v1, partials through a bf16 workspace, then .sum(1) (bf16 result), then the DownU product (:586-624)
+    S_v1_bf = _bf(sum(_bf(t) for t in tiles))
+    y_v1_bf = _bf(S_v1_bf @ DownU.to(d64) + b2.to(d64))
+    # v1 with fp32 partials / v2: fp32 sum, one rounding of S (:686-721)
+    S_f32 = _bf(sum(tiles))
+    y_f32 = _bf(S_f32 @ DownU.to(d64) + b2.to(d64))
+    got_bf = O.dual_split_mlp(PUp, PGate, GateU, UpU, DownV, DownU, b2, BD=BD, variant="v1", work_dtype=bf)
+    got_f32 = O.dual_split_mlp(PUp, PGate, GateU, UpU, DownV, DownU, b2, BD=BD, variant="v1", work_dtype=torch.float32)
+    got_v2 = O.dual_split_mlp(PUp, PGate, GateU, UpU, DownV, DownU, b2, BD=BD, variant="v2")
+    assert torch.equal(got_bf.reshape(B, Hd).to(d64), y_v1_bf)
+    assert torch.equal(got_f32.reshape(B, Hd).to(d64), y_f32)
+    assert torch.equal(got_v2.reshape(B, Hd).to(d64), y_f32)
+    assert not torch.equal(y_v1_bf, y_f32), "operands too tame: the workspace rounding changes nothing"
+    # v3: s per (D tile, BR2 slice) rounded to bf16, Y summed in fp32, rounded once, b2 added afterwards in bf16 (:427-532,858-966)
+    Y = torch.zeros(B, Hd, dtype=d64)
+    for d0 in range(0, D, BD):
+        for r0 in range(0, R, BR2):
+            s = _bf(h[:, d0:d0 + BD] @ DownV[d0:d0 + BD, r0:r0 + BR2].to(d64))
+            Y += s @ DownU[r0:r0 + BR2].to(d64)
+    y_v3 = _bf(_bf(Y) + b2.to(d64))
+    got_v3 = O.dual_split_mlp_v3(PUp, PGate, GateU, UpU, DownV, DownU, b2, BD=BD, BR2=BR2)
+    assert torch.equal(got_v3.reshape(B, Hd).to(d64), y_v3)
+    assert not torch.equal(y_v3, y_f32)
+
+
+def test_exact_mode_matches_float64_restatement_and_bounds_the_bf16_run():
+    """The exact mode (fp64 activations, stored bf16 weights, no rounding between operators) against an independent
+    float64 restatement of one block written with numpy and explicit loops over heads and positions; the bf16 run of
+    the same block must then sit within a few bf16 roundings of it."""
+    mw = _tiny(torch.bfloat16, n_layers=1, kvh=2)
+    T, d, H, Hk, Dh = 5, 32, 4, 2, 8
+    x = _rand(1, T, d, seed=9).to(torch.bfloat16)
+    cos, sin = O.rope_tables(T, Dh, dtype=torch.bfloat16)
+    got = O.block_forward(mw, 0, x.double(), 0, None, cos, sin)[0].numpy()
+    assert got.dtype == np.float64
+    b = mw.blocks[0]
+    W = {k: getattr(b, k).double().numpy() for k in ("q_v", "q_u", "k_v", "k_u", "v_v", "v_u", "o_v", "o_u", "gate_v", "gate_u",
+                                                      "up_v", "up_u", "down_v", "down_u", "ln1", "ln2")}
+    xn = x[0].double().numpy()
+    c, s = cos.double().numpy(), sin.double().numpy()
+
+    def rms(v, w):
+        return w * (v / np.sqrt((v * v).mean(-1, keepdims=True) + mw.eps))
+
+    def rope(v, t):     # v [Dh]
+        half = Dh // 2
+        out = np.empty(Dh)
+        for i in range(half):
+            out[i] = v[i] * c[t, i] - v[i + half] * s[t, i]
+            out[i + half] = v[i + half] * c[t, i] + v[i] * s[t, i]
+        return out
+
+    h1 = rms(xn, W["ln1"])
+    q = (h1 @ W["q_v"].T) @ W["q_u"].T
+    k = (h1 @ W["k_v"].T) @ W["k_u"].T
+    v = (h1 @ W["v_v"].T) @ W["v_u"].T
+    attn = np.zeros((T, H * Dh))
+    for t in range(T):
+        for hh in range(H):
+            hk = hh // (H // Hk)
+            qt = rope(q[t, hh * Dh:(hh + 1) * Dh], t)
+            sc = np.array([qt @ rope(k[n, hk * Dh:(hk + 1) * Dh], n) for n in range(t + 1)]) / math.sqrt(Dh)
+            p = np.exp(sc - sc.max())
+            p /= p.sum()
+            attn[t, hh * Dh:(hh + 1) * Dh] = sum(p[n] * v[n, hk * Dh:(hk + 1) * Dh] for n in range(t + 1))
+    x2 = xn + (attn @ W["o_v"].T) @ W["o_u"].T
+    h2 = rms(x2, W["ln2"])
+    gg = (h2 @ W["gate_v"].T) @ W["gate_u"].T
+    uu = (h2 @ W["up_v"].T) @ W["up_u"].T
+    ref = x2 + (((gg / (1 + np.exp(-gg))) * uu) @ W["down_v"].T) @ W["down_u"].T
+    assert np.allclose(got, ref, rtol=1e-11, atol=1e-12)
+    # fp32 activations: the same up to fp32 accumulation noise
+    got32 = O.block_forward(mw, 0, x.float(), 0, None, cos, sin)[0].double().numpy()
+    assert np.abs(got32 - ref).max() <= 1e-5 * np.abs(ref).max()
+    # the bf16 run differs from the exact one, by bf16 roundings only
+    got16 = O.block_forward(mw, 0, x, 0, None, cos, sin)[0].double().numpy()
+    err = np.abs(got16 - ref).max() / np.abs(ref).max()
+    assert 1e-4 < err < 3e-2, err
+
+
+def test_teacher_forced_decode_and_layer_trace():
+    """forced= feeds the given tokens; with a run's own tokens it reproduces that run; layer_trace returns every
+    block's input, chained by block_forward."""
+    mw = _tiny(torch.float32)
+    prompt = torch.randint(0, 50, (1, 6), generator=torch.Generator().manual_seed(8))
+    toks, hid, _, logits = O.greedy_decode(mw, prompt, 5, return_logits=True)
+    trace = []
+    toks2, hid2, cache2, logits2 = O.greedy_decode(mw, prompt, 5, return_logits=True, forced=toks, layer_trace=trace)
+    assert torch.equal(toks, toks2) and torch.equal(logits, logits2)
+    assert len(trace) == 4 and all(len(t) == len(mw.blocks) + 1 for t in trace)
+    assert torch.equal(trace[2][0][0, 0], mw.embed[toks[0, 2]])
+    assert torch.equal(trace[2][-1][:, -1], hid[:, 3])
+    other = (toks + 7) % 50
+    toks3, _, _, _ = O.greedy_decode(mw, prompt, 5, return_logits=True, forced=other)
+    seq = torch.cat([prompt, other[:, :1]], 1)
+    assert int(O.model_forward(mw, seq)[0, -1].argmax()) == int(toks3[0, 1])
