@@ -174,11 +174,16 @@ def _manual_llama_decode_step(model, input_ids: torch.Tensor, *, past_key_values
 def _build_generation_cache(model, *, prompt_len: int, max_new_tokens: int, batch_size: int, device):
     """(cache, use_manual_decode).  The dense FlashSVD cache is used when the dense-attention decode
     route or the dense-KV baseline is switched on; this build has no other cache for its modules."""
-    from .runtime.cache import FlashSVDV15DenseKVCache
+    from .runtime.cache import FlashSVDLegacySparseKVCache, FlashSVDV15DenseKVCache
     dtype = next(iter(model.parameters())).dtype
     use_flash = _env_truthy("FLASH_SVD_ENABLE_DENSE_ATTN_DECODE") and not _env_truthy("SVDLLM_FLASH_FALLBACK")
-    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=int(batch_size),
-                                    max_cache_len=int(prompt_len) + int(max_new_tokens) + 4, device=device, dtype=dtype)
+    # the rank-space cache when the checkpoint asks for it (config side channel written by the loader,
+    # utils/model_utils.py:438-439) or the rank-space baseline switch is on (utils/evaluator.py:418-456)
+    use_rank = (bool(getattr(model.config, "flash_svd_use_lowrank_cache", False)) or _env_truthy("FLASH_SVD_BASELINE_LR_KVCACHE")) \
+        and not use_flash
+    kind = FlashSVDLegacySparseKVCache if use_rank else FlashSVDV15DenseKVCache
+    cache = kind(model.config, max_batch_size=int(batch_size), max_cache_len=int(prompt_len) + int(max_new_tokens) + 4,
+                 device=device, dtype=dtype)
     return cache, bool(use_flash)
 
 
@@ -238,6 +243,8 @@ def generate_text(model, tokenizer, *, prompt: str, max_new_tokens: int = 64, de
             out = _manual_llama_decode_step(model, next_token, past_key_values=cache,
                                             cache_position=torch.tensor([prompt_len + step]))
             next_token = _sample_next_token(out.logits[:, -1, :], **sample)
+    if pdec is not None:
+        pdec.check()      # a step that gave up waiting leaves stale token ids behind: raise instead of returning them
     completion = output_ids[prompt_len:]
     return {"prompt_token_count": prompt_len, "generated_token_count": len(completion), "output_ids": output_ids,
             "completion_ids": completion, "text": tokenizer.decode(output_ids, skip_special_tokens=False),
@@ -247,16 +254,25 @@ def generate_text(model, tokenizer, *, prompt: str, max_new_tokens: int = 64, de
 @torch.no_grad()
 def decode_kvcache_eval(model, *, prompt_len: int = 2048, new_tokens: int = 128, batch_size: int = 1, device: str = "cuda",
                         warmup: int = 5, max_cache_len: Optional[int] = None, lowrank_cache: bool = False,
-                        flashsvd_dense_cache: bool = True, baseline_dense_kvcache: bool = False, use_graph: bool = True,
+                        flashsvd_dense_cache: Optional[bool] = None, baseline_dense_kvcache: bool = False, use_graph: bool = True,
                         profile_decode: bool = False, profile_decode_steps: int = 20) -> dict:
     """Prefill a random prompt, run `warmup` untimed decode tokens, then time `new_tokens` tokens
-    between two device synchronisations.  Result keys follow the reference's dict."""
+    between two device synchronisations.  Result keys follow the reference's dict.
+
+    Cache choice as in utils/evaluator.py:352-388: ``lowrank_cache`` decodes over the rank-space cache
+    (FlashSVDLegacySparseKVCache: per-layer, possibly unequal q/k/v ranks, shaped at the first write), otherwise the
+    dense cache (this build has no third, HF-static one, so ``flashsvd_dense_cache`` left unset means "dense unless
+    lowrank_cache").  Two modes switched on together raise, as there."""
     from .graphs import GraphedDecoder
-    from .runtime.cache import FlashSVDV15DenseKVCache
-    if lowrank_cache:
-        raise NotImplementedError("the rank-space cache is driven through flashsvd_amd.kernels.rank_decode, not this loop")
-    if sum(map(bool, (lowrank_cache, flashsvd_dense_cache, baseline_dense_kvcache))) > 1:
-        raise ValueError("cache modes are mutually exclusive.")
+    from .runtime.cache import FlashSVDLegacySparseKVCache, FlashSVDV15DenseKVCache
+    if flashsvd_dense_cache is None:
+        flashsvd_dense_cache = not (lowrank_cache or baseline_dense_kvcache)
+    if lowrank_cache and flashsvd_dense_cache:
+        raise ValueError("lowrank_cache and flashsvd_dense_cache are mutually exclusive.")
+    if lowrank_cache and baseline_dense_kvcache:
+        raise ValueError("lowrank_cache and baseline_dense_kvcache are mutually exclusive.")
+    if flashsvd_dense_cache and baseline_dense_kvcache:
+        raise ValueError("flashsvd_dense_cache and baseline_dense_kvcache are mutually exclusive.")
     model.eval()
     dev = torch.device(device)
     if max_cache_len is None:
@@ -264,7 +280,8 @@ def decode_kvcache_eval(model, *, prompt_len: int = 2048, new_tokens: int = 128,
     dtype = next(iter(model.parameters())).dtype
     vocab = int(getattr(model.config, "vocab_size", 32000))
     input_ids = torch.randint(0, vocab, (int(batch_size), int(prompt_len)), device=dev, dtype=torch.long)
-    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=int(batch_size), max_cache_len=int(max_cache_len), device=dev, dtype=dtype)
+    kind = FlashSVDLegacySparseKVCache if lowrank_cache else FlashSVDV15DenseKVCache
+    cache = kind(model.config, max_batch_size=int(batch_size), max_cache_len=int(max_cache_len), device=dev, dtype=dtype)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     out = model(input_ids=input_ids, past_key_values=cache, cache_position=torch.arange(int(prompt_len)), logits_to_keep=1)

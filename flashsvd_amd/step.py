@@ -51,6 +51,17 @@ class PersistentDecoder:
         dev = model.lm_head.weight.device
         if model.lm_head.weight.dtype != torch.bfloat16:
             raise ValueError("PersistentDecoder is bf16 only")
+        # the kernel reinterprets every buffer it is pointed at as bf16 bits (int4 factors aside): refuse anything else
+        # here, so that the driver falls back to the per-operator engine instead of decoding garbage
+        if getattr(cache, "_dtype", torch.bfloat16) != torch.bfloat16:
+            raise ValueError(f"PersistentDecoder needs a bfloat16 KV cache, got {cache._dtype} "
+                             "(FlashSVDV15DenseKVCache defaults to float16: pass dtype=torch.bfloat16)")
+        if inner.embed_tokens.weight.dtype != torch.bfloat16 or inner.norm.weight.dtype != torch.bfloat16:
+            raise ValueError("PersistentDecoder needs a bfloat16 embedding table and final norm")
+        for li, layer in enumerate(inner.layers):
+            for nm, p_ in layer.named_parameters():
+                if p_.is_floating_point() and p_.dtype != torch.bfloat16:
+                    raise ValueError(f"PersistentDecoder needs bfloat16 weights; layer {li} {nm} is {p_.dtype}")
         self.nwg = int(lib.fsvd_decode_step_workgroups())
         if self.nwg <= 0:
             raise RuntimeError("fsvd_decode_step_workgroups: cannot query the device")
@@ -122,6 +133,12 @@ class PersistentDecoder:
 
         def sz_words(scales, zeros):
             """uint32 [N, G]: fp16 scale bits in the low half, zero point + 128 in the high half (what a piece needs in one load)."""
+            if scales.dtype != torch.float16:
+                raise ValueError(f"int4 scales must be float16, got {scales.dtype}")
+            zmin, zmax = int(zeros.min()), int(zeros.max())
+            if zmin < -128 or zmax > 65535 - 128:
+                raise ValueError(f"int4 zero points {zmin}..{zmax} do not fit the unsigned 16-bit field of the packed "
+                                 "scale | zero word (zero + 128)")
             lo = scales.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
             hi = (zeros.to(torch.int32) + 128) << 16
             return (lo | hi).contiguous()

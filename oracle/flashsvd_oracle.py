@@ -476,6 +476,17 @@ def make_model(*, d: int, n_heads: int, n_kv_heads: int, head_dim: int, ffn: int
                                   n_layers=n_layers, seed=seed, std=std))
 
 
+def hold_weights_as(mw: ModelWeights, dtype: torch.dtype) -> ModelWeights:
+    """The same model with every factor and the lm_head held in ``dtype`` (values unchanged: widening bf16 is exact).
+    The embedding and the norm weights keep their dtype, which is what names the activation dtype.  Results are
+    bit-identical to those of ``mw``; the per-call widening of every weight is what goes away (decode steps of a deep
+    model are several times faster on the host)."""
+    import dataclasses
+    blocks = [BlockWeights(**{f.name: (getattr(b, f.name) if f.name in ("ln1", "ln2") else getattr(b, f.name).to(dtype))
+                              for f in dataclasses.fields(BlockWeights)}) for b in mw.blocks]
+    return dataclasses.replace(mw, blocks=blocks, lm_head=mw.lm_head.to(dtype))
+
+
 def mlp_forward(bw: BlockWeights, h2: torch.Tensor) -> torch.Tensor:
     """Chain-of-linears SwiGLU: down(silu(gate(x)) * up(x)), every op rounded in dtype.
     src/legacy/FlashSVD-V1/decoders/llama/profile_asvd_llama_decode.py:311-314."""

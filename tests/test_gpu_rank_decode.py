@@ -151,3 +151,47 @@ def test_model_rank_cache_greedy_matches_oracle_rank_cache():
         same += int(torch.equal(nxt, ref_tok[:, s:s + 1]))
         dec.tokens.copy_(ref_tok[:, s:s + 1])
     assert same >= n_new - 2, f"only {same}/{n_new} teacher-forced tokens identical"
+
+
+def test_decode_driver_serves_the_rank_space_cache(monkeypatch):
+    """decode_kvcache_eval(lowrank_cache=True) (utils/evaluator.py:358-371) decodes over FlashSVDLegacySparseKVCache through
+    the per-operator graph engine, with per-layer and unequal q/k/v ranks; generate_text takes the same cache when the
+    checkpoint's config asks for it, and then produces the oracle's rank-cache tokens."""
+    from flashsvd_amd import api, llama
+    from types import SimpleNamespace
+    monkeypatch.setenv("FLASHSVD_AMD_DECODE_ENGINE", "auto")
+    cfg = SimpleNamespace(hidden_size=256, num_attention_heads=2, num_key_value_heads=2, head_dim=128, intermediate_size=512,
+                          num_hidden_layers=2, vocab_size=500, rope_theta=10000.0, rms_norm_eps=1e-6, hidden_act="silu",
+                          max_position_embeddings=256)
+    with torch.device("meta"):
+        hetero = llama.SVDLlamaForCausalLM(cfg, attn_ranks=dict(q=64, k=40, v=72, o=64), mlp_rank=96)
+    hetero = llama.materialize(hetero, "cuda", BF16, seed=1, std=0.05)
+    r = api.decode_kvcache_eval(hetero, prompt_len=33, new_tokens=5, warmup=2, batch_size=2, lowrank_cache=True)
+    assert r["lowrank_cache"] and not r["flashsvd_dense_cache"] and r["decode_engine"] == "graph" and r["decode_tok_s"] > 0
+    with pytest.raises(ValueError, match="mutually exclusive"):
+        api.decode_kvcache_eval(hetero, prompt_len=8, new_tokens=1, warmup=0, lowrank_cache=True, flashsvd_dense_cache=True)
+
+    mw = O.make_model(d=256, n_heads=2, n_kv_heads=2, head_dim=128, ffn=512, attn_rank=64, mlp_rank=96, n_layers=2,
+                      vocab=500, dtype=BF16, seed=5, std=0.05)
+    model = model_from_oracle(mw)
+    model.config.flash_svd_use_lowrank_cache = True
+    prompt = torch.randint(0, 500, (1, 21), generator=torch.Generator().manual_seed(4))
+
+    class Tok:
+        eos_token_id = None
+        pad_token_id = 0
+
+        def __call__(self, text, return_tensors="pt", add_special_tokens=False):
+            return {"input_ids": prompt}
+
+        def decode(self, ids, skip_special_tokens=False):
+            return " ".join(map(str, ids))
+
+    out = api.generate_text(model, Tok(), prompt="x", max_new_tokens=6, use_graph=True)
+    ref_tok, _, _, ref_logits = O.greedy_decode(mw, prompt, 6, "rank", return_logits=True)
+    got, ref = out["completion_ids"], ref_tok[0].tolist()
+    same = next((s for s in range(6) if got[s] != ref[s]), 6)
+    if same < 6:    # the first differing token must be a near-tie in the oracle (rank path: fp32 K rebuild, V applied in rank space)
+        lo = ref_logits[0, same].float()
+        assert float(lo[ref[same]] - lo[got[same]]) <= 2e-2 * float(lo.abs().max()), f"{got} vs {ref}"
+    assert same >= 3, f"{got} vs {ref}"
