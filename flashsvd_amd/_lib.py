@@ -42,7 +42,7 @@ class Phase(ctypes.Structure):
                 ("plain_out", c_void_p),
                 ("inp", TagBuf), ("aux0", TagBuf), ("aux1", TagBuf), ("out0", TagBuf),
                 ("qsz", c_void_p * 2), ("ldg", ctypes.c_int32), ("gshift", ctypes.c_int32), ("wbits", ctypes.c_int32),
-                ("rsv0", ctypes.c_int32),
+                ("shared_in", ctypes.c_int32),
                 ("share_q", ctypes.c_int32), ("share_r", ctypes.c_int32), ("m_kp", ctypes.c_uint32), ("dk", ctypes.c_int32)]
 
 

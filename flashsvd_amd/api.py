@@ -163,9 +163,11 @@ def _manual_llama_decode_step(model, input_ids: torch.Tensor, *, past_key_values
             out = out[0]
         hidden = out
     norm = inner.norm
-    if hasattr(model, "decode_step"):   # fused final norm + lm_head
-        from . import hip_ops
-        logits = hip_ops.linear(hidden[:, -1:, :], model.lm_head.weight, norm_weight=norm.weight, eps=norm.variance_epsilon)
+    head_w = getattr(model.lm_head, "weight", None)
+    if head_w is not None and head_w.is_cuda and head_w.dtype == torch.bfloat16 and hidden.dtype == torch.bfloat16 \
+            and getattr(model.lm_head, "bias", None) is None and hasattr(norm, "variance_epsilon"):
+        from . import hip_ops   # fused final norm + lm_head
+        logits = hip_ops.linear(hidden[:, -1:, :], head_w, norm_weight=norm.weight, eps=norm.variance_epsilon)
     else:
         logits = model.lm_head(norm(hidden)[:, -1:, :])
     return SimpleNamespace(logits=logits, past_key_values=past_key_values)
@@ -431,12 +433,14 @@ def format_decode_profile(profile: dict, topk: int = 10) -> list[str]:
 
 
 def enable_flashsvd_llama_layer_tail_cuda_graph() -> None:
-    """Process-global, idempotent switch: decoder layers of this package run "residual +
-    post-attention norm + MLP + residual" as one captured graph when FLASH_SVD_MLP_CUDA_GRAPH is on
-    with scope layer_tail (the role of the patch of the same name in the reference, called from
-    utils/model_utils.py:768-786)."""
+    """Process-global and idempotent, like the patch of the same name in the reference (called from
+    utils/model_utils.py:768-786 and benchmark/mlp/bench_svd_llama_decode_graph.py:227): transformers'
+    LlamaDecoderLayer, used unmodified with SVD_LlamaMLP (and SVD_LlamaAttention) swapped in, and this package's own
+    decoder layer run "residual + post-attention norm + MLP + residual" as one captured graph when
+    FLASH_SVD_MLP_CUDA_GRAPH is on with scope layer_tail (or auto)."""
     from . import llama
     llama.LAYER_TAIL_GRAPH_ENABLED = True
+    llama.patch_hf_llama_decoder_layer()
 
 
 __all__ = ["cast_model_for_inference", "configure_runtime", "decode_kvcache_eval", "generate_text", "runtime_env_snapshot",

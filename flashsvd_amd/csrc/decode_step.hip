@@ -142,6 +142,7 @@ __device__ __forceinline__ uint64_t desc_u64(uint32_t dv, int word) {
 // ---------------------------------------------------------------------------------------------
 struct GemvCtx {
   int K, kp, nmat, r0, srows, pps, nsteps, dk;
+  int xk;                    // staged elements between the inputs of matrix 0 and matrix 1 (K, or 0 when they share one input)
   uint64_t base0, base1;     // byte addresses of the slab in matrix 0 / 1
   int q4, ldg, gshift;       // int4 weights: a piece is 32 columns; scale | zero words [N, ldg], group = 32 << gshift columns
   uint64_t sz0, sz1;         // byte addresses of the slab's scale | zero rows
@@ -152,6 +153,7 @@ __device__ __forceinline__ void gemv_ctx(uint32_t dv, int w, GemvCtx& c) {
   c.q4 = Q4 && DF_I(dv, wbits) == 4;
   c.kp = c.q4 ? c.K >> 5 : c.K >> 3;
   c.nmat = DF_I(dv, nmat);
+  c.xk = DF_I(dv, shared_in) ? 0 : c.K;
   const int q = DF_I(dv, share_q), r = DF_I(dv, share_r);
   c.r0 = w * q + min(w, r);
   c.srows = q + (w < r ? 1 : 0);
@@ -220,7 +222,7 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
     for (int u = 0; u < kU; ++u) {
       if (s0 + u / NMAT >= c.nsteps) break;     // the rest of the window lies past the slab (uniform)
       const int mat = u % NMAT;
-      int xo = mat * c.K + kofs * 8;
+      int xo = mat * c.xk + kofs * 8;
       if (GROUPED) xo += ((row >= g1 ? 1 : 0) + (row >= g2 ? 1 : 0)) * c.K;
       const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xs + xo);
       d[u] = dot8_bf16(R[u], xv, 0.f);
@@ -295,7 +297,7 @@ __device__ __forceinline__ void gemv_stream_q4(const GemvCtx& c, uint32_t m_kp, 
     for (int u = 0; u < kU; ++u) {
       if (s0 + u / NMAT >= c.nsteps) break;     // the rest of the window lies past the slab (uniform)
       const int mat = u % NMAT;
-      int sel = mat;
+      int sel = c.xk ? mat : 0;
       if (GROUPED) sel += (c.r0 + lrow >= g1 ? 1 : 0) + (c.r0 + lrow >= g2 ? 1 : 0);
       const float dp = dot32_q4(R[u], reinterpret_cast<const u32x4_t*>(xs + sel * c.K + kofs * 32));
       const uint32_t sz = sztab[mat * szper + min(lrow, c.srows - 1) * c.ldg + (kofs >> c.gshift)];
@@ -556,7 +558,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       const int epi = DF_I(dv, epilogue);
       if (epi == FSVD_EP_RESID && (tid >> 3) < gc.srows) resid = ld_coh32(DF_P(dv, aux0), gc.r0 + (tid >> 3));
       const int gH = DF_I(dv, H);                 // > 0: rows are q | k | v groups with their own inputs
-      const int in_len = (gH > 0 ? 3 : gc.nmat) * gc.K;
+      const int in_len = (gH > 0 ? 3 : (gc.xk ? gc.nmat : 1)) * gc.K;
       const uint32_t tin = DF_TAG16(dv, in, epoch);
       const uint32_t* nw = static_cast<const uint32_t*>(DF_P(dv, norm_w));
       bool ok;
@@ -938,8 +940,10 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
           if (d.Hk <= 0 || d.Dh <= 0 || d.N != (d.H + 2 * d.Hk) * d.Dh) return bad("grouped GEMV needs N = (H + 2*Hk) * Dh", p);
           if (3 * d.K > kMaxIn) return bad("input vector longer than the staging buffer", p);
         }
-        if (d.nmat * d.K > kMaxIn) return bad("input vector longer than the staging buffer", p);
-        if (d.norm_w && d.nmat * d.K > kT * 12 * 2) return bad("normalised input too long for one staging round", p);
+        if (d.shared_in != 0 && (d.nmat != 2 || d.H > 0)) return bad("shared_in is for a pair of matrices over one input", p);
+        const int n_in = d.shared_in ? 1 : d.nmat;
+        if (n_in * d.K > kMaxIn) return bad("input vector longer than the staging buffer", p);
+        if (d.norm_w && n_in * d.K > kT * 12 * 2) return bad("normalised input too long for one staging round", p);
         const int64_t rows = ((int64_t)d.N + nwg - 1) / nwg;
         if (rows * d.nmat * (d.K / (q4 ? 256 : 128)) > kMaxChunks) return bad("too many rows per workgroup for the partial buffer", p);
         if ((d.epilogue == FSVD_EP_SWIGLU) != (d.nmat == 2)) return bad("SwiGLU epilogue needs exactly two matrices", p);
@@ -959,8 +963,10 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         if (d.H <= 0 || d.Hk <= 0 || d.H % d.Hk != 0) return bad("bad head counts", p);
         if (d.nsplit <= 0 || d.H * d.nsplit != nwg) return bad("H * nsplit must equal the workgroup count", p);
         if (!d.in.ptr || !d.out0.ptr || !d.k_cache || !d.v_cache) return bad("attention needs in = [q|k|v], out0 and the caches", p);
+        // the producer is the grouped head expansion (H > 0, same geometry) or a plain GEMV of that many rows (a dense
+        // [q; k; v] projection)
         if (p == 0 || ph[p - 1].type != FSVD_PH_GEMV || ph[p - 1].epilogue != FSVD_EP_STORE || ph[p - 1].N != (d.H + 2 * d.Hk) * d.Dh ||
-            ph[p - 1].H != d.H || ph[p - 1].Hk != d.Hk || ph[p - 1].Dh != d.Dh)
+            (ph[p - 1].H != 0 && (ph[p - 1].H != d.H || ph[p - 1].Hk != d.Hk || ph[p - 1].Dh != d.Dh)))
           return bad("attention must follow the GEMV that writes (H + 2*Hk) * Dh values of q, k, v", p);
         if ((d.cos == nullptr) != (d.sin == nullptr) || (d.cos && d.rope_len <= 0)) return bad("rope tables incomplete", p);
         if ((d.sc_s % 8) || (d.sc_h % 8) || (reinterpret_cast<uintptr_t>(d.k_cache) & 15) || (reinterpret_cast<uintptr_t>(d.v_cache) & 15))

@@ -10,6 +10,7 @@ from typing import Optional
 import torch
 
 from . import _lib
+from .torch_ops import ops as _OPS
 
 _BF16 = torch.bfloat16
 
@@ -78,7 +79,14 @@ def release_split_workspace(device: Optional[torch.device] = None) -> None:
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
            norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
            residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:
-    """out = (residual +) linear(rmsnorm?(x), weight, bias); weight is nn.Linear layout [N, K]."""
+    """out = (residual +) linear(rmsnorm?(x), weight, bias); weight is nn.Linear layout [N, K].
+    Dispatches to the custom operator flashsvd_hip::linear (``.out`` when ``out`` is given)."""
+    if out is None:
+        return _OPS.linear.default(x, weight, bias, norm_weight, float(eps), residual, int(cfg))
+    return _OPS.linear.out(x, weight, bias, norm_weight, float(eps), residual, int(cfg), out=out)
+
+
+def _linear_impl(x, weight, bias, norm_weight, eps, residual, out, cfg):
     _need(x, "x"); _need(weight, "weight")
     if weight.dim() != 2 or weight.stride(1) != 1:
         raise ValueError(f"weight must be [N, K] with unit inner stride, got {tuple(weight.shape)} strides {weight.stride()}")
@@ -109,7 +117,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     if norm_weight is not None and B >= 3 and cfg == 0 and K % 32 == 0:
         # three rows and more run on the matrix cores, which take the activations as they are: normalise once
         # up front (same rounding points as the fused prologue)
-        x2 = rmsnorm(x2, norm_weight, eps)
+        x2 = _rmsnorm_impl(x2, norm_weight, eps, None)
         norm_weight = None
     rc = lib.fsvd_linear(x2.data_ptr(), x2.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias), _ptr(norm_weight),
                          float(eps), _ptr(r2), 0 if r2 is None else r2.stride(0), o2.data_ptr(), o2.stride(0),
@@ -120,7 +128,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
 
 def swiglu_linear(p: torch.Tensor, gate_u: torch.Tensor, up_u: torch.Tensor, *, up_off: int, mode: int = 0,
                   out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:
-    """h = silu(p[..., :R] @ gate_u.T) * (p[..., up_off:up_off+R] @ up_u.T); gate_u/up_u are [D, R]."""
+    """h = silu(p[..., :R] @ gate_u.T) * (p[..., up_off:up_off+R] @ up_u.T); gate_u/up_u are [D, R].
+    Custom operator flashsvd_hip::swiglu_linear."""
+    if out is None:
+        return _OPS.swiglu_linear.default(p, gate_u, up_u, int(up_off), int(mode), int(cfg))
+    return _OPS.swiglu_linear.out(p, gate_u, up_u, int(up_off), int(mode), int(cfg), out=out)
+
+
+def _swiglu_linear_impl(p, gate_u, up_u, up_off, mode, out, cfg):
     _need(p, "p"); _need(gate_u, "gate_u"); _need(up_u, "up_u")
     if gate_u.dim() != 2 or gate_u.shape != up_u.shape or gate_u.stride() != up_u.stride() or gate_u.stride(1) != 1:
         raise ValueError(f"gate_u/up_u must be matching [D, R] weights, got {tuple(gate_u.shape)} / {tuple(up_u.shape)}")
@@ -236,7 +251,13 @@ def qkv_rope_append(p: torch.Tensor, q_u: torch.Tensor, k_u: torch.Tensor, v_u: 
                     cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                     k_cache: torch.Tensor, v_cache: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int,
                     q_out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:
-    """q (rotated) -> q_out [B,H,Dh]; rotated k and v written into the caches [B,S,Hk,Dh] at positions[b]."""
+    """q (rotated) -> q_out [B,H,Dh]; rotated k and v written into the caches [B,S,Hk,Dh] at positions[b].
+    Custom operator flashsvd_hip::qkv_rope_append (the caches are mutated arguments)."""
+    a = (p, q_u, k_u, v_u, cos, sin, positions, k_cache, v_cache, int(num_heads), int(num_kv_heads), int(head_dim), int(cfg))
+    return _OPS.qkv_rope_append.default(*a) if q_out is None else _OPS.qkv_rope_append.out(*a, q_out=q_out)
+
+
+def _qkv_rope_append_impl(p, q_u, k_u, v_u, cos, sin, positions, k_cache, v_cache, num_heads, num_kv_heads, head_dim, q_out, cfg):
     for t, nm in ((p, "p"), (q_u, "q_u"), (k_u, "k_u"), (v_u, "v_u"), (k_cache, "k_cache"), (v_cache, "v_cache")):
         _need(t, nm)
     _need(positions, "positions", dtype=torch.int32)
@@ -296,7 +317,15 @@ def attn_decode_densekv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
                         out: Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None,
                         static_scratch: bool = False) -> torch.Tensor:
     """q [B,H,Dh] over caches [B,S,Hk,Dh]; see fsvd_attn_decode_densekv in include/flashsvd_hip.h.
-    static_scratch=True takes fsvd_attn_decode_densekv_static (the library's own fixed scratch array)."""
+    static_scratch=True takes fsvd_attn_decode_densekv_static (the library's own fixed scratch array).
+    Custom operator flashsvd_hip::attn_decode_densekv."""
+    a = (q, k_cache, v_cache, cache_seqlens, k_new, v_new, cos, sin, int(seqlen_add), None if nsplit is None else int(nsplit),
+         workspace, None if not softmax_scale else float(softmax_scale), bool(static_scratch))
+    return _OPS.attn_decode_densekv.default(*a) if out is None else _OPS.attn_decode_densekv.out(*a, out=out)
+
+
+def _attn_decode_densekv_impl(q, k_cache, v_cache, cache_seqlens, k_new, v_new, cos, sin, seqlen_add, nsplit, workspace, out,
+                              softmax_scale, static_scratch):
     _need(q, "q"); _need(k_cache, "k_cache"); _need(v_cache, "v_cache")
     _need(cache_seqlens, "cache_seqlens", dtype=torch.int32)
     if q.dim() != 3 or q.stride(2) != 1:
@@ -356,6 +385,11 @@ def attn_decode_densekv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """w * bf16(x * rsqrt(mean(x^2) + eps)); custom operator flashsvd_hip::rmsnorm."""
+    return _OPS.rmsnorm.default(x, weight, float(eps)) if out is None else _OPS.rmsnorm.out(x, weight, float(eps), out=out)
+
+
+def _rmsnorm_impl(x, weight, eps, out):
     _need(x, "x"); _need(weight, "weight")
     K = x.shape[-1]
     if weight.shape != (K,) or not weight.is_contiguous():
@@ -411,7 +445,14 @@ def lowrank_expand_heads(p: torch.Tensor, u: torch.Tensor, *, num_heads: int, he
                          positions: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
                          dst_by_position: bool = False, head_stride: Optional[int] = None) -> torch.Tensor:
     """out[b, row, h, :] = rope(p[b, m, (h), :] @ u[h*Dh:(h+1)*Dh].T + bias); see fsvd_lowrank_expand_heads.
-    p is [B, M, R] (shared by all heads) or [B, M, heads, R]; out is [B, rows, heads, Dh]."""
+    p is [B, M, R] (shared by all heads) or [B, M, heads, R]; out is [B, rows, heads, Dh].
+    Custom operator flashsvd_hip::lowrank_expand_heads (``out`` is the mutated argument)."""
+    _OPS.lowrank_expand_heads.default(p, u, int(num_heads), int(head_dim), out, cos, sin, positions, bias, bool(dst_by_position),
+                                      None if head_stride is None else int(head_stride))
+    return out
+
+
+def _lowrank_expand_heads_impl(p, u, num_heads, head_dim, out, cos, sin, positions, bias, dst_by_position, head_stride):
     heads, Dh = int(num_heads), int(head_dim)
     B, M, R, sp = _expand_operands(p, u, heads, Dh, out, bias, head_stride)
     rope_len = _rope_tables(cos, sin, Dh)
@@ -466,7 +507,13 @@ def lowrank_expand_heads_multi(items, *, head_dim: int, cos: Optional[torch.Tens
 def attn_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, q_pos0: Optional[torch.Tensor] = None, causal: bool = True,
                  pad_mask: Optional[torch.Tensor] = None, add_mask: Optional[torch.Tensor] = None,
                  out: Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None) -> torch.Tensor:
-    """q [B,M,H,Dh] (rotated), k/v [B,S,Hk,Dh] -> out [B,M,H,Dh]; keys n < q_pos0[b]+M, causal n <= q_pos0[b]+m."""
+    """q [B,M,H,Dh] (rotated), k/v [B,S,Hk,Dh] -> out [B,M,H,Dh]; keys n < q_pos0[b]+M, causal n <= q_pos0[b]+m.
+    Custom operator flashsvd_hip::rope_attn_prefill."""
+    a = (q, k, v, q_pos0, bool(causal), pad_mask, add_mask, None if not softmax_scale else float(softmax_scale))
+    return _OPS.rope_attn_prefill.default(*a) if out is None else _OPS.rope_attn_prefill.out(*a, out=out)
+
+
+def _attn_prefill_impl(q, k, v, q_pos0, causal, pad_mask, add_mask, out, softmax_scale):
     _need(q, "q"); _need(k, "k"); _need(v, "v")
     if q.dim() != 4 or k.dim() != 4 or k.shape != v.shape or k.stride() != v.stride():
         raise ValueError(f"q must be [B,M,H,Dh] and k/v matching [B,S,Hk,Dh], got {tuple(q.shape)} {tuple(k.shape)} {tuple(v.shape)}")

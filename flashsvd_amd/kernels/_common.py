@@ -39,3 +39,25 @@ def check(name: str, rc: int) -> None:
 
 def inner_contig(t: torch.Tensor) -> torch.Tensor:
     return t if t.stride(-1) == 1 else t.contiguous()
+
+
+_TRANSPOSED: dict = {}
+
+
+def linear_layout_of(W: torch.Tensor) -> torch.Tensor:
+    """The nn.Linear-layout twin ``W.T.contiguous()`` of a reference-layout operand ``W [K, N]`` (``x @ W``), built once
+    per tensor and kept while the tensor lives and is not written to (keyed by storage address, shape, strides and
+    version counter, checked against a weak reference).  The reference re-lays its operands out on every call
+    (``.contiguous()``, kernels/mlp/decode/dual_split_triton.py:576-581; ``pack_qkv_shared_bases`` is the same idea for
+    the head bases); here the copy is what lets the reference-layout operators stream weights the way the product path
+    does — every output a contiguous row."""
+    import weakref
+    key = (W.data_ptr(), tuple(W.shape), tuple(W.stride()), W._version, W.dtype)
+    hit = _TRANSPOSED.get(key)
+    if hit is not None and hit[0]() is W:
+        return hit[1]
+    out = W.t().contiguous()
+    if len(_TRANSPOSED) > 512:
+        _TRANSPOSED.clear()
+    _TRANSPOSED[key] = (weakref.ref(W), out)
+    return out

@@ -11,6 +11,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
+from ..torch_ops import ops as _OPS
 from ._common import check, dtype_code, inner_contig, scratch, stream
 
 
@@ -27,7 +28,57 @@ def _bias_ok(b: Optional[torch.Tensor], name: str, heads: int, dh: int) -> Optio
 
 
 def _launch(Pq, Pk, Pv, sP, Vq, Vk, Vv, bq, bk, bv, B, H, Hk, Dh, Rq, Rk, Rv):
-    """sP: per matrix (stride_b, stride_h, stride_r) of the coefficient tensors."""
+    """sP: per matrix (stride_b, stride_h, stride_r) of the coefficient tensors.  Goes through the custom operator
+    flashsvd_hip::reconstruct_qkv_token, which takes head-wise views [B, heads, R] (a head stride of 0 = shared)."""
+    views = [P.as_strided((B, h, r), st) for P, h, r, st in ((Pq, H, Rq, sP[0]), (Pk, Hk, Rk, sP[1]), (Pv, Hk, Rv, sP[2]))]
+    return _OPS.reconstruct_qkv_token.default(*views, Vq, Vk, Vv, bq, bk, bv)
+
+
+def _heads_as_linear_layout(V: torch.Tensor) -> torch.Tensor:
+    """[heads, R, Dh] basis -> nn.Linear layout [heads*Dh, R], built once per tensor (see rank_decode._as_linear_layout)."""
+    from .rank_decode import _as_linear_layout
+    return _as_linear_layout(V)
+
+
+def _reconstruct_fast(Pq, Pk, Pv, Vq, Vk, Vv, bq, bk, bv):
+    """Shared coefficients (head stride 0), bf16: the head expansion of the product path on nn.Linear-layout twins of the
+    bases — one launch (fsvd_qkv_rope_append without rotation, K and V written to one-row "caches") when there are no
+    biases, else one fused-bias projection per matrix.  Same arithmetic as the reference kernels: fp32 sum (+ bias), one
+    rounding (kernels/attn/decode/densekv_reconstruct_triton.py:170-237)."""
+    import os
+    from .. import hip_ops
+    B, H, Rq = Pq.shape
+    Hk, Rk, Rv, Dh = Pk.shape[1], Pk.shape[2], Pv.shape[2], Vq.shape[2]
+    if os.getenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST", "1") == "0" or Dh not in (64, 128):
+        return None
+    if any(t.dtype != torch.bfloat16 for t in (Pq, Pk, Pv, Vq, Vk, Vv)) or any(t.stride(1) != 0 or t.stride(2) != 1 for t in (Pq, Pk, Pv)):
+        return None
+    if Rq % 8 or Rk % 8 or Rv % 8:
+        return None
+    uq, uk, uv = _heads_as_linear_layout(Vq), _heads_as_linear_layout(Vk), _heads_as_linear_layout(Vv)
+    pq, pk, pv = (t.as_strided((B, r), (t.stride(0), 1)) for t, r in ((Pq, Rq), (Pk, Rk), (Pv, Rv)))
+    if bq is not None or bk is not None or bv is not None:
+        flat = lambda b: None if b is None else b.reshape(-1).contiguous()
+        return (hip_ops.linear(pq, uq, flat(bq)).view(B, H, Dh), hip_ops.linear(pk, uk, flat(bk)).view(B, Hk, Dh),
+                hip_ops.linear(pv, uv, flat(bv)).view(B, Hk, Dh))
+    adjacent = pk.data_ptr() == pq.data_ptr() + Rq * 2 and pv.data_ptr() == pk.data_ptr() + Rk * 2 and \
+        pq.stride(0) == pk.stride(0) == pv.stride(0) >= Rq + Rk + Rv
+    p = pq.as_strided((B, Rq + Rk + Rv), (pq.stride(0), 1)) if adjacent else torch.cat([pq, pk, pv], dim=1)
+    K = torch.empty((B, 1, Hk, Dh), device=Pq.device, dtype=Pq.dtype)
+    V = torch.empty_like(K)
+    pos = scratch(Pq.device, 4096, "reconstruct_pos")[:B]          # zeros: every row writes its one cache slot
+    Q = hip_ops.qkv_rope_append(p, uq, uk, uv, None, None, pos, K, V, num_heads=H, num_kv_heads=Hk, head_dim=Dh)
+    return Q, K.view(B, Hk, Dh), V.view(B, Hk, Dh)
+
+
+def _reconstruct_impl(Pq, Pk, Pv, Vq, Vk, Vv, bq, bk, bv):
+    B, H, Rq = Pq.shape
+    Hk, Rk, Rv, Dh = Pk.shape[1], Pk.shape[2], Pv.shape[2], Vq.shape[2]
+    if B <= 64:       # decode batches; more rows take the input-major kernel below
+        fast = _reconstruct_fast(Pq, Pk, Pv, Vq, Vk, Vv, bq, bk, bv)
+        if fast is not None:
+            return fast
+    sP = [tuple(t.stride()) for t in (Pq, Pk, Pv)]
     Vq, Vk, Vv = inner_contig(Vq), inner_contig(Vk), inner_contig(Vv)
     for t, nm in ((Pk, "Pk"), (Pv, "Pv"), (Vq, "Vq"), (Vk, "Vk"), (Vv, "Vv")):
         if t.dtype != Pq.dtype:
@@ -138,6 +189,11 @@ def pack_qkv_shared_bases(Vq, Vk, Vv):
 
 
 def _xw(x: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], bias_post: bool) -> torch.Tensor:
+    """Custom operator flashsvd_hip::xw_linear."""
+    return _OPS.xw_linear.default(x, W, bias, bool(bias_post))
+
+
+def _xw_impl(x, W, bias, bias_post):
     lib = _lib.load()
     B, K = x.shape
     N = W.shape[1]

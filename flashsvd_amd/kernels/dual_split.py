@@ -14,6 +14,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
+from ..torch_ops import ops as _OPS
 from ._common import check, dtype_code, scratch, stream
 
 
@@ -98,6 +99,42 @@ def _check_workspace(ws, shape, device, name):
 
 def _run(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, b2, *, variant: int, BD: int, partials_fp32: bool = True,
          s_out: Optional[torch.Tensor] = None):
+    """Custom operator flashsvd_hip::mlp_dual_split on [T, R] coefficient rows."""
+    return _OPS.mlp_dual_split.default(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, b2, int(variant), int(BD), bool(partials_fp32), s_out)
+
+
+def _fast_path_ok(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, variant, partials_fp32, s_out) -> bool:
+    """bf16, fp32 partial sums rounded once (v2 / v2_sm80 / pcat_s, and v1 with fp32 partials), no caller workspace:
+    the arithmetic of three product-path launches on nn.Linear-layout twins of the operands."""
+    if os.getenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST", "1") == "0":
+        return False
+    if s_out is not None or not (variant == 2 or (variant == 1 and partials_fp32)):
+        return False
+    if any(t.dtype != torch.bfloat16 for t in (p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU)):
+        return False
+    R, D, Hd = p_up_2d.shape[1], GateU.shape[1], DownU.shape[1]
+    return p_up_2d.stride(1) == 1 and p_gate_2d.stride(1) == 1 and R % 8 == 0 and D % 8 == 0 and Hd % 8 == 0
+
+
+def _run_fast(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, b2):
+    from .. import hip_ops
+    from ._common import linear_layout_of
+    T, R = p_up_2d.shape
+    # the coefficient rows as one [T, 2R] buffer [PGate | PUp]: adjacent views of such a packed tensor are used in place,
+    # anything else (separate tensors, the [PUp | PGate] order of the pcat_s variant) is packed by one small copy
+    if p_up_2d.data_ptr() == p_gate_2d.data_ptr() + R * 2 and p_up_2d.stride(0) == p_gate_2d.stride(0) >= 2 * R:
+        p = p_gate_2d.as_strided((T, 2 * R), (p_gate_2d.stride(0), 1))
+    else:
+        p = torch.cat([p_gate_2d, p_up_2d], dim=1)
+    gate_u, up_u = linear_layout_of(GateU), linear_layout_of(UpU)          # [D, R]
+    h = hip_ops.swiglu_linear(p, gate_u, up_u, up_off=R, mode=1)           # h = bf16(silu(g32) * u32), dual_split_triton.py:207
+    s = hip_ops.linear(h, linear_layout_of(DownV))                        # S: fp32 sum over D, one rounding (:719-720)
+    return hip_ops.linear(s, linear_layout_of(DownU), None if b2 is None else b2.to(torch.bfloat16).contiguous())
+
+
+def _run_impl(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, b2, variant, BD, partials_fp32, s_out):
+    if _fast_path_ok(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, variant, partials_fp32, s_out):
+        return _run_fast(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, b2)
     T, R = p_up_2d.shape
     D, Hd = int(GateU.shape[1]), int(DownU.shape[1])
     dt = dtype_code(p_up_2d)

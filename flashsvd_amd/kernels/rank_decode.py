@@ -19,6 +19,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
+from ..torch_ops import ops as _OPS
 from ._common import check, stream
 
 
@@ -56,7 +57,17 @@ def rank_decode(q: torch.Tensor, pk_cache: torch.Tensor, pv_cache: torch.Tensor,
                 cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], seqlens: torch.Tensor, *, num_kv_heads: int,
                 seqlen_add: int = 0, rotate_q: bool = False, bv: Optional[torch.Tensor] = None, nsplit: Optional[int] = None,
                 workspace=None, out: Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None) -> torch.Tensor:
-    """q [B,H,Dh]; pk_cache/pv_cache [B,S,R] (shared) or [B,S,Hk,R]; k_u/v_u nn.Linear weights [Hk*Dh,R]."""
+    """q [B,H,Dh]; pk_cache/pv_cache [B,S,R] (shared) or [B,S,Hk,R]; k_u/v_u nn.Linear weights [Hk*Dh,R].
+    Custom operator flashsvd_hip::attn_decode_rankkv; ``workspace`` = (M, L, Acc)."""
+    ws_m, ws_l, ws_acc = workspace if workspace is not None else (None, None, None)
+    a = (q, pk_cache, pv_cache, k_u, v_u, cos, sin, seqlens, int(num_kv_heads), int(seqlen_add), bool(rotate_q), bv,
+         None if nsplit is None else int(nsplit), ws_m, ws_l, ws_acc, None if not softmax_scale else float(softmax_scale))
+    return _OPS.attn_decode_rankkv.default(*a) if out is None else _OPS.attn_decode_rankkv.out(*a, out=out)
+
+
+def _rank_decode_impl(q, pk_cache, pv_cache, k_u, v_u, cos, sin, seqlens, num_kv_heads, seqlen_add, rotate_q, bv, nsplit,
+                      ws_m, ws_l, ws_acc, out, softmax_scale):
+    workspace = None if ws_m is None else (ws_m, ws_l, ws_acc)
     for t, nm in ((q, "q"), (pk_cache, "pk_cache"), (pv_cache, "pv_cache"), (k_u, "k_u"), (v_u, "v_u")):
         if not t.is_cuda:
             raise ValueError(f"{nm} must be a GPU tensor")
@@ -111,7 +122,12 @@ def rank_decode(q: torch.Tensor, pk_cache: torch.Tensor, pv_cache: torch.Tensor,
 def rankkv_append(pk: torch.Tensor, pv: torch.Tensor, pk_cache: torch.Tensor, pv_cache: torch.Tensor, positions: torch.Tensor) -> None:
     """pk_cache[b, positions[b]] = pk[b], pv_cache[b, positions[b]] = pv[b] in one launch: the one-token case of
     FlashSVDLegacySparseKVCache.update (runtime/cache/attn_legacy_sparse_kv.py:113-169).  pk / pv [B,R] (row views of a
-    wider buffer are fine), caches [>=B,S,R] bf16, positions int32 [B] on the device; positions outside the cache are dropped."""
+    wider buffer are fine), caches [>=B,S,R] bf16, positions int32 [B] on the device; positions outside the cache are dropped.
+    Custom operator flashsvd_hip::rankkv_append."""
+    _OPS.rankkv_append.default(pk, pv, pk_cache, pv_cache, positions)
+
+
+def _rankkv_append_impl(pk, pv, pk_cache, pv_cache, positions):
     for t, nm in ((pk, "pk"), (pv, "pv"), (pk_cache, "pk_cache"), (pv_cache, "pv_cache")):
         if not t.is_cuda or t.dtype != torch.bfloat16:
             raise ValueError(f"{nm} must be a bfloat16 GPU tensor")

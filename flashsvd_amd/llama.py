@@ -615,50 +615,123 @@ class SVDLlamaDecoderLayer(nn.Module):
 
     def decode_token(self, x: torch.Tensor, cache, positions: torch.Tensor, *, rope=None, attn_ws=None, nsplit=None):
         """x [B,d] -> [B,d]; both RMSNorms and both residual adds are fused into the projections."""
-        n1, n2 = self.input_layernorm, self.post_attention_layernorm
-        x2 = self.self_attn.decode_token(x, cache, positions, norm_weight=n1.weight, eps=n1.variance_epsilon,
-                                         residual=x, rope=rope, attn_ws=attn_ws, nsplit=nsplit)
-        return self._layer_tail(x2)
+        return decoder_layer_decode_token(self, x, cache, positions, rope=rope, attn_ws=attn_ws, nsplit=nsplit)
 
     def _layer_tail(self, x2: torch.Tensor) -> torch.Tensor:
-        """residual + post-attention norm + MLP + residual; replayed from a captured graph when the
-        layer-tail scope is enabled and no outer capture is running."""
-        n2 = self.post_attention_layernorm
-        want_graph = (LAYER_TAIL_GRAPH_ENABLED and _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH")
-                      and os.getenv("FLASH_SVD_MLP_CUDA_GRAPH_SCOPE", "auto").strip().lower() in ("auto", "layer_tail")
-                      and not torch.cuda.is_current_stream_capturing())
-        if not want_graph:
-            return self.mlp.run(x2, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=x2)
-        from .graphs import GraphedCallable
-        mode = mlp_rounding_mode()
-        cache = self.mlp._flashsvd_layer_graph_cache
-        key = (tuple(x2.shape), x2.dtype, x2.device, mode)
-        g = cache.get(key)
-        if g is None:
-            g = GraphedCallable(lambda t: self.mlp.run(t, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=t, mode=mode), x2)
-            cache[key] = g
-        out = g(x2)
-        return out if _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH_ALIAS_OUTPUT") else out.clone()
+        return decoder_layer_tail(self, x2)
 
     def forward(self, hidden_states: torch.Tensor, attention_mask=None, position_ids=None, past_key_values=None,
                 cache_position=None, position_embeddings=None, **kwargs):
-        _require_gpu(hidden_states, "SVDLlamaDecoderLayer")
-        cache = past_key_values if past_key_values is not None else kwargs.get("past_key_value")
-        B, T, d = hidden_states.shape
-        n1, n2 = self.input_layernorm, self.post_attention_layernorm
-        if cache is None:
-            cache = FlashSVDV15DenseKVCache(SimpleNamespace(num_hidden_layers=self.layer_idx + 1,
-                                                            rope_theta=self.self_attn.rotary_emb.base),
-                                            max_batch_size=B, max_cache_len=T, device=hidden_states.device,
-                                            dtype=hidden_states.dtype)
-        if T == 1:
-            positions = self.self_attn._positions_for(cache, B, cache_position, hidden_states.device)
-            out = self.decode_token(hidden_states[:, 0], cache, positions).unsqueeze(1)
-            cache.advance_after_fa2(self.layer_idx, q_len=1, cache_position=cache_position)
-            return out
-        x2 = self.self_attn.prefill_tokens(hidden_states, cache, cache_position, norm_weight=n1.weight,
-                                           eps=n1.variance_epsilon, residual=hidden_states)
-        return self.mlp.run(x2, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=x2)
+        return decoder_layer_forward(self, hidden_states, past_key_values=past_key_values, cache_position=cache_position, **kwargs)
+
+
+# The three functions below are the decoder layer.  They take any module that carries ``input_layernorm``, ``self_attn``
+# (SVD_LlamaAttention), ``post_attention_layernorm`` and ``mlp`` (SVD_LlamaMLP): this package's SVDLlamaDecoderLayer, or an
+# unmodified transformers LlamaDecoderLayer whose two sub-modules were swapped for the low-rank ones (the reference's
+# arrangement, utils/model_utils.py:586-671), once enable_flashsvd_llama_layer_tail_cuda_graph() has patched that class.
+def decoder_layer_decode_token(layer, x: torch.Tensor, cache, positions: torch.Tensor, *, rope=None, attn_ws=None, nsplit=None):
+    n1 = layer.input_layernorm
+    x2 = layer.self_attn.decode_token(x, cache, positions, norm_weight=n1.weight, eps=n1.variance_epsilon,
+                                      residual=x, rope=rope, attn_ws=attn_ws, nsplit=nsplit)
+    return decoder_layer_tail(layer, x2)
+
+
+def decoder_layer_tail(layer, x2: torch.Tensor) -> torch.Tensor:
+    """residual + post-attention norm + MLP + residual; replayed from a captured graph when the
+    layer-tail scope is enabled and no outer capture is running."""
+    n2, mlp = layer.post_attention_layernorm, layer.mlp
+    want_graph = (LAYER_TAIL_GRAPH_ENABLED and _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH")
+                  and os.getenv("FLASH_SVD_MLP_CUDA_GRAPH_SCOPE", "auto").strip().lower() in ("auto", "layer_tail")
+                  and not torch.cuda.is_current_stream_capturing())
+    if not want_graph:
+        return mlp.run(x2, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=x2)
+    from .graphs import GraphedCallable
+    mode = mlp_rounding_mode()
+    cache = mlp._flashsvd_layer_graph_cache
+    key = (tuple(x2.shape), x2.dtype, x2.device, mode)
+    g = cache.get(key)
+    if g is None:
+        g = GraphedCallable(lambda t: mlp.run(t, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=t, mode=mode), x2)
+        cache[key] = g
+    out = g(x2)
+    return out if _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH_ALIAS_OUTPUT") else out.clone()
+
+
+def decoder_layer_forward(layer, hidden_states: torch.Tensor, *, past_key_values=None, cache_position=None, **kwargs):
+    _require_gpu(hidden_states, type(layer).__name__)
+    attn = layer.self_attn
+    cache = past_key_values if past_key_values is not None else kwargs.get("past_key_value")
+    B, T, d = hidden_states.shape
+    n1 = layer.input_layernorm
+    if cache is None:
+        cache = FlashSVDV15DenseKVCache(SimpleNamespace(num_hidden_layers=attn.layer_idx + 1, rope_theta=attn.rotary_emb.base),
+                                        max_batch_size=B, max_cache_len=T, device=hidden_states.device, dtype=hidden_states.dtype)
+    if T == 1:
+        positions = attn._positions_for(cache, B, cache_position, hidden_states.device)
+        out = decoder_layer_decode_token(layer, hidden_states[:, 0], cache, positions).unsqueeze(1)
+        cache.advance_after_fa2(attn.layer_idx, q_len=1, cache_position=cache_position)
+        return out
+    x2 = attn.prefill_tokens(hidden_states, cache, cache_position, norm_weight=n1.weight, eps=n1.variance_epsilon,
+                             residual=hidden_states)
+    n2 = layer.post_attention_layernorm      # prompt rows: no graph (the captured tail is a decode-step device)
+    return layer.mlp.run(x2, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=x2)
+
+
+_HF_PATCH = {}
+
+
+def patch_hf_llama_decoder_layer() -> bool:
+    """Idempotent, process-global: give transformers' LlamaDecoderLayer a forward that, for a layer whose ``mlp`` is an
+    SVD_LlamaMLP, runs "residual + post-attention norm + MLP + residual" through the fused kernels (and from one captured
+    graph under the layer_tail scope); when ``self_attn`` is an SVD_LlamaAttention too the whole layer takes the same
+    route as SVDLlamaDecoderLayer, bit for bit.  Layers with other modules, and tensors that are not bf16 on the GPU, keep
+    the original forward.  Returns False when transformers is not importable."""
+    if _HF_PATCH:
+        return True
+    try:
+        from transformers.models.llama.modeling_llama import LlamaDecoderLayer
+    except Exception:
+        return False
+    orig = LlamaDecoderLayer.forward
+    returns_tensor = orig.__annotations__.get("return") in (torch.Tensor, "torch.Tensor")
+
+    def forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
+                position_embeddings=None, **kwargs):
+        if not isinstance(self.mlp, SVD_LlamaMLP) or not hidden_states.is_cuda or hidden_states.dtype != torch.bfloat16:
+            return orig(self, hidden_states, attention_mask=attention_mask, position_ids=position_ids,
+                        past_key_values=past_key_values, use_cache=use_cache, position_embeddings=position_embeddings, **kwargs)
+        if _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH") and os.getenv("FLASH_SVD_MLP_CUDA_GRAPH_SCOPE", "auto").strip().lower() == "mlp":
+            # scope "mlp": the graph covers the MLP module alone (SVD_LlamaMLP.forward replays it); the layer around it
+            # stays the original one
+            return orig(self, hidden_states, attention_mask=attention_mask, position_ids=position_ids,
+                        past_key_values=past_key_values, use_cache=use_cache, position_embeddings=position_embeddings, **kwargs)
+        if past_key_values is None:
+            past_key_values = kwargs.pop("past_key_value", None)
+        if isinstance(self.self_attn, SVD_LlamaAttention) and \
+                (past_key_values is None or isinstance(past_key_values, (FlashSVDV15DenseKVCache, FlashSVDLegacySparseKVCache))):
+            out = decoder_layer_forward(self, hidden_states, past_key_values=past_key_values,
+                                        cache_position=kwargs.get("cache_position"))
+        else:
+            # attention half as the unmodified layer runs it (any attention module), fused tail
+            h = self.input_layernorm(hidden_states)
+            h = self.self_attn(hidden_states=h, attention_mask=attention_mask, position_ids=position_ids,
+                               past_key_values=past_key_values, use_cache=use_cache, position_embeddings=position_embeddings, **kwargs)
+            h = h[0] if isinstance(h, (tuple, list)) else h
+            x2 = hidden_states + h
+            shape = x2.shape
+            out = decoder_layer_tail(self, x2.reshape(-1, shape[-1]) if x2.dim() == 3 and shape[1] == 1 else x2).reshape(shape)
+        return out if returns_tensor else (out,)
+
+    LlamaDecoderLayer.forward = forward
+    _HF_PATCH.update(cls=LlamaDecoderLayer, orig=orig)
+    return True
+
+
+def unpatch_hf_llama_decoder_layer() -> None:
+    """Put the original forward back (tests)."""
+    if _HF_PATCH:
+        _HF_PATCH["cls"].forward = _HF_PATCH["orig"]
+        _HF_PATCH.clear()
 
 
 class SVDLlamaModel(nn.Module):

@@ -259,6 +259,11 @@ class PersistentDecoder:
         g.plain_out = self.token_log.data_ptr()
         ph.append(g)
 
+        self._finish(ph, dev)
+
+    def _finish(self, ph, dev) -> None:
+        """Derived fields, host-side validation, upload of the phase list."""
+        lib = self.lib
         self.nph = len(ph)
         self.host_phases = (Phase * self.nph)(*ph)
         _lib.check("fsvd_decode_step_prepare", lib.fsvd_decode_step_prepare(ctypes.addressof(self.host_phases), self.nph, self.nwg))
@@ -301,6 +306,9 @@ class PersistentDecoder:
 
     PHASE_NAMES = ("embed", "attn_rank_proj", "qkv_u", "attn", "attn_merge", "o_v", "o_u", "mlp_rank_proj", "swiglu",
                    "down_v", "down_u")
+
+    def phase_names(self) -> list:
+        return ["embed"] + [n for _ in range(self.L) for n in self.PHASE_NAMES[1:]] + ["lm_head", "argmax"]
 
     def trace_step(self, wg_stride: int = 32) -> torch.Tensor:
         """Run ONE step with per-phase time stamps; returns int64 [workgroups/stride, phases, 4] in
@@ -361,7 +369,7 @@ class PersistentDecoder:
         """Per-phase microseconds of one traced step, averaged over layers and traced workgroups:
         {phase name: {"wait": input wait, "stream": weight stream, "publish": epilogue, "total": ...}}."""
         t = self.trace_step(wg_stride)
-        names = ["embed"] + [n for _ in range(self.L) for n in self.PHASE_NAMES[1:]] + ["lm_head", "argmax"]
+        names = self.phase_names()
         acc: dict = {}
         for p, nm in enumerate(names):
             e, s_, c, d_ = (t[:, p, k] for k in range(4))
@@ -373,6 +381,104 @@ class PersistentDecoder:
             row["total"] += float((d_ - e).mean())
             row["n"] += 1
         return {k: {m: v[m] / v["n"] for m in ("wait", "stream", "publish", "total")} for k, v in acc.items()}
+
+
+class DenseStepDecoder(PersistentDecoder):
+    """The same resident step over DENSE bf16 Llama weights: per layer [q; k; v] projection (RMSNorm fused) -> attention
+    -> merge -> o projection (+ residual) -> gate / up pair (RMSNorm fused, SwiGLU, both matrices over one input) ->
+    down projection (+ residual), then final norm + lm_head + argmax.  It exists as the like-for-like comparator of the
+    low-rank step ("the same model run as dense bf16 on the same GPU"): same kernel, same hand-off, same attention
+    phase, only the weight streams differ.
+
+    ``layers``: one dict per layer with ``wqkv`` [(H + 2*Hk)*Dh, d], ``wo`` [d, H*Dh], ``wg``, ``wu`` [D, d],
+    ``wd`` [d, D], ``n1``, ``n2`` [d] (bf16, contiguous, on the cache's device)."""
+
+    PHASE_NAMES = ("embed", "qkv", "attn", "attn_merge", "o", "gate_up", "down")
+
+    def __init__(self, *, embed, layers, norm, lm_head, cache, num_heads: int, num_kv_heads: int, head_dim: int,
+                 eps: float = 1e-6, mode: int = 0, max_new_tokens: int = 4096):
+        if not isinstance(cache, FlashSVDV15DenseKVCache) or getattr(cache, "_dtype", None) != torch.bfloat16:
+            raise TypeError("DenseStepDecoder needs a bfloat16 FlashSVDV15DenseKVCache")
+        lib = _lib.load()
+        self.lib, self.cache, self.model = lib, cache, None
+        dev = lm_head.device
+        self.nwg = int(lib.fsvd_decode_step_workgroups())
+        H, Hk, Dh = int(num_heads), int(num_kv_heads), int(head_dim)
+        V, d = lm_head.shape
+        L = len(layers)
+        D = int(layers[0]["wg"].shape[0])
+        if self.nwg <= 0 or self.nwg % H != 0:
+            raise ValueError(f"{self.nwg} workgroups are not a multiple of {H} heads")
+        nsplit = self.nwg // H
+        S = int(cache.max_cache_len)
+        self.H, self.Hk, self.Dh, self.d, self.L, self.V, self.S, self.nsplit = H, Hk, Dh, d, L, V, S, nsplit
+        for t in (embed, norm, lm_head, *(w for lw in layers for w in lw.values())):
+            if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.device != dev:
+                raise ValueError("DenseStepDecoder needs contiguous bfloat16 tensors on one device")
+
+        def tagged(n, dt=torch.int32):
+            return torch.zeros(n, dtype=dt, device=dev)
+
+        self.XA, self.XB = tagged(d), tagged(d)
+        self.QKV, self.A, self.HB = tagged((H + 2 * Hk) * Dh), tagged(H * Dh), tagged(D)
+        self.PART, self.CAND = tagged(H * nsplit * (Dh + 2), torch.int64), tagged(self.nwg, torch.int64)
+        self.logits = torch.zeros(V, dtype=torch.bfloat16, device=dev)
+        self.token_log = torch.zeros(int(max_new_tokens), dtype=torch.int64, device=dev)
+        self.state = torch.zeros(8, dtype=torch.int32, device=dev)
+        cos, sin = cache.get_rope_tables(seqlen=S, head_dim=Dh, device=dev, dtype=torch.bfloat16)
+        self.rope = (cos, sin)
+        self._keep = [embed, norm, lm_head, layers]
+        ph = []
+
+        def gemv(W, N, K, inp, out, *, norm_w=None, epi=EP_STORE, aux=None, plain=None, shared=False):
+            p = Phase()
+            p.type, p.epilogue, p.N, p.K, p.nmat, p.mode = PH_GEMV, epi, N, K, len(W), int(mode)
+            p.shared_in = int(shared)
+            for i, w in enumerate(W):
+                if tuple(w.shape) != (N, K):
+                    raise ValueError(f"weight {tuple(w.shape)} is not [{N},{K}]")
+                p.W[i] = w.data_ptr()
+            if norm_w is not None:
+                p.norm_w, p.fparam = norm_w.data_ptr(), float(eps)
+            p.inp, p.out0 = inp, out
+            if aux is not None:
+                p.aux0 = aux
+            if plain is not None:
+                p.plain_out = plain.data_ptr()
+            ph.append(p)
+
+        e = Phase()
+        e.type, e.N = PH_EMBED, d
+        e.W[0] = embed.data_ptr()
+        e.out0 = _tb(self.XA, L + 1, 0)
+        ph.append(e)
+        for l, lw in enumerate(layers):
+            cache._ensure_layer_spec(l, h=Hk, dh=Dh)
+            kc, vc = cache.key_cache[l][0], cache.value_cache[l][0]
+            xin, xmid, xout = _tb(self.XA, L + 1, l), _tb(self.XB, L, l), _tb(self.XA, L + 1, l + 1)
+            gemv([lw["wqkv"]], (H + 2 * Hk) * Dh, d, xin, _tb(self.QKV, L, l), norm_w=lw["n1"])
+            a = Phase()
+            a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
+            a.fparam = 1.0 / math.sqrt(Dh)
+            a.cos, a.sin, a.rope_len = cos.data_ptr(), sin.data_ptr(), int(cos.shape[0])
+            a.k_cache, a.v_cache, a.sc_s, a.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
+            a.inp, a.out0 = _tb(self.QKV, L, l), _tb(self.PART, L, l)
+            ph.append(a)
+            m = Phase()
+            m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
+            m.inp, m.out0 = _tb(self.PART, L, l), _tb(self.A, L, l)
+            ph.append(m)
+            gemv([lw["wo"]], d, H * Dh, _tb(self.A, L, l), xmid, epi=EP_RESID, aux=xin)
+            gemv([lw["wg"], lw["wu"]], D, d, xmid, _tb(self.HB, L, l), norm_w=lw["n2"], epi=EP_SWIGLU, shared=True)
+            gemv([lw["wd"]], d, D, _tb(self.HB, L, l), xout, epi=EP_RESID, aux=xmid)
+            cache._layer_initialized[l] = True
+        gemv([lm_head], V, d, _tb(self.XA, L + 1, L), _tb(self.CAND, 1, 0), norm_w=norm, epi=EP_LOGITS, plain=self.logits)
+        g = Phase()
+        g.type = PH_ARGMAX
+        g.inp = _tb(self.CAND, 1, 0)
+        g.plain_out = self.token_log.data_ptr()
+        ph.append(g)
+        self._finish(ph, dev)
 
 
 def decode_engine_choice() -> str:

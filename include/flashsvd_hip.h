@@ -291,7 +291,8 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
 #define FSVD_PH_EMBED 0   /* out0[n] = W[0][token, n]                                   (N = hidden)        */
 #define FSVD_PH_GEMV 1    /* out0 = epilogue(W[m] . norm(in)), m < nmat; bf16 weights, or int4 when wbits == 4  */
 #define FSVD_PH_ATTN 3    /* in = un-rotated [q | k | v] of the current token ((H + 2*Hk) * Dh values, the   */
-                          /* output of a GEMV over the row-packed [q_u; k_u; v_u]): rotate-half RoPE on q, k */
+                          /* output of a GEMV over the row-packed [q_u; k_u; v_u], or of a plain GEMV of that   */
+                          /* many rows): rotate-half RoPE on q, k                                            */
                           /* at state->pos, append k, v to the cache, split-KV attention; out0 = partials    */
 #define FSVD_PH_MERGE 4   /* out0 = merged attention output from in = partials                               */
 #define FSVD_PH_ARGMAX 5  /* token = argmax of the per-workgroup candidates in `in`; advances the state      */
@@ -299,6 +300,7 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
 #define FSVD_EP_STORE 0   /* out0[n] = bf16(dot)                                                              */
 #define FSVD_EP_RESID 1   /* out0[n] = bf16(aux0[n] + bf16(dot))                                              */
 #define FSVD_EP_SWIGLU 2  /* nmat = 2: out0[n] = silu(W[0][n].in[0:K]) * (W[1][n].in[K:2K]), rounding `mode`  */
+                          /* (shared_in: both over in[0:K])                                                   */
 #define FSVD_EP_LOGITS 3  /* plain_out[n] = bf16(dot) and out0[wg] = (best value, best index) of the workgroup */
 
 typedef struct fsvd_tagbuf {
@@ -326,7 +328,9 @@ typedef struct fsvd_phase {
    * the fp16 scale bits of a group in the low half and (zero point + 128) in the high half; a group is
    * 32 << gshift columns.  K % 256 == 0.  Arithmetic as fsvd_linear_q4: y = sum_g s_g * sum_k x_k (q_k - z_g), fp32. */
   const void* qsz[2];
-  int32_t ldg, gshift, wbits, rsv0;
+  int32_t ldg, gshift, wbits;
+  int32_t shared_in;            /* nmat == 2: both matrices read the same K-long input (a dense gate / up pair) instead   */
+                                /* of in[0:K] and in[K:2K]                                                                 */
   /* derived by fsvd_decode_step_prepare (do not fill by hand): work items (rows, merge outputs) are
    * dealt as share_q per workgroup plus one more for the first share_r workgroups; m_kp is the 32-bit
    * reciprocal of K/8 and dk = (threads per workgroup) mod (K/8) */

@@ -165,3 +165,47 @@ def test_dual_split_errors(K):
         K.flashsvd_mlp_dual_split_triton_pcat_s(c(1, 1, 9), c(4, 32), c(4, 32), c(32, 4), c(4, 16))
     with pytest.raises(AssertionError):
         K.flashsvd_mlp_dual_split_triton_v2(rnd(1, 1, 8), c(1, 1, 8), c(8, 32), c(8, 32), c(32, 8), c(8, 16))
+
+
+def test_reference_layout_fast_route_against_the_input_major_kernels(K, monkeypatch):
+    """bf16 v2-type MLP calls and shared-coefficient reconstruction run on nn.Linear-layout twins of their operands (one
+    copy per tensor, reused while the tensor is unchanged) through the product-path kernels; the input-major kernels
+    (FLASHSVD_AMD_REFERENCE_LAYOUT_FAST=0) are the same arithmetic in another summation order.  Both at the 7B shapes."""
+    from flashsvd_amd.kernels import _common
+    dt = torch.bfloat16
+    B, R, D, Hd = 8, 1536, 11008, 4096
+    PUp, PGate = rnd(B, 1, R, seed=1), rnd(B, 1, R, seed=2)
+    GateU, UpU = rnd(R, D, std=0.03, seed=3), rnd(R, D, std=0.03, seed=4)
+    DownV, DownU, b2 = rnd(D, R, std=0.03, seed=5), rnd(R, Hd, std=0.03, seed=6), rnd(Hd, std=0.1, seed=7)
+    ref = O.dual_split_mlp(PUp, PGate, GateU, UpU, DownV, DownU, b2)
+    g = [t.cuda() for t in (PUp, PGate, GateU, UpU, DownV, DownU)]
+    n0 = len(_common._TRANSPOSED)
+    fast = K.flashsvd_mlp_dual_split_triton_v2(*g, b2.cuda())
+    assert len(_common._TRANSPOSED) == n0 + 4                       # GateU, UpU, DownV, DownU
+    again = K.flashsvd_mlp_dual_split_triton_v2(*g, b2.cuda())
+    assert len(_common._TRANSPOSED) == n0 + 4 and torch.equal(fast, again)
+    monkeypatch.setenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST", "0")
+    slow = K.flashsvd_mlp_dual_split_triton_v2(*g, b2.cuda())
+    monkeypatch.delenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST")
+    for got, nm in ((fast, "product-path route"), (slow, "input-major route")):
+        assert_close_bf16(got, ref, nm, **tol(ref, dt))
+    # an operand written in place must not be served from a stale twin
+    g[5].mul_(2.0)
+    doubled = K.flashsvd_mlp_dual_split_triton_v2(*g, None)
+    ref2 = O.dual_split_mlp(PUp, PGate, GateU, UpU, DownV, (DownU.float() * 2).to(dt))
+    assert_close_bf16(doubled, ref2, "after an in-place update of DownU", **tol(ref2, dt))
+    # reconstruction: coefficients as adjacent views of one packed row (the reference's split of hidden @ packed_qkv_rank)
+    Bq, H, Dh, Ra = 1, 32, 128, 1024
+    packed = rnd(Bq, 3 * Ra, seed=11)
+    Vq, Vk, Vv = (rnd(H, Ra, Dh, std=0.03, seed=12 + i) for i in range(3))
+    pg = packed.cuda()
+    gq, gk, gv = pg[:, :Ra], pg[:, Ra:2 * Ra], pg[:, 2 * Ra:]
+    vq, vk, vv = Vq.cuda(), Vk.cuda(), Vv.cuda()
+    refq = O.reconstruct_qkv_token_shared(packed[:, :Ra], packed[:, Ra:2 * Ra], packed[:, 2 * Ra:], Vq, Vk, Vv)
+    fastq = K.reconstruct_qkv_token_shared(gq, gk, gv, vq, vk, vv)
+    monkeypatch.setenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST", "0")
+    slowq = K.reconstruct_qkv_token_shared(gq, gk, gv, vq, vk, vv)
+    for got, nm in ((fastq, "product-path route"), (slowq, "input-major route")):
+        for a, b, c in zip(got, refq, "QKV"):
+            assert a.shape == b.shape and a.is_contiguous()
+            assert_close_bf16(a, b, f"reconstruct {nm} {c}", **tol(b, dt))

@@ -319,3 +319,50 @@ def test_checkpoint_round_trip_decodes_identically(tmp_path):
         dec.step(n_new - 1)
         toks.append([int(tok0)] + dec.tokens().cpu().tolist())
     assert toks[0] == toks[1]
+
+
+def test_dense_step_decoder_matches_the_oracle():
+    """The resident step over DENSE weights (the like-for-like dense-bf16 comparator of the benchmark: plain [q;k;v]
+    projection in front of the attention phase, gate / up pair over one shared input).  The oracle runs the same
+    network as factor pairs whose first factor is the identity, which reproduces a dense linear exactly."""
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    from flashsvd_amd.step import DenseStepDecoder
+    d, H, Hk, Dh, D, L, V = 256, 4, 2, 128, 512, 2, 512
+    g = torch.Generator().manual_seed(21)
+    rn = lambda *s: (torch.randn(*s, generator=g) * 0.05).to(BF16)
+    eye = lambda n: torch.eye(n, dtype=BF16)
+    embed, head, ones = rn(V, d), rn(V, d), torch.ones(d, dtype=BF16)
+    dense, blocks = [], []
+    for _ in range(L):
+        wq, wk, wv, wo = rn(H * Dh, d), rn(Hk * Dh, d), rn(Hk * Dh, d), rn(d, H * Dh)
+        wg, wu, wd = rn(D, d), rn(D, d), rn(d, D)
+        n1, n2 = (1.0 + rn(d)).to(BF16), (1.0 + rn(d)).to(BF16)
+        dense.append(dict(wqkv=torch.cat([wq, wk, wv]).contiguous(), wo=wo, wg=wg, wu=wu, wd=wd, n1=n1, n2=n2))
+        blocks.append(O.BlockWeights(q_v=eye(d), q_u=wq, k_v=eye(d), k_u=wk, v_v=eye(d), v_u=wv, o_v=eye(H * Dh), o_u=wo,
+                                     gate_v=eye(d), gate_u=wg, up_v=eye(d), up_u=wu, down_v=eye(D), down_u=wd, ln1=n1, ln2=n2))
+    mw = O.ModelWeights(embed=embed, blocks=blocks, norm=ones, lm_head=head, n_heads=H, n_kv_heads=Hk, head_dim=Dh)
+    prompt = torch.randint(0, V, (1, 11), generator=torch.Generator().manual_seed(3))
+    n_new, Lp = 7, 11
+    ref_tok, ref_hid, ref_cache, ref_logits = O.greedy_decode(mw, prompt, n_new, "dense", return_logits=True)
+    from types import SimpleNamespace
+    cache = FlashSVDV15DenseKVCache(SimpleNamespace(num_hidden_layers=L, rope_theta=10000.0), max_batch_size=1,
+                                    max_cache_len=Lp + n_new + 2, device="cuda", dtype=BF16)
+    dec = DenseStepDecoder(embed=embed.cuda(), layers=[{k: v.cuda() for k, v in lw.items()} for lw in dense], norm=ones.cuda(),
+                           lm_head=head.cuda(), cache=cache, num_heads=H, num_kv_heads=Hk, head_dim=Dh, max_new_tokens=32)
+    for i in range(Lp):                       # the prompt token by token: every step appends its K / V rows
+        dec.set_state(int(prompt[0, i]), i)
+        dec.step(1)
+    dec.check()
+    assert_close_bf16(dec.hidden()[None].cpu(), ref_hid[:, 0], "hidden state after the prompt", rel_tol=3e-2,
+                      abs_tol=3 * bounds(ref_hid[:, 0])["abs_tol"])
+    for li in range(L):
+        assert_close_bf16(cache.key_cache[li][:, :Lp], ref_cache.k[li][:, :Lp], f"K rows layer {li}", abs_tol=float("inf"), rel_tol=3e-2)
+    tok = int(dec.tokens()[-1])
+    n_equal = int(tok == int(ref_tok[0, 0]))
+    for s in range(1, n_new):                 # teacher-forced with the oracle's tokens
+        dec.set_state(ref_tok[:, s - 1], Lp + s - 1)
+        dec.step(1)
+        assert_close_bf16(dec.hidden()[None].cpu(), ref_hid[:, s], f"hidden state at step {s}", rel_tol=3e-2,
+                          abs_tol=3 * bounds(ref_hid[:, s])["abs_tol"])
+        n_equal += _tie_aware(int(dec.tokens()[0]), int(ref_tok[0, s]), ref_logits[0, s], f"step {s}")
+    assert n_equal >= n_new - 1
