@@ -42,6 +42,7 @@ def inner_contig(t: torch.Tensor) -> torch.Tensor:
 
 
 _TRANSPOSED: dict = {}
+TWIN_BUILDS = [0]          # how many twins have been built (tests count copies with it)
 
 
 def linear_layout_of(W: torch.Tensor) -> torch.Tensor:
@@ -57,7 +58,13 @@ def linear_layout_of(W: torch.Tensor) -> torch.Tensor:
     if hit is not None and hit[0]() is W:
         return hit[1]
     out = W.t().contiguous()
+    TWIN_BUILDS[0] += 1
     if len(_TRANSPOSED) > 512:
         _TRANSPOSED.clear()
-    _TRANSPOSED[key] = (weakref.ref(W), out)
+
+    def _drop(ref, key=key):                     # the operand died: its twin goes with it
+        cur = _TRANSPOSED.get(key)
+        if cur is not None and cur[0] is ref:
+            del _TRANSPOSED[key]
+    _TRANSPOSED[key] = (weakref.ref(W, _drop), out)
     return out

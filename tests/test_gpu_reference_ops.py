@@ -179,11 +179,11 @@ def test_reference_layout_fast_route_against_the_input_major_kernels(K, monkeypa
     DownV, DownU, b2 = rnd(D, R, std=0.03, seed=5), rnd(R, Hd, std=0.03, seed=6), rnd(Hd, std=0.1, seed=7)
     ref = O.dual_split_mlp(PUp, PGate, GateU, UpU, DownV, DownU, b2)
     g = [t.cuda() for t in (PUp, PGate, GateU, UpU, DownV, DownU)]
-    n0 = len(_common._TRANSPOSED)
+    n0 = _common.TWIN_BUILDS[0]
     fast = K.flashsvd_mlp_dual_split_triton_v2(*g, b2.cuda())
-    assert len(_common._TRANSPOSED) == n0 + 4                       # GateU, UpU, DownV, DownU
+    assert _common.TWIN_BUILDS[0] == n0 + 4                         # GateU, UpU, DownV, DownU
     again = K.flashsvd_mlp_dual_split_triton_v2(*g, b2.cuda())
-    assert len(_common._TRANSPOSED) == n0 + 4 and torch.equal(fast, again)
+    assert _common.TWIN_BUILDS[0] == n0 + 4 and torch.equal(fast, again)
     monkeypatch.setenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST", "0")
     slow = K.flashsvd_mlp_dual_split_triton_v2(*g, b2.cuda())
     monkeypatch.delenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST")
