@@ -853,7 +853,12 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     if (type == FSVD_PH_EMBED) {
       const int q = DF_I(dv, share_q), r = DF_I(dv, share_r), N = DF_I(dv, N);
       const int n0 = w * q + min(w, r), n1 = n0 + q + (w < r ? 1 : 0);
-      const uint16_t* row = static_cast<const uint16_t*>(DF_P(dv, W)) + token * (int64_t)N;
+      // K > 0 is the number of rows of the table: a token outside it (a caller's mistake, or the index the argmax
+      // leaves when no logit compares) must not become an address; row 0 is read instead and the step reports it
+      const int V = DF_I(dv, K);
+      long long tk = token;
+      if (V > 0 && (tk < 0 || tk >= V)) { tk = 0; raise_error(st, p, w); }
+      const uint16_t* row = static_cast<const uint16_t*>(DF_P(dv, W)) + tk * (int64_t)N;
       const uint32_t tg = DF_TAG16(dv, out0, epoch);
       void* out = DF_P(dv, out0);
       for (int n = n0 + tid; n < n1; n += kT) st_tag16(out, n, tg, row[n]);
@@ -920,6 +925,12 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         if (tid == 0) {
           for (int i = 1; i < kT / 64; ++i)
             if (red[i] > best || (red[i] == best && ired[i] < best_i)) { best = red[i]; best_i = ired[i]; }
+          // no logit compared greater than -inf (all NaN): there is no greedy token; token 0 stands in and the step says so
+          if (best_i == 0x7fffffff) {
+            best_i = 0;
+            __hip_atomic_store(&st->err, p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            st->err_wg = w;
+          }
           long long* log = static_cast<long long*>(DF_P(dv, plain_out));
           if (log) log[st->step] = best_i;
           st->token = best_i;

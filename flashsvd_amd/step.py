@@ -177,6 +177,7 @@ class PersistentDecoder:
         e = Phase()
         e.type, e.N = PH_EMBED, d
         emb = inner.embed_tokens.weight
+        e.K = int(emb.shape[0])          # rows of the table: the kernel refuses a token outside it
         if tuple(emb.shape)[1] != d or not emb.is_contiguous():
             raise ValueError("embedding table must be a contiguous [V, hidden] matrix")
         e.W[0] = emb.data_ptr()
@@ -333,11 +334,16 @@ class PersistentDecoder:
         return (t - t0).clamp_min(0).float() / 100.0
 
     def check(self) -> None:
-        """Synchronise and raise if a step timed out waiting for a hand-off."""
+        """Synchronise and raise if a step reported an error: a hand-off that never arrived (time-out), an input token
+        outside the embedding table, or logits none of which compares (all NaN: there is no greedy token)."""
         st = self.state.cpu()
         if int(st[1]) != 0:
-            raise DecodeStepError(f"decode step gave up in phase {int(st[1]) - 1} (workgroup {int(st[6])}); "
-                                  "clear with reset_error() after finding the cause")
+            p = int(st[1]) - 1
+            names = self.phase_names() if hasattr(self, "phase_names") else []
+            what = f" ({names[p]})" if 0 <= p < len(names) else ""
+            raise DecodeStepError(f"decode step failed in phase {p}{what} (workgroup {int(st[6])}): time-out of a hand-off, "
+                                  "token outside the embedding table, or no comparable logit; clear with reset_error() "
+                                  "after finding the cause")
 
     def reset_error(self) -> None:
         """Clear a time-out.  The failed step left half-written vectors that carry its tags, so the
@@ -448,7 +454,7 @@ class DenseStepDecoder(PersistentDecoder):
             ph.append(p)
 
         e = Phase()
-        e.type, e.N = PH_EMBED, d
+        e.type, e.N, e.K = PH_EMBED, d, int(embed.shape[0])
         e.W[0] = embed.data_ptr()
         e.out0 = _tb(self.XA, L + 1, 0)
         ph.append(e)

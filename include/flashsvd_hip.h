@@ -312,7 +312,8 @@ typedef struct fsvd_tagbuf {
 typedef struct fsvd_phase {
   int32_t type, epilogue;
   int32_t N, K, nmat, mode;     /* rows per matrix, row length, matrices, SwiGLU rounding mode; the staged     */
-                                /* input has nmat * K elements                                                 */
+                                /* input has nmat * K elements.  EMBED: K = rows of the table (0: unchecked);  */
+                                /* a token outside [0, K) reads row 0 and sets state->err                      */
   int32_t H, Hk, Dh, nsplit, rope_len, S;   /* on a GEMV, H > 0 marks the q | k | v head expansion: N = (H + 2*Hk) * Dh  */
                                 /* rows in three groups that read in[0:K], in[K:2K], in[2K:3K]                 */
   float fparam;                 /* GEMV with norm_w: RMSNorm eps; ATTN: softmax scale                          */
@@ -341,7 +342,8 @@ typedef struct fsvd_phase {
 
 typedef struct fsvd_step_state {
   int32_t epoch;      /* advanced by every completed step; seeds the tags                                     */
-  int32_t err;        /* 0 ok; else 1 + index of the phase whose input never arrived                          */
+  int32_t err;        /* 0 ok; else 1 + index of the phase whose input never arrived, of the EMBED phase that */
+                      /* met a token outside its table, or of the ARGMAX phase that found no comparable logit */
   int32_t pos;        /* position of the token being decoded = number of keys already in the cache            */
   int32_t step;       /* tokens generated so far (index into the token log)                                   */
   int64_t token;      /* input token of the next step (written by ARGMAX)                                     */

@@ -209,6 +209,41 @@ def test_timeout_path_leaves_cleanly_and_recovers():
     assert torch.equal(toks, ref_tok), f"after recovery: {toks.tolist()} vs {ref_tok.tolist()}"
 
 
+def test_bad_token_and_nan_logits_are_errors_not_addresses():
+    """A token outside the embedding table must not become a row address, and logits none of which compares (NaN) must
+    not leave the argmax's 'nothing yet' index as the next token: both end the step normally with its error flag set."""
+    from flashsvd_amd.step import DecodeStepError, PersistentDecoder
+    mw, prompt = _small()
+    model = model_from_oracle(mw)
+    ref_tok, _, _ = O.greedy_decode(mw, prompt, 4, "dense", return_hidden=True)
+    Lp = prompt.shape[1]
+    cache, tok0 = _prefill(model, prompt, 12)
+    dec = PersistentDecoder(model, cache)
+    for bad in (2048 + 7, -3, 2 ** 31 - 1):
+        dec.set_state(torch.tensor([[bad]]), Lp)
+        dec.step(1)
+        with pytest.raises(DecodeStepError):
+            dec.check()
+        dec.reset_error()
+    norm_w = model.model.norm.weight
+    keep = norm_w.detach().clone()
+    norm_w.data.fill_(float("nan"))
+    cache._seen_tokens = Lp
+    dec.set_state(tok0, Lp)
+    dec.step(2)                           # the second launch returns at once: the flag is already set
+    with pytest.raises(DecodeStepError):
+        dec.check()
+    dec.reset_error()
+    assert int(dec.tokens()[0]) == 0
+    norm_w.data.copy_(keep)
+    cache._seen_tokens = Lp
+    dec.set_state(tok0, Lp)
+    dec.step(3)
+    dec.check()
+    toks = torch.cat([tok0.cpu(), dec.tokens().cpu()[None, :]], 1)
+    assert torch.equal(toks, ref_tok), f"after recovery: {toks.tolist()} vs {ref_tok.tolist()}"
+
+
 def test_phase_list_validation():
     """The host check rejects lists the kernel cannot run (no launch happens)."""
     import ctypes
