@@ -43,6 +43,8 @@ def _parse():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense bf16 comparator leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-breakdown", action="store_true", help="also time every kernel type of the step")
+    ap.add_argument("--no-kernel-configs", action="store_true",
+                    help="skip the kernel-level configurations (for profiler runs: their launches share kernel names with the step's)")
     ap.add_argument("--engine", choices=["persistent", "graph", "both"], default="both",
                     help="persistent: one resident kernel per token (fsvd_decode_step); graph: one HIP graph of the "
                          "per-operator kernels per token; both: time both, the headline value is the persistent step")
@@ -146,6 +148,32 @@ def kernel_configs(model, cache, dec, n_layers: int) -> dict:
         us = per_layer_kernel_us(mlp, n_layers)
         nb = 3 * (d + CFG["intermediate_size"]) * CFG["mlp_rank"] * 2 + B * 2 * d * 2
         out[f"swiglu_mlp_bs{B}"] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3, "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS}
+    # the same two blocks as short phase lists of the resident step kernel (embedding row -> the block's phases, one launch
+    # per call, hand-off between phases inside the kernel): 8 layers' weights in rotation, launches queued back to back
+    from flashsvd_amd.step import PersistentDecoder
+    nrot = min(8, n_layers)
+    nb_attn = out["attention_block_bs1_ctx512"]["bytes_per_call"]
+    nb_mlp = out["swiglu_mlp_bs1"]["bytes_per_call"]
+    for part, key, nb in (("attention", "attention_block_bs1_ctx512_resident_step", nb_attn), ("mlp", "swiglu_mlp_bs1_resident_step", nb_mlp)):
+        decs = [PersistentDecoder(model, cache, part=part, layer=i, max_new_tokens=8) for i in range(nrot)]
+        for dd in decs:
+            dd.set_state(1234, PROMPT_LEN)
+            dd.step(2)
+        torch.cuda.synchronize()
+        reps = 40
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for dd in decs:
+                dd.step(1)
+        e1.record()
+        torch.cuda.synchronize()
+        for dd in decs:
+            dd.check()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * nrot)
+        out[key] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3, "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS,
+                    "phases": len(decs[0].phase_names())}
+        del decs
     # the operators under the reference's own names and operand layouts (x @ W): flashsvd_mlp_dual_split_triton_v2 on
     # PUp / PGate [B,1,R], GateU / UpU [R,D], DownV [D,R], DownU [R,d], and reconstruct_qkv_token_shared on the split of a
     # packed coefficient row and bases [H,R,Dh]; operands of 8 layers in rotation (1.1 GB: nothing comes from a cache)
@@ -307,10 +335,16 @@ def run_lowrank(args):
         res["persistent"] = dict(tok_s=B * args.steps / t_decode, ms_per_step=t_decode * 1000.0 / args.steps,
                                  kernel_us_per_launch=e0.elapsed_time(e1) * 1000.0 / args.steps,
                                  workgroups=pdec.nwg, last_token=int(pdec.tokens()[-1]))
+        # where the launch's time goes, from inside the kernel: per phase kind (averaged over layers and 8 workgroups)
+        # wait for the input | weight stream | epilogue and publication, microseconds
+        prof = pdec.phase_profile(32)
+        res["persistent"]["phase_profile_us"] = {k: {m: round(x, 2) for m, x in v.items()} for k, v in prof.items()}
+        pdec.check()
         del pdec
     best = res.get("persistent") or res["graph"]
     res["tok_s"], res["ms_per_step"] = best["tok_s"], best["ms_per_step"]
-    res["kernel_configs"] = kernel_configs(model, cache, dec, args.layers)
+    if not args.no_kernel_configs:
+        res["kernel_configs"] = kernel_configs(model, cache, dec, args.layers)
     legs = kernel_legs(model, cache, dec)
     name = "mlp_gate_up_u+swiglu"
     fn, nbytes = legs[name]
@@ -549,6 +583,84 @@ def run_stress():
     }
 
 
+def run_stress_model(steps: int = 8, warmup: int = 2, layers: int = 32):
+    """The stress configuration as one model: the 7B shape at parameter ratio ~0.8 (attention rank 1664, MLP rank 2432),
+    bf16.  Leg 1: prefill of 8 prompts x 2048 tokens into the rank-space cache.  Leg 2: greedy decode at batch 16 over
+    a 4096-token context held in rank space (the prompt is prefilled for real, 16 x 4096 tokens, untimed), K rebuilt
+    in-kernel, one HIP graph per token.  Both legs are matrix-core bound at these sizes, so each reports flop / time
+    against the dense bf16 peak next to its token rate; `attention_share` prices the rank-space attention kernels alone
+    (their per-layer time, measured separately, x layers / step time)."""
+    import torch
+    from flashsvd_amd import llama
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.runtime.cache import FlashSVDLegacySparseKVCache
+    R, RM, ctx, Bd, Bp, Tp = 1664, 2432, 4096, 16, 8, 2048
+    cfg = dict(CFG, attn_rank=R, mlp_rank=RM, num_layers=int(layers), max_position_embeddings=ctx + 64)
+    d, H, Dh, D, V, L = cfg["hidden_size"], cfg["num_heads"], cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"], int(layers)
+    def say(msg):                       # progress on stderr: the legs take tens of seconds
+        print(f"[stress] {msg}", file=sys.stderr, flush=True)
+
+    model = llama.materialize(llama.build_model(**cfg), "cuda", torch.bfloat16, seed=0)
+    model.eval()
+    say(f"model of {L} layers on the device")
+    gen = torch.Generator().manual_seed(11)
+    peak = 2500e12
+    lin_flop_tok = 2.0 * (8 * d * R + 3 * (d + D) * RM)          # factor products per token per layer
+
+    # ---- leg 1: prefill 8 x 2048
+    ids = torch.randint(0, V, (Bp, Tp), generator=gen).cuda()
+    times = []
+    with torch.no_grad():
+        for it in range(3):
+            cache = FlashSVDLegacySparseKVCache(model.config, max_batch_size=Bp, max_cache_len=Tp + 8, device="cuda", dtype=torch.bfloat16)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = model(ids, past_key_values=cache, cache_position=torch.arange(Tp), logits_to_keep=1)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            say(f"prefill {Bp} x {Tp}: {times[-1]:.3f} s")
+            del cache, out
+    t_pre = min(times[1:])
+    attn_flop_pre = 3 * 2.0 * Bp * Tp * R * H * Dh + 2 * 2.0 * Bp * H * Dh * Tp * (Tp + 1) / 2     # head expansion + causal attention
+    flop_pre = L * (Bp * Tp * lin_flop_tok + attn_flop_pre) + 2.0 * Bp * d * V
+    prefill = {"batch": Bp, "prompt_len": Tp, "s": t_pre, "cold_s": times[0], "tok_s": Bp * Tp / t_pre, "flop": flop_pre,
+               "TFLOPs": flop_pre / t_pre / 1e12, "frac_of_bf16_mfma_peak": flop_pre / t_pre / peak}
+
+    # ---- leg 2: decode at batch 16, context 4096, rank-space cache
+    ids = torch.randint(0, V, (Bd, ctx), generator=gen).cuda()
+    cache = FlashSVDLegacySparseKVCache(model.config, max_batch_size=Bd, max_cache_len=ctx + steps + warmup + 8, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        out = model(ids, past_key_values=cache, cache_position=torch.arange(ctx), logits_to_keep=1)
+    tok = out.logits[:, -1].float().argmax(-1, keepdim=True)
+    del out
+    torch.cuda.synchronize()
+    say(f"context of {Bd} x {ctx} tokens prefilled into the rank-space cache")
+    dec = GraphedDecoder(model, cache, Bd)
+    dec.set_state(tok, ctx)
+    dec.capture()
+    say("decode step captured")
+    for _ in range(warmup):
+        dec.step()
+    torch.cuda.synchronize()
+    say("timing the decode steps")
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        dec.step()
+    torch.cuda.synchronize()
+    t_step = (time.perf_counter() - t0) / steps
+    attn_flop_dec = 2.0 * Bd * ctx * R * H * Dh + 2.0 * Bd * H * ctx * R + 2.0 * Bd * H * R * Dh     # K rebuild, rank-space PV, expansion
+    flop_step = L * (Bd * lin_flop_tok + attn_flop_dec) + 2.0 * Bd * d * V
+    cache_bytes = L * 2 * Bd * ctx * R * 2
+    weight_bytes = L * 2 * (8 * d * R + 3 * (d + D) * RM) + 2 * d * V
+    decode = {"batch": Bd, "context": ctx, "steps": steps, "ms_per_step": t_step * 1e3, "tok_s": Bd / t_step, "flop_per_step": flop_step,
+              "TFLOPs": flop_step / t_step / 1e12, "frac_of_bf16_mfma_peak": flop_step / t_step / peak,
+              "attention_flop_per_layer": attn_flop_dec, "bytes_per_step": cache_bytes + weight_bytes,
+              "GB/s": (cache_bytes + weight_bytes) / t_step / 1e9, "engine": "per-operator HIP graph", "kv_cache": "rank space (FlashSVDLegacySparseKVCache)"}
+    del dec, cache, model
+    torch.cuda.empty_cache()
+    return {"model": f"{L}-layer 7B shape, attention rank {R}, MLP rank {RM}", "prefill": prefill, "decode": decode}
+
+
 def run_quant(args):
     """Config 4 with every factor linear as group-wise int4 (PackedQuantLinear, group 128, asymmetric): the persistent step
     streams the packed nibbles (phases with wbits == 4), the per-operator graph uses fsvd_linear_q4 / fsvd_swiglu_linear_q4."""
@@ -647,8 +759,16 @@ def main():
                           "data": "synthetic", "quant": q}))
         return
     if args.stress:
-        print(json.dumps({"metric": "stress attention kernels, 7B-shape rank-0.8, per layer", "n_gpus": 1, "dtype": "bf16", "data": "synthetic",
-                          "stress": run_stress()}))
+        kern = run_stress()
+        print("[stress] attention kernels timed", file=sys.stderr, flush=True)
+        mp = run_stress_model(steps=max(2, min(args.steps, 8)), warmup=max(1, min(args.warmup, 2)), layers=args.layers)
+        t_att = kern["rank_space_decode_attention_b16_ctx4096_r1664"]["ms_per_layer"]
+        mp["decode"]["attention_share"] = t_att * args.layers / mp["decode"]["ms_per_step"]
+        mp["decode"]["attention_kernel_frac_of_bf16_mfma_peak"] = kern["rank_space_decode_attention_b16_ctx4096_r1664"]["frac_of_bf16_mfma_peak"]
+        print(json.dumps({"metric": "stress decode tok/s, 7B-shape rank-0.8, batch 16, context 4096, rank-space cache", "value": mp["decode"]["tok_s"],
+                          "unit": "tok/s", "n_gpus": 1, "steps": mp["decode"]["steps"], "dtype": "bf16", "data": "synthetic",
+                          "config": {"workload": mp["model"] + "; prefill 8 x 2048, then decode batch 16 at context 4096", "layers": args.layers},
+                          "model_pass": mp, "kernels": kern}))
         return
     lr = run_lowrank(args)
     if args.prefill_only:
@@ -668,7 +788,7 @@ def main():
         "step_hbm": {"bytes_per_token": lr["step_bytes"], "GB/s": lr["step_GBs"], "frac_of_peak": lr["step_GBs"] / HBM_PEAK_GBS},
         "prefill_s": lr["prefill_s"],
         "prefill": lr["prefill"],
-        "kernel_configs": lr["kernel_configs"],
+        "kernel_configs": lr.get("kernel_configs"),
     }
     for k in ("persistent", "graph", "swiglu_roofline"):
         if k in lr:

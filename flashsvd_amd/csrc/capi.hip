@@ -596,7 +596,7 @@ int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host
   if (validate) {
     FSVD_REQUIRE_PTR(phases_host, fn);
     const int nwg = decode_step_workgroups();
-    if (nwg <= 0) { set_last_error("%s: cannot query the device", fn); return kErrLaunch; }
+    if (nwg <= 0) return kErrLaunch;   // decode_step_workgroups left the reason in the last-error text
     const int rc = validate_decode_step(phases_host, nphase, nwg);
     if (rc != kOk) return rc;
   }
@@ -608,7 +608,7 @@ int fsvd_decode_step_trace(const fsvd_phase* phases_dev, const fsvd_phase* phase
   const char* fn = "fsvd_decode_step_trace";
   FSVD_REQUIRE_PTR(phases_dev, fn); FSVD_REQUIRE_PTR(state, fn); FSVD_REQUIRE_PTR(trace, fn);
   const int nwg = decode_step_workgroups();
-  if (nwg <= 0) { set_last_error("%s: cannot query the device", fn); return kErrLaunch; }
+  if (nwg <= 0) return kErrLaunch;
   if (nphase <= 0 || wg_stride <= 0) { set_last_error("%s: bad arguments", fn); return kErrBadShape; }
   const size_t need = (size_t)((nwg + wg_stride - 1) / wg_stride) * nphase * 4;
   if (trace_words < need) { set_last_error("%s: trace buffer holds %zu words, %zu needed", fn, trace_words, need); return kErrWorkspace; }

@@ -953,23 +953,34 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
 // ---------------------------------------------------------------------------------------------
 static int g_step_wgs = 0;
 
+// One workgroup per compute unit, all of them resident at once: a workgroup that waits for a hand-off spins, so a
+// workgroup that is still waiting for a free compute unit would never get one.  The grid is therefore refused unless the
+// runtime's own occupancy calculation places at least one workgroup of every instantiation on a compute unit (registers,
+// LDS, waves); what the calculation cannot see - other kernels holding compute units while a step runs - is the
+// caller's to avoid: nothing else may execute on the device during a step (a starved step ends by its spin limit with
+// the error flag set, it does not hang).
 int decode_step_workgroups() {
   if (g_step_wgs > 0) return g_step_wgs;
   int dev = 0;
   hipDeviceProp_t prop;
-  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<false, false>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)kSmemBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<true, false>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)kSmemBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<false, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)kSmemBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(decode_step_kernel<true, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)kSmemBytes) != hipSuccess)
+  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+    set_last_error("fsvd_decode_step: cannot query the device");
+    return 0;
+  }
+  const void* fns[4] = {reinterpret_cast<const void*>(decode_step_kernel<false, false>), reinterpret_cast<const void*>(decode_step_kernel<true, false>),
+                        reinterpret_cast<const void*>(decode_step_kernel<false, true>), reinterpret_cast<const void*>(decode_step_kernel<true, true>)};
+  for (const void* fn : fns) {
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSmemBytes) != hipSuccess) {
+      set_last_error("fsvd_decode_step: the device refuses %zu bytes of dynamic LDS per workgroup", kSmemBytes);
       return 0;
-    attr_set = true;
+    }
+    int resident = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, fn, kT, kSmemBytes) != hipSuccess || resident < 1) {
+      set_last_error("fsvd_decode_step: a workgroup of the step kernel (%d threads, %zu bytes of LDS) does not fit a compute unit of "
+                     "this device, so its grid of one workgroup per compute unit cannot be co-resident", kT, kSmemBytes);
+      (void)hipGetLastError();
+      return 0;
+    }
   }
   g_step_wgs = prop.multiProcessorCount;
   return g_step_wgs;
@@ -1145,7 +1156,7 @@ bool decode_step_has_q4(const fsvd_phase* host, int nph) {
 int launch_decode_step(const fsvd_phase* dev, int nph, fsvd_step_state* st, unsigned long long* trace, int trace_stride, bool q4,
                        hipStream_t stream) {
   const int nwg = decode_step_workgroups();
-  if (nwg <= 0) { set_last_error("fsvd_decode_step: cannot query the device"); return kErrLaunch; }
+  if (nwg <= 0) return kErrLaunch;   // the reason is in the last-error text
   if (trace) {
     if (q4) hipLaunchKernelGGL((decode_step_kernel<true, true>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, trace, trace_stride);
     else hipLaunchKernelGGL((decode_step_kernel<true, false>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, trace, trace_stride);

@@ -437,9 +437,13 @@ class SVD_LlamaAttention(nn.Module):
 
 
 def _prefill_tokens_rank(self, x, cache, cache_position=None, *, norm_weight=None, eps=1e-6, residual=None):
-    """Rank-space prefill with the decode kernel: coefficients of all T tokens go into the cache,
-    then the tokens of a sequence are the kernel's batch rows bound to one cache row (batch stride 0)
-    with key counts start+t+1.  K tiles are rebuilt once per query, so this is meant for short prompts."""
+    """Rank-space prefill: the coefficients of all T tokens go into the cache.  head_dim 128 with ranks that are multiples
+    of 8 (and T >= 16) then takes the matrix-core route of the dense-cache prompt pass: q of the new tokens and K / V of
+    the whole context (cached coefficients included) are rebuilt ONCE into temporaries, rotation fused, and causal flash
+    attention runs over them — K rounded to bf16 before the scores, as the reference's prompt kernel does
+    (kernels/attn/prefill/rope_sdpa.py:133-199).  Other shapes (or FLASHSVD_AMD_PREFILL=decode) use the decode kernel:
+    the tokens of a sequence are its batch rows bound to one cache row (batch stride 0) with key counts start+t+1, K
+    tiles rebuilt per query — short prompts only."""
     from .kernels.rank_decode import rank_decode
     from .quant import is_quantized
     if is_quantized(*self._factor_modules()):
@@ -458,9 +462,34 @@ def _prefill_tokens_rank(self, x, cache, cache_position=None, *, norm_weight=Non
     pvc[:B, start:start + T] = p[..., rq + rk:]
     cache._layer_initialized[self.layer_idx] = True
     cache._note_seen(self.layer_idx, T, cache_position)
+    a = torch.empty(B, T, H * Dh, device=x.device, dtype=x.dtype)
+    mfma_ok = Dh == 128 and rq % 8 == 0 and rk % 8 == 0 and rv % 8 == 0 and T >= 16 \
+        and os.getenv("FLASHSVD_AMD_PREFILL", "mfma").strip().lower() != "decode"
+    if mfma_ok:
+        n_ctx = start + T
+        q = torch.empty(B, T, H, Dh, device=x.device, dtype=x.dtype)
+        kt = torch.empty(B, n_ctx, Hk, Dh, device=x.device, dtype=x.dtype)
+        vt = torch.empty_like(kt)
+        zero = torch.zeros(B, device=x.device, dtype=torch.int32)
+        pos_q = torch.full((B,), start, device=x.device, dtype=torch.int32)
+        wq, wk, wv = self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight
+        if start == 0:
+            hip_ops.lowrank_expand_heads_multi(
+                [dict(p=p[..., :rq], u=wq, num_heads=H, out=q, rotate=True),
+                 dict(p=p[..., rq:rq + rk], u=wk, num_heads=Hk, out=kt, rotate=True),
+                 dict(p=p[..., rq + rk:], u=wv, num_heads=Hk, out=vt)],
+                head_dim=Dh, cos=rope[0], sin=rope[1], positions=zero)
+        else:
+            hip_ops.lowrank_expand_heads(p[..., :rq], wq, num_heads=H, head_dim=Dh, out=q, cos=rope[0], sin=rope[1], positions=pos_q)
+            hip_ops.lowrank_expand_heads_multi(
+                [dict(p=pkc[:B, :n_ctx], u=wk, num_heads=Hk, out=kt, rotate=True),
+                 dict(p=pvc[:B, :n_ctx], u=wv, num_heads=Hk, out=vt)],
+                head_dim=Dh, cos=rope[0], sin=rope[1], positions=zero)
+        hip_ops.attn_prefill(q, kt, vt, q_pos0=pos_q, causal=True, out=a.view(B, T, H, Dh))
+        po = hip_ops.linear(a, self.o_v_proj.weight)
+        return hip_ops.linear(po, self.o_u_proj.weight, residual=residual)
     q = hip_ops.linear(p[..., :rq].contiguous(), self.q_u_proj.weight).view(B, T, H, Dh)
     lens = torch.arange(start + 1, start + T + 1, device=x.device, dtype=torch.int32)
-    a = torch.empty(B, T, H * Dh, device=x.device, dtype=x.dtype)
     for b in range(B):
         # the rotation position of query t is its own key count - 1, which rotate_q uses
         rank_decode(q[b], pkc[b:b + 1].expand(T, -1, -1), pvc[b:b + 1].expand(T, -1, -1), self.k_u_proj.weight,

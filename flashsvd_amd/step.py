@@ -39,8 +39,16 @@ class PersistentDecoder:
     number of heads.  Models outside these limits decode through ``graphs.GraphedDecoder``.
     """
 
-    def __init__(self, model, cache, *, mode: int | None = None, max_new_tokens: int = 4096):
+    def __init__(self, model, cache, *, mode: int | None = None, max_new_tokens: int = 4096, part: str = "model",
+                 layer: int = 0):
+        """``part``: "model" (the whole token), or — for timing one block through the same machinery — "attention"
+        (embedding row -> the attention half of layer ``layer``, ending at its residual add) or "mlp" (embedding row ->
+        the MLP half of that layer).  A part has no argmax phase: token and position stay where ``set_state`` put them."""
         from .llama import _packed_rows, mlp_rounding_mode
+        if part not in ("model", "attention", "mlp"):
+            raise ValueError(f"part must be 'model', 'attention' or 'mlp', got {part!r}")
+        self.part = part
+        layer_index = int(layer)
         if not isinstance(cache, FlashSVDV15DenseKVCache):
             raise TypeError("PersistentDecoder needs a FlashSVDV15DenseKVCache")
         lib = _lib.load()
@@ -58,18 +66,19 @@ class PersistentDecoder:
                              "(FlashSVDV15DenseKVCache defaults to float16: pass dtype=torch.bfloat16)")
         if inner.embed_tokens.weight.dtype != torch.bfloat16 or inner.norm.weight.dtype != torch.bfloat16:
             raise ValueError("PersistentDecoder needs a bfloat16 embedding table and final norm")
-        for li, layer in enumerate(inner.layers):
+        layers = list(inner.layers) if part == "model" else [inner.layers[layer_index]]
+        for li, layer in enumerate(layers):
             for nm, p_ in layer.named_parameters():
                 if p_.is_floating_point() and p_.dtype != torch.bfloat16:
                     raise ValueError(f"PersistentDecoder needs bfloat16 weights; layer {li} {nm} is {p_.dtype}")
         self.nwg = int(lib.fsvd_decode_step_workgroups())
         if self.nwg <= 0:
-            raise RuntimeError("fsvd_decode_step_workgroups: cannot query the device")
+            raise RuntimeError((lib.fsvd_last_error() or b"").decode() or "fsvd_decode_step_workgroups: cannot query the device")
         H = int(cfg.num_attention_heads)
         Hk = int(getattr(cfg, "num_key_value_heads", H))
         Dh = int(getattr(cfg, "head_dim", None) or cfg.hidden_size // H)
         d = int(cfg.hidden_size)
-        L = len(inner.layers)
+        L = len(layers)
         V = int(model.lm_head.weight.shape[0])
         if self.nwg % H != 0:
             raise ValueError(f"{self.nwg} workgroups are not a multiple of {H} heads")
@@ -87,7 +96,7 @@ class PersistentDecoder:
         from .quant import PackedQuantLinear, is_quantized, pack_quant_rows
         # a layer is either all bf16 factors or all group-wise int4 factors (PackedQuantLinear, no bias, K % 256 == 0)
         layer_q4 = []
-        for li, layer in enumerate(inner.layers):
+        for li, layer in enumerate(layers):
             mods = [*layer.self_attn._factor_modules(), *layer.mlp._factor_modules()]
             if not is_quantized(*mods):
                 layer_q4.append(False)
@@ -103,7 +112,7 @@ class PersistentDecoder:
         # ranks may differ from layer to layer (buffers take the largest); within a layer q, k and v share
         # one rank because their head expansion is a single grouped product
         ranks = []
-        for li, layer in enumerate(inner.layers):
+        for li, layer in enumerate(layers):
             at, mlp = layer.self_attn, layer.mlp
             rq, rk, rv = at._qkv_rank_tuple()
             if not (rq == rk == rv):
@@ -116,7 +125,7 @@ class PersistentDecoder:
         if not ranks:
             raise ValueError("PersistentDecoder needs at least one layer")
         Rq, Ro, Rm, Rd = (max(r[i] for r in ranks) for i in range(4))
-        D = int(inner.layers[0].mlp.gate_u_proj.out_features)
+        D = int(layers[0].mlp.gate_u_proj.out_features)
         self.XA, self.XB = tagged(d), tagged(d)
         self.P, self.QKV = tagged(3 * Rq), tagged((H + 2 * Hk) * Dh)
         self.PART, self.A = tagged64(H * nsplit * (Dh + 2)), tagged(H * Dh)
@@ -181,15 +190,16 @@ class PersistentDecoder:
         if tuple(emb.shape)[1] != d or not emb.is_contiguous():
             raise ValueError("embedding table must be a contiguous [V, hidden] matrix")
         e.W[0] = emb.data_ptr()
-        e.out0 = _tb(self.XA, L + 1, 0)
+        e.out0 = _tb(self.XB, L, 0) if part == "mlp" else _tb(self.XA, L + 1, 0)     # an MLP part starts at the mid-layer state
         ph.append(e)
-        for l, layer in enumerate(inner.layers):
+        for l, layer in enumerate(layers):
             at, mlp = layer.self_attn, layer.mlp
             at._ensure_runtime_state()
             mlp._ensure_runtime_state()
             rq, ro, rm, rd = ranks[l]
-            cache._ensure_layer_spec(l, h=Hk, dh=Dh)
-            kc, vc = cache.key_cache[l][0], cache.value_cache[l][0]      # [S, Hk, Dh]
+            lc = l if part == "model" else layer_index                    # the layer's index in the cache
+            cache._ensure_layer_spec(lc, h=Hk, dh=Dh)
+            kc, vc = cache.key_cache[lc][0], cache.value_cache[lc][0]    # [S, Hk, Dh]
             n1, n2 = layer.input_layernorm, layer.post_attention_layernorm
             xin, xmid, xout = _tb(self.XA, L + 1, l), _tb(self.XB, L, l), _tb(self.XA, L + 1, l + 1)
             q4 = layer_q4[l]
@@ -204,7 +214,9 @@ class PersistentDecoder:
                     raise ValueError(f"PersistentDecoder: int4 factors of layer {l} cannot share a stream (group sizes differ)")
                 return pk, int(mods[0].group_size)
 
-            if q4:
+            if part == "mlp":
+                pass
+            elif q4:
                 w, gs = triple(at.q_v_proj, at.k_v_proj, at.v_v_proj)
                 gemv([w], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon, q4=gs)
                 w, gs = triple(at.q_u_proj, at.k_u_proj, at.v_u_proj)
@@ -216,22 +228,29 @@ class PersistentDecoder:
                 qkv_u = _packed_rows([at.q_u_proj, at.k_u_proj, at.v_u_proj])
                 self._keep.append(qkv_u)
                 gemv([qkv_u], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
-            a = Phase()
-            a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
-            a.fparam = 1.0 / math.sqrt(Dh)
-            a.cos, a.sin, a.rope_len = cos.data_ptr(), sin.data_ptr(), int(cos.shape[0])
-            a.k_cache, a.v_cache, a.sc_s, a.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
-            a.inp, a.out0 = _tb(self.QKV, L, l), _tb(self.PART, L, l)
-            ph.append(a)
-            m = Phase()
-            m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
-            m.inp, m.out0 = _tb(self.PART, L, l), _tb(self.A, L, l)
-            ph.append(m)
-            if q4:
-                w, gs = triple(at.o_v_proj)
-                gemv([w], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l), q4=gs)
-                w, gs = triple(at.o_u_proj)
-                gemv([w], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin, q4=gs)
+            if part != "mlp":
+                a = Phase()
+                a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
+                a.fparam = 1.0 / math.sqrt(Dh)
+                a.cos, a.sin, a.rope_len = cos.data_ptr(), sin.data_ptr(), int(cos.shape[0])
+                a.k_cache, a.v_cache, a.sc_s, a.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
+                a.inp, a.out0 = _tb(self.QKV, L, l), _tb(self.PART, L, l)
+                ph.append(a)
+                m = Phase()
+                m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
+                m.inp, m.out0 = _tb(self.PART, L, l), _tb(self.A, L, l)
+                ph.append(m)
+                if q4:
+                    w, gs = triple(at.o_v_proj)
+                    gemv([w], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l), q4=gs)
+                    w, gs = triple(at.o_u_proj)
+                    gemv([w], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin, q4=gs)
+                else:
+                    gemv([at.o_v_proj.weight], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
+                    gemv([at.o_u_proj.weight], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
+            if part == "attention":
+                pass
+            elif q4:
                 w, gs = triple(mlp.gate_v_proj, mlp.up_v_proj)
                 gemv([w], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon, q4=gs)
                 (wg, gs), (wu, gs2) = triple(mlp.gate_u_proj), triple(mlp.up_u_proj)
@@ -243,22 +262,21 @@ class PersistentDecoder:
                 w, gs = triple(mlp.down_u_proj)
                 gemv([w], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid, q4=gs)
             else:
-                gemv([at.o_v_proj.weight], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
-                gemv([at.o_u_proj.weight], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
                 gemv([mlp._packed_gu_v], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
                 gemv([mlp.gate_u_proj.weight, mlp.up_u_proj.weight], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2,
                      epi=EP_SWIGLU)
                 gemv([mlp.down_v_proj.weight], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
                 gemv([mlp.down_u_proj.weight], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
-            cache._layer_initialized[l] = True
-        fn = inner.norm
-        gemv([model.lm_head.weight], V, d, _tb(self.XA, L + 1, L), _tb(self.CAND, 1, 0), norm=fn.weight,
-             eps=fn.variance_epsilon, epi=EP_LOGITS, plain=self.logits)
-        g = Phase()
-        g.type = PH_ARGMAX
-        g.inp = _tb(self.CAND, 1, 0)
-        g.plain_out = self.token_log.data_ptr()
-        ph.append(g)
+            cache._layer_initialized[lc] = True
+        if part == "model":
+            fn = inner.norm
+            gemv([model.lm_head.weight], V, d, _tb(self.XA, L + 1, L), _tb(self.CAND, 1, 0), norm=fn.weight,
+                 eps=fn.variance_epsilon, epi=EP_LOGITS, plain=self.logits)
+            g = Phase()
+            g.type = PH_ARGMAX
+            g.inp = _tb(self.CAND, 1, 0)
+            g.plain_out = self.token_log.data_ptr()
+            ph.append(g)
 
         self._finish(ph, dev)
 
@@ -290,7 +308,16 @@ class PersistentDecoder:
         self._host_steps = 0
 
     def step(self, n: int = 1) -> None:
-        """Decode ``n`` tokens greedily (asynchronous; read them with ``tokens()``)."""
+        """Decode ``n`` tokens greedily (asynchronous; read them with ``tokens()``).  A part ("attention" / "mlp") runs its
+        phases ``n`` times at the position of ``set_state``: nothing advances."""
+        if getattr(self, "part", "model") != "model":
+            stream = torch.cuda.current_stream().cuda_stream
+            for _ in range(int(n)):
+                rc = self.lib.fsvd_decode_step(self.dev_phases.data_ptr(), ctypes.addressof(self.host_phases), self.nph,
+                                               self.state.data_ptr(), 0 if self._validated else 1, stream)
+                _lib.check("fsvd_decode_step", rc)
+                self._validated = True
+            return
         if self._host_pos + n > self.S:
             raise IndexError(f"decode position {self._host_pos + n - 1} outside the cache (max {self.S})")
         if self._host_steps + n > self.token_log.numel():
@@ -309,6 +336,11 @@ class PersistentDecoder:
                    "down_v", "down_u")
 
     def phase_names(self) -> list:
+        part = getattr(self, "part", "model")
+        if part == "attention":
+            return ["embed", *self.PHASE_NAMES[1:7]]
+        if part == "mlp":
+            return ["embed", *self.PHASE_NAMES[7:]]
         return ["embed"] + [n for _ in range(self.L) for n in self.PHASE_NAMES[1:]] + ["lm_head", "argmax"]
 
     def trace_step(self, wg_stride: int = 32) -> torch.Tensor:
@@ -361,8 +393,10 @@ class PersistentDecoder:
         return self.token_log[: self._host_steps].clone()
 
     def hidden(self) -> torch.Tensor:
-        """Final-layer hidden state of the last step, bf16 [hidden]."""
-        return ((self.XA & 0xFFFF) << 16).view(torch.float32).to(torch.bfloat16)
+        """Final-layer hidden state of the last step, bf16 [hidden] (part "attention": the state after the attention
+        half's residual add; part "mlp": after the MLP half's)."""
+        buf = self.XB if getattr(self, "part", "model") == "attention" else self.XA
+        return ((buf & 0xFFFF) << 16).view(torch.float32).to(torch.bfloat16)
 
 
     # ------------------------------------------------------------------ GraphedDecoder-compatible face

@@ -351,7 +351,10 @@ typedef struct fsvd_step_state {
   int32_t spin_limit; /* polls before a workgroup gives up; 0 = default (about a second)                       */
 } fsvd_step_state;
 
-/* Workgroups the step kernel runs with on the current device (one per compute unit). */
+/* Workgroups the step kernel runs with on the current device (one per compute unit), or 0 with fsvd_last_error() when
+ * the device cannot hold one workgroup of the kernel per compute unit (the grid must be co-resident: workgroups wait
+ * for each other's results).  While a step runs nothing else may execute on the device; a step that is starved of
+ * compute units ends by its spin limit with state->err set. */
 int fsvd_decode_step_workgroups(void);
 /* Fill the derived fields of a host-side phase list for `workgroups` workgroups (call before uploading it). */
 int fsvd_decode_step_prepare(fsvd_phase* phases_host, int nphase, int workgroups);

@@ -244,6 +244,42 @@ def test_bad_token_and_nan_logits_are_errors_not_addresses():
     assert torch.equal(toks, ref_tok), f"after recovery: {toks.tolist()} vs {ref_tok.tolist()}"
 
 
+def test_block_parts_match_the_per_operator_blocks():
+    """PersistentDecoder(part="attention" | "mlp", layer=i): embedding row -> one block's phases, the lists the benchmark
+    times.  Same arithmetic and rounding points as the per-operator block on the same input (fp32 sums split
+    differently): outputs agree to bf16 resolution, and the attention part appends the same K / V row."""
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.step import PersistentDecoder
+    mw, prompt = _small()
+    model = model_from_oracle(mw)
+    Lp = prompt.shape[1]
+    cache, _ = _prefill(model, prompt, 8)
+    ref_cache, _ = _prefill(model, prompt, 8)
+    gd = GraphedDecoder(model, ref_cache, 1)
+    tok = 77
+    x = model.model.embed_tokens.weight[tok][None].clone()
+    pos = torch.full((1,), Lp, dtype=torch.int32, device="cuda")
+    for li in (0, 2):
+        layer = model.model.layers[li]
+        n1, n2 = layer.input_layernorm, layer.post_attention_layernorm
+        want_a = layer.self_attn.decode_token(x, ref_cache, pos, norm_weight=n1.weight, eps=n1.variance_epsilon, residual=x,
+                                              rope=gd.rope, attn_ws=gd.attn_ws, nsplit=gd.nsplit)
+        want_m = layer.mlp.run(x, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=x)
+        for part, want in (("attention", want_a), ("mlp", want_m)):
+            dec = PersistentDecoder(model, cache, part=part, layer=li)
+            assert dec.phase_names()[0] == "embed" and len(dec.phase_names()) == dec.nph
+            dec.set_state(tok, Lp)
+            dec.step(3)                   # a part leaves token and position alone: three identical runs
+            dec.check()
+            assert int(dec.state.cpu()[2]) == Lp
+            b = bounds(want.float().cpu())
+            assert_close_bf16(dec.hidden()[None].cpu(), want.float().cpu(), f"{part} part of layer {li}", abs_tol=2 * b["abs_tol"], rel_tol=2e-2)
+        for got, ref, nm in ((cache.key_cache[li], ref_cache.key_cache[li], "K"), (cache.value_cache[li], ref_cache.value_cache[li], "V")):
+            assert_close_bf16(got[:, Lp:Lp + 1].cpu(), ref[:, Lp:Lp + 1].cpu(), f"{nm} row of layer {li}", abs_tol=float("inf"), rel_tol=2e-2)
+    with pytest.raises(ValueError):
+        PersistentDecoder(model, cache, part="sideways")
+
+
 def test_phase_list_validation():
     """The host check rejects lists the kernel cannot run (no launch happens)."""
     import ctypes
