@@ -428,16 +428,30 @@ __device__ __forceinline__ bool stage_input(const void* in, int in_len, uint32_t
 // 16-byte loads, 2.2 us as 4-byte loads, whatever the number of workgroups reading), and every word carries its own tag,
 // so a load wider than the atomic unit loses nothing: a word that is torn or stale fails its tag and is polled again.
 // The loads are written as instructions: the compiler's forms of a coherent 16-byte load are a volatile access, which
-// it follows with a full wait (one round trip per load), or four atomic ones.  All loads of a round are issued, then
-// ONE wait covers them; the operands of that wait tie every later use of the registers to it.
-__device__ __forceinline__ void ld_coh128_issue(u32x4_t& dst, const void* base, int idx128) {
-  const uint64_t addr = reinterpret_cast<uint64_t>(base) + ((uint64_t)(uint32_t)idx128 << 4);
-  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(dst) : "v"(addr) : "memory");
+// it follows with a full wait (one round trip per load), or four atomic ones.  All loads of a round AND the wait for
+// them are ONE asm statement: the compiler takes an asm statement's outputs as valid the moment it ends, so a load
+// left in flight behind its statement may find its destination registers copied, or handed to something else (an
+// address), before the data lands.  Outputs are early-clobber: every address is read before the statement ends.
+#define FSVD_LDC "global_load_dwordx4 %"
+__device__ __forceinline__ void ld_coh128_round(u32x4_t (&v)[2], const uint64_t (&a)[2]) {
+  asm volatile(FSVD_LDC "0, %2, off sc0 sc1\n\t" FSVD_LDC "1, %3, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+               : "=&v"(v[0]), "=&v"(v[1])
+               : "v"(a[0]), "v"(a[1])
+               : "memory");
 }
+__device__ __forceinline__ void ld_coh128_round(u32x4_t (&v)[8], const uint64_t (&a)[8]) {
+  asm volatile(FSVD_LDC "0, %8, off sc0 sc1\n\t" FSVD_LDC "1, %9, off sc0 sc1\n\t" FSVD_LDC "2, %10, off sc0 sc1\n\t"
+               FSVD_LDC "3, %11, off sc0 sc1\n\t" FSVD_LDC "4, %12, off sc0 sc1\n\t" FSVD_LDC "5, %13, off sc0 sc1\n\t"
+               FSVD_LDC "6, %14, off sc0 sc1\n\t" FSVD_LDC "7, %15, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+               : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+               : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7])
+               : "memory");
+}
+#undef FSVD_LDC
 template <int NS>
 __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uint32_t tin, const uint32_t* norm_w, float eps,
                                                  const fsvd_step_state* st, int limit, uint16_t* xs, float* red) {
-  static_assert(NS == 2 || NS == 8, "the wait below names the registers of a round");
+  static_assert(NS == 2 || NS == 8, "ld_coh128_round exists for rounds of 2 and of 8 loads");
   const int tid = threadIdx.x;
   const int nw128 = in_len >> 2;                 // in_len is a multiple of 128
   const bool norm = norm_w != nullptr;
@@ -450,15 +464,13 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
 #pragma unroll
       for (int j = 0; j < NS; ++j) nwt[j] = reinterpret_cast<const uint2*>(norm_w)[min(base + j * kT + tid, nw128 - 1)];
     }
+    // every slot of the round is loaded, index clamped (a slot past the end re-reads the last word and is not used)
     u32x4_t v[NS];
+    uint64_t adr[NS];
 #pragma unroll
-    for (int j = 0; j < NS; ++j) {
-      v[j] = u32x4_t{0u, 0u, 0u, 0u};
-      if (base + j * kT < nw128) ld_coh128_issue(v[j], in, min(base + j * kT + tid, nw128 - 1));
-    }
-    if (NS == 2) asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1])::"memory");
-    else asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2 % NS]), "+v"(v[3 % NS]), "+v"(v[4 % NS]), "+v"(v[5 % NS]),
-                      "+v"(v[6 % NS]), "+v"(v[7 % NS])::"memory");
+    for (int j = 0; j < NS; ++j)
+      adr[j] = reinterpret_cast<uint64_t>(in) + ((uint64_t)(uint32_t)min(base + j * kT + tid, nw128 - 1) << 4);
+    ld_coh128_round(v, adr);
 #pragma unroll
     for (int j = 0; j < NS; ++j) {
       if (base + j * kT >= nw128) break;
