@@ -34,9 +34,11 @@ def _tb(t: torch.Tensor, uses: int, use: int) -> TagBuf:
 class PersistentDecoder:
     """``PersistentDecoder(model, cache)`` then ``set_state(token, position)``, ``step(n)``, ``tokens()``.
 
-    Requirements (checked): batch 1, bf16, dense KV cache, head_dim 128, equal q/k/v ranks, every
-    matrix row length a multiple of 128, and a device whose compute-unit count is a multiple of the
-    number of heads.  Models outside these limits decode through ``graphs.GraphedDecoder``.
+    Requirements (checked): batch 1, bf16, dense KV cache, head_dim 128, hidden and intermediate sizes that are multiples
+    of 128, and a device whose compute-unit count is a multiple of the number of heads.  Factor ranks are free for bf16
+    factors (unequal q / k / v ranks, ranks that are not multiples of 128 or smaller than the workgroup count are served
+    from zero-padded copies made once, at the cost of their memory); int4 layers need equal q / k / v ranks and row
+    lengths that are multiples of 256.  Models outside these limits decode through ``graphs.GraphedDecoder``.
     """
 
     def __init__(self, model, cache, *, mode: int | None = None, max_new_tokens: int = 4096, part: str = "model",
@@ -109,19 +111,30 @@ class PersistentDecoder:
                 if gs < m.in_features and (gs < 32 or gs & (gs - 1)):
                     raise ValueError(f"PersistentDecoder: int4 group size {gs} is not a power of two >= 32")
             layer_q4.append(True)
-        # ranks may differ from layer to layer (buffers take the largest); within a layer q, k and v share
-        # one rank because their head expansion is a single grouped product
-        ranks = []
+        # Ranks may differ from layer to layer and, for bf16 factors, between q, k and v: the kernel wants one rank per
+        # row group, a multiple of 128 (a lane group covers 128 elements of a row) and at least one row per workgroup,
+        # so factors that do not fit are copied once into zero-padded twins (zero rows / columns contribute nothing:
+        # results are bit-identical to the unpadded product).  int4 factors are streamed as stored and must fit as they are.
+        def rank_up(r: int) -> int:
+            return max((int(r) + 127) // 128 * 128, (self.nwg + 127) // 128 * 128)
+
+        ranks, padded = [], []
         for li, layer in enumerate(layers):
             at, mlp = layer.self_attn, layer.mlp
             rq, rk, rv = at._qkv_rank_tuple()
-            if not (rq == rk == rv):
-                raise ValueError(f"PersistentDecoder needs equal q/k/v ranks in layer {li} (got {rq}/{rk}/{rv}; pad them "
-                                 "to a common multiple of 128)")
             rm = int(mlp.gate_v_proj.out_features)
             if int(mlp.up_v_proj.out_features) != rm:
                 raise ValueError(f"PersistentDecoder needs equal gate/up ranks in layer {li}")
-            ranks.append((rq, int(at.o_v_proj.out_features), rm, int(mlp.down_v_proj.out_features)))
+            ro, rd = int(at.o_v_proj.out_features), int(mlp.down_v_proj.out_features)
+            if layer_q4[li]:
+                if not (rq == rk == rv):
+                    raise ValueError(f"PersistentDecoder needs equal q/k/v ranks in an int4 layer (layer {li}: {rq}/{rk}/{rv})")
+                ranks.append((rq, ro, rm, rd))
+                padded.append(None)
+                continue
+            Rq, Ro, Rm, Rd = rank_up(max(rq, rk, rv)), rank_up(ro), rank_up(rm), rank_up(rd)
+            ranks.append((Rq, Ro, Rm, Rd))
+            padded.append(dict(qkv=not (rq == rk == rv == Rq), o=ro != Ro, gu=rm != Rm, d=rd != Rd))
         if not ranks:
             raise ValueError("PersistentDecoder needs at least one layer")
         Rq, Ro, Rm, Rd = (max(r[i] for r in ranks) for i in range(4))
@@ -151,6 +164,16 @@ class PersistentDecoder:
             lo = scales.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
             hi = (zeros.to(torch.int32) + 128) << 16
             return (lo | hi).contiguous()
+
+        def pad_rows(w, n):       # zero rows below: outputs that are zero
+            out_ = torch.zeros(n, w.shape[1], dtype=torch.bfloat16, device=dev)
+            out_[:w.shape[0]] = w.data
+            return out_
+
+        def pad_cols(w, n):       # zero columns to the right: inputs that are multiplied by zero
+            out_ = torch.zeros(w.shape[0], n, dtype=torch.bfloat16, device=dev)
+            out_[:, :w.shape[1]] = w.data
+            return out_
 
         def gemv(W, N, K, inp, out, *, nmat=1, norm=None, eps=0.0, epi=EP_STORE, aux=None, plain=None, groups=None, q4=None):
             p = Phase()
@@ -221,6 +244,18 @@ class PersistentDecoder:
                 gemv([w], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon, q4=gs)
                 w, gs = triple(at.q_u_proj, at.k_u_proj, at.v_u_proj)
                 gemv([w], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh), q4=gs)
+            elif padded[l]["qkv"]:
+                # unequal or unaligned q / k / v ranks: [q_v; k_v; v_v] with each block padded to rq rows, and the head bases
+                # with their columns padded to rq
+                aq, ak, av = at._qkv_rank_tuple()
+                pv = torch.zeros(3 * rq, d, dtype=torch.bfloat16, device=dev)
+                qu = torch.zeros((H + 2 * Hk) * Dh, rq, dtype=torch.bfloat16, device=dev)
+                for i, (m_v, m_u, r_, row0, rows) in enumerate(((at.q_v_proj, at.q_u_proj, aq, 0, H * Dh), (at.k_v_proj, at.k_u_proj, ak, H * Dh, Hk * Dh),
+                                                                (at.v_v_proj, at.v_u_proj, av, (H + Hk) * Dh, Hk * Dh))):
+                    pv[i * rq:i * rq + r_] = m_v.weight.data
+                    qu[row0:row0 + rows, :r_] = m_u.weight.data
+                gemv([pv], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
+                gemv([qu], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
             else:
                 gemv([at._packed_qkv_v], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
                 # q, k, v head expansion as one GEMV over the row-packed [q_u; k_u; v_u] (the three module
@@ -246,8 +281,11 @@ class PersistentDecoder:
                     w, gs = triple(at.o_u_proj)
                     gemv([w], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin, q4=gs)
                 else:
-                    gemv([at.o_v_proj.weight], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
-                    gemv([at.o_u_proj.weight], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
+                    w_ov, w_ou = at.o_v_proj.weight, at.o_u_proj.weight
+                    if padded[l]["o"]:
+                        w_ov, w_ou = pad_rows(w_ov, ro), pad_cols(w_ou, ro)
+                    gemv([w_ov], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
+                    gemv([w_ou], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
             if part == "attention":
                 pass
             elif q4:
@@ -262,11 +300,20 @@ class PersistentDecoder:
                 w, gs = triple(mlp.down_u_proj)
                 gemv([w], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid, q4=gs)
             else:
-                gemv([mlp._packed_gu_v], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
-                gemv([mlp.gate_u_proj.weight, mlp.up_u_proj.weight], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2,
-                     epi=EP_SWIGLU)
-                gemv([mlp.down_v_proj.weight], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
-                gemv([mlp.down_u_proj.weight], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
+                w_guv, w_gu, w_uu = mlp._packed_gu_v, mlp.gate_u_proj.weight, mlp.up_u_proj.weight
+                if padded[l]["gu"]:
+                    am = int(mlp.gate_v_proj.out_features)
+                    w_guv = torch.zeros(2 * rm, d, dtype=torch.bfloat16, device=dev)
+                    w_guv[:am] = mlp.gate_v_proj.weight.data
+                    w_guv[rm:rm + am] = mlp.up_v_proj.weight.data
+                    w_gu, w_uu = pad_cols(w_gu, rm), pad_cols(w_uu, rm)
+                w_dv, w_du = mlp.down_v_proj.weight, mlp.down_u_proj.weight
+                if padded[l]["d"]:
+                    w_dv, w_du = pad_rows(w_dv, rd), pad_cols(w_du, rd)
+                gemv([w_guv], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
+                gemv([w_gu, w_uu], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2, epi=EP_SWIGLU)
+                gemv([w_dv], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
+                gemv([w_du], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
             cache._layer_initialized[lc] = True
         if part == "model":
             fn = inner.norm

@@ -280,6 +280,44 @@ def test_block_parts_match_the_per_operator_blocks():
         PersistentDecoder(model, cache, part="sideways")
 
 
+def test_unequal_and_unaligned_ranks_are_served_from_padded_twins():
+    """Real checkpoints carry per-matrix ranks such as 1492: q / k / v ranks that differ, ranks that are not multiples of
+    128 or that are smaller than the workgroup count.  The persistent step copies such factors once into zero-padded
+    twins; zero rows and columns add nothing, so every step must agree with the per-operator engine on the same model
+    (same rounding points, fp32 sums split differently) exactly as it does for aligned ranks."""
+    from types import SimpleNamespace
+    from flashsvd_amd import llama
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.step import PersistentDecoder
+    cfg = SimpleNamespace(hidden_size=1024, num_attention_heads=8, num_key_value_heads=4, head_dim=128, intermediate_size=2048,
+                          num_hidden_layers=2, vocab_size=2048, rope_theta=10000.0, rms_norm_eps=1e-6, hidden_act="silu",
+                          max_position_embeddings=256)
+    with torch.device("meta"):
+        model = llama.SVDLlamaForCausalLM(cfg, attn_ranks=dict(q=200, k=136, v=264, o=72), mlp_rank=300)
+    model = llama.materialize(model, "cuda", BF16, seed=9, std=0.05)
+    prompt = torch.randint(0, 2048, (1, 29), generator=torch.Generator().manual_seed(2))
+    Lp, n_new = prompt.shape[1], 9
+    cache_k, tok0 = _prefill(model, prompt, n_new + 4)
+    dec_k = GraphedDecoder(model, cache_k, 1)
+    dec_k.set_state(tok0, Lp)
+    toks_k, logits_k = [tok0.clone()], [None]
+    for _ in range(n_new - 1):
+        toks_k.append(dec_k.eager_step().clone())
+        logits_k.append(dec_k.logits[0, -1].float().cpu())
+    toks_k = torch.cat(toks_k, 1).cpu()
+    cache_p, tok0p = _prefill(model, prompt, n_new + 4)
+    dec = PersistentDecoder(model, cache_p)
+    for s in range(1, n_new):                 # teacher-forced with the per-operator engine's tokens
+        dec.set_state(toks_k[:, s - 1], Lp + s - 1)
+        dec.step(1)
+        lk = logits_k[s]
+        assert_close_bf16(dec.logits[None].cpu(), lk[None], f"logits at step {s}", abs_tol=3 * bounds(lk)["abs_tol"], rel_tol=3e-2)
+        _tie_aware(int(dec.tokens()[0]), int(toks_k[0, s]), lk, f"step {s}")
+    for li in range(2):
+        for got, ref, nm in ((cache_p.key_cache[li], cache_k.key_cache[li], "K"), (cache_p.value_cache[li], cache_k.value_cache[li], "V")):
+            assert_close_bf16(got[:, Lp:Lp + n_new - 1], ref[:, Lp:Lp + n_new - 1], f"{nm} rows layer {li}", abs_tol=float("inf"), rel_tol=3e-2)
+
+
 def test_phase_list_validation():
     """The host check rejects lists the kernel cannot run (no launch happens)."""
     import ctypes
