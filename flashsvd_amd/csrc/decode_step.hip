@@ -470,20 +470,27 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
 #pragma unroll
     for (int j = 0; j < NS; ++j)
       adr[j] = reinterpret_cast<uint64_t>(in) + ((uint64_t)(uint32_t)min(base + j * kT + tid, nw128 - 1) << 4);
-    ld_coh128_round(v, adr);
+    // A round whose words have not all arrived is read again as a whole after a short sleep: one trip through memory per
+    // attempt for the whole vector, however many producers are late (retrying word by word pays a trip per late word)
+    for (int spins = 0;; ++spins) {
+      ld_coh128_round(v, adr);
+      bool late = false;
+#pragma unroll
+      for (int j = 0; j < NS; ++j) {
+        if (base + j * kT >= nw128) break;
+        if (base + j * kT + tid < nw128)
+          late = late || (v[j].x >> 16) != tin || (v[j].y >> 16) != tin || (v[j].z >> 16) != tin || (v[j].w >> 16) != tin;
+      }
+      if (!__any(late ? 1 : 0)) break;
+      if (spins >= limit || ((spins & 255) == 255 && ld_err(st) != 0)) { fail = fail || late; break; }
+      __builtin_amdgcn_s_sleep(2);
+    }
 #pragma unroll
     for (int j = 0; j < NS; ++j) {
       if (base + j * kT >= nw128) break;
       const int q = base + j * kT + tid;
       if (q < nw128) {
-        uint32_t a0 = v[j].x, a1 = v[j].y, a2 = v[j].z, a3 = v[j].w;
-        if ((a0 >> 16) != tin || (a1 >> 16) != tin) {
-          if (!poll_pair(in, 2 * q, tin, st, limit, a0, a1)) fail = true;
-        }
-        if ((a2 >> 16) != tin || (a3 >> 16) != tin) {
-          if (!poll_pair(in, 2 * q + 1, tin, st, limit, a2, a3)) fail = true;
-        }
-        a0 &= 0xffffu; a1 &= 0xffffu; a2 &= 0xffffu; a3 &= 0xffffu;
+        const uint32_t a0 = v[j].x & 0xffffu, a1 = v[j].y & 0xffffu, a2 = v[j].z & 0xffffu, a3 = v[j].w & 0xffffu;
         if (norm) {
           const float f0 = bf16_bits_to_f32(a0), f1 = bf16_bits_to_f32(a1), f2 = bf16_bits_to_f32(a2), f3 = bf16_bits_to_f32(a3);
           ss += (f0 * f0 + f1 * f1) + (f2 * f2 + f3 * f3);
