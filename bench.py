@@ -43,6 +43,7 @@ def _parse():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense bf16 comparator leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-breakdown", action="store_true", help="also time every kernel type of the step")
+    ap.add_argument("--no-stress", action="store_true", help="skip the stress configuration's whole-model pass in the default line")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the kernel-level configurations (for profiler runs: their launches share kernel names with the step's)")
     ap.add_argument("--engine", choices=["persistent", "graph", "both"], default="both",
@@ -809,6 +810,13 @@ def main():
             "torch_graph": dict(dn, how="same shape, dense bf16 weights, torch.matmul (hipBLASLt) projections, torch elementwise ops, "
                                         "same attention kernel, one HIP graph per token"),
             "bandwidth_ratio_dense_over_lowrank": ds["bytes_per_token"] / lr["step_bytes"]}
+    if not args.no_stress and args.layers == CFG["num_layers"]:
+        # the stress configuration (rank ratio ~0.8) as one model: prefill 8 x 2048, decode batch 16 at context 4096 over the
+        # rank-space cache; `bench.py --stress` prints the same with the attention kernels timed alone
+        try:
+            line["stress_rank08"] = run_stress_model(steps=4, warmup=1, layers=args.layers)
+        except Exception as exc:      # the headline line must not be lost to a failure of a side leg
+            line["stress_rank08"] = {"error": f"{type(exc).__name__}: {exc}"}
     line["cpu_baseline"] = None if args.no_cpu else run_cpu_baseline()
     print(json.dumps(line))
 
