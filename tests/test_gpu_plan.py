@@ -73,16 +73,22 @@ def test_exact_and_packed_backends_agree(monkeypatch):
 
 
 def test_persistent_step_with_ranks_that_differ_per_layer():
-    """Layer 0 padded to 256 / 384, layer 1 to 384 / 512: the step takes each layer's own ranks."""
+    """Unpadded ranks first, then layer 0 padded to 256 / 384 and layer 1 to 384 / 512: the step takes each layer's own ranks."""
     from flashsvd_amd import plan as P
     from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
     from flashsvd_amd.step import PersistentDecoder
     mw, prompt = _odd()
     model = model_from_oracle(mw)
-    from flashsvd_amd._lib import FlashSVDHipError
-    with pytest.raises(FlashSVDHipError, match="multiple of 128"):
-        cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=64, device="cuda", dtype=BF16)
-        PersistentDecoder(model, cache).step(1)
+    # ranks off the 128 grid (204 / 300 here) are served from zero-padded twins the decoder builds itself
+    n0, Lp0 = 5, prompt.shape[1]
+    toks_0, _ = _decode(model, prompt, n0)
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=Lp0 + n0 + 4, device="cuda", dtype=BF16)
+    out = model(prompt.cuda(), past_key_values=cache, cache_position=torch.arange(Lp0))
+    t0 = out.logits[:, -1].float().argmax(-1, keepdim=True)
+    dec0 = PersistentDecoder(model, cache)
+    dec0.set_state(t0, Lp0)
+    dec0.step(n0 - 1)
+    assert [int(t0)] + dec0.tokens().cpu().tolist() == toks_0
     l0, l1 = model.model.layers
     P.pad_attention_ranks(l0.self_attn, 128, "uniform_layer")
     P.pad_mlp_ranks(l0.mlp, 128)
