@@ -106,6 +106,7 @@ struct RankDecodeArgs {
   uint16_t* out; int64_t so_b, so_h;                // [B,H,Dh]
   int B, H, Hk, Dh, S, Rk, Rv, nsplit;
   float scale;
+  float* scores = nullptr; int64_t score_ld = 0;    // [B,H,score_ld] fp32 in the registered scratch (set by the launcher for long caches)
 };
 int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st);
 int launch_rankkv_append(const uint16_t* pk, int64_t ldpk, const uint16_t* pv, int64_t ldpv, uint16_t* pkc, int64_t spk_b, int64_t spk_s,

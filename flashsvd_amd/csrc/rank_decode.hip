@@ -13,6 +13,14 @@
 //   The 8 accumulator tiles of a wave hold K[16 keys x 128 d]; d and d+64 sit in the same lane,
 //   so the rotate-half RoPE is register-local; scores fold over the 16 lanes of a DPP row.
 // Stage 2, grid (H, B): merge the splits in order, normalise, multiply by v_u[h].
+//
+// Long caches shared by the heads (B * H * S of a million and more), when the caller has registered scratch: stage 1 is
+// three launches.  The score kernel is stage 1 cut after the scores (it keeps neither softmax state nor rank-space sums,
+// which frees the registers for four key sub-tiles per wave, and stages k_u as well as Pk with loads that write LDS
+// directly); rank_decode_softmax_kernel turns the scores of a split into weights in place; rank_decode_pv_kernel
+// accumulates p . Pv on the matrix cores for up to 32 heads at once, so that a Pv row is read once per head tile instead
+// of once per head.  In the one-kernel form every head re-reads the Pv rows of its batch row from L2 (as much traffic
+// again as k_u and Pk together) and multiplies them on the vector ALU.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -47,7 +55,10 @@ template <int KS, bool PKL, bool DEEP> struct RankDecodeLds {
 // are loaded straight into a ring of three LDS stages as well, two chunks ahead, and the Pk pieces two chunks ahead into
 // two slots per wave; the wave's load counter and one barrier per chunk are the synchronisation.  Batch 1, 512 keys,
 // rank 1024: 24 us -> see the launcher.
-template <int REP, int KS, bool PKL, bool DEEP = false>
+// SC (long caches, scratch registered): the kernel stops at the scores.  It writes s[b, key, h] = q_h . K_key * scale to
+// a.scores and leaves the softmax and the rank-space accumulation to rank_decode_softmax_kernel / rank_decode_pv_kernel,
+// which read every Pv row once for a group of heads instead of once per head.
+template <int REP, int KS, bool PKL, bool DEEP = false, bool SC = false>
 __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(RankDecodeArgs a) {
   static_assert(!DEEP || (PKL && KS == 1), "the deep form is built for single sub-tiles with Pk through LDS");
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
@@ -240,6 +251,64 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         }
       }
       __syncthreads();                                           // the last stages are read out before the next tile refills them
+    } else if constexpr (PKL && SC) {
+      // k_u chunks straight into the two LDS stages as well (no registers, no LDS stores), one chunk ahead: lane -> LDS row
+      // wave * 32 + i * 8 + lane / 8 and position lane % 8 of the stage, which holds piece (lane % 8) ^ (row % 8) of head
+      // dimension kd(row) -- the placement store_ku gives the register form.  Addresses are a wave-uniform base plus a
+      // 32-bit byte offset per lane (the launcher checks that the cache of a batch row fits): no 64-bit pointer per piece
+      // to keep and to advance
+      uint32_t kuoff[4], pkoff[KS][2];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = wave * 32 + i * 8 + (lane >> 3);
+        const int rd = ((row >> 4) / 4) * HALF + (row & 15) * 4 + ((row >> 4) % 4);
+        kuoff[i] = (uint32_t)((rd * (int)a.ldku + (((lane & 7) ^ (row & 7)) * 8)) * 2);
+      }
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int row = i * 8 + (lane >> 3);
+          const int pkey = min(kt + (4 * j + wave) * 16 + row, k1 - 1);
+          pkoff[j][i] = (uint32_t)pkey * (uint32_t)(a.spk_s * 2) + (uint32_t)((((lane & 7) ^ (row & 7)) * 8) * 2);
+        }
+      const char* kub = reinterpret_cast<const char*>(ku_h);
+      const char* pkb = reinterpret_cast<const char*>(pk_b);
+      const auto issue_ku = [&](int c) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          __builtin_amdgcn_global_load_lds((gptr_t)(kub + c * 128 + (size_t)kuoff[i]), (lptr_t)(smem + (c & 1) * (DH * KROW * 2) + (wave * 32 + i * 8) * 128), 16, 0, 0);
+      };
+      const auto issue_pk = [&](int c) {
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(pkb + c * 128 + (size_t)pkoff[j][i]), (lptr_t)(myslot + j * 2048 + i * 1024), 16, 0, 0);
+      };
+      // (the barrier that ended the previous tile's last chunk also freed both stages and the slot)
+      issue_ku(0);
+      issue_pk(0);
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      for (int st = 0; st < nstep; ++st) {
+        const int cur = st & 1;
+        read_pk();
+        __builtin_amdgcn_s_waitcnt(0);             // fragments in registers: the slot is free again
+        __builtin_amdgcn_sched_barrier(0);
+        if (st + 1 < nstep) { issue_pk(st + 1); issue_ku(st + 1); }
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+#pragma unroll
+            for (int j = 0; j < KS; ++j) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][k], bf, accs[j][t], 0, 0, 0);
+          }
+        }
+        __builtin_amdgcn_s_waitcnt(0);             // this wave's pieces of chunk st + 1 have landed ...
+        __syncthreads();                           // ... everybody's have, and stage cur is read out
+      }
     } else {
     // (the barrier that ended the previous tile's last chunk also freed both buffers)
     load_ku(0);
@@ -311,6 +380,16 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         sc[i] = (wkey0 + lg * 4 + i < k1) ? d : -INFINITY;
         tmax = fmaxf(tmax, sc[i]);
       }
+      if constexpr (SC) {
+        // every lane of a row group holds the group's four scores: lane 0 of the group stores them
+        if (lr == 0) {
+          float* sp = a.scores + ((int64_t)b * a.H + h0 + g) * a.score_ld + wkey0 + lg * 4;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (wkey0 + lg * 4 + i < k1) sp[i] = sc[i];
+        }
+        continue;
+      }
       tmax = wave_max(tmax);
       const float m_new = fmaxf(m_run[g], tmax);
       const float alpha = (m_run[g] == -INFINITY) ? 0.f : __expf(m_run[g] - m_new);
@@ -350,6 +429,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
     }
   }
 
+  if constexpr (SC) return;
   // ---- merge the 4 waves (each has its own running max) and write the split's partial
 #pragma unroll
   for (int g = 0; g < REP; ++g) {
@@ -369,6 +449,161 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
     for (int r = tid; r < a.Rv; r += kRdThreads)
       a.ws_acc[slot * a.Rv + r] = w[0] * tbuf[0][r] + w[1] * tbuf[1][r] + w[2] * tbuf[2][r] + w[3] * tbuf[3][r];
     if (tid == 0) { a.ws_m[slot] = M; a.ws_l[slot] = L; }
+  }
+}
+
+// Softmax weights of one split of one (batch row, head), in place: scores[b, h, key] -> exp(s - m[b,h,split]), with the
+// split's maximum and sum to ws_m / ws_l (the merge kernel folds the splits as it does for the one-kernel form).
+// grid (nsplit, H, B), 256 threads.  Rows of the score buffer are a.score_ld floats apart.
+__global__ __launch_bounds__(kRdThreads) void rank_decode_softmax_kernel(RankDecodeArgs a) {
+  __shared__ float red[4];
+  const int s = blockIdx.x, h = blockIdx.y, b = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int n_keys = a.seqlens[b] + a.seqlen_add;
+  n_keys = max(0, min(n_keys, a.S));
+  int per = (n_keys + a.nsplit - 1) / a.nsplit;
+  per = (per + kRdTileKeys - 1) / kRdTileKeys * kRdTileKeys;
+  const int k0 = min(s * per, n_keys), k1 = min(n_keys, k0 + per);
+  float* sp = a.scores + ((int64_t)b * a.H + h) * a.score_ld;
+  float m = -INFINITY;
+  for (int k = k0 + tid; k < k1; k += kRdThreads) m = fmaxf(m, sp[k]);
+  m = wave_max(m);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float l = 0.f;
+  for (int k = k0 + tid; k < k1; k += kRdThreads) {
+    const float p = __expf(sp[k] - M);
+    sp[k] = p;
+    l += p;
+  }
+  l = wave_sum(l);
+  if (lane == 0) red[wave] = l;
+  __syncthreads();
+  if (tid == 0) {
+    const int64_t slot = ((int64_t)b * a.H + h) * a.nsplit + s;
+    a.ws_m[slot] = M;                              // -inf for an empty split: the merge gives it weight 0
+    a.ws_l[slot] = ((red[0] + red[1]) + red[2]) + red[3];
+  }
+}
+
+// Acc[b, h, split, r] = sum over the split's keys of p[b, h, key] * Pv[b, key, r] on the matrix cores, for 16 * MT heads at
+// once: a Pv row is read once per head tile instead of once per head (coefficient caches shared by the heads only).
+// grid (r slices of 64, nsplit * head tiles, B), 4 waves; wave w owns the 16 columns r0 + 16 w of the slice.  Per block of
+// 64 keys the workgroup stages Pv[64 keys x 64 r] in LDS (one 16-byte load per thread and 32 keys, a block ahead in
+// registers) and every lane gathers its B fragment (8 keys of one column) with 2-byte LDS reads; the A fragments are the
+// weights p[h, 8 keys] straight from the score buffer, split into two bf16 terms (p = hi + lo to 2^-17) so that the sum
+// keeps fp32 weights; fp32 accumulation in key order.
+template <int MT>
+__global__ __launch_bounds__(kRdThreads) void rank_decode_pv_kernel(RankDecodeArgs a) {
+  constexpr int KB = 64, PITCH = 132;              // bytes per LDS row: 8 rows apart = 8 banks apart, the four key groups of a fragment read disjoint banks
+  __shared__ __align__(16) unsigned char tile[2][KB * PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 15, lg = lane >> 4;
+  const int ntile = (a.H + 16 * MT - 1) / (16 * MT);
+  const int s = blockIdx.y / ntile, ht = blockIdx.y % ntile, b = blockIdx.z;
+  const int h0 = ht * 16 * MT;
+  int n_keys = a.seqlens[b] + a.seqlen_add;
+  n_keys = max(0, min(n_keys, a.S));
+  int per = (n_keys + a.nsplit - 1) / a.nsplit;
+  per = (per + kRdTileKeys - 1) / kRdTileKeys * kRdTileKeys;
+  const int k0 = min(s * per, n_keys), k1 = min(n_keys, k0 + per);
+  const int c0 = blockIdx.x * 64;                  // first column of the slice
+  // staging: thread -> key row tid / 8 (+ 32) of the block, 16-byte piece tid % 8 of the 128-byte row slice
+  const int srow = tid >> 3, spiece = tid & 7;
+  const bool scol = c0 + spiece * 8 < a.Rv;        // Rv is a multiple of 8: a piece is inside or outside as a whole
+  const uint16_t* pv_b = a.pv + (int64_t)b * a.spv_b + (scol ? c0 + spiece * 8 : 0);
+  const auto load_block = [&](int kb, u32x4_t (&v)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int key = min(kb + i * 32 + srow, k1 - 1);   // clamped rows carry weight 0
+      v[i] = scol ? *reinterpret_cast<const u32x4_t*>(pv_b + (int64_t)key * a.spv_s) : u32x4_t{0u, 0u, 0u, 0u};
+    }
+  };
+  const auto store_block = [&](int buf, const u32x4_t (&v)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      uint32_t* d = reinterpret_cast<uint32_t*>(&tile[buf][(i * 32 + srow) * PITCH + spiece * 16]);
+      d[0] = v[i].x; d[1] = v[i].y; d[2] = v[i].z; d[3] = v[i].w;
+    }
+  };
+  // weights: lane -> head h0 + mt * 16 + lr, keys kb + ks * 32 + lg * 8 .. + 8
+  const float* prow[MT];
+  bool hlive[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int h = h0 + mt * 16 + lr;
+    hlive[mt] = h < a.H;
+    prow[mt] = a.scores + ((int64_t)b * a.H + (hlive[mt] ? h : 0)) * a.score_ld + lg * 8;
+  }
+  f32x4_t pw[MT][2][2];
+  const auto load_p = [&](int kb) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        // the score rows are padded to a multiple of 64 floats: the loads stay inside the row, keys past k1 are masked below
+        const float* p = prow[mt] + kb + ks * 32;
+        pw[mt][ks][0] = *reinterpret_cast<const f32x4_t*>(p);
+        pw[mt][ks][1] = *reinterpret_cast<const f32x4_t*>(p + 4);
+      }
+  };
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  if (k0 < k1) {
+    u32x4_t nxt[2];
+    load_block(k0, nxt);
+    store_block(0, nxt);
+    int buf = 0;
+    for (int kb = k0; kb < k1; kb += KB, buf ^= 1) {
+      const bool more = kb + KB < k1;
+      if (more) load_block(kb + KB, nxt);
+      load_p(kb);
+      __syncthreads();                             // block kb is in tile[buf]; everybody has left tile[buf ^ 1]
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        uint16_t e[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = *reinterpret_cast<const uint16_t*>(&tile[buf][(ks * 32 + lg * 8 + j) * PITCH + (wave * 16 + lr) * 2]);
+        const u32x4_t bw{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
+                         (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+        const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, bw);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          uint32_t hi[4], lo[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            float x[2];
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+              const int kk = j * 2 + q;
+              const float v = pw[mt][ks][kk >> 2][kk & 3];
+              x[q] = (hlive[mt] && kb + ks * 32 + lg * 8 + kk < k1) ? v : 0.f;
+            }
+            const uint32_t h0b = f32_to_bf16_bits(x[0]), h1b = f32_to_bf16_bits(x[1]);
+            const uint32_t l0b = f32_to_bf16_bits(x[0] - bf16_bits_to_f32((uint16_t)h0b)), l1b = f32_to_bf16_bits(x[1] - bf16_bits_to_f32((uint16_t)h1b));
+            hi[j] = (h0b & 0xffffu) | (h1b << 16);
+            lo[j] = (l0b & 0xffffu) | (l1b << 16);
+          }
+          const bf16x8_t ah = __builtin_bit_cast(bf16x8_t, u32x4_t{hi[0], hi[1], hi[2], hi[3]});
+          const bf16x8_t al = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], lo[2], lo[3]});
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bf, acc[mt], 0, 0, 0);
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, bf, acc[mt], 0, 0, 0);
+        }
+      }
+      if (more) store_block(buf ^ 1, nxt);         // tile[buf ^ 1] was read out before this iteration's barrier
+    }
+  }
+  // element i of a lane: head h0 + mt * 16 + lg * 4 + i, column c0 + wave * 16 + lr
+  const int r = c0 + wave * 16 + lr;
+  if (r < a.Rv) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int h = h0 + mt * 16 + lg * 4 + i;
+        if (h < a.H) a.ws_acc[(((int64_t)b * a.H + h) * a.nsplit + s) * a.Rv + r] = acc[mt][i];
+      }
   }
 }
 
@@ -482,6 +717,16 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   }
   const int rep = a.H / a.Hk;
   dim3 block(kRdThreads);
+  // long caches shared by the heads, with registered scratch: scores -> softmax -> rank-space accumulation per head tile,
+  // as three launches; the scores of the call live in the scratch, [B,H,score_ld] fp32
+  const SplitWorkspace sw = split_workspace();
+  const int64_t score_ld = ((int64_t)a.S + 63) / 64 * 64;
+  const size_t score_floats = (size_t)a.B * a.H * score_ld;
+  const bool three = a.spv_h == 0 && a.S >= 1024 && score_floats >= ((size_t)1 << 20) && sw.part != nullptr &&
+                     sw.part_floats >= score_floats;
+  RankDecodeArgs a3 = a;
+  a3.scores = three ? sw.part : nullptr;
+  a3.score_ld = score_ld;
   // key sub-tiles per pass: long splits amortise every k_u fragment over more keys (any value is correct for any
   // length; short splits would only rebuild clamped keys)
   const int per = (a.S + a.nsplit - 1) / a.nsplit;
@@ -502,12 +747,42 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     }                                                                                                                               \
     hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, PKL_, DEEP_>), dim3(a.nsplit, GY_, a.B), block, lds, st, a);          \
   } while (0)
+#define FSVD_RD_LAUNCH_SC(REP_, KS_, PKL_, GY_)                                                                                      \
+  do {                                                                                                                              \
+    constexpr int lds = RankDecodeLds<KS_, PKL_, false>::kBytes;                                                                    \
+    static bool granted = false;                                                                                                    \
+    if (!granted && lds >= 48 * 1024) {                                                                                             \
+      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_decode_partial_kernel<REP_, KS_, PKL_, false, true>), \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);                                         \
+      if (ea != hipSuccess) { set_last_error("%s: cannot reserve %d bytes of LDS: %s", fn, lds, hipGetErrorString(ea)); return kErrLaunch; } \
+      granted = true;                                                                                                               \
+    }                                                                                                                               \
+    hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, PKL_, false, true>), dim3(a.nsplit, GY_, a.B), block, lds, st, a3);   \
+  } while (0)
 #define FSVD_RD_LAUNCH(REP_, KS_, GY_)                                                                                              \
   do {                                                                                                                              \
     if (KS_ == 1 && deep) FSVD_RD_LAUNCH_T(REP_, 1, true, true, GY_);                                                               \
     else if (pkl) FSVD_RD_LAUNCH_T(REP_, KS_, true, false, GY_);                                                                    \
     else FSVD_RD_LAUNCH_T(REP_, KS_, false, false, GY_);                                                                            \
   } while (0)
+  if (three) {
+    // the score kernel addresses the Pk rows of a batch row and the k_u rows of a head with 32-bit byte offsets when it
+    // loads them straight into LDS
+    const bool pk3 = pkl && ((int64_t)a.S * a.spk_s + a.Rk) * 2 < ((int64_t)1 << 32) && ((int64_t)a.Dh * a.ldku + a.Rk) * 2 < ((int64_t)1 << 32);
+    if (rep % 4 == 0) { if (pk3) FSVD_RD_LAUNCH_SC(4, 1, true, a.Hk * (rep / 4)); else FSVD_RD_LAUNCH_SC(4, 1, false, a.Hk * (rep / 4)); }
+    else if (rep % 2 == 0) { if (pk3) FSVD_RD_LAUNCH_SC(2, 2, true, a.Hk * (rep / 2)); else FSVD_RD_LAUNCH_SC(2, 2, false, a.Hk * (rep / 2)); }
+    else if (per >= 256) { if (pk3) FSVD_RD_LAUNCH_SC(1, 4, true, a.Hk * rep); else FSVD_RD_LAUNCH_SC(1, 4, false, a.Hk * rep); }
+    else { if (pk3) FSVD_RD_LAUNCH_SC(1, 2, true, a.Hk * rep); else FSVD_RD_LAUNCH_SC(1, 2, false, a.Hk * rep); }
+    hipError_t e3 = hipGetLastError();
+    if (e3 != hipSuccess) { set_last_error("%s: score launch failed: %s", fn, hipGetErrorString(e3)); return kErrLaunch; }
+    hipLaunchKernelGGL(rank_decode_softmax_kernel, dim3(a.nsplit, a.H, a.B), block, 0, st, a3);
+    const int mt = a.H > 16 ? 2 : 1;
+    const dim3 gpv((a.Rv + 63) / 64, a.nsplit * ((a.H + 16 * mt - 1) / (16 * mt)), a.B);
+    if (mt == 2) hipLaunchKernelGGL(rank_decode_pv_kernel<2>, gpv, block, 0, st, a3);
+    else hipLaunchKernelGGL(rank_decode_pv_kernel<1>, gpv, block, 0, st, a3);
+    e3 = hipGetLastError();
+    if (e3 != hipSuccess) { set_last_error("%s: softmax / accumulation launch failed: %s", fn, hipGetErrorString(e3)); return kErrLaunch; }
+  } else
   if (rep % 4 == 0) FSVD_RD_LAUNCH(4, 1, a.Hk * (rep / 4));
   else if (rep % 2 == 0) {
     if (ks >= 2) FSVD_RD_LAUNCH(2, 2, a.Hk * (rep / 2));
@@ -517,6 +792,7 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     else FSVD_RD_LAUNCH(1, 1, a.Hk * rep);
   }
 #undef FSVD_RD_LAUNCH_T
+#undef FSVD_RD_LAUNCH_SC
 #undef FSVD_RD_LAUNCH
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: stage 1 launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }

@@ -108,6 +108,10 @@ def _rank_decode_impl(q, pk_cache, pv_cache, k_u, v_u, cos, sin, seqlens, num_kv
     if out is None:
         out = torch.empty(B, H, Dh, device=q.device, dtype=q.dtype)
     rope_len = 0 if cos is None else int(cos.shape[0])
+    if B * S * H >= (1 << 20):
+        # long caches: the library keeps the scores of a call in the registered scratch and accumulates per head group
+        from ..hip_ops import ensure_split_workspace
+        ensure_split_workspace(q.device)
     lib = _lib.load()
     rc = lib.fsvd_attn_decode_rankkv(
         q.data_ptr(), q.stride(0), q.stride(1), pk_cache.data_ptr(), *spk, pv_cache.data_ptr(), *spv,

@@ -207,7 +207,11 @@ int fsvd_mlp_dual_split(const void* PUp, int64_t sPUp_t, const void* PGate, int6
  * [Hk*Dh, R] (= per-head bases V[h][r][d] = u[h*Dh+d][r]), workspaces are the reference's split-K
  * buffers M, L [B,H,nsplit] and Acc [B,H,nsplit,Rv] (fp32), n_keys = cache_seqlens[b] + seqlen_add.
  * spk_h / spv_h are the kv-head strides of head-wise coefficient caches [B,S,Hk,R] (0 when shared).
- * bf16 only; head_dim 128; ranks multiples of 8, Rv <= 2048. */
+ * bf16 only; head_dim 128; ranks multiples of 8, Rv <= 2048.
+ * With scratch registered (fsvd_set_workspace) of at least B*H*ceil64(S) floats behind its 64 KiB counter block, shared
+ * caches (spv_h == 0) with S >= 1024 and B*H*S >= 2^20 run as score, softmax and accumulation launches that keep the
+ * scores of the call in that scratch (same results up to the order of fp32 sums); calls that use it must be ordered on
+ * one stream, like the K-split projections. */
 int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,
                             const void* pk_cache, int64_t spk_b, int64_t spk_s, int64_t spk_h,
                             const void* pv_cache, int64_t spv_b, int64_t spv_s, int64_t spv_h,

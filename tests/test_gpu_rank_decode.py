@@ -49,6 +49,55 @@ def test_rank_decode_vs_oracle(RD, B, H, Hk, L, S, Rk, Rv, nsplit):
     assert_close_bf16(out[:1], O.dense_decode_attn(q[:1].float(), K[:1, :n], V[:1, :n]), "vs dense")
 
 
+LONG_CASES = [  # B, H, Hk, S, Rk, Rv, nsplit: long caches with registered scratch take the three-launch form
+    (4, 32, 32, 8200, 192, 200, 2),     # one query head per kv head: four key sub-tiles per pass, Pk and k_u straight into LDS
+    (4, 32, 8, 8200, 128, 64, 3),       # four query heads per kv head
+    (4, 32, 16, 8200, 72, 136, 2),      # two query heads per kv head, ranks off the 64 grid (fragments straight from memory)
+    (9, 16, 16, 7300, 64, 72, 5),       # 16 heads: one head tile; short last split
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,S,Rk,Rv,nsplit", LONG_CASES)
+def test_long_cache_three_launch_form(RD, monkeypatch, B, H, Hk, S, Rk, Rv, nsplit):
+    """Scores -> softmax -> rank-space accumulation per head tile (long caches shared by the heads, scratch registered)
+    against the one-kernel form on the same inputs (same arithmetic up to the order of fp32 sums: one bf16 ulp) and against
+    the oracle on sampled batch rows."""
+    from flashsvd_amd import hip_ops
+    Dh = 128
+    cos, sin = O.rope_tables(S, Dh, dtype=BF16)
+    q = rand_bf16(B, H, Dh, seed=11)
+    Pk, Pv = rand_bf16(B, S, Rk, seed=12), rand_bf16(B, S, Rv, seed=13)
+    Vk, Vv = rand_bf16(Hk, Rk, Dh, std=Rk ** -0.5, seed=14), rand_bf16(Hk, Rv, Dh, std=Rv ** -0.5, seed=15)
+    lens = torch.tensor([max(0, S - 5 - 1031 * b) for b in range(B)], dtype=torch.int32)
+    lens[-1] = 0 if B > 4 else lens[-1]                 # an empty batch row in the widest case
+    args = (q.cuda(), Pk.cuda(), Pv.cuda(), _lin_layout(Vk).cuda(), _lin_layout(Vv).cuda(), cos.cuda(), sin.cuda(), lens.cuda())
+    # one-kernel form: no scratch registered
+    monkeypatch.setenv("FLASHSVD_AMD_SPLITK", "0")
+    hip_ops.release_split_workspace(torch.device("cuda", torch.cuda.current_device()))
+    one = RD.rank_decode(*args, num_kv_heads=Hk, nsplit=nsplit).float().cpu()
+    monkeypatch.delenv("FLASHSVD_AMD_SPLITK")
+    hip_ops.release_split_workspace(torch.device("cuda", torch.cuda.current_device()))
+    three = RD.rank_decode(*args, num_kv_heads=Hk, nsplit=nsplit)
+    torch.cuda.synchronize()
+    # the scratch now holds the softmax weights of the call, [B,H,ld] fp32 behind the 64 KiB counter block: the largest
+    # weight of a non-empty row is exp(0) in at least one split -- which proves the form that ran
+    ws = hip_ops._SPLIT_WS[torch.cuda.current_device()]
+    ld = (S + 63) // 64 * 64
+    w = ws[64 * 1024:64 * 1024 + B * H * ld * 4].view(torch.float32).view(B, H, ld)
+    n0 = int(lens[0])
+    assert n0 > 0 and float(w[0, :, :n0].max(dim=-1).values.min()) == 1.0 and float(w[0, :, :n0].min()) >= 0.0
+    three = three.float().cpu()
+    assert torch.isfinite(three).all()
+    assert_close_bf16(three, one, "three-launch form vs one-kernel form", abs_tol=2e-3, rel_tol=1e-2)
+    for b in (0, B - 1):
+        n = int(lens[b])
+        if n == 0:
+            assert float(three[b].abs().max()) == 0.0 and float(one[b].abs().max()) == 0.0
+            continue
+        ref = O.rank_decode_attn(q[b:b + 1], Pk[b:b + 1, :n], Pv[b:b + 1, :n], Vk, Vv, cos[:n], sin[:n])
+        assert_close_bf16(three[b:b + 1], ref, f"three-launch form, b={b} n={n}")
+
+
 def test_packed_api_shared_and_headwise(RD):
     B, H, Hk, L, R, Dh = 2, 8, 4, 150, 96, 128
     cos, sin = O.rope_tables(L, Dh, dtype=BF16)
