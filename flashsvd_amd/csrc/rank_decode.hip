@@ -40,8 +40,8 @@ __device__ __forceinline__ bf16x8_t zero_frag() { return __builtin_bit_cast(bf16
 
 // dynamic LDS of the partial kernel: k_u stages [stage][128 d][64 r] bf16 (two, or three in the deep form), reused for the
 // four waves' rank-space partials [4][kRdMaxChunks * 512] fp32 at the end; then the waves' Pk slots
-template <int KS, bool PKL, bool DEEP> struct RankDecodeLds {
-  static constexpr int kStages = DEEP ? 3 : 2;
+template <int KS, bool PKL, bool DEEP, bool SC = false> struct RankDecodeLds {
+  static constexpr int kStages = (DEEP || (SC && PKL)) ? 3 : 2;
   static constexpr int kKu = kStages * 128 * 64 * 2, kTb = 4 * kRdMaxChunks * 512 * 4;
   static constexpr int kMain = kKu > kTb ? kKu : kTb;
   static constexpr int kPkSlots = DEEP ? 2 : 1;
@@ -62,7 +62,6 @@ template <int REP, int KS, bool PKL, bool DEEP = false, bool SC = false>
 __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(RankDecodeArgs a) {
   static_assert(!DEEP || (PKL && KS == 1), "the deep form is built for single sub-tiles with Pk through LDS");
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
-  __shared__ float qs[REP][DH];
   __shared__ float wm[4][REP], wl[4][REP];
   // one LDS block, used twice: k_u chunks [2][128 d][64 r] bf16 while the keys stream, the four waves'
   // rank-space partials [4][kRdMaxChunks*512] fp32 for the merge at the end
@@ -70,12 +69,13 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   // (lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of a half wave), and with this placement the fragment reads (lane =
   // row % 16 + 16 * piece) touch every bank once per group (rows padded to 144 bytes put two lanes on a bank)
   constexpr int KROW = 64;
-  typedef RankDecodeLds<KS, PKL, DEEP> Lds;
+  typedef RankDecodeLds<KS, PKL, DEEP, SC> Lds;
   extern __shared__ __align__(16) unsigned char rd_smem[];
   unsigned char* smem = rd_smem;                                 // k_u stages, then the waves' partials
   unsigned char* pkslot = rd_smem + Lds::kMain;                  // [wave][slot][sub-tile][16 keys][128 bytes]
   uint16_t (*kus)[DH][KROW] = reinterpret_cast<uint16_t (*)[DH][KROW]>(smem);
   float (*tbuf)[kRdMaxChunks * 512] = reinterpret_cast<float (*)[kRdMaxChunks * 512]>(smem);
+  float (*qs)[DH] = reinterpret_cast<float (*)[DH]>(smem);         // the queries, before the first k_u chunk takes the place
 
   const int groups = a.H / a.Hk / REP;             // q-head groups per kv head handled by separate blocks
   // the head groups of one key range (they read the same cache rows) are neighbours on one XCD
@@ -113,6 +113,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   for (int g = 0; g < REP; ++g)
 #pragma unroll
     for (int t = 0; t < NT; ++t) qv[g][t] = qs[g][(t / 4) * HALF + lr * 4 + (t % 4)];
+  __syncthreads();                                                 // the queries are in registers: the LDS block is free
 
   const int nchunk = (a.Rv + 511) / 512;
   float m_run[REP], l_run[REP];
@@ -252,7 +253,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
       }
       __syncthreads();                                           // the last stages are read out before the next tile refills them
     } else if constexpr (PKL && SC) {
-      // k_u chunks straight into the two LDS stages as well (no registers, no LDS stores), one chunk ahead: lane -> LDS row
+      // k_u chunks straight into LDS stages as well (no registers, no LDS stores): lane -> LDS row
       // wave * 32 + i * 8 + lane / 8 and position lane % 8 of the stage, which holds piece (lane % 8) ^ (row % 8) of head
       // dimension kd(row) -- the placement store_ku gives the register form.  Addresses are a wave-uniform base plus a
       // 32-bit byte offset per lane (the launcher checks that the cache of a batch row fits): no 64-bit pointer per piece
@@ -277,7 +278,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
       const auto issue_ku = [&](int c) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          __builtin_amdgcn_global_load_lds((gptr_t)(kub + c * 128 + (size_t)kuoff[i]), (lptr_t)(smem + (c & 1) * (DH * KROW * 2) + (wave * 32 + i * 8) * 128), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((gptr_t)(kub + c * 128 + (size_t)kuoff[i]), (lptr_t)(smem + (c % 3) * (DH * KROW * 2) + (wave * 32 + i * 8) * 128), 16, 0, 0);
       };
       const auto issue_pk = [&](int c) {
 #pragma unroll
@@ -286,17 +287,30 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
           for (int i = 0; i < 2; ++i)
             __builtin_amdgcn_global_load_lds((gptr_t)(pkb + c * 128 + (size_t)pkoff[j][i]), (lptr_t)(myslot + j * 2048 + i * 1024), 16, 0, 0);
       };
-      // (the barrier that ended the previous tile's last chunk also freed both stages and the slot)
+      // k_u chunks run two ahead through a ring of three stages, the Pk pieces one ahead (a wave reads its slot out at the
+      // top of a step and refills it at once); the wave's load counter and one barrier per step are the synchronisation.
+      // Requests in issue order: ... Pk(st) [2 KS], k_u(st + 1) [4]: chunk st is complete once only the 4 newest are out.
+      // (the barrier that ended the previous tile freed every stage and the slot)
+      constexpr int kNoLgkm = (7 << 4) | (15 << 8);              // wait on the load counter only
       issue_ku(0);
       issue_pk(0);
-      __builtin_amdgcn_s_waitcnt(0);
-      __syncthreads();
+      if (nstep > 1) issue_ku(1);
       for (int st = 0; st < nstep; ++st) {
-        const int cur = st & 1;
-        read_pk();
-        __builtin_amdgcn_s_waitcnt(0);             // fragments in registers: the slot is free again
+        if (st + 1 < nstep) __builtin_amdgcn_s_waitcnt(kNoLgkm | 4);
+        else __builtin_amdgcn_s_waitcnt(kNoLgkm | 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (st + 1 < nstep) { issue_pk(st + 1); issue_ku(st + 1); }
+        read_pk();
+        __builtin_amdgcn_s_waitcnt(0xc07f);         // LDS reads done (fragments in registers, the previous step's k_u reads too); loads stay in flight
+        // everybody's pieces of chunk st are in, stage (st + 2) % 3 is read out (step st - 1), the slot is free.  The bare
+        // barrier instruction: __syncthreads() carries a fence that waits for all of the wave's loads, the chunk requested
+        // ahead included
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (st + 1 < nstep) issue_pk(st + 1);
+        if (st + 2 < nstep) issue_ku(st + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        const int cur = st % 3;
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
 #pragma unroll
@@ -306,9 +320,8 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
             for (int j = 0; j < KS; ++j) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][k], bf, accs[j][t], 0, 0, 0);
           }
         }
-        __builtin_amdgcn_s_waitcnt(0);             // this wave's pieces of chunk st + 1 have landed ...
-        __syncthreads();                           // ... everybody's have, and stage cur is read out
       }
+      __syncthreads();                             // the last stages are read out before the next tile refills them
     } else {
     // (the barrier that ended the previous tile's last chunk also freed both buffers)
     load_ku(0);
@@ -452,9 +465,13 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   }
 }
 
-// Softmax weights of one split of one (batch row, head), in place: scores[b, h, key] -> exp(s - m[b,h,split]), with the
-// split's maximum and sum to ws_m / ws_l (the merge kernel folds the splits as it does for the one-kernel form).
-// grid (nsplit, H, B), 256 threads.  Rows of the score buffer are a.score_ld floats apart.
+// Softmax weights of one split of one (batch row, head), in place: the scores s[b, h, key] of the split become the
+// weights p = exp(s - m[b,h,split]) in the form the accumulation kernel multiplies with, and the split's maximum and sum
+// go to ws_m / ws_l (the merge kernel folds the splits as it does for the one-kernel form).  Every group of 8 keys (32
+// bytes of the row) is rewritten as two matrix-core fragments of 8 bf16 each: hi = bf16(p) of the 8 keys, then
+// lo = bf16(p - hi), so that hi + lo carries p to 2^-17 and the consumer needs no arithmetic on them.  Keys between the end
+// of the cache row and the next multiple of 64 get weight 0.  grid (nsplit, H, B), 256 threads; rows of the score buffer
+// are a.score_ld floats apart (a multiple of 64).
 __global__ __launch_bounds__(kRdThreads) void rank_decode_softmax_kernel(RankDecodeArgs a) {
   __shared__ float red[4];
   const int s = blockIdx.x, h = blockIdx.y, b = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -463,147 +480,177 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_softmax_kernel(RankDec
   int per = (n_keys + a.nsplit - 1) / a.nsplit;
   per = (per + kRdTileKeys - 1) / kRdTileKeys * kRdTileKeys;
   const int k0 = min(s * per, n_keys), k1 = min(n_keys, k0 + per);
+  if (k0 >= k1) {
+    if (tid == 0) {
+      const int64_t slot = ((int64_t)b * a.H + h) * a.nsplit + s;
+      a.ws_m[slot] = -INFINITY;                    // an empty split: the merge gives it weight 0
+      a.ws_l[slot] = 0.f;
+    }
+    return;
+  }
   float* sp = a.scores + ((int64_t)b * a.H + h) * a.score_ld;
+  const int kend = (k1 + 63) / 64 * 64;            // k0 is a multiple of 64; only the last split of a row ends off the grid
+  // a thread takes groups of 8 keys: both passes read the same 32 bytes, the second rewrites them
   float m = -INFINITY;
-  for (int k = k0 + tid; k < k1; k += kRdThreads) m = fmaxf(m, sp[k]);
+  for (int k = k0 + tid * 8; k < k1; k += kRdThreads * 8) {
+    const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(sp + k), x1 = *reinterpret_cast<const f32x4_t*>(sp + k + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (k + i < k1) m = fmaxf(m, x0[i]);
+      if (k + 4 + i < k1) m = fmaxf(m, x1[i]);
+    }
+  }
   m = wave_max(m);
   if (lane == 0) red[wave] = m;
   __syncthreads();
   const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   __syncthreads();
   float l = 0.f;
-  for (int k = k0 + tid; k < k1; k += kRdThreads) {
-    const float p = __expf(sp[k] - M);
-    sp[k] = p;
-    l += p;
+  for (int k = k0 + tid * 8; k < kend; k += kRdThreads * 8) {
+    const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(sp + k), x1 = *reinterpret_cast<const f32x4_t*>(sp + k + 4);
+    uint32_t hi[8], lo[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p = (k + i < k1) ? __expf((i < 4 ? x0[i] : x1[i - 4]) - M) : 0.f;
+      l += p;
+      hi[i] = f32_to_bf16_bits(p);
+      lo[i] = f32_to_bf16_bits(p - bf16_bits_to_f32(hi[i]));
+    }
+    uint32_t* wp = reinterpret_cast<uint32_t*>(sp + k);
+    *reinterpret_cast<u32x4_t*>(wp) = u32x4_t{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)};
+    *reinterpret_cast<u32x4_t*>(wp + 4) = u32x4_t{lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)};
   }
   l = wave_sum(l);
   if (lane == 0) red[wave] = l;
   __syncthreads();
   if (tid == 0) {
     const int64_t slot = ((int64_t)b * a.H + h) * a.nsplit + s;
-    a.ws_m[slot] = M;                              // -inf for an empty split: the merge gives it weight 0
+    a.ws_m[slot] = M;
     a.ws_l[slot] = ((red[0] + red[1]) + red[2]) + red[3];
   }
 }
 
 // Acc[b, h, split, r] = sum over the split's keys of p[b, h, key] * Pv[b, key, r] on the matrix cores, for 16 * MT heads at
 // once: a Pv row is read once per head tile instead of once per head (coefficient caches shared by the heads only).
-// grid (r slices of 64, nsplit * head tiles, B), 4 waves; wave w owns the 16 columns r0 + 16 w of the slice.  Per block of
-// 64 keys the workgroup stages Pv[64 keys x 64 r] in LDS (one 16-byte load per thread and 32 keys, a block ahead in
-// registers) and every lane gathers its B fragment (8 keys of one column) with 2-byte LDS reads; the A fragments are the
-// weights p[h, 8 keys] straight from the score buffer, split into two bf16 terms (p = hi + lo to 2^-17) so that the sum
-// keeps fp32 weights; fp32 accumulation in key order.
+// grid (r slices of 128, nsplit * head tiles, B), 4 waves; wave w owns the 32 columns c0 + 32 w of the slice.  Per block of
+// 64 keys the workgroup stages Pv[64 keys x 128 r] and the weight fragments of its heads (the hi and lo term the softmax
+// kernel left in the score buffer, 32 bytes per head and 8 keys) in LDS, two blocks ahead in registers; a lane gathers its
+// B fragment (8 keys of one column) with 2-byte LDS reads and takes its A fragments with 16-byte ones; two matrix
+// products per tile so that the sum keeps fp32 weights; fp32 accumulation in key order.
 template <int MT>
 __global__ __launch_bounds__(kRdThreads) void rank_decode_pv_kernel(RankDecodeArgs a) {
-  constexpr int KB = 64, PITCH = 132;              // bytes per LDS row: 8 rows apart = 8 banks apart, the four key groups of a fragment read disjoint banks
+  // LDS rows: 128 columns of a key in 260 bytes (8 rows apart = 8 banks apart: the four key groups of a fragment gather
+  // from disjoint banks), the 64 keys of a head in 272 bytes (16 heads read 16 bytes each from disjoint banks)
+  constexpr int KB = 64, NT = 2, PITCH = 260, WPITCH = 272, HT = 16 * MT;
   __shared__ __align__(16) unsigned char tile[2][KB * PITCH];
+  __shared__ __align__(16) unsigned char wtile[2][HT * WPITCH];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 15, lg = lane >> 4;
-  const int ntile = (a.H + 16 * MT - 1) / (16 * MT);
+  const int ntile = (a.H + HT - 1) / HT;
   const int s = blockIdx.y / ntile, ht = blockIdx.y % ntile, b = blockIdx.z;
-  const int h0 = ht * 16 * MT;
+  const int h0 = ht * HT;
   int n_keys = a.seqlens[b] + a.seqlen_add;
   n_keys = max(0, min(n_keys, a.S));
   int per = (n_keys + a.nsplit - 1) / a.nsplit;
   per = (per + kRdTileKeys - 1) / kRdTileKeys * kRdTileKeys;
   const int k0 = min(s * per, n_keys), k1 = min(n_keys, k0 + per);
-  const int c0 = blockIdx.x * 64;                  // first column of the slice
-  // staging: thread -> key row tid / 8 (+ 32) of the block, 16-byte piece tid % 8 of the 128-byte row slice
-  const int srow = tid >> 3, spiece = tid & 7;
+  const int c0 = blockIdx.x * 128;                 // first column of the slice
+  // staging of Pv: thread -> key row tid / 16 (+ 16 i) of the block, 16-byte piece tid % 16 of the 256-byte row slice
+  const int srow = tid >> 4, spiece = tid & 15;
   const bool scol = c0 + spiece * 8 < a.Rv;        // Rv is a multiple of 8: a piece is inside or outside as a whole
   const uint16_t* pv_b = a.pv + (int64_t)b * a.spv_b + (scol ? c0 + spiece * 8 : 0);
-  const auto load_block = [&](int kb, u32x4_t (&v)[2]) {
+  // staging of the weights: thread -> head tid / 8 of the tile (32 heads: all threads; 16 heads: the first half), the 32
+  // bytes of key group tid % 8
+  const int whead = tid >> 3, wgrp = tid & 7;
+  const bool wlive = whead < HT && h0 + whead < a.H;
+  const float* wsrc = a.scores + ((int64_t)b * a.H + (wlive ? h0 + whead : 0)) * a.score_ld + wgrp * 8;
+  struct Regs { u32x4_t v[4]; u32x4_t w[2]; };
+  const auto load_block = [&](int kb, Regs& r) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int key = min(kb + i * 32 + srow, k1 - 1);   // clamped rows carry weight 0
-      v[i] = scol ? *reinterpret_cast<const u32x4_t*>(pv_b + (int64_t)key * a.spv_s) : u32x4_t{0u, 0u, 0u, 0u};
+    for (int i = 0; i < 4; ++i) {
+      const int key = min(kb + i * 16 + srow, k1 - 1);   // clamped rows carry weight 0
+      r.v[i] = scol ? *reinterpret_cast<const u32x4_t*>(pv_b + (int64_t)key * a.spv_s) : u32x4_t{0u, 0u, 0u, 0u};
+    }
+    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(wsrc + kb);
+    r.w[0] = wlive ? p[0] : u32x4_t{0u, 0u, 0u, 0u};
+    r.w[1] = wlive ? p[1] : u32x4_t{0u, 0u, 0u, 0u};
+  };
+  const auto store_block = [&](int buf, const Regs& r) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint32_t* d = reinterpret_cast<uint32_t*>(&tile[buf][(i * 16 + srow) * PITCH + spiece * 16]);
+      d[0] = r.v[i].x; d[1] = r.v[i].y; d[2] = r.v[i].z; d[3] = r.v[i].w;
+    }
+    if (whead < HT) {
+      u32x4_t* d = reinterpret_cast<u32x4_t*>(&wtile[buf][whead * WPITCH + wgrp * 32]);
+      d[0] = r.w[0];
+      d[1] = r.w[1];
     }
   };
-  const auto store_block = [&](int buf, const u32x4_t (&v)[2]) {
+  f32x4_t acc[MT][NT];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      uint32_t* d = reinterpret_cast<uint32_t*>(&tile[buf][(i * 32 + srow) * PITCH + spiece * 16]);
-      d[0] = v[i].x; d[1] = v[i].y; d[2] = v[i].z; d[3] = v[i].w;
-    }
-  };
-  // weights: lane -> head h0 + mt * 16 + lr, keys kb + ks * 32 + lg * 8 .. + 8
-  const float* prow[MT];
-  bool hlive[MT];
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int h = h0 + mt * 16 + lr;
-    hlive[mt] = h < a.H;
-    prow[mt] = a.scores + ((int64_t)b * a.H + (hlive[mt] ? h : 0)) * a.score_ld + lg * 8;
-  }
-  f32x4_t pw[MT][2][2];
-  const auto load_p = [&](int kb) {
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const auto products = [&](int buf) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int ks = 0; ks < 2; ++ks) {
+      u32x4_t af[MT][2];
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        // the score rows are padded to a multiple of 64 floats: the loads stay inside the row, keys past k1 are masked below
-        const float* p = prow[mt] + kb + ks * 32;
-        pw[mt][ks][0] = *reinterpret_cast<const f32x4_t*>(p);
-        pw[mt][ks][1] = *reinterpret_cast<const f32x4_t*>(p + 4);
+      for (int mt = 0; mt < MT; ++mt) {
+        const u32x4_t* p = reinterpret_cast<const u32x4_t*>(&wtile[buf][(mt * 16 + lr) * WPITCH + (ks * 4 + lg) * 32]);
+        af[mt][0] = p[0];
+        af[mt][1] = p[1];
       }
-  };
-  f32x4_t acc[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  if (k0 < k1) {
-    u32x4_t nxt[2];
-    load_block(k0, nxt);
-    store_block(0, nxt);
-    int buf = 0;
-    for (int kb = k0; kb < k1; kb += KB, buf ^= 1) {
-      const bool more = kb + KB < k1;
-      if (more) load_block(kb + KB, nxt);
-      load_p(kb);
-      __syncthreads();                             // block kb is in tile[buf]; everybody has left tile[buf ^ 1]
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
+      for (int nt = 0; nt < NT; ++nt) {
         uint16_t e[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = *reinterpret_cast<const uint16_t*>(&tile[buf][(ks * 32 + lg * 8 + j) * PITCH + (wave * 16 + lr) * 2]);
+        for (int j = 0; j < 8; ++j) e[j] = *reinterpret_cast<const uint16_t*>(&tile[buf][(ks * 32 + lg * 8 + j) * PITCH + (wave * 32 + nt * 16 + lr) * 2]);
         const u32x4_t bw{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
                          (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
         const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, bw);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          uint32_t hi[4], lo[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            float x[2];
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-              const int kk = j * 2 + q;
-              const float v = pw[mt][ks][kk >> 2][kk & 3];
-              x[q] = (hlive[mt] && kb + ks * 32 + lg * 8 + kk < k1) ? v : 0.f;
-            }
-            const uint32_t h0b = f32_to_bf16_bits(x[0]), h1b = f32_to_bf16_bits(x[1]);
-            const uint32_t l0b = f32_to_bf16_bits(x[0] - bf16_bits_to_f32((uint16_t)h0b)), l1b = f32_to_bf16_bits(x[1] - bf16_bits_to_f32((uint16_t)h1b));
-            hi[j] = (h0b & 0xffffu) | (h1b << 16);
-            lo[j] = (l0b & 0xffffu) | (l1b << 16);
-          }
-          const bf16x8_t ah = __builtin_bit_cast(bf16x8_t, u32x4_t{hi[0], hi[1], hi[2], hi[3]});
-          const bf16x8_t al = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], lo[2], lo[3]});
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bf, acc[mt], 0, 0, 0);
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, bf, acc[mt], 0, 0, 0);
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[mt][0]), bf, acc[mt][nt], 0, 0, 0);
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[mt][1]), bf, acc[mt][nt], 0, 0, 0);
         }
       }
-      if (more) store_block(buf ^ 1, nxt);         // tile[buf ^ 1] was read out before this iteration's barrier
+    }
+  };
+  if (k0 < k1) {
+    // two register sets, each with the Pv pieces and the weights of one block: while block i is multiplied out of LDS,
+    // block i + 1 sits in one set (requested an iteration ago, stored to the other tile after the products) and block i + 2
+    // is requested into the other, so that two blocks per workgroup are always on their way from memory
+    Regs ra, rb;
+    load_block(k0, ra);
+    if (k0 + KB < k1) load_block(k0 + KB, rb);
+    store_block(0, ra);
+    for (int kb = k0; kb < k1; kb += 2 * KB) {
+      if (kb + 2 * KB < k1) load_block(kb + 2 * KB, ra);
+      __syncthreads();                             // block kb is in tile 0; everybody has left tile 1
+      products(0);
+      if (kb + KB >= k1) break;
+      store_block(1, rb);
+      if (kb + 3 * KB < k1) load_block(kb + 3 * KB, rb);
+      __syncthreads();                             // block kb + KB is in tile 1; everybody has left tile 0
+      products(1);
+      if (kb + 2 * KB >= k1) break;
+      store_block(0, ra);
     }
   }
-  // element i of a lane: head h0 + mt * 16 + lg * 4 + i, column c0 + wave * 16 + lr
-  const int r = c0 + wave * 16 + lr;
-  if (r < a.Rv) {
+  // element i of a lane: head h0 + mt * 16 + lg * 4 + i, column c0 + wave * 32 + nt * 16 + lr
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+  for (int nt = 0; nt < NT; ++nt) {
+    const int r = c0 + wave * 32 + nt * 16 + lr;
+    if (r < a.Rv) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int h = h0 + mt * 16 + lg * 4 + i;
-        if (h < a.H) a.ws_acc[(((int64_t)b * a.H + h) * a.nsplit + s) * a.Rv + r] = acc[mt][i];
-      }
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int h = h0 + mt * 16 + lg * 4 + i;
+          if (h < a.H) a.ws_acc[(((int64_t)b * a.H + h) * a.nsplit + s) * a.Rv + r] = acc[mt][nt][i];
+        }
+    }
   }
 }
 
@@ -749,7 +796,7 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   } while (0)
 #define FSVD_RD_LAUNCH_SC(REP_, KS_, PKL_, GY_)                                                                                      \
   do {                                                                                                                              \
-    constexpr int lds = RankDecodeLds<KS_, PKL_, false>::kBytes;                                                                    \
+    constexpr int lds = RankDecodeLds<KS_, PKL_, false, true>::kBytes;                                                              \
     static bool granted = false;                                                                                                    \
     if (!granted && lds >= 48 * 1024) {                                                                                             \
       hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_decode_partial_kernel<REP_, KS_, PKL_, false, true>), \
@@ -777,7 +824,7 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     if (e3 != hipSuccess) { set_last_error("%s: score launch failed: %s", fn, hipGetErrorString(e3)); return kErrLaunch; }
     hipLaunchKernelGGL(rank_decode_softmax_kernel, dim3(a.nsplit, a.H, a.B), block, 0, st, a3);
     const int mt = a.H > 16 ? 2 : 1;
-    const dim3 gpv((a.Rv + 63) / 64, a.nsplit * ((a.H + 16 * mt - 1) / (16 * mt)), a.B);
+    const dim3 gpv((a.Rv + 127) / 128, a.nsplit * ((a.H + 16 * mt - 1) / (16 * mt)), a.B);
     if (mt == 2) hipLaunchKernelGGL(rank_decode_pv_kernel<2>, gpv, block, 0, st, a3);
     else hipLaunchKernelGGL(rank_decode_pv_kernel<1>, gpv, block, 0, st, a3);
     e3 = hipGetLastError();

@@ -79,13 +79,21 @@ def test_long_cache_three_launch_form(RD, monkeypatch, B, H, Hk, S, Rk, Rv, nspl
     hip_ops.release_split_workspace(torch.device("cuda", torch.cuda.current_device()))
     three = RD.rank_decode(*args, num_kv_heads=Hk, nsplit=nsplit)
     torch.cuda.synchronize()
-    # the scratch now holds the softmax weights of the call, [B,H,ld] fp32 behind the 64 KiB counter block: the largest
-    # weight of a non-empty row is exp(0) in at least one split -- which proves the form that ran
+    # the scratch now holds the softmax weights of the call, [B,H,ld] words behind the 64 KiB counter block, per 8 keys four
+    # words of bf16 pairs hi(p) and four of lo(p) = bf16(p - hi): the largest weight of a non-empty row is exp(0) in at
+    # least one split -- which proves the form that ran
     ws = hip_ops._SPLIT_WS[torch.cuda.current_device()]
     ld = (S + 63) // 64 * 64
-    w = ws[64 * 1024:64 * 1024 + B * H * ld * 4].view(torch.float32).view(B, H, ld)
+    w = ws[64 * 1024:64 * 1024 + B * H * ld * 4].view(torch.int32).view(B, H, ld // 8, 2, 4)[0].cpu()
     n0 = int(lens[0])
-    assert n0 > 0 and float(w[0, :, :n0].max(dim=-1).values.min()) == 1.0 and float(w[0, :, :n0].min()) >= 0.0
+    def pairs(x):                                       # [H, groups, 4] words -> [H, groups * 8] values
+        lo16 = ((x & 0xffff) << 16).view(torch.float32)
+        hi16 = (x & -65536).view(torch.float32)
+        return torch.stack([lo16, hi16], dim=-1).reshape(x.shape[0], -1)
+    p_hi, p_lo = pairs(w[:, :, 0].contiguous()), pairs(w[:, :, 1].contiguous())
+    p = (p_hi + p_lo)[:, :n0]
+    assert float(p.max(dim=-1).values.min()) == 1.0 and float(p.min()) >= 0.0
+    assert float((p_hi + p_lo)[:, n0:(n0 + 63) // 64 * 64].abs().max() if n0 % 64 else 0.0) == 0.0   # the tail of the last block
     three = three.float().cpu()
     assert torch.isfinite(three).all()
     assert_close_bf16(three, one, "three-launch form vs one-kernel form", abs_tol=2e-3, rel_tol=1e-2)
