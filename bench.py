@@ -550,7 +550,7 @@ def run_stress():
     cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)     # half tables [S, Dh/2]
     lens = torch.full((B,), ctx, dtype=torch.int32, device="cuda")
     out = torch.empty(B, H, Dh, device="cuda", dtype=torch.bfloat16)
-    t_dec = timed(lambda: rank_decode(q, pk, pv, ku, vu, cos, sin, lens, num_kv_heads=Hk, rotate_q=True, out=out))
+    t_dec = timed(lambda: rank_decode(q, pk, pv, ku, vu, cos, sin, lens, num_kv_heads=Hk, rotate_q=True, out=out), reps=20, warm=5)
     flop_dec = 2.0 * B * ctx * R * Hk * Dh + 2.0 * B * H * ctx * R
     cache_bytes = 2 * B * ctx * R * 2
     del pk, pv
