@@ -192,10 +192,11 @@ def test_swiglu_batched_matrix_cores(ops, B, D, R, mode):
 
 # ---- 128 rows and more (prefill): the tiled matrix-core kernel (csrc/mfma_gemm.hip) behind the same entry points
 #      (shapes chosen to reach every tile form: 64 x 64 in K steps of 64 / 128, 128 x 64 and 128 x 128 with four and with
-#      eight waves, loads through registers and straight into LDS, ragged edges in rows and columns)
+#      eight waves, 128 x 256 from 2048 big tiles on, loads through registers and straight into LDS, ragged edges in rows
+#      and columns)
 @pytest.mark.parametrize("B,N,K", [(512, 3072, 4096), (128, 128, 64), (200, 1000, 1536), (129, 130, 192), (384, 1536, 11008),
                                    (1024, 64, 1024), (500, 3050, 1152), (1000, 3000, 1088), (1024, 3072, 1024), (2048, 4096, 256),
-                                   (2040, 2900, 192), (1150, 4090, 320)])
+                                   (2040, 2900, 192), (1150, 4090, 320), (4096, 8192, 64), (4100, 8200, 96)])
 def test_linear_prefill_rows_tiled_kernel(ops, B, N, K):
     x, w = rand_bf16(B, K, seed=1), rand_bf16(N, K, std=0.02, seed=2)
     bias, res = rand_bf16(N, std=0.1, seed=4), rand_bf16(B, N, seed=5)
