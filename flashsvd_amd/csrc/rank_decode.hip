@@ -14,8 +14,8 @@
 //   so the rotate-half RoPE is register-local; scores fold over the 16 lanes of a DPP row.
 // Stage 2, grid (H, B): merge the splits in order, normalise, multiply by v_u[h].
 //
-// Long caches shared by the heads (B * H * S of a million and more), when the caller has registered scratch: stage 1 is
-// three launches.  The score kernel is stage 1 cut after the scores (it keeps neither softmax state nor rank-space sums,
+// Caches shared by the heads with B * H * S of 2^17 and more (4096 keys of 32 heads: from there on it is the faster form
+// at every batch size measured), when the caller has registered scratch: stage 1 is three launches.  The score kernel is stage 1 cut after the scores (it keeps neither softmax state nor rank-space sums,
 // which frees the registers for four key sub-tiles per wave, and stages k_u as well as Pk with loads that write LDS
 // directly); rank_decode_softmax_kernel turns the scores of a split into weights in place; rank_decode_pv_kernel
 // accumulates p . Pv on the matrix cores for up to 32 heads at once, so that a Pv row is read once per head tile instead
@@ -764,12 +764,12 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   }
   const int rep = a.H / a.Hk;
   dim3 block(kRdThreads);
-  // long caches shared by the heads, with registered scratch: scores -> softmax -> rank-space accumulation per head tile,
+  // caches shared by the heads from 2^17 (head, key) pairs on, with registered scratch: scores -> softmax -> rank-space accumulation per head tile,
   // as three launches; the scores of the call live in the scratch, [B,H,score_ld] fp32
   const SplitWorkspace sw = split_workspace();
   const int64_t score_ld = ((int64_t)a.S + 63) / 64 * 64;
   const size_t score_floats = (size_t)a.B * a.H * score_ld;
-  const bool three = a.spv_h == 0 && a.S >= 1024 && score_floats >= ((size_t)1 << 20) && sw.part != nullptr &&
+  const bool three = a.spv_h == 0 && a.S >= 256 && score_floats >= ((size_t)1 << 17) && sw.part != nullptr &&
                      sw.part_floats >= score_floats;
   RankDecodeArgs a3 = a;
   a3.scores = three ? sw.part : nullptr;

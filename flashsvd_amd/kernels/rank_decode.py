@@ -108,8 +108,8 @@ def _rank_decode_impl(q, pk_cache, pv_cache, k_u, v_u, cos, sin, seqlens, num_kv
     if out is None:
         out = torch.empty(B, H, Dh, device=q.device, dtype=q.dtype)
     rope_len = 0 if cos is None else int(cos.shape[0])
-    if B * S * H >= (1 << 20):
-        # long caches: the library keeps the scores of a call in the registered scratch and accumulates per head group
+    if B * S * H >= (1 << 16):
+        # 4096 keys of 32 heads and more: the library keeps the scores of a call in the registered scratch and accumulates per head group
         from ..hip_ops import ensure_split_workspace
         ensure_split_workspace(q.device)
     lib = _lib.load()

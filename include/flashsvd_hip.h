@@ -209,7 +209,7 @@ int fsvd_mlp_dual_split(const void* PUp, int64_t sPUp_t, const void* PGate, int6
  * spk_h / spv_h are the kv-head strides of head-wise coefficient caches [B,S,Hk,R] (0 when shared).
  * bf16 only; head_dim 128; ranks multiples of 8, Rv <= 2048.
  * With scratch registered (fsvd_set_workspace) of at least B*H*ceil64(S) floats behind its 64 KiB counter block, shared
- * caches (spv_h == 0) with S >= 1024 and B*H*S >= 2^20 run as score, softmax and accumulation launches that keep the
+ * caches (spv_h == 0) with S >= 256 and B*H*ceil64(S) >= 2^17 run as score, softmax and accumulation launches that keep the
  * scores of the call in that scratch (same results up to the order of fp32 sums); calls that use it must be ordered on
  * one stream, like the K-split projections. */
 int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,

@@ -49,11 +49,13 @@ def test_rank_decode_vs_oracle(RD, B, H, Hk, L, S, Rk, Rv, nsplit):
     assert_close_bf16(out[:1], O.dense_decode_attn(q[:1].float(), K[:1, :n], V[:1, :n]), "vs dense")
 
 
-LONG_CASES = [  # B, H, Hk, S, Rk, Rv, nsplit: long caches with registered scratch take the three-launch form
+LONG_CASES = [  # B, H, Hk, S, Rk, Rv, nsplit: shared caches of 2^17 (head, key) pairs and more take the three-launch form
     (4, 32, 32, 8200, 192, 200, 2),     # one query head per kv head: four key sub-tiles per pass, Pk and k_u straight into LDS
     (4, 32, 8, 8200, 128, 64, 3),       # four query heads per kv head
     (4, 32, 16, 8200, 72, 136, 2),      # two query heads per kv head, ranks off the 64 grid (fragments straight from memory)
     (9, 16, 16, 7300, 64, 72, 5),       # 16 heads: one head tile; short last split
+    (2, 32, 32, 2100, 128, 128, None),  # just above the size from which the form is taken; the wrapper's own split count
+    (16, 8, 4, 1030, 64, 64, 2),        # 8 heads in a 16-head tile
 ]
 
 
@@ -68,7 +70,7 @@ def test_long_cache_three_launch_form(RD, monkeypatch, B, H, Hk, S, Rk, Rv, nspl
     q = rand_bf16(B, H, Dh, seed=11)
     Pk, Pv = rand_bf16(B, S, Rk, seed=12), rand_bf16(B, S, Rv, seed=13)
     Vk, Vv = rand_bf16(Hk, Rk, Dh, std=Rk ** -0.5, seed=14), rand_bf16(Hk, Rv, Dh, std=Rv ** -0.5, seed=15)
-    lens = torch.tensor([max(0, S - 5 - 1031 * b) for b in range(B)], dtype=torch.int32)
+    lens = torch.tensor([max(0, S - 5 - (S // (B + 1)) * b) for b in range(B)], dtype=torch.int32)
     lens[-1] = 0 if B > 4 else lens[-1]                 # an empty batch row in the widest case
     args = (q.cuda(), Pk.cuda(), Pv.cuda(), _lin_layout(Vk).cuda(), _lin_layout(Vv).cuda(), cos.cuda(), sin.cuda(), lens.cuda())
     # one-kernel form: no scratch registered
