@@ -48,27 +48,38 @@ _SPLIT_WS: dict = {}                      # device index -> scratch tensor regis
 _SPLIT_WS_BYTES = (64 << 20) + (64 << 10)
 
 
-def ensure_split_workspace(device: torch.device) -> bool:
-    """Register, once per device, the scratch the library's K-split projections (3..127 rows) work in.  The library
-    allocates nothing itself; this hands it 64 MiB of torch memory.  ``FLASHSVD_AMD_SPLITK=0`` keeps the projections
-    unsplit; so does a first call made under stream capture (an allocation there would belong to the graph's pool).
-    Launches that use the scratch must be ordered on one stream per device."""
+_SPLIT_WS_OLD: list = []                  # replaced scratch buffers: captured graphs may still hold their addresses
+_SPLIT_WS_MAX = 1 << 30
+
+
+def ensure_split_workspace(device: torch.device, min_bytes: int = 0) -> bool:
+    """Register, once per device, the scratch the library's K-split projections (3..127 rows) and its rank-space decode
+    attention (scores of a call) work in.  The library allocates nothing itself; this hands it 64 MiB of torch memory, or
+    ``min_bytes`` (up to 1 GiB) when a caller needs more: a larger buffer then replaces the registered one, and the old one
+    is kept alive because graphs captured earlier hold its address.  ``FLASHSVD_AMD_SPLITK=0`` keeps the library without
+    scratch; so does a first call made under stream capture (an allocation there would belong to the graph's pool), and
+    a registered buffer is never replaced under capture.  Launches that use the scratch must be ordered on one stream per
+    device.  Returns whether a buffer of at least ``min_bytes`` is registered."""
     idx = device.index if device.index is not None else torch.cuda.current_device()
-    if idx in _SPLIT_WS:
-        return _SPLIT_WS[idx] is not None
-    if os.environ.get("FLASHSVD_AMD_SPLITK", "1") == "0" or torch.cuda.is_current_stream_capturing():
-        return False
+    need = max(int(min_bytes), _SPLIT_WS_BYTES)
+    have = _SPLIT_WS.get(idx)
+    if have is not None and have.numel() >= need:
+        return True
+    if os.environ.get("FLASHSVD_AMD_SPLITK", "1") == "0" or torch.cuda.is_current_stream_capturing() or need > _SPLIT_WS_MAX:
+        return have is not None and min_bytes <= 0
     with torch.cuda.device(idx):
-        ws = torch.empty(_SPLIT_WS_BYTES, dtype=torch.uint8, device=f"cuda:{idx}")
+        ws = torch.empty(need, dtype=torch.uint8, device=f"cuda:{idx}")
         rc = _lib.load().fsvd_set_workspace(ws.data_ptr(), ws.numel(), _stream())
         _lib.check("fsvd_set_workspace", rc)
         torch.cuda.current_stream().synchronize()      # cleared before any other stream can use it
+    if have is not None:
+        _SPLIT_WS_OLD.append(have)
     _SPLIT_WS[idx] = ws
     return True
 
 
 def release_split_workspace(device: Optional[torch.device] = None) -> None:
-    """Unregister (and free) the scratch of ``device``; projections run unsplit until it is registered again."""
+    """Unregister (and free) the scratch of ``device``; the library runs without scratch until it is registered again."""
     idx = torch.cuda.current_device() if device is None or device.index is None else device.index
     if _SPLIT_WS.pop(idx, None) is not None:
         with torch.cuda.device(idx):

@@ -111,7 +111,7 @@ def _rank_decode_impl(q, pk_cache, pv_cache, k_u, v_u, cos, sin, seqlens, num_kv
     if B * S * H >= (1 << 16):
         # 4096 keys of 32 heads and more: the library keeps the scores of a call in the registered scratch and accumulates per head group
         from ..hip_ops import ensure_split_workspace
-        ensure_split_workspace(q.device)
+        ensure_split_workspace(q.device, (64 << 10) + 4 * B * H * ((S + 63) // 64 * 64))
     lib = _lib.load()
     rc = lib.fsvd_attn_decode_rankkv(
         q.data_ptr(), q.stride(0), q.stride(1), pk_cache.data_ptr(), *spk, pv_cache.data_ptr(), *spv,

@@ -108,6 +108,34 @@ def test_long_cache_three_launch_form(RD, monkeypatch, B, H, Hk, S, Rk, Rv, nspl
         assert_close_bf16(three[b:b + 1], ref, f"three-launch form, b={b} n={n}")
 
 
+def test_scratch_grows_to_the_capacity_of_a_long_cache(RD):
+    """The scores of a call are indexed by cache position: a cache with room for 600 000 tokens needs 77 MB of scratch
+    whatever its fill; the wrapper registers a larger buffer (the old one stays alive for graphs that hold its address)."""
+    from flashsvd_amd import hip_ops
+    B, H, Hk, S, R, Dh, n = 1, 32, 32, 600_000, 64, 128, 3000
+    dev = torch.device("cuda", torch.cuda.current_device())
+    hip_ops.ensure_split_workspace(dev)
+    before = hip_ops._SPLIT_WS[dev.index]
+    cos, sin = O.rope_tables(n, Dh, dtype=BF16)
+    q = rand_bf16(B, H, Dh, seed=21)
+    Pk, Pv = rand_bf16(B, n, R, seed=22), rand_bf16(B, n, R, seed=23)
+    Vk, Vv = rand_bf16(Hk, R, Dh, std=R ** -0.5, seed=24), rand_bf16(Hk, R, Dh, std=R ** -0.5, seed=25)
+    pkc = torch.zeros(B, S, R, dtype=BF16, device="cuda")
+    pvc = torch.zeros(B, S, R, dtype=BF16, device="cuda")
+    pkc[:, :n], pvc[:, :n] = Pk.cuda(), Pv.cuda()
+    lens = torch.tensor([n], dtype=torch.int32, device="cuda")
+    out = RD.rank_decode(q.cuda(), pkc, pvc, _lin_layout(Vk).cuda(), _lin_layout(Vv).cuda(), cos.cuda(), sin.cuda(), lens,
+                         num_kv_heads=Hk, nsplit=4)
+    after = hip_ops._SPLIT_WS[dev.index]
+    need = (64 << 10) + 4 * B * H * ((S + 63) // 64 * 64)
+    assert after.numel() >= need > before.numel() and any(t is before for t in hip_ops._SPLIT_WS_OLD)
+    ref = O.rank_decode_attn(q, Pk, Pv, Vk, Vv, cos, sin)
+    assert_close_bf16(out, ref, "long-capacity cache")
+    # the weights of the call sit in the new buffer (row 0: head 0): the three-launch form ran
+    w = after[64 * 1024:64 * 1024 + 64 * 4].view(torch.int32).cpu()
+    assert int(w.abs().max()) != 0
+
+
 def test_packed_api_shared_and_headwise(RD):
     B, H, Hk, L, R, Dh = 2, 8, 4, 150, 96, 128
     cos, sin = O.rope_tables(L, Dh, dtype=BF16)
