@@ -341,89 +341,33 @@ __device__ __forceinline__ float row_sum8(const float* cp, int row, int cpr) {
   return t;
 }
 
-// poll the tagged input of a GEMV phase into LDS as packed bf16, RMS-normalised when asked.
-// NS 64-bit words per lane per round; a normalised input fits one round (checked on the host).
-// one packed pair of staged values (elements 2q, 2q + 1) into LDS.  For an int4 phase the eight values of four
-// neighbouring lanes are stored in the order the nibble masks deliver the weights (columns 0,4 | 1,5 | 2,6 | 3,7) and the
-// sum of every 32-column piece (16 lanes) is left in xsum.
-__device__ __forceinline__ void stage_store(uint16_t* xs, float* xsum, int q, uint32_t word, bool q4) {
-  uint32_t* xs32 = reinterpret_cast<uint32_t*>(xs);
-  if (!q4) { xs32[q] = word; return; }
-  const uint32_t partner = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)word, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
-  const int pos = threadIdx.x & 3;
-  const uint32_t out = (pos & 2) ? (partner >> 16) | (word & 0xffff0000u) : (word & 0xffffu) | (partner << 16);
-  xs32[(q & ~3) + ((pos & 1) * 2 + (pos >> 1))] = out;
-  const float s = row16_sum(bf16_lo(word) + bf16_hi(word));
-  if ((threadIdx.x & 15) == 0) xsum[q >> 4] = s;
-}
-template <int NS>
-__device__ __forceinline__ bool stage_input(const void* in, int in_len, uint32_t tin, const uint32_t* norm_w, float eps,
-                                            const fsvd_step_state* st, int limit, uint16_t* xs, float* red, bool q4, float* xsum) {
-  const int tid = threadIdx.x;
-  const int nw64 = in_len >> 1;
-  const bool norm = norm_w != nullptr;
-  bool fail = false;
-  float ss = 0.f;
-  for (int base = 0; base < nw64; base += kT * NS) {
-    uint32_t nwt[NS];
-    if (norm) {
-#pragma unroll
-      for (int j = 0; j < NS; ++j) {
-        if (base + j * kT >= nw64) break;
-        const int q = base + j * kT + tid;
-        nwt[j] = norm_w[q < nw64 ? q : 0];
-      }
-    }
-    uint64_t v[NS];
-#pragma unroll
-    for (int j = 0; j < NS; ++j) {
-      if (base + j * kT >= nw64) break;
-      const int q = base + j * kT + tid;
-      v[j] = ld_coh64(in, q < nw64 ? q : 0);
-    }
-#pragma unroll
-    for (int j = 0; j < NS; ++j) {
-      if (base + j * kT >= nw64) break;
-      const int q = base + j * kT + tid;
-      if (q < nw64) {
-        uint32_t lo = (uint32_t)v[j], hi = (uint32_t)(v[j] >> 32);
-        if ((lo >> 16) != tin || (hi >> 16) != tin) {
-          if (!poll_pair(in, q, tin, st, limit, lo, hi)) fail = true;
-        }
-        lo &= 0xffffu;
-        hi &= 0xffffu;
-        if (norm) {
-          const float a = bf16_bits_to_f32(lo), b = bf16_bits_to_f32(hi);
-          ss += a * a + b * b;
-          v[j] = ((uint64_t)hi << 32) | lo;   // raw values; scaled once the sum is known
-        } else {
-          stage_store(xs, xsum, q, lo | (hi << 16), q4);
-        }
-      }
-    }
-    if (norm) {
-      ss = wave_sum(ss);
-      if ((tid & 63) == 0) red[tid >> 6] = ss;
-      __syncthreads();
-      float tot = 0.f;
-#pragma unroll
-      for (int i = 0; i < kT / 64; ++i) tot += red[i];
-      const float rs = rsqrtf(tot / (float)in_len + eps);
-#pragma unroll
-      for (int j = 0; j < NS; ++j) {
-        if (base + j * kT >= nw64) break;
-        const int q = base + j * kT + tid;
-        if (q < nw64) {
-          const float a = bf16_bits_to_f32((uint32_t)v[j]), b = bf16_bits_to_f32((uint32_t)(v[j] >> 32));
-          stage_store(xs, xsum, q, pack_bf16x2(bf16_lo(nwt[j]) * round_bf16(a * rs), bf16_hi(nwt[j]) * round_bf16(b * rs)), q4);
-        }
-      }
-    }
+// Staging of the tagged input of a GEMV phase into LDS as packed bf16, RMS-normalised when asked (a normalised input
+// fits one round of loads; checked on the host).
+// One lane's four consecutive staged values (two packed words, elements 4q .. 4q + 3) into LDS.  For an int4 phase the
+// eight values of two neighbouring lanes (columns 0..3 and 4..7 of a group) are stored in the order the nibble masks
+// deliver the weights (columns 0,4 | 1,5 | 2,6 | 3,7) and the sum of every 32-column piece (8 lanes) is left in xsum,
+// added pairwise: columns, lane pairs, quads, halves.
+__device__ __forceinline__ void stage_store_wide(uint16_t* xs, float* xsum, int q, uint32_t w0, uint32_t w1, bool q4) {
+  uint2* xs64 = reinterpret_cast<uint2*>(xs);
+  if (!q4) { xs64[q] = make_uint2(w0, w1); return; }
+  const uint32_t p0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w0, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+  const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w1, 0xB1, 0xF, 0xF, true);
+  uint2 out;
+  if ((threadIdx.x & 1) == 0) {   // columns (0,4), (1,5)
+    out.x = (w0 & 0xffffu) | (p0 << 16);
+    out.y = (w0 >> 16) | (p0 & 0xffff0000u);
+  } else {                        // columns (2,6), (3,7): this lane holds 4..7, its partner 0..3
+    out.x = (p1 & 0xffffu) | (w1 << 16);
+    out.y = (p1 >> 16) | (w1 & 0xffff0000u);
   }
-  return !fail;
+  xs64[q] = out;                  // q and the lane have the same parity: words 0,1 of the group from the even lane, 2,3 from the odd
+  float s = (bf16_lo(w0) + bf16_hi(w0)) + (bf16_lo(w1) + bf16_hi(w1));
+  s += dpp_f32<0xB1>(s);
+  s += dpp_f32<0x4E>(s);
+  s += dpp_f32<0x141>(s);
+  if ((threadIdx.x & 7) == 0) xsum[q >> 3] = s;
 }
-
-// The same for bf16 phases with 16-byte loads: four tagged values per lane and load.  A workgroup's rate of coherent
+// The input arrives through 16-byte loads: four tagged values per lane and load.  A workgroup's rate of coherent
 // loads is set by their number, not by their bytes (measured on this machine: 44 KB in 1.3 us as 8-byte loads, 0.9 us as
 // 16-byte loads, 2.2 us as 4-byte loads, whatever the number of workgroups reading), and every word carries its own tag,
 // so a load wider than the atomic unit loses nothing: a word that is torn or stale fails its tag and is polled again.
@@ -450,14 +394,13 @@ __device__ __forceinline__ void ld_coh128_round(u32x4_t (&v)[8], const uint64_t 
 #undef FSVD_LDC
 template <int NS>
 __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uint32_t tin, const uint32_t* norm_w, float eps,
-                                                 const fsvd_step_state* st, int limit, uint16_t* xs, float* red) {
+                                                 const fsvd_step_state* st, int limit, uint16_t* xs, float* red, bool q4, float* xsum) {
   static_assert(NS == 2 || NS == 8, "ld_coh128_round exists for rounds of 2 and of 8 loads");
   const int tid = threadIdx.x;
   const int nw128 = in_len >> 2;                 // in_len is a multiple of 128
   const bool norm = norm_w != nullptr;
   bool fail = false;
   float ss = 0.f;
-  uint2* xs64 = reinterpret_cast<uint2*>(xs);
   for (int base = 0; base < nw128; base += kT * NS) {
     uint2 nwt[NS];
     if (norm) {   // every slot of the round, index clamped: loads under a condition leave the compiler guarding their registers
@@ -497,7 +440,7 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
           v[j].x = a0 | (a1 << 16);       // raw values; scaled once the sum is known
           v[j].y = a2 | (a3 << 16);
         } else {
-          xs64[q] = make_uint2(a0 | (a1 << 16), a2 | (a3 << 16));
+          stage_store_wide(xs, xsum, q, a0 | (a1 << 16), a2 | (a3 << 16), q4);
         }
       }
     }
@@ -515,8 +458,8 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
         const int q = base + j * kT + tid;
         if (q < nw128) {
           const float f0 = bf16_lo(v[j].x), f1 = bf16_hi(v[j].x), f2 = bf16_lo(v[j].y), f3 = bf16_hi(v[j].y);
-          xs64[q] = make_uint2(pack_bf16x2(bf16_lo(nwt[j].x) * round_bf16(f0 * rs), bf16_hi(nwt[j].x) * round_bf16(f1 * rs)),
-                               pack_bf16x2(bf16_lo(nwt[j].y) * round_bf16(f2 * rs), bf16_hi(nwt[j].y) * round_bf16(f3 * rs)));
+          stage_store_wide(xs, xsum, q, pack_bf16x2(bf16_lo(nwt[j].x) * round_bf16(f0 * rs), bf16_hi(nwt[j].x) * round_bf16(f1 * rs)),
+                           pack_bf16x2(bf16_lo(nwt[j].y) * round_bf16(f2 * rs), bf16_hi(nwt[j].y) * round_bf16(f3 * rs)), q4);
         }
       }
     }
@@ -664,11 +607,8 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       const uint32_t* nw = static_cast<const uint32_t*>(DF_P(dv, norm_w));
       bool ok;
       const void* inp = DF_P(dv, in);
-      if (!(Q4 && gc.q4)) {      // bf16 weights: 16-byte polls
-        if (in_len <= 2 * kT * 4) ok = stage_input_wide<2>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red);
-        else ok = stage_input_wide<8>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red);
-      } else if (in_len <= 4 * kT * 2) ok = stage_input<4>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
-      else ok = stage_input<12>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+      if (in_len <= 2 * kT * 4) ok = stage_input_wide<2>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+      else ok = stage_input_wide<8>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
       // Every load of the staging code has been consumed by now (and the window, requested before the polls, has landed
       // with them: loads complete in order).  The compiler's bookkeeping cannot see that for loads issued under a
       // condition; without this explicit (and free) wait it protects the registers they used with full waits in the
