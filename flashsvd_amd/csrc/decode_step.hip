@@ -76,29 +76,6 @@ __device__ __forceinline__ u32x4_t ld_stream(uint64_t base, uint32_t byte_off) {
 }
 __device__ __forceinline__ u32x4_t ld_global16(const uint16_t* p) { return *(gptr16_t)(uintptr_t)p; }
 
-// poll one 64-bit word holding two tagged bf16 values; returns false on time-out / foreign error
-__device__ __forceinline__ bool poll_pair(const void* buf, int idx64, uint32_t tag, const fsvd_step_state* st, int limit,
-                                          uint32_t& lo, uint32_t& hi) {
-  int spins = 0;
-  for (;;) {
-    const uint64_t v = ld_coh64(buf, idx64);
-    lo = (uint32_t)v; hi = (uint32_t)(v >> 32);
-    if ((lo >> 16) == tag && (hi >> 16) == tag) return true;
-    if (++spins > limit) return false;
-    if ((spins & 1023) == 0 && ld_err(st) != 0) return false;
-  }
-}
-// poll one 32-bit tagged bf16 word
-__device__ __forceinline__ bool poll_w32(const void* buf, int idx, uint32_t tag, const fsvd_step_state* st, int limit, uint32_t& bits) {
-  int spins = 0;
-  for (;;) {
-    const uint32_t v = ld_coh32(buf, idx);
-    bits = v & 0xffffu;
-    if ((v >> 16) == tag) return true;
-    if (++spins > limit) return false;
-    if ((spins & 1023) == 0 && ld_err(st) != 0) return false;
-  }
-}
 // poll one 64-bit word with a 32-bit tag in the high half
 __device__ __forceinline__ bool poll_w64(const void* buf, int idx64, uint32_t tag, const fsvd_step_state* st, int limit,
                                          uint32_t& payload) {
@@ -660,9 +637,15 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           c = bf16_bits_to_f32(cosT[(int64_t)tp * half + dd]);
           sn = bf16_bits_to_f32(sinT[(int64_t)tp * half + dd]);
         }
+        // the two halves of a rotation pair in one trip through memory: both loads, then both tags
         uint32_t b0, b1;
-        if (!poll_w32(qkv, ebase + dd, tq, st, limit, b0)) fail = true;
-        if (!poll_w32(qkv, ebase + dd + half, tq, st, limit, b1)) fail = true;
+        for (int spins = 0;;) {
+          const uint32_t v0 = ld_coh32(qkv, ebase + dd), v1 = ld_coh32(qkv, ebase + dd + half);
+          b0 = v0 & 0xffffu;
+          b1 = v1 & 0xffffu;
+          if ((v0 >> 16) == tq && (v1 >> 16) == tq) break;
+          if (++spins > limit || ((spins & 1023) == 0 && ld_err(st) != 0)) { fail = true; break; }
+        }
         float x0 = bf16_bits_to_f32(b0), x1 = bf16_bits_to_f32(b1);
         if (role != 2 && cosT) {
           // eager bf16 arithmetic: one rounding per multiply and per add
