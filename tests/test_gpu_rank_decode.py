@@ -240,6 +240,42 @@ def test_model_rank_cache_greedy_matches_oracle_rank_cache():
     assert same >= n_new - 2, f"only {same}/{n_new} teacher-forced tokens identical"
 
 
+def test_graph_replays_of_the_three_launch_form_match_eager_steps():
+    """Batch 16 over a 1000-token rank-space context (8 heads: 2^17 (head, key) pairs): the decode step captured in a HIP
+    graph (score, softmax, accumulation and merge launches, scores in the registered scratch) replayed three times, with
+    synchronisations between the replays, gives the tokens and hidden states of eager steps from the same state."""
+    from flashsvd_amd import hip_ops
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.runtime.cache import FlashSVDLegacySparseKVCache
+    mw = O.make_model(d=1024, n_heads=8, n_kv_heads=8, head_dim=128, ffn=512, attn_rank=64, mlp_rank=64, n_layers=1,
+                      vocab=300, dtype=BF16, seed=9, std=0.05)
+    model = model_from_oracle(mw)
+    B, Lp, S = 16, 1000, 1100
+    prompt = torch.randint(0, 300, (B, Lp), generator=torch.Generator().manual_seed(6)).cuda()
+    runs = []
+    for graphed in (True, False):
+        cache = FlashSVDLegacySparseKVCache(model.config, max_batch_size=B, max_cache_len=S, device="cuda", dtype=BF16)
+        out = model(prompt, past_key_values=cache, cache_position=torch.arange(Lp), logits_to_keep=1)
+        tok = out.logits[:, -1].float().argmax(-1, keepdim=True)
+        dec = GraphedDecoder(model, cache, B)
+        dec.set_state(tok, Lp)
+        if graphed:
+            dec.capture()
+        toks, hids = [tok.cpu()], []
+        for _ in range(3):
+            t = dec.step() if graphed else dec.eager_step()
+            torch.cuda.synchronize()
+            toks.append(t.clone().cpu())
+            hids.append(dec.hidden.float().cpu().clone())
+        runs.append((torch.cat(toks, 1), torch.stack(hids)))
+    assert torch.equal(runs[0][0], runs[1][0]), "graph replays and eager steps disagree on tokens"
+    assert torch.equal(runs[0][1], runs[1][1]), "graph replays and eager steps disagree on hidden states"
+    assert torch.isfinite(runs[0][1]).all()
+    # (the projections that follow the attention in a step reuse the scratch, so the weights cannot be read back here;
+    # the shape is above the size from which fsvd_attn_decode_rankkv takes the form, with scratch registered)
+    assert hip_ops._SPLIT_WS.get(torch.cuda.current_device()) is not None and B * 8 * ((S + 63) // 64 * 64) >= 1 << 17
+
+
 def test_decode_driver_serves_the_rank_space_cache(monkeypatch):
     """decode_kvcache_eval(lowrank_cache=True) (utils/evaluator.py:358-371) decodes over FlashSVDLegacySparseKVCache through
     the per-operator graph engine, with per-layer and unequal q/k/v ranks; generate_text takes the same cache when the
