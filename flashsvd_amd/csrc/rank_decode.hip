@@ -21,6 +21,8 @@
 // accumulates p . Pv on the matrix cores for up to 32 heads at once, so that a Pv row is read once per head tile instead
 // of once per head.  In the one-kernel form every head re-reads the Pv rows of its batch row from L2 (as much traffic
 // again as k_u and Pk together) and multiplies them on the vector ALU.
+// With one query head per kv head the score launch takes two heads per workgroup (rank_scores_pair_kernel), which share
+// the Pk rows in LDS as well.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -465,6 +467,179 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   }
 }
 
+// The score launch for caches shared by the heads, one query head per kv head, ranks on the 64 grid: a workgroup of eight
+// waves takes TWO heads over the same 64 KS keys, waves 0-3 head 2 gy and waves 4-7 head 2 gy + 1.  Wave w and wave w + 4
+// work on the same key sub-tiles and read their Pk fragments from one LDS slot, which the two of them fill (half of the
+// sub-tiles each): the Pk rows of a batch row cross from L2 to LDS once per pair of heads instead of once per head (at
+// batch 16 x 4096 keys x rank 1664 the score launch moves 7 GB per layer through the compute units' load path instead of
+// 10.5).  Every head has its own two stages of k_u chunks; both operands are requested one chunk ahead, straight into
+// LDS; per chunk: the wave's load counter, one barrier (everybody's pieces of this chunk are in, everybody has left the
+// previous chunk), the requests for the next chunk, the fragments, the products.  grid (nsplit, Hk / 2, B), 512 threads,
+// one workgroup per compute unit (128 KB of LDS).
+constexpr int kRdPairThreads = 512;
+template <int KS> struct RankPairLds {
+  static constexpr int kKu = 2 * 128 * 64 * 2;                   // two stages of one head's k_u chunk [128 d][64 r] bf16
+  static constexpr int kSlot = KS * 2048;                        // Pk of KS sub-tiles x 16 keys x 128 bytes
+  static constexpr int kBytes = 2 * kKu + 4 * 2 * kSlot;         // both heads' stages, then [pair of waves][2 slots]
+};
+template <int KS>
+__global__ __launch_bounds__(kRdPairThreads, 1) void rank_scores_pair_kernel(RankDecodeArgs a) {
+  static_assert(KS == 2 || KS == 4, "the two waves of a pair fill half of the sub-tiles each");
+  constexpr int DH = 128, NT = DH / 16, HALF = DH / 2, KROW = 64;
+  typedef RankPairLds<KS> Lds;
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  extern __shared__ __align__(16) unsigned char rd_smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hp = wave >> 2, w4 = wave & 3;
+  const int lr = lane & 15, lg = lane >> 4;
+  unsigned char* kubase = rd_smem + hp * Lds::kKu;                // this head's two k_u stages
+  unsigned char* slots = rd_smem + 2 * Lds::kKu + w4 * 2 * Lds::kSlot;   // the pair's two Pk slots
+  uint16_t (*kus)[DH][KROW] = reinterpret_cast<uint16_t (*)[DH][KROW]>(kubase);
+  float (*qs)[DH] = reinterpret_cast<float (*)[DH]>(rd_smem);      // the two queries, before the first chunk takes the place
+
+  const int GY = gridDim.y;
+  const int t = xcd_run_index(blockIdx.x + (int)gridDim.x * (blockIdx.y + GY * blockIdx.z), (int)gridDim.x * GY * gridDim.z);
+  const int gy = t % GY, s = (t / GY) % (int)gridDim.x, b = t / (GY * (int)gridDim.x);
+  const int h = 2 * gy + hp;                       // query head = kv head
+
+  int n_keys = a.seqlens[b] + a.seqlen_add;
+  n_keys = max(0, min(n_keys, a.S));
+  int per = (n_keys + a.nsplit - 1) / a.nsplit;
+  per = (per + kRdTileKeys - 1) / kRdTileKeys * kRdTileKeys;
+  const int k0 = min(s * per, n_keys), k1 = min(n_keys, k0 + per);
+
+  for (int i = tid; i < 2 * HALF; i += kRdPairThreads) {
+    const int g = i / HALF, d = i % HALF;
+    const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)(2 * gy + g) * a.sq_h;
+    float x0 = bf16_bits_to_f32(qp[d]), x1 = bf16_bits_to_f32(qp[d + HALF]);
+    if (a.rotate_q) {
+      const int tp = min(max(n_keys - 1, 0), a.rope_len - 1);
+      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * HALF + d]), sn = bf16_bits_to_f32(a.sin[(int64_t)tp * HALF + d]);
+      const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
+      x0 = r0; x1 = r1;
+    }
+    qs[g][d] = x0 * a.scale;
+    qs[g][d + HALF] = x1 * a.scale;
+  }
+  __syncthreads();
+  float qv[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) qv[t] = qs[hp][(t / 4) * HALF + lr * 4 + (t % 4)];
+  __syncthreads();                                                 // the queries are in registers: the LDS block is free
+
+  const char* pkb = reinterpret_cast<const char*>(a.pk + (int64_t)b * a.spk_b);
+  const char* kub = reinterpret_cast<const char*>(a.k_u + (int64_t)h * DH * a.ldku);
+  const int nstep = a.Rk / 64;
+  // k_u: lane -> LDS row w4 * 32 + i * 8 + lane / 8 and position lane % 8 of a stage, which holds piece (lane % 8) ^ (row % 8)
+  // of head dimension kd(row): row t * 16 + lr of a stage is head dimension (t / 4) * 64 + lr * 4 + t % 4, so that a
+  // lane's accumulator tiles t = 0..3 cover four consecutive dimensions and tiles t, t + 4 a rotation pair
+  uint32_t kuoff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = w4 * 32 + i * 8 + (lane >> 3);
+    const int rd = ((row >> 4) / 4) * HALF + (row & 15) * 4 + ((row >> 4) % 4);
+    kuoff[i] = (uint32_t)((rd * (int)a.ldku + (((lane & 7) ^ (row & 7)) * 8)) * 2);
+  }
+  const auto issue_ku = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t)(kub + c * 128 + (size_t)kuoff[i]), (lptr_t)(kubase + (c & 1) * (DH * KROW * 2) + (w4 * 32 + i * 8) * 128), 16, 0, 0);
+  };
+
+  for (int kt = k0; kt < k1; kt += kRdTileKeys * KS) {
+    // sub-tile j of the pair starts at key kt + (4 j + w4) * 16; this wave requests sub-tiles hp * KS / 2 .. + KS / 2
+    f32x4_t accs[KS][NT];
+#pragma unroll
+    for (int j = 0; j < KS; ++j)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) accs[j][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    uint32_t pkoff[KS / 2][2];
+#pragma unroll
+    for (int jj = 0; jj < KS / 2; ++jj)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int j = hp * (KS / 2) + jj, row = i * 8 + (lane >> 3);
+        const int pkey = min(kt + (4 * j + w4) * 16 + row, k1 - 1);
+        pkoff[jj][i] = (uint32_t)pkey * (uint32_t)(a.spk_s * 2) + (uint32_t)((((lane & 7) ^ (row & 7)) * 8) * 2);
+      }
+    const auto issue_pk = [&](int c) {
+#pragma unroll
+      for (int jj = 0; jj < KS / 2; ++jj)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          __builtin_amdgcn_global_load_lds((gptr_t)(pkb + c * 128 + (size_t)pkoff[jj][i]),
+                                           (lptr_t)(slots + (c & 1) * Lds::kSlot + (hp * (KS / 2) + jj) * 2048 + i * 1024), 16, 0, 0);
+    };
+    // (the barrier that ended the previous tile freed every stage and slot)
+    issue_ku(0);
+    issue_pk(0);
+    for (int st = 0; st < nstep; ++st) {
+      __builtin_amdgcn_s_waitcnt(0);               // this wave's pieces of chunk st have landed (and its LDS reads of chunk st - 1 are done)
+      // everybody's pieces of chunk st are in; everybody has left chunk st - 1, whose stage and slot take chunk st + 1.  The
+      // bare barrier instruction (nothing is in flight here that a fence would have to wait for)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (st + 1 < nstep) { issue_pk(st + 1); issue_ku(st + 1); }
+      __builtin_amdgcn_sched_barrier(0);
+      const int cur = st & 1;
+      const unsigned char* slot = slots + cur * Lds::kSlot;
+      bf16x8_t af[KS][2];
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+#pragma unroll
+        for (int k = 0; k < 2; ++k)
+          af[j][k] = *reinterpret_cast<const bf16x8_t*>(slot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+#pragma unroll
+          for (int j = 0; j < KS; ++j) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][k], bf, accs[j][t], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();                               // the last chunk is read out before the next tile refills the stages
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+      const int wkey0 = kt + (4 * j + w4) * 16;    // first key of this sub-tile
+      if (wkey0 >= k1) break;                      // wave-uniform; later sub-tiles start even further out
+      f32x4_t (&acc)[NT] = accs[j];
+      if (a.cos) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int pos = min(wkey0 + lg * 4 + i, a.rope_len - 1);
+          const uint2 cw = *reinterpret_cast<const uint2*>(a.cos + (int64_t)pos * HALF + lr * 4);
+          const uint2 sw = *reinterpret_cast<const uint2*>(a.sin + (int64_t)pos * HALF + lr * 4);
+          const float cv[4] = {bf16_lo(cw.x), bf16_hi(cw.x), bf16_lo(cw.y), bf16_hi(cw.y)};
+          const float sv[4] = {bf16_lo(sw.x), bf16_hi(sw.x), bf16_lo(sw.y), bf16_hi(sw.y)};
+#pragma unroll
+          for (int t = 0; t < NT / 2; ++t) {
+            const float x0 = acc[t][i], x1 = acc[t + NT / 2][i];
+            acc[t][i] = x0 * cv[t] - x1 * sv[t];
+            acc[t + NT / 2][i] = x0 * sv[t] + x1 * cv[t];
+          }
+        }
+      }
+      float sc[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float d = 0.f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) d += qv[t] * acc[t][i];
+        sc[i] = row16_sum(d);
+      }
+      if (lr == 0) {
+        float* sp = a.scores + ((int64_t)b * a.H + h) * a.score_ld + wkey0 + lg * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (wkey0 + lg * 4 + i < k1) sp[i] = sc[i];
+      }
+    }
+  }
+}
+
 // Softmax weights of one split of one (batch row, head), in place: the scores s[b, h, key] of the split become the
 // weights p = exp(s - m[b,h,split]) in the form the accumulation kernel multiplies with, and the split's maximum and sum
 // go to ws_m / ws_l (the merge kernel folds the splits as it does for the one-kernel form).  Every group of 8 keys (32
@@ -816,6 +991,24 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     // the score kernel addresses the Pk rows of a batch row and the k_u rows of a head with 32-bit byte offsets when it
     // loads them straight into LDS
     const bool pk3 = pkl && ((int64_t)a.S * a.spk_s + a.Rk) * 2 < ((int64_t)1 << 32) && ((int64_t)a.Dh * a.ldku + a.Rk) * 2 < ((int64_t)1 << 32);
+    // one query head per kv head over caches shared by the heads: two heads per workgroup read every Pk row once
+    const bool pair = rep == 1 && (a.Hk % 2) == 0 && a.spk_h == 0 && pk3 && per >= 128;
+    if (pair) {
+#define FSVD_RD_LAUNCH_PAIR(KS_)                                                                                                    \
+  do {                                                                                                                              \
+    constexpr int lds = RankPairLds<KS_>::kBytes;                                                                                   \
+    static bool granted = false;                                                                                                    \
+    if (!granted) {                                                                                                                 \
+      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_scores_pair_kernel<KS_>),                             \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);                                         \
+      if (ea != hipSuccess) { set_last_error("%s: cannot reserve %d bytes of LDS: %s", fn, lds, hipGetErrorString(ea)); return kErrLaunch; } \
+      granted = true;                                                                                                               \
+    }                                                                                                                               \
+    hipLaunchKernelGGL((rank_scores_pair_kernel<KS_>), dim3(a.nsplit, a.Hk / 2, a.B), dim3(kRdPairThreads), lds, st, a3);           \
+  } while (0)
+      if (per >= 256) FSVD_RD_LAUNCH_PAIR(4); else FSVD_RD_LAUNCH_PAIR(2);
+#undef FSVD_RD_LAUNCH_PAIR
+    } else
     if (rep % 4 == 0) { if (pk3) FSVD_RD_LAUNCH_SC(4, 1, true, a.Hk * (rep / 4)); else FSVD_RD_LAUNCH_SC(4, 1, false, a.Hk * (rep / 4)); }
     else if (rep % 2 == 0) { if (pk3) FSVD_RD_LAUNCH_SC(2, 2, true, a.Hk * (rep / 2)); else FSVD_RD_LAUNCH_SC(2, 2, false, a.Hk * (rep / 2)); }
     else if (per >= 256) { if (pk3) FSVD_RD_LAUNCH_SC(1, 4, true, a.Hk * rep); else FSVD_RD_LAUNCH_SC(1, 4, false, a.Hk * rep); }

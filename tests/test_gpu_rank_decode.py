@@ -50,12 +50,14 @@ def test_rank_decode_vs_oracle(RD, B, H, Hk, L, S, Rk, Rv, nsplit):
 
 
 LONG_CASES = [  # B, H, Hk, S, Rk, Rv, nsplit: shared caches of 2^17 (head, key) pairs and more take the three-launch form
-    (4, 32, 32, 8200, 192, 200, 2),     # one query head per kv head: four key sub-tiles per pass, Pk and k_u straight into LDS
+    (4, 32, 32, 8200, 192, 200, 2),     # one query head per kv head: two heads per workgroup share the Pk rows, four key sub-tiles per wave
     (4, 32, 8, 8200, 128, 64, 3),       # four query heads per kv head
     (4, 32, 16, 8200, 72, 136, 2),      # two query heads per kv head, ranks off the 64 grid (fragments straight from memory)
     (9, 16, 16, 7300, 64, 72, 5),       # 16 heads: one head tile; short last split
     (2, 32, 32, 2100, 128, 128, None),  # just above the size from which the form is taken; the wrapper's own split count
     (16, 8, 4, 1030, 64, 64, 2),        # 8 heads in a 16-head tile
+    (4, 32, 32, 8200, 72, 72, 2),       # one query head per kv head, ranks off the 64 grid: one head per workgroup
+    (12, 3, 3, 4000, 64, 64, 2),        # an odd number of heads: one head per workgroup, operands straight into LDS
 ]
 
 
