@@ -209,6 +209,23 @@ def kernel_configs(model, cache, dec, n_layers: int) -> dict:
     out["reference_layout_reconstruct_qkv_token_shared"] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3,
                                                             "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS}
     del refw
+    # the dense-cache attention kernel alone at a serving shape (batch 16 over 4096 cached tokens, 32 heads): the cache
+    # rows are its algorithmic bytes; two caches in rotation (2.1 GB) so that nothing comes from a cache
+    from flashsvd_amd import hip_ops
+    Bs, ctx, Hk = 16, 4096, CFG["num_kv_heads"]
+    kcs = [torch.randn(Bs, ctx + 8, Hk, Dh, device="cuda").to(torch.bfloat16) for _ in range(2)]
+    vcs = [torch.randn(Bs, ctx + 8, Hk, Dh, device="cuda").to(torch.bfloat16) for _ in range(2)]
+    qb = torch.randn(Bs, H, Dh, device="cuda").to(torch.bfloat16)
+    lens = torch.full((Bs,), ctx, dtype=torch.int32, device="cuda")
+    ob = torch.empty(Bs, H, Dh, device="cuda", dtype=torch.bfloat16)
+    ws = hip_ops.attn_workspace(Bs, H, Dh, 4, "cuda")
+
+    def dense_attn(i):
+        return hip_ops.attn_decode_densekv(qb, kcs[i % 2], vcs[i % 2], lens, nsplit=4, workspace=ws, out=ob)
+    us = per_layer_kernel_us(dense_attn, 8)
+    nb = 2 * Bs * ctx * Hk * Dh * 2
+    out["dense_kv_attention_b16_ctx4096"] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3, "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS}
+    del kcs, vcs
     return out
 
 
