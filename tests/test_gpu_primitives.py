@@ -100,7 +100,10 @@ def test_qkv_rope_append(ops, B, H, Hk, Dh, Rq, Rk, Rv):
 
 @pytest.mark.parametrize("B,H,Hk,Dh,L,S,nsplit", [(1, 32, 32, 128, 512, 560, 8), (1, 32, 32, 128, 513, 560, 16),
                                                  (2, 8, 2, 64, 37, 64, 3), (3, 4, 4, 128, 1, 16, 2),
-                                                 (1, 32, 8, 128, 4096, 4100, 16), (2, 4, 4, 64, 100, 128, 1)])
+                                                 (1, 32, 8, 128, 4096, 4100, 16), (2, 4, 4, 64, 100, 128, 1),
+                                                 # grouped-query caches with the chip full: four / two query heads per workgroup
+                                                 (16, 32, 8, 128, 300, 320, 4), (16, 32, 16, 128, 130, 160, 2), (64, 32, 8, 128, 70, 96, 1),
+                                                 (32, 16, 4, 128, 260, 300, 5)])
 def test_attn_decode_densekv_prerotated(ops, B, H, Hk, Dh, L, S, nsplit):
     q = rand_bf16(B, H, Dh, seed=1)
     kc, vc = rand_bf16(B, S, Hk, Dh, seed=2), rand_bf16(B, S, Hk, Dh, seed=3)
