@@ -81,12 +81,12 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = min(c0 + u * KPB + slot, k1 - 1);
-      kv[u] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)key * a.sc_s);
+      kv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(kbase + (int64_t)key * a.sc_s));
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = min(c0 + u * KPB + slot, k1 - 1);
-      vv[u] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)key * a.sc_s);
+      vv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vbase + (int64_t)key * a.sc_s));
     }
     if (it == 0) __syncthreads();  // qs ready
     const u32x4_t qv = *reinterpret_cast<const u32x4_t*>(qs + part * 8);
@@ -247,12 +247,12 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_gqa_kernel(AttnDecod
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = min(c0 + u * KPB + slot, k1 - 1);
-      kv[u] = *reinterpret_cast<const u32x4_t*>(kbase + (int64_t)key * a.sc_s);
+      kv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(kbase + (int64_t)key * a.sc_s));
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = min(c0 + u * KPB + slot, k1 - 1);
-      vv[u] = *reinterpret_cast<const u32x4_t*>(vbase + (int64_t)key * a.sc_s);
+      vv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vbase + (int64_t)key * a.sc_s));
     }
     if (it == 0) __syncthreads();  // qs ready
     float sc[G][U];
