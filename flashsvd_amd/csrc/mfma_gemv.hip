@@ -250,7 +250,7 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
     for (int m = 0; m < NM; ++m) {
 #pragma unroll
       for (int q = 0; q < NI; ++q)
-        __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[m][q] + k0), (lptr_t)(ring + slot * kStage + m * 16 * CKB + q * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[m][q] + k0), (lptr_t)(ring + slot * kStage + m * 16 * CKB + q * 1024), 16, 0, 2);
 #pragma unroll
       for (int s = 0; s < KST; ++s)
 #pragma unroll

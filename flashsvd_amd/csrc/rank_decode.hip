@@ -743,7 +743,7 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_pv_kernel(RankDecodeAr
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = min(kb + i * 16 + srow, k1 - 1);   // clamped rows carry weight 0
-      r.v[i] = scol ? *reinterpret_cast<const u32x4_t*>(pv_b + (int64_t)key * a.spv_s) : u32x4_t{0u, 0u, 0u, 0u};
+      r.v[i] = scol ? __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(pv_b + (int64_t)key * a.spv_s)) : u32x4_t{0u, 0u, 0u, 0u};
     }
     const u32x4_t* p = reinterpret_cast<const u32x4_t*>(wsrc + kb);
     r.w[0] = wlive ? p[0] : u32x4_t{0u, 0u, 0u, 0u};
