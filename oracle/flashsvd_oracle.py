@@ -532,8 +532,8 @@ class RankCache:
 
 def block_forward(mw: ModelWeights, li: int, x: torch.Tensor, pos0: int, cache, cos, sin) -> torch.Tensor:
     """x [B,T,d] at absolute positions pos0..pos0+T-1; the cache already holds pos0 earlier
-    tokens and is extended in place.  Appendix-C math of the survey; op order of an HF
-    LlamaDecoderLayer with factored linears."""
+    tokens and is extended in place.  Pre-norm block: x + o_u(o_v(attn(...))) then x + down(swiglu(...)); op order of an HF
+    LlamaDecoderLayer with factored linears (utils/model_utils.py:586-671)."""
     bw = mw.blocks[li]
     B, T, d = x.shape
     H, Hk, Dh = mw.n_heads, mw.n_kv_heads, mw.head_dim
