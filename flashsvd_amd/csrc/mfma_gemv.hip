@@ -297,6 +297,216 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
   else mfma_finish<NB, DUAL, KS>(a, red, acc);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Wide matrices (at least two 16-row tiles per compute unit) at up to 32 rows: the same wave-private LDS ring, but one
+// workgroup per compute unit that stays for the whole matrix.  Workgroup g takes tiles g, g + G, g + 2G, ...; its eight
+// waves split K as above, and because a wave's share of K is the same for every tile, its activation fragments are loaded
+// ONCE into registers (CW chunks x KST steps x NB batch tiles).  The loop then holds nothing but weight pieces on their way
+// into LDS: the ring runs on across tile boundaries (the pieces of the next tile are in flight while this tile's partial
+// sums are added through LDS and stored), and the load counter counts only them.  In the kernel above the activation
+// fragments travel with every chunk, and the compiler, which cannot follow register loads around the loop, waits for all
+// outstanding loads — the chunk requested ahead included — before every second product.
+// ---------------------------------------------------------------------------------------------
+constexpr int kResPitch = 68;                      // floats between the four row groups of a parked tile: conflict-free reads below
+template <bool DUAL, int NB, int CW, int D>
+__global__ __launch_bounds__(kMfThreads) void mfma_resident_kernel(MfmaArgs a) {
+  typedef StreamShape<DUAL> SS;
+  constexpr int NM = SS::NM, CKB = SS::CKB, kStage = SS::kStage;
+  constexpr int PPR = CKB / 16, KST = CKB / 64, RPI = 64 / PPR, NI = 16 / RPI;
+  constexpr int kGroup = NM * NI;                  // loads per chunk
+  constexpr int E = NB * 256;                      // output elements of a tile
+  static_assert(D >= 2 && D <= 4 && 3 * kGroup < 64, "the waits below cover up to three groups in flight");
+  extern __shared__ __align__(16) unsigned char st_smem[];     // [8 waves][D][kStage], then the parked partial tiles
+  constexpr int kRedWave = NM * NB * 4 * kResPitch;
+  float* red = reinterpret_cast<float*>(st_smem + (size_t)kMfWaves * D * kStage);   // [8][NM][NB][4][kResPitch]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lr = lane & 15, lg = lane >> 4;
+  const int tiles = (a.N + 15) / 16, G = gridDim.x, g = blockIdx.x;
+  const int nt = (tiles - g + G - 1) / G;          // this workgroup's tiles: g, g + G, ...
+  const int nchunk = a.K / (CKB / 2);
+  const int cw = min(CW, max(0, (nchunk - wave + kMfWaves - 1) / kMfWaves));   // this wave's chunks: wave, wave + 8, ...
+  unsigned char* ring = st_smem + (size_t)wave * D * kStage;
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  const int lrow = lane / PPR, lpc = lane % PPR;
+
+  const int total = nt * cw;
+  int issued = 0, it = 0, ic = 0, islot = 0;
+  const auto issue = [&]() {
+    const int n0 = (g + it * G) * 16;
+    const int k0 = (ic * kMfWaves + wave) * (CKB / 2);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+      for (int q = 0; q < NI; ++q) {
+        const int row = q * RPI + lrow;
+        const uint16_t* src = (m ? a.W2 : a.W) + (int64_t)min(n0 + row, a.N - 1) * a.ldw + ((lpc ^ (row % PPR)) * 8) + k0;
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(ring + islot * kStage + m * 16 * CKB + q * 1024), 16, 0, 2);
+      }
+    __builtin_amdgcn_sched_barrier(0);
+    ++issued;
+    if (++ic == cw) { ic = 0; ++it; }
+    islot = islot + 1 == D ? 0 : islot + 1;
+  };
+  constexpr int kW0 = (7 << 4) | (15 << 8);
+  const auto vm = [](int n) { return (n & 15) | ((n >> 4) << 14); };
+#pragma unroll
+  for (int p = 0; p < D; ++p)
+    if (issued < total) issue();
+  // the wave's activation fragments, requested behind the first weight stages so that both are on their way together
+  bf16x8_t xf[CW][NM][KST][NB];
+  const bf16x8_t zero = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+#pragma unroll
+  for (int c = 0; c < CW; ++c)
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+      for (int s = 0; s < KST; ++s)
+#pragma unroll
+        for (int t = 0; t < NB; ++t)
+          xf[c][m][s][t] = c < cw ? ldx_frag(a.x + (int64_t)min(t * 16 + lr, a.B - 1) * a.ldx + lg * 8 + (m ? a.up_off : 0) +
+                                             (int64_t)(c * kMfWaves + wave) * (CKB / 2) + s * 32)
+                                  : zero;
+  __builtin_amdgcn_s_waitcnt(0);                   // (the first stages land with them) from here on the load counter counts weight pieces only
+  __builtin_amdgcn_sched_barrier(0);
+
+  int done = 0, cslot = 0;
+  // one thread per output element, 16 consecutive lanes on 16 consecutive columns of one batch row (32-byte stores):
+  // element i of lane l of a tile is weight row (l / 16) * 4 + i, batch row l % 16
+  const int nn = tid & 15, b = tid >> 4;
+  const int ro = ((b >> 4) * 4 + (nn & 3)) * kResPitch + (nn >> 2) * 16 + (b & 15);
+  for (int ti = 0; ti < nt; ++ti) {
+    f32x4_t acc[NM][NB];
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+      for (int t = 0; t < NB; ++t) acc[m][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < CW; ++c) {
+      if (c < cw) {
+        // chunk `done` has landed once no more than the groups requested after it are outstanding (stores of the
+        // epilogue below, where they sit between two groups, only make this wait a little stricter)
+        const int newer = issued - done - 1;
+        if (newer >= 3) __builtin_amdgcn_s_waitcnt(kW0 | vm(3 * kGroup));
+        else if (newer == 2) __builtin_amdgcn_s_waitcnt(kW0 | vm(2 * kGroup));
+        else if (newer == 1) __builtin_amdgcn_s_waitcnt(kW0 | vm(kGroup));
+        else __builtin_amdgcn_s_waitcnt(kW0 | vm(0));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KST; ++s)
+#pragma unroll
+          for (int m = 0; m < NM; ++m) {
+            const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(ring + cslot * kStage + m * 16 * CKB + lr * CKB + (((s * 4 + lg) ^ (lr % PPR)) * 16));
+#pragma unroll
+            for (int t = 0; t < NB; ++t) acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[c][m][s][t], acc[m][t], 0, 0, 0);
+          }
+        ++done;
+        cslot = cslot + 1 == D ? 0 : cslot + 1;
+        // the stage is free again (its fragments are in registers): the chunk D ahead goes into it at once, so that a
+        // tile's last stages are on their way again before the partial sums are added
+        if (issued < total) issue();
+      }
+    }
+    // the waves' partial tiles through LDS, added in wave order; bare barrier instructions: __syncthreads() carries a
+    // fence that waits for all of the wave's loads, the pieces requested ahead included
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+      for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave * kRedWave + ((m * NB + t) * 4 + i) * kResPitch + lane] = acc[m][t][i];
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const int n = (g + ti * G) * 16 + nn;
+    if (tid < E) {
+      float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+      for (int w = 0; w < kMfWaves; ++w) {
+        v0 += red[w * kRedWave + ro];
+        if (DUAL) v1 += red[w * kRedWave + (NM - 1) * NB * 4 * kResPitch + ro];
+      }
+      if (n < a.N && b < a.B) {
+        float v;
+        if (DUAL) {
+          if (a.mode == 0) {
+            v0 = round_bf16(v0);
+            v1 = round_bf16(v1);
+            v = round_bf16(round_bf16(silu_f32(v0)) * v1);
+          } else {
+            v = round_bf16((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
+          }
+        } else {
+          if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
+          v = round_bf16(v0);
+          if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)b * a.ldres + n]) + v);
+        }
+        a.y[(int64_t)b * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);            // the sums are in registers before the next tile's partials overwrite them
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  }
+}
+
+static int compute_units() {
+  static int cus[16] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 0;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cus[dev] = n;
+  }
+  return cus[dev];
+}
+// The resident form applies to 8..32 rows of a matrix with at least two tiles per compute unit whose K is a whole number
+// of chunks, one to six per wave.  Measured against the one-shot kernels at the 7B shapes (us per call at 8 / 16 / 32
+// rows): gate/up pair 14.5 -> 13.6 / 17.5 -> 14.9 / 24.7 -> 18.7, q|k|v expansion 8.1 -> 8.1 / 9.3 -> 8.5 / 11.2 -> 10.0,
+// lm_head 45.2 -> 45.3 / 54.9 -> 46.7 / 78.1 -> 53.4; at 3 rows it is 3-5 % behind, and narrower matrices (one tile per
+// workgroup, with or without K split over workgroups as well) are where they were or slower, so both stay where they are.
+constexpr int kResidentCW = 6;
+template <bool DUAL>
+static bool resident_applies(const MfmaArgs& a) {
+  constexpr int ck = StreamShape<DUAL>::CKB / 2;
+  const int cu = compute_units();
+  if (cu <= 0 || a.B < 8 || a.B > 32 || (a.K % ck) != 0) return false;
+  const int nchunk = a.K / ck;
+  return (a.N + 15) / 16 >= 2 * cu && nchunk >= kMfWaves && nchunk <= kMfWaves * kResidentCW;
+}
+template <bool DUAL, int NB, int CW>
+static int launch_mfma_resident_t(const MfmaArgs& a, hipStream_t st, const char* who) {
+  static bool granted = false;
+  constexpr int D = 3;
+  constexpr int NM = StreamShape<DUAL>::NM;
+  const size_t lds = (size_t)kMfWaves * D * StreamShape<DUAL>::kStage + (size_t)kMfWaves * NM * NB * 4 * kResPitch * sizeof(float);
+  const void* f = reinterpret_cast<const void*>(&mfma_resident_kernel<DUAL, NB, CW, D>);
+  if (!granted) {
+    hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
+    granted = true;
+  }
+  const int G = std::min(compute_units(), (a.N + 15) / 16);
+  hipLaunchKernelGGL((mfma_resident_kernel<DUAL, NB, CW, D>), dim3(G), dim3(kMfThreads), lds, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
+  return kOk;
+}
+template <bool DUAL, int NB>
+static int launch_mfma_resident_nb(const MfmaArgs& a, hipStream_t st, const char* who) {
+  const int per = (a.K / (StreamShape<DUAL>::CKB / 2) + kMfWaves - 1) / kMfWaves;   // chunks of the busiest wave
+  if (per <= 2) return launch_mfma_resident_t<DUAL, NB, 2>(a, st, who);
+  if (per <= 4) return launch_mfma_resident_t<DUAL, NB, 4>(a, st, who);
+  return launch_mfma_resident_t<DUAL, NB, 6>(a, st, who);
+}
+template <bool DUAL>
+static int launch_mfma_resident(const MfmaArgs& a, hipStream_t st, const char* who) {
+  return a.B <= 16 ? launch_mfma_resident_nb<DUAL, 1>(a, st, who) : launch_mfma_resident_nb<DUAL, 2>(a, st, who);
+}
+
 template <int NB, bool DUAL>
 static void launch_mfma_ks(const MfmaArgs& a, int ks, hipStream_t st) {
   const int tiles = (a.N + 15) / 16;
@@ -400,6 +610,7 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
   // rows on (up to 32 rows the streaming form is faster: 12.3 / 25.3 / 6.7 us against 13.4 / 28.8 / 8.8 us on the wide
   // matrices of the 7B MLP; matrices with fewer than 128 weight tiles take its split form above, or the 32-row tiles
   // when their K does not divide into chunks)
+  if (resident_applies<DUAL>(a0)) return launch_mfma_resident<DUAL>(a0, st, who);
   const bool streamed = a0.B <= 32 && tiles >= 128 && stream_applies<DUAL>(a0, ks);
   if constexpr (!DUAL) {
     const int z = stream_split_shares(a0);

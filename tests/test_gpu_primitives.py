@@ -193,6 +193,34 @@ def test_swiglu_batched_matrix_cores(ops, B, D, R, mode):
     assert_close_bf16(h, ref, f"batched swiglu mode {mode}", **bounds(ref))
 
 
+# ---- 8..32 rows of a wide matrix (two 16-row tiles per compute unit and more): one workgroup per compute unit walks its
+#      tiles with the activation fragments in registers (mfma_resident_kernel); one to six chunks of K per wave, ragged N,
+#      bias and residual, both SwiGLU rounding modes
+@pytest.mark.parametrize("B,N,K", [(8, 12288, 1024), (16, 8200, 2048), (32, 8200, 4096), (20, 8192, 6144), (9, 32000, 4096)])
+def test_linear_wide_matrix_resident_form(ops, B, N, K):
+    x, w = rand_bf16(B, K, seed=1), rand_bf16(N, K, std=0.02, seed=2)
+    bias, res = rand_bf16(N, std=0.1, seed=4), rand_bf16(B, N, seed=5)
+    y = ops.linear(x.cuda(), w.cuda(), bias.cuda(), residual=res.cuda())
+    assert_close_bf16(y, res + O.lin(x, w, bias), f"resident linear {B}x{N}x{K}")
+    y2 = ops.linear(x.cuda(), w.cuda())
+    assert_close_bf16(y2, O.lin(x, w), f"resident linear {B}x{N}x{K}, no epilogue terms")
+    assert torch.equal(y2, ops.linear(x.cuda(), w.cuda())), "repeat differs"
+
+
+@pytest.mark.parametrize("B,D,R,mode", [(16, 8200, 2432, 0), (32, 11008, 2432, 1), (8, 8200, 512, 1), (24, 14336, 2048, 0)])
+def test_swiglu_wide_matrix_resident_form(ops, B, D, R, mode):
+    p = rand_bf16(B, 2 * R, seed=1)
+    gu, uu = rand_bf16(D, R, std=0.05, seed=2), rand_bf16(D, R, std=0.05, seed=3)
+    h = ops.swiglu_linear(p.cuda(), gu.cuda(), uu.cuda(), up_off=R, mode=mode)
+    g, u = p[:, :R].float() @ gu.float().t(), p[:, R:].float() @ uu.float().t()
+    if mode == 0:
+        ref = torch.nn.functional.silu(g.to(torch.bfloat16)) * u.to(torch.bfloat16)
+    else:
+        ref = ((g * torch.sigmoid(g)) * u).to(torch.bfloat16)
+    assert_close_bf16(h, ref, f"resident swiglu mode {mode}", **bounds(ref))
+    assert torch.equal(h, ops.swiglu_linear(p.cuda(), gu.cuda(), uu.cuda(), up_off=R, mode=mode)), "repeat differs"
+
+
 # ---- 128 rows and more (prefill): the tiled matrix-core kernel (csrc/mfma_gemm.hip) behind the same entry points
 #      (shapes chosen to reach every tile form: 64 x 64 in K steps of 64 / 128, 128 x 64 and 128 x 128 with four and with
 #      eight waves, 128 x 256 from 2048 big tiles on, loads through registers and straight into LDS, ragged edges in rows
