@@ -46,6 +46,8 @@ def _parse():
     ap.add_argument("--no-stress", action="store_true", help="skip the stress configuration's whole-model pass in the default line")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the kernel-level configurations (for profiler runs: their launches share kernel names with the step's)")
+    ap.add_argument("--kernel-configs-only", action="store_true",
+                    help="only the kernel-level configurations (attention block, MLP at 1 / 8 / 32 rows): the run to trace per kernel")
     ap.add_argument("--engine", choices=["persistent", "graph", "both"], default="both",
                     help="persistent: one resident kernel per token (fsvd_decode_step); graph: one HIP graph of the "
                          "per-operator kernels per token; both: time both, the headline value is the persistent step")
@@ -323,6 +325,9 @@ def run_lowrank(args):
         return res
     dec = GraphedDecoder(model, cache, B)
     dec.set_state(tok, PROMPT_LEN)
+    if args.kernel_configs_only:
+        res["kernel_configs"] = kernel_configs(model, cache, dec, args.layers)
+        return res
     if args.engine in ("graph", "both"):
         dec.capture()
         for _ in range(args.warmup):
@@ -789,6 +794,10 @@ def main():
                           "model_pass": mp, "kernels": kern}))
         return
     lr = run_lowrank(args)
+    if args.kernel_configs_only:
+        print(json.dumps({"metric": "kernel-level configurations, 7B shape rank 0.5: microseconds per call", "unit": "us", "n_gpus": 1,
+                          "dtype": "bf16", "data": "synthetic", "layers": args.layers, "kernel_configs": lr["kernel_configs"]}))
+        return
     if args.prefill_only:
         print(json.dumps({"metric": "prefill tok/s, 7B-shape rank-0.5 bs1 prompt 512", "value": lr["prefill"]["tok_s"], "unit": "tok/s",
                           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16", "data": "synthetic",
