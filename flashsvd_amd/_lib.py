@@ -30,20 +30,54 @@ class TagBuf(ctypes.Structure):
     _fields_ = [("ptr", c_void_p), ("uses_per_step", ctypes.c_int32), ("use", ctypes.c_int32)]
 
 
+class _PhaseU1(ctypes.Union):
+    _fields_ = [("nsplit", ctypes.c_int32), ("rows0", ctypes.c_int32)]
+
+
+class _PhaseU2(ctypes.Union):
+    _fields_ = [("rope_len", ctypes.c_int32), ("in_off", ctypes.c_int32)]
+
+
+class _PhaseU3(ctypes.Union):
+    _fields_ = [("S", ctypes.c_int32), ("in2_len", ctypes.c_int32)]
+
+
+class _PhaseAttnPtrs(ctypes.Structure):
+    _fields_ = [("cos", c_void_p), ("sin", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p)]
+
+
+class _PhaseGemvBufs(ctypes.Structure):
+    _fields_ = [("aux2", TagBuf), ("out1", TagBuf)]
+
+
+class _PhaseU4(ctypes.Union):
+    _anonymous_ = ("attn_ptrs", "gemv_bufs")
+    _fields_ = [("attn_ptrs", _PhaseAttnPtrs), ("gemv_bufs", _PhaseGemvBufs)]
+
+
+class _PhaseU5(ctypes.Union):
+    _fields_ = [("sc_s", c_int64), ("in2_off", ctypes.c_int32)]
+
+
 class Phase(ctypes.Structure):
-    """fsvd_phase (include/flashsvd_hip.h), field for field."""
+    """fsvd_phase (include/flashsvd_hip.h), field for field; the unions overlay the fields of an attention phase with
+    those of a GEMV phase."""
+    _anonymous_ = ("u1", "u2", "u3", "u4", "u5")
     _fields_ = [("type", ctypes.c_int32), ("epilogue", ctypes.c_int32),
                 ("N", ctypes.c_int32), ("K", ctypes.c_int32), ("nmat", ctypes.c_int32), ("mode", ctypes.c_int32),
-                ("H", ctypes.c_int32), ("Hk", ctypes.c_int32), ("Dh", ctypes.c_int32), ("nsplit", ctypes.c_int32),
-                ("rope_len", ctypes.c_int32), ("S", ctypes.c_int32),
-                ("fparam", c_float),
-                ("W", c_void_p * 3), ("norm_w", c_void_p), ("cos", c_void_p), ("sin", c_void_p),
-                ("k_cache", c_void_p), ("v_cache", c_void_p), ("sc_s", c_int64), ("sc_h", c_int64),
+                ("H", ctypes.c_int32), ("Hk", ctypes.c_int32), ("Dh", ctypes.c_int32), ("u1", _PhaseU1),
+                ("u2", _PhaseU2), ("u3", _PhaseU3),
+                ("fparam", c_float), ("flags", ctypes.c_int32),
+                ("W", c_void_p * 3), ("norm_w", c_void_p), ("u4", _PhaseU4),
+                ("u5", _PhaseU5), ("sc_h", c_int64),
                 ("plain_out", c_void_p),
-                ("inp", TagBuf), ("aux0", TagBuf), ("aux1", TagBuf), ("out0", TagBuf),
+                ("inp", TagBuf), ("aux0", TagBuf), ("in2", TagBuf), ("out0", TagBuf),
                 ("qsz", c_void_p * 2), ("ldg", ctypes.c_int32), ("gshift", ctypes.c_int32), ("wbits", ctypes.c_int32),
                 ("shared_in", ctypes.c_int32),
                 ("share_q", ctypes.c_int32), ("share_r", ctypes.c_int32), ("m_kp", ctypes.c_uint32), ("dk", ctypes.c_int32)]
+
+
+assert ctypes.sizeof(Phase) == 256, "fsvd_phase is 64 words: the kernel carries a descriptor in one register per lane"
 
 
 class StepState(ctypes.Structure):
@@ -53,7 +87,8 @@ class StepState(ctypes.Structure):
 
 
 PH_EMBED, PH_GEMV, _PH_RESERVED, PH_ATTN, PH_MERGE, PH_ARGMAX = range(6)
-EP_STORE, EP_RESID, EP_SWIGLU, EP_LOGITS = range(4)
+EP_STORE, EP_RESID, EP_SWIGLU, EP_LOGITS, EP_F32 = range(5)
+PF_NOWAIT, PF_STAGE2, PF_SPLIT = 1, 2, 4
 
 # name -> (restype, argtypes); mirrors include/flashsvd_hip.h declaration by declaration
 SIGNATURES = {

@@ -362,8 +362,10 @@ def decode_profile_from_phases(phases_us: dict, n_layers: int, total_ms_per_tok:
     """The persistent step's per-phase microseconds (averages over layers) as a per-token module profile."""
     def ms(*names):
         return sum(float(phases_us.get(n, {}).get("total", 0.0)) for n in names) / 1000.0
-    attn = ms("attn_rank_proj", "qkv_u", "attn", "attn_merge", "o_v", "o_u")
-    mlp = ms("mlp_rank_proj", "swiglu", "down_v", "down_u")
+    # the composed form of the step takes a layer's rank projections inside other phases: the product with the hidden
+    # state behind the q / k / v expansion or the SwiGLU pair (mlp_rank_x, attn_rank_x), the rest with o_u / down_u
+    attn = ms("attn_rank_proj", "qkv_u", "attn", "attn_merge", "o_v", "o_u", "attn_rank_x", "down_u+attn_rank")
+    mlp = ms("mlp_rank_proj", "swiglu", "down_v", "down_u", "mlp_rank_x", "o_u+mlp_rank")
     per_mod = {"embed_tokens": ms("embed"), "lm_head": ms("lm_head", "argmax")}
     for i in range(int(n_layers)):
         per_mod[f"layer{i}.attn"] = attn

@@ -600,7 +600,7 @@ int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host
     const int rc = validate_decode_step(phases_host, nphase, nwg);
     if (rc != kOk) return rc;
   }
-  return launch_decode_step(phases_dev, nphase, state, nullptr, 1, decode_step_has_q4(phases_host, nphase), static_cast<hipStream_t>(stream));
+  return launch_decode_step(phases_dev, nphase, state, nullptr, 1, decode_step_build(phases_host, nphase), static_cast<hipStream_t>(stream));
 }
 
 int fsvd_decode_step_trace(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase, fsvd_step_state* state,
@@ -613,7 +613,7 @@ int fsvd_decode_step_trace(const fsvd_phase* phases_dev, const fsvd_phase* phase
   const size_t need = (size_t)((nwg + wg_stride - 1) / wg_stride) * nphase * 4;
   if (trace_words < need) { set_last_error("%s: trace buffer holds %zu words, %zu needed", fn, trace_words, need); return kErrWorkspace; }
   return launch_decode_step(phases_dev, nphase, state, reinterpret_cast<unsigned long long*>(trace), wg_stride,
-                            decode_step_has_q4(phases_host, nphase), static_cast<hipStream_t>(stream));
+                            decode_step_build(phases_host, nphase), static_cast<hipStream_t>(stream));
 }
 
 int fsvd_handoff_probe(void* scratch, size_t scratch_bytes, int rounds, int delay, void* stream) {

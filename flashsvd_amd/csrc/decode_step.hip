@@ -17,6 +17,7 @@
 // ~0.2 us.  Hence: descriptors travel in a VGPR and are read with readlane where needed, work splits and
 // reciprocals are precomputed on the host, per-piece address arithmetic is incremental, and waves that
 // own no output rows skip the epilogue.
+#include <algorithm>
 #include <cstddef>
 #include <type_traits>
 #include <vector>
@@ -120,6 +121,7 @@ __device__ __forceinline__ uint64_t desc_u64(uint32_t dv, int word) {
 struct GemvCtx {
   int K, kp, nmat, r0, srows, pps, nsteps, dk;
   int xk;                    // staged elements between the inputs of matrix 0 and matrix 1 (K, or 0 when they share one input)
+  int xoff;                  // element offset of the phase's input in the staging area
   uint64_t base0, base1;     // byte addresses of the slab in matrix 0 / 1
   int q4, ldg, gshift;       // int4 weights: a piece is 32 columns; scale | zero words [N, ldg], group = 32 << gshift columns
   uint64_t sz0, sz1;         // byte addresses of the slab's scale | zero rows
@@ -131,6 +133,7 @@ __device__ __forceinline__ void gemv_ctx(uint32_t dv, int w, GemvCtx& c) {
   c.kp = c.q4 ? c.K >> 5 : c.K >> 3;
   c.nmat = DF_I(dv, nmat);
   c.xk = DF_I(dv, shared_in) ? 0 : c.K;
+  c.xoff = DF_I(dv, in_off);
   const int q = DF_I(dv, share_q), r = DF_I(dv, share_r);
   c.r0 = w * q + min(w, r);
   c.srows = q + (w < r ? 1 : 0);
@@ -360,6 +363,13 @@ __device__ __forceinline__ void ld_coh128_round(u32x4_t (&v)[2], const uint64_t 
                : "v"(a[0]), "v"(a[1])
                : "memory");
 }
+__device__ __forceinline__ void ld_coh128_round(u32x4_t (&v)[5], const uint64_t (&a)[5]) {
+  asm volatile(FSVD_LDC "0, %5, off sc0 sc1\n\t" FSVD_LDC "1, %6, off sc0 sc1\n\t" FSVD_LDC "2, %7, off sc0 sc1\n\t"
+               FSVD_LDC "3, %8, off sc0 sc1\n\t" FSVD_LDC "4, %9, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+               : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4])
+               : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4])
+               : "memory");
+}
 __device__ __forceinline__ void ld_coh128_round(u32x4_t (&v)[8], const uint64_t (&a)[8]) {
   asm volatile(FSVD_LDC "0, %8, off sc0 sc1\n\t" FSVD_LDC "1, %9, off sc0 sc1\n\t" FSVD_LDC "2, %10, off sc0 sc1\n\t"
                FSVD_LDC "3, %11, off sc0 sc1\n\t" FSVD_LDC "4, %12, off sc0 sc1\n\t" FSVD_LDC "5, %13, off sc0 sc1\n\t"
@@ -440,6 +450,71 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
         }
       }
     }
+  }
+  return !fail;
+}
+
+// Staging for the composed form of a layer (FSVD_PF_STAGE2): `a` holds `na` fp32 sums in 64-bit tagged words (products
+// with a hidden state that were completed, unrounded, by the previous phases), `b` the `nb` bf16 values of that hidden
+// state itself.  One round of loads brings both; b goes to LDS as it is (at boff, for a phase that follows without a
+// hand-off) and gives rs = rsqrt(mean(b^2) + eps); a goes to LDS as bf16(a * rs) at 0: the RMSNorm of the hidden state
+// applied as a scalar behind the product (its weight vector is folded into the matrix).
+template <int NS>
+__device__ __forceinline__ bool stage_pair(const void* a, int na, uint32_t ta, const void* b, int nb, uint32_t tb, int boff, float eps,
+                                           const fsvd_step_state* st, int limit, uint16_t* xs, float* red) {
+  const int tid = threadIdx.x;
+  const int npa = na >> 1, npb = nb >> 2;          // 16-byte pieces: two 64-bit words of a, four 32-bit words of b
+  const int sa = (npa + kT - 1) / kT;              // slots of a round that belong to a; the others to b (sa + sb <= NS, host-checked)
+  u32x4_t v[NS];
+  uint64_t adr[NS];
+#pragma unroll
+  for (int j = 0; j < NS; ++j) {                   // every slot is loaded, index clamped
+    const bool isa = j < sa;
+    const int q = (isa ? j : j - sa) * kT + tid;
+    adr[j] = reinterpret_cast<uint64_t>(isa ? a : b) + ((uint64_t)(uint32_t)min(q, (isa ? npa : npb) - 1) << 4);
+  }
+  bool fail = false;
+  for (int spins = 0;; ++spins) {
+    ld_coh128_round(v, adr);
+    bool late = false;
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+      const bool isa = j < sa;
+      const int q = (isa ? j : j - sa) * kT + tid;
+      if (isa) {
+        if (q < npa) late = late || v[j].y != ta || v[j].w != ta;
+      } else if (q < npb) {
+        late = late || (v[j].x >> 16) != tb || (v[j].y >> 16) != tb || (v[j].z >> 16) != tb || (v[j].w >> 16) != tb;
+      }
+    }
+    if (!__any(late ? 1 : 0)) break;
+    if (spins >= limit || ((spins & 255) == 255 && ld_err(st) != 0)) { fail = late; break; }
+    __builtin_amdgcn_s_sleep(2);
+  }
+  float ss = 0.f;
+  uint2* xb = reinterpret_cast<uint2*>(xs + boff);
+#pragma unroll
+  for (int j = 0; j < NS; ++j) {
+    const int q = (j - sa) * kT + tid;
+    if (j >= sa && q < npb) {
+      const uint32_t a0 = v[j].x & 0xffffu, a1 = v[j].y & 0xffffu, a2 = v[j].z & 0xffffu, a3 = v[j].w & 0xffffu;
+      const float f0 = bf16_bits_to_f32(a0), f1 = bf16_bits_to_f32(a1), f2 = bf16_bits_to_f32(a2), f3 = bf16_bits_to_f32(a3);
+      ss += (f0 * f0 + f1 * f1) + (f2 * f2 + f3 * f3);
+      xb[q] = make_uint2(a0 | (a1 << 16), a2 | (a3 << 16));
+    }
+  }
+  ss = wave_sum(ss);
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int i = 0; i < kT / 64; ++i) tot += red[i];
+  const float rs = rsqrtf(tot / (float)nb + eps);
+  uint32_t* xa = reinterpret_cast<uint32_t*>(xs);
+#pragma unroll
+  for (int j = 0; j < NS; ++j) {
+    const int q = j * kT + tid;
+    if (j < sa && q < npa) xa[q] = pack_bf16x2(__uint_as_float(v[j].x) * rs, __uint_as_float(v[j].z) * rs);
   }
   return !fail;
 }
@@ -533,7 +608,8 @@ __device__ __forceinline__ void raise_error(fsvd_step_state* st, int p, int w) {
 // TRACE: workgroups 0, stride, 2*stride, ... record wall-clock ticks (100 MHz) per phase:
 // [0] phase entered, [1] input staged, [2] weights consumed, [3] epilogue done
 // Q4: the list may hold int4 GEMV phases (wbits == 4); the build without them keeps the bf16 walk free of their code
-template <bool TRACE, bool Q4>
+// CX: the list may hold the phases of the composed form (FSVD_PF_* flags, fp32 rows); likewise a build of its own
+template <bool TRACE, bool Q4, bool CX>
 __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __restrict__ phases, int nph, fsvd_step_state* st,
                                                          unsigned long long* trace, int trace_stride) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -568,6 +644,8 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     GemvCtx gc;
     AttnWork aw;
     uint32_t resid = 0;
+    int rows0 = 0x7fffffff;                // GEMV: first row of the fp32 group
+    float addend = 0.f;                    // GEMV: this lane group's fp32 addend (second row group)
     // addresses of the next phase's first window, worked out now (behind the wait for this phase's input) so that the
     // request after publication is nothing but the loads
     uint64_t nxt[kU], nxt_sz[kSzLoads];
@@ -577,25 +655,58 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     if (type == FSVD_PH_GEMV) {
       gemv_ctx<Q4>(dv, w, gc);
       const int epi = DF_I(dv, epilogue);
-      if (epi == FSVD_EP_RESID && (tid >> 3) < gc.srows) resid = ld_coh32(DF_P(dv, aux0), gc.r0 + (tid >> 3));
+      const int flags = CX ? DF_I(dv, flags) : 0;
+      if (CX) rows0 = (flags & FSVD_PF_SPLIT) ? DF_I(dv, rows0) : (epi == FSVD_EP_F32 ? 0 : 0x7fffffff);
+      const int myrow = gc.r0 + (tid >> 3);          // the row whose epilogue this lane group runs (one pass: host-checked)
+      if (epi == FSVD_EP_RESID && (tid >> 3) < gc.srows && myrow < rows0) resid = ld_coh32(DF_P(dv, aux0), myrow);
+      // fp32 addend of a row of the second group: requested now, its tag checked behind the staging (it was published
+      // several hand-offs ago, but by another workgroup and to no reader before this one: nothing else proves it visible)
+      const void* aux2p = CX && desc_u64(dv, FSVD_DW(aux2)) != 0 ? DF_P(dv, aux2) : nullptr;
+      const bool want2 = aux2p != nullptr && (tid >> 3) < gc.srows && myrow >= rows0;
+      uint64_t a2w = 0;
+      if (want2) a2w = ld_coh64(aux2p, myrow - rows0);
       const int gH = DF_I(dv, H);                 // > 0: rows are q | k | v groups with their own inputs
       const int in_len = (gH > 0 ? 3 : (gc.xk ? gc.nmat : 1)) * gc.K;
       const uint32_t tin = DF_TAG16(dv, in, epoch);
       const uint32_t* nw = static_cast<const uint32_t*>(DF_P(dv, norm_w));
-      bool ok;
+      bool ok = true;
       const void* inp = DF_P(dv, in);
-      if (in_len <= 2 * kT * 4) ok = stage_input_wide<2>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
-      else ok = stage_input_wide<8>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+      if (flags & FSVD_PF_NOWAIT) {
+        // the previous phase of this workgroup staged the input; its epilogue may still be reading the partial buffer
+      } else if (flags & FSVD_PF_STAGE2) {
+        const int n2 = DF_I(dv, in2_len);
+        const int slots = ((in_len >> 1) + kT - 1) / kT + ((n2 >> 2) + kT - 1) / kT;
+        if (slots <= 5)
+          ok = stage_pair<5>(inp, in_len, DF_TAG32(dv, in, epoch), DF_P(dv, in2), n2, DF_TAG16(dv, in2, epoch), DF_I(dv, in2_off),
+                             DF_F(dv, fparam), st, limit, xs, red);
+        else
+          ok = stage_pair<8>(inp, in_len, DF_TAG32(dv, in, epoch), DF_P(dv, in2), n2, DF_TAG16(dv, in2, epoch), DF_I(dv, in2_off),
+                             DF_F(dv, fparam), st, limit, xs, red);
+      } else if (in_len <= 2 * kT * 4) {
+        ok = stage_input_wide<2>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+      } else {
+        ok = stage_input_wide<8>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+      }
       // Every load of the staging code has been consumed by now (and the window, requested before the polls, has landed
       // with them: loads complete in order).  The compiler's bookkeeping cannot see that for loads issued under a
       // condition; without this explicit (and free) wait it protects the registers they used with full waits in the
       // middle of the weight stream's batches, which halves the loads in flight there.
       __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), no wait on the other counters
+      if (want2) {
+        const uint32_t t2 = DF_TAG32(dv, aux2, epoch);
+        uint32_t pay = (uint32_t)a2w;
+        if ((uint32_t)(a2w >> 32) != t2 && !poll_w64(aux2p, myrow - rows0, t2, st, limit, pay)) ok = false;
+        addend = __uint_as_float(pay);
+      }
       if (Q4 && gc.q4) {   // the slab's scale | zero table came with the window, ahead of the polls; the barrier publishes it
 #pragma unroll
         for (int j = 0; j < kSzLoads; ++j) sztab[j * kT + tid] = SZ[j];
       }
-      if (__syncthreads_or((ok && (Q4 || DF_I(dv, wbits) != 4)) ? 0 : 1)) { raise_error(st, p, w); return; }   // int4 phase in the bf16 build
+      // an int4 phase in the bf16 build, or a phase of the composed form in a build without it, is an error too
+      if (__syncthreads_or((ok && (Q4 || DF_I(dv, wbits) != 4) && (CX || (DF_I(dv, flags) == 0 && epi != FSVD_EP_F32))) ? 0 : 1)) {
+        raise_error(st, p, w);
+        return;
+      }
       if (TRACE && tr) tr[1] = wall_clock64();
       const uint32_t m_kp = desc_u32(dv, FSVD_DW(m_kp));
       if (Q4 && gc.q4) {
@@ -609,11 +720,11 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         }
       } else if (gH > 0) {
         const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
-        gemv_stream<1, true>(gc, m_kp, g1, g2, R, xs, cp);
+        gemv_stream<1, true>(gc, m_kp, g1, g2, R, xs + (CX ? gc.xoff : 0), cp);
       } else if (gc.nmat == 1) {
-        gemv_stream<1, false>(gc, m_kp, 0, 0, R, xs, cp);
+        gemv_stream<1, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cp);
       } else {
-        gemv_stream<2, false>(gc, m_kp, 0, 0, R, xs, cp);
+        gemv_stream<2, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cp);
       }
       __syncthreads();
     } else if (type == FSVD_PH_ATTN) {
@@ -738,6 +849,11 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           const int t = min(ps * (kT / 8) + grp, gc.srows - 1);
           const bool live = lead && ps * (kT / 8) + grp < gc.srows;
           float v;
+          if (CX && gc.r0 + t >= rows0) {      // fp32 row group: the unrounded sum (+ the part of it an earlier phase left)
+            v = row_sum8(cp, t, cpr) + addend;
+            if (live) st_tag64(DF_P(dv, out1), gc.r0 + t - rows0, DF_TAG32(dv, out1, epoch), __float_as_uint(v));
+            continue;
+          }
           if (epi == FSVD_EP_SWIGLU) {
             float gv = row_sum8(cp, t, cpr), uv = row_sum8(cp, gc.srows + t, cpr);
             if (mode == 0) {
@@ -909,8 +1025,9 @@ int decode_step_workgroups() {
     set_last_error("fsvd_decode_step: cannot query the device");
     return 0;
   }
-  const void* fns[4] = {reinterpret_cast<const void*>(decode_step_kernel<false, false>), reinterpret_cast<const void*>(decode_step_kernel<true, false>),
-                        reinterpret_cast<const void*>(decode_step_kernel<false, true>), reinterpret_cast<const void*>(decode_step_kernel<true, true>)};
+  const void* fns[6] = {reinterpret_cast<const void*>(decode_step_kernel<false, false, false>), reinterpret_cast<const void*>(decode_step_kernel<true, false, false>),
+                        reinterpret_cast<const void*>(decode_step_kernel<false, true, false>), reinterpret_cast<const void*>(decode_step_kernel<true, true, false>),
+                        reinterpret_cast<const void*>(decode_step_kernel<false, false, true>), reinterpret_cast<const void*>(decode_step_kernel<true, false, true>)};
   for (const void* fn : fns) {
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSmemBytes) != hipSuccess) {
       set_last_error("fsvd_decode_step: the device refuses %zu bytes of dynamic LDS per workgroup", kSmemBytes);
@@ -952,13 +1069,44 @@ static int bad(const char* what, int p) {
   return kErrBadShape;
 }
 
+// staged elements of a GEMV phase's own input
+static int gemv_in_len(const fsvd_phase& d) { return (d.H > 0 ? 3 : (d.shared_in ? 1 : d.nmat)) * d.K; }
+
 int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
   if (nph < 2) return bad("a step needs at least two phases", 0);
+  {
+    bool any_q4 = false, any_cx = false;
+    for (int p = 0; p < nph; ++p) {
+      if (ph[p].type != FSVD_PH_GEMV) continue;
+      any_q4 = any_q4 || ph[p].wbits == 4;
+      any_cx = any_cx || ph[p].flags != 0 || ph[p].epilogue == FSVD_EP_F32;
+    }
+    if (any_q4 && any_cx) return bad("a list holds int4 phases or phases of the composed form, not both (they run on different builds of the kernel)", 0);
+  }
 
-  // last phase index that wrote each buffer and whether a "closing" GEMV consumed a fully-shared vector since
-  struct Seen { const void* ptr; int last_write; fsvd_tagbuf tb; };
+  // Every tagged buffer with the phase that wrote it last.  `full`: every workgroup wrote part of it in that phase (a
+  // consumer that has polled all of it knows that every workgroup is through that phase); `half`: it is one of the two
+  // outputs of a phase with two row groups, which cover the workgroups only together.
+  struct Seen { const void* ptr; int last_write; fsvd_tagbuf tb; bool full, half; };
   std::vector<Seen> seen;
-  std::vector<char> writes_all(nph, 0);
+  auto find = [&](const void* ptr) -> Seen* {
+    for (auto& s : seen)
+      if (s.ptr == ptr) return &s;
+    return nullptr;
+  };
+  auto reads = [&](const fsvd_phase& d, const void* o) -> bool {
+    if (!o) return false;
+    if (d.type == FSVD_PH_GEMV) {
+      if (!(d.flags & FSVD_PF_NOWAIT) && d.in.ptr == o) return true;
+      if ((d.flags & FSVD_PF_STAGE2) && d.in2.ptr == o) return true;
+      if (d.epilogue == FSVD_EP_RESID && d.aux0.ptr == o) return true;
+      return d.aux2.ptr == o;
+    }
+    return d.in.ptr == o;
+  };
+  // the phase up to which every workgroup is known to have come once phase q has staged its input: the producer of a
+  // fully polled vector that every workgroup helped to write (-1: none)
+  std::vector<int> closes(nph, -1);
   for (int p = 0; p < nph; ++p) {
     const fsvd_phase& d = ph[p];
     {
@@ -971,10 +1119,11 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         ok = ok && d.m_kp == 0xffffffffu / (uint32_t)(d.K / pc) + 1u && d.dk == kT % (d.K / pc);
       if (!ok) return bad("derived fields missing: call fsvd_decode_step_prepare", p);
     }
+    bool out0_written = true, out1_written = false;
     switch (d.type) {
       case FSVD_PH_EMBED:
+        if (p != 0) return bad("the embedding phase must come first", p);
         if (!d.W[0] || !d.out0.ptr || d.N < nwg) return bad("embedding phase needs W[0], out0 and N >= workgroups", p);
-        writes_all[p] = 1;
         break;
       case FSVD_PH_GEMV: {
         if (d.nmat < 1 || d.nmat > 2 || !d.W[0] || (d.nmat == 2 && !d.W[1])) return bad("GEMV needs 1 or 2 matrices", p);
@@ -990,46 +1139,84 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
             if (reinterpret_cast<uintptr_t>(d.qsz[m]) & 3) return bad("scale | zero words must be 4-byte aligned", p);
         }
         if (d.N < nwg) return bad("fewer rows than workgroups", p);
+        if (d.flags & ~(FSVD_PF_NOWAIT | FSVD_PF_STAGE2 | FSVD_PF_SPLIT)) return bad("unknown flag", p);
+        const bool nowait = d.flags & FSVD_PF_NOWAIT, stage2 = d.flags & FSVD_PF_STAGE2, split = d.flags & FSVD_PF_SPLIT;
+        const bool f32rows = split || d.epilogue == FSVD_EP_F32;
+        if ((d.flags != 0 || f32rows || d.in_off != 0) && q4) return bad("flags, fp32 rows and input offsets are for bf16 weights", p);
         if (d.H > 0) {   // q | k | v row groups reading [Pq | Pk | Pv]
-          if (d.nmat != 1 || d.epilogue != FSVD_EP_STORE || d.norm_w) return bad("grouped GEMV is a plain single-matrix store", p);
+          if (d.nmat != 1 || d.epilogue != FSVD_EP_STORE || d.norm_w || split) return bad("grouped GEMV is a plain single-matrix store", p);
           if (d.Hk <= 0 || d.Dh <= 0 || d.N != (d.H + 2 * d.Hk) * d.Dh) return bad("grouped GEMV needs N = (H + 2*Hk) * Dh", p);
-          if (3 * d.K > kMaxIn) return bad("input vector longer than the staging buffer", p);
         }
         if (d.shared_in != 0 && (d.nmat != 2 || d.H > 0)) return bad("shared_in is for a pair of matrices over one input", p);
-        const int n_in = d.shared_in ? 1 : d.nmat;
-        if (n_in * d.K > kMaxIn) return bad("input vector longer than the staging buffer", p);
-        if (d.norm_w && n_in * d.K > kT * 12 * 2) return bad("normalised input too long for one staging round", p);
+        const int n_in = gemv_in_len(d);
+        if (d.in_off < 0 || d.in_off % 8 != 0 || (int64_t)d.in_off + n_in > kMaxIn) return bad("input does not fit the staging buffer", p);
+        if (d.norm_w && n_in > kT * 12 * 2) return bad("normalised input too long for one staging round", p);
+        if (nowait) {
+          // the input is what the previous phase of the same workgroup left in its staging area
+          if (stage2 || d.norm_w || d.aux2.ptr) return bad("a phase without a hand-off stages nothing and takes no addend", p);
+          if (p == 0 || ph[p - 1].type != FSVD_PH_GEMV) return bad("a phase without a hand-off must follow a GEMV phase", p);
+          const fsvd_phase& q = ph[p - 1];
+          const bool from_in2 = (q.flags & FSVD_PF_STAGE2) && d.in_off == q.in2_off && n_in == q.in2_len;
+          const bool same_in = d.in_off == q.in_off && n_in <= gemv_in_len(q) && !q.norm_w && !(q.flags & FSVD_PF_STAGE2);
+          if (!from_in2 && !same_in) return bad("a phase without a hand-off must read what the previous phase staged", p);
+        } else if (d.in_off != 0) {
+          return bad("a staged input starts at offset 0", p);
+        }
+        if (stage2) {
+          if (d.norm_w) return bad("two-vector staging applies the norm as a scalar: fold norm_w into the matrix", p);
+          if (!d.in2.ptr || d.in2_len <= 0 || d.in2_len % 8 != 0 || d.in2_off % 8 != 0 || d.in2_off < n_in ||
+              (int64_t)d.in2_off + d.in2_len > kMaxIn)
+            return bad("second staged vector missing, misaligned, overlapping the first or past the staging buffer", p);
+          if (((n_in / 2) + kT - 1) / kT + ((d.in2_len / 4) + kT - 1) / kT > 8) return bad("two-vector staging needs more than one round of loads", p);
+        }
         const int64_t rows = ((int64_t)d.N + nwg - 1) / nwg;
         if (rows * d.nmat * (d.K / (q4 ? 256 : 128)) > kMaxChunks) return bad("too many rows per workgroup for the partial buffer", p);
+        if (d.epilogue < 0 || d.epilogue > FSVD_EP_F32) return bad("unknown epilogue", p);
         if ((d.epilogue == FSVD_EP_SWIGLU) != (d.nmat == 2)) return bad("SwiGLU epilogue needs exactly two matrices", p);
         if (d.epilogue == FSVD_EP_RESID && !d.aux0.ptr) return bad("residual epilogue needs aux0", p);
         if (d.epilogue == FSVD_EP_RESID && rows > kT / 8) return bad("residual epilogue handles at most kT/8 rows per workgroup", p);
+        if (split) {
+          if (d.rows0 <= 0 || d.rows0 >= d.N) return bad("rows0 must cut the rows into two non-empty groups", p);
+          if (d.epilogue != FSVD_EP_STORE && d.epilogue != FSVD_EP_RESID) return bad("the first row group stores or adds a residual", p);
+        }
+        if (f32rows) {
+          if (d.nmat != 1) return bad("fp32 rows come from a single matrix", p);
+          if (!d.out1.ptr) return bad("fp32 rows need out1", p);
+          if ((d.aux2.ptr || split) && rows > kT / 8) return bad("a phase with two row groups or an addend handles at most kT/8 rows per workgroup", p);
+        } else if (d.aux2.ptr || d.out1.ptr) {
+          // aux2 / out1 overlay the attention pointers; a GEMV without fp32 rows must leave them empty
+          return bad("aux2 / out1 without fp32 rows", p);
+        }
         if ((rows + kU) * d.nmat * (d.K / (q4 ? 32 : 8)) * (int64_t)(d.K / (q4 ? 32 : 8)) >= (1ll << 32)) return bad("slab too large for the index arithmetic", p);
         if (d.epilogue == FSVD_EP_LOGITS && !d.plain_out) return bad("logits epilogue needs plain_out", p);
-        if (d.epilogue < 0 || d.epilogue > FSVD_EP_LOGITS) return bad("unknown epilogue", p);
-        if (!d.in.ptr || !d.out0.ptr) return bad("GEMV needs in and out0", p);
+        if ((!nowait && !d.in.ptr) || (d.epilogue != FSVD_EP_F32 && !d.out0.ptr)) return bad("GEMV needs in and out0", p);
         for (int m = 0; m < d.nmat; ++m)
           if (reinterpret_cast<uintptr_t>(d.W[m]) & 15) return bad("weights must be 16-byte aligned", p);
-        writes_all[p] = 1;
+        out0_written = d.epilogue != FSVD_EP_F32;
+        out1_written = f32rows;
         break;
       }
-      case FSVD_PH_ATTN:
+      case FSVD_PH_ATTN: {
         if (d.Dh != 128) return bad("attention phase needs head_dim 128", p);
         if (d.H <= 0 || d.Hk <= 0 || d.H % d.Hk != 0) return bad("bad head counts", p);
         if (d.nsplit <= 0 || d.H * d.nsplit != nwg) return bad("H * nsplit must equal the workgroup count", p);
         if (!d.in.ptr || !d.out0.ptr || !d.k_cache || !d.v_cache) return bad("attention needs in = [q|k|v], out0 and the caches", p);
         // the producer is the grouped head expansion (H > 0, same geometry) or a plain GEMV of that many rows (a dense
-        // [q; k; v] projection)
-        if (p == 0 || ph[p - 1].type != FSVD_PH_GEMV || ph[p - 1].epilogue != FSVD_EP_STORE || ph[p - 1].N != (d.H + 2 * d.Hk) * d.Dh ||
-            (ph[p - 1].H != 0 && (ph[p - 1].H != d.H || ph[p - 1].Hk != d.Hk || ph[p - 1].Dh != d.Dh)))
-          return bad("attention must follow the GEMV that writes (H + 2*Hk) * Dh values of q, k, v", p);
+        // [q; k; v] projection); phases without a hand-off may sit between the two
+        const Seen* s = find(d.in.ptr);
+        const fsvd_phase* pr = s ? &ph[s->last_write] : nullptr;
+        if (!pr || pr->type != FSVD_PH_GEMV || pr->epilogue != FSVD_EP_STORE || (pr->flags & FSVD_PF_SPLIT) || pr->out0.ptr != d.in.ptr ||
+            pr->N != (d.H + 2 * d.Hk) * d.Dh || (pr->H != 0 && (pr->H != d.H || pr->Hk != d.Hk || pr->Dh != d.Dh)))
+          return bad("attention must read the output of the GEMV that writes (H + 2*Hk) * Dh values of q, k, v", p);
+        for (int q = s->last_write + 1; q < p; ++q)
+          if (ph[q].type != FSVD_PH_GEMV || !(ph[q].flags & FSVD_PF_NOWAIT)) return bad("only phases without a hand-off may sit between the q, k, v projection and its attention phase", p);
         if ((d.cos == nullptr) != (d.sin == nullptr) || (d.cos && d.rope_len <= 0)) return bad("rope tables incomplete", p);
         if ((d.sc_s % 8) || (d.sc_h % 8) || (reinterpret_cast<uintptr_t>(d.k_cache) & 15) || (reinterpret_cast<uintptr_t>(d.v_cache) & 15))
           return bad("cache strides/pointers must be 16-byte aligned", p);
         if (d.S <= 0) return bad("cache length missing", p);
         if (kSlots * (d.Dh + 2) + kSlots + 1 > kMaxChunks) return bad("internal: slot buffer", p);
-        writes_all[p] = 1;
         break;
+      }
       case FSVD_PH_MERGE:
         if (p == 0 || ph[p - 1].type != FSVD_PH_ATTN) return bad("merge must follow an attention phase", p);
         if (d.H != ph[p - 1].H || d.Dh != ph[p - 1].Dh || d.nsplit != ph[p - 1].nsplit || d.in.ptr != ph[p - 1].out0.ptr)
@@ -1037,75 +1224,96 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         if (!d.out0.ptr || (d.H * d.Dh) % nwg != 0 || d.Dh % ((d.H * d.Dh) / nwg) != 0)
           return bad("merge needs out0 and H*Dh split evenly over the workgroups inside heads", p);
         if (d.nsplit * ((d.H * d.Dh) / nwg + 2) > kMaxChunks) return bad("internal: merge buffer", p);
-        writes_all[p] = 1;
         break;
       case FSVD_PH_ARGMAX:
         if (p == 0 || ph[p - 1].type != FSVD_PH_GEMV || ph[p - 1].epilogue != FSVD_EP_LOGITS || d.in.ptr != ph[p - 1].out0.ptr)
           return bad("argmax must follow a logits GEMV and read its candidates", p);
         if (p != nph - 1) return bad("argmax must be the last phase", p);
+        out0_written = false;
         break;
       default:
         return bad("unknown phase type", p);
     }
     // every read must find its producer's tag schedule
-    auto check_read = [&](const fsvd_tagbuf& r) -> bool {
-      for (auto& s : seen)
-        if (s.ptr == r.ptr) return s.tb.uses_per_step == r.uses_per_step && s.tb.use == r.use;
-      return false;
+    auto check_read = [&](const fsvd_tagbuf& r) -> const Seen* {
+      const Seen* s = find(r.ptr);
+      return (s && s->tb.uses_per_step == r.uses_per_step && s->tb.use == r.use) ? s : nullptr;
     };
-    if (d.type != FSVD_PH_EMBED) {
-      if (p == 0 || d.in.ptr != ph[p - 1].out0.ptr) return bad("a phase must read the previous phase's out0", p);
-      if (!check_read(d.in)) return bad("input tag schedule differs from the producer's", p);
-      if (d.type == FSVD_PH_GEMV && d.epilogue == FSVD_EP_RESID && !check_read(d.aux0))
-        return bad("residual tag schedule differs from the producer's", p);
-    } else if (p != 0) {
-      return bad("the embedding phase must come first", p);
+    const bool nowait = d.type == FSVD_PH_GEMV && (d.flags & FSVD_PF_NOWAIT);
+    if (d.type != FSVD_PH_EMBED && !nowait) {
+      const Seen* s = check_read(d.in);
+      if (!s) return bad("the input was not written by an earlier phase of the step, or with another tag schedule", p);
+      if (d.type == FSVD_PH_GEMV) {
+        // a fully polled input that every workgroup helped to write tells the reader that all of them are through its
+        // producer; the two outputs of a phase with two row groups say so only together
+        if (s->full) closes[p] = s->last_write;
+        if (d.flags & FSVD_PF_STAGE2) {
+          const Seen* s2 = check_read(d.in2);
+          if (!s2) return bad("the second staged vector was not written by an earlier phase, or with another tag schedule", p);
+          if (s2->full) closes[p] = std::max(closes[p], s2->last_write);
+          if (s->half && s2->half && s->last_write == s2->last_write) closes[p] = std::max(closes[p], s->last_write);
+        }
+      }
     }
-    // write-after-read safety: between two writes of one buffer there must be a GEMV phase (which reads
-    // its whole input) whose input every workgroup helped to write, and that phase must come after the
-    // last reader of the old contents (readers are the next phase, or a residual / attention aux read).
-    const fsvd_tagbuf* outs[1] = {&d.out0};
+    if (d.type == FSVD_PH_GEMV) {
+      if (d.epilogue == FSVD_EP_RESID && !check_read(d.aux0)) return bad("residual tag schedule differs from the producer's", p);
+      if (d.aux2.ptr && !check_read(d.aux2)) return bad("addend tag schedule differs from the producer's", p);
+    }
+    // write-after-read safety: between two writes of one buffer every workgroup must be known to have finished reading
+    // the old contents, i.e. some phase q in (last reader, this phase] has staged an input that closes a phase at or
+    // behind the last reader (a phase stages before it writes, so q may be this phase itself).
+    const fsvd_tagbuf* outs[2] = {out0_written ? &d.out0 : nullptr, out1_written ? &d.out1 : nullptr};
     for (const fsvd_tagbuf* ob : outs) {
       if (!ob || !ob->ptr) continue;
-      void* o = ob->ptr;
+      const void* o = ob->ptr;
       if (ob->uses_per_step <= 0 || ob->use < 0 || ob->use >= ob->uses_per_step) return bad("bad tag schedule", p);
-      int prev = -1;
-      for (auto& s : seen)
-        if (s.ptr == o) { prev = s.last_write; s.last_write = p; s.tb = *ob; }
-      if (prev < 0) { seen.push_back({o, p, *ob}); continue; }
-      // last reader of the previous contents
-      int last_read = prev + 1;
-      for (int q = prev + 1; q < p; ++q)
-        if (ph[q].in.ptr == o || ph[q].aux0.ptr == o) last_read = q;
+      const bool split = d.type == FSVD_PH_GEMV && (d.flags & FSVD_PF_SPLIT);
+      Seen* s = find(o);
+      if (!s) { seen.push_back({o, p, *ob, !split, split}); continue; }
+      const int prev = s->last_write;
+      int last_read = prev;
+      for (int q = prev + 1; q <= p; ++q)
+        if (reads(ph[q], o)) last_read = q;
+      if (last_read == p) return bad("a phase must not write a buffer that it reads", p);
       bool closed = false;
-      for (int q = last_read + 1; q <= p && !closed; ++q)
-        if (ph[q].type == FSVD_PH_GEMV && q > 0 && writes_all[q - 1] && q - 1 >= last_read) closed = true;
+      for (int q = last_read + 1; q <= p && !closed; ++q) closed = closes[q] >= last_read;
       if (!closed) return bad("buffer is rewritten before a full hand-off separates it from its last reader", p);
+      *s = {o, p, *ob, !split, split};
     }
   }
   return kOk;
 }
 
-bool decode_step_has_q4(const fsvd_phase* host, int nph) {
-  if (!host) return false;
-  for (int p = 0; p < nph; ++p)
-    if (host[p].type == FSVD_PH_GEMV && host[p].wbits == 4) return true;
-  return false;
+// Which build of the kernel a list needs: 0 plain bf16, 1 with the int4 code (~5 % slower on a bf16 list), 2 with the
+// code of the composed form.  A build that meets a phase it was not compiled for raises the step's error flag.
+int decode_step_build(const fsvd_phase* host, int nph) {
+  if (!host) return 0;
+  int build = 0;
+  for (int p = 0; p < nph; ++p) {
+    if (host[p].type != FSVD_PH_GEMV) continue;
+    if (host[p].wbits == 4) return 1;
+    if (host[p].flags != 0 || host[p].epilogue == FSVD_EP_F32) build = 2;
+  }
+  return build;
 }
 
-// q4: the list holds int4 GEMV phases (the build without their code is ~5 % faster on a bf16 list; it raises the
-// step's error flag if it meets one)
-int launch_decode_step(const fsvd_phase* dev, int nph, fsvd_step_state* st, unsigned long long* trace, int trace_stride, bool q4,
+int launch_decode_step(const fsvd_phase* dev, int nph, fsvd_step_state* st, unsigned long long* trace, int trace_stride, int build,
                        hipStream_t stream) {
   const int nwg = decode_step_workgroups();
   if (nwg <= 0) return kErrLaunch;   // the reason is in the last-error text
+  unsigned long long* tp = trace ? trace : nullptr;
+  const int ts = trace ? trace_stride : 1;
+#define FSVD_LAUNCH(T, Q, C) hipLaunchKernelGGL((decode_step_kernel<T, Q, C>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, tp, ts)
   if (trace) {
-    if (q4) hipLaunchKernelGGL((decode_step_kernel<true, true>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, trace, trace_stride);
-    else hipLaunchKernelGGL((decode_step_kernel<true, false>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, trace, trace_stride);
+    if (build == 1) FSVD_LAUNCH(true, true, false);
+    else if (build == 2) FSVD_LAUNCH(true, false, true);
+    else FSVD_LAUNCH(true, false, false);
   } else {
-    if (q4) hipLaunchKernelGGL((decode_step_kernel<false, true>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, nullptr, 1);
-    else hipLaunchKernelGGL((decode_step_kernel<false, false>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, nullptr, 1);
+    if (build == 1) FSVD_LAUNCH(false, true, false);
+    else if (build == 2) FSVD_LAUNCH(false, false, true);
+    else FSVD_LAUNCH(false, false, false);
   }
+#undef FSVD_LAUNCH
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("fsvd_decode_step: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
   return kOk;

@@ -15,11 +15,13 @@ from __future__ import annotations
 
 import ctypes
 import math
+import os
 
 import torch
 
 from . import _lib
-from ._lib import EP_LOGITS, EP_RESID, EP_STORE, EP_SWIGLU, PH_ARGMAX, PH_ATTN, PH_EMBED, PH_GEMV, PH_MERGE, Phase, TagBuf
+from ._lib import (EP_F32, EP_LOGITS, EP_RESID, EP_STORE, EP_SWIGLU, PF_NOWAIT, PF_SPLIT, PF_STAGE2, PH_ARGMAX, PH_ATTN, PH_EMBED,
+                   PH_GEMV, PH_MERGE, Phase, TagBuf)
 from .runtime.cache import FlashSVDV15DenseKVCache
 
 
@@ -42,10 +44,13 @@ class PersistentDecoder:
     """
 
     def __init__(self, model, cache, *, mode: int | None = None, max_new_tokens: int = 4096, part: str = "model",
-                 layer: int = 0):
+                 layer: int = 0, composed: bool | None = None):
         """``part``: "model" (the whole token), or — for timing one block through the same machinery — "attention"
         (embedding row -> the attention half of layer ``layer``, ending at its residual add) or "mlp" (embedding row ->
-        the MLP half of that layer).  A part has no argmax phase: token and position stay where ``set_state`` put them."""
+        the MLP half of that layer).  A part has no argmax phase: token and position stay where ``set_state`` put them.
+
+        ``composed`` (default: FLASHSVD_AMD_STEP_COMPOSED, off) selects the composed form of a bf16 layer, see
+        ``_composed_layers``; the default ten-phase form follows the module walk one projection per phase."""
         from .llama import _packed_rows, mlp_rounding_mode
         if part not in ("model", "attention", "mlp"):
             raise ValueError(f"part must be 'model', 'attention' or 'mlp', got {part!r}")
@@ -152,6 +157,7 @@ class PersistentDecoder:
         self._keep = []   # tensors whose storage the phase list points into
 
         ph: list[Phase] = []
+        names: list[str] = []
 
         def sz_words(scales, zeros):
             """uint32 [N, G]: fp16 scale bits in the low half, zero point + 128 in the high half (what a piece needs in one load)."""
@@ -175,7 +181,8 @@ class PersistentDecoder:
             out_[:, :w.shape[1]] = w.data
             return out_
 
-        def gemv(W, N, K, inp, out, *, nmat=1, norm=None, eps=0.0, epi=EP_STORE, aux=None, plain=None, groups=None, q4=None):
+        def gemv(name, W, N, K, inp, out, *, nmat=1, norm=None, eps=0.0, epi=EP_STORE, aux=None, plain=None, groups=None, q4=None,
+                 flags=0, in_off=0, in2=None, in2_len=0, in2_off=0, rows0=0, aux2=None, out1=None):
             p = Phase()
             p.type, p.epilogue, p.N, p.K, p.nmat, p.mode = PH_GEMV, epi, N, K, nmat, mode
             if groups is not None:          # rows are q | k | v heads, each group reads its own K-long input
@@ -199,12 +206,78 @@ class PersistentDecoder:
             if norm is not None:
                 p.norm_w, p.fparam = norm.data_ptr(), float(eps)
                 self._keep.append(norm)
-            p.inp, p.out0 = inp, out
+            elif flags & PF_STAGE2:
+                p.fparam = float(eps)
+            p.flags, p.in_off = int(flags), int(in_off)
+            if flags & PF_STAGE2:
+                p.in2, p.in2_len, p.in2_off = in2, int(in2_len), int(in2_off)
+            if flags & PF_SPLIT:
+                p.rows0 = int(rows0)
+            if inp is not None:
+                p.inp = inp
+            if out is not None:
+                p.out0 = out
             if aux is not None:
                 p.aux0 = aux
+            if aux2 is not None:
+                p.aux2 = aux2
+            if out1 is not None:
+                p.out1 = out1
             if plain is not None:
                 p.plain_out = plain.data_ptr()
             ph.append(p)
+            names.append(name)
+
+        def attention(l, lc):
+            kc, vc = cache.key_cache[lc][0], cache.value_cache[lc][0]    # [S, Hk, Dh]
+            a = Phase()
+            a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
+            a.fparam = 1.0 / math.sqrt(Dh)
+            a.cos, a.sin, a.rope_len = cos.data_ptr(), sin.data_ptr(), int(cos.shape[0])
+            a.k_cache, a.v_cache, a.sc_s, a.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
+            a.inp, a.out0 = _tb(self.QKV, L, l), _tb(self.PART, L, l)
+            ph.append(a)
+            names.append("attn")
+            m = Phase()
+            m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
+            m.inp, m.out0 = _tb(self.PART, L, l), _tb(self.A, L, l)
+            ph.append(m)
+            names.append("attn_merge")
+
+        def bf16_weights(l):
+            """The nine matrices of a bf16 layer as the kernel streams them: [q_v; k_v; v_v], [q_u; k_u; v_u], o_v, o_u,
+            [gate_v; up_v], gate_u, up_u, down_v, down_u, zero-padded to the layer's working ranks where needed."""
+            layer = layers[l]
+            at, mlp = layer.self_attn, layer.mlp
+            rq, ro, rm, rd = ranks[l]
+            if padded[l]["qkv"]:
+                # unequal or unaligned q / k / v ranks: [q_v; k_v; v_v] with each block padded to rq rows, and the head bases
+                # with their columns padded to rq
+                aq, ak, av = at._qkv_rank_tuple()
+                pv = torch.zeros(3 * rq, d, dtype=torch.bfloat16, device=dev)
+                qu = torch.zeros((H + 2 * Hk) * Dh, rq, dtype=torch.bfloat16, device=dev)
+                for i, (m_v, m_u, r_, row0, rows) in enumerate(((at.q_v_proj, at.q_u_proj, aq, 0, H * Dh), (at.k_v_proj, at.k_u_proj, ak, H * Dh, Hk * Dh),
+                                                                (at.v_v_proj, at.v_u_proj, av, (H + Hk) * Dh, Hk * Dh))):
+                    pv[i * rq:i * rq + r_] = m_v.weight.data
+                    qu[row0:row0 + rows, :r_] = m_u.weight.data
+            else:
+                pv = at._packed_qkv_v
+                # the three module weights become views of one buffer
+                qu = _packed_rows([at.q_u_proj, at.k_u_proj, at.v_u_proj])
+            w_ov, w_ou = at.o_v_proj.weight, at.o_u_proj.weight
+            if padded[l]["o"]:
+                w_ov, w_ou = pad_rows(w_ov, ro), pad_cols(w_ou, ro)
+            w_guv, w_gu, w_uu = mlp._packed_gu_v, mlp.gate_u_proj.weight, mlp.up_u_proj.weight
+            if padded[l]["gu"]:
+                am = int(mlp.gate_v_proj.out_features)
+                w_guv = torch.zeros(2 * rm, d, dtype=torch.bfloat16, device=dev)
+                w_guv[:am] = mlp.gate_v_proj.weight.data
+                w_guv[rm:rm + am] = mlp.up_v_proj.weight.data
+                w_gu, w_uu = pad_cols(w_gu, rm), pad_cols(w_uu, rm)
+            w_dv, w_du = mlp.down_v_proj.weight, mlp.down_u_proj.weight
+            if padded[l]["d"]:
+                w_dv, w_du = pad_rows(w_dv, rd), pad_cols(w_du, rd)
+            return dict(qkv_v=pv, qkv_u=qu, o_v=w_ov, o_u=w_ou, gu_v=w_guv, gate_u=w_gu, up_u=w_uu, down_v=w_dv, down_u=w_du)
 
         e = Phase()
         e.type, e.N = PH_EMBED, d
@@ -215,14 +288,30 @@ class PersistentDecoder:
         e.W[0] = emb.data_ptr()
         e.out0 = _tb(self.XB, L, 0) if part == "mlp" else _tb(self.XA, L + 1, 0)     # an MLP part starts at the mid-layer state
         ph.append(e)
+        names.append("embed")
+        for layer in layers:
+            layer.self_attn._ensure_runtime_state()
+            layer.mlp._ensure_runtime_state()
+        if composed is None:
+            composed = os.getenv("FLASHSVD_AMD_STEP_COMPOSED", "0").strip().lower() in ("1", "true", "on", "yes")
+        # the composed form is for whole bf16 models whose two-vector stagings fit one round of loads
+        in2_off_a = (3 * Rq + 127) // 128 * 128
+        in2_off_m = (2 * Rm + 127) // 128 * 128
+
+        def slots(n_sums):
+            return (n_sums // 2 + 511) // 512 + (d // 4 + 511) // 512
+
+        self.composed = bool(composed) and part == "model" and not any(layer_q4) and max(slots(3 * Rq), slots(2 * Rm)) <= 8 \
+            and max(in2_off_a, in2_off_m) + d <= 16384 and d + max(3 * Rq, 2 * Rm) <= 64 * self.nwg
+        if self.composed:
+            self._composed_layers(layers, ranks, bf16_weights, gemv, attention, in2_off_a, in2_off_m)
         for l, layer in enumerate(layers):
+            if self.composed:
+                break
             at, mlp = layer.self_attn, layer.mlp
-            at._ensure_runtime_state()
-            mlp._ensure_runtime_state()
             rq, ro, rm, rd = ranks[l]
             lc = l if part == "model" else layer_index                    # the layer's index in the cache
             cache._ensure_layer_spec(lc, h=Hk, dh=Dh)
-            kc, vc = cache.key_cache[lc][0], cache.value_cache[lc][0]    # [S, Hk, Dh]
             n1, n2 = layer.input_layernorm, layer.post_attention_layernorm
             xin, xmid, xout = _tb(self.XA, L + 1, l), _tb(self.XB, L, l), _tb(self.XA, L + 1, l + 1)
             q4 = layer_q4[l]
@@ -237,95 +326,133 @@ class PersistentDecoder:
                     raise ValueError(f"PersistentDecoder: int4 factors of layer {l} cannot share a stream (group sizes differ)")
                 return pk, int(mods[0].group_size)
 
+            bw = None if q4 else bf16_weights(l)
             if part == "mlp":
                 pass
             elif q4:
                 w, gs = triple(at.q_v_proj, at.k_v_proj, at.v_v_proj)
-                gemv([w], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon, q4=gs)
+                gemv("attn_rank_proj", [w], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon, q4=gs)
                 w, gs = triple(at.q_u_proj, at.k_u_proj, at.v_u_proj)
-                gemv([w], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh), q4=gs)
-            elif padded[l]["qkv"]:
-                # unequal or unaligned q / k / v ranks: [q_v; k_v; v_v] with each block padded to rq rows, and the head bases
-                # with their columns padded to rq
-                aq, ak, av = at._qkv_rank_tuple()
-                pv = torch.zeros(3 * rq, d, dtype=torch.bfloat16, device=dev)
-                qu = torch.zeros((H + 2 * Hk) * Dh, rq, dtype=torch.bfloat16, device=dev)
-                for i, (m_v, m_u, r_, row0, rows) in enumerate(((at.q_v_proj, at.q_u_proj, aq, 0, H * Dh), (at.k_v_proj, at.k_u_proj, ak, H * Dh, Hk * Dh),
-                                                                (at.v_v_proj, at.v_u_proj, av, (H + Hk) * Dh, Hk * Dh))):
-                    pv[i * rq:i * rq + r_] = m_v.weight.data
-                    qu[row0:row0 + rows, :r_] = m_u.weight.data
-                gemv([pv], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
-                gemv([qu], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
+                gemv("qkv_u", [w], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh), q4=gs)
             else:
-                gemv([at._packed_qkv_v], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
-                # q, k, v head expansion as one GEMV over the row-packed [q_u; k_u; v_u] (the three module
-                # weights become views of one buffer); RoPE and the cache append happen in the attention phase
-                qkv_u = _packed_rows([at.q_u_proj, at.k_u_proj, at.v_u_proj])
-                self._keep.append(qkv_u)
-                gemv([qkv_u], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
+                gemv("attn_rank_proj", [bw["qkv_v"]], 3 * rq, d, xin, _tb(self.P, L, l), norm=n1.weight, eps=n1.variance_epsilon)
+                # q, k, v head expansion as one GEMV over the row-packed [q_u; k_u; v_u]; RoPE and the cache append
+                # happen in the attention phase
+                gemv("qkv_u", [bw["qkv_u"]], (H + 2 * Hk) * Dh, rq, _tb(self.P, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh))
             if part != "mlp":
-                a = Phase()
-                a.type, a.H, a.Hk, a.Dh, a.S, a.nsplit = PH_ATTN, H, Hk, Dh, S, nsplit
-                a.fparam = 1.0 / math.sqrt(Dh)
-                a.cos, a.sin, a.rope_len = cos.data_ptr(), sin.data_ptr(), int(cos.shape[0])
-                a.k_cache, a.v_cache, a.sc_s, a.sc_h = kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1)
-                a.inp, a.out0 = _tb(self.QKV, L, l), _tb(self.PART, L, l)
-                ph.append(a)
-                m = Phase()
-                m.type, m.H, m.Dh, m.nsplit = PH_MERGE, H, Dh, nsplit
-                m.inp, m.out0 = _tb(self.PART, L, l), _tb(self.A, L, l)
-                ph.append(m)
+                attention(l, lc)
                 if q4:
                     w, gs = triple(at.o_v_proj)
-                    gemv([w], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l), q4=gs)
+                    gemv("o_v", [w], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l), q4=gs)
                     w, gs = triple(at.o_u_proj)
-                    gemv([w], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin, q4=gs)
+                    gemv("o_u", [w], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin, q4=gs)
                 else:
-                    w_ov, w_ou = at.o_v_proj.weight, at.o_u_proj.weight
-                    if padded[l]["o"]:
-                        w_ov, w_ou = pad_rows(w_ov, ro), pad_cols(w_ou, ro)
-                    gemv([w_ov], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
-                    gemv([w_ou], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
+                    gemv("o_v", [bw["o_v"]], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
+                    gemv("o_u", [bw["o_u"]], d, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin)
             if part == "attention":
                 pass
             elif q4:
                 w, gs = triple(mlp.gate_v_proj, mlp.up_v_proj)
-                gemv([w], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon, q4=gs)
+                gemv("mlp_rank_proj", [w], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon, q4=gs)
                 (wg, gs), (wu, gs2) = triple(mlp.gate_u_proj), triple(mlp.up_u_proj)
                 if gs != gs2:
                     raise ValueError(f"PersistentDecoder: gate_u / up_u of layer {l} use different int4 group sizes")
-                gemv([wg, wu], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2, epi=EP_SWIGLU, q4=gs)
+                gemv("swiglu", [wg, wu], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2, epi=EP_SWIGLU, q4=gs)
                 w, gs = triple(mlp.down_v_proj)
-                gemv([w], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l), q4=gs)
+                gemv("down_v", [w], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l), q4=gs)
                 w, gs = triple(mlp.down_u_proj)
-                gemv([w], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid, q4=gs)
+                gemv("down_u", [w], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid, q4=gs)
             else:
-                w_guv, w_gu, w_uu = mlp._packed_gu_v, mlp.gate_u_proj.weight, mlp.up_u_proj.weight
-                if padded[l]["gu"]:
-                    am = int(mlp.gate_v_proj.out_features)
-                    w_guv = torch.zeros(2 * rm, d, dtype=torch.bfloat16, device=dev)
-                    w_guv[:am] = mlp.gate_v_proj.weight.data
-                    w_guv[rm:rm + am] = mlp.up_v_proj.weight.data
-                    w_gu, w_uu = pad_cols(w_gu, rm), pad_cols(w_uu, rm)
-                w_dv, w_du = mlp.down_v_proj.weight, mlp.down_u_proj.weight
-                if padded[l]["d"]:
-                    w_dv, w_du = pad_rows(w_dv, rd), pad_cols(w_du, rd)
-                gemv([w_guv], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
-                gemv([w_gu, w_uu], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2, epi=EP_SWIGLU)
-                gemv([w_dv], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
-                gemv([w_du], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
+                gemv("mlp_rank_proj", [bw["gu_v"]], 2 * rm, d, xmid, _tb(self.PM, L, l), norm=n2.weight, eps=n2.variance_epsilon)
+                gemv("swiglu", [bw["gate_u"], bw["up_u"]], D, rm, _tb(self.PM, L, l), _tb(self.HB, L, l), nmat=2, epi=EP_SWIGLU)
+                gemv("down_v", [bw["down_v"]], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
+                gemv("down_u", [bw["down_u"]], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
             cache._layer_initialized[lc] = True
         if part == "model":
             fn = inner.norm
-            gemv([model.lm_head.weight], V, d, _tb(self.XA, L + 1, L), _tb(self.CAND, 1, 0), norm=fn.weight,
+            gemv("lm_head", [model.lm_head.weight], V, d, _tb(self.XA, L + 1, L), _tb(self.CAND, 1, 0), norm=fn.weight,
                  eps=fn.variance_epsilon, epi=EP_LOGITS, plain=self.logits)
             g = Phase()
             g.type = PH_ARGMAX
             g.inp = _tb(self.CAND, 1, 0)
             g.plain_out = self.token_log.data_ptr()
             ph.append(g)
+            names.append("argmax")
+        self._names = names
 
         self._finish(ph, dev)
+
+    def _composed_layers(self, layers, ranks, bf16_weights, gemv, attention, off_a, off_m) -> None:
+        """The eight-phase form of a bf16 layer.
+
+        RMSNorm is a scalar behind a product once its weight vector is folded into the matrix (W' = W diag(w)), and a
+        product with a hidden state that is itself ``x + U t`` splits as ``W' x + (W' U) t``.  So the two rank
+        projections of a layer leave the critical path: ``[gate_v; up_v]' x`` is taken (as unrounded fp32 sums) right
+        behind the q / k / v expansion, from the copy of x that phase has staged, and the o_u phase streams
+        ``[o_u; [gate_v; up_v]' o_u]`` — its first rows give the new hidden state, the others complete the sums, which the
+        SwiGLU phase scales by 1 / rms of that state while staging them; the same with down_u and the NEXT layer's
+        ``[q_v; k_v; v_v]'``, whose product with the mid-layer state rides behind the SwiGLU pair.  Per layer: ten
+        hand-offs become eight, the two moved products (25 MB each at the 7B shape) stream while the hand-off behind the
+        expansion and behind the pair is in flight, and the two composed blocks add 6 % to the layer's bytes.
+
+        Arithmetic: the hidden states take the same roundings as in the ten-phase form; the rank coefficients are formed
+        from the unrounded residual sum and rounded once (the ten-phase form rounds the hidden state, the normalised
+        state and its product with the norm weight first), and the composed blocks ``W' U`` are products in fp32 of the
+        stored factors, rounded to bf16 once.
+        """
+        dev = self.XA.device
+        H, Hk, Dh, d, L = self.H, self.Hk, self.Dh, self.d, self.L
+        D = int(layers[0].mlp.gate_u_proj.out_features)
+        Rq = max(r[0] for r in ranks)
+        Rm = max(r[2] for r in ranks)
+
+        def tagged64(n):
+            return torch.zeros(n, dtype=torch.int64, device=dev)
+
+        self.PRAW, self.G0, self.PMRAW, self.Q0 = tagged64(3 * Rq), tagged64(2 * Rm), tagged64(2 * Rm), tagged64(3 * Rq)
+        nq0 = max(L - 1, 1)
+
+        def folded(w, norm):
+            """W diag(norm) in fp32; as a bf16 matrix it is W itself when the norm weights are all one."""
+            nw = norm.weight.data.float()
+            wf = w.data.float() * nw[None, :]
+            return wf, (w if bool((nw == 1).all()) else wf.to(torch.bfloat16).contiguous())
+
+        bw = [bf16_weights(l) for l in range(L)]
+        fq = [folded(bw[l]["qkv_v"], layers[l].input_layernorm) for l in range(L)]
+        for l, layer in enumerate(layers):
+            rq, ro, rm, rd = ranks[l]
+            n1, n2 = layer.input_layernorm, layer.post_attention_layernorm
+            self.cache._ensure_layer_spec(l, h=Hk, dh=Dh)
+            xin, xmid, xout = _tb(self.XA, L + 1, l), _tb(self.XB, L, l), _tb(self.XA, L + 1, l + 1)
+            w = bw[l]
+            gu32, gu16 = folded(w["gu_v"], n2)
+            # [o_u; [gate_v; up_v]' o_u] and [down_u; [q_v; k_v; v_v]'(next layer) down_u]: one stream each
+            cat_o = torch.cat([w["o_u"].data, (gu32 @ w["o_u"].data.float()).to(torch.bfloat16)]).contiguous()
+            if l == 0:
+                gemv("attn_rank_proj", [fq[0][1]], 3 * rq, d, xin, None, epi=EP_F32, out1=_tb(self.PRAW, L, 0))
+            gemv("qkv_u", [w["qkv_u"]], (H + 2 * Hk) * Dh, rq, _tb(self.PRAW, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh),
+                 flags=PF_STAGE2, eps=n1.variance_epsilon, in2=xin, in2_len=d, in2_off=off_a)
+            gemv("mlp_rank_x", [gu16], 2 * rm, d, None, None, epi=EP_F32, flags=PF_NOWAIT, in_off=off_a, out1=_tb(self.G0, L, l))
+            attention(l, l)
+            gemv("o_v", [w["o_v"]], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
+            gemv("o_u+mlp_rank", [cat_o], d + 2 * rm, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin, flags=PF_SPLIT, rows0=d,
+                 aux2=_tb(self.G0, L, l), out1=_tb(self.PMRAW, L, l))
+            gemv("swiglu", [w["gate_u"], w["up_u"]], D, rm, _tb(self.PMRAW, L, l), _tb(self.HB, L, l), nmat=2, epi=EP_SWIGLU,
+                 flags=PF_STAGE2, eps=n2.variance_epsilon, in2=xmid, in2_len=d, in2_off=off_m)
+            if l + 1 < L:
+                rq_n = ranks[l + 1][0]
+                gemv("attn_rank_x", [fq[l + 1][1]], 3 * rq_n, d, None, None, epi=EP_F32, flags=PF_NOWAIT, in_off=off_m,
+                     out1=_tb(self.Q0, nq0, l))
+            gemv("down_v", [w["down_v"]], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
+            if l + 1 < L:
+                cat_d = torch.cat([w["down_u"].data, (fq[l + 1][0] @ w["down_u"].data.float()).to(torch.bfloat16)]).contiguous()
+                gemv("down_u+attn_rank", [cat_d], d + 3 * rq_n, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid, flags=PF_SPLIT,
+                     rows0=d, aux2=_tb(self.Q0, nq0, l), out1=_tb(self.PRAW, L, l + 1))
+            else:
+                gemv("down_u", [w["down_u"]], d, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid)
+            self.cache._layer_initialized[l] = True
+            fq[l] = None      # the fp32 copies are only needed while the blocks are composed
 
     def _finish(self, ph, dev) -> None:
         """Derived fields, host-side validation, upload of the phase list."""
@@ -379,16 +506,8 @@ class PersistentDecoder:
         self._host_steps += int(n)
         self.cache._seen_tokens += int(n)
 
-    PHASE_NAMES = ("embed", "attn_rank_proj", "qkv_u", "attn", "attn_merge", "o_v", "o_u", "mlp_rank_proj", "swiglu",
-                   "down_v", "down_u")
-
     def phase_names(self) -> list:
-        part = getattr(self, "part", "model")
-        if part == "attention":
-            return ["embed", *self.PHASE_NAMES[1:7]]
-        if part == "mlp":
-            return ["embed", *self.PHASE_NAMES[7:]]
-        return ["embed"] + [n for _ in range(self.L) for n in self.PHASE_NAMES[1:]] + ["lm_head", "argmax"]
+        return list(self._names)
 
     def trace_step(self, wg_stride: int = 32) -> torch.Tensor:
         """Run ONE step with per-phase time stamps; returns int64 [workgroups/stride, phases, 4] in
@@ -565,6 +684,8 @@ class DenseStepDecoder(PersistentDecoder):
         g.inp = _tb(self.CAND, 1, 0)
         g.plain_out = self.token_log.data_ptr()
         ph.append(g)
+        self.composed = False
+        self._names = ["embed"] + [n for _ in range(L) for n in self.PHASE_NAMES[1:]] + ["lm_head", "argmax"]
         self._finish(ph, dev)
 
 

@@ -306,6 +306,20 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
 #define FSVD_EP_SWIGLU 2  /* nmat = 2: out0[n] = silu(W[0][n].in[0:K]) * (W[1][n].in[K:2K]), rounding `mode`  */
                           /* (shared_in: both over in[0:K])                                                   */
 #define FSVD_EP_LOGITS 3  /* plain_out[n] = bf16(dot) and out0[wg] = (best value, best index) of the workgroup */
+#define FSVD_EP_F32 4     /* out1[n - rows0] = dot (+ aux2[n - rows0]) as fp32 in a 64-bit tagged word: a sum that a  */
+                          /* later phase completes or scales before it is rounded                                */
+
+/* GEMV phase flags.  They exist for the composed form of a low-rank layer, in which RMSNorm is applied as a scalar
+ * after the product (norm weights folded into the matrix): W.(x + U.t) = W.x + (W.U).t, so the product with the hidden
+ * state x can be taken in an earlier phase that has x staged anyway (as an FSVD_PF_NOWAIT phase behind the publication
+ * of that phase's own outputs, where its weight stream hides the hand-off), and the phase that applies U also applies
+ * the pre-multiplied W.U and emits the finished sum unrounded (FSVD_PF_SPLIT).  No counterpart in the reference, whose
+ * walk (utils/evaluator.py:39-82) launches one operator per projection. */
+#define FSVD_PF_NOWAIT 1  /* the input was staged by the previous phase of this workgroup (at in_off): no polling   */
+#define FSVD_PF_STAGE2 2  /* `in` holds fp32 sums (64-bit tagged words, nmat * K or 3 * K of them) and in2 the raw   */
+                          /* bf16 hidden state they were taken from: staged input = bf16(in * rsqrt(mean(in2^2) +  */
+                          /* fparam)) at 0, and in2 itself, unscaled, at in2_off for a following NOWAIT phase     */
+#define FSVD_PF_SPLIT 4   /* two row groups with their own epilogues and outputs, see rows0                       */
 
 typedef struct fsvd_tagbuf {
   void* ptr;              /* uint32 [len] (bf16 payload) or uint64 [len] (fp32 / candidate payload)           */
@@ -318,16 +332,32 @@ typedef struct fsvd_phase {
   int32_t N, K, nmat, mode;     /* rows per matrix, row length, matrices, SwiGLU rounding mode; the staged     */
                                 /* input has nmat * K elements.  EMBED: K = rows of the table (0: unchecked);  */
                                 /* a token outside [0, K) reads row 0 and sets state->err                      */
-  int32_t H, Hk, Dh, nsplit, rope_len, S;   /* on a GEMV, H > 0 marks the q | k | v head expansion: N = (H + 2*Hk) * Dh  */
+  int32_t H, Hk, Dh;            /* on a GEMV, H > 0 marks the q | k | v head expansion: N = (H + 2*Hk) * Dh    */
                                 /* rows in three groups that read in[0:K], in[K:2K], in[2K:3K]                 */
-  float fparam;                 /* GEMV with norm_w: RMSNorm eps; ATTN: softmax scale                          */
+  union { int32_t nsplit;       /* ATTN, MERGE: key splits per head                                            */
+          int32_t rows0; };     /* GEMV with FSVD_PF_SPLIT: rows [0, rows0) take `epilogue` into out0, rows    */
+                                /* [rows0, N) take FSVD_EP_F32 into out1 (+ aux2)                              */
+  union { int32_t rope_len;     /* ATTN: rows of cos / sin                                                     */
+          int32_t in_off; };    /* GEMV: element offset of this phase's input in the workgroup's staging area  */
+  union { int32_t S;            /* ATTN: cache rows                                                            */
+          int32_t in2_len; };   /* GEMV with FSVD_PF_STAGE2: elements of in2                                   */
+  float fparam;                 /* GEMV with norm_w or FSVD_PF_STAGE2: RMSNorm eps; ATTN: softmax scale        */
+  int32_t flags;                /* GEMV: FSVD_PF_* bits                                                        */
   const void* W[3];             /* nn.Linear-layout weights [N, K] (EMBED: table [V, N]); W[2] unused         */
   const void* norm_w;           /* RMSNorm weight over `in` or NULL                                            */
-  const void* cos; const void* sin;   /* [rope_len, Dh/2]                                                      */
-  void* k_cache; void* v_cache; /* batch row of the dense cache, [S, Hk, Dh] with strides sc_s, sc_h          */
-  int64_t sc_s, sc_h;
+  union {
+    struct { const void* cos; const void* sin;     /* ATTN: [rope_len, Dh/2]                                   */
+             void* k_cache; void* v_cache; };      /* ATTN: batch row of the dense cache, [S, Hk, Dh], strides sc_s, sc_h */
+    struct { fsvd_tagbuf aux2;                     /* GEMV: fp32 addend of the FSVD_EP_F32 rows (ptr NULL: none) */
+             fsvd_tagbuf out1; };                  /* GEMV: fp32 output of the FSVD_EP_F32 rows                */
+  };
+  union { int64_t sc_s;         /* ATTN: cache stride between tokens (elements)                                */
+          int32_t in2_off; };   /* GEMV with FSVD_PF_STAGE2: element offset at which in2 is staged             */
+  int64_t sc_h;                 /* ATTN: cache stride between heads                                            */
   void* plain_out;              /* EP_LOGITS: bf16 logits [N]; ARGMAX: int64 token log indexed by state->step */
-  fsvd_tagbuf in, aux0, aux1, out0;   /* aux0: residual of EP_RESID; aux1 reserved                            */
+  fsvd_tagbuf in, aux0;         /* aux0: residual of EP_RESID                                                  */
+  fsvd_tagbuf in2;              /* GEMV with FSVD_PF_STAGE2: the raw hidden state behind `in` (see the flag)   */
+  fsvd_tagbuf out0;
   /* GEMV over group-wise int4 weights (wbits == 4; 0 or 16 = bf16): W[m] is the packed matrix [N, K/2] bytes (two
    * columns per byte, even column in the low nibble, as PackedQuantLinear.qweight); qsz[m] is uint32 [N, ldg] with
    * the fp16 scale bits of a group in the low half and (zero point + 128) in the high half; a group is
@@ -373,8 +403,9 @@ int fsvd_decode_step_prepare(fsvd_phase* phases_host, int nphase, int workgroups
 /* The host-side check of fsvd_decode_step alone (no launch): 0, or a negative status with fsvd_last_error(). */
 int fsvd_decode_step_validate(const fsvd_phase* phases_host, int nphase, int workgroups);
 /* phases_dev: the list in device memory; phases_host: the same list in host memory (validated on every
- * call unless validate == 0; it also tells the launcher whether the list holds int4 phases, so it may be NULL
- * only for lists without them — the kernel build without int4 code raises state->err on such a phase);
+ * call unless validate == 0; it also tells the launcher which build of the kernel the list needs — plain bf16, with
+ * the int4 code, or with the code of the composed form — so it may be NULL only for plain bf16 lists: a build that
+ * meets a phase it was not compiled for raises state->err);
  * state: device.  Launch is asynchronous on `stream`. */
 int fsvd_decode_step(const fsvd_phase* phases_dev, const fsvd_phase* phases_host, int nphase,
                      fsvd_step_state* state, int validate, void* stream);

@@ -45,7 +45,8 @@ def _tie_aware(g, o, ref_logits_row, what):
     return False
 
 
-def test_small_model_teacher_forced_against_oracle():
+@pytest.mark.parametrize("composed", [False, True], ids=["ten_phase", "composed"])
+def test_small_model_teacher_forced_against_oracle(composed):
     from flashsvd_amd.step import PersistentDecoder
     mw, prompt = _small()
     n_new = 12
@@ -53,7 +54,8 @@ def test_small_model_teacher_forced_against_oracle():
     ref_tok, ref_hid, _, ref_logits = O.greedy_decode(mw, prompt, n_new, "dense", return_logits=True)
     cache, tok0 = _prefill(model, prompt, n_new + 4)
     assert int(tok0) == int(ref_tok[0, 0])
-    dec = PersistentDecoder(model, cache)
+    dec = PersistentDecoder(model, cache, composed=composed)
+    assert dec.composed == composed
     Lp = prompt.shape[1]
     n_equal = 0
     for s in range(1, n_new):
@@ -69,7 +71,8 @@ def test_small_model_teacher_forced_against_oracle():
     assert n_equal >= n_new - 3
 
 
-def test_small_model_free_running_matches_kernel_path():
+@pytest.mark.parametrize("composed", [False, True], ids=["ten_phase", "composed"])
+def test_small_model_free_running_matches_kernel_path(composed):
     """16 launches queued without host synchronisation: same greedy tokens and cache rows as the
     per-kernel decode path (both GPU paths, same rounding points; fp32 sums are split differently, so a
     token may differ where the per-kernel path itself holds the two candidates within bf16 resolution —
@@ -89,7 +92,7 @@ def test_small_model_free_running_matches_kernel_path():
         logits_k.append(dec_k.logits[0, -1].float().cpu())
     toks_k = torch.cat(toks_k, 1).cpu()
     cache_p, tok0p = _prefill(model, prompt, n_new + 4)
-    dec = PersistentDecoder(model, cache_p)
+    dec = PersistentDecoder(model, cache_p, composed=composed)
     dec.set_state(tok0p, Lp)
     dec.step(n_new - 1)
     toks_p = torch.cat([tok0p.cpu(), dec.tokens().cpu()[None, :]], 1)
@@ -110,7 +113,8 @@ def test_small_model_free_running_matches_kernel_path():
                           abs_tol=3 * bounds(dec_k.logits.float())["abs_tol"])
 
 
-def test_7b_width_two_layers_teacher_forced_tie_aware():
+@pytest.mark.parametrize("composed", [False, True], ids=["ten_phase", "composed"])
+def test_7b_width_two_layers_teacher_forced_tie_aware(composed):
     from flashsvd_amd.step import PersistentDecoder
     mw = O.make_model(d=4096, n_heads=32, n_kv_heads=32, head_dim=128, ffn=11008, attn_rank=1024, mlp_rank=1536,
                       n_layers=2, vocab=32000, dtype=BF16, seed=0)
@@ -119,7 +123,7 @@ def test_7b_width_two_layers_teacher_forced_tie_aware():
     model = model_from_oracle(mw)
     ref_tok, ref_hid, _, ref_logits = O.greedy_decode(mw, prompt, n_new, "dense", return_logits=True)
     cache, _ = _prefill(model, prompt, n_new + 4)
-    dec = PersistentDecoder(model, cache)
+    dec = PersistentDecoder(model, cache, composed=composed)
     n_equal = 0
     for s in range(1, n_new):
         dec.set_state(ref_tok[:, s - 1], prompt.shape[1] + s - 1)      # teacher forcing: the oracle's token
@@ -345,6 +349,40 @@ def test_phase_list_validation():
     dec.host_phases[2].inp.use = saved_use
     rc = lib.fsvd_decode_step(None, ctypes.addressof(dec.host_phases), dec.nph, dec.state.data_ptr(), 1, stream)
     assert rc == -4
+    # the composed form: phases without a hand-off, two-vector staging, two row groups
+    cache2, _ = _prefill(model, prompt, 8)
+    dc = PersistentDecoder(model, cache2, composed=True)
+    names = dc.phase_names()
+    hp, n = dc.host_phases, dc.nph
+
+    def verdict():
+        return lib.fsvd_decode_step_validate(ctypes.addressof(hp), n, dc.nwg), lib.fsvd_last_error()
+
+    assert verdict()[0] == 0
+    i = names.index("mlp_rank_x")
+    saved = hp[i].in_off
+    hp[i].in_off = saved + 128                 # not where the previous phase staged the hidden state
+    rc, msg = verdict()
+    assert rc == -1 and b"previous phase staged" in msg
+    hp[i].in_off = saved
+    j = names.index("o_u+mlp_rank")
+    saved = hp[j].rows0
+    hp[j].rows0 = hp[j].N                      # an empty second row group
+    rc, msg = verdict()
+    assert rc == -1 and b"two non-empty groups" in msg
+    hp[j].rows0 = saved
+    k = names.index("swiglu")
+    saved = hp[k].in2_off
+    hp[k].in2_off = 8                          # the hidden state staged over the coefficients
+    rc, msg = verdict()
+    assert rc == -1 and b"second staged vector" in msg
+    hp[k].in2_off = saved
+    saved = hp[j].aux2.use
+    hp[j].aux2.use = saved + 1                 # addend expected with a tag nobody writes
+    rc, msg = verdict()
+    assert rc == -1 and b"addend tag schedule" in msg
+    hp[j].aux2.use = saved
+    assert verdict()[0] == 0
 
 
 def test_decode_driver_picks_the_persistent_engine(monkeypatch):
@@ -428,6 +466,14 @@ def test_checkpoint_round_trip_decodes_identically(tmp_path):
         dec.step(n_new - 1)
         toks.append([int(tok0)] + dec.tokens().cpu().tolist())
     assert toks[0] == toks[1]
+    # and the loaded weights are the oracle's: its greedy tokens for the same model, tie-aware as in the tests above
+    ref_tok, _, _, ref_logits = O.greedy_decode(mw, prompt, n_new, "dense", return_logits=True)
+    for s_ in range(n_new):
+        if not _tie_aware(toks[1][s_], int(ref_tok[0, s_]), ref_logits[0, s_], f"loaded model, step {s_}"):
+            break                      # past a near-tie the two runs follow different prefixes
+    else:
+        s_ = n_new
+    assert s_ >= 4, f"loaded model {toks[1]} vs oracle {ref_tok[0].tolist()}"
 
 
 def test_dense_step_decoder_matches_the_oracle():
