@@ -477,12 +477,16 @@ int fsvd_mlp_dual_split(const void* PUp, int64_t sPUp_t, const void* PGate, int6
   return launch_xw(m.du.a, dtype, m.du.tx, m.du.bt, counters, partials, st);
 }
 
+size_t fsvd_attn_decode_rankkv_scores_bytes(int B, int H, int S, int shared_by_heads) {
+  return rank_decode_scores_floats(B, H, S, shared_by_heads ? 0 : 1) * sizeof(float);
+}
+
 int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h, const void* pk_cache, int64_t spk_b, int64_t spk_s, int64_t spk_h,
                             const void* pv_cache, int64_t spv_b, int64_t spv_s, int64_t spv_h, const void* k_u, int64_t ldku, const void* v_u,
                             int64_t ldvu, const void* bv, const void* cos, const void* sin, int rope_len, int rotate_q,
                             const int32_t* cache_seqlens, int seqlen_add, float* ws_m, float* ws_l, float* ws_acc, void* out,
                             int64_t so_b, int64_t so_h, int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit,
-                            float scale, void* stream) {
+                            float scale, float* scores, size_t scores_bytes, void* stream) {
   const char* fn = "fsvd_attn_decode_rankkv";
   FSVD_REQUIRE_PTR(q, fn); FSVD_REQUIRE_PTR(pk_cache, fn); FSVD_REQUIRE_PTR(pv_cache, fn); FSVD_REQUIRE_PTR(k_u, fn);
   FSVD_REQUIRE_PTR(v_u, fn); FSVD_REQUIRE_PTR(cache_seqlens, fn); FSVD_REQUIRE_PTR(ws_m, fn); FSVD_REQUIRE_PTR(ws_l, fn);
@@ -493,6 +497,15 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h, const voi
   RankDecodeArgs a{cu16(q), sq_b, sq_h, cu16(pk_cache), spk_b, spk_s, spk_h, cu16(pv_cache), spv_b, spv_s, spv_h, cu16(k_u), ldku, cu16(v_u), ldvu,
                    cu16(bv), cu16(cos), cu16(sin), rope_len, rotate_q, cache_seqlens, seqlen_add, ws_m, ws_l, ws_acc, u16(out),
                    so_b, so_h, B, H, Hk, Dh, S, Rk, Rv, nsplit, scale > 0.f ? scale : 1.0f / sqrtf((float)Dh)};
+  if (scores != nullptr) {
+    const size_t need = rank_decode_scores_floats(B, H, S, spv_h) * sizeof(float);
+    if (need != 0 && scores_bytes < need) {
+      set_last_error("%s: the score buffer holds %zu bytes, this shape needs %zu (fsvd_attn_decode_rankkv_scores_bytes)", fn, scores_bytes, need);
+      return kErrWorkspace;
+    }
+    if ((reinterpret_cast<uintptr_t>(scores) & 15) != 0) { set_last_error("%s: the score buffer must be 16-byte aligned", fn); return kErrBadAlign; }
+    a.scores = scores;
+  }
   return launch_rank_decode(a, static_cast<hipStream_t>(stream));
 }
 

@@ -106,8 +106,9 @@ struct RankDecodeArgs {
   uint16_t* out; int64_t so_b, so_h;                // [B,H,Dh]
   int B, H, Hk, Dh, S, Rk, Rv, nsplit;
   float scale;
-  float* scores = nullptr; int64_t score_ld = 0;    // [B,H,score_ld] fp32 in the registered scratch (set by the launcher for long caches)
+  float* scores = nullptr; int64_t score_ld = 0;    // the caller's score buffer [B,H,ceil64(S)] fp32 or null; score_ld is set by the launcher
 };
+size_t rank_decode_scores_floats(int B, int H, int S, int64_t spv_h);
 int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st);
 int launch_rankkv_append(const uint16_t* pk, int64_t ldpk, const uint16_t* pv, int64_t ldpv, uint16_t* pkc, int64_t spk_b, int64_t spk_s,
                          uint16_t* pvc, int64_t spv_b, int64_t spv_s, const int32_t* positions, int B, int S, int Rk, int Rv, hipStream_t st);

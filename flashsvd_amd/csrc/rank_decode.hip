@@ -915,6 +915,13 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_merge_kernel(RankDecod
   }
 }
 
+// floats of the score buffer with which a call of this shape runs as three launches; 0: the shape keeps the one-kernel form
+size_t rank_decode_scores_floats(int B, int H, int S, int64_t spv_h) {
+  if (B <= 0 || H <= 0 || S < 256 || spv_h != 0) return 0;
+  const size_t n = (size_t)B * H * (((size_t)S + 63) / 64 * 64);
+  return n >= ((size_t)1 << 17) ? n : 0;
+}
+
 int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   const char* fn = "fsvd_attn_decode_rankkv";
   if (a.B <= 0 || a.H <= 0 || a.Hk <= 0 || a.H % a.Hk != 0 || a.S <= 0 || a.nsplit <= 0) {
@@ -939,15 +946,13 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   }
   const int rep = a.H / a.Hk;
   dim3 block(kRdThreads);
-  // caches shared by the heads from 2^17 (head, key) pairs on, with registered scratch: scores -> softmax -> rank-space accumulation per head tile,
-  // as three launches; the scores of the call live in the scratch, [B,H,score_ld] fp32
-  const SplitWorkspace sw = split_workspace();
+  // caches shared by the heads from 2^17 (head, key) pairs on, when the caller brings a buffer for the scores of the call
+  // ([B,H,score_ld] fp32): scores -> softmax -> rank-space accumulation per head tile, as three launches.  The form
+  // depends on the shape and on that argument alone, never on process state.
   const int64_t score_ld = ((int64_t)a.S + 63) / 64 * 64;
-  const size_t score_floats = (size_t)a.B * a.H * score_ld;
-  const bool three = a.spv_h == 0 && a.S >= 256 && score_floats >= ((size_t)1 << 17) && sw.part != nullptr &&
-                     sw.part_floats >= score_floats;
+  const bool three = a.scores != nullptr && rank_decode_scores_floats(a.B, a.H, a.S, a.spv_h) != 0;
   RankDecodeArgs a3 = a;
-  a3.scores = three ? sw.part : nullptr;
+  a3.scores = three ? a.scores : nullptr;
   a3.score_ld = score_ld;
   // key sub-tiles per pass: long splits amortise every k_u fragment over more keys (any value is correct for any
   // length; short splits would only rebuild clamped keys)

@@ -46,20 +46,19 @@ def _rows(t: torch.Tensor, name: str) -> torch.Tensor:
 
 _SPLIT_WS: dict = {}                      # device index -> scratch tensor registered with the library (kept alive here)
 _SPLIT_WS_BYTES = (64 << 20) + (64 << 10)
-
-
-_SPLIT_WS_OLD: list = []                  # replaced scratch buffers: captured graphs may still hold their addresses
+_SPLIT_WS_OLD: dict = {}                  # device index -> replaced buffers: graphs captured earlier may hold their addresses
 _SPLIT_WS_MAX = 1 << 30
 
 
 def ensure_split_workspace(device: torch.device, min_bytes: int = 0) -> bool:
-    """Register, once per device, the scratch the library's K-split projections (3..127 rows) and its rank-space decode
-    attention (scores of a call) work in.  The library allocates nothing itself; this hands it 64 MiB of torch memory, or
-    ``min_bytes`` (up to 1 GiB) when a caller needs more: a larger buffer then replaces the registered one, and the old one
-    is kept alive because graphs captured earlier hold its address.  ``FLASHSVD_AMD_SPLITK=0`` keeps the library without
-    scratch; so does a first call made under stream capture (an allocation there would belong to the graph's pool), and
-    a registered buffer is never replaced under capture.  Launches that use the scratch must be ordered on one stream per
-    device.  Returns whether a buffer of at least ``min_bytes`` is registered."""
+    """Register, once per device, the scratch the library's K-split projections (3..127 rows) work in.  The library
+    allocates nothing itself; this hands it 64 MiB of torch memory, or ``min_bytes`` rounded up to a power of two (up to
+    1 GiB) when a caller needs more: a larger buffer then replaces the registered one (a doubling each time at least, so
+    a growing demand costs a logarithmic number of replacements), and the old one is kept alive until
+    ``release_split_workspace`` because graphs captured earlier hold its address.  ``FLASHSVD_AMD_SPLITK=0`` keeps the
+    library without scratch; so does a first call made under stream capture (an allocation there would belong to the
+    graph's pool), and a registered buffer is never replaced under capture.  Launches that use the scratch must be
+    ordered on one stream per device.  Returns whether a buffer of at least ``min_bytes`` is registered."""
     idx = device.index if device.index is not None else torch.cuda.current_device()
     need = max(int(min_bytes), _SPLIT_WS_BYTES)
     have = _SPLIT_WS.get(idx)
@@ -67,20 +66,24 @@ def ensure_split_workspace(device: torch.device, min_bytes: int = 0) -> bool:
         return True
     if os.environ.get("FLASHSVD_AMD_SPLITK", "1") == "0" or torch.cuda.is_current_stream_capturing() or need > _SPLIT_WS_MAX:
         return have is not None and min_bytes <= 0
+    if need > _SPLIT_WS_BYTES:
+        need = min(_SPLIT_WS_MAX, 1 << (need - 1).bit_length())
     with torch.cuda.device(idx):
         ws = torch.empty(need, dtype=torch.uint8, device=f"cuda:{idx}")
         rc = _lib.load().fsvd_set_workspace(ws.data_ptr(), ws.numel(), _stream())
         _lib.check("fsvd_set_workspace", rc)
         torch.cuda.current_stream().synchronize()      # cleared before any other stream can use it
     if have is not None:
-        _SPLIT_WS_OLD.append(have)
+        _SPLIT_WS_OLD.setdefault(idx, []).append(have)
     _SPLIT_WS[idx] = ws
     return True
 
 
 def release_split_workspace(device: Optional[torch.device] = None) -> None:
-    """Unregister (and free) the scratch of ``device``; the library runs without scratch until it is registered again."""
+    """Unregister (and free) the scratch of ``device`` and the buffers it replaced; the library runs without scratch
+    until it is registered again.  Graphs captured while a buffer was registered must not be replayed afterwards."""
     idx = torch.cuda.current_device() if device is None or device.index is None else device.index
+    _SPLIT_WS_OLD.pop(idx, None)
     if _SPLIT_WS.pop(idx, None) is not None:
         with torch.cuda.device(idx):
             torch.cuda.synchronize()

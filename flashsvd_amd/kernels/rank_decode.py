@@ -53,6 +53,11 @@ def _as_linear_layout(V: torch.Tensor) -> torch.Tensor:
     return out
 
 
+# test hooks: force the one-kernel form for every shape; a list that receives the score buffer of each call (or None)
+_FORCE_ONE_KERNEL = False
+_KEEP_SCORES: Optional[list] = None
+
+
 def rank_decode(q: torch.Tensor, pk_cache: torch.Tensor, pv_cache: torch.Tensor, k_u: torch.Tensor, v_u: torch.Tensor,
                 cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], seqlens: torch.Tensor, *, num_kv_heads: int,
                 seqlen_add: int = 0, rotate_q: bool = False, bv: Optional[torch.Tensor] = None, nsplit: Optional[int] = None,
@@ -108,17 +113,21 @@ def _rank_decode_impl(q, pk_cache, pv_cache, k_u, v_u, cos, sin, seqlens, num_kv
     if out is None:
         out = torch.empty(B, H, Dh, device=q.device, dtype=q.dtype)
     rope_len = 0 if cos is None else int(cos.shape[0])
-    if B * S * H >= (1 << 16):
-        # 4096 keys of 32 heads and more: the library keeps the scores of a call in the registered scratch and accumulates per head group
-        from ..hip_ops import ensure_split_workspace
-        ensure_split_workspace(q.device, (64 << 10) + 4 * B * H * ((S + 63) // 64 * 64))
     lib = _lib.load()
+    # long caches shared by the heads: the library runs score / softmax / accumulation launches when the call brings a
+    # buffer for its scores; the size query depends on the shape alone, so a captured graph and an eager call of the
+    # same shape take the same form, and the buffer is the call's own (nothing shared between streams)
+    need = 0 if _FORCE_ONE_KERNEL else int(lib.fsvd_attn_decode_rankkv_scores_bytes(B, H, S, 1 if spv[2] == 0 else 0))
+    scores = torch.empty(need // 4, device=q.device, dtype=torch.float32) if need else None
+    if _KEEP_SCORES is not None:
+        _KEEP_SCORES.append(scores)
     rc = lib.fsvd_attn_decode_rankkv(
         q.data_ptr(), q.stride(0), q.stride(1), pk_cache.data_ptr(), *spk, pv_cache.data_ptr(), *spv,
         k_u.data_ptr(), k_u.stride(0), v_u.data_ptr(), v_u.stride(0), None if bv is None else bv.data_ptr(),
         None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rope_len, int(bool(rotate_q)),
         seqlens.data_ptr(), int(seqlen_add), M.data_ptr(), L.data_ptr(), Acc.data_ptr(), out.data_ptr(), out.stride(0),
-        out.stride(1), B, H, Hk, Dh, S, Rk, Rv, int(nsplit), float(softmax_scale) if softmax_scale else 0.0, stream())
+        out.stride(1), B, H, Hk, Dh, S, Rk, Rv, int(nsplit), float(softmax_scale) if softmax_scale else 0.0,
+        None if scores is None else scores.data_ptr(), need, stream())
     check("fsvd_attn_decode_rankkv", rc)
     return out
 

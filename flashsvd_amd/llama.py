@@ -722,7 +722,32 @@ def patch_hf_llama_decoder_layer() -> bool:
     except Exception:
         return False
     orig = LlamaDecoderLayer.forward
-    returns_tensor = orig.__annotations__.get("return") in (torch.Tensor, "torch.Tensor")
+    # Whether the installed transformers returns the hidden state itself or a 1-tuple: releases that return a tuple build
+    # it as `outputs = (hidden_states,)` in the layer's forward; the return annotation is the fallback where the source
+    # cannot be read.
+    try:
+        import inspect
+        returns_tensor = "outputs = (hidden_states,)" not in inspect.getsource(orig)
+    except (OSError, TypeError):
+        returns_tensor = orig.__annotations__.get("return") in (torch.Tensor, "torch.Tensor")
+    _cache_kw = {}
+
+    def cache_kwarg(attn_mod) -> str:
+        """The name under which this attention class takes the cache (`past_key_values` in transformers 4.56+ / 5.x,
+        `past_key_value` before): passing it under the other name would drop it into **kwargs unnoticed."""
+        cls = type(attn_mod)
+        if cls not in _cache_kw:
+            import inspect
+            names = inspect.signature(cls.forward).parameters
+            if "past_key_values" in names:
+                _cache_kw[cls] = "past_key_values"
+            elif "past_key_value" in names:
+                _cache_kw[cls] = "past_key_value"
+            elif any(p.kind is inspect.Parameter.VAR_KEYWORD for p in names.values()):
+                _cache_kw[cls] = "past_key_values"       # an open signature: the spelling the installed layer itself uses
+            else:
+                raise TypeError(f"{cls.__name__}.forward takes neither past_key_values nor past_key_value")
+        return _cache_kw[cls]
 
     def forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
                 position_embeddings=None, **kwargs):
@@ -743,12 +768,17 @@ def patch_hf_llama_decoder_layer() -> bool:
         else:
             # attention half as the unmodified layer runs it (any attention module), fused tail
             h = self.input_layernorm(hidden_states)
-            h = self.self_attn(hidden_states=h, attention_mask=attention_mask, position_ids=position_ids,
-                               past_key_values=past_key_values, use_cache=use_cache, position_embeddings=position_embeddings, **kwargs)
+            h = self.self_attn(hidden_states=h, attention_mask=attention_mask, position_ids=position_ids, use_cache=use_cache,
+                               position_embeddings=position_embeddings, **{cache_kwarg(self.self_attn): past_key_values}, **kwargs)
             h = h[0] if isinstance(h, (tuple, list)) else h
             x2 = hidden_states + h
             shape = x2.shape
-            out = decoder_layer_tail(self, x2.reshape(-1, shape[-1]) if x2.dim() == 3 and shape[1] == 1 else x2).reshape(shape)
+            if x2.dim() == 3 and shape[1] == 1:
+                out = decoder_layer_tail(self, x2.reshape(-1, shape[-1])).reshape(shape)
+            else:
+                # prompt rows: no graph (one would be captured and kept per prompt shape and layer), as decoder_layer_forward
+                n2 = self.post_attention_layernorm
+                out = self.mlp.run(x2, norm_weight=n2.weight, eps=n2.variance_epsilon, residual=x2)
         return out if returns_tensor else (out,)
 
     LlamaDecoderLayer.forward = forward

@@ -208,10 +208,12 @@ int fsvd_mlp_dual_split(const void* PUp, int64_t sPUp_t, const void* PGate, int6
  * buffers M, L [B,H,nsplit] and Acc [B,H,nsplit,Rv] (fp32), n_keys = cache_seqlens[b] + seqlen_add.
  * spk_h / spv_h are the kv-head strides of head-wise coefficient caches [B,S,Hk,R] (0 when shared).
  * bf16 only; head_dim 128; ranks multiples of 8, Rv <= 2048.
- * With scratch registered (fsvd_set_workspace) of at least B*H*ceil64(S) floats behind its 64 KiB counter block, shared
- * caches (spv_h == 0) with S >= 256 and B*H*ceil64(S) >= 2^17 run as score, softmax and accumulation launches that keep the
- * scores of the call in that scratch (same results up to the order of fp32 sums); calls that use it must be ordered on
- * one stream, like the K-split projections. */
+ * Long caches shared by the heads (spv_h == 0, S >= 256, B*H*ceil64(S) >= 2^17) can run as score, softmax and
+ * accumulation launches (same results up to the order of fp32 sums) when the caller passes `scores`, a buffer of
+ * fsvd_attn_decode_rankkv_scores_bytes(B, H, S, 1) bytes that holds the scores of the call; with scores == NULL, or for a
+ * shape for which that size is 0, the call is one kernel + merge.  Which form runs therefore depends on the arguments
+ * alone; the buffer belongs to the call, so calls on different streams need different buffers. */
+size_t fsvd_attn_decode_rankkv_scores_bytes(int B, int H, int S, int shared_by_heads);
 int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,
                             const void* pk_cache, int64_t spk_b, int64_t spk_s, int64_t spk_h,
                             const void* pv_cache, int64_t spv_b, int64_t spv_s, int64_t spv_h,
@@ -220,7 +222,8 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,
                             const int32_t* cache_seqlens, int seqlen_add,
                             float* ws_m, float* ws_l, float* ws_acc,
                             void* out, int64_t so_b, int64_t so_h,
-                            int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit, float scale, void* stream);
+                            int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit, float scale,
+                            float* scores, size_t scores_bytes, void* stream);
 
 /* One decoded token per batch row into a rank-space cache: pk_cache[b, positions[b], :] = pk[b, :] and the same for pv
  * (FlashSVDLegacySparseKVCache.update with one position per row, runtime/cache/attn_legacy_sparse_kv.py:113-169: two

@@ -63,10 +63,9 @@ LONG_CASES = [  # B, H, Hk, S, Rk, Rv, nsplit: shared caches of 2^17 (head, key)
 
 @pytest.mark.parametrize("B,H,Hk,S,Rk,Rv,nsplit", LONG_CASES)
 def test_long_cache_three_launch_form(RD, monkeypatch, B, H, Hk, S, Rk, Rv, nsplit):
-    """Scores -> softmax -> rank-space accumulation per head tile (long caches shared by the heads, scratch registered)
-    against the one-kernel form on the same inputs (same arithmetic up to the order of fp32 sums: one bf16 ulp) and against
-    the oracle on sampled batch rows."""
-    from flashsvd_amd import hip_ops
+    """Scores -> softmax -> rank-space accumulation per head tile (long caches shared by the heads, the call brings a score
+    buffer) against the one-kernel form on the same inputs (same arithmetic up to the order of fp32 sums: one bf16 ulp) and
+    against the oracle on sampled batch rows."""
     Dh = 128
     cos, sin = O.rope_tables(S, Dh, dtype=BF16)
     q = rand_bf16(B, H, Dh, seed=11)
@@ -75,20 +74,20 @@ def test_long_cache_three_launch_form(RD, monkeypatch, B, H, Hk, S, Rk, Rv, nspl
     lens = torch.tensor([max(0, S - 5 - (S // (B + 1)) * b) for b in range(B)], dtype=torch.int32)
     lens[-1] = 0 if B > 4 else lens[-1]                 # an empty batch row in the widest case
     args = (q.cuda(), Pk.cuda(), Pv.cuda(), _lin_layout(Vk).cuda(), _lin_layout(Vv).cuda(), cos.cuda(), sin.cuda(), lens.cuda())
-    # one-kernel form: no scratch registered
-    monkeypatch.setenv("FLASHSVD_AMD_SPLITK", "0")
-    hip_ops.release_split_workspace(torch.device("cuda", torch.cuda.current_device()))
+    # one-kernel form: the call brings no score buffer
+    monkeypatch.setattr(RD, "_FORCE_ONE_KERNEL", True)
     one = RD.rank_decode(*args, num_kv_heads=Hk, nsplit=nsplit).float().cpu()
-    monkeypatch.delenv("FLASHSVD_AMD_SPLITK")
-    hip_ops.release_split_workspace(torch.device("cuda", torch.cuda.current_device()))
+    monkeypatch.setattr(RD, "_FORCE_ONE_KERNEL", False)
+    kept = []
+    monkeypatch.setattr(RD, "_KEEP_SCORES", kept)
     three = RD.rank_decode(*args, num_kv_heads=Hk, nsplit=nsplit)
     torch.cuda.synchronize()
-    # the scratch now holds the softmax weights of the call, [B,H,ld] words behind the 64 KiB counter block, per 8 keys four
-    # words of bf16 pairs hi(p) and four of lo(p) = bf16(p - hi): the largest weight of a non-empty row is exp(0) in at
-    # least one split -- which proves the form that ran
-    ws = hip_ops._SPLIT_WS[torch.cuda.current_device()]
+    # the call's score buffer now holds its softmax weights, [B,H,ld] words, per 8 keys four words of bf16 pairs hi(p) and
+    # four of lo(p) = bf16(p - hi): the largest weight of a non-empty row is exp(0) in at least one split -- which proves
+    # the form that ran
+    assert len(kept) == 1 and kept[0] is not None
     ld = (S + 63) // 64 * 64
-    w = ws[64 * 1024:64 * 1024 + B * H * ld * 4].view(torch.int32).view(B, H, ld // 8, 2, 4)[0].cpu()
+    w = kept[0][:B * H * ld].view(torch.int32).view(B, H, ld // 8, 2, 4)[0].cpu()
     n0 = int(lens[0])
     def pairs(x):                                       # [H, groups, 4] words -> [H, groups * 8] values
         lo16 = ((x & 0xffff) << 16).view(torch.float32)
@@ -110,14 +109,13 @@ def test_long_cache_three_launch_form(RD, monkeypatch, B, H, Hk, S, Rk, Rv, nspl
         assert_close_bf16(three[b:b + 1], ref, f"three-launch form, b={b} n={n}")
 
 
-def test_scratch_grows_to_the_capacity_of_a_long_cache(RD):
-    """The scores of a call are indexed by cache position: a cache with room for 600 000 tokens needs 77 MB of scratch
-    whatever its fill; the wrapper registers a larger buffer (the old one stays alive for graphs that hold its address)."""
+def test_score_buffer_follows_the_capacity_of_a_long_cache(RD, monkeypatch):
+    """The scores of a call are indexed by cache position: a cache with room for 600 000 tokens takes a 77 MB score buffer
+    whatever its fill.  The buffer belongs to the call; nothing registered with the library is involved."""
     from flashsvd_amd import hip_ops
     B, H, Hk, S, R, Dh, n = 1, 32, 32, 600_000, 64, 128, 3000
     dev = torch.device("cuda", torch.cuda.current_device())
-    hip_ops.ensure_split_workspace(dev)
-    before = hip_ops._SPLIT_WS[dev.index]
+    hip_ops.release_split_workspace(dev)
     cos, sin = O.rope_tables(n, Dh, dtype=BF16)
     q = rand_bf16(B, H, Dh, seed=21)
     Pk, Pv = rand_bf16(B, n, R, seed=22), rand_bf16(B, n, R, seed=23)
@@ -126,16 +124,52 @@ def test_scratch_grows_to_the_capacity_of_a_long_cache(RD):
     pvc = torch.zeros(B, S, R, dtype=BF16, device="cuda")
     pkc[:, :n], pvc[:, :n] = Pk.cuda(), Pv.cuda()
     lens = torch.tensor([n], dtype=torch.int32, device="cuda")
+    kept = []
+    monkeypatch.setattr(RD, "_KEEP_SCORES", kept)
     out = RD.rank_decode(q.cuda(), pkc, pvc, _lin_layout(Vk).cuda(), _lin_layout(Vv).cuda(), cos.cuda(), sin.cuda(), lens,
                          num_kv_heads=Hk, nsplit=4)
-    after = hip_ops._SPLIT_WS[dev.index]
-    need = (64 << 10) + 4 * B * H * ((S + 63) // 64 * 64)
-    assert after.numel() >= need > before.numel() and any(t is before for t in hip_ops._SPLIT_WS_OLD)
+    assert len(kept) == 1 and kept[0].numel() == B * H * ((S + 63) // 64 * 64)
+    assert dev.index not in hip_ops._SPLIT_WS
     ref = O.rank_decode_attn(q, Pk, Pv, Vk, Vv, cos, sin)
     assert_close_bf16(out, ref, "long-capacity cache")
-    # the weights of the call sit in the new buffer (row 0: head 0): the three-launch form ran
-    w = after[64 * 1024:64 * 1024 + 64 * 4].view(torch.int32).cpu()
-    assert int(w.abs().max()) != 0
+    # the weights of the call sit in its buffer (row 0: head 0): the three-launch form ran
+    assert int(kept[0][:64].view(torch.int32).abs().max()) != 0
+
+
+def test_graph_and_eager_take_the_same_form(RD, monkeypatch):
+    """Which form runs depends on the shape alone: a call captured into a HIP graph and the same call made eagerly give
+    the same bits, replay after replay, and a second stream with its own call does not disturb them."""
+    B, H, Hk, S, R, Dh = 4, 32, 32, 2048, 256, 128
+    cos, sin = O.rope_tables(S, Dh, dtype=BF16)
+    q = rand_bf16(B, H, Dh, seed=31).cuda()
+    Pk, Pv = rand_bf16(B, S, R, seed=32).cuda(), rand_bf16(B, S, R, seed=33).cuda()
+    Vk, Vv = rand_bf16(Hk, R, Dh, std=R ** -0.5, seed=34), rand_bf16(Hk, R, Dh, std=R ** -0.5, seed=35)
+    ku, vu = _lin_layout(Vk).cuda(), _lin_layout(Vv).cuda()
+    lens = torch.tensor([S - 3, S // 2, 700, 64], dtype=torch.int32, device="cuda")
+    cosg, sing = cos.cuda(), sin.cuda()
+    kept = []
+    monkeypatch.setattr(RD, "_KEEP_SCORES", kept)
+    eager = RD.rank_decode(q, Pk, Pv, ku, vu, cosg, sing, lens, num_kv_heads=Hk, nsplit=4).clone()
+    assert kept[-1] is not None                       # this shape takes the three-launch form
+    out = torch.empty_like(eager)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            RD.rank_decode(q, Pk, Pv, ku, vu, cosg, sing, lens, num_kv_heads=Hk, nsplit=4, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        RD.rank_decode(q, Pk, Pv, ku, vu, cosg, sing, lens, num_kv_heads=Hk, nsplit=4, out=out)
+    assert kept[-1] is not None                       # and so does the captured call
+    for rep in range(3):
+        out.zero_()
+        g.replay()
+        with torch.cuda.stream(side):                 # an eager call of another shape on another stream, its own buffers
+            other = RD.rank_decode(q[:2], Pk[:2], Pv[:2], ku, vu, cosg, sing, lens[:2].contiguous(), num_kv_heads=Hk, nsplit=4)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager call"
+        assert torch.equal(other, eager[:2])
 
 
 def test_packed_api_shared_and_headwise(RD):
