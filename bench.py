@@ -43,6 +43,10 @@ def _parse():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense bf16 comparator leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-breakdown", action="store_true", help="also time every kernel type of the step")
+    ap.add_argument("--handoff-probe", action="store_true",
+                    help="also time the step kernel's hand-off alone (a diagnostic: 256 workgroups exchange a tagged vector, nothing else)")
+    ap.add_argument("--composed", action="store_true",
+                    help="time the persistent step in its composed form as well (rank projections folded into the u-factor phases)")
     ap.add_argument("--no-stress", action="store_true", help="skip the stress configuration's whole-model pass in the default line")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the kernel-level configurations (for profiler runs: their launches share kernel names with the step's)")
@@ -191,16 +195,29 @@ def kernel_configs(model, cache, dec, n_layers: int) -> dict:
                          Vq=a.q_u_proj.weight.view(H, Dh, Ra).transpose(1, 2).contiguous(),
                          Vk=a.k_u_proj.weight.view(H, Dh, Ra).transpose(1, 2).contiguous(),
                          Vv=a.v_u_proj.weight.view(H, Dh, Ra).transpose(1, 2).contiguous()))
+    twin_note = ("bf16 v2-type calls stream cached nn.Linear-layout twins of GateU / UpU / DownV / DownU (a second copy of each operand, "
+                 "built at the first call and kept while the operand lives); the *_xw_kernel entry is the same call on the "
+                 "operands as given (x @ W kernel, FLASHSVD_AMD_REFERENCE_LAYOUT_FAST=0)")
     for B in (1, 8):
         pcat = torch.randn(B, 1, 2 * R, device="cuda").to(torch.bfloat16)          # [PGate | PUp] of one rank projection
 
         def ref_mlp(i, pcat=pcat):
             w = refw[i % nref]
             return DS.flashsvd_mlp_dual_split_triton_v2(pcat[..., R:], pcat[..., :R], w["GateU"], w["UpU"], w["DownV"], w["DownU"])
-        us = per_layer_kernel_us(ref_mlp, n_layers)
         nb = 3 * CFG["intermediate_size"] * R * 2 + d * R * 2 + B * (2 * R + d) * 2
-        out[f"reference_layout_mlp_dual_split_v2_bs{B}"] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3,
-                                                             "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS}
+        for nm, fast in ((f"reference_layout_mlp_dual_split_v2_bs{B}", "1"), (f"reference_layout_mlp_dual_split_v2_xw_kernel_bs{B}", "0")):
+            keep = os.environ.get("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST")
+            os.environ["FLASHSVD_AMD_REFERENCE_LAYOUT_FAST"] = fast
+            try:
+                us = per_layer_kernel_us(ref_mlp, n_layers)
+            finally:
+                if keep is None:
+                    os.environ.pop("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST", None)
+                else:
+                    os.environ["FLASHSVD_AMD_REFERENCE_LAYOUT_FAST"] = keep
+            out[nm] = {"us_per_call": us, "bytes_per_call": nb, "GB/s": nb / us / 1e3, "frac_of_peak": nb / us / 1e3 / HBM_PEAK_GBS,
+                       "operands": "cached transposed twins (warm)" if fast == "1" else "as given (x @ W)"}
+    out["reference_layout_note"] = twin_note
     packed = torch.randn(1, 3 * Ra, device="cuda").to(torch.bfloat16)
 
     def ref_rec(i):
@@ -362,13 +379,34 @@ def run_lowrank(args):
         # wait for the input | weight stream | epilogue and publication, microseconds
         # the hand-off alone (every workgroup writes 16 tagged words and polls the whole vector, nothing else in a round),
         # with the first poll sent at once and held back 0.85 / 1.3 us: what a dependent phase costs before it streams a byte
-        from flashsvd_amd import hip_ops as _ops
-        res["persistent"]["handoff_alone_us_per_round"] = {f"first_poll_after_{64 * dl}_clocks": round(_ops.handoff_probe(2000, dl)["us_per_round"], 3)
-                                                           for dl in (0, 32, 48)}
+        if args.handoff_probe:
+            from flashsvd_amd import hip_ops as _ops
+            res["persistent"]["handoff_alone_us_per_round"] = {f"first_poll_after_{64 * dl}_clocks": round(_ops.handoff_probe(2000, dl)["us_per_round"], 3)
+                                                               for dl in (0, 32, 48)}
         prof = pdec.phase_profile(32)
         res["persistent"]["phase_profile_us"] = {k: {m: round(x, 2) for m, x in v.items()} for k, v in prof.items()}
         pdec.check()
         del pdec
+        if args.composed:
+            # the same step with the rank projections folded into the u-factor phases (PersistentDecoder(composed=True)):
+            # fewer hand-offs, 6 % more bytes; reported beside the default form, never as the headline value
+            scratch_c = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=torch.bfloat16)
+            model(prompt, past_key_values=scratch_c, cache_position=torch.arange(PROMPT_LEN), logits_to_keep=1)
+            cdec = PersistentDecoder(model, scratch_c, composed=True)
+            cdec.set_state(tok, PROMPT_LEN)
+            cdec.step(args.warmup)
+            cdec.check()
+            torch.cuda.synchronize()
+            e0.record()
+            cdec.step(args.steps)
+            e1.record()
+            torch.cuda.synchronize()
+            cdec.check()
+            us_c = e0.elapsed_time(e1) * 1000.0 / args.steps
+            prof = cdec.phase_profile(32)
+            res["persistent_composed"] = dict(tok_s=1e6 / us_c, kernel_us_per_launch=us_c, phases=cdec.nph, last_token=int(cdec.tokens()[-1]),
+                                              phase_profile_us={k: {m: round(x, 2) for m, x in v.items()} for k, v in prof.items()})
+            del cdec, scratch_c
     best = res.get("persistent") or res["graph"]
     res["tok_s"], res["ms_per_step"] = best["tok_s"], best["ms_per_step"]
     if not args.no_kernel_configs:
@@ -641,18 +679,27 @@ def run_stress_model(steps: int = 8, warmup: int = 2, layers: int = 32):
     with torch.no_grad():
         for it in range(3):
             cache = FlashSVDLegacySparseKVCache(model.config, max_batch_size=Bp, max_cache_len=Tp + 8, device="cuda", dtype=torch.bfloat16)
+            for li in range(L):             # the cache sizes a layer at its first use: do it before the measurement
+                cache.ensure_layer_ranks(li, R, R)
             torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            resident = torch.cuda.memory_allocated()
             t0 = time.perf_counter()
             out = model(ids, past_key_values=cache, cache_position=torch.arange(Tp), logits_to_keep=1)
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t0)
+            transient = torch.cuda.max_memory_allocated() - resident
             say(f"prefill {Bp} x {Tp}: {times[-1]:.3f} s")
             del cache, out
     t_pre = min(times[1:])
     attn_flop_pre = 3 * 2.0 * Bp * Tp * R * H * Dh + 2 * 2.0 * Bp * H * Dh * Tp * (Tp + 1) / 2     # head expansion + causal attention
     flop_pre = L * (Bp * Tp * lin_flop_tok + attn_flop_pre) + 2.0 * Bp * d * V
     prefill = {"batch": Bp, "prompt_len": Tp, "s": t_pre, "cold_s": times[0], "tok_s": Bp * Tp / t_pre, "flop": flop_pre,
-               "TFLOPs": flop_pre / t_pre / 1e12, "frac_of_bf16_mfma_peak": flop_pre / t_pre / peak}
+               "TFLOPs": flop_pre / t_pre / 1e12, "frac_of_bf16_mfma_peak": flop_pre / t_pre / peak,
+               # the prompt pass expands q and the context's K / V of a layer to HBM once and attends over them (the reference's
+               # kernel rebuilds K / V tiles per query tile and never writes them): what that costs in memory
+               "transient_bytes_peak": int(transient), "qkv_temporaries_bytes_per_layer": 3 * Bp * Tp * H * Dh * 2,
+               "rank_cache_bytes_per_layer": 2 * Bp * (Tp + 8) * R * 2}
 
     # ---- leg 2: decode at batch 16, context 4096, rank-space cache
     ids = torch.randint(0, V, (Bd, ctx), generator=gen).cuda()
@@ -724,9 +771,14 @@ def run_quant(args):
 
 
 def run_cpu_baseline():
-    """The CPU oracle in fp32 (the precision of the reference's CPU path) on a bounded sample:
-    2 of the 32 layers + final norm + lm_head, prompt 512 (the context of the headline configuration), 6 greedy
-    tokens; per-token decode time is scaled to 32 layers."""
+    """The CPU oracle in fp32 (the precision of the reference's CPU path, scripts/demo_support/api.py:128-143,161-165) on
+    the host cores of this box, every leg a bounded sample:
+      value      the headline shape: 2 of the 32 layers + final norm + lm_head at context 512, 5 timed greedy tokens,
+                 per-layer time scaled to 32 layers;
+      legs.C1    configuration 1 whole: one block of d 512, prompt 128, then 16 greedy decode steps;
+      legs.K2    one attention block call (norm, q / k / v factor pairs, rotation, cache append, attention over 513 keys,
+                 o factor pair, residual) at the 7B shape, batch 1;
+      legs.K3    one SwiGLU MLP call (three factor pairs) at the 7B shape for 1, 8 and 32 rows."""
     import torch
     from oracle import flashsvd_oracle as O
     cores = os.cpu_count() or 1
@@ -755,9 +807,55 @@ def run_cpu_baseline():
             t_layers += t1 - t0
             t_head += t2 - t1
     per_tok = (t_layers / n_s * CFG["num_layers"] + t_head) / (n_new - 1)
+
+    def med_ms(fn, reps):
+        fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return _median(ts) * 1e3
+
+    legs = {}
+    # K2: the attention half of a block (the oracle's block_forward up to its first residual), one token at position 512
+    bw, H, Hk, Dh = mw.blocks[0], mw.n_heads, mw.n_kv_heads, mw.head_dim
+    pos = PROMPT_LEN
+    xk = torch.randn(1, 1, CFG["hidden_size"], generator=torch.Generator().manual_seed(2))
+
+    def attention_block():
+        h1 = O.rms_norm(xk, bw.ln1, mw.eps)
+        c, s_ = cos[pos:pos + 1][None, :, None, :], sin[pos:pos + 1][None, :, None, :]
+        q = O.apply_rope(O.lowrank_pair(h1, bw.q_v, bw.q_u).reshape(1, 1, H, Dh), c, s_)
+        cache.k[0][:1, pos:pos + 1] = O.apply_rope(O.lowrank_pair(h1, bw.k_v, bw.k_u).reshape(1, 1, Hk, Dh), c, s_)
+        cache.v[0][:1, pos:pos + 1] = O.lowrank_pair(h1, bw.v_v, bw.v_u).reshape(1, 1, Hk, Dh)
+        a = O._attend(q, cache.k[0][:1, :pos + 1], cache.v[0][:1, :pos + 1], pos)
+        return xk + O.lowrank_pair(a, bw.o_v, bw.o_u)
+    legs["K2_attention_block_bs1_ctx512"] = {"ms_per_call": med_ms(attention_block, 10)}
+    # K3: the oracle's mlp_forward on RMS-normalised N(0,1) rows
+    for B in (1, 8, 32):
+        h2 = O.rms_norm(torch.randn(B, 1, CFG["hidden_size"], generator=torch.Generator().manual_seed(3)), bw.ln2, mw.eps)
+        legs[f"K3_swiglu_mlp_bs{B}"] = {"ms_per_call": med_ms(lambda: O.mlp_forward(bw, h2), 10)}
+    del mw, cache
+    # C1 on its own protocol: prefill 128, then 16 greedy decode steps
+    mw1, p1 = O.config_c1(torch.float32)
+    runs = []
+    for _ in range(3):
+        c1 = O.DenseCache(mw1, 1, 128 + 20, torch.float32)
+        cs1, sn1 = O.rope_tables(128 + 20, mw1.head_dim, mw1.rope_theta, torch.float32)
+        t0 = time.perf_counter()
+        tk = O.model_forward(mw1, p1, 0, c1, cs1, sn1)[:, -1].argmax(-1, keepdim=True)
+        t1 = time.perf_counter()
+        for s in range(16):
+            tk = O.model_forward(mw1, tk, 128 + s, c1, cs1, sn1)[:, -1].argmax(-1, keepdim=True)
+        t2 = time.perf_counter()
+        runs.append((t1 - t0, (t2 - t1) / 16))
+    pre, dec = _median([r[0] for r in runs]), _median([r[1] for r in runs])
+    legs["C1_one_block_d512_prompt128_16steps"] = {"prefill_ms": pre * 1e3, "decode_ms_per_token": dec * 1e3, "decode_tok_s": 1.0 / dec}
     return {"value": 1.0 / per_tok, "unit": "tok/s", "cores": int(torch.get_num_threads()), "kind": "port",
             "sample": f"CPU oracle fp32, {n_s} of 32 layers + lm_head, context {PROMPT_LEN}-{PROMPT_LEN + n_new - 1}, {n_new - 1} timed greedy tokens, "
-                      f"per-layer time x32 + head time ({per_tok * 1e3:.1f} ms/token)"}
+                      f"per-layer time x32 + head time ({per_tok * 1e3:.1f} ms/token)",
+            "legs": legs}
 
 
 def main():
@@ -822,7 +920,7 @@ def main():
         "prefill": lr["prefill"],
         "kernel_configs": lr.get("kernel_configs"),
     }
-    for k in ("persistent", "graph", "swiglu_roofline"):
+    for k in ("persistent", "persistent_composed", "graph", "swiglu_roofline"):
         if k in lr:
             line[k if k != "graph" else "per_operator_graph"] = lr[k]
     if "kernels" in lr:
