@@ -45,8 +45,11 @@ def _parse():
     ap.add_argument("--kernel-breakdown", action="store_true", help="also time every kernel type of the step")
     ap.add_argument("--handoff-probe", action="store_true",
                     help="also time the step kernel's hand-off alone (a diagnostic: 256 workgroups exchange a tagged vector, nothing else)")
-    ap.add_argument("--composed", action="store_true",
-                    help="time the persistent step in its composed form as well (rank projections folded into the u-factor phases)")
+    ap.add_argument("--no-composed", dest="composed", action="store_false",
+                    help="skip the leg that times the persistent step in its composed form (rank projections folded into the "
+                         "u-factor phases, products with the hidden state streamed as leading phases); the form is opt-in in the "
+                         "library (FLASHSVD_AMD_STEP_COMPOSED=1) because it moves rounding points, and is never the headline value")
+    ap.add_argument("--composed", dest="composed", action="store_true", help=argparse.SUPPRESS)   # the old spelling; now the default
     ap.add_argument("--no-stress", action="store_true", help="skip the stress configuration's whole-model pass in the default line")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the kernel-level configurations (for profiler runs: their launches share kernel names with the step's)")
@@ -389,7 +392,8 @@ def run_lowrank(args):
         del pdec
         if args.composed:
             # the same step with the rank projections folded into the u-factor phases (PersistentDecoder(composed=True)):
-            # fewer hand-offs, 6 % more bytes; reported beside the default form, never as the headline value
+            # eight hand-offs per layer instead of ten, 6 % more bytes; reported beside the default form, never as the headline
+            # value (its rank coefficients come from unrounded sums: closer to exact arithmetic, but not the reference's roundings)
             scratch_c = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=torch.bfloat16)
             model(prompt, past_key_values=scratch_c, cache_position=torch.arange(PROMPT_LEN), logits_to_keep=1)
             cdec = PersistentDecoder(model, scratch_c, composed=True)
@@ -404,7 +408,8 @@ def run_lowrank(args):
             cdec.check()
             us_c = e0.elapsed_time(e1) * 1000.0 / args.steps
             prof = cdec.phase_profile(32)
-            res["persistent_composed"] = dict(tok_s=1e6 / us_c, kernel_us_per_launch=us_c, phases=cdec.nph, last_token=int(cdec.tokens()[-1]),
+            res["persistent_composed"] = dict(tok_s=1e6 / us_c, kernel_us_per_launch=us_c, phases=cdec.nph, leading_phases=bool(cdec.leading),
+                                              last_token=int(cdec.tokens()[-1]),
                                               phase_profile_us={k: {m: round(x, 2) for m, x in v.items()} for k, v in prof.items()})
             del cdec, scratch_c
     best = res.get("persistent") or res["graph"]
@@ -939,6 +944,8 @@ def main():
             "torch_graph": dict(dn, how="same shape, dense bf16 weights, torch.matmul (hipBLASLt) projections, torch elementwise ops, "
                                         "same attention kernel, one HIP graph per token"),
             "bandwidth_ratio_dense_over_lowrank": ds["bytes_per_token"] / lr["step_bytes"]}
+        if "persistent_composed" in lr:
+            line["dense_bf16"]["speedup_composed_form_vs_dense"] = lr["persistent_composed"]["tok_s"] / best
     if not args.no_stress and args.layers == CFG["num_layers"]:
         # the stress configuration (rank ratio ~0.8) as one model: prefill 8 x 2048, decode batch 16 at context 4096 over the
         # rank-space cache; `bench.py --stress` prints the same with the attention kernels timed alone

@@ -231,6 +231,43 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
   for (; s0 + SPB < c.nsteps; s0 += SPB) batch(s0, std::true_type{});
   if (s0 < c.nsteps) batch(s0, std::false_type{});
 }
+// A leading phase (FSVD_PF_LEAD): a slab whose input this workgroup staged long ago is streamed in front of the next
+// phase's slab as one run of the window - the refills of its last batch already fetch the first pieces of the main
+// slab, so the request never pauses between the two, and the main phase polls for its input only after this stream, when
+// the producers have long published.  Every step is full and the steps are a multiple of kU (host-checked), so the
+// window slots come out holding steps 0 .. kU-1 of the main slab in order.
+__device__ __forceinline__ void lead_stream(const GemvCtx& a, const GemvCtx& b, uint32_t m_kp, u32x4_t (&R)[kU], const uint16_t* xs,
+                                            float* cp) {
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lastB = (uint32_t)(b.pps - 1);
+  const int nA = a.nsteps;
+  const int row = (int)__umulhi(tid, m_kp);     // tid / kp
+  int kofs = (int)tid - row * a.kp;             // tid % kp
+  const bool lead = (tid & 15) == 0;
+  // one batch; TAIL: the last one, whose refills are steps 0 .. kU-1 of the main slab (a copy of the body rather than a
+  // choice of base per load: with a branch in the loop the compiler waits for every load at the top of a batch)
+  auto batch = [&](int s0, auto tail) {
+    constexpr bool TAIL = decltype(tail)::value;
+    float d[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xs + kofs * 8);
+      d[u] = dot8_bf16(R[u], xv, 0.f);
+      if (TAIL) R[u] = ld_stream(b.base0, min((uint32_t)(u * kT) + tid, lastB) << 4);
+      else R[u] = ld_stream(a.base0, ((uint32_t)((s0 + u + kU) * kT) + tid) << 4);
+      d[u] = row16_sum(d[u]);
+      kofs += a.dk;
+      kofs = kofs >= a.kp ? kofs - a.kp : kofs;
+    }
+    if (lead) {
+#pragma unroll
+      for (int u = 0; u < kU; ++u) cp[((s0 + u) * kT + (int)tid) >> 4] = d[u];
+    }
+  };
+  int s0 = 0;
+  for (; s0 + kU < nA; s0 += kU) batch(s0, std::false_type{});
+  batch(s0, std::true_type{});
+}
 // ---------------------------------------------------------------------------------------------
 // the same walk over group-wise int4 weights: a 16-byte piece is 32 columns, 8 consecutive lanes form a chunk of
 // 256 columns of one row (K % 256 == 0).  No weight becomes a float: OR-ing 0x4300 over a nibble n gives the bf16
@@ -631,17 +668,24 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
   uint32_t dvA = desc_fetch(phases, 0, nph), dvB = dvA;   // descriptors of phase p and p+1
 
   // Iteration p: finish phase p (its first weights were requested one iteration earlier), publish its
-  // outputs, request the first weights of phase p+1.
-  for (int p = -1; p < nph; ++p) {
+  // outputs, request the first weights of phase p+1.  A leading phase (FSVD_PF_LEAD) and the phase behind it are one
+  // iteration: the leading slab is streamed first, then the main phase runs as usual.
+  for (int p = -1; p < nph;) {
     const uint32_t dvC = desc_fetch(phases, p + 2, nph);   // needed one iteration from now
-    const uint32_t dv = dvA;
+    const uint32_t dvD = CX ? desc_fetch(phases, p + 3, nph) : dvC;
+    const bool lead = CX && p >= 0 && DF_I(dvA, type) == FSVD_PH_GEMV && (DF_I(dvA, flags) & FSVD_PF_LEAD) != 0;
+    const uint32_t dvF = dvA;                              // the leading phase, when there is one
+    const uint32_t dv = lead ? dvB : dvA;                  // the phase this iteration completes
+    const uint32_t dvN = lead ? dvC : dvB;                 // the phase whose first window it requests
+    const int pm = lead ? p + 1 : p;
     const int type = p < 0 ? -1 : DF_I(dv, type);
     unsigned long long* tr = nullptr;
     if (TRACE && p >= 0 && tid == 0 && (w % trace_stride) == 0) {
-      tr = trace + ((size_t)(w / trace_stride) * nph + p) * 4;
+      tr = trace + ((size_t)(w / trace_stride) * nph + pm) * 4;
       tr[0] = wall_clock64();
     }
-    GemvCtx gc;
+    GemvCtx gc, fc;
+    float* cpm = cp;                       // chunk partials of the main phase (behind those of a leading phase)
     AttnWork aw;
     uint32_t resid = 0;
     int rows0 = 0x7fffffff;                // GEMV: first row of the fp32 group
@@ -649,9 +693,23 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     // addresses of the next phase's first window, worked out now (behind the wait for this phase's input) so that the
     // request after publication is nothing but the loads
     uint64_t nxt[kU], nxt_sz[kSzLoads];
-    window_addresses<Q4>(dvB, w, pos, reinterpret_cast<uint64_t>(phases), nxt, nxt_sz);
+    window_addresses<Q4>(dvN, w, pos, reinterpret_cast<uint64_t>(phases), nxt, nxt_sz);
 
     // ------------------------------------------------------------------ stage + stream
+    if (CX && lead) {
+      gemv_ctx<false>(dvF, w, fc);
+      gemv_ctx<false>(dv, w, gc);
+      // the epilogue of the previous phase may still be reading the partial buffer in another wave (its LDS reads are
+      // complete by the time that wave's stores have been issued, i.e. before it arrives here)
+      __builtin_amdgcn_s_barrier();
+      lead_stream(fc, gc, desc_u32(dvF, FSVD_DW(m_kp)), R, xs + fc.xoff, cp);
+      cpm = cp + (fc.pps >> 4);
+      if (TRACE && tr) {                   // the leading phase: entered, (nothing staged), streamed, (published with the main phase)
+        unsigned long long* trf = tr - 4;
+        trf[0] = trf[1] = tr[0];
+        trf[2] = trf[3] = tr[0] = wall_clock64();
+      }
+    }
     if (type == FSVD_PH_GEMV) {
       gemv_ctx<Q4>(dv, w, gc);
       const int epi = DF_I(dv, epilogue);
@@ -704,7 +762,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       }
       // an int4 phase in the bf16 build, or a phase of the composed form in a build without it, is an error too
       if (__syncthreads_or((ok && (Q4 || DF_I(dv, wbits) != 4) && (CX || (DF_I(dv, flags) == 0 && epi != FSVD_EP_F32))) ? 0 : 1)) {
-        raise_error(st, p, w);
+        raise_error(st, pm, w);
         return;
       }
       if (TRACE && tr) tr[1] = wall_clock64();
@@ -722,7 +780,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
         gemv_stream<1, true>(gc, m_kp, g1, g2, R, xs + (CX ? gc.xoff : 0), cp);
       } else if (gc.nmat == 1) {
-        gemv_stream<1, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cp);
+        gemv_stream<1, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cpm);
       } else {
         gemv_stream<2, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cp);
       }
@@ -774,7 +832,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           cb[half] = o1;
         }
       }
-      if (__syncthreads_or(fail ? 1 : 0)) { raise_error(st, p, w); return; }
+      if (__syncthreads_or(fail ? 1 : 0)) { raise_error(st, pm, w); return; }
       if (TRACE && tr) tr[1] = wall_clock64();
       const float scale = DF_F(dv, fparam);
       const int part = tid & 15, slot = tid >> 4;
@@ -813,7 +871,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       const uint32_t tout = DF_TAG16(dv, out0, epoch);
       void* out = DF_P(dv, out0);
       const int grp = tid >> 3;
-      const bool lead = (tid & 7) == 0;
+      const bool lead8 = (tid & 7) == 0;
       const int npass = (gc.srows + kT / 8 - 1) / (kT / 8);
       if (epi == FSVD_EP_LOGITS) {
         float best = -INFINITY;
@@ -822,7 +880,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         for (int ps = 0; ps < npass; ++ps) {
           const int t = min(ps * (kT / 8) + grp, gc.srows - 1);
           const float v = round_bf16(row_sum8(cp, t, cpr));
-          if (lead && ps * (kT / 8) + grp < gc.srows) {
+          if (lead8 && ps * (kT / 8) + grp < gc.srows) {
             logits[gc.r0 + t] = (uint16_t)f32_to_bf16_bits(v);
             if (v > best) { best = v; best_i = gc.r0 + t; }
           }
@@ -847,10 +905,10 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         const int mode = DF_I(dv, mode);
         for (int ps = 0; ps < npass; ++ps) {
           const int t = min(ps * (kT / 8) + grp, gc.srows - 1);
-          const bool live = lead && ps * (kT / 8) + grp < gc.srows;
+          const bool live = lead8 && ps * (kT / 8) + grp < gc.srows;
           float v;
           if (CX && gc.r0 + t >= rows0) {      // fp32 row group: the unrounded sum (+ the part of it an earlier phase left)
-            v = row_sum8(cp, t, cpr) + addend;
+            v = row_sum8(cpm, t, cpr) + addend;
             if (live) st_tag64(DF_P(dv, out1), gc.r0 + t - rows0, DF_TAG32(dv, out1, epoch), __float_as_uint(v));
             continue;
           }
@@ -864,14 +922,23 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
               v = round_bf16((gv * (1.0f / (1.0f + expf(-gv)))) * uv);
             }
           } else {
-            v = round_bf16(row_sum8(cp, t, cpr));
+            v = round_bf16(row_sum8(cpm, t, cpr));
             if (epi == FSVD_EP_RESID) v = round_bf16(bf16_bits_to_f32(resid & 0xffffu) + v);
           }
           if (live) st_tag16(out, gc.r0 + t, tout, f32_to_bf16_bits(v));
         }
       }
-      // no barrier here: the next phase writes cp only after its staging barrier, which every wave reaches
-      // after this epilogue
+      if (CX && lead) {
+        // the rows of the leading phase: unrounded sums, taken by the lane groups from the top of the workgroup down
+        // while those from the bottom up run the main epilogue
+        const int t = kT / 8 - 1 - grp;
+        if (t < fc.srows) {
+          const float v = row_sum8(cp, t, fc.kp >> 4);
+          if (lead8) st_tag64(DF_P(dvF, out1), fc.r0 + t, DF_TAG32(dvF, out1, epoch), __float_as_uint(v));
+        }
+      }
+      // no barrier here: the next phase writes cp only after its staging barrier (a leading phase: after a barrier of
+      // its own), which every wave reaches after this epilogue
     } else if (type == FSVD_PH_ATTN) {
       // fold the key slots and publish this split's (acc, m, l)
       const int Dh = 128;
@@ -915,7 +982,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       // leaves when no logit compares) must not become an address; row 0 is read instead and the step reports it
       const int V = DF_I(dv, K);
       long long tk = token;
-      if (V > 0 && (tk < 0 || tk >= V)) { tk = 0; raise_error(st, p, w); }
+      if (V > 0 && (tk < 0 || tk >= V)) { tk = 0; raise_error(st, pm, w); }
       const uint16_t* row = static_cast<const uint16_t*>(DF_P(dv, W)) + tk * (int64_t)N;
       const uint32_t tg = DF_TAG16(dv, out0, epoch);
       void* out = DF_P(dv, out0);
@@ -939,7 +1006,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         if (!poll_w64(in, (head * nsplit + sp) * (Dh + 2) + col, tin, st, limit, payload)) fail = true;
         cp[it] = __uint_as_float(payload);
       }
-      if (__syncthreads_or(fail ? 1 : 0)) { raise_error(st, p, w); return; }
+      if (__syncthreads_or(fail ? 1 : 0)) { raise_error(st, pm, w); return; }
       if (tid < cnt) {
         float M = -INFINITY, num = 0.f, den = 0.f;
         for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, cp[sp * per + cnt]);
@@ -979,14 +1046,14 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
         }
         if ((tid & 63) == 0) { red[tid >> 6] = best; ired[tid >> 6] = best_i; }
-        if (__syncthreads_or(fail ? 1 : 0)) { raise_error(st, p, w); return; }
+        if (__syncthreads_or(fail ? 1 : 0)) { raise_error(st, pm, w); return; }
         if (tid == 0) {
           for (int i = 1; i < kT / 64; ++i)
             if (red[i] > best || (red[i] == best && ired[i] < best_i)) { best = red[i]; best_i = ired[i]; }
           // no logit compared greater than -inf (all NaN): there is no greedy token; token 0 stands in and the step says so
           if (best_i == 0x7fffffff) {
             best_i = 0;
-            __hip_atomic_store(&st->err, p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&st->err, pm + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             st->err_wg = w;
           }
           long long* log = static_cast<long long*>(DF_P(dv, plain_out));
@@ -998,8 +1065,15 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       }
     }
     if (TRACE && tr) tr[3] = wall_clock64();
-    if (p >= 0) dvA = dvB;   // iteration -1 already holds descriptor 0 in both
-    dvB = dvC;
+    if (CX && lead) {
+      dvA = dvC;
+      dvB = dvD;
+      p += 2;
+    } else {
+      if (p >= 0) dvA = dvB;   // iteration -1 already holds descriptor 0 in both
+      dvB = dvC;
+      ++p;
+    }
   }
   // Every workgroup read the state before it produced anything, and workgroup 0 cannot get here before
   // it has consumed data from all the others, so bumping the epoch now cannot be seen by this launch.
@@ -1139,8 +1213,9 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
             if (reinterpret_cast<uintptr_t>(d.qsz[m]) & 3) return bad("scale | zero words must be 4-byte aligned", p);
         }
         if (d.N < nwg) return bad("fewer rows than workgroups", p);
-        if (d.flags & ~(FSVD_PF_NOWAIT | FSVD_PF_STAGE2 | FSVD_PF_SPLIT)) return bad("unknown flag", p);
+        if (d.flags & ~(FSVD_PF_NOWAIT | FSVD_PF_STAGE2 | FSVD_PF_SPLIT | FSVD_PF_LEAD)) return bad("unknown flag", p);
         const bool nowait = d.flags & FSVD_PF_NOWAIT, stage2 = d.flags & FSVD_PF_STAGE2, split = d.flags & FSVD_PF_SPLIT;
+        const bool leading = d.flags & FSVD_PF_LEAD;
         const bool f32rows = split || d.epilogue == FSVD_EP_F32;
         if ((d.flags != 0 || f32rows || d.in_off != 0) && q4) return bad("flags, fp32 rows and input offsets are for bf16 weights", p);
         if (d.H > 0) {   // q | k | v row groups reading [Pq | Pk | Pv]
@@ -1154,11 +1229,45 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         if (nowait) {
           // the input is what the previous phase of the same workgroup left in its staging area
           if (stage2 || d.norm_w || d.aux2.ptr) return bad("a phase without a hand-off stages nothing and takes no addend", p);
+          if (leading) {
+            // streamed in front of the next phase: the input is what an earlier two-vector staging left at in_off, and
+            // nothing since may have been staged over it
+            if (d.epilogue != FSVD_EP_F32 || d.nmat != 1 || d.H > 0 || split)
+              return bad("a leading phase is a single matrix whose rows leave as unrounded fp32 sums", p);
+            if (d.N % nwg != 0 || d.N / nwg > kT / 8) return bad("a leading phase deals the same number of rows, at most kT/8, to every workgroup", p);
+            if (((int64_t)(d.N / nwg) * (d.K / 8)) % (kT * kU) != 0) return bad("the slab of a leading phase must fill whole windows (rows per workgroup x K/8 a multiple of kT x kU)", p);
+            if (p + 1 >= nph) return bad("a leading phase needs a phase behind it", p);
+            const fsvd_phase& m = ph[p + 1];
+            if (m.type != FSVD_PH_GEMV || m.nmat != 1 || m.H > 0 || m.flags != 0 || m.wbits == 4 ||
+                (m.epilogue != FSVD_EP_STORE && m.epilogue != FSVD_EP_RESID))
+              return bad("the phase behind a leading phase must be a plain single-matrix bf16 GEMV that stores or adds a residual", p);
+            if (d.in_off < gemv_in_len(m)) return bad("the staged input of a leading phase overlaps the input of the phase behind it", p);
+            if ((int64_t)(d.N / nwg) * (d.K / 128) + (((int64_t)m.N + nwg - 1) / nwg) * (m.K / 128) > kMaxChunks)
+              return bad("a leading phase and the phase behind it overflow the partial buffer", p);
+            bool found = false;
+            for (int q = p - 1; q >= 0 && !found; --q) {
+              const fsvd_phase& e = ph[q];
+              if (e.type == FSVD_PH_GEMV) {
+                if ((e.flags & FSVD_PF_STAGE2) && e.in2_off == d.in_off && e.in2_len == n_in) { found = true; break; }
+                if (e.flags & FSVD_PF_NOWAIT) continue;
+                const bool hits2 = (e.flags & FSVD_PF_STAGE2) && e.in2_off < d.in_off + n_in && d.in_off < e.in2_off + e.in2_len;
+                if (gemv_in_len(e) > d.in_off || hits2) return bad("the staged input of a leading phase was overwritten by a later staging", p);
+              } else if (e.type == FSVD_PH_ATTN) {
+                if (3 * e.Dh > d.in_off) return bad("the staged input of a leading phase was overwritten by an attention phase", p);
+              } else if (e.type != FSVD_PH_MERGE) {
+                break;
+              }
+            }
+            if (!found) return bad("a leading phase must read a vector that an earlier two-vector staging left in place", p);
+          } else {
           if (p == 0 || ph[p - 1].type != FSVD_PH_GEMV) return bad("a phase without a hand-off must follow a GEMV phase", p);
           const fsvd_phase& q = ph[p - 1];
           const bool from_in2 = (q.flags & FSVD_PF_STAGE2) && d.in_off == q.in2_off && n_in == q.in2_len;
           const bool same_in = d.in_off == q.in_off && n_in <= gemv_in_len(q) && !q.norm_w && !(q.flags & FSVD_PF_STAGE2);
           if (!from_in2 && !same_in) return bad("a phase without a hand-off must read what the previous phase staged", p);
+          }
+        } else if (leading) {
+          return bad("a leading phase reads a staged input: FSVD_PF_NOWAIT must be set with FSVD_PF_LEAD", p);
         } else if (d.in_off != 0) {
           return bad("a staged input starts at offset 0", p);
         }

@@ -20,7 +20,7 @@ import os
 import torch
 
 from . import _lib
-from ._lib import (EP_F32, EP_LOGITS, EP_RESID, EP_STORE, EP_SWIGLU, PF_NOWAIT, PF_SPLIT, PF_STAGE2, PH_ARGMAX, PH_ATTN, PH_EMBED,
+from ._lib import (EP_F32, EP_LOGITS, EP_RESID, EP_STORE, EP_SWIGLU, PF_LEAD, PF_NOWAIT, PF_SPLIT, PF_STAGE2, PH_ARGMAX, PH_ATTN, PH_EMBED,
                    PH_GEMV, PH_MERGE, Phase, TagBuf)
 from .runtime.cache import FlashSVDV15DenseKVCache
 
@@ -303,6 +303,17 @@ class PersistentDecoder:
 
         self.composed = bool(composed) and part == "model" and not any(layer_q4) and max(slots(3 * Rq), slots(2 * Rm)) <= 8 \
             and max(in2_off_a, in2_off_m) + d <= 16384 and d + max(3 * Rq, 2 * Rm) <= 64 * self.nwg
+        # The products with the hidden state as leading phases (streamed in front of o_v / down_v): the hidden state
+        # must stay in the staging area until then, i.e. behind everything staged in between, and a workgroup's share of
+        # each product must fill whole windows of loads
+        lead_off_a = (max(3 * Rq, H * Dh, 3 * Dh) + 127) // 128 * 128
+        lead_off_m = (max(2 * Rm, D) + 127) // 128 * 128
+        want_lead = os.getenv("FLASHSVD_AMD_STEP_LEAD", "1").strip().lower() in ("1", "true", "on", "yes")
+        self.leading = self.composed and want_lead and max(lead_off_a, lead_off_m) + d <= 16384 and all(
+            n % self.nwg == 0 and n // self.nwg <= 64 and ((n // self.nwg) * (d // 8)) % 2048 == 0
+            for r in ranks for n in (3 * r[0], 2 * r[2]))
+        if self.leading:
+            in2_off_a, in2_off_m = lead_off_a, lead_off_m
         if self.composed:
             self._composed_layers(layers, ranks, bf16_weights, gemv, attention, in2_off_a, in2_off_m)
         for l, layer in enumerate(layers):
@@ -392,8 +403,14 @@ class PersistentDecoder:
         ``[o_u; [gate_v; up_v]' o_u]`` — its first rows give the new hidden state, the others complete the sums, which the
         SwiGLU phase scales by 1 / rms of that state while staging them; the same with down_u and the NEXT layer's
         ``[q_v; k_v; v_v]'``, whose product with the mid-layer state rides behind the SwiGLU pair.  Per layer: ten
-        hand-offs become eight, the two moved products (25 MB each at the 7B shape) stream while the hand-off behind the
-        expansion and behind the pair is in flight, and the two composed blocks add 6 % to the layer's bytes.
+        hand-offs become eight and the two composed blocks add 6 % to the layer's bytes.
+
+        Where the two moved products (25 MB each at the 7B shape) run: as *leading phases* (``self.leading``) when a
+        workgroup's share of each fills whole windows of loads and the staging area can keep the hidden state that long -
+        ``[gate_v; up_v]' x`` is then streamed in front of o_v and the next layer's ``[q_v; k_v; v_v]' x2`` in front of
+        down_v, in one run of loads with the slab behind them, so that neither pays a pipeline drain of its own and o_v /
+        down_v poll for their input when it has long been published; otherwise as phases of their own behind the
+        expansion and behind the pair (the older arrangement, FLASHSVD_AMD_STEP_LEAD=0 forces it).  Same sums, same bits.
 
         Arithmetic: the hidden states take the same roundings as in the ten-phase form; the rank coefficients are formed
         from the unrounded residual sum and rounded once (the ten-phase form rounds the hidden state, the normalised
@@ -433,8 +450,12 @@ class PersistentDecoder:
                 gemv("attn_rank_proj", [fq[0][1]], 3 * rq, d, xin, None, epi=EP_F32, out1=_tb(self.PRAW, L, 0))
             gemv("qkv_u", [w["qkv_u"]], (H + 2 * Hk) * Dh, rq, _tb(self.PRAW, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh),
                  flags=PF_STAGE2, eps=n1.variance_epsilon, in2=xin, in2_len=d, in2_off=off_a)
-            gemv("mlp_rank_x", [gu16], 2 * rm, d, None, None, epi=EP_F32, flags=PF_NOWAIT, in_off=off_a, out1=_tb(self.G0, L, l))
+            if not self.leading:
+                gemv("mlp_rank_x", [gu16], 2 * rm, d, None, None, epi=EP_F32, flags=PF_NOWAIT, in_off=off_a, out1=_tb(self.G0, L, l))
             attention(l, l)
+            if self.leading:
+                gemv("mlp_rank_x", [gu16], 2 * rm, d, None, None, epi=EP_F32, flags=PF_NOWAIT | PF_LEAD, in_off=off_a,
+                     out1=_tb(self.G0, L, l))
             gemv("o_v", [w["o_v"]], ro, H * Dh, _tb(self.A, L, l), _tb(self.PO, L, l))
             gemv("o_u+mlp_rank", [cat_o], d + 2 * rm, ro, _tb(self.PO, L, l), xmid, epi=EP_RESID, aux=xin, flags=PF_SPLIT, rows0=d,
                  aux2=_tb(self.G0, L, l), out1=_tb(self.PMRAW, L, l))
@@ -442,8 +463,8 @@ class PersistentDecoder:
                  flags=PF_STAGE2, eps=n2.variance_epsilon, in2=xmid, in2_len=d, in2_off=off_m)
             if l + 1 < L:
                 rq_n = ranks[l + 1][0]
-                gemv("attn_rank_x", [fq[l + 1][1]], 3 * rq_n, d, None, None, epi=EP_F32, flags=PF_NOWAIT, in_off=off_m,
-                     out1=_tb(self.Q0, nq0, l))
+                gemv("attn_rank_x", [fq[l + 1][1]], 3 * rq_n, d, None, None, epi=EP_F32,
+                     flags=PF_NOWAIT | (PF_LEAD if self.leading else 0), in_off=off_m, out1=_tb(self.Q0, nq0, l))
             gemv("down_v", [w["down_v"]], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
             if l + 1 < L:
                 cat_d = torch.cat([w["down_u"].data, (fq[l + 1][0] @ w["down_u"].data.float()).to(torch.bfloat16)]).contiguous()
@@ -685,6 +706,7 @@ class DenseStepDecoder(PersistentDecoder):
         g.plain_out = self.token_log.data_ptr()
         ph.append(g)
         self.composed = False
+        self.leading = False
         self._names = ["embed"] + [n for _ in range(L) for n in self.PHASE_NAMES[1:]] + ["lm_head", "argmax"]
         self._finish(ph, dev)
 

@@ -133,6 +133,69 @@ def test_7b_width_two_layers_teacher_forced_tie_aware(composed):
         assert_close_bf16(dec.hidden()[None].cpu(), ref_hid[:, s], f"hidden state at step {s}", abs_tol=3 * b["abs_tol"], rel_tol=3e-2)
         n_equal += _tie_aware(g, int(ref_tok[0, s]), ref_logits[0, s], f"step {s}")
     assert n_equal >= n_new - 3
+    if not composed:
+        return
+    # At this width the products with the hidden state run as leading phases (streamed in front of o_v / down_v); the
+    # host-side check refuses a leading phase whose staged input is gone, whose slab leaves a window half filled, or
+    # whose follower is not a plain GEMV
+    import ctypes
+    from flashsvd_amd import _lib
+    from flashsvd_amd._lib import PF_LEAD, PF_NOWAIT
+    assert dec.leading
+    names, hp, n, lib = dec.phase_names(), dec.host_phases, dec.nph, _lib.load()
+    assert names.index("mlp_rank_x") + 1 == names.index("o_v") and names.index("attn_rank_x") + 1 == names.index("down_v")
+
+    def verdict():
+        return lib.fsvd_decode_step_validate(ctypes.addressof(hp), n, dec.nwg), lib.fsvd_last_error()
+
+    assert verdict()[0] == 0
+    i = names.index("mlp_rank_x")
+    assert hp[i].flags == PF_LEAD | PF_NOWAIT
+    saved = hp[i].in_off
+    hp[i].in_off = saved + 128
+    rc, msg = verdict()
+    assert rc == -1 and b"overwritten by a later staging" in msg
+    hp[i].in_off = saved
+    hp[i].flags = PF_LEAD
+    rc, msg = verdict()
+    assert rc == -1 and b"FSVD_PF_NOWAIT must be set" in msg
+    hp[i].flags = PF_LEAD | PF_NOWAIT
+    saved = hp[i + 1].norm_w, hp[i + 1].epilogue
+    hp[i + 1].epilogue = 2                       # a SwiGLU pair cannot sit behind a leading phase
+    rc, msg = verdict()
+    assert rc == -1 and b"behind a leading phase" in msg
+    hp[i + 1].epilogue = saved[1]
+    j = names.index("qkv_u")
+    saved = hp[j].in2_off
+    hp[j].in2_off = saved - 1024                 # the hidden state would be staged where o_v's input goes later
+    hp[i].in_off = saved - 1024
+    rc, msg = verdict()
+    assert rc == -1 and b"overlaps the input of the phase behind it" in msg
+    hp[j].in2_off = hp[i].in_off = saved
+    assert verdict()[0] == 0
+
+
+def test_composed_form_without_leading_phases_matches_the_leading_arrangement(monkeypatch):
+    """The composed form keeps its older arrangement (the product with the hidden state as a phase of its own behind the
+    q | k | v expansion and behind the SwiGLU pair) for shapes whose slabs do not fill whole windows; at the 7B width both
+    arrangements are possible, compute the same sums in the same order, and must give the same bits."""
+    from flashsvd_amd.step import PersistentDecoder
+    mw = O.make_model(d=4096, n_heads=32, n_kv_heads=32, head_dim=128, ffn=11008, attn_rank=1024, mlp_rank=1536,
+                      n_layers=2, vocab=32000, dtype=BF16, seed=3)
+    prompt = torch.randint(0, 32000, (1, 40), generator=torch.Generator().manual_seed(2))
+    model = model_from_oracle(mw)
+    outs = []
+    for lead in ("1", "0"):
+        monkeypatch.setenv("FLASHSVD_AMD_STEP_LEAD", lead)
+        cache, tok0 = _prefill(model, prompt, 12)
+        dec = PersistentDecoder(model, cache, composed=True)
+        assert dec.composed and dec.leading == (lead == "1")
+        dec.set_state(tok0, prompt.shape[1])
+        dec.step(8)
+        dec.check()
+        outs.append((dec.tokens().cpu().clone(), dec.hidden().cpu().clone(), dec.logits.cpu().clone()))
+    assert torch.equal(outs[0][0], outs[1][0])
+    assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2])
 
 
 def test_tag_wrap_decodes_the_same_tokens():
