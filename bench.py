@@ -43,8 +43,6 @@ def _parse():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense bf16 comparator leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-breakdown", action="store_true", help="also time every kernel type of the step")
-    ap.add_argument("--handoff-probe", action="store_true",
-                    help="also time the step kernel's hand-off alone (a diagnostic: 256 workgroups exchange a tagged vector, nothing else)")
     ap.add_argument("--no-composed", dest="composed", action="store_false",
                     help="skip the leg that times the persistent step in its composed form (rank projections folded into the "
                          "u-factor phases, products with the hidden state streamed as leading phases); the form is opt-in in the "
@@ -380,12 +378,6 @@ def run_lowrank(args):
                                  workgroups=pdec.nwg, last_token=int(pdec.tokens()[-1]))
         # where the launch's time goes, from inside the kernel: per phase kind (averaged over layers and 8 workgroups)
         # wait for the input | weight stream | epilogue and publication, microseconds
-        # the hand-off alone (every workgroup writes 16 tagged words and polls the whole vector, nothing else in a round),
-        # with the first poll sent at once and held back 0.85 / 1.3 us: what a dependent phase costs before it streams a byte
-        if args.handoff_probe:
-            from flashsvd_amd import hip_ops as _ops
-            res["persistent"]["handoff_alone_us_per_round"] = {f"first_poll_after_{64 * dl}_clocks": round(_ops.handoff_probe(2000, dl)["us_per_round"], 3)
-                                                               for dl in (0, 32, 48)}
         prof = pdec.phase_profile(32)
         res["persistent"]["phase_profile_us"] = {k: {m: round(x, 2) for m, x in v.items()} for k, v in prof.items()}
         pdec.check()

@@ -142,7 +142,6 @@ SIGNATURES = {
                                    + [c_void_p, c_size_t, c_void_p]),
     "fsvd_mlp_dual_split_workspace_bytes": (c_size_t, [c_int] * 6),
     "fsvd_decode_step_workgroups": (c_int, []),
-    "fsvd_handoff_probe": (c_int, [c_void_p, c_size_t, c_int, c_int, c_void_p]),
     "fsvd_decode_step_prepare": (c_int, [c_void_p, c_int, c_int]),
     "fsvd_decode_step_validate": (c_int, [c_void_p, c_int, c_int]),
     "fsvd_set_workspace": (c_int, [c_void_p, c_size_t, c_void_p]),

@@ -629,22 +629,4 @@ int fsvd_decode_step_trace(const fsvd_phase* phases_dev, const fsvd_phase* phase
                             decode_step_build(phases_host, nphase), static_cast<hipStream_t>(stream));
 }
 
-int fsvd_handoff_probe(void* scratch, size_t scratch_bytes, int rounds, int delay, void* stream) {
-  const char* fn = "fsvd_handoff_probe";
-  FSVD_REQUIRE_PTR(scratch, fn);
-  const int nwg = decode_step_workgroups();
-  if (nwg <= 0) return kErrLaunch;
-  if (rounds <= 0 || rounds > 60000 || delay < 0 || delay > 1024) { set_last_error("%s: rounds must be 1..60000 and delay 0..1024", fn); return kErrBadShape; }
-  const size_t need = 256 + (size_t)2 * 16 * nwg * sizeof(uint32_t);
-  if (scratch_bytes < need || (reinterpret_cast<uintptr_t>(scratch) & 15) != 0) {
-    set_last_error("%s: scratch of %zu bytes (16-byte aligned) needed, %zu given", fn, need, scratch_bytes);
-    return kErrWorkspace;
-  }
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  hipError_t e = hipMemsetAsync(scratch, 0, need, st);
-  if (e != hipSuccess) { set_last_error("%s: cannot clear the scratch: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
-  uint32_t* out = static_cast<uint32_t*>(scratch);
-  return launch_handoff_probe(out + 64, out, nwg, rounds, delay, 1 << 15, st);
-}
-
 }  // extern "C"

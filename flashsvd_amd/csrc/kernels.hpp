@@ -200,7 +200,6 @@ int decode_step_workgroups();
 int prepare_decode_step(fsvd_phase* host_phases, int nph, int nwg);
 int validate_decode_step(const fsvd_phase* host_phases, int nph, int nwg);
 int decode_step_build(const fsvd_phase* host_phases, int nph);   // 0 bf16, 1 with int4 phases, 2 with the composed form's phases
-int launch_handoff_probe(uint32_t* vec, uint32_t* out, int workgroups, int rounds, int delay, int spin, hipStream_t st);   // handoff_probe.hip
 int launch_decode_step(const fsvd_phase* dev_phases, int nph, fsvd_step_state* state, unsigned long long* trace,
                        int trace_stride, int build, hipStream_t stream);
 }  // namespace fsvd

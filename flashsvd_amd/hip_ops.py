@@ -90,30 +90,6 @@ def release_split_workspace(device: Optional[torch.device] = None) -> None:
             _lib.check("fsvd_set_workspace", _lib.load().fsvd_set_workspace(None, 0, None))
 
 
-def handoff_probe(rounds: int = 2000, delay: int = 32, device: Optional[torch.device] = None) -> dict:
-    """Microseconds per round of the persistent step's hand-off alone (``fsvd_handoff_probe``: every workgroup writes its
-    16 tagged words and polls the whole vector, nothing else in a round), the stale polling rounds per workgroup and
-    round, and the number of workgroups that gave up (0 unless something else held compute units)."""
-    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else device
-    lib = _lib.load()
-    with torch.cuda.device(dev):
-        nwg = int(lib.fsvd_decode_step_workgroups())
-        if nwg <= 0:
-            raise RuntimeError((lib.fsvd_last_error() or b"").decode() or "fsvd_decode_step_workgroups: cannot query the device")
-        scratch = torch.empty(256 + 128 * nwg, dtype=torch.uint8, device=dev)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        times = []
-        for _ in range(3):
-            e0.record()
-            _lib.check("fsvd_handoff_probe", lib.fsvd_handoff_probe(scratch.data_ptr(), scratch.numel(), rounds, delay, _stream()))
-            e1.record()
-            e1.synchronize()
-            times.append(e0.elapsed_time(e1))
-        words = scratch[:8].view(torch.int32).tolist()
-    return {"us_per_round": min(times) * 1000.0 / rounds, "stale_polls_per_round": words[1] / (nwg * rounds), "gave_up": words[0],
-            "workgroups": nwg, "rounds": rounds, "delay_clocks": 64 * delay}
-
-
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
            norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
            residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:

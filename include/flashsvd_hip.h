@@ -398,14 +398,6 @@ typedef struct fsvd_step_state {
  * for each other's results).  While a step runs nothing else may execute on the device; a step that is starved of
  * compute units ends by its spin limit with state->err set. */
 int fsvd_decode_step_workgroups(void);
-/* No counterpart in the reference: a diagnostic of the step kernel's hand-off.  The grid of fsvd_decode_step_workgroups()
- * workgroups exchanges a tagged vector (16 words written per workgroup, all of it polled by every workgroup, with the
- * step kernel's stores and loads) `rounds` times in one launch, with nothing else in a round; `delay` x 64 clocks pass
- * between a workgroup's stores and its first poll.  Time the launch on `stream`: duration / rounds is what a dependent
- * phase costs before it streams a byte.  scratch: device memory, 16-byte aligned, 256 + 128 * workgroups bytes, cleared
- * by the call (with a memset: do not capture it); afterwards word 0 = workgroups that gave up (0 unless the grid was
- * starved of compute units), word 1 = polling rounds that came back stale, summed over workgroups. */
-int fsvd_handoff_probe(void* scratch, size_t scratch_bytes, int rounds, int delay, void* stream);
 /* Fill the derived fields of a host-side phase list for `workgroups` workgroups (call before uploading it). */
 int fsvd_decode_step_prepare(fsvd_phase* phases_host, int nphase, int workgroups);
 /* The host-side check of fsvd_decode_step alone (no launch): 0, or a negative status with fsvd_last_error(). */
