@@ -670,32 +670,52 @@ def run_stress_model(steps: int = 8, warmup: int = 2, layers: int = 32):
     peak = 2500e12
     lin_flop_tok = 2.0 * (8 * d * R + 3 * (d + D) * RM)          # factor products per token per layer
 
-    # ---- leg 1: prefill 8 x 2048
+    # ---- leg 1: prefill 8 x 2048.  The prompt pass rebuilds q and the context's K / V from the rank coefficients into
+    # temporaries and attends over them; the heads can be taken in groups sized by a byte budget (default 1 GiB: all heads
+    # at once at this shape), and the same pass with a 64 MiB budget is timed beside it: what the temporaries cost in
+    # memory, and what the grouping costs in time.  (The reference's kernel rebuilds K / V tiles per query tile inside its
+    # attention loop and writes none.)
+    from flashsvd_amd import hip_ops as _ops
     ids = torch.randint(0, V, (Bp, Tp), generator=gen).cuda()
-    times = []
-    with torch.no_grad():
-        for it in range(3):
-            cache = FlashSVDLegacySparseKVCache(model.config, max_batch_size=Bp, max_cache_len=Tp + 8, device="cuda", dtype=torch.bfloat16)
-            for li in range(L):             # the cache sizes a layer at its first use: do it before the measurement
-                cache.ensure_layer_ranks(li, R, R)
-            torch.cuda.synchronize()
-            torch.cuda.reset_peak_memory_stats()
-            resident = torch.cuda.memory_allocated()
-            t0 = time.perf_counter()
-            out = model(ids, past_key_values=cache, cache_position=torch.arange(Tp), logits_to_keep=1)
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-            transient = torch.cuda.max_memory_allocated() - resident
-            say(f"prefill {Bp} x {Tp}: {times[-1]:.3f} s")
-            del cache, out
-    t_pre = min(times[1:])
+    legs = {}
+    saved_budget = os.environ.get("FLASHSVD_AMD_PREFILL_TEMP_BYTES")
+    for name, budget in (("default", None), ("head_groups_64MiB", str(64 << 20))):
+        if budget is None:
+            os.environ.pop("FLASHSVD_AMD_PREFILL_TEMP_BYTES", None)
+        else:
+            os.environ["FLASHSVD_AMD_PREFILL_TEMP_BYTES"] = budget
+        times = []
+        with torch.no_grad():
+            for it in range(3):
+                cache = FlashSVDLegacySparseKVCache(model.config, max_batch_size=Bp, max_cache_len=Tp + 8, device="cuda", dtype=torch.bfloat16)
+                for li in range(L):             # the cache sizes a layer at its first use: do it before the measurement
+                    cache.ensure_layer_ranks(li, R, R)
+                torch.cuda.synchronize()
+                torch.cuda.reset_peak_memory_stats()
+                resident = torch.cuda.memory_allocated()
+                t0 = time.perf_counter()
+                out = model(ids, past_key_values=cache, cache_position=torch.arange(Tp), logits_to_keep=1)
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                transient = torch.cuda.max_memory_allocated() - resident
+                say(f"prefill {Bp} x {Tp} ({name}): {times[-1]:.3f} s")
+                del cache, out
+        gk = _ops.prefill_head_groups(Bp, Tp, Tp, H, H, Dh)   # under the budget of this leg
+        legs[name] = {"s": min(times[1:]), "cold_s": times[0], "transient_bytes_peak": int(transient), "kv_heads_per_pass": gk,
+                      "qkv_temporaries_bytes": 3 * Bp * Tp * gk * Dh * 2}
+    if saved_budget is None:
+        os.environ.pop("FLASHSVD_AMD_PREFILL_TEMP_BYTES", None)
+    else:
+        os.environ["FLASHSVD_AMD_PREFILL_TEMP_BYTES"] = saved_budget
+    t_pre = legs["default"]["s"]
     attn_flop_pre = 3 * 2.0 * Bp * Tp * R * H * Dh + 2 * 2.0 * Bp * H * Dh * Tp * (Tp + 1) / 2     # head expansion + causal attention
     flop_pre = L * (Bp * Tp * lin_flop_tok + attn_flop_pre) + 2.0 * Bp * d * V
-    prefill = {"batch": Bp, "prompt_len": Tp, "s": t_pre, "cold_s": times[0], "tok_s": Bp * Tp / t_pre, "flop": flop_pre,
+    prefill = {"batch": Bp, "prompt_len": Tp, "s": t_pre, "cold_s": legs["default"]["cold_s"], "tok_s": Bp * Tp / t_pre, "flop": flop_pre,
                "TFLOPs": flop_pre / t_pre / 1e12, "frac_of_bf16_mfma_peak": flop_pre / t_pre / peak,
-               # the prompt pass expands q and the context's K / V of a layer to HBM once and attends over them (the reference's
-               # kernel rebuilds K / V tiles per query tile and never writes them): what that costs in memory
-               "transient_bytes_peak": int(transient), "qkv_temporaries_bytes_per_layer": 3 * Bp * Tp * H * Dh * 2,
+               "transient_bytes_peak": legs["default"]["transient_bytes_peak"],
+               "kv_heads_per_pass": legs["default"]["kv_heads_per_pass"],
+               "qkv_temporaries_bytes": legs["default"]["qkv_temporaries_bytes"],
+               "head_groups_64MiB": legs["head_groups_64MiB"],
                "rank_cache_bytes_per_layer": 2 * Bp * (Tp + 8) * R * 2}
 
     # ---- leg 2: decode at batch 16, context 4096, rank-space cache

@@ -482,6 +482,22 @@ def _lowrank_expand_heads_impl(p, u, num_heads, head_dim, out, cos, sin, positio
     return out
 
 
+def prefill_head_groups(B: int, M: int, n_ctx: int, H: int, Hk: int, Dh: int, itemsize: int = 2) -> int:
+    """How many kv heads (with their query heads) the expand-then-attend prompt pass takes at a time.
+
+    The pass rebuilds q [B,M,H,Dh] and K, V [B,n_ctx,Hk,Dh] from rank coefficients into temporaries and runs the prompt
+    attention over them; nothing forces all heads to exist at once.  The largest group of kv heads whose temporaries
+    fit FLASHSVD_AMD_PREFILL_TEMP_BYTES (default 1 GiB) is taken, at least one; 0 or a negative budget means all heads in
+    one pass.  Groups cost a few per cent of the pass (8 x 2048 tokens at rank 1664: +4 % at 64 MiB, five kv heads per
+    group), so the default only bounds the temporaries of very long batches."""
+    import os
+    budget = int(float(os.getenv("FLASHSVD_AMD_PREFILL_TEMP_BYTES", str(1 << 30))))
+    if budget <= 0:
+        return Hk
+    per_kv_head = (B * M * (H // Hk) + 2 * B * n_ctx) * Dh * itemsize
+    return max(1, min(Hk, budget // max(per_kv_head, 1)))
+
+
 def lowrank_expand_heads_multi(items, *, head_dim: int, cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
                                positions: Optional[torch.Tensor] = None) -> None:
     """The q / k / v expansions of one prompt pass in one call (fsvd_lowrank_expand_heads_multi): ``items`` is a list of one

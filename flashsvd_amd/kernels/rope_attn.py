@@ -110,15 +110,9 @@ class FlashSVDRoPEAttention(nn.Module):
         def bias(b, heads):
             return None if b is None else b.reshape(-1)[: heads * dh].to(dt).contiguous()
 
-        q = torch.empty(B, M, H, dh, device=dev, dtype=dt)
-        k = torch.empty(B, M, Hk, dh, device=dev, dtype=dt)
-        v = torch.empty(B, M, Hk, dh, device=dev, dtype=dt)
-        hip_ops.lowrank_expand_heads_multi(
-            [dict(p=coeff(f.Pq), u=_as_linear_layout(f.Vq), num_heads=H, out=q, rotate=True, bias=bias(f.bq, H)),
-             dict(p=coeff(f.Pk), u=_as_linear_layout(f.Vk), num_heads=Hk, out=k, rotate=True, bias=bias(f.bk, Hk)),
-             dict(p=coeff(f.Pv), u=_as_linear_layout(f.Vv), num_heads=Hk, out=v, bias=bias(f.bv, Hk))],
-            head_dim=dh, cos=cos, sin=sin, positions=offs)
-
+        uq, uk, uv = _as_linear_layout(f.Vq), _as_linear_layout(f.Vk), _as_linear_layout(f.Vv)
+        Pq, Pk, Pv = coeff(f.Pq), coeff(f.Pk), coeff(f.Pv)
+        bq, bk, bv = bias(f.bq, H), bias(f.bk, Hk), bias(f.bv, Hk)
         pad = add = None
         if attention_mask is not None:
             if attention_mask.dim() == 2:
@@ -129,7 +123,31 @@ class FlashSVDRoPEAttention(nn.Module):
                 raise ValueError(f"Unsupported attention_mask shape: {attention_mask.shape}")
         if sliding_window_mask is not None:
             add = sliding_window_mask[:, 0].to(torch.float32).expand(B, M, M).contiguous()
-        return hip_ops.attn_prefill(q, k, v, causal=self.causal, pad_mask=pad, add_mask=add)
+        # q, K, V are rebuilt and consumed one group of kv heads at a time (hip_ops.prefill_head_groups): the temporaries of
+        # a group are reused by the next, so the pass never holds q / k / v of all heads (the activation-memory property of
+        # the reference's kernel, which rebuilds its tiles inside the attention loop, without its rebuild per query tile)
+        G = H // Hk
+        gk = hip_ops.prefill_head_groups(B, M, M, H, Hk, dh)
+        q = torch.empty(B, M, gk * G, dh, device=dev, dtype=dt)
+        k = torch.empty(B, M, gk, dh, device=dev, dtype=dt)
+        v = torch.empty_like(k)
+        out = torch.empty(B, M, H, dh, device=dev, dtype=dt)
+
+        def rows(t, r0, r1):
+            return None if t is None else t[r0:r1]
+
+        for k0 in range(0, Hk, gk):
+            k1 = min(k0 + gk, Hk)
+            nk, nq = k1 - k0, (k1 - k0) * G
+            hip_ops.lowrank_expand_heads_multi(
+                [dict(p=Pq[:, :, k0 * G:k1 * G], u=uq[k0 * G * dh:k1 * G * dh], num_heads=nq, out=q[:, :, :nq], rotate=True,
+                      bias=rows(bq, k0 * G * dh, k1 * G * dh)),
+                 dict(p=Pk[:, :, k0:k1], u=uk[k0 * dh:k1 * dh], num_heads=nk, out=k[:, :, :nk], rotate=True, bias=rows(bk, k0 * dh, k1 * dh)),
+                 dict(p=Pv[:, :, k0:k1], u=uv[k0 * dh:k1 * dh], num_heads=nk, out=v[:, :, :nk], bias=rows(bv, k0 * dh, k1 * dh))],
+                head_dim=dh, cos=cos, sin=sin, positions=offs)
+            hip_ops.attn_prefill(q[:, :, :nq], k[:, :, :nk], v[:, :, :nk], causal=self.causal, pad_mask=pad, add_mask=add,
+                                 out=out[:, :, k0 * G:k1 * G])
+        return out
 
 
 __all__ = ["FlashSVDRoPEAttention", "QKVFactors", "apply_rotary_bmhd", "rotate_half"]

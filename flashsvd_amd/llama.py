@@ -466,26 +466,36 @@ def _prefill_tokens_rank(self, x, cache, cache_position=None, *, norm_weight=Non
     mfma_ok = Dh == 128 and rq % 8 == 0 and rk % 8 == 0 and rv % 8 == 0 and T >= 16 \
         and os.getenv("FLASHSVD_AMD_PREFILL", "mfma").strip().lower() != "decode"
     if mfma_ok:
+        # q, K and V never exist for all heads at once: the heads are taken in groups whose temporaries stay inside a byte
+        # budget (hip_ops.prefill_head_groups), each group expanded and attended before the next reuses the buffers
         n_ctx = start + T
-        q = torch.empty(B, T, H, Dh, device=x.device, dtype=x.dtype)
-        kt = torch.empty(B, n_ctx, Hk, Dh, device=x.device, dtype=x.dtype)
+        G = H // Hk
+        gk = hip_ops.prefill_head_groups(B, T, n_ctx, H, Hk, Dh)
+        q = torch.empty(B, T, gk * G, Dh, device=x.device, dtype=x.dtype)
+        kt = torch.empty(B, n_ctx, gk, Dh, device=x.device, dtype=x.dtype)
         vt = torch.empty_like(kt)
         zero = torch.zeros(B, device=x.device, dtype=torch.int32)
         pos_q = torch.full((B,), start, device=x.device, dtype=torch.int32)
         wq, wk, wv = self.q_u_proj.weight, self.k_u_proj.weight, self.v_u_proj.weight
-        if start == 0:
-            hip_ops.lowrank_expand_heads_multi(
-                [dict(p=p[..., :rq], u=wq, num_heads=H, out=q, rotate=True),
-                 dict(p=p[..., rq:rq + rk], u=wk, num_heads=Hk, out=kt, rotate=True),
-                 dict(p=p[..., rq + rk:], u=wv, num_heads=Hk, out=vt)],
-                head_dim=Dh, cos=rope[0], sin=rope[1], positions=zero)
-        else:
-            hip_ops.lowrank_expand_heads(p[..., :rq], wq, num_heads=H, head_dim=Dh, out=q, cos=rope[0], sin=rope[1], positions=pos_q)
-            hip_ops.lowrank_expand_heads_multi(
-                [dict(p=pkc[:B, :n_ctx], u=wk, num_heads=Hk, out=kt, rotate=True),
-                 dict(p=pvc[:B, :n_ctx], u=wv, num_heads=Hk, out=vt)],
-                head_dim=Dh, cos=rope[0], sin=rope[1], positions=zero)
-        hip_ops.attn_prefill(q, kt, vt, q_pos0=pos_q, causal=True, out=a.view(B, T, H, Dh))
+        av = a.view(B, T, H, Dh)
+        for k0 in range(0, Hk, gk):
+            k1 = min(k0 + gk, Hk)
+            nk, nq = k1 - k0, (k1 - k0) * G
+            qg, kg, vg = q[:, :, :nq], kt[:, :, :nk], vt[:, :, :nk]
+            wqg, wkg, wvg = wq[k0 * G * Dh:k1 * G * Dh], wk[k0 * Dh:k1 * Dh], wv[k0 * Dh:k1 * Dh]
+            if start == 0:
+                hip_ops.lowrank_expand_heads_multi(
+                    [dict(p=p[..., :rq], u=wqg, num_heads=nq, out=qg, rotate=True),
+                     dict(p=p[..., rq:rq + rk], u=wkg, num_heads=nk, out=kg, rotate=True),
+                     dict(p=p[..., rq + rk:], u=wvg, num_heads=nk, out=vg)],
+                    head_dim=Dh, cos=rope[0], sin=rope[1], positions=zero)
+            else:
+                hip_ops.lowrank_expand_heads(p[..., :rq], wqg, num_heads=nq, head_dim=Dh, out=qg, cos=rope[0], sin=rope[1], positions=pos_q)
+                hip_ops.lowrank_expand_heads_multi(
+                    [dict(p=pkc[:B, :n_ctx], u=wkg, num_heads=nk, out=kg, rotate=True),
+                     dict(p=pvc[:B, :n_ctx], u=wvg, num_heads=nk, out=vg)],
+                    head_dim=Dh, cos=rope[0], sin=rope[1], positions=zero)
+            hip_ops.attn_prefill(qg, kg, vg, q_pos0=pos_q, causal=True, out=av[:, :, k0 * G:k1 * G])
         po = hip_ops.linear(a, self.o_v_proj.weight)
         return hip_ops.linear(po, self.o_u_proj.weight, residual=residual)
     q = hip_ops.linear(p[..., :rq].contiguous(), self.q_u_proj.weight).view(B, T, H, Dh)

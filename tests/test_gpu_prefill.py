@@ -44,6 +44,37 @@ def test_rope_attention_module_vs_oracle(B, H, Hk, M, R, shared):
     assert_close_bf16(out, ref, "prefill", **bounds(ref))
 
 
+@pytest.mark.parametrize("H,Hk,shared", [(8, 8, True), (8, 2, False)])
+def test_rope_attention_in_head_groups_gives_the_same_bits(monkeypatch, H, Hk, shared):
+    """q, K, V are rebuilt and attended one group of kv heads at a time when their temporaries would exceed the byte budget
+    (FLASHSVD_AMD_PREFILL_TEMP_BYTES); a head's result does not depend on which heads share its pass.  Biases, a padding
+    mask and grouped queries included; budgets that give groups of one, of three (a ragged last group) and all heads."""
+    from flashsvd_amd import hip_ops
+    from flashsvd_amd.kernels.rope_attn import FlashSVDRoPEAttention, QKVFactors
+    B, M, R, dh = 2, 200, 64, 128
+    Pq, Pk, Pv, Vq, Vk, Vv = _factors(B, H, Hk, M, R, dh, shared, seed=30)
+    bq = rand_bf16(H * dh, std=0.1, seed=40)
+    bk = bv = None
+    if H == Hk:
+        bk, bv = rand_bf16(H * dh, std=0.1, seed=41), rand_bf16(H * dh, std=0.1, seed=42)
+    pad = torch.ones(B, M, dtype=torch.long)
+    pad[1, :5] = 0
+    mod = FlashSVDRoPEAttention(H, dh, _Rot(dh))
+    g = [t.cuda() for t in (Pq, Pk, Pv, Vq, Vk, Vv)]
+    f = QKVFactors(*g, bq=bq.cuda(), bk=None if bk is None else bk.cuda(), bv=None if bv is None else bv.cuda())
+    per_kv_head = (B * M * (H // Hk) + 2 * B * M) * dh * 2
+    outs = {}
+    for name, budget in (("all", 0), ("one", 1), ("three", 3 * per_kv_head)):
+        monkeypatch.setenv("FLASHSVD_AMD_PREFILL_TEMP_BYTES", str(budget))
+        want = {"all": Hk, "one": 1, "three": min(3, Hk)}[name]
+        assert hip_ops.prefill_head_groups(B, M, M, H, Hk, dh) == want
+        outs[name] = mod(f, pad.cuda(), torch.arange(M, device="cuda")[None]).cpu()
+    assert torch.equal(outs["all"], outs["one"]) and torch.equal(outs["all"], outs["three"])
+    cos, sin = O.rope_tables(M, dh, dtype=BF16)
+    ref = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin, bq=bq, bk=bk, bv=bv, pad_mask=pad)
+    assert_close_bf16(outs["one"], ref, "prefill in head groups", **bounds(ref))
+
+
 @pytest.mark.parametrize("M", [70, 150])     # 64-query kernel / 128-query kernel with LDS-shared tiles
 def test_rope_attention_masks_biases_positions(M):
     from flashsvd_amd.kernels.rope_attn import FlashSVDRoPEAttention, QKVFactors
