@@ -231,30 +231,27 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
   for (; s0 + SPB < c.nsteps; s0 += SPB) batch(s0, std::true_type{});
   if (s0 < c.nsteps) batch(s0, std::false_type{});
 }
-// A leading phase (FSVD_PF_LEAD): a slab whose input this workgroup staged long ago is streamed in front of the next
-// phase's slab as one run of the window - the refills of its last batch already fetch the first pieces of the main
-// slab, so the request never pauses between the two, and the main phase polls for its input only after this stream, when
-// the producers have long published.  Every step is full and the steps are a multiple of kU (host-checked), so the
-// window slots come out holding steps 0 .. kU-1 of the main slab in order.
-__device__ __forceinline__ void lead_stream(const GemvCtx& a, const GemvCtx& b, uint32_t m_kp, u32x4_t (&R)[kU], const uint16_t* xs,
-                                            float* cp) {
+// A leading phase (FSVD_PF_LEAD): a slab whose input this workgroup staged long ago (it sits at an offset of the staging
+// area that nothing has overwritten since) is streamed in an iteration of its own that neither polls nor publishes: the
+// sums stay in the partial buffer, the window request at the end of the iteration fetches the first pieces of the phase
+// behind it, and that phase - which polls for its input only now, when the producers have long published - puts its own
+// partial sums behind these and publishes both.  Every step is full and the steps are a multiple of kU (host-checked).
+__device__ __forceinline__ void lead_stream(const GemvCtx& a, uint32_t m_kp, u32x4_t (&R)[kU], const uint16_t* xs, float* cp) {
   const uint32_t tid = threadIdx.x;
-  const uint32_t lastB = (uint32_t)(b.pps - 1);
   const int nA = a.nsteps;
   const int row = (int)__umulhi(tid, m_kp);     // tid / kp
   int kofs = (int)tid - row * a.kp;             // tid % kp
   const bool lead = (tid & 15) == 0;
-  // one batch; TAIL: the last one, whose refills are steps 0 .. kU-1 of the main slab (a copy of the body rather than a
-  // choice of base per load: with a branch in the loop the compiler waits for every load at the top of a batch)
-  auto batch = [&](int s0, auto tail) {
-    constexpr bool TAIL = decltype(tail)::value;
+  // one batch; the last one issues no loads (a copy of the body rather than a condition per load: with a branch in the
+  // loop the compiler waits for every load at the top of a batch)
+  auto batch = [&](int s0, auto refill) {
+    constexpr bool REFILL = decltype(refill)::value;
     float d[kU];
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
       const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xs + kofs * 8);
       d[u] = dot8_bf16(R[u], xv, 0.f);
-      if (TAIL) R[u] = ld_stream(b.base0, min((uint32_t)(u * kT) + tid, lastB) << 4);
-      else R[u] = ld_stream(a.base0, ((uint32_t)((s0 + u + kU) * kT) + tid) << 4);
+      if (REFILL) R[u] = ld_stream(a.base0, ((uint32_t)((s0 + u + kU) * kT) + tid) << 4);
       d[u] = row16_sum(d[u]);
       kofs += a.dk;
       kofs = kofs >= a.kp ? kofs - a.kp : kofs;
@@ -265,8 +262,8 @@ __device__ __forceinline__ void lead_stream(const GemvCtx& a, const GemvCtx& b, 
     }
   };
   int s0 = 0;
-  for (; s0 + kU < nA; s0 += kU) batch(s0, std::false_type{});
-  batch(s0, std::true_type{});
+  for (; s0 + kU < nA; s0 += kU) batch(s0, std::true_type{});
+  batch(s0, std::false_type{});
 }
 // ---------------------------------------------------------------------------------------------
 // the same walk over group-wise int4 weights: a 16-byte piece is 32 columns, 8 consecutive lanes form a chunk of
@@ -668,24 +665,22 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
   uint32_t dvA = desc_fetch(phases, 0, nph), dvB = dvA;   // descriptors of phase p and p+1
 
   // Iteration p: finish phase p (its first weights were requested one iteration earlier), publish its
-  // outputs, request the first weights of phase p+1.  A leading phase (FSVD_PF_LEAD) and the phase behind it are one
-  // iteration: the leading slab is streamed first, then the main phase runs as usual.
-  for (int p = -1; p < nph;) {
+  // outputs, request the first weights of phase p+1.  (A leading phase, FSVD_PF_LEAD, only streams: its sums wait in
+  // the partial buffer for the epilogue of the phase behind it.)
+  int lead_chunks = 0;                     // chunk partials a leading phase left for this iteration's epilogue
+  uint32_t dvL = dvA;                      // and its descriptor
+  for (int p = -1; p < nph; ++p) {
     const uint32_t dvC = desc_fetch(phases, p + 2, nph);   // needed one iteration from now
-    const uint32_t dvD = CX ? desc_fetch(phases, p + 3, nph) : dvC;
-    const bool lead = CX && p >= 0 && DF_I(dvA, type) == FSVD_PH_GEMV && (DF_I(dvA, flags) & FSVD_PF_LEAD) != 0;
-    const uint32_t dvF = dvA;                              // the leading phase, when there is one
-    const uint32_t dv = lead ? dvB : dvA;                  // the phase this iteration completes
-    const uint32_t dvN = lead ? dvC : dvB;                 // the phase whose first window it requests
-    const int pm = lead ? p + 1 : p;
-    const int type = p < 0 ? -1 : DF_I(dv, type);
+    const uint32_t dv = dvA;
+    const int pm = p;
+    int type = p < 0 ? -1 : DF_I(dv, type);
     unsigned long long* tr = nullptr;
     if (TRACE && p >= 0 && tid == 0 && (w % trace_stride) == 0) {
-      tr = trace + ((size_t)(w / trace_stride) * nph + pm) * 4;
+      tr = trace + ((size_t)(w / trace_stride) * nph + p) * 4;
       tr[0] = wall_clock64();
     }
-    GemvCtx gc, fc;
-    float* cpm = cp;                       // chunk partials of the main phase (behind those of a leading phase)
+    GemvCtx gc;
+    float* cpm = cp + lead_chunks;         // chunk partials of this phase (behind those of a leading phase)
     AttnWork aw;
     uint32_t resid = 0;
     int rows0 = 0x7fffffff;                // GEMV: first row of the fp32 group
@@ -693,22 +688,19 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     // addresses of the next phase's first window, worked out now (behind the wait for this phase's input) so that the
     // request after publication is nothing but the loads
     uint64_t nxt[kU], nxt_sz[kSzLoads];
-    window_addresses<Q4>(dvN, w, pos, reinterpret_cast<uint64_t>(phases), nxt, nxt_sz);
+    window_addresses<Q4>(dvB, w, pos, reinterpret_cast<uint64_t>(phases), nxt, nxt_sz);
 
     // ------------------------------------------------------------------ stage + stream
-    if (CX && lead) {
-      gemv_ctx<false>(dvF, w, fc);
+    if (CX && type == FSVD_PH_GEMV && (DF_I(dv, flags) & FSVD_PF_LEAD) != 0) {
       gemv_ctx<false>(dv, w, gc);
       // the epilogue of the previous phase may still be reading the partial buffer in another wave (its LDS reads are
       // complete by the time that wave's stores have been issued, i.e. before it arrives here)
       __builtin_amdgcn_s_barrier();
-      lead_stream(fc, gc, desc_u32(dvF, FSVD_DW(m_kp)), R, xs + fc.xoff, cp);
-      cpm = cp + (fc.pps >> 4);
-      if (TRACE && tr) {                   // the leading phase: entered, (nothing staged), streamed, (published with the main phase)
-        unsigned long long* trf = tr - 4;
-        trf[0] = trf[1] = tr[0];
-        trf[2] = trf[3] = tr[0] = wall_clock64();
-      }
+      lead_stream(gc, desc_u32(dv, FSVD_DW(m_kp)), R, xs + gc.xoff, cp);
+      lead_chunks = gc.pps >> 4;
+      dvL = dv;
+      if (TRACE && tr) tr[1] = tr[0];      // nothing staged
+      type = -2;                           // no staging, no epilogue: on to the window request
     }
     if (type == FSVD_PH_GEMV) {
       gemv_ctx<Q4>(dv, w, gc);
@@ -928,14 +920,17 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           if (live) st_tag16(out, gc.r0 + t, tout, f32_to_bf16_bits(v));
         }
       }
-      if (CX && lead) {
-        // the rows of the leading phase: unrounded sums, taken by the lane groups from the top of the workgroup down
-        // while those from the bottom up run the main epilogue
+      if (CX && lead_chunks != 0) {
+        // the rows of the leading phase in front of this one: unrounded sums, taken by the lane groups from the top of the
+        // workgroup down while those from the bottom up run this phase's epilogue
+        GemvCtx fc;
+        gemv_ctx<false>(dvL, w, fc);
         const int t = kT / 8 - 1 - grp;
         if (t < fc.srows) {
           const float v = row_sum8(cp, t, fc.kp >> 4);
-          if (lead8) st_tag64(DF_P(dvF, out1), fc.r0 + t, DF_TAG32(dvF, out1, epoch), __float_as_uint(v));
+          if (lead8) st_tag64(DF_P(dvL, out1), fc.r0 + t, DF_TAG32(dvL, out1, epoch), __float_as_uint(v));
         }
+        lead_chunks = 0;
       }
       // no barrier here: the next phase writes cp only after its staging barrier (a leading phase: after a barrier of
       // its own), which every wave reaches after this epilogue
@@ -1065,15 +1060,8 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       }
     }
     if (TRACE && tr) tr[3] = wall_clock64();
-    if (CX && lead) {
-      dvA = dvC;
-      dvB = dvD;
-      p += 2;
-    } else {
-      if (p >= 0) dvA = dvB;   // iteration -1 already holds descriptor 0 in both
-      dvB = dvC;
-      ++p;
-    }
+    if (p >= 0) dvA = dvB;   // iteration -1 already holds descriptor 0 in both
+    dvB = dvC;
   }
   // Every workgroup read the state before it produced anything, and workgroup 0 cannot get here before
   // it has consumed data from all the others, so bumping the epoch now cannot be seen by this launch.

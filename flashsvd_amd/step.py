@@ -408,9 +408,10 @@ class PersistentDecoder:
         Where the two moved products (25 MB each at the 7B shape) run: as *leading phases* (``self.leading``) when a
         workgroup's share of each fills whole windows of loads and the staging area can keep the hidden state that long -
         ``[gate_v; up_v]' x`` is then streamed in front of o_v and the next layer's ``[q_v; k_v; v_v]' x2`` in front of
-        down_v, in one run of loads with the slab behind them, so that neither pays a pipeline drain of its own and o_v /
-        down_v poll for their input when it has long been published; otherwise as phases of their own behind the
-        expansion and behind the pair (the older arrangement, FLASHSVD_AMD_STEP_LEAD=0 forces it).  Same sums, same bits.
+        down_v, in iterations that neither poll nor publish (the sums wait in the workgroup's partial buffer and leave
+        with o_v's / down_v's), so that o_v / down_v poll for their input when it has long been published; otherwise as
+        phases of their own behind the expansion and behind the pair (the older arrangement, FLASHSVD_AMD_STEP_LEAD=0
+        forces it).  Same sums, same bits.
 
         Arithmetic: the hidden states take the same roundings as in the ten-phase form; the rank coefficients are formed
         from the unrounded residual sum and rounded once (the ten-phase form rounds the hidden state, the normalised

@@ -323,11 +323,12 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
                           /* bf16 hidden state they were taken from: staged input = bf16(in * rsqrt(mean(in2^2) +  */
                           /* fparam)) at 0, and in2 itself, unscaled, at in2_off for a following NOWAIT phase     */
 #define FSVD_PF_SPLIT 4   /* two row groups with their own epilogues and outputs, see rows0                       */
-#define FSVD_PF_LEAD 8    /* with FSVD_PF_NOWAIT, on a single-matrix FSVD_EP_F32 phase: its slab is streamed in     */
-                          /* front of the NEXT phase's slab as one run of loads (its input is a vector that an      */
-                          /* earlier FSVD_PF_STAGE2 staging left at in_off and nothing has overwritten since); the   */
-                          /* next phase, a plain single-matrix bf16 GEMV, polls for its own input only behind that   */
-                          /* stream, and the two publish together.  The slab must fill whole windows of loads.      */
+#define FSVD_PF_LEAD 8    /* with FSVD_PF_NOWAIT, on a single-matrix FSVD_EP_F32 phase: the phase only streams (its   */
+                          /* input is a vector that an earlier FSVD_PF_STAGE2 staging left at in_off and nothing has  */
+                          /* overwritten since); it neither polls nor publishes, its sums wait in the workgroup's     */
+                          /* partial buffer, and the NEXT phase - a plain single-matrix bf16 GEMV, which polls for    */
+                          /* its own input only behind that stream - publishes them with its own.  The slab must     */
+                          /* fill whole windows of loads.                                                            */
 
 typedef struct fsvd_tagbuf {
   void* ptr;              /* uint32 [len] (bf16 payload) or uint64 [len] (fp32 / candidate payload)           */
