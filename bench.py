@@ -401,6 +401,7 @@ def run_lowrank(args):
             us_c = e0.elapsed_time(e1) * 1000.0 / args.steps
             prof = cdec.phase_profile(32)
             res["persistent_composed"] = dict(tok_s=1e6 / us_c, kernel_us_per_launch=us_c, phases=cdec.nph, leading_phases=bool(cdec.leading),
+                                              traffic=_traffic("decode_step_kernel_composed"),   # measured HBM bytes per launch (1.08x the token's algorithmic bytes: the composed blocks)
                                               last_token=int(cdec.tokens()[-1]),
                                               phase_profile_us={k: {m: round(x, 2) for m, x in v.items()} for k, v in prof.items()})
             del cdec, scratch_c
