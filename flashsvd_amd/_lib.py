@@ -95,9 +95,9 @@ SIGNATURES = {
     "fsvd_version": (c_int, []),
     "fsvd_last_error": (c_char_p, []),
     "fsvd_linear": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_float, c_void_p, c_int64,
-                            c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+                            c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_swiglu_linear": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
-                                   c_int, c_int, c_int, c_int, c_int, c_void_p]),
+                                   c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_linear_q4": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p,
                                c_float, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "fsvd_dequant_q4": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
@@ -106,18 +106,18 @@ SIGNATURES = {
     "fsvd_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                      c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int64, c_int64, c_int64,
-                                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_attn_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "fsvd_attn_decode_densekv": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                          c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int,
                                          c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
-                                         c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
+                                         c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "fsvd_attn_decode_densekv_static_max_bytes": (c_size_t, []),
     "fsvd_attn_decode_densekv_static": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                                 c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int,
                                                 c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
-                                                c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
-    "fsvd_rmsnorm": (c_int, [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int, c_int, c_void_p]),
+                                                c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
+    "fsvd_rmsnorm": (c_int, [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "fsvd_attn_decode_rankkv": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
                                         c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                         c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
@@ -127,12 +127,12 @@ SIGNATURES = {
                                    c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_lowrank_expand_heads": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
                                           c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
-                                          c_int, c_void_p]),
+                                          c_int, c_int, c_void_p]),
     "fsvd_lowrank_expand_heads_multi": (c_int, [ctypes.POINTER(ExpandDesc), c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
-                                                c_void_p]),
+                                                c_int, c_void_p]),
     "fsvd_attn_prefill": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p,
                                   c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
-                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
+                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "fsvd_xw_linear_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "fsvd_xw_linear": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int,
                                c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -164,7 +164,7 @@ def _manual_llama_decode_step(model, input_ids: torch.Tensor, *, past_key_values
         hidden = out
     norm = inner.norm
     head_w = getattr(model.lm_head, "weight", None)
-    if head_w is not None and head_w.is_cuda and head_w.dtype == torch.bfloat16 and hidden.dtype == torch.bfloat16 \
+    if head_w is not None and head_w.is_cuda and head_w.dtype in (torch.bfloat16, torch.float16) and hidden.dtype == head_w.dtype \
             and getattr(model.lm_head, "bias", None) is None and hasattr(norm, "variance_epsilon"):
         from . import hip_ops   # fused final norm + lm_head
         logits = hip_ops.linear(hidden[:, -1:, :], head_w, norm_weight=norm.weight, eps=norm.variance_epsilon)

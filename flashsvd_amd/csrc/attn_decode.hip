@@ -31,8 +31,9 @@ __device__ __forceinline__ void decode_work_item(int B, int H, int nsplit, int& 
 __device__ __forceinline__ void st_agent(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float ld_agent(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-template <int DH, int U>
+template <int DT, int DH, int U>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArgs a) {
+  typedef E16<DT> E;
   constexpr int LPK = DH / 8;                 // lanes that share one key (8 bf16 each)
   constexpr int KPB = kAttnThreads / LPK;     // keys per block pass
   constexpr int CH = KPB * U;                 // keys in flight per workgroup
@@ -55,16 +56,16 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
   // query chunk (optionally rotated at position seqlens[b], fp32 math, one rounding)
   const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)h * a.sq_h;
   if (tid < DH / 2) {
-    float x0 = bf16_bits_to_f32(qp[tid]), x1 = bf16_bits_to_f32(qp[tid + DH / 2]);
+    float x0 = E::val(qp[tid]), x1 = E::val(qp[tid + DH / 2]);
     if (a.cos) {
       const int tp = min(max(a.seqlens[b], 0), a.rope_len - 1);
-      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * (DH / 2) + tid]);
-      const float sn = bf16_bits_to_f32(a.sin[(int64_t)tp * (DH / 2) + tid]);
+      const float c = E::val(a.cos[(int64_t)tp * (DH / 2) + tid]);
+      const float sn = E::val(a.sin[(int64_t)tp * (DH / 2) + tid]);
       const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
       x0 = r0; x1 = r1;
     }
-    qs[tid] = (uint16_t)f32_to_bf16_bits(x0);
-    qs[tid + DH / 2] = (uint16_t)f32_to_bf16_bits(x1);
+    qs[tid] = (uint16_t)E::bits(x0);
+    qs[tid + DH / 2] = (uint16_t)E::bits(x1);
   }
   const int part = tid % LPK, slot = tid / LPK;
   const uint16_t* kbase = a.k_cache + (int64_t)b * a.sc_b + (int64_t)hk * a.sc_h + part * 8;
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
     float lmax = -INFINITY;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      float d = dot8_bf16(kv[u], qv, 0.f);
+      float d = E::dot8(kv[u], qv, 0.f);
       d += dpp_f32<0xB1>(d);
       d += dpp_f32<0x4E>(d);
       d += dpp_f32<0x141>(d);
@@ -116,10 +117,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
     for (int u = 0; u < U; ++u) {
       const float p = (sc[u] == -INFINITY) ? 0.f : __expf(sc[u] - m_new);
       psum += p;
-      acc[0] += p * bf16_lo(vv[u].x); acc[1] += p * bf16_hi(vv[u].x);
-      acc[2] += p * bf16_lo(vv[u].y); acc[3] += p * bf16_hi(vv[u].y);
-      acc[4] += p * bf16_lo(vv[u].z); acc[5] += p * bf16_hi(vv[u].z);
-      acc[6] += p * bf16_lo(vv[u].w); acc[7] += p * bf16_hi(vv[u].w);
+      acc[0] += p * E::lo(vv[u].x); acc[1] += p * E::hi(vv[u].x);
+      acc[2] += p * E::lo(vv[u].y); acc[3] += p * E::hi(vv[u].y);
+      acc[4] += p * E::lo(vv[u].z); acc[5] += p * E::hi(vv[u].z);
+      acc[6] += p * E::lo(vv[u].w); acc[7] += p * E::hi(vv[u].w);
     }
     l_thr = l_thr * alpha + (part == 0 ? psum : 0.f);
     m_run = m_new;
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
 
   uint16_t* outp = a.out + (int64_t)b * a.so_b + (int64_t)h * a.so_h;
   if (a.nsplit == 1) {
-    if (tid < DH) outp[tid] = (uint16_t)f32_to_bf16_bits(l > 0.f ? o / l : 0.f);
+    if (tid < DH) outp[tid] = (uint16_t)E::bits(l > 0.f ? o / l : 0.f);
     return;
   }
   float* part_ws = a.ws_part + ((int64_t)(b * a.H + h) * a.nsplit) * (DH + 2);
@@ -187,7 +188,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
         den += w * li[u];
       }
     }
-    outp[tid] = (uint16_t)f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
+    outp[tid] = (uint16_t)E::bits(den > 0.f ? num / den : 0.f);
   }
   if (tid == 0) __hip_atomic_store(&a.ws_count[b * a.H + h], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -196,8 +197,9 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(AttnDecodeArg
 // scored against the G queries (with one workgroup per query head every head of a group re-reads its kv head's rows from
 // L2); running maximum, sum and accumulators per query head; the heads' partials and merges go one after the other
 // through the same LDS block and the same last-arriver protocol as above.  G divides H / Hk.
-template <int DH, int U, int G>
+template <int DT, int DH, int U, int G>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_gqa_kernel(AttnDecodeArgs a) {
+  typedef E16<DT> E;
   constexpr int LPK = DH / 8, KPB = kAttnThreads / LPK, CH = KPB * U;
   static_assert(G * DH / 2 <= kAttnThreads, "one thread per rotation pair of every query of the group");
   __shared__ __align__(16) float accs[KPB * DH];
@@ -219,16 +221,16 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_gqa_kernel(AttnDecod
   if (tid < G * (DH / 2)) {
     const int g = tid / (DH / 2), d = tid % (DH / 2);
     const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)(h0 + g) * a.sq_h;
-    float x0 = bf16_bits_to_f32(qp[d]), x1 = bf16_bits_to_f32(qp[d + DH / 2]);
+    float x0 = E::val(qp[d]), x1 = E::val(qp[d + DH / 2]);
     if (a.cos) {
       const int tp = min(max(a.seqlens[b], 0), a.rope_len - 1);
-      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * (DH / 2) + d]);
-      const float sn = bf16_bits_to_f32(a.sin[(int64_t)tp * (DH / 2) + d]);
+      const float c = E::val(a.cos[(int64_t)tp * (DH / 2) + d]);
+      const float sn = E::val(a.sin[(int64_t)tp * (DH / 2) + d]);
       const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
       x0 = r0; x1 = r1;
     }
-    qs[g][d] = (uint16_t)f32_to_bf16_bits(x0);
-    qs[g][d + DH / 2] = (uint16_t)f32_to_bf16_bits(x1);
+    qs[g][d] = (uint16_t)E::bits(x0);
+    qs[g][d + DH / 2] = (uint16_t)E::bits(x1);
   }
   const int part = tid % LPK, slot = tid / LPK;
   const uint16_t* kbase = a.k_cache + (int64_t)b * a.sc_b + (int64_t)hk * a.sc_h + part * 8;
@@ -263,7 +265,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_gqa_kernel(AttnDecod
       float lmax = -INFINITY;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        float d = dot8_bf16(kv[u], qv, 0.f);
+        float d = E::dot8(kv[u], qv, 0.f);
         d += dpp_f32<0xB1>(d);
         d += dpp_f32<0x4E>(d);
         d += dpp_f32<0x141>(d);
@@ -287,10 +289,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_gqa_kernel(AttnDecod
       for (int u = 0; u < U; ++u) {
         const float p = (sc[g][u] == -INFINITY) ? 0.f : __expf(sc[g][u] - m_new);
         psum += p;
-        acc[g][0] += p * bf16_lo(vv[u].x); acc[g][1] += p * bf16_hi(vv[u].x);
-        acc[g][2] += p * bf16_lo(vv[u].y); acc[g][3] += p * bf16_hi(vv[u].y);
-        acc[g][4] += p * bf16_lo(vv[u].z); acc[g][5] += p * bf16_hi(vv[u].z);
-        acc[g][6] += p * bf16_lo(vv[u].w); acc[g][7] += p * bf16_hi(vv[u].w);
+        acc[g][0] += p * E::lo(vv[u].x); acc[g][1] += p * E::hi(vv[u].x);
+        acc[g][2] += p * E::lo(vv[u].y); acc[g][3] += p * E::hi(vv[u].y);
+        acc[g][4] += p * E::lo(vv[u].z); acc[g][5] += p * E::hi(vv[u].z);
+        acc[g][6] += p * E::lo(vv[u].w); acc[g][7] += p * E::hi(vv[u].w);
       }
       l_thr[g] = l_thr[g] * alpha + (part == 0 ? psum : 0.f);
       m_run[g] = m_new;
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_gqa_kernel(AttnDecod
     }
     uint16_t* outp = a.out + (int64_t)b * a.so_b + (int64_t)h * a.so_h;
     if (a.nsplit == 1) {
-      if (tid < DH) outp[tid] = (uint16_t)f32_to_bf16_bits(l > 0.f ? o / l : 0.f);
+      if (tid < DH) outp[tid] = (uint16_t)E::bits(l > 0.f ? o / l : 0.f);
       __syncthreads();                             // accs and red are read out before the next head refills them
       continue;
     }
@@ -361,7 +363,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_gqa_kernel(AttnDecod
             den += w * li[u];
           }
         }
-        outp[tid] = (uint16_t)f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
+        outp[tid] = (uint16_t)E::bits(den > 0.f ? num / den : 0.f);
       }
       if (tid == 0) __hip_atomic_store(&a.ws_count[b * a.H + h], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -370,7 +372,9 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_gqa_kernel(AttnDecod
 }
 
 // rotate k_new at position seqlens[b] (fp32 math, one rounding) and write k/v into the caches
+template <int DT>
 __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
+  typedef E16<DT> E;
   const int half = a.Dh >> 1;
   const int total = a.B * a.Hk * half;
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
@@ -379,17 +383,17 @@ __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
     if (pos < 0 || pos >= a.S) continue;
     const uint16_t* kp = a.k_new + (int64_t)b * a.sk_b + (int64_t)hk * a.sk_h;
     const uint16_t* vp = a.v_new + (int64_t)b * a.sv_b + (int64_t)hk * a.sv_h;
-    float x0 = bf16_bits_to_f32(kp[d]), x1 = bf16_bits_to_f32(kp[d + half]);
+    float x0 = E::val(kp[d]), x1 = E::val(kp[d + half]);
     if (a.cos) {
       const int tp = min(pos, a.rope_len - 1);
-      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * half + d]);
-      const float s = bf16_bits_to_f32(a.sin[(int64_t)tp * half + d]);
+      const float c = E::val(a.cos[(int64_t)tp * half + d]);
+      const float s = E::val(a.sin[(int64_t)tp * half + d]);
       const float r0 = x0 * c - x1 * s, r1 = x0 * s + x1 * c;
       x0 = r0; x1 = r1;
     }
     const int64_t off = (int64_t)b * a.sc_b + (int64_t)pos * a.sc_s + (int64_t)hk * a.sc_h;
-    a.k_cache[off + d] = (uint16_t)f32_to_bf16_bits(x0);
-    a.k_cache[off + d + half] = (uint16_t)f32_to_bf16_bits(x1);
+    a.k_cache[off + d] = (uint16_t)E::bits(x0);
+    a.k_cache[off + d + half] = (uint16_t)E::bits(x1);
     a.v_cache[off + d] = vp[d];
     a.v_cache[off + d + half] = vp[d + half];
   }
@@ -397,7 +401,17 @@ __global__ __launch_bounds__(256) void kv_append_kernel(KvAppendArgs a) {
 
 size_t attn_decode_ws_floats(int B, int H, int nsplit, int Dh) { return (size_t)B * H * nsplit * (Dh + 2); }
 
+template <int DT>
+static void launch_attn_decode_t(const AttnDecodeArgs& a, int G, hipStream_t st) {
+  dim3 grid(a.B * (a.H / G) * a.nsplit);
+  if (G == 4) hipLaunchKernelGGL((attn_decode_gqa_kernel<DT, 128, 8, 4>), grid, dim3(kAttnThreads), 0, st, a);
+  else if (G == 2) hipLaunchKernelGGL((attn_decode_gqa_kernel<DT, 128, 8, 2>), grid, dim3(kAttnThreads), 0, st, a);
+  else if (a.Dh == 128) hipLaunchKernelGGL((attn_decode_kernel<DT, 128, 8>), grid, dim3(kAttnThreads), 0, st, a);
+  else hipLaunchKernelGGL((attn_decode_kernel<DT, 64, 4>), grid, dim3(kAttnThreads), 0, st, a);
+}
+
 int launch_attn_decode(const AttnDecodeArgs& a, hipStream_t st) {
+  if (a.dt != 0 && a.dt != 1) { set_last_error("fsvd_attn_decode_densekv: dtype code %d (bf16 = 0 and fp16 = 1 are served)", a.dt); return kErrBadDtype; }
   if (a.B <= 0 || a.H <= 0 || a.Hk <= 0 || a.H % a.Hk != 0 || a.S <= 0 || a.nsplit <= 0) {
     set_last_error("fsvd_attn_decode_densekv: bad shape B=%d H=%d Hk=%d S=%d nsplit=%d", a.B, a.H, a.Hk, a.S, a.nsplit);
     return kErrBadShape;
@@ -423,11 +437,8 @@ int launch_attn_decode(const AttnDecodeArgs& a, hipStream_t st) {
     if (rep % 4 == 0 && (int64_t)a.B * (a.H / 4) * a.nsplit >= 512) G = 4;
     else if (rep % 2 == 0 && (int64_t)a.B * (a.H / 2) * a.nsplit >= 512) G = 2;
   }
-  dim3 grid(a.B * (a.H / G) * a.nsplit);
-  if (G == 4) hipLaunchKernelGGL((attn_decode_gqa_kernel<128, 8, 4>), grid, dim3(kAttnThreads), 0, st, a);
-  else if (G == 2) hipLaunchKernelGGL((attn_decode_gqa_kernel<128, 8, 2>), grid, dim3(kAttnThreads), 0, st, a);
-  else if (a.Dh == 128) hipLaunchKernelGGL((attn_decode_kernel<128, 8>), grid, dim3(kAttnThreads), 0, st, a);
-  else hipLaunchKernelGGL((attn_decode_kernel<64, 4>), grid, dim3(kAttnThreads), 0, st, a);
+  if (a.dt == 1) launch_attn_decode_t<1>(a, G, st);
+  else launch_attn_decode_t<0>(a, G, st);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("fsvd_attn_decode_densekv: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
@@ -436,7 +447,9 @@ int launch_attn_decode(const AttnDecodeArgs& a, hipStream_t st) {
 int launch_kv_append(const KvAppendArgs& a, hipStream_t st) {
   if (a.B <= 0 || a.Hk <= 0 || a.Dh <= 0 || (a.Dh & 1) || a.S <= 0) { set_last_error("fsvd_kv_append: bad shape"); return kErrBadShape; }
   const int total = a.B * a.Hk * (a.Dh / 2);
-  hipLaunchKernelGGL(kv_append_kernel, dim3((total + 255) / 256), dim3(256), 0, st, a);
+  if (a.dt != 0 && a.dt != 1) { set_last_error("fsvd_kv_append: dtype code %d (bf16 = 0 and fp16 = 1 are served)", a.dt); return kErrBadDtype; }
+  if (a.dt == 1) hipLaunchKernelGGL(kv_append_kernel<1>, dim3((total + 255) / 256), dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(kv_append_kernel<0>, dim3((total + 255) / 256), dim3(256), 0, st, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("fsvd_kv_append: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
   return kOk;

@@ -48,7 +48,7 @@ static inline uint16_t* u16(void* p) { return static_cast<uint16_t*>(p); }
 
 extern "C" {
 
-int fsvd_version(void) { return 100; }
+int fsvd_version(void) { return 101; }
 const char* fsvd_last_error(void) { return g_last_error; }
 
 int fsvd_set_workspace(void* ws, size_t bytes, void* stream) {
@@ -68,19 +68,19 @@ int fsvd_set_workspace(void* ws, size_t bytes, void* stream) {
 }
 
 int fsvd_linear(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* bias, const void* norm_w, float eps,
-                const void* res, int64_t ldres, void* y, int64_t ldy, int B, int N, int K, int cfg, void* stream) {
+                const void* res, int64_t ldres, void* y, int64_t ldy, int B, int N, int K, int cfg, int dtype, void* stream) {
   FSVD_REQUIRE_PTR(x, "fsvd_linear"); FSVD_REQUIRE_PTR(W, "fsvd_linear"); FSVD_REQUIRE_PTR(y, "fsvd_linear");
   if (ldx < K || ldw < K || ldy < N || (res && ldres < N)) {
     set_last_error("fsvd_linear: leading dimension smaller than the row (ldx=%lld ldw=%lld ldy=%lld ldres=%lld K=%d N=%d)",
                    (long long)ldx, (long long)ldw, (long long)ldy, (long long)ldres, K, N);
     return kErrBadShape;
   }
-  LinearArgs a{cu16(x), ldx, cu16(W), ldw, cu16(bias), cu16(norm_w), eps, cu16(res), ldres, u16(y), ldy, B, N, K};
+  LinearArgs a{cu16(x), ldx, cu16(W), ldw, cu16(bias), cu16(norm_w), eps, cu16(res), ldres, u16(y), ldy, B, N, K, dtype};
   return launch_linear(a, cfg, static_cast<hipStream_t>(stream));
 }
 
 int fsvd_swiglu_linear(const void* p, int64_t ldp, int64_t up_off, const void* gate_u, const void* up_u, int64_t ldw,
-                       void* h, int64_t ldh, int B, int D, int R, int mode, int cfg, void* stream) {
+                       void* h, int64_t ldh, int B, int D, int R, int mode, int cfg, int dtype, void* stream) {
   FSVD_REQUIRE_PTR(p, "fsvd_swiglu_linear"); FSVD_REQUIRE_PTR(gate_u, "fsvd_swiglu_linear");
   FSVD_REQUIRE_PTR(up_u, "fsvd_swiglu_linear"); FSVD_REQUIRE_PTR(h, "fsvd_swiglu_linear");
   if (up_off < 0 || ldp < up_off + R || ldw < R || ldh < D || (mode != 0 && mode != 1)) {
@@ -88,7 +88,7 @@ int fsvd_swiglu_linear(const void* p, int64_t ldp, int64_t up_off, const void* g
                    (long long)ldp, (long long)up_off, R, (long long)ldw, (long long)ldh, D, mode);
     return kErrBadShape;
   }
-  SwigluArgs a{cu16(p), ldp, up_off, cu16(gate_u), cu16(up_u), ldw, u16(h), ldh, B, D, R, mode};
+  SwigluArgs a{cu16(p), ldp, up_off, cu16(gate_u), cu16(up_u), ldw, u16(h), ldh, B, D, R, mode, dtype};
   return launch_swiglu(a, cfg, static_cast<hipStream_t>(stream));
 }
 
@@ -133,7 +133,7 @@ int fsvd_swiglu_linear_q4(const void* p, int64_t ldp, int64_t up_off, const void
 int fsvd_qkv_rope_append(const void* p, int64_t ldp, const void* q_u, int64_t ldq, const void* k_u, int64_t ldk,
                          const void* v_u, int64_t ldv, const void* cos, const void* sin, int rope_len,
                          const int32_t* positions, void* q_out, void* k_cache, void* v_cache, int64_t sc_b, int64_t sc_s,
-                         int64_t sc_h, int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int S, int cfg, void* stream) {
+                         int64_t sc_h, int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int S, int cfg, int dtype, void* stream) {
   const char* fn = "fsvd_qkv_rope_append";
   FSVD_REQUIRE_PTR(p, fn); FSVD_REQUIRE_PTR(q_u, fn); FSVD_REQUIRE_PTR(k_u, fn); FSVD_REQUIRE_PTR(v_u, fn);
   FSVD_REQUIRE_PTR(positions, fn); FSVD_REQUIRE_PTR(q_out, fn); FSVD_REQUIRE_PTR(k_cache, fn); FSVD_REQUIRE_PTR(v_cache, fn);
@@ -143,7 +143,7 @@ int fsvd_qkv_rope_append(const void* p, int64_t ldp, const void* q_u, int64_t ld
     return kErrBadShape;
   }
   QkvArgs a{cu16(p), ldp, cu16(q_u), ldq, cu16(k_u), ldk, cu16(v_u), ldv, cu16(cos), cu16(sin), rope_len, positions,
-            u16(q_out), u16(k_cache), u16(v_cache), sc_b, sc_s, sc_h, B, H, Hk, Dh, Rq, Rk, Rv, S};
+            u16(q_out), u16(k_cache), u16(v_cache), sc_b, sc_s, sc_h, B, H, Hk, Dh, Rq, Rk, Rv, S, dtype};
   return launch_qkv(a, cfg, static_cast<hipStream_t>(stream));
 }
 
@@ -160,7 +160,7 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h, void* k_
                              int64_t sc_s, int64_t sc_h, const void* k_new, int64_t sk_b, int64_t sk_h, const void* v_new, int64_t sv_b, int64_t sv_h,
                              const int32_t* cache_seqlens, int seqlen_add, const void* cos, const void* sin, int rope_len,
                              void* out, int64_t so_b, int64_t so_h, void* workspace, size_t workspace_bytes, int B, int H,
-                             int Hk, int Dh, int S, int nsplit, float scale, void* stream) {
+                             int Hk, int Dh, int S, int nsplit, float scale, int dtype, void* stream) {
   const char* fn = "fsvd_attn_decode_densekv";
   FSVD_REQUIRE_PTR(q, fn); FSVD_REQUIRE_PTR(k_cache, fn); FSVD_REQUIRE_PTR(v_cache, fn);
   FSVD_REQUIRE_PTR(cache_seqlens, fn); FSVD_REQUIRE_PTR(out, fn);
@@ -185,14 +185,14 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h, void* k_
   }
   if (k_new) {
     KvAppendArgs ka{cu16(k_new), cu16(v_new), sk_b, sk_h, sv_b, sv_h, u16(k_cache), u16(v_cache), sc_b, sc_s, sc_h,
-                    cache_seqlens, cu16(cos), cu16(sin), rope_len, B, Hk, Dh, S};
+                    cache_seqlens, cu16(cos), cu16(sin), rope_len, B, Hk, Dh, S, dtype};
     int rc = launch_kv_append(ka, st);
     if (rc != kOk) return rc;
     seqlen_add = 1;
   }
   AttnDecodeArgs a{cu16(q), sq_b, sq_h, cu16(k_cache), cu16(v_cache), sc_b, sc_s, sc_h, cache_seqlens, seqlen_add,
                    cu16(cos), cu16(sin), rope_len, u16(out), so_b, so_h, ws_part, ws_count, B, H, Hk, Dh, S, nsplit,
-                   scale > 0.f ? scale : 1.0f / sqrtf((float)Dh)};
+                   scale > 0.f ? scale : 1.0f / sqrtf((float)Dh), dtype};
   return launch_attn_decode(a, st);
 }
 
@@ -224,7 +224,7 @@ int fsvd_attn_decode_densekv_static(const void* q, int64_t sq_b, int64_t sq_h, v
                                     int64_t sc_s, int64_t sc_h, const void* k_new, int64_t sk_b, int64_t sk_h, const void* v_new,
                                     int64_t sv_b, int64_t sv_h, const int32_t* cache_seqlens, int seqlen_add, const void* cos,
                                     const void* sin, int rope_len, void* out, int64_t so_b, int64_t so_h, int B, int H, int Hk,
-                                    int Dh, int S, int nsplit, float scale, void* stream) {
+                                    int Dh, int S, int nsplit, float scale, int dtype, void* stream) {
   const char* fn = "fsvd_attn_decode_densekv_static";
   if (B <= 0 || H <= 0 || Dh <= 0 || nsplit <= 0) { set_last_error("%s: bad shape", fn); return kErrBadShape; }
   void* ws = nullptr;
@@ -247,12 +247,12 @@ int fsvd_attn_decode_densekv_static(const void* q, int64_t sq_b, int64_t sq_h, v
     if (e != hipSuccess) { set_last_error("%s: launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
   }
   return fsvd_attn_decode_densekv(q, sq_b, sq_h, k_cache, v_cache, sc_b, sc_s, sc_h, k_new, sk_b, sk_h, v_new, sv_b, sv_h, cache_seqlens,
-                                  seqlen_add, cos, sin, rope_len, out, so_b, so_h, ws, need, B, H, Hk, Dh, S, nsplit, scale, stream);
+                                  seqlen_add, cos, sin, rope_len, out, so_b, so_h, ws, need, B, H, Hk, Dh, S, nsplit, scale, dtype, stream);
 }
 
-int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, void* stream) {
+int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, int dtype, void* stream) {
   FSVD_REQUIRE_PTR(x, "fsvd_rmsnorm"); FSVD_REQUIRE_PTR(w, "fsvd_rmsnorm"); FSVD_REQUIRE_PTR(y, "fsvd_rmsnorm");
-  return launch_rmsnorm(cu16(x), ldx, cu16(w), eps, u16(y), ldy, rows, K, static_cast<hipStream_t>(stream));
+  return launch_rmsnorm(cu16(x), ldx, cu16(w), eps, u16(y), ldy, rows, K, dtype, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"
@@ -529,18 +529,18 @@ int fsvd_rankkv_append(const void* pk, int64_t ldpk, const void* pv, int64_t ldp
 int fsvd_lowrank_expand_heads(const void* p, int64_t sp_b, int64_t sp_m, int64_t sp_h, const void* u, int64_t ldu, const void* bias,
                               const void* cos, const void* sin, int rope_len, const int32_t* positions, void* y, int64_t sy_b,
                               int64_t sy_m, int64_t sy_h, int dst_by_position, int dst_rows, int B, int M, int heads, int Dh, int R,
-                              void* stream) {
+                              int dtype, void* stream) {
   const char* fn = "fsvd_lowrank_expand_heads";
   FSVD_REQUIRE_PTR(p, fn); FSVD_REQUIRE_PTR(u, fn); FSVD_REQUIRE_PTR(y, fn);
   if ((cos == nullptr) != (sin == nullptr) || (cos && rope_len <= 0)) { set_last_error("%s: cos/sin must both be set with rope_len > 0", fn); return kErrBadShape; }
   if (ldu < R || sy_h < Dh || dst_rows <= 0) { set_last_error("%s: inconsistent strides (ldu=%lld R=%d sy_h=%lld dst_rows=%d)", fn, (long long)ldu, R, (long long)sy_h, dst_rows); return kErrBadShape; }
   ExpandArgs a{cu16(p), sp_b, sp_m, sp_h, cu16(u), ldu, cu16(bias), cu16(cos), cu16(sin), rope_len, positions, u16(y), sy_b, sy_m,
-               sy_h, dst_by_position, dst_rows, B, M, heads, Dh, R};
+               sy_h, dst_by_position, dst_rows, B, M, heads, Dh, R, dtype};
   return launch_expand(a, static_cast<hipStream_t>(stream));
 }
 
 int fsvd_lowrank_expand_heads_multi(const fsvd_expand_desc* desc, int n, const void* cos, const void* sin, int rope_len,
-                                    const int32_t* positions, int B, int M, int Dh, void* stream) {
+                                    const int32_t* positions, int B, int M, int Dh, int dtype, void* stream) {
   const char* fn = "fsvd_lowrank_expand_heads_multi";
   FSVD_REQUIRE_PTR(desc, fn);
   if (n < 1 || n > 3) { set_last_error("%s: %d descriptors (1..3)", fn, n); return kErrBadShape; }
@@ -556,7 +556,7 @@ int fsvd_lowrank_expand_heads_multi(const fsvd_expand_desc* desc, int n, const v
     }
     a[k] = ExpandArgs{cu16(d.p), d.sp_b, d.sp_m, d.sp_h, cu16(d.u), d.ldu, cu16(d.bias), d.rotate ? cu16(cos) : nullptr,
                       d.rotate ? cu16(sin) : nullptr, rope_len, positions, u16(d.y), d.sy_b, d.sy_m, d.sy_h, d.dst_by_position,
-                      d.dst_rows, B, M, d.heads, Dh, d.R};
+                      d.dst_rows, B, M, d.heads, Dh, d.R, dtype};
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (expand_multi_apply(a, n)) {
@@ -576,12 +576,12 @@ int fsvd_lowrank_expand_heads_multi(const fsvd_expand_desc* desc, int n, const v
 int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h, const void* k, const void* v, int64_t sk_b,
                       int64_t sk_s, int64_t sk_h, const int32_t* q_pos0, const uint8_t* pad_mask, int64_t spm_b,
                       const float* add_mask, int64_t sam_b, int64_t sam_q, void* out, int64_t so_b, int64_t so_m, int64_t so_h,
-                      int B, int M, int H, int Hk, int Dh, int S, int causal, float scale, void* stream) {
+                      int B, int M, int H, int Hk, int Dh, int S, int causal, float scale, int dtype, void* stream) {
   const char* fn = "fsvd_attn_prefill";
   FSVD_REQUIRE_PTR(q, fn); FSVD_REQUIRE_PTR(k, fn); FSVD_REQUIRE_PTR(v, fn); FSVD_REQUIRE_PTR(out, fn);
   if (S <= 0 || (!q_pos0 && M > S)) { set_last_error("%s: %d queries do not fit %d cache rows", fn, M, S); return kErrBadShape; }
   PrefillAttnArgs a{cu16(q), sq_b, sq_m, sq_h, cu16(k), cu16(v), sk_b, sk_s, sk_h, q_pos0, pad_mask, spm_b, add_mask, sam_b, sam_q,
-                    u16(out), so_b, so_m, so_h, B, M, H, Hk, Dh, S, causal, scale > 0.f ? scale : 1.0f / sqrtf((float)Dh)};
+                    u16(out), so_b, so_m, so_h, B, M, H, Hk, Dh, S, causal, scale > 0.f ? scale : 1.0f / sqrtf((float)Dh), dtype};
   return launch_prefill_attn(a, static_cast<hipStream_t>(stream));
 }
 

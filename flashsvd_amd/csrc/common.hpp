@@ -52,6 +52,53 @@ __device__ __forceinline__ float dot8_bf16(const u32x4_t& w, const u32x4_t& x, f
   return acc;
 }
 
+// The 16-bit element types of the fused product kernels (dtype codes of the C ABI: 0 = bf16, 1 = fp16).  The kernels
+// move bit patterns; an element type says how a pattern widens to fp32, how fp32 rounds to it (nearest even, as
+// torch does) and which packed dot-product instruction multiplies it (fp32 accumulation in both).
+// frag_t / mfma: eight elements as a matrix-core operand and V_MFMA_F32_16X16X32_{BF16,F16}.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+template <int DT> struct E16;
+template <> struct E16<0> {
+  static constexpr int code = 0;
+  typedef bf16x8_t frag_t;
+  static __device__ __forceinline__ f32x4_t mfma(frag_t a, frag_t b, f32x4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ float lo(uint32_t packed) { return bf16_lo(packed); }
+  static __device__ __forceinline__ float hi(uint32_t packed) { return bf16_hi(packed); }
+  static __device__ __forceinline__ float val(uint32_t h) { return bf16_bits_to_f32(h); }      // pattern in the low 16 bits
+  static __device__ __forceinline__ uint32_t bits(float f) { return f32_to_bf16_bits(f); }
+  static __device__ __forceinline__ float rnd(float f) { return round_bf16(f); }
+  static __device__ __forceinline__ uint32_t pack2(float l, float h) { return pack_bf16x2(l, h); }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) { return dot2_bf16(a, b, acc); }
+  static __device__ __forceinline__ float dot8(const u32x4_t& w, const u32x4_t& x, float acc) { return dot8_bf16(w, x, acc); }
+};
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <> struct E16<1> {
+  static constexpr int code = 1;
+  typedef f16x8_t frag_t;
+  static __device__ __forceinline__ f32x4_t mfma(frag_t a, frag_t b, f32x4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ float val(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (unsigned short)h); }
+  static __device__ __forceinline__ float lo(uint32_t packed) { return val(packed & 0xffffu); }
+  static __device__ __forceinline__ float hi(uint32_t packed) { return val(packed >> 16); }
+  static __device__ __forceinline__ uint32_t bits(float f) {
+    return static_cast<uint32_t>(__builtin_bit_cast(unsigned short, static_cast<_Float16>(f)));
+  }
+  static __device__ __forceinline__ float rnd(float f) { return (float)static_cast<_Float16>(f); }
+  static __device__ __forceinline__ uint32_t pack2(float l, float h) { return bits(l) | (bits(h) << 16); }
+  // V_DOT2_F32_F16
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), acc, false);
+  }
+  static __device__ __forceinline__ float dot8(const u32x4_t& w, const u32x4_t& x, float acc) {
+    acc = dot2(w.x, x.x, acc);
+    acc = dot2(w.y, x.y, acc);
+    acc = dot2(w.z, x.z, acc);
+    acc = dot2(w.w, x.w, acc);
+    return acc;
+  }
+};
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));

@@ -15,9 +15,10 @@ constexpr int kWaves = kThreads / kWave;
 // stage the activation rows of one batch tile into LDS (packed bf16), optionally RMS-normed
 //   xs layout: [BATCH][Kp] bf16, Kp = K rounded up to 8
 // ---------------------------------------------------------------------------------------
-template <int BATCH>
+template <int DT, int BATCH>
 __device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int64_t ldx, int nb, int K, int Kp,
                                         const uint16_t* __restrict__ norm_w, float eps, uint16_t* xs, float* red) {
+  typedef E16<DT> E;
   const int tid = threadIdx.x;
   const bool vec = ((K & 7) == 0) && ((ldx & 7) == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
   for (int b = 0; b < BATCH; ++b) {
@@ -42,13 +43,13 @@ __device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int64_t 
     if (vnorm) {
       for (int k = tid * 8; k < K; k += kThreads * 8) {
         const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + k);
-        const float a0 = bf16_lo(v.x), a1 = bf16_hi(v.x), a2 = bf16_lo(v.y), a3 = bf16_hi(v.y);
-        const float a4 = bf16_lo(v.z), a5 = bf16_hi(v.z), a6 = bf16_lo(v.w), a7 = bf16_hi(v.w);
+        const float a0 = E::lo(v.x), a1 = E::hi(v.x), a2 = E::lo(v.y), a3 = E::hi(v.y);
+        const float a4 = E::lo(v.z), a5 = E::hi(v.z), a6 = E::lo(v.w), a7 = E::hi(v.w);
         ss += ((a0 * a0 + a1 * a1) + (a2 * a2 + a3 * a3)) + ((a4 * a4 + a5 * a5) + (a6 * a6 + a7 * a7));
       }
     } else {
       for (int k = tid; k < K; k += kThreads) {
-        float v = bf16_bits_to_f32(src[k]);
+        float v = E::val(src[k]);
         ss += v * v;
       }
     }
@@ -65,18 +66,18 @@ __device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int64_t 
         const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + k);
         const u32x4_t g = *reinterpret_cast<const u32x4_t*>(norm_w + k);
         u32x4_t o;
-        o.x = pack_bf16x2(bf16_lo(g.x) * round_bf16(bf16_lo(v.x) * rs), bf16_hi(g.x) * round_bf16(bf16_hi(v.x) * rs));
-        o.y = pack_bf16x2(bf16_lo(g.y) * round_bf16(bf16_lo(v.y) * rs), bf16_hi(g.y) * round_bf16(bf16_hi(v.y) * rs));
-        o.z = pack_bf16x2(bf16_lo(g.z) * round_bf16(bf16_lo(v.z) * rs), bf16_hi(g.z) * round_bf16(bf16_hi(v.z) * rs));
-        o.w = pack_bf16x2(bf16_lo(g.w) * round_bf16(bf16_lo(v.w) * rs), bf16_hi(g.w) * round_bf16(bf16_hi(v.w) * rs));
+        o.x = E::pack2(E::lo(g.x) * E::rnd(E::lo(v.x) * rs), E::hi(g.x) * E::rnd(E::hi(v.x) * rs));
+        o.y = E::pack2(E::lo(g.y) * E::rnd(E::lo(v.y) * rs), E::hi(g.y) * E::rnd(E::hi(v.y) * rs));
+        o.z = E::pack2(E::lo(g.z) * E::rnd(E::lo(v.z) * rs), E::hi(g.z) * E::rnd(E::hi(v.z) * rs));
+        o.w = E::pack2(E::lo(g.w) * E::rnd(E::lo(v.w) * rs), E::hi(g.w) * E::rnd(E::hi(v.w) * rs));
         *reinterpret_cast<u32x4_t*>(dst + k) = o;
       }
     } else {
       for (int k = tid; k < Kp; k += kThreads) {
         uint16_t o = 0;
         if (k < K) {
-          float v = round_bf16(bf16_bits_to_f32(src[k]) * rs);
-          o = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(norm_w[k]) * v);
+          float v = E::rnd(E::val(src[k]) * rs);
+          o = (uint16_t)E::bits(E::val(norm_w[k]) * v);
         }
         dst[k] = o;
       }
@@ -87,9 +88,10 @@ __device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int64_t 
 
 // dot of NR weight rows against BATCH staged vectors; `first`/`step` give this thread's
 // 8-element chunk walk (lane walk for a wave-owned row, thread walk for a block-owned row)
-template <int NR, int BATCH>
+template <int DT, int NR, int BATCH>
 __device__ __forceinline__ void dot_rows_vec8(const uint16_t* const (&wrow)[NR], const uint16_t* const (&xrow)[NR],
                                               int Kp, int K, int first, int step, float (&acc)[NR][BATCH]) {
+  typedef E16<DT> E;
 #pragma unroll 4
   for (int k = first; k < K; k += step) {
     u32x4_t w[NR];
@@ -100,7 +102,7 @@ __device__ __forceinline__ void dot_rows_vec8(const uint16_t* const (&wrow)[NR],
 #pragma unroll
       for (int b = 0; b < BATCH; ++b) {
         u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xrow[r] + b * Kp + k);
-        acc[r][b] = dot8_bf16(w[r], xv, acc[r][b]);
+        acc[r][b] = E::dot8(w[r], xv, acc[r][b]);
       }
     }
   }
@@ -121,9 +123,10 @@ __device__ __forceinline__ void prefetch_rows(const uint16_t* const (&wrow)[NR],
     }
   }
 }
-template <int NR, int PF, int BATCH>
+template <int DT, int NR, int PF, int BATCH>
 __device__ __forceinline__ void consume_rows(const u32x4_t (&w)[NR][PF], const uint16_t* const (&xrow)[NR], int Kp, int K,
                                              int first, int step, float (&acc)[NR][BATCH]) {
+  typedef E16<DT> E;
 #pragma unroll
   for (int c = 0; c < PF; ++c) {
     const int k = first + c * step;
@@ -133,22 +136,23 @@ __device__ __forceinline__ void consume_rows(const u32x4_t (&w)[NR][PF], const u
 #pragma unroll
         for (int b = 0; b < BATCH; ++b) {
           const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xrow[r] + b * Kp + k);
-          acc[r][b] = dot8_bf16(w[r][c], xv, acc[r][b]);
+          acc[r][b] = E::dot8(w[r][c], xv, acc[r][b]);
         }
     }
   }
 }
 
 // fallback walk for rows whose start is not 16-byte aligned or whose length is not a multiple of 8
-template <int NR, int BATCH>
+template <int DT, int NR, int BATCH>
 __device__ __forceinline__ void dot_rows_scalar(const uint16_t* const (&wrow)[NR], const uint16_t* const (&xrow)[NR],
                                                 int Kp, int K, int first, int step, float (&acc)[NR][BATCH]) {
+  typedef E16<DT> E;
   for (int k = first; k < K; k += step) {
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
-      float w = bf16_bits_to_f32(wrow[r][k]);
+      float w = E::val(wrow[r][k]);
 #pragma unroll
-      for (int b = 0; b < BATCH; ++b) acc[r][b] += w * bf16_bits_to_f32(xrow[r][b * Kp + k]);
+      for (int b = 0; b < BATCH; ++b) acc[r][b] += w * E::val(xrow[r][b * Kp + k]);
     }
   }
 }
@@ -185,8 +189,9 @@ __device__ __forceinline__ void reduce_acc(float (&acc)[NR][BATCH], float* red) 
 // ---------------------------------------------------------------------------------------
 // y[b,n] = (res[b,n] +) bf16( W[n,:] . xn[b,:] (+ bias[n]) )
 // ---------------------------------------------------------------------------------------
-template <int BATCH, int ROWS, bool BLOCKROW, bool VEC>
+template <int DT, int BATCH, int ROWS, bool BLOCKROW, bool VEC>
 __global__ __launch_bounds__(kThreads) void linear_kernel(LinearArgs a) {
+  typedef E16<DT> E;
   extern __shared__ __align__(16) uint16_t smem[];
   __shared__ float red[kWaves * ROWS * BATCH > kWaves ? kWaves * ROWS * BATCH : kWaves];
   constexpr int PF = (8 / ROWS) > 1 ? (8 / ROWS) : 2;
@@ -214,7 +219,7 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(LinearArgs a) {
     prefetch_rows<ROWS, PF>(wrow, a.K, first, step, pf);
     have_pf = true;
   }
-  stage_x<BATCH>(a.x + (int64_t)b0 * a.ldx, a.ldx, nb, a.K, Kp, a.norm_w, a.eps, smem, red);
+  stage_x<DT, BATCH>(a.x + (int64_t)b0 * a.ldx, a.ldx, nb, a.K, Kp, a.norm_w, a.eps, smem, red);
 
   // BLOCKROW needs every thread of the block in the loop (barriers inside reduce_acc)
   for (; g < ngrp_rows; g += ngroups) {
@@ -226,15 +231,15 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(LinearArgs a) {
       for (int b = 0; b < BATCH; ++b) acc[r][b] = 0.f;
     int kstart = first;
     if (have_pf) {
-      consume_rows<ROWS, PF, BATCH>(pf, xrow, Kp, a.K, first, step, acc);
+      consume_rows<DT, ROWS, PF, BATCH>(pf, xrow, Kp, a.K, first, step, acc);
       kstart = first + PF * step;
       have_pf = false;
     } else {
 #pragma unroll
       for (int r = 0; r < ROWS; ++r) wrow[r] = a.W + (int64_t)min(n0 + r, a.N - 1) * a.ldw;
     }
-    if (VEC) dot_rows_vec8<ROWS, BATCH>(wrow, xrow, Kp, a.K, kstart, step, acc);
-    else dot_rows_scalar<ROWS, BATCH>(wrow, xrow, Kp, a.K, kstart, step, acc);
+    if (VEC) dot_rows_vec8<DT, ROWS, BATCH>(wrow, xrow, Kp, a.K, kstart, step, acc);
+    else dot_rows_scalar<DT, ROWS, BATCH>(wrow, xrow, Kp, a.K, kstart, step, acc);
     reduce_acc<ROWS, BATCH, BLOCKROW>(acc, red);
     // epilogue: lane/thread (r*BATCH+b) stores one value
     const int who = BLOCKROW ? tid : lane;
@@ -245,10 +250,10 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(LinearArgs a) {
         if (who == r * BATCH + b && n0 + r < a.N && b < nb) {
           const int n = n0 + r;
           float v = acc[r][b];
-          if (a.bias) v += bf16_bits_to_f32(a.bias[n]);
-          v = round_bf16(v);
-          if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)(b0 + b) * a.ldres + n]) + v);
-          a.y[(int64_t)(b0 + b) * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+          if (a.bias) v += E::val(a.bias[n]);
+          v = E::rnd(v);
+          if (a.res) v = E::rnd(E::val(a.res[(int64_t)(b0 + b) * a.ldres + n]) + v);
+          a.y[(int64_t)(b0 + b) * a.ldy + n] = (uint16_t)E::bits(v);
         }
       }
   }
@@ -259,8 +264,9 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(LinearArgs a) {
 //   mode 0 (chain of nn.Linear): g,u rounded to bf16, silu rounded, product rounded
 //   mode 1 (fused-kernel rounding): h = bf16( silu(g32) * u32 )
 // ---------------------------------------------------------------------------------------
-template <int BATCH, int ROWS, bool VEC>
+template <int DT, int BATCH, int ROWS, bool VEC>
 __global__ __launch_bounds__(kThreads) void swiglu_kernel(SwigluArgs a) {
+  typedef E16<DT> E;
   extern __shared__ __align__(16) uint16_t smem[];
   __shared__ float red[kWaves];
   const int Kp = (a.R + 7) & ~7;
@@ -290,8 +296,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_kernel(SwigluArgs a) {
     have_pf = true;
   }
   // two staged vectors per batch row: gate input then up input
-  stage_x<BATCH>(a.p + (int64_t)b0 * a.ldp, a.ldp, nb, a.R, Kp, nullptr, 0.f, smem, red);
-  stage_x<BATCH>(a.p + (int64_t)b0 * a.ldp + a.up_off, a.ldp, nb, a.R, Kp, nullptr, 0.f, smem + BATCH * Kp, red);
+  stage_x<DT, BATCH>(a.p + (int64_t)b0 * a.ldp, a.ldp, nb, a.R, Kp, nullptr, 0.f, smem, red);
+  stage_x<DT, BATCH>(a.p + (int64_t)b0 * a.ldp + a.up_off, a.ldp, nb, a.R, Kp, nullptr, 0.f, smem + BATCH * Kp, red);
 
   for (; g < ngrp_rows; g += ngroups) {
     const int n0 = g * ROWS;
@@ -302,7 +308,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_kernel(SwigluArgs a) {
       for (int b = 0; b < BATCH; ++b) acc[r][b] = 0.f;
     int kstart = first;
     if (have_pf) {
-      consume_rows<2 * ROWS, PF, BATCH>(pf, xrow, Kp, a.R, first, step, acc);
+      consume_rows<DT, 2 * ROWS, PF, BATCH>(pf, xrow, Kp, a.R, first, step, acc);
       kstart = first + PF * step;
       have_pf = false;
     } else {
@@ -313,8 +319,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_kernel(SwigluArgs a) {
         wrow[ROWS + r] = a.up_u + off;
       }
     }
-    if (VEC) dot_rows_vec8<2 * ROWS, BATCH>(wrow, xrow, Kp, a.R, kstart, step, acc);
-    else dot_rows_scalar<2 * ROWS, BATCH>(wrow, xrow, Kp, a.R, kstart, step, acc);
+    if (VEC) dot_rows_vec8<DT, 2 * ROWS, BATCH>(wrow, xrow, Kp, a.R, kstart, step, acc);
+    else dot_rows_scalar<DT, 2 * ROWS, BATCH>(wrow, xrow, Kp, a.R, kstart, step, acc);
     reduce_acc<2 * ROWS, BATCH, false>(acc, red);
 #pragma unroll
     for (int r = 0; r < ROWS; ++r)
@@ -323,13 +329,13 @@ __global__ __launch_bounds__(kThreads) void swiglu_kernel(SwigluArgs a) {
         if (lane == r * BATCH + b && n0 + r < a.D && b < nb) {
           float gv = acc[r][b], uv = acc[ROWS + r][b], hv;
           if (a.mode == 0) {
-            gv = round_bf16(gv);
-            uv = round_bf16(uv);
-            hv = round_bf16(round_bf16(silu_f32(gv)) * uv);
+            gv = E::rnd(gv);
+            uv = E::rnd(uv);
+            hv = E::rnd(E::rnd(silu_f32(gv)) * uv);
           } else {
-            hv = round_bf16((gv * (1.0f / (1.0f + expf(-gv)))) * uv);
+            hv = E::rnd((gv * (1.0f / (1.0f + expf(-gv)))) * uv);
           }
-          a.h[(int64_t)(b0 + b) * a.ldh + n0 + r] = (uint16_t)f32_to_bf16_bits(hv);
+          a.h[(int64_t)(b0 + b) * a.ldh + n0 + r] = (uint16_t)E::bits(hv);
         }
       }
   }
@@ -339,8 +345,9 @@ __global__ __launch_bounds__(kThreads) void swiglu_kernel(SwigluArgs a) {
 // current-token q/k/v from rank coefficients, rotate-half RoPE on q and k, append k/v
 //   p[b] = [Pq | Pk | Pv]; a work item is a row pair (d, d+Dh/2) of one head
 // ---------------------------------------------------------------------------------------
-template <int BATCH, int PAIRS, bool VEC>
+template <int DT, int BATCH, int PAIRS, bool VEC>
 __global__ __launch_bounds__(kThreads) void qkv_rope_append_kernel(QkvArgs a) {
+  typedef E16<DT> E;
   extern __shared__ __align__(16) uint16_t smem[];
   __shared__ float red[kWaves];
   const int Rq8 = (a.Rq + 7) & ~7, Rk8 = (a.Rk + 7) & ~7, Rv8 = (a.Rv + 7) & ~7;
@@ -350,9 +357,9 @@ __global__ __launch_bounds__(kThreads) void qkv_rope_append_kernel(QkvArgs a) {
   uint16_t* xk = xq + BATCH * Rq8;
   uint16_t* xv = xk + BATCH * Rk8;
   const uint16_t* pb = a.p + (int64_t)b0 * a.ldp;
-  stage_x<BATCH>(pb, a.ldp, nb, a.Rq, Rq8, nullptr, 0.f, xq, red);
-  stage_x<BATCH>(pb + a.Rq, a.ldp, nb, a.Rk, Rk8, nullptr, 0.f, xk, red);
-  stage_x<BATCH>(pb + a.Rq + a.Rk, a.ldp, nb, a.Rv, Rv8, nullptr, 0.f, xv, red);
+  stage_x<DT, BATCH>(pb, a.ldp, nb, a.Rq, Rq8, nullptr, 0.f, xq, red);
+  stage_x<DT, BATCH>(pb + a.Rq, a.ldp, nb, a.Rk, Rk8, nullptr, 0.f, xk, red);
+  stage_x<DT, BATCH>(pb + a.Rq + a.Rk, a.ldp, nb, a.Rv, Rv8, nullptr, 0.f, xv, red);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = a.Dh >> 1;
@@ -399,8 +406,8 @@ __global__ __launch_bounds__(kThreads) void qkv_rope_append_kernel(QkvArgs a) {
       float acc2[2][BATCH];
 #pragma unroll
       for (int b = 0; b < BATCH; ++b) acc2[0][b] = acc2[1][b] = 0.f;
-      if (VEC) dot_rows_vec8<2, BATCH>(w2, x2, Kp[i], K[i], lane * 8, kWave * 8, acc2);
-      else dot_rows_scalar<2, BATCH>(w2, x2, Kp[i], K[i], lane, kWave, acc2);
+      if (VEC) dot_rows_vec8<DT, 2, BATCH>(w2, x2, Kp[i], K[i], lane * 8, kWave * 8, acc2);
+      else dot_rows_scalar<DT, 2, BATCH>(w2, x2, Kp[i], K[i], lane, kWave, acc2);
 #pragma unroll
       for (int b = 0; b < BATCH; ++b) { acc[2 * i][b] = acc2[0][b]; acc[2 * i + 1][b] = acc2[1][b]; }
     }
@@ -412,17 +419,17 @@ __global__ __launch_bounds__(kThreads) void qkv_rope_append_kernel(QkvArgs a) {
         if (lane == i * BATCH + b && g * PAIRS + i < npairs && b < nb) {
           const int bb = b0 + b;
           const int pos = a.positions[bb];
-          float x0 = round_bf16(acc[2 * i][b]), x1 = round_bf16(acc[2 * i + 1][b]);
+          float x0 = E::rnd(acc[2 * i][b]), x1 = E::rnd(acc[2 * i + 1][b]);
           if (kind[i] != 2 && a.cos) {
             // eager bf16 arithmetic: x0*c - x1*s and x1*c + x0*s, one rounding per op
             const int tp = min(max(pos, 0), a.rope_len - 1);
-            const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * half + dd[i]]);
-            const float s = bf16_bits_to_f32(a.sin[(int64_t)tp * half + dd[i]]);
-            const float r0 = round_bf16(round_bf16(x0 * c) - round_bf16(x1 * s));
-            const float r1 = round_bf16(round_bf16(x1 * c) + round_bf16(x0 * s));
+            const float c = E::val(a.cos[(int64_t)tp * half + dd[i]]);
+            const float s = E::val(a.sin[(int64_t)tp * half + dd[i]]);
+            const float r0 = E::rnd(E::rnd(x0 * c) - E::rnd(x1 * s));
+            const float r1 = E::rnd(E::rnd(x1 * c) + E::rnd(x0 * s));
             x0 = r0; x1 = r1;
           }
-          const uint16_t o0 = (uint16_t)f32_to_bf16_bits(x0), o1 = (uint16_t)f32_to_bf16_bits(x1);
+          const uint16_t o0 = (uint16_t)E::bits(x0), o1 = (uint16_t)E::bits(x1);
           if (kind[i] == 0) {
             uint16_t* q = a.q_out + ((int64_t)bb * a.H + head[i]) * a.Dh + dd[i];
             q[0] = o0; q[half] = o1;
@@ -439,15 +446,17 @@ __global__ __launch_bounds__(kThreads) void qkv_rope_append_kernel(QkvArgs a) {
 // ---------------------------------------------------------------------------------------
 // stand-alone RMSNorm (one block per row)
 // ---------------------------------------------------------------------------------------
+template <int DT>
 __global__ __launch_bounds__(kThreads) void rmsnorm_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                           const uint16_t* __restrict__ w, float eps,
                                                           uint16_t* __restrict__ y, int64_t ldy, int K) {
+  typedef E16<DT> E;
   __shared__ float red[kWaves];
   const uint16_t* src = x + (int64_t)blockIdx.x * ldx;
   uint16_t* dst = y + (int64_t)blockIdx.x * ldy;
   float ss = 0.f;
   for (int k = threadIdx.x; k < K; k += kThreads) {
-    float v = bf16_bits_to_f32(src[k]);
+    float v = E::val(src[k]);
     ss += v * v;
   }
   ss = wave_sum(ss);
@@ -458,17 +467,18 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_kernel(const uint16_t* __res
   for (int i = 0; i < kWaves; ++i) tot += red[i];
   const float rs = rsqrtf(tot / (float)K + eps);
   for (int k = threadIdx.x; k < K; k += kThreads) {
-    float v = round_bf16(bf16_bits_to_f32(src[k]) * rs);
-    dst[k] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(w[k]) * v);
+    float v = E::rnd(E::val(src[k]) * rs);
+    dst[k] = (uint16_t)E::bits(E::val(w[k]) * v);
   }
 }
 
 // the same with 16-byte accesses and the row kept in registers between the two passes (K a multiple of 8, at most
 // 8 * NC * kThreads, rows 16-byte aligned): a prompt of 512 rows x 4096 took 9.9 us with 2-byte accesses
-template <int NC>
+template <int DT, int NC>
 __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(const uint16_t* __restrict__ x, int64_t ldx,
                                                               const uint16_t* __restrict__ w, float eps,
                                                               uint16_t* __restrict__ y, int64_t ldy, int K) {
+  typedef E16<DT> E;
   __shared__ float red[kWaves];
   const uint16_t* src = x + (int64_t)blockIdx.x * ldx;
   uint16_t* dst = y + (int64_t)blockIdx.x * ldy;
@@ -482,7 +492,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(const uint16_t* _
     const uint32_t e[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float a = bf16_lo(e[i]), b = bf16_hi(e[i]);
+      const float a = E::lo(e[i]), b = E::hi(e[i]);
       ss += a * a;
       ss += b * b;
     }
@@ -503,8 +513,8 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(const uint16_t* _
     uint32_t o[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float a = round_bf16(bf16_lo(e[i]) * rs), b = round_bf16(bf16_hi(e[i]) * rs);
-      o[i] = f32_to_bf16_bits(bf16_lo(g[i]) * a) | (f32_to_bf16_bits(bf16_hi(g[i]) * b) << 16);
+      const float a = E::rnd(E::lo(e[i]) * rs), b = E::rnd(E::hi(e[i]) * rs);
+      o[i] = E::bits(E::lo(g[i]) * a) | (E::bits(E::hi(g[i]) * b) << 16);
     }
     *reinterpret_cast<u32x4_t*>(dst + ch * 8) = u32x4_t{o[0], o[1], o[2], o[3]};
   }
@@ -524,7 +534,7 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
     }                                                                       \
   } while (0)
 
-template <int BATCH, bool VEC>
+template <int DT, int BATCH, bool VEC>
 static int launch_linear_b(const LinearArgs& a, int cfg, hipStream_t st) {
   const int Kp = (a.K + 7) & ~7;
   const size_t smem = (size_t)BATCH * Kp * 2;
@@ -541,7 +551,7 @@ static int launch_linear_b(const LinearArgs& a, int cfg, hipStream_t st) {
   {                                                                                              \
     const int groups = (a.N + R - 1) / R;                                                        \
     dim3 grid(BR ? groups : (groups + kWaves - 1) / kWaves, nby);                                \
-    hipLaunchKernelGGL((linear_kernel<BATCH, R, BR, VEC>), grid, dim3(kThreads), smem, st, a);   \
+    hipLaunchKernelGGL((linear_kernel<DT, BATCH, R, BR, VEC>), grid, dim3(kThreads), smem, st, a);   \
   }
   if (blockrow) {
     if (rows >= 2) FSVD_LAUNCH_LIN(2, true) else FSVD_LAUNCH_LIN(1, true)
@@ -553,23 +563,29 @@ static int launch_linear_b(const LinearArgs& a, int cfg, hipStream_t st) {
   return kOk;
 }
 
-int launch_linear(const LinearArgs& a, int cfg, hipStream_t st) {
-  if (a.B <= 0 || a.N <= 0 || a.K <= 0) { set_last_error("fsvd_linear: empty shape B=%d N=%d K=%d", a.B, a.N, a.K); return kErrBadShape; }
-  if (cfg == 0 && mfma_linear_applies(a)) return launch_linear_mfma(a, st);
-  if (a.K > 32768) { set_last_error("fsvd_linear: K=%d exceeds the 32768 LDS staging limit", a.K); return kErrBadShape; }
+template <int DT>
+static int launch_linear_t(const LinearArgs& a, int cfg, hipStream_t st) {
   const bool vec = (a.K % 8 == 0) && (a.ldw % 8 == 0) && aligned16(a.W);
   const int batch = a.B >= 4 && a.K <= 16384 ? 4 : (a.B >= 2 ? 2 : 1);
   if (vec) {
-    if (batch == 4) return launch_linear_b<4, true>(a, cfg, st);
-    if (batch == 2) return launch_linear_b<2, true>(a, cfg, st);
-    return launch_linear_b<1, true>(a, cfg, st);
+    if (batch == 4) return launch_linear_b<DT, 4, true>(a, cfg, st);
+    if (batch == 2) return launch_linear_b<DT, 2, true>(a, cfg, st);
+    return launch_linear_b<DT, 1, true>(a, cfg, st);
   }
-  if (batch == 4) return launch_linear_b<4, false>(a, cfg, st);
-  if (batch == 2) return launch_linear_b<2, false>(a, cfg, st);
-  return launch_linear_b<1, false>(a, cfg, st);
+  if (batch == 4) return launch_linear_b<DT, 4, false>(a, cfg, st);
+  if (batch == 2) return launch_linear_b<DT, 2, false>(a, cfg, st);
+  return launch_linear_b<DT, 1, false>(a, cfg, st);
 }
 
-template <int BATCH, bool VEC>
+int launch_linear(const LinearArgs& a, int cfg, hipStream_t st) {
+  if (a.B <= 0 || a.N <= 0 || a.K <= 0) { set_last_error("fsvd_linear: empty shape B=%d N=%d K=%d", a.B, a.N, a.K); return kErrBadShape; }
+  if (a.dt != 0 && a.dt != 1) { set_last_error("fsvd_linear: dtype code %d (bf16 = 0 and fp16 = 1 are served)", a.dt); return kErrBadDtype; }
+  if (cfg == 0 && mfma_linear_applies(a)) return launch_linear_mfma(a, st);
+  if (a.K > 32768) { set_last_error("fsvd_linear: K=%d exceeds the 32768 LDS staging limit", a.K); return kErrBadShape; }
+  return a.dt == 1 ? launch_linear_t<1>(a, cfg, st) : launch_linear_t<0>(a, cfg, st);
+}
+
+template <int DT, int BATCH, bool VEC>
 static int launch_swiglu_b(const SwigluArgs& a, int cfg, hipStream_t st) {
   const int Kp = (a.R + 7) & ~7;
   const size_t smem = (size_t)2 * BATCH * Kp * 2;
@@ -580,7 +596,7 @@ static int launch_swiglu_b(const SwigluArgs& a, int cfg, hipStream_t st) {
   {                                                                                        \
     const int groups = (a.D + R - 1) / R;                                                  \
     dim3 grid((groups + kWaves - 1) / kWaves, nby);                                        \
-    hipLaunchKernelGGL((swiglu_kernel<BATCH, R, VEC>), grid, dim3(kThreads), smem, st, a); \
+    hipLaunchKernelGGL((swiglu_kernel<DT, BATCH, R, VEC>), grid, dim3(kThreads), smem, st, a); \
   }
   if (rows >= 2 && BATCH <= 2) FSVD_LAUNCH_SW(2) else FSVD_LAUNCH_SW(1)
 #undef FSVD_LAUNCH_SW
@@ -588,23 +604,29 @@ static int launch_swiglu_b(const SwigluArgs& a, int cfg, hipStream_t st) {
   return kOk;
 }
 
-int launch_swiglu(const SwigluArgs& a, int cfg, hipStream_t st) {
-  if (a.B <= 0 || a.D <= 0 || a.R <= 0) { set_last_error("fsvd_swiglu_linear: empty shape"); return kErrBadShape; }
-  if (cfg == 0 && mfma_swiglu_applies(a)) return launch_swiglu_mfma(a, st);
-  if (a.R > 16384) { set_last_error("fsvd_swiglu_linear: R=%d exceeds 16384", a.R); return kErrBadShape; }
+template <int DT>
+static int launch_swiglu_t(const SwigluArgs& a, int cfg, hipStream_t st) {
   const bool vec = (a.R % 8 == 0) && (a.ldw % 8 == 0) && aligned16(a.gate_u) && aligned16(a.up_u);
   const int batch = a.B >= 4 && a.R <= 4096 ? 4 : (a.B >= 2 ? 2 : 1);
   if (vec) {
-    if (batch == 4) return launch_swiglu_b<4, true>(a, cfg, st);
-    if (batch == 2) return launch_swiglu_b<2, true>(a, cfg, st);
-    return launch_swiglu_b<1, true>(a, cfg, st);
+    if (batch == 4) return launch_swiglu_b<DT, 4, true>(a, cfg, st);
+    if (batch == 2) return launch_swiglu_b<DT, 2, true>(a, cfg, st);
+    return launch_swiglu_b<DT, 1, true>(a, cfg, st);
   }
-  if (batch == 4) return launch_swiglu_b<4, false>(a, cfg, st);
-  if (batch == 2) return launch_swiglu_b<2, false>(a, cfg, st);
-  return launch_swiglu_b<1, false>(a, cfg, st);
+  if (batch == 4) return launch_swiglu_b<DT, 4, false>(a, cfg, st);
+  if (batch == 2) return launch_swiglu_b<DT, 2, false>(a, cfg, st);
+  return launch_swiglu_b<DT, 1, false>(a, cfg, st);
 }
 
-template <int BATCH, bool VEC>
+int launch_swiglu(const SwigluArgs& a, int cfg, hipStream_t st) {
+  if (a.B <= 0 || a.D <= 0 || a.R <= 0) { set_last_error("fsvd_swiglu_linear: empty shape"); return kErrBadShape; }
+  if (a.dt != 0 && a.dt != 1) { set_last_error("fsvd_swiglu_linear: dtype code %d (bf16 = 0 and fp16 = 1 are served)", a.dt); return kErrBadDtype; }
+  if (cfg == 0 && mfma_swiglu_applies(a)) return launch_swiglu_mfma(a, st);
+  if (a.R > 16384) { set_last_error("fsvd_swiglu_linear: R=%d exceeds 16384", a.R); return kErrBadShape; }
+  return a.dt == 1 ? launch_swiglu_t<1>(a, cfg, st) : launch_swiglu_t<0>(a, cfg, st);
+}
+
+template <int DT, int BATCH, bool VEC>
 static int launch_qkv_b(const QkvArgs& a, int cfg, hipStream_t st) {
   const int Rq8 = (a.Rq + 7) & ~7, Rk8 = (a.Rk + 7) & ~7, Rv8 = (a.Rv + 7) & ~7;
   const size_t smem = (size_t)BATCH * (Rq8 + Rk8 + Rv8) * 2;
@@ -616,7 +638,7 @@ static int launch_qkv_b(const QkvArgs& a, int cfg, hipStream_t st) {
   {                                                                                                 \
     const int groups = (npairs + P - 1) / P;                                                        \
     dim3 grid((groups + kWaves - 1) / kWaves, nby);                                                 \
-    hipLaunchKernelGGL((qkv_rope_append_kernel<BATCH, P, VEC>), grid, dim3(kThreads), smem, st, a); \
+    hipLaunchKernelGGL((qkv_rope_append_kernel<DT, BATCH, P, VEC>), grid, dim3(kThreads), smem, st, a); \
   }
   if (pairs >= 2 && BATCH == 1) FSVD_LAUNCH_QKV(2) else FSVD_LAUNCH_QKV(1)
 #undef FSVD_LAUNCH_QKV
@@ -624,33 +646,53 @@ static int launch_qkv_b(const QkvArgs& a, int cfg, hipStream_t st) {
   return kOk;
 }
 
-int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st) {
+static int check_qkv(const QkvArgs& a) {
   if (a.B <= 0 || a.H <= 0 || a.Hk <= 0 || a.Dh <= 0 || (a.Dh & 1) || a.Rq <= 0 || a.Rk <= 0 || a.Rv <= 0) {
     set_last_error("fsvd_qkv_rope_append: bad shape B=%d H=%d Hk=%d Dh=%d R=(%d,%d,%d)", a.B, a.H, a.Hk, a.Dh, a.Rq, a.Rk, a.Rv);
     return kErrBadShape;
   }
   if (a.Rq + a.Rk + a.Rv > 24576) { set_last_error("fsvd_qkv_rope_append: ranks too large for LDS staging"); return kErrBadShape; }
+  if (a.dt != 0 && a.dt != 1) { set_last_error("fsvd_qkv_rope_append: dtype code %d (bf16 = 0 and fp16 = 1 are served)", a.dt); return kErrBadDtype; }
+  return kOk;
+}
+
+template <int DT>
+static int launch_qkv_t(const QkvArgs& a, int cfg, hipStream_t st) {
   const bool vec = (a.Rq % 8 == 0) && (a.Rk % 8 == 0) && (a.Rv % 8 == 0) && (a.ldq % 8 == 0) && (a.ldk % 8 == 0) &&
                    (a.ldv % 8 == 0) && aligned16(a.q_u) && aligned16(a.k_u) && aligned16(a.v_u);
   const int batch = a.B >= 4 && (a.Rq + a.Rk + a.Rv) <= 8192 ? 4 : (a.B >= 2 ? 2 : 1);
   if (vec) {
-    if (batch == 4) return launch_qkv_b<4, true>(a, cfg, st);
-    if (batch == 2) return launch_qkv_b<2, true>(a, cfg, st);
-    return launch_qkv_b<1, true>(a, cfg, st);
+    if (batch == 4) return launch_qkv_b<DT, 4, true>(a, cfg, st);
+    if (batch == 2) return launch_qkv_b<DT, 2, true>(a, cfg, st);
+    return launch_qkv_b<DT, 1, true>(a, cfg, st);
   }
-  if (batch == 4) return launch_qkv_b<4, false>(a, cfg, st);
-  if (batch == 2) return launch_qkv_b<2, false>(a, cfg, st);
-  return launch_qkv_b<1, false>(a, cfg, st);
+  if (batch == 4) return launch_qkv_b<DT, 4, false>(a, cfg, st);
+  if (batch == 2) return launch_qkv_b<DT, 2, false>(a, cfg, st);
+  return launch_qkv_b<DT, 1, false>(a, cfg, st);
+}
+
+int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st) {
+  const int rc = check_qkv(a);
+  if (rc != kOk) return rc;
+  return a.dt == 1 ? launch_qkv_t<1>(a, cfg, st) : launch_qkv_t<0>(a, cfg, st);
+}
+
+template <int DT>
+static void launch_rmsnorm_t(const uint16_t* x, int64_t ldx, const uint16_t* w, float eps, uint16_t* y, int64_t ldy, int rows,
+                             int K, hipStream_t st) {
+  const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool vec = (K % 8) == 0 && al(x) && al(w) && al(y) && (ldx % 8) == 0 && (ldy % 8) == 0;
+  if (vec && K <= 8 * 2 * kThreads) hipLaunchKernelGGL((rmsnorm_vec_kernel<DT, 2>), dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
+  else if (vec && K <= 8 * 8 * kThreads) hipLaunchKernelGGL((rmsnorm_vec_kernel<DT, 8>), dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
+  else hipLaunchKernelGGL(rmsnorm_kernel<DT>, dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
 }
 
 int launch_rmsnorm(const uint16_t* x, int64_t ldx, const uint16_t* w, float eps, uint16_t* y, int64_t ldy, int rows,
-                   int K, hipStream_t st) {
+                   int K, int dt, hipStream_t st) {
   if (rows <= 0 || K <= 0) { set_last_error("fsvd_rmsnorm: empty shape"); return kErrBadShape; }
-  const auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  const bool vec = (K % 8) == 0 && al(x) && al(w) && al(y) && (ldx % 8) == 0 && (ldy % 8) == 0;
-  if (vec && K <= 8 * 2 * kThreads) hipLaunchKernelGGL(rmsnorm_vec_kernel<2>, dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
-  else if (vec && K <= 8 * 8 * kThreads) hipLaunchKernelGGL(rmsnorm_vec_kernel<8>, dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
-  else hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(kThreads), 0, st, x, ldx, w, eps, y, ldy, K);
+  if (dt != 0 && dt != 1) { set_last_error("fsvd_rmsnorm: dtype code %d (bf16 = 0 and fp16 = 1 are served)", dt); return kErrBadDtype; }
+  if (dt == 1) launch_rmsnorm_t<1>(x, ldx, w, eps, y, ldy, rows, K, st);
+  else launch_rmsnorm_t<0>(x, ldx, w, eps, y, ldy, rows, K, st);
   FSVD_CHECK_LAUNCH("fsvd_rmsnorm");
   return kOk;
 }

@@ -13,6 +13,7 @@ struct LinearArgs {
   const uint16_t* res; int64_t ldres;    // residual [B, N] or null
   uint16_t* y; int64_t ldy;              // [B, N]
   int B, N, K;
+  int dt = 0;                            // element type: 0 bf16, 1 fp16
 };
 
 struct SwigluArgs {
@@ -21,6 +22,7 @@ struct SwigluArgs {
   uint16_t* h; int64_t ldh;              // [B, D]
   int B, D, R;
   int mode;                              // 0 chain-of-linears rounding, 1 fused-kernel rounding
+  int dt = 0;
 };
 
 struct QkvArgs {
@@ -34,6 +36,7 @@ struct QkvArgs {
   uint16_t* k_cache; uint16_t* v_cache;  // [B, S, Hk, Dh] with element strides below
   int64_t sc_b, sc_s, sc_h;
   int B, H, Hk, Dh, Rq, Rk, Rv, S;
+  int dt = 0;
 };
 
 struct AttnDecodeArgs {
@@ -49,6 +52,7 @@ struct AttnDecodeArgs {
   int32_t* ws_count;                     // [B, H] arrival counters (zero before first use; self-resetting)
   int B, H, Hk, Dh, S, nsplit;
   float scale;
+  int dt = 0;
 };
 
 struct KvAppendArgs {
@@ -58,6 +62,7 @@ struct KvAppendArgs {
   const int32_t* seqlens;
   const uint16_t* cos; const uint16_t* sin; int rope_len;
   int B, Hk, Dh, S;
+  int dt = 0;
 };
 
 // one x @ W problem of the input-major GEMV (a launch carries up to three: q, k, v)
@@ -123,6 +128,7 @@ struct ExpandArgs {
   int dst_by_position;                              // 1: destination row = absolute position (cache), 0: row = m
   int dst_rows;                                     // rows the destination has (bounds check)
   int B, M, heads, Dh, R;
+  int dt = 0;
 };
 struct PrefillAttnArgs {
   const uint16_t* q; int64_t sq_b, sq_m, sq_h;      // [B,M,H,Dh], rotated
@@ -133,6 +139,7 @@ struct PrefillAttnArgs {
   uint16_t* out; int64_t so_b, so_m, so_h;          // [B,M,H,Dh]
   int B, M, H, Hk, Dh, S, causal;
   float scale;
+  int dt = 0;
 };
 int launch_expand(const ExpandArgs& a, hipStream_t st);
 bool expand_tiles_apply(const ExpandArgs& a);                               // mfma_gemm.hip
@@ -152,6 +159,7 @@ struct MfmaArgs {
   // K split over gridDim.z workgroups per output tile (filled by the launcher when a workspace is registered):
   // fp32 partial tiles and one arrival counter per tile; the last workgroup to arrive adds the partials in order
   int ksplit; float* ws_part; int32_t* ws_count;
+  int dt = 0;
 };
 // caller-owned scratch of the current device for the K-split projections (null when none is registered)
 struct SplitWorkspace { float* part; size_t part_floats; int32_t* count; int ncount; };
@@ -185,7 +193,7 @@ int launch_dequant_q4(const uint8_t* qw, int64_t ldq, const uint16_t* sc, const 
                       int64_t ldw, int N, int K, hipStream_t st);
 int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st);
 int launch_rmsnorm(const uint16_t* x, int64_t ldx, const uint16_t* w, float eps, uint16_t* y, int64_t ldy, int rows,
-                   int K, hipStream_t st);
+                   int K, int dt, hipStream_t st);
 int launch_attn_decode(const AttnDecodeArgs& a, hipStream_t st);
 int launch_kv_append(const KvAppendArgs& a, hipStream_t st);
 size_t attn_decode_ws_floats(int B, int H, int nsplit, int Dh);

@@ -19,7 +19,6 @@
 
 namespace fsvd {
 
-typedef __bf16 gm_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float gm_f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kGT4 = 256;           // threads of the four-wave form: 2 x 2 waves
@@ -45,8 +44,10 @@ struct ExpandEpi {
 // gate partners through LDS once, before the SwiGLU epilogue.  8, single matrix: waves 4-7 take the second half of the
 // k slices of every step and hand their sums to waves 0-3 through LDS at the end.
 // PF > 0: register sets in flight; PF < 0: loads straight into LDS with -PF stages.
-template <bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
+template <int DT, bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
 __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandEpi& ep, const int tile_m, const int tile_n) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   static_assert(!EXPAND || (!DUAL && WT == 4), "head expansion takes whole 128-wide heads");
   static_assert(NW == 4 || (NW == 8 && DUAL && WT == 4 && WTM == 4) || (NW == 8 && !DUAL && !EXPAND && BK >= 64),
                 "eight waves: the split form of the 128 x 128 pair tile, or two halves of every K step of a single matrix");
@@ -190,17 +191,17 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
       // next stage and the global loads that refill their registers: the other stage was last read before the
       // barrier that ended step ks - 1, and past the last step both are harmless (clamped addresses, a dead stage).
       constexpr int Q = KHALF ? BK / 64 : (BK / 32) * NMA;
-      gm_bf16x8_t fx[2][WTM], fw[2][WT];
+      frag_t fx[2][WTM], fw[2][WT];
       const auto load_frags = [&](int q, int set) {
         const int kk = KHALF ? mat * (BK / 64) + q : q / NMA, m = SPLIT ? mat : (KHALF ? 0 : q % NMA);
         const int fcol = (((kk * 4) ^ fr_hi) + fr_lo) * 8;
 #pragma unroll
         for (int i = 0; i < WTM; ++i)
-          fx[set][i] = *reinterpret_cast<const gm_bf16x8_t*>(base + m * kTileX + (wm * 16 * WTM + i * 16 + lr) * kGLd + fcol);
+          fx[set][i] = *reinterpret_cast<const frag_t*>(base + m * kTileX + (wm * 16 * WTM + i * 16 + lr) * kGLd + fcol);
 #pragma unroll
         for (int i = 0; i < WT; ++i) {
           const int wrow = EXPAND ? (i < 2 ? wn * 32 + i * 16 : 64 + wn * 32 + (i - 2) * 16) : wn * 16 * WT + i * 16;
-          fw[set][i] = *reinterpret_cast<const gm_bf16x8_t*>(base + NM * kTileX + m * kTileW + (wrow + lr) * kGLd + fcol);
+          fw[set][i] = *reinterpret_cast<const frag_t*>(base + NM * kTileX + m * kTileW + (wrow + lr) * kGLd + fcol);
         }
       };
       load_frags(0, 0);
@@ -217,7 +218,7 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
         for (int i = 0; i < WTM; ++i)
 #pragma unroll
           for (int j = 0; j < WT; ++j)
-            acc[q % NMA][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[q & 1][j], fx[q & 1][i], acc[q % NMA][i][j], 0, 0, 0);
+            acc[q % NMA][i][j] = E::mfma(fw[q & 1][j], fx[q & 1][i], acc[q % NMA][i][j]);
         // issue order: memory instructions spread between the products instead of ahead of them
         constexpr int kMf = WTM * WT;
         if (q + 1 < Q) {
@@ -374,13 +375,13 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
           if (tab8) {
             const u32x2_t cw = *reinterpret_cast<const u32x2_t*>(ep.cos + (int64_t)tp * 64 + d0);
             const u32x2_t sw = *reinterpret_cast<const u32x2_t*>(ep.sin + (int64_t)tp * 64 + d0);
-            c[0] = bf16_lo(cw.x); c[1] = bf16_hi(cw.x); c[2] = bf16_lo(cw.y); c[3] = bf16_hi(cw.y);
-            sn[0] = bf16_lo(sw.x); sn[1] = bf16_hi(sw.x); sn[2] = bf16_lo(sw.y); sn[3] = bf16_hi(sw.y);
+            c[0] = E::lo(cw.x); c[1] = E::hi(cw.x); c[2] = E::lo(cw.y); c[3] = E::hi(cw.y);
+            sn[0] = E::lo(sw.x); sn[1] = E::hi(sw.x); sn[2] = E::lo(sw.y); sn[3] = E::hi(sw.y);
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              c[e] = bf16_bits_to_f32(ep.cos[(int64_t)tp * 64 + d0 + e]);
-              sn[e] = bf16_bits_to_f32(ep.sin[(int64_t)tp * 64 + d0 + e]);
+              c[e] = E::val(ep.cos[(int64_t)tp * 64 + d0 + e]);
+              sn[e] = E::val(ep.sin[(int64_t)tp * 64 + d0 + e]);
             }
           }
         }
@@ -389,16 +390,16 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
         for (int e = 0; e < 4; ++e) {
           const int d = d0 + e;
           float x0 = acc[0][i][j][e], x1 = acc[0][i][j + 2][e];
-          if (a.bias) { x0 += bf16_bits_to_f32(a.bias[head * 128 + d]); x1 += bf16_bits_to_f32(a.bias[head * 128 + d + 64]); }
-          x0 = round_bf16(x0);                          // the projection's own rounding point
-          x1 = round_bf16(x1);
+          if (a.bias) { x0 += E::val(a.bias[head * 128 + d]); x1 += E::val(a.bias[head * 128 + d + 64]); }
+          x0 = E::rnd(x0);                          // the projection's own rounding point
+          x1 = E::rnd(x1);
           if (ep.cos) {                                 // eager bf16 arithmetic, one rounding per op
-            const float r0 = round_bf16(round_bf16(x0 * c[e]) - round_bf16(x1 * sn[e]));
-            const float r1 = round_bf16(round_bf16(x1 * c[e]) + round_bf16(x0 * sn[e]));
+            const float r0 = E::rnd(E::rnd(x0 * c[e]) - E::rnd(x1 * sn[e]));
+            const float r1 = E::rnd(E::rnd(x1 * c[e]) + E::rnd(x0 * sn[e]));
             x0 = r0; x1 = r1;
           }
-          o0[e] = f32_to_bf16_bits(x0);
-          o1[e] = f32_to_bf16_bits(x1);
+          o0[e] = E::bits(x0);
+          o1[e] = E::bits(x1);
         }
         if (dst8) {
           *reinterpret_cast<u32x2_t*>(dst + d0) = u32x2_t{o0[0] | (o0[1] << 16), o0[2] | (o0[3] << 16)};
@@ -422,11 +423,11 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
       if (!DUAL && rrow) {
         if (whole && r8) {
           const u32x2_t rw = *reinterpret_cast<const u32x2_t*>(rrow + nb);
-          r[0] = bf16_lo(rw.x); r[1] = bf16_hi(rw.x); r[2] = bf16_lo(rw.y); r[3] = bf16_hi(rw.y);
+          r[0] = E::lo(rw.x); r[1] = E::hi(rw.x); r[2] = E::lo(rw.y); r[3] = E::hi(rw.y);
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (nb + e < a.N) r[e] = bf16_bits_to_f32(rrow[nb + e]);
+            if (nb + e < a.N) r[e] = E::val(rrow[nb + e]);
         }
       }
       uint32_t o[4];
@@ -437,18 +438,18 @@ __device__ __forceinline__ void gemm_tiles_body(const MfmaArgs& a, const ExpandE
         if (DUAL) {
           float v1 = SPLIT ? upv[SPLIT ? i : 0][SPLIT ? j : 0][e] : acc[NMA - 1][i][j][e];
           if (a.mode == 0) {
-            v0 = round_bf16(v0);
-            v1 = round_bf16(v1);
-            v = round_bf16(round_bf16(silu_f32(v0)) * v1);
+            v0 = E::rnd(v0);
+            v1 = E::rnd(v1);
+            v = E::rnd(E::rnd(silu_f32(v0)) * v1);
           } else {
-            v = round_bf16((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
+            v = E::rnd((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
           }
         } else {
-          if (a.bias && nb + e < a.N) v0 += bf16_bits_to_f32(a.bias[nb + e]);
-          v = round_bf16(v0);
-          if (rrow) v = round_bf16(r[e] + v);
+          if (a.bias && nb + e < a.N) v0 += E::val(a.bias[nb + e]);
+          v = E::rnd(v0);
+          if (rrow) v = E::rnd(r[e] + v);
         }
-        o[e] = f32_to_bf16_bits(v);
+        o[e] = E::bits(v);
       }
       if (whole && y8) {
         *reinterpret_cast<u32x2_t*>(yrow + nb) = u32x2_t{o[0] | (o[1] << 16), o[2] | (o[3] << 16)};
@@ -471,23 +472,23 @@ __device__ __forceinline__ void tile_of_workgroup(int NT, int MT, int& tile_m, i
   tile_m = band * 8 + tb - tile_n * bh;
 }
 
-template <bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
+template <int DT, bool DUAL, int WTM, int WT, int PF, bool EXPAND, int BK, int NW>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void gemm_tiles_kernel(MfmaArgs a, ExpandEpi ep) {
   int tile_m, tile_n;
   tile_of_workgroup(gridDim.x, gridDim.y, tile_m, tile_n);
-  gemm_tiles_body<DUAL, WTM, WT, PF, EXPAND, BK, NW>(a, ep, tile_m, tile_n);
+  gemm_tiles_body<DT, DUAL, WTM, WT, PF, EXPAND, BK, NW>(a, ep, tile_m, tile_n);
 }
 
 // up to three head expansions of the same token rows (q, k, v of a prompt pass) in one launch: column tile = one head
 // of one of them.  At 512 rows a single expansion has one workgroup per compute unit and waits on its own loads; the
 // three together give every compute unit three.
 struct ExpandBatch { MfmaArgs a[3]; ExpandEpi ep[3]; int first_head[4]; };
-template <int WTM>
+template <int DT, int WTM>
 __global__ __launch_bounds__(kGT4, 2) void expand_multi_kernel(ExpandBatch eb) {
   int tile_m, tile_n;
   tile_of_workgroup(gridDim.x, gridDim.y, tile_m, tile_n);
   const int k = tile_n >= eb.first_head[2] ? 2 : (tile_n >= eb.first_head[1] ? 1 : 0);
-  gemm_tiles_body<false, WTM, 4, 2, true, kGBK, 4>(eb.a[k], eb.ep[k], tile_m, tile_n - eb.first_head[k]);
+  gemm_tiles_body<DT, false, WTM, 4, 2, true, kGBK, 4>(eb.a[k], eb.ep[k], tile_m, tile_n - eb.first_head[k]);
 }
 
 bool gemm_tiles_apply(const MfmaArgs& a) {
@@ -518,7 +519,7 @@ static int pick_ksplit_prompt(int64_t tiles, int ksteps, int K, size_t floats_pe
   return z > 1 ? fit_ksplit(z, tiles, ksteps, floats_per_share, ws, 8) : 1;
 }
 
-template <bool DUAL, int WTM, int WT, int BK, int NW = 4, int PFSEL = 99>
+template <int DT, bool DUAL, int WTM, int WT, int BK, int NW = 4, int PFSEL = 99>
 static int launch_gemm_tiles_t(const MfmaArgs& a0, hipStream_t st, const char* who) {
   static bool granted = false;
   constexpr int BM = 32 * WTM, BN = 32 * WT;
@@ -528,7 +529,7 @@ static int launch_gemm_tiles_t(const MfmaArgs& a0, hipStream_t st, const char* w
   constexpr int PF = PFSEL != 99 ? PFSEL : (!DUAL && WT == 2 && WTM == 2 && BK == 64) ? 4 : 2;
   const size_t lds = (size_t)(PF < 0 ? -PF : 2) * (DUAL ? 2 : 1) * (BM + BN) * kGLd * 2;
   if (lds > 64 * 1024 && !granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DUAL, WTM, WT, PF, false, BK, NW>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DT, DUAL, WTM, WT, PF, false, BK, NW>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
@@ -545,13 +546,14 @@ static int launch_gemm_tiles_t(const MfmaArgs& a0, hipStream_t st, const char* w
   a.ws_part = ws.part;
   a.ws_count = ws.count;
   grid.z = a.ksplit;
-  hipLaunchKernelGGL((gemm_tiles_kernel<DUAL, WTM, WT, PF, false, BK, NW>), grid, dim3(NW * 64), lds, st, a, ExpandEpi{});
+  hipLaunchKernelGGL((gemm_tiles_kernel<DT, DUAL, WTM, WT, PF, false, BK, NW>), grid, dim3(NW * 64), lds, st, a, ExpandEpi{});
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
 }
 
-int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
+template <int DT>
+static int launch_gemm_tiles_dt(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
   const int64_t big = (int64_t)((a.N + 127) / 128) * ((a.B + 127) / 128);
   // Forms by tile count (measured on the projections of the 7B shape at 128..4096 rows).  The pair kernel: the
   // eight-wave 128 x 128 form from two big tiles per compute unit on, else 64 x 64.  A single matrix: 128 x 128 from
@@ -560,32 +562,32 @@ int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* 
   // with one workgroup or less per compute unit and a long K only loads issued several steps ahead hide the latency.
   // The pair at four big tiles per compute unit and more: four waves with both accumulator sets, K steps of 32
   // loaded straight into LDS (two workgroups per compute unit; 243 -> 214 us at 2048 rows of the 7B MLP)
-  if (dual && big >= 1024) return launch_gemm_tiles_t<true, 4, 4, 32, 4, -2>(a, st, who);
-  if (dual && big >= 512) return launch_gemm_tiles_t<true, 4, 4, 64, 8>(a, st, who);
+  if (dual && big >= 1024) return launch_gemm_tiles_t<DT, true, 4, 4, 32, 4, -2>(a, st, who);
+  if (dual && big >= 512) return launch_gemm_tiles_t<DT, true, 4, 4, 64, 8>(a, st, who);
   // two and a half to four 64 x 128 tiles per compute unit: that tile, K steps of 32 straight into LDS, three
   // workgroups per compute unit (7B MLP at 512 rows 83 -> 77 us, at 768 rows 114 -> 110; slower outside this range)
   const int64_t wide = (int64_t)((a.N + 127) / 128) * ((a.B + 63) / 64);
-  if (dual && wide >= 640 && wide <= 1100) return launch_gemm_tiles_t<true, 2, 4, 32, 4, -2>(a, st, who);
-  if (dual) return launch_gemm_tiles_t<true, 2, 2, 64>(a, st, who);
+  if (dual && wide >= 640 && wide <= 1100) return launch_gemm_tiles_t<DT, true, 2, 4, 32, 4, -2>(a, st, who);
+  if (dual) return launch_gemm_tiles_t<DT, true, 2, 2, 64>(a, st, who);
   // a single matrix with more than one big tile per compute unit: loads straight into LDS, two stages (the second and
   // third workgroup of a compute unit cover the one-step load distance; 5..8 % faster than the register pipeline with
   // weights that come from HBM, and slower than it below these tile counts)
   // many tiles per compute unit (long prompts): 128 x 256 tiles, a wave on 64 x 128 of it -- a third fewer fragment
   // reads from LDS per product; K steps of 32 keep two workgroups per compute unit (16384 rows of the 7B shape at
   // ratio 0.8: 1..6 % faster per projection, same results bit for bit)
-  if (big >= 2048) return launch_gemm_tiles_t<false, 4, 8, 32, 4, -2>(a, st, who);
-  if (big >= 448) return launch_gemm_tiles_t<false, 4, 4, 64, 4, -2>(a, st, who);
-  if (big >= 320) return launch_gemm_tiles_t<false, 4, 2, 64, 4, -2>(a, st, who);
+  if (big >= 2048) return launch_gemm_tiles_t<DT, false, 4, 8, 32, 4, -2>(a, st, who);
+  if (big >= 448) return launch_gemm_tiles_t<DT, false, 4, 4, 64, 4, -2>(a, st, who);
+  if (big >= 320) return launch_gemm_tiles_t<DT, false, 4, 2, 64, 4, -2>(a, st, who);
   // about one tile per compute unit: eight waves on a 128 x 128 or 128 x 64 tile, each half of them on half of the k
   // slices of a step, so that a workgroup alone on its compute unit still runs two waves per SIMD (rank projections at
   // 512 rows 36 -> 29 us, at 1024 rows 50 -> 43; down_v at 2048 rows 131 -> 109; with fewer tiles than ~0.6 per
   // compute unit the 64 x 64 tiles below win, with more the four-wave forms that share a compute unit)
-  if (big >= 144 && big <= 256) return launch_gemm_tiles_t<false, 4, 4, 64, 8>(a, st, who);
-  if (big >= 256) return launch_gemm_tiles_t<false, 4, 2, 64>(a, st, who);
+  if (big >= 144 && big <= 256) return launch_gemm_tiles_t<DT, false, 4, 4, 64, 8>(a, st, who);
+  if (big >= 256) return launch_gemm_tiles_t<DT, false, 4, 2, 64>(a, st, who);
   const int64_t half = (int64_t)((a.N + 63) / 64) * ((a.B + 127) / 128);
-  if (half >= 160 && half <= 256 && (a.K % 128) == 0) return launch_gemm_tiles_t<false, 4, 2, 128, 8>(a, st, who);
+  if (half >= 160 && half <= 256 && (a.K % 128) == 0) return launch_gemm_tiles_t<DT, false, 4, 2, 128, 8>(a, st, who);
   const int64_t small = (int64_t)((a.N + 63) / 64) * ((a.B + 63) / 64);
-  return (small < 320 && (a.K % 128) == 0) ? launch_gemm_tiles_t<false, 2, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 2, 2, 64>(a, st, who);
+  return (small < 320 && (a.K % 128) == 0) ? launch_gemm_tiles_t<DT, false, 2, 2, 128>(a, st, who) : launch_gemm_tiles_t<DT, false, 2, 2, 64>(a, st, who);
 }
 
 // 17..127 rows (batched decoding): 32-row tiles, 64 columns wide, K split over workgroups.  Needs the registered
@@ -598,9 +600,17 @@ bool gemm_rows_apply(const MfmaArgs& a) {
   return rows && a.B < 128 && (a.K % kGBK) == 0 && (a.ldw % 8) == 0 && (a.ldx % 8) == 0 && (a.up_off % 8) == 0 &&
          split_workspace().part != nullptr;
 }
+int launch_gemm_tiles(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
+  return a.dt == 1 ? launch_gemm_tiles_dt<1>(a, dual, st, who) : launch_gemm_tiles_dt<0>(a, dual, st, who);
+}
+template <int DT>
+static int launch_gemm_rows_dt(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
+  if (dual) return launch_gemm_tiles_t<DT, true, 1, 2, 64>(a, st, who);
+  return (a.K % 128) == 0 ? launch_gemm_tiles_t<DT, false, 1, 2, 128>(a, st, who) : launch_gemm_tiles_t<DT, false, 1, 2, 64>(a, st, who);
+}
+
 int launch_gemm_rows(const MfmaArgs& a, bool dual, hipStream_t st, const char* who) {
-  if (dual) return launch_gemm_tiles_t<true, 1, 2, 64>(a, st, who);
-  return (a.K % 128) == 0 ? launch_gemm_tiles_t<false, 1, 2, 128>(a, st, who) : launch_gemm_tiles_t<false, 1, 2, 64>(a, st, who);
+  return a.dt == 1 ? launch_gemm_rows_dt<1>(a, dual, st, who) : launch_gemm_rows_dt<0>(a, dual, st, who);
 }
 
 // head expansion of the prefill on the tiled kernel: 128 token rows and more, head_dim 128, rank a multiple of 64,
@@ -610,7 +620,7 @@ bool expand_tiles_apply(const ExpandArgs& a) {
          (a.ldu % 8) == 0;
 }
 
-template <int WTM>
+template <int DT, int WTM>
 static int launch_expand_tiles_t(const ExpandArgs& a, hipStream_t st) {
   const char* who = "fsvd_lowrank_expand_heads";
   static bool granted = false;
@@ -619,7 +629,7 @@ static int launch_expand_tiles_t(const ExpandArgs& a, hipStream_t st) {
   constexpr int BM = 32 * WTM;
   const size_t lds = (size_t)2 * (BM + 128) * kGLd * 2;
   if (!granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<false, WTM, 4, PF, true, kGBK, 4>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<DT, false, WTM, 4, PF, true, kGBK, 4>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
@@ -628,20 +638,20 @@ static int launch_expand_tiles_t(const ExpandArgs& a, hipStream_t st) {
   MfmaArgs g{a.p, 0, 0, a.u, nullptr, a.ldu, a.bias, nullptr, 0, a.y, 0, rows, a.heads * 128, a.R, 0};
   ExpandEpi ep{a.cos, a.sin, a.rope_len, a.positions, a.M, a.sp_b, a.sp_m, a.sy_b, a.sy_m, a.sy_h, a.dst_by_position, a.dst_rows};
   const dim3 grid(a.heads, (rows + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_tiles_kernel<false, WTM, 4, PF, true, kGBK, 4>), grid, dim3(kGT4), lds, st, g, ep);
+  hipLaunchKernelGGL((gemm_tiles_kernel<DT, false, WTM, 4, PF, true, kGBK, 4>), grid, dim3(kGT4), lds, st, g, ep);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
 }
 
-template <int WTM>
+template <int DT, int WTM>
 static int launch_expand_multi_t(const ExpandArgs* d, int n, hipStream_t st) {
   const char* who = "fsvd_lowrank_expand_heads_multi";
   static bool granted = false;
   constexpr int BM = 32 * WTM;
   const size_t lds = (size_t)2 * (BM + 128) * kGBK * 2;
   if (!granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&expand_multi_kernel<WTM>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&expand_multi_kernel<DT, WTM>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
   }
@@ -658,7 +668,7 @@ static int launch_expand_multi_t(const ExpandArgs* d, int n, hipStream_t st) {
   eb.first_head[3] = heads;
   for (int k = n; k < 3; ++k) eb.first_head[k] = heads;    // unused sets start past the last head
   const dim3 grid(heads, (rows + BM - 1) / BM);
-  hipLaunchKernelGGL(expand_multi_kernel<WTM>, grid, dim3(kGT4), lds, st, eb);
+  hipLaunchKernelGGL((expand_multi_kernel<DT, WTM>), grid, dim3(kGT4), lds, st, eb);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
@@ -668,20 +678,22 @@ static int launch_expand_multi_t(const ExpandArgs* d, int n, hipStream_t st) {
 bool expand_multi_apply(const ExpandArgs* d, int n) {
   if (n < 2 || n > 3) return false;
   for (int k = 0; k < n; ++k)
-    if (!expand_tiles_apply(d[k]) || d[k].B != d[0].B || d[k].M != d[0].M) return false;
+    if (!expand_tiles_apply(d[k]) || d[k].B != d[0].B || d[k].M != d[0].M || d[k].dt != d[0].dt) return false;
   return true;
 }
 int launch_expand_multi(const ExpandArgs* d, int n, hipStream_t st) {
   int heads = 0;
   for (int k = 0; k < n; ++k) heads += d[k].heads;
   const int64_t big = (int64_t)heads * (((int64_t)d[0].B * d[0].M + 127) / 128);
-  return big >= 384 ? launch_expand_multi_t<4>(d, n, st) : launch_expand_multi_t<2>(d, n, st);
+  if (d[0].dt == 1) return big >= 384 ? launch_expand_multi_t<1, 4>(d, n, st) : launch_expand_multi_t<1, 2>(d, n, st);
+  return big >= 384 ? launch_expand_multi_t<0, 4>(d, n, st) : launch_expand_multi_t<0, 2>(d, n, st);
 }
 
 int launch_expand_tiles(const ExpandArgs& a, hipStream_t st) {
   // a column tile is always one head; 128 token rows per workgroup when that gives every compute unit two tiles, else 64
   const int64_t big = (int64_t)a.heads * (((int64_t)a.B * a.M + 127) / 128);
-  return big >= 384 ? launch_expand_tiles_t<4>(a, st) : launch_expand_tiles_t<2>(a, st);
+  if (a.dt == 1) return big >= 384 ? launch_expand_tiles_t<1, 4>(a, st) : launch_expand_tiles_t<1, 2>(a, st);
+  return big >= 384 ? launch_expand_tiles_t<0, 4>(a, st) : launch_expand_tiles_t<0, 2>(a, st);
 }
 
 }  // namespace fsvd

@@ -16,24 +16,26 @@
 
 namespace fsvd {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) u32x4_t* gp16_t;
 
 constexpr int kMfThreads = 512;
 constexpr int kMfWaves = kMfThreads / 64;
 
-__device__ __forceinline__ bf16x8_t ldw_frag(const uint16_t* p) {
-  return __builtin_bit_cast(bf16x8_t, __builtin_nontemporal_load((gp16_t)(uintptr_t)p));
+template <class F>
+__device__ __forceinline__ F ldw_frag(const uint16_t* p) {
+  return __builtin_bit_cast(F, __builtin_nontemporal_load((gp16_t)(uintptr_t)p));
 }
-__device__ __forceinline__ bf16x8_t ldx_frag(const uint16_t* p) {
-  return __builtin_bit_cast(bf16x8_t, *(gp16_t)(uintptr_t)p);
+template <class F>
+__device__ __forceinline__ F ldx_frag(const uint16_t* p) {
+  return __builtin_bit_cast(F, *(gp16_t)(uintptr_t)p);
 }
 
 
 // the waves' partial tiles through LDS, added in wave order, then the epilogue of the vector kernels
-template <int NB, bool DUAL, int KS>
+template <int DT, int NB, bool DUAL, int KS>
 __device__ __forceinline__ void mfma_finish(const MfmaArgs& a, float (*red)[DUAL ? 2 : 1][NB][4][64], const f32x4_t (&acc)[DUAL ? 2 : 1][NB]) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   constexpr int NM = DUAL ? 2 : 1;
   constexpr int RT = kMfWaves / KS;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -60,18 +62,18 @@ __device__ __forceinline__ void mfma_finish(const MfmaArgs& a, float (*red)[DUAL
     float v;
     if (DUAL) {
       if (a.mode == 0) {
-        v0 = round_bf16(v0);
-        v1 = round_bf16(v1);
-        v = round_bf16(round_bf16(silu_f32(v0)) * v1);
+        v0 = E::rnd(v0);
+        v1 = E::rnd(v1);
+        v = E::rnd(E::rnd(silu_f32(v0)) * v1);
       } else {
-        v = round_bf16((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
+        v = E::rnd((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
       }
     } else {
-      if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
-      v = round_bf16(v0);
-      if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)b * a.ldres + n]) + v);
+      if (a.bias) v0 += E::val(a.bias[n]);
+      v = E::rnd(v0);
+      if (a.res) v = E::rnd(E::val(a.res[(int64_t)b * a.ldres + n]) + v);
     }
-    a.y[(int64_t)b * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+    a.y[(int64_t)b * a.ldy + n] = (uint16_t)E::bits(v);
   }
 }
 
@@ -80,10 +82,12 @@ __device__ __forceinline__ void mfma_finish(const MfmaArgs& a, float (*red)[DUAL
 // acknowledged, and the last workgroup to arrive adds the gridDim.y shares in split order (its own included, so the sum
 // does not depend on who came last) through agent-scope loads, all in flight at once, then applies the epilogue.  No
 // fence: a release or acquire fence writes back or empties a whole L2 under the weight streams of the other workgroups.
-template <int NB, int KS>
+template <int DT, int NB, int KS>
 __device__ __forceinline__ void mfma_finish_split(const MfmaArgs& a, float (*red)[1][NB][4][64], const f32x4_t (&acc)[1][NB]) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   constexpr int RT = kMfWaves / KS;
-  constexpr int E = RT * NB * 256;                 // output elements of this workgroup
+  constexpr int NE = RT * NB * 256;                 // output elements of this workgroup
   constexpr int kMaxZ = 8;
   __shared__ int last_flag;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -93,14 +97,14 @@ __device__ __forceinline__ void mfma_finish_split(const MfmaArgs& a, float (*red
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[wave][0][t][i][lane] = acc[0][t][i];
   __syncthreads();
-  uint32_t* part = reinterpret_cast<uint32_t*>(a.ws_part) + (size_t)blockIdx.x * Z * E;
-  for (int o = tid; o < E; o += kMfThreads) {
+  uint32_t* part = reinterpret_cast<uint32_t*>(a.ws_part) + (size_t)blockIdx.x * Z * NE;
+  for (int o = tid; o < NE; o += kMfThreads) {
     const int q = o / (NB * 256), oo = o - q * (NB * 256);
     const int t = oo >> 8, r = oo & 255, i = r >> 6, l = r & 63;
     float v0 = 0.f;
 #pragma unroll
     for (int w = 0; w < KS; ++w) v0 += red[q * KS + w][0][t][i][l];
-    __hip_atomic_store(part + (size_t)blockIdx.y * E + o, __float_as_uint(v0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(part + (size_t)blockIdx.y * NE + o, __float_as_uint(v0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
@@ -112,29 +116,31 @@ __device__ __forceinline__ void mfma_finish_split(const MfmaArgs& a, float (*red
   }
   __syncthreads();
   if (last_flag == 0) return;
-  for (int o = tid; o < E; o += kMfThreads) {
+  for (int o = tid; o < NE; o += kMfThreads) {
     const int q = o / (NB * 256), oo = o - q * (NB * 256);
     const int t = oo >> 8, r = oo & 255, i = r >> 6, l = r & 63;
     const int n = (blockIdx.x * RT + q) * 16 + (l >> 4) * 4 + i, b = t * 16 + (l & 15);
     uint32_t sh[kMaxZ];
 #pragma unroll
-    for (int z = 0; z < kMaxZ; ++z) sh[z] = __hip_atomic_load(part + (size_t)min(z, Z - 1) * E + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int z = 0; z < kMaxZ; ++z) sh[z] = __hip_atomic_load(part + (size_t)min(z, Z - 1) * NE + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     float v0 = 0.f;
 #pragma unroll
     for (int z = 0; z < kMaxZ; ++z)
       if (z < Z) v0 += __uint_as_float(sh[z]);
     if (n >= a.N || b >= a.B) continue;
-    if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
-    float v = round_bf16(v0);
-    if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)b * a.ldres + n]) + v);
-    a.y[(int64_t)b * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+    if (a.bias) v0 += E::val(a.bias[n]);
+    float v = E::rnd(v0);
+    if (a.res) v = E::rnd(E::val(a.res[(int64_t)b * a.ldres + n]) + v);
+    a.y[(int64_t)b * a.ldy + n] = (uint16_t)E::bits(v);
   }
 }
 
 // NB: 16-row batch tiles (B <= 16 * NB); KS: waves that split K for one 16-row weight tile, so a workgroup
 // of 8 waves covers 8 / KS weight tiles
-template <int NB, bool DUAL, int KS>
+template <int DT, int NB, bool DUAL, int KS>
 __global__ __launch_bounds__(kMfThreads) void mfma_linear_kernel(MfmaArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   constexpr int NM = DUAL ? 2 : 1;
   constexpr int RT = kMfWaves / KS;
   __shared__ float red[kMfWaves][NM][NB][4][64];
@@ -159,32 +165,32 @@ __global__ __launch_bounds__(kMfThreads) void mfma_linear_kernel(MfmaArgs a) {
   // four k-steps per trip, all loads of a trip requested before the first product; steps past the end of
   // this wave's slice read the last step again and contribute zero
   constexpr int UN = 4;
-  const bf16x8_t zero = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+  const frag_t zero = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
   for (int s = s0; s < s1; s += UN) {
-    bf16x8_t fa0[UN], fa1[UN], fb0[UN][NB], fb1[UN][NB];
+    frag_t fa0[UN], fa1[UN], fb0[UN][NB], fb1[UN][NB];
 #pragma unroll
     for (int j = 0; j < UN; ++j) {
       const int k = (min(s + j, s1 - 1) * KS + ks) << 5;
-      fa0[j] = ldw_frag(w0 + k);
-      if (DUAL) fa1[j] = ldw_frag(w1 + k);
+      fa0[j] = ldw_frag<frag_t>(w0 + k);
+      if (DUAL) fa1[j] = ldw_frag<frag_t>(w1 + k);
 #pragma unroll
       for (int t = 0; t < NB; ++t) {
-        fb0[j][t] = ldx_frag(xr[t] + k);
-        if (DUAL) fb1[j][t] = ldx_frag(xr[t] + a.up_off + k);
+        fb0[j][t] = ldx_frag<frag_t>(xr[t] + k);
+        if (DUAL) fb1[j][t] = ldx_frag<frag_t>(xr[t] + a.up_off + k);
       }
     }
 #pragma unroll
     for (int j = 0; j < UN; ++j) {
       const bool live = s + j < s1;
-      const bf16x8_t a0 = live ? fa0[j] : zero;
+      const frag_t a0 = live ? fa0[j] : zero;
 #pragma unroll
       for (int t = 0; t < NB; ++t) {
-        acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, fb0[j][t], acc[0][t], 0, 0, 0);
-        if (DUAL) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(live ? fa1[j] : zero, fb1[j][t], acc[1][t], 0, 0, 0);
+        acc[0][t] = E::mfma(a0, fb0[j][t], acc[0][t]);
+        if (DUAL) acc[1][t] = E::mfma(live ? fa1[j] : zero, fb1[j][t], acc[1][t]);
       }
     }
   }
-  mfma_finish<NB, DUAL, KS>(a, red, acc);
+  mfma_finish<DT, NB, DUAL, KS>(a, red, acc);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -205,8 +211,10 @@ template <bool DUAL> struct StreamShape {
 // D: chunks in a wave's ring (D - 1 in flight while one multiplies)
 // ZS: K also split over the gridDim.y workgroups of a tile (single matrix; narrow projections that would otherwise
 // leave compute units idle): the KS waves of workgroup z act as waves z * KS .. z * KS + KS - 1 of KS * gridDim.y
-template <bool DUAL, int KS, int D, int NB, bool ZS = false>
+template <int DT, bool DUAL, int KS, int D, int NB, bool ZS = false>
 __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   static_assert(!ZS || !DUAL, "the split over workgroups is built for a single matrix");
   typedef StreamShape<DUAL> SS;
   constexpr int NM = SS::NM, CKB = SS::CKB, kStage = SS::kStage;
@@ -240,7 +248,7 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
   const uint16_t* xsrc[NB];
 #pragma unroll
   for (int t = 0; t < NB; ++t) xsrc[t] = a.x + (int64_t)min(t * 16 + lr, a.B - 1) * a.ldx + lg * 8;
-  bf16x8_t xf[D][NM][KST][NB];
+  frag_t xf[D][NM][KST][NB];
   // The wave's load counter is the only synchronisation: it counts weight pieces and activation fragments alike, in
   // issue order, so the loads of one chunk must stay together in the instruction stream (scheduling fences around them).
   const auto issue = [&](int c, int slot) {
@@ -254,7 +262,7 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
 #pragma unroll
       for (int s = 0; s < KST; ++s)
 #pragma unroll
-        for (int t = 0; t < NB; ++t) xf[slot][m][s][t] = ldx_frag(xsrc[t] + (m ? a.up_off : 0) + k0 + s * 32);
+        for (int t = 0; t < NB; ++t) xf[slot][m][s][t] = ldx_frag<frag_t>(xsrc[t] + (m ? a.up_off : 0) + k0 + s * 32);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -286,15 +294,15 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
       for (int s = 0; s < KST; ++s)
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
-          const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(ring + u * kStage + m * 16 * CKB + lr * CKB + (((s * 4 + lg) ^ (lr % PPR)) * 16));
+          const frag_t wf = *reinterpret_cast<const frag_t*>(ring + u * kStage + m * 16 * CKB + lr * CKB + (((s * 4 + lg) ^ (lr % PPR)) * 16));
 #pragma unroll
-          for (int t = 0; t < NB; ++t) acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[u][m][s][t], acc[m][t], 0, 0, 0);
+          for (int t = 0; t < NB; ++t) acc[m][t] = E::mfma(wf, xf[u][m][s][t], acc[m][t]);
         }
     }
   }
   __syncthreads();                                 // every wave is done with its ring: the partial tiles take its place
-  if constexpr (ZS) mfma_finish_split<NB, KS>(a, red, acc);
-  else mfma_finish<NB, DUAL, KS>(a, red, acc);
+  if constexpr (ZS) mfma_finish_split<DT, NB, KS>(a, red, acc);
+  else mfma_finish<DT, NB, DUAL, KS>(a, red, acc);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -308,13 +316,15 @@ __global__ __launch_bounds__(kMfThreads) void mfma_stream_kernel(MfmaArgs a) {
 // outstanding loads — the chunk requested ahead included — before every second product.
 // ---------------------------------------------------------------------------------------------
 constexpr int kResPitch = 68;                      // floats between the four row groups of a parked tile: conflict-free reads below
-template <bool DUAL, int NB, int CW, int D>
+template <int DT, bool DUAL, int NB, int CW, int D>
 __global__ __launch_bounds__(kMfThreads) void mfma_resident_kernel(MfmaArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   typedef StreamShape<DUAL> SS;
   constexpr int NM = SS::NM, CKB = SS::CKB, kStage = SS::kStage;
   constexpr int PPR = CKB / 16, KST = CKB / 64, RPI = 64 / PPR, NI = 16 / RPI;
   constexpr int kGroup = NM * NI;                  // loads per chunk
-  constexpr int E = NB * 256;                      // output elements of a tile
+  constexpr int NE = NB * 256;                      // output elements of a tile
   static_assert(D >= 2 && D <= 4 && 3 * kGroup < 64, "the waits below cover up to three groups in flight");
   extern __shared__ __align__(16) unsigned char st_smem[];     // [8 waves][D][kStage], then the parked partial tiles
   constexpr int kRedWave = NM * NB * 4 * kResPitch;
@@ -354,8 +364,8 @@ __global__ __launch_bounds__(kMfThreads) void mfma_resident_kernel(MfmaArgs a) {
   for (int p = 0; p < D; ++p)
     if (issued < total) issue();
   // the wave's activation fragments, requested behind the first weight stages so that both are on their way together
-  bf16x8_t xf[CW][NM][KST][NB];
-  const bf16x8_t zero = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+  frag_t xf[CW][NM][KST][NB];
+  const frag_t zero = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
 #pragma unroll
   for (int c = 0; c < CW; ++c)
 #pragma unroll
@@ -364,7 +374,7 @@ __global__ __launch_bounds__(kMfThreads) void mfma_resident_kernel(MfmaArgs a) {
       for (int s = 0; s < KST; ++s)
 #pragma unroll
         for (int t = 0; t < NB; ++t)
-          xf[c][m][s][t] = c < cw ? ldx_frag(a.x + (int64_t)min(t * 16 + lr, a.B - 1) * a.ldx + lg * 8 + (m ? a.up_off : 0) +
+          xf[c][m][s][t] = c < cw ? ldx_frag<frag_t>(a.x + (int64_t)min(t * 16 + lr, a.B - 1) * a.ldx + lg * 8 + (m ? a.up_off : 0) +
                                              (int64_t)(c * kMfWaves + wave) * (CKB / 2) + s * 32)
                                   : zero;
   __builtin_amdgcn_s_waitcnt(0);                   // (the first stages land with them) from here on the load counter counts weight pieces only
@@ -396,9 +406,9 @@ __global__ __launch_bounds__(kMfThreads) void mfma_resident_kernel(MfmaArgs a) {
         for (int s = 0; s < KST; ++s)
 #pragma unroll
           for (int m = 0; m < NM; ++m) {
-            const bf16x8_t wf = *reinterpret_cast<const bf16x8_t*>(ring + cslot * kStage + m * 16 * CKB + lr * CKB + (((s * 4 + lg) ^ (lr % PPR)) * 16));
+            const frag_t wf = *reinterpret_cast<const frag_t*>(ring + cslot * kStage + m * 16 * CKB + lr * CKB + (((s * 4 + lg) ^ (lr % PPR)) * 16));
 #pragma unroll
-            for (int t = 0; t < NB; ++t) acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[c][m][s][t], acc[m][t], 0, 0, 0);
+            for (int t = 0; t < NB; ++t) acc[m][t] = E::mfma(wf, xf[c][m][s][t], acc[m][t]);
           }
         ++done;
         cslot = cslot + 1 == D ? 0 : cslot + 1;
@@ -420,7 +430,7 @@ __global__ __launch_bounds__(kMfThreads) void mfma_resident_kernel(MfmaArgs a) {
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     const int n = (g + ti * G) * 16 + nn;
-    if (tid < E) {
+    if (tid < NE) {
       float v0 = 0.f, v1 = 0.f;
 #pragma unroll
       for (int w = 0; w < kMfWaves; ++w) {
@@ -431,18 +441,18 @@ __global__ __launch_bounds__(kMfThreads) void mfma_resident_kernel(MfmaArgs a) {
         float v;
         if (DUAL) {
           if (a.mode == 0) {
-            v0 = round_bf16(v0);
-            v1 = round_bf16(v1);
-            v = round_bf16(round_bf16(silu_f32(v0)) * v1);
+            v0 = E::rnd(v0);
+            v1 = E::rnd(v1);
+            v = E::rnd(E::rnd(silu_f32(v0)) * v1);
           } else {
-            v = round_bf16((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
+            v = E::rnd((v0 * (1.0f / (1.0f + expf(-v0)))) * v1);
           }
         } else {
-          if (a.bias) v0 += bf16_bits_to_f32(a.bias[n]);
-          v = round_bf16(v0);
-          if (a.res) v = round_bf16(bf16_bits_to_f32(a.res[(int64_t)b * a.ldres + n]) + v);
+          if (a.bias) v0 += E::val(a.bias[n]);
+          v = E::rnd(v0);
+          if (a.res) v = E::rnd(E::val(a.res[(int64_t)b * a.ldres + n]) + v);
         }
-        a.y[(int64_t)b * a.ldy + n] = (uint16_t)f32_to_bf16_bits(v);
+        a.y[(int64_t)b * a.ldy + n] = (uint16_t)E::bits(v);
       }
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);            // the sums are in registers before the next tile's partials overwrite them
@@ -477,43 +487,43 @@ static bool resident_applies(const MfmaArgs& a) {
   const int nchunk = a.K / ck;
   return (a.N + 15) / 16 >= 2 * cu && nchunk >= kMfWaves && nchunk <= kMfWaves * kResidentCW;
 }
-template <bool DUAL, int NB, int CW>
+template <int DT, bool DUAL, int NB, int CW>
 static int launch_mfma_resident_t(const MfmaArgs& a, hipStream_t st, const char* who) {
   static bool granted = false;
   constexpr int D = 3;
   constexpr int NM = StreamShape<DUAL>::NM;
   const size_t lds = (size_t)kMfWaves * D * StreamShape<DUAL>::kStage + (size_t)kMfWaves * NM * NB * 4 * kResPitch * sizeof(float);
-  const void* f = reinterpret_cast<const void*>(&mfma_resident_kernel<DUAL, NB, CW, D>);
+  const void* f = reinterpret_cast<const void*>(&mfma_resident_kernel<DT, DUAL, NB, CW, D>);
   if (!granted) {
     hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = true;
   }
   const int G = std::min(compute_units(), (a.N + 15) / 16);
-  hipLaunchKernelGGL((mfma_resident_kernel<DUAL, NB, CW, D>), dim3(G), dim3(kMfThreads), lds, st, a);
+  hipLaunchKernelGGL((mfma_resident_kernel<DT, DUAL, NB, CW, D>), dim3(G), dim3(kMfThreads), lds, st, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
 }
-template <bool DUAL, int NB>
+template <int DT, bool DUAL, int NB>
 static int launch_mfma_resident_nb(const MfmaArgs& a, hipStream_t st, const char* who) {
   const int per = (a.K / (StreamShape<DUAL>::CKB / 2) + kMfWaves - 1) / kMfWaves;   // chunks of the busiest wave
-  if (per <= 2) return launch_mfma_resident_t<DUAL, NB, 2>(a, st, who);
-  if (per <= 4) return launch_mfma_resident_t<DUAL, NB, 4>(a, st, who);
-  return launch_mfma_resident_t<DUAL, NB, 6>(a, st, who);
+  if (per <= 2) return launch_mfma_resident_t<DT, DUAL, NB, 2>(a, st, who);
+  if (per <= 4) return launch_mfma_resident_t<DT, DUAL, NB, 4>(a, st, who);
+  return launch_mfma_resident_t<DT, DUAL, NB, 6>(a, st, who);
 }
-template <bool DUAL>
+template <int DT, bool DUAL>
 static int launch_mfma_resident(const MfmaArgs& a, hipStream_t st, const char* who) {
-  return a.B <= 16 ? launch_mfma_resident_nb<DUAL, 1>(a, st, who) : launch_mfma_resident_nb<DUAL, 2>(a, st, who);
+  return a.B <= 16 ? launch_mfma_resident_nb<DT, DUAL, 1>(a, st, who) : launch_mfma_resident_nb<DT, DUAL, 2>(a, st, who);
 }
 
-template <int NB, bool DUAL>
+template <int DT, int NB, bool DUAL>
 static void launch_mfma_ks(const MfmaArgs& a, int ks, hipStream_t st) {
   const int tiles = (a.N + 15) / 16;
   const dim3 block(kMfThreads);
-  if (ks == 2) hipLaunchKernelGGL((mfma_linear_kernel<NB, DUAL, 2>), dim3((tiles + 3) / 4), block, 0, st, a);
-  else if (ks == 4) hipLaunchKernelGGL((mfma_linear_kernel<NB, DUAL, 4>), dim3((tiles + 1) / 2), block, 0, st, a);
-  else hipLaunchKernelGGL((mfma_linear_kernel<NB, DUAL, 8>), dim3(tiles), block, 0, st, a);
+  if (ks == 2) hipLaunchKernelGGL((mfma_linear_kernel<DT, NB, DUAL, 2>), dim3((tiles + 3) / 4), block, 0, st, a);
+  else if (ks == 4) hipLaunchKernelGGL((mfma_linear_kernel<DT, NB, DUAL, 4>), dim3((tiles + 1) / 2), block, 0, st, a);
+  else hipLaunchKernelGGL((mfma_linear_kernel<DT, NB, DUAL, 8>), dim3(tiles), block, 0, st, a);
 }
 
 // the streaming form: up to 16 rows, K a whole number of chunks with at least one chunk per wave of a tile
@@ -522,7 +532,7 @@ static bool stream_applies(const MfmaArgs& a, int ks) {
   constexpr int ck = StreamShape<DUAL>::CKB / 2;
   return a.B <= 32 && (a.K % ck) == 0 && a.K / ck >= ks;
 }
-template <bool DUAL, int D, int NB>
+template <int DT, bool DUAL, int D, int NB>
 static int launch_mfma_stream_d(const MfmaArgs& a, int ks, hipStream_t st, const char* who) {
   static bool granted[3] = {false, false, false};
   const int tiles = (a.N + 15) / 16;
@@ -535,14 +545,14 @@ static int launch_mfma_stream_d(const MfmaArgs& a, int ks, hipStream_t st, const
   };
   const dim3 block(kMfThreads);
   if (ks == 2) {
-    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 2, D, NB>), 0)) return kErrLaunch;
-    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 2, D, NB>), dim3((tiles + 3) / 4), block, lds, st, a);
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DT, DUAL, 2, D, NB>), 0)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DT, DUAL, 2, D, NB>), dim3((tiles + 3) / 4), block, lds, st, a);
   } else if (ks == 4) {
-    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 4, D, NB>), 1)) return kErrLaunch;
-    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 4, D, NB>), dim3((tiles + 1) / 2), block, lds, st, a);
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DT, DUAL, 4, D, NB>), 1)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DT, DUAL, 4, D, NB>), dim3((tiles + 1) / 2), block, lds, st, a);
   } else {
-    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DUAL, 8, D, NB>), 2)) return kErrLaunch;
-    hipLaunchKernelGGL((mfma_stream_kernel<DUAL, 8, D, NB>), dim3(tiles), block, lds, st, a);
+    if (!grant(reinterpret_cast<const void*>(&mfma_stream_kernel<DT, DUAL, 8, D, NB>), 2)) return kErrLaunch;
+    hipLaunchKernelGGL((mfma_stream_kernel<DT, DUAL, 8, D, NB>), dim3(tiles), block, lds, st, a);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
@@ -551,10 +561,10 @@ static int launch_mfma_stream_d(const MfmaArgs& a, int ks, hipStream_t st, const
 // Eight waves per weight tile whenever K has a chunk for each, and a ring of two chunks: 64 KB of LDS, so two
 // workgroups share a compute unit — measured better than deeper rings with one workgroup per compute unit or fewer waves
 // per tile (7B MLP at 8 rows, ring 4 / 2: rank projection 8.9 / 7.9 us, pair 19.7 / 15.9, down_u 4.9 / 4.9).
-template <bool DUAL>
+template <int DT, bool DUAL>
 static int launch_mfma_stream(const MfmaArgs& a, int ks, hipStream_t st, const char* who) {
   if (a.K / (StreamShape<DUAL>::CKB / 2) >= 8) ks = 8;
-  return a.B <= 16 ? launch_mfma_stream_d<DUAL, 2, 1>(a, ks, st, who) : launch_mfma_stream_d<DUAL, 2, 2>(a, ks, st, who);
+  return a.B <= 16 ? launch_mfma_stream_d<DT, DUAL, 2, 1>(a, ks, st, who) : launch_mfma_stream_d<DT, DUAL, 2, 2>(a, ks, st, who);
 }
 
 // Narrow projections (fewer than 128 weight tiles, e.g. down_v of the 7B MLP: 96) at 3..32 rows: the streaming form with
@@ -574,12 +584,12 @@ static int stream_split_shares(const MfmaArgs& a) {
   while (z > 1 && (nchunk < kMfWaves * z || (size_t)tiles * z * share > ws.part_floats)) --z;
   return z;
 }
-template <int NB>
+template <int DT, int NB>
 static int launch_mfma_stream_split(const MfmaArgs& a0, int z, hipStream_t st, const char* who) {
   static bool granted = false;
   constexpr int D = 2;
   const size_t lds = (size_t)kMfWaves * D * StreamShape<false>::kStage;
-  const void* f = reinterpret_cast<const void*>(&mfma_stream_kernel<false, 8, D, NB, true>);
+  const void* f = reinterpret_cast<const void*>(&mfma_stream_kernel<DT, false, 8, D, NB, true>);
   if (!granted && lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", who, lds, hipGetErrorString(e)); return kErrLaunch; }
@@ -590,13 +600,13 @@ static int launch_mfma_stream_split(const MfmaArgs& a0, int z, hipStream_t st, c
   a.ksplit = z;
   a.ws_part = ws.part;
   a.ws_count = ws.count;
-  hipLaunchKernelGGL((mfma_stream_kernel<false, 8, D, NB, true>), dim3((a.N + 15) / 16, z), dim3(kMfThreads), lds, st, a);
+  hipLaunchKernelGGL((mfma_stream_kernel<DT, false, 8, D, NB, true>), dim3((a.N + 15) / 16, z), dim3(kMfThreads), lds, st, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
 }
 
-template <bool DUAL>
+template <int DT, bool DUAL>
 static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
   // K is split over as few waves as still give every compute unit a workgroup: long slices amortise the
   // reduction, but a small matrix needs all eight waves of a workgroup on one weight tile to fill the chip
@@ -610,11 +620,11 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
   // rows on (up to 32 rows the streaming form is faster: 12.3 / 25.3 / 6.7 us against 13.4 / 28.8 / 8.8 us on the wide
   // matrices of the 7B MLP; matrices with fewer than 128 weight tiles take its split form above, or the 32-row tiles
   // when their K does not divide into chunks)
-  if (resident_applies<DUAL>(a0)) return launch_mfma_resident<DUAL>(a0, st, who);
+  if (resident_applies<DUAL>(a0)) return launch_mfma_resident<DT, DUAL>(a0, st, who);
   const bool streamed = a0.B <= 32 && tiles >= 128 && stream_applies<DUAL>(a0, ks);
   if constexpr (!DUAL) {
     const int z = stream_split_shares(a0);
-    if (z > 1) return a0.B <= 16 ? launch_mfma_stream_split<1>(a0, z, st, who) : launch_mfma_stream_split<2>(a0, z, st, who);
+    if (z > 1) return a0.B <= 16 ? launch_mfma_stream_split<DT, 1>(a0, z, st, who) : launch_mfma_stream_split<DT, 2>(a0, z, st, who);
   }
   if (gemm_rows_apply(a0) && !streamed) return launch_gemm_rows(a0, DUAL, st, who);
   // batches above 64 rows go in slices of 64
@@ -626,14 +636,14 @@ static int launch_mfma(const MfmaArgs& a0, hipStream_t st, const char* who) {
     if (a0.res) a.res = a0.res + (int64_t)b0 * a0.ldres;
     const int nb = (a.B + 15) / 16;
     if (nb <= 2 && stream_applies<DUAL>(a, ks)) {
-      const int rc = launch_mfma_stream<DUAL>(a, ks, st, who);
+      const int rc = launch_mfma_stream<DT, DUAL>(a, ks, st, who);
       if (rc != kOk) return rc;
       continue;
     }
-    if (nb == 1) launch_mfma_ks<1, DUAL>(a, ks, st);
-    else if (nb == 2) launch_mfma_ks<2, DUAL>(a, ks, st);
-    else if (nb == 3) launch_mfma_ks<3, DUAL>(a, ks, st);
-    else launch_mfma_ks<4, DUAL>(a, ks, st);
+    if (nb == 1) launch_mfma_ks<DT, 1, DUAL>(a, ks, st);
+    else if (nb == 2) launch_mfma_ks<DT, 2, DUAL>(a, ks, st);
+    else if (nb == 3) launch_mfma_ks<DT, 3, DUAL>(a, ks, st);
+    else launch_mfma_ks<DT, 4, DUAL>(a, ks, st);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_last_error("%s: launch failed: %s", who, hipGetErrorString(e)); return kErrLaunch; }
   }
@@ -648,7 +658,8 @@ bool mfma_linear_applies(const LinearArgs& a) {
 }
 int launch_linear_mfma(const LinearArgs& a, hipStream_t st) {
   MfmaArgs m{a.x, a.ldx, 0, a.W, nullptr, a.ldw, a.bias, a.res, a.ldres, a.y, a.ldy, a.B, a.N, a.K, 0};
-  return launch_mfma<false>(m, st, "fsvd_linear");
+  m.dt = a.dt;
+  return a.dt == 1 ? launch_mfma<1, false>(m, st, "fsvd_linear") : launch_mfma<0, false>(m, st, "fsvd_linear");
 }
 bool mfma_swiglu_applies(const SwigluArgs& a) {
   return a.B >= 3 && (a.R % 32) == 0 && (a.ldw % 8) == 0 && (a.ldp % 8) == 0 && (a.up_off % 8) == 0 && al16(a.gate_u) &&
@@ -656,7 +667,8 @@ bool mfma_swiglu_applies(const SwigluArgs& a) {
 }
 int launch_swiglu_mfma(const SwigluArgs& a, hipStream_t st) {
   MfmaArgs m{a.p, a.ldp, a.up_off, a.gate_u, a.up_u, a.ldw, nullptr, nullptr, 0, a.h, a.ldh, a.B, a.D, a.R, a.mode};
-  return launch_mfma<true>(m, st, "fsvd_swiglu_linear");
+  m.dt = a.dt;
+  return a.dt == 1 ? launch_mfma<1, true>(m, st, "fsvd_swiglu_linear") : launch_mfma<0, true>(m, st, "fsvd_swiglu_linear");
 }
 
 }  // namespace fsvd

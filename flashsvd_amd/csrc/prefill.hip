@@ -19,21 +19,24 @@
 
 namespace fsvd {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-
 constexpr int kPfThreads = 256;
 
-__device__ __forceinline__ bf16x8_t pf_ld(const uint16_t* p) {
-  return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(p));
+// eight elements as a matrix-core operand (F = the element type's fragment)
+template <class F>
+__device__ __forceinline__ F pf_ld(const uint16_t* p) {
+  return __builtin_bit_cast(F, *reinterpret_cast<const u32x4_t*>(p));
 }
-__device__ __forceinline__ bf16x8_t pf_zero() { return __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u}); }
+template <class F>
+__device__ __forceinline__ F pf_zero() { return __builtin_bit_cast(F, u32x4_t{0u, 0u, 0u, 0u}); }
 
 // ---------------------------------------------------------------------------------------------
 // 1. Y[token, head, :] = epilogue( P[token, (head), :] @ u[head*128 + :, :]^T )
 //    grid (ceil(T/128), heads), 4 waves x 32 tokens
 // ---------------------------------------------------------------------------------------------
+template <int DT>
 __global__ __launch_bounds__(kPfThreads) void lowrank_expand_kernel(ExpandArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   constexpr int DH = 128, NT = 8, HALF = 64;
   const int head = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -59,15 +62,15 @@ __global__ __launch_bounds__(kPfThreads) void lowrank_expand_kernel(ExpandArgs a
 #pragma unroll 2
   for (int r0 = 0; r0 < a.R; r0 += 32) {
     const bool in = r0 + lg * 8 < a.R;
-    bf16x8_t af[2], bf[NT];
+    frag_t af[2], bf[NT];
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) af[mi] = in ? pf_ld(arow[mi] + r0) : pf_zero();
+    for (int mi = 0; mi < 2; ++mi) af[mi] = in ? pf_ld<frag_t>(arow[mi] + r0) : pf_zero<frag_t>();
 #pragma unroll
-    for (int t = 0; t < NT; ++t) bf[t] = in ? pf_ld(brow + (int64_t)t * 16 * a.ldu + r0) : pf_zero();
+    for (int t = 0; t < NT; ++t) bf[t] = in ? pf_ld<frag_t>(brow + (int64_t)t * 16 * a.ldu + r0) : pf_zero<frag_t>();
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) acc[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mi], bf[t], acc[mi][t], 0, 0, 0);
+      for (int t = 0; t < NT; ++t) acc[mi][t] = E::mfma(af[mi], bf[t], acc[mi][t]);
   }
 
   // epilogue on the accumulator layout: lane holds rows lg*4+i, column t*16+lr of each tile
@@ -83,33 +86,36 @@ __global__ __launch_bounds__(kPfThreads) void lowrank_expand_kernel(ExpandArgs a
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         float v = acc[mi][t][i];
-        if (a.bias) v += bf16_bits_to_f32(a.bias[head * DH + t * 16 + lr]);
-        x[t] = round_bf16(v);                       // the projection's own rounding point
+        if (a.bias) v += E::val(a.bias[head * DH + t * 16 + lr]);
+        x[t] = E::rnd(v);                       // the projection's own rounding point
       }
       if (a.cos) {
         // eager bf16 arithmetic: x0*c - x1*s and x1*c + x0*s, one rounding per op
         const int tp = min(max(pos, 0), a.rope_len - 1);
 #pragma unroll
         for (int t = 0; t < NT / 2; ++t) {
-          const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * HALF + t * 16 + lr]);
-          const float s = bf16_bits_to_f32(a.sin[(int64_t)tp * HALF + t * 16 + lr]);
+          const float c = E::val(a.cos[(int64_t)tp * HALF + t * 16 + lr]);
+          const float s = E::val(a.sin[(int64_t)tp * HALF + t * 16 + lr]);
           const float x0 = x[t], x1 = x[t + NT / 2];
-          x[t] = round_bf16(round_bf16(x0 * c) - round_bf16(x1 * s));
-          x[t + NT / 2] = round_bf16(round_bf16(x1 * c) + round_bf16(x0 * s));
+          x[t] = E::rnd(E::rnd(x0 * c) - E::rnd(x1 * s));
+          x[t + NT / 2] = E::rnd(E::rnd(x1 * c) + E::rnd(x0 * s));
         }
       }
       const int slot = a.dst_by_position ? pos : m;
       if (slot < 0 || slot >= a.dst_rows) continue;   // outside the destination: dropped
       uint16_t* dst = a.y + (int64_t)b * a.sy_b + (int64_t)slot * a.sy_m + (int64_t)head * a.sy_h;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) dst[t * 16 + lr] = (uint16_t)f32_to_bf16_bits(x[t]);
+      for (int t = 0; t < NT; ++t) dst[t * 16 + lr] = (uint16_t)E::bits(x[t]);
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // 2. causal flash attention, head_dim 128, 64 queries per workgroup (16 per wave), 64-key tiles
 // ---------------------------------------------------------------------------------------------
+template <int DT>
 __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   constexpr int DH = 128, BN = 64, PSTR = BN + 8, VSTR = BN + 8;
   __shared__ __align__(16) uint16_t Ps[4][16][PSTR];    // softmax weights, bf16 high part
   __shared__ __align__(16) uint16_t Pl[4][16][PSTR];    // and the bf16 residual, so that P carries ~16 mantissa bits
@@ -124,12 +130,12 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
   const int n_keys_all = max(1, min(q0 + a.M, a.S));  // keys that exist once the block is appended
 
   // Q fragments (A operand): row m_base+lr, d = step*32 + lg*8
-  bf16x8_t qf[4];
+  frag_t qf[4];
   {
     const int m = min(m_base + lr, a.M - 1);
     const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)m * a.sq_m + (int64_t)h * a.sq_h + lg * 8;
 #pragma unroll
-    for (int st = 0; st < 4; ++st) qf[st] = pf_ld(qp + st * 32);
+    for (int st = 0; st < 4; ++st) qf[st] = pf_ld<frag_t>(qp + st * 32);
   }
   float m_run[4], l_run[4];
   f32x4_t o[8];
@@ -166,7 +172,7 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
       const int key = min(n0 + j * 16 + lr, n_keys_all - 1);
       const uint16_t* kp = kb + (int64_t)key * a.sk_s + lg * 8;
 #pragma unroll
-      for (int st = 0; st < 4; ++st) s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[st], pf_ld(kp + st * 32), s[j], 0, 0, 0);
+      for (int st = 0; st < 4; ++st) s[j] = E::mfma(qf[st], pf_ld<frag_t>(kp + st * 32), s[j]);
     }
     // ---- masks + online softmax on the accumulator layout (rows lg*4+i, key column j*16+lr)
     float p[4][4];
@@ -209,21 +215,21 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t hi = f32_to_bf16_bits(p[j][i]);
+        const uint32_t hi = E::bits(p[j][i]);
         Ps[wave][lg * 4 + i][j * 16 + lr] = (uint16_t)hi;
-        Pl[wave][lg * 4 + i][j * 16 + lr] = (uint16_t)f32_to_bf16_bits(p[j][i] - bf16_bits_to_f32(hi));
+        Pl[wave][lg * 4 + i][j * 16 + lr] = (uint16_t)E::bits(p[j][i] - E::val(hi));
       }
     __syncthreads();   // Vt and Ps visible
     // ---- O += P V : A = Ps[row lr][keys st*32 + lg*8 ..], B = Vt[d = t*16+lr][keys st*32 + lg*8 ..]
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
-      const bf16x8_t pa = pf_ld(&Ps[wave][lr][st * 32 + lg * 8]);
-      const bf16x8_t pb = pf_ld(&Pl[wave][lr][st * 32 + lg * 8]);
+      const frag_t pa = pf_ld<frag_t>(&Ps[wave][lr][st * 32 + lg * 8]);
+      const frag_t pb = pf_ld<frag_t>(&Pl[wave][lr][st * 32 + lg * 8]);
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
-        const bf16x8_t vf = pf_ld(&Vt[t * 16 + lr][st * 32 + lg * 8]);
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vf, o[t], 0, 0, 0);
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pb, vf, o[t], 0, 0, 0);
+        const frag_t vf = pf_ld<frag_t>(&Vt[t * 16 + lr][st * 32 + lg * 8]);
+        o[t] = E::mfma(pa, vf, o[t]);
+        o[t] = E::mfma(pb, vf, o[t]);
       }
     }
   }
@@ -236,7 +242,7 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
     const float inv = l_run[i] > 0.f ? 1.0f / l_run[i] : 0.f;
     uint16_t* op = a.out + (int64_t)b * a.so_b + (int64_t)m * a.so_m + (int64_t)h * a.so_h;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) op[t * 16 + lr] = (uint16_t)f32_to_bf16_bits(o[t][i] * inv);
+    for (int t = 0; t < 8; ++t) op[t * 16 + lr] = (uint16_t)E::bits(o[t][i] * inv);
   }
 }
 
@@ -260,8 +266,10 @@ __global__ __launch_bounds__(kPfThreads) void attn_prefill_kernel(PrefillAttnArg
 // two groups' running statistics and outputs are merged through LDS at the end — for prompts whose (query tile, head)
 // pairs number no more than the compute units, where a workgroup alone on its compute unit walks its key tiles with
 // one wave per SIMD and waits out every load and barrier.
-template <int MI, int NG>
+template <int DT, int MI, int NG>
 __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill_wide_kernel(PrefillAttnArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   constexpr int DH = 128, BN = 64, QW = 16 * MI, BM = 4 * QW, VSTR = BN;
   // K rows of 288 bytes: a 16-byte LDS read is served 16 lanes a cycle (lanes 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of a
   // half wave); rows 16 r apart with r odd multiples of 32 bytes give those lanes 16 different bank groups
@@ -285,13 +293,13 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
   const int m_base = mt * BM + wave * QW;
   const int n_keys_all = max(1, min(q0 + a.M, a.S));
 
-  bf16x8_t qf[MI][4];
+  frag_t qf[MI][4];
 #pragma unroll
   for (int mi = 0; mi < MI; ++mi) {
     const int m = min(m_base + mi * 16 + lr, a.M - 1);
     const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)m * a.sq_m + (int64_t)h * a.sq_h + lg * 8;
 #pragma unroll
-    for (int st = 0; st < 4; ++st) qf[mi][st] = pf_ld(qp + st * 32);
+    for (int st = 0; st < 4; ++st) qf[mi][st] = pf_ld<frag_t>(qp + st * 32);
   }
   float m_run[MI], l_run[MI];          // statistics of query m_base + 16 mi + lr (the same in the four lanes lg of a column)
   f32x4_t o[MI][8];                    // O^T: tile t, element i = dimension 16 t + 4 lg + i of that query
@@ -358,20 +366,20 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
     f32x4_t sacc[MI][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      bf16x8_t kf[4];
+      frag_t kf[4];
 #pragma unroll
-      for (int st = 0; st < 4; ++st) kf[st] = pf_ld(&Ks[j * 16 + lr][st * 32 + lg * 8]);
+      for (int st = 0; st < 4; ++st) kf[st] = pf_ld<frag_t>(&Ks[j * 16 + lr][st * 32 + lg * 8]);
 #pragma unroll
       for (int mi = 0; mi < MI; ++mi) {
         sacc[mi][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int st = 0; st < 4; ++st) sacc[mi][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[st], qf[mi][st], sacc[mi][j], 0, 0, 0);
+        for (int st = 0; st < 4; ++st) sacc[mi][j] = E::mfma(kf[st], qf[mi][st], sacc[mi][j]);
       }
     }
     // ---- masks + online softmax, one query per lane and block; tiles that need no mask take the short way
     const bool plain = !a.pad_mask && !a.add_mask && !rows_ragged && n0 + BN <= n_keys_all &&
                        (!a.causal || n0 + BN - 1 <= q0 + m_base);
-    bf16x8_t ph[MI][2], pl[MI][2];     // P^T fragments (high part, residual) of the two 32-key steps
+    frag_t ph[MI][2], pl[MI][2];     // P^T fragments (high part, residual) of the two 32-key steps
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi) {
       const int m = m_base + mi * 16 + lr;
@@ -419,12 +427,12 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
 #pragma unroll
         for (int c = 0; c < 4; ++c) {                  // k-slots 2c, 2c + 1: block 2 st + c / 2, elements 2 (c % 2), + 1
           const float x0 = e[2 * st + (c >> 1)][2 * (c & 1)], x1 = e[2 * st + (c >> 1)][2 * (c & 1) + 1];
-          const uint32_t h0 = f32_to_bf16_bits(x0), h1 = f32_to_bf16_bits(x1);
+          const uint32_t h0 = E::bits(x0), h1 = E::bits(x1);
           hw[c] = h0 | (h1 << 16);
-          lw[c] = f32_to_bf16_bits(x0 - bf16_bits_to_f32(h0)) | (f32_to_bf16_bits(x1 - bf16_bits_to_f32(h1)) << 16);
+          lw[c] = E::bits(x0 - E::val(h0)) | (E::bits(x1 - E::val(h1)) << 16);
         }
-        ph[mi][st] = __builtin_bit_cast(bf16x8_t, u32x4_t{hw[0], hw[1], hw[2], hw[3]});
-        pl[mi][st] = __builtin_bit_cast(bf16x8_t, u32x4_t{lw[0], lw[1], lw[2], lw[3]});
+        ph[mi][st] = __builtin_bit_cast(frag_t, u32x4_t{hw[0], hw[1], hw[2], hw[3]});
+        pl[mi][st] = __builtin_bit_cast(frag_t, u32x4_t{lw[0], lw[1], lw[2], lw[3]});
       }
     }
     // ---- O^T += V^T P^T : A = Vt rows (dimension 16 t + lr; keys in the permuted order), B = P^T fragments
@@ -432,11 +440,11 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
     for (int st = 0; st < 2; ++st) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
-        const bf16x8_t vf = pf_ld(&Vt[t * 16 + lr][(st * 32 + lg * 8) ^ (8 * ((lr >> 1) ^ ((2 * t + (lr >> 3)) & 7)))]);
+        const frag_t vf = pf_ld<frag_t>(&Vt[t * 16 + lr][(st * 32 + lg * 8) ^ (8 * ((lr >> 1) ^ ((2 * t + (lr >> 3)) & 7)))]);
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
-          o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph[mi][st], o[mi][t], 0, 0, 0);
-          o[mi][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[mi][st], o[mi][t], 0, 0, 0);
+          o[mi][t] = E::mfma(vf, ph[mi][st], o[mi][t]);
+          o[mi][t] = E::mfma(vf, pl[mi][st], o[mi][t]);
         }
       }
     }
@@ -477,8 +485,8 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       u32x2_t w;
-      w.x = f32_to_bf16_bits(o[mi][t][0] * inv) | (f32_to_bf16_bits(o[mi][t][1] * inv) << 16);
-      w.y = f32_to_bf16_bits(o[mi][t][2] * inv) | (f32_to_bf16_bits(o[mi][t][3] * inv) << 16);
+      w.x = E::bits(o[mi][t][0] * inv) | (E::bits(o[mi][t][1] * inv) << 16);
+      w.y = E::bits(o[mi][t][2] * inv) | (E::bits(o[mi][t][3] * inv) << 16);
       *reinterpret_cast<u32x2_t*>(op + t * 16) = w;
     }
   }
@@ -486,6 +494,7 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
 
 int launch_expand(const ExpandArgs& a, hipStream_t st) {
   const char* fn = "fsvd_lowrank_expand_heads";
+  if (a.dt != 0 && a.dt != 1) { set_last_error("%s: dtype code %d (bf16 = 0 and fp16 = 1 are served)", fn, a.dt); return kErrBadDtype; }
   if (a.B <= 0 || a.M <= 0 || a.heads <= 0 || a.R <= 0) { set_last_error("%s: empty shape", fn); return kErrBadShape; }
   if (a.Dh != 128) { set_last_error("%s: head_dim %d is not 128", fn, a.Dh); return kErrBadShape; }
   if (a.R % 8) { set_last_error("%s: rank %d is not a multiple of 8; pad the factors", fn, a.R); return kErrBadShape; }
@@ -496,21 +505,16 @@ int launch_expand(const ExpandArgs& a, hipStream_t st) {
   }
   if (expand_tiles_apply(a)) return launch_expand_tiles(a, st);   // long prompts: the LDS-tiled kernel
   const int T = a.B * a.M;
-  hipLaunchKernelGGL(lowrank_expand_kernel, dim3((T + 127) / 128, a.heads), dim3(kPfThreads), 0, st, a);
+  if (a.dt == 1) hipLaunchKernelGGL(lowrank_expand_kernel<1>, dim3((T + 127) / 128, a.heads), dim3(kPfThreads), 0, st, a);
+  else hipLaunchKernelGGL(lowrank_expand_kernel<0>, dim3((T + 127) / 128, a.heads), dim3(kPfThreads), 0, st, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
 }
 
-int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
+template <int DT>
+static int launch_prefill_attn_t(const PrefillAttnArgs& a, hipStream_t st) {
   const char* fn = "fsvd_attn_prefill";
-  if (a.B <= 0 || a.M <= 0 || a.H <= 0 || a.Hk <= 0 || a.H % a.Hk) { set_last_error("%s: bad shape", fn); return kErrBadShape; }
-  if (a.Dh != 128) { set_last_error("%s: head_dim %d is not 128", fn, a.Dh); return kErrBadShape; }
-  const auto mis = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
-  if (mis(a.q) || mis(a.k) || mis(a.v) || (a.sq_b % 8) || (a.sq_m % 8) || (a.sq_h % 8) || (a.sk_b % 8) || (a.sk_s % 8) || (a.sk_h % 8)) {
-    set_last_error("%s: q / k / v pointers and strides must be 16-byte aligned", fn);
-    return kErrBadAlign;
-  }
   // the LDS-shared kernel stores four dimensions of a row with one 8-byte write
   const bool out8 = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.so_b % 4) == 0 && (a.so_m % 4) == 0 && (a.so_h % 4) == 0;
   if (a.M >= 128 && out8) {   // long prompts: 64 or 128 queries per workgroup, K / V tiles shared through LDS
@@ -522,19 +526,32 @@ int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
     if (pair) {
       static bool granted = false;
       if (!granted) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * lds));
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_wide_kernel<DT, 1, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * lds));
         if (e != hipSuccess) { set_last_error("%s: cannot reserve %zu bytes of LDS: %s", fn, 2 * lds, hipGetErrorString(e)); return kErrLaunch; }
         granted = true;
       }
-      hipLaunchKernelGGL((attn_prefill_wide_kernel<1, 2>), dim3((a.M + 63) / 64, a.H, a.B), dim3(2 * kPfThreads), 2 * lds, st, a);
-    } else if (wide) hipLaunchKernelGGL((attn_prefill_wide_kernel<2, 1>), dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
-    else hipLaunchKernelGGL((attn_prefill_wide_kernel<1, 1>), dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), lds, st, a);
+      hipLaunchKernelGGL((attn_prefill_wide_kernel<DT, 1, 2>), dim3((a.M + 63) / 64, a.H, a.B), dim3(2 * kPfThreads), 2 * lds, st, a);
+    } else if (wide) hipLaunchKernelGGL((attn_prefill_wide_kernel<DT, 2, 1>), dim3((a.M + 127) / 128, a.H, a.B), dim3(kPfThreads), lds, st, a);
+    else hipLaunchKernelGGL((attn_prefill_wide_kernel<DT, 1, 1>), dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), lds, st, a);
   } else {
-    hipLaunchKernelGGL(attn_prefill_kernel, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), 0, st, a);
+    hipLaunchKernelGGL(attn_prefill_kernel<DT>, dim3((a.M + 63) / 64, a.H, a.B), dim3(kPfThreads), 0, st, a);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
+}
+
+int launch_prefill_attn(const PrefillAttnArgs& a, hipStream_t st) {
+  const char* fn = "fsvd_attn_prefill";
+  if (a.dt != 0 && a.dt != 1) { set_last_error("%s: dtype code %d (bf16 = 0 and fp16 = 1 are served)", fn, a.dt); return kErrBadDtype; }
+  if (a.B <= 0 || a.M <= 0 || a.H <= 0 || a.Hk <= 0 || a.H % a.Hk) { set_last_error("%s: bad shape", fn); return kErrBadShape; }
+  if (a.Dh != 128) { set_last_error("%s: head_dim %d is not 128", fn, a.Dh); return kErrBadShape; }
+  const auto mis = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+  if (mis(a.q) || mis(a.k) || mis(a.v) || (a.sq_b % 8) || (a.sq_m % 8) || (a.sq_h % 8) || (a.sk_b % 8) || (a.sk_s % 8) || (a.sk_h % 8)) {
+    set_last_error("%s: q / k / v pointers and strides must be 16-byte aligned", fn);
+    return kErrBadAlign;
+  }
+  return a.dt == 1 ? launch_prefill_attn_t<1>(a, st) : launch_prefill_attn_t<0>(a, st);
 }
 
 }  // namespace fsvd

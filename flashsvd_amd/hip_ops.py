@@ -30,6 +30,20 @@ def _need(t: torch.Tensor, name: str, *, dtype=_BF16) -> None:
         raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
 
 
+_ELEM_CODES = {torch.bfloat16: 0, torch.float16: 1}     # FSVD_BF16, FSVD_FP16
+
+
+def _elem(t: torch.Tensor, name: str):
+    """Element type of a call on the fused product path, named by its first operand: (torch dtype, C-ABI code).  Every
+    other 16-bit tensor of the call must be of the same type."""
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor, got device {t.device}")
+    code = _ELEM_CODES.get(t.dtype)
+    if code is None:
+        raise ValueError(f"{name} must be torch.bfloat16 or torch.float16, got {t.dtype}")
+    return t.dtype, code
+
+
 def _rows(t: torch.Tensor, name: str) -> torch.Tensor:
     """View as [rows, last] with unit stride on the last axis (copies only if it must)."""
     if t.stride(-1) != 1:
@@ -101,7 +115,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
 
 
 def _linear_impl(x, weight, bias, norm_weight, eps, residual, out, cfg):
-    _need(x, "x"); _need(weight, "weight")
+    dt, code = _elem(x, "x")
+    _need(weight, "weight", dtype=dt)
     if weight.dim() != 2 or weight.stride(1) != 1:
         raise ValueError(f"weight must be [N, K] with unit inner stride, got {tuple(weight.shape)} strides {weight.stride()}")
     N, K = weight.shape
@@ -110,19 +125,20 @@ def _linear_impl(x, weight, bias, norm_weight, eps, residual, out, cfg):
     x2 = _rows(x, "x")
     B = x2.shape[0]
     if out is None:
-        out = torch.empty(*x.shape[:-1], N, device=x.device, dtype=_BF16)
+        out = torch.empty(*x.shape[:-1], N, device=x.device, dtype=dt)
+    _need(out, "out", dtype=dt)
     o2 = _rows(out, "out")
     if o2.shape != (B, N) or o2.data_ptr() != out.data_ptr():
         raise ValueError("out must be a dense [..., N] tensor matching x")
     r2 = None
     if residual is not None:
-        _need(residual, "residual")
+        _need(residual, "residual", dtype=dt)
         r2 = _rows(residual, "residual")
         if r2.shape != (B, N):
             raise ValueError(f"residual shape {tuple(residual.shape)} does not match output [{B}, {N}]")
     for t, nm, n in ((bias, "bias", N), (norm_weight, "norm_weight", K)):
         if t is not None:
-            _need(t, nm)
+            _need(t, nm, dtype=dt)
             if t.shape != (n,) or not t.is_contiguous():
                 raise ValueError(f"{nm} must be a contiguous [{n}] tensor")
     lib = _lib.load()
@@ -135,7 +151,7 @@ def _linear_impl(x, weight, bias, norm_weight, eps, residual, out, cfg):
         norm_weight = None
     rc = lib.fsvd_linear(x2.data_ptr(), x2.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias), _ptr(norm_weight),
                          float(eps), _ptr(r2), 0 if r2 is None else r2.stride(0), o2.data_ptr(), o2.stride(0),
-                         B, N, K, int(cfg), _stream())
+                         B, N, K, int(cfg), code, _stream())
     _lib.check("fsvd_linear", rc)
     return out
 
@@ -150,7 +166,8 @@ def swiglu_linear(p: torch.Tensor, gate_u: torch.Tensor, up_u: torch.Tensor, *, 
 
 
 def _swiglu_linear_impl(p, gate_u, up_u, up_off, mode, out, cfg):
-    _need(p, "p"); _need(gate_u, "gate_u"); _need(up_u, "up_u")
+    dt, code = _elem(p, "p")
+    _need(gate_u, "gate_u", dtype=dt); _need(up_u, "up_u", dtype=dt)
     if gate_u.dim() != 2 or gate_u.shape != up_u.shape or gate_u.stride() != up_u.stride() or gate_u.stride(1) != 1:
         raise ValueError(f"gate_u/up_u must be matching [D, R] weights, got {tuple(gate_u.shape)} / {tuple(up_u.shape)}")
     D, R = gate_u.shape
@@ -159,13 +176,14 @@ def _swiglu_linear_impl(p, gate_u, up_u, up_off, mode, out, cfg):
         raise ValueError(f"p last dim {p2.shape[1]} too small for up_off {up_off} + R {R}")
     B = p2.shape[0]
     if out is None:
-        out = torch.empty(*p.shape[:-1], D, device=p.device, dtype=_BF16)
+        out = torch.empty(*p.shape[:-1], D, device=p.device, dtype=dt)
+    _need(out, "out", dtype=dt)
     o2 = _rows(out, "out")
     lib = _lib.load()
     if 3 <= B < 128:
         ensure_split_workspace(p.device)
     rc = lib.fsvd_swiglu_linear(p2.data_ptr(), p2.stride(0), int(up_off), gate_u.data_ptr(), up_u.data_ptr(),
-                                gate_u.stride(0), o2.data_ptr(), o2.stride(0), B, D, R, int(mode), int(cfg), _stream())
+                                gate_u.stride(0), o2.data_ptr(), o2.stride(0), B, D, R, int(mode), int(cfg), code, _stream())
     _lib.check("fsvd_swiglu_linear", rc)
     return out
 
@@ -272,8 +290,9 @@ def qkv_rope_append(p: torch.Tensor, q_u: torch.Tensor, k_u: torch.Tensor, v_u: 
 
 
 def _qkv_rope_append_impl(p, q_u, k_u, v_u, cos, sin, positions, k_cache, v_cache, num_heads, num_kv_heads, head_dim, q_out, cfg):
-    for t, nm in ((p, "p"), (q_u, "q_u"), (k_u, "k_u"), (v_u, "v_u"), (k_cache, "k_cache"), (v_cache, "v_cache")):
-        _need(t, nm)
+    dt, code = _elem(p, "p")
+    for t, nm in ((q_u, "q_u"), (k_u, "k_u"), (v_u, "v_u"), (k_cache, "k_cache"), (v_cache, "v_cache")):
+        _need(t, nm, dtype=dt)
     _need(positions, "positions", dtype=torch.int32)
     H, Hk, Dh = int(num_heads), int(num_kv_heads), int(head_dim)
     Rq, Rk, Rv = q_u.shape[1], k_u.shape[1], v_u.shape[1]
@@ -291,20 +310,20 @@ def _qkv_rope_append_impl(p, q_u, k_u, v_u, cos, sin, positions, k_cache, v_cach
         raise ValueError(f"positions must be a contiguous int32 [{B}] tensor")
     rope_len = 0
     if cos is not None:
-        _need(cos, "cos"); _need(sin, "sin")
+        _need(cos, "cos", dtype=dt); _need(sin, "sin", dtype=dt)
         if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2 or not cos.is_contiguous() or not sin.is_contiguous():
             raise ValueError(f"cos/sin must be contiguous [len, {Dh // 2}] tables")
         rope_len = cos.shape[0]
     if q_out is None:
-        q_out = torch.empty(B, H, Dh, device=p.device, dtype=_BF16)
-    elif q_out.shape != (B, H, Dh) or not q_out.is_contiguous():
+        q_out = torch.empty(B, H, Dh, device=p.device, dtype=dt)
+    elif q_out.shape != (B, H, Dh) or not q_out.is_contiguous() or q_out.dtype != dt:
         raise ValueError("q_out must be contiguous [B,H,Dh]")
     lib = _lib.load()
     rc = lib.fsvd_qkv_rope_append(p2.data_ptr(), p2.stride(0), q_u.data_ptr(), q_u.stride(0), k_u.data_ptr(), k_u.stride(0),
                                   v_u.data_ptr(), v_u.stride(0), _ptr(cos), _ptr(sin), rope_len, positions.data_ptr(),
                                   q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                   k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
-                                  B, H, Hk, Dh, Rq, Rk, Rv, k_cache.shape[1], int(cfg), _stream())
+                                  B, H, Hk, Dh, Rq, Rk, Rv, k_cache.shape[1], int(cfg), code, _stream())
     _lib.check("fsvd_qkv_rope_append", rc)
     return q_out
 
@@ -340,7 +359,8 @@ def attn_decode_densekv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
 
 def _attn_decode_densekv_impl(q, k_cache, v_cache, cache_seqlens, k_new, v_new, cos, sin, seqlen_add, nsplit, workspace, out,
                               softmax_scale, static_scratch):
-    _need(q, "q"); _need(k_cache, "k_cache"); _need(v_cache, "v_cache")
+    dt, code = _elem(q, "q")
+    _need(k_cache, "k_cache", dtype=dt); _need(v_cache, "v_cache", dtype=dt)
     _need(cache_seqlens, "cache_seqlens", dtype=torch.int32)
     if q.dim() != 3 or q.stride(2) != 1:
         raise ValueError(f"q must be [B,H,Dh] with unit inner stride, got {tuple(q.shape)}")
@@ -355,21 +375,21 @@ def _attn_decode_densekv_impl(q, k_cache, v_cache, cache_seqlens, k_new, v_new, 
         raise ValueError(f"cache_seqlens must be a contiguous int32 [{B}] tensor")
     sk_b = sk_h = sv_b = sv_h = 0
     if k_new is not None:
-        _need(k_new, "k_new"); _need(v_new, "v_new")
+        _need(k_new, "k_new", dtype=dt); _need(v_new, "v_new", dtype=dt)
         if k_new.shape != (B, Hk, Dh) or v_new.shape != (B, Hk, Dh) or k_new.stride(2) != 1 or v_new.stride(2) != 1:
             raise ValueError(f"k_new/v_new must be [B,Hk,Dh] tensors with unit inner stride, got {tuple(k_new.shape)} / {tuple(v_new.shape)}")
         sk_b, sk_h, sv_b, sv_h = k_new.stride(0), k_new.stride(1), v_new.stride(0), v_new.stride(1)
     rope_len = 0
     if cos is not None:
-        _need(cos, "cos"); _need(sin, "sin")
+        _need(cos, "cos", dtype=dt); _need(sin, "sin", dtype=dt)
         if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2 or not cos.is_contiguous() or not sin.is_contiguous():
             raise ValueError(f"cos/sin must be contiguous [len, {Dh // 2}] tables")
         rope_len = cos.shape[0]
     if nsplit is None:
         nsplit = pick_nsplit(S, B, H, Dh)
     if out is None:
-        out = torch.empty(B, H, Dh, device=q.device, dtype=_BF16)
-    elif out.shape != (B, H, Dh) or out.stride(2) != 1:
+        out = torch.empty(B, H, Dh, device=q.device, dtype=dt)
+    elif out.shape != (B, H, Dh) or out.stride(2) != 1 or out.dtype != dt:
         raise ValueError("out must be [B,H,Dh] with unit inner stride")
     lib = _lib.load()
     if static_scratch:
@@ -380,7 +400,7 @@ def _attn_decode_densekv_impl(q, k_cache, v_cache, cache_seqlens, k_new, v_new, 
                                                  _ptr(k_new), sk_b, sk_h, _ptr(v_new), sv_b, sv_h, cache_seqlens.data_ptr(),
                                                  int(seqlen_add), _ptr(cos), _ptr(sin), rope_len, out.data_ptr(), out.stride(0),
                                                  out.stride(1), B, H, Hk, Dh, S, int(nsplit),
-                                                 float(softmax_scale) if softmax_scale else 0.0, _stream())
+                                                 float(softmax_scale) if softmax_scale else 0.0, code, _stream())
         _lib.check("fsvd_attn_decode_densekv_static", rc)
         return out
     ws_ptr, ws_bytes = None, 0
@@ -393,7 +413,7 @@ def _attn_decode_densekv_impl(q, k_cache, v_cache, cache_seqlens, k_new, v_new, 
                                       _ptr(k_new), sk_b, sk_h, _ptr(v_new), sv_b, sv_h, cache_seqlens.data_ptr(), int(seqlen_add),
                                       _ptr(cos), _ptr(sin), rope_len, out.data_ptr(), out.stride(0), out.stride(1),
                                       ws_ptr, ws_bytes, B, H, Hk, Dh, S, int(nsplit),
-                                      float(softmax_scale) if softmax_scale else 0.0, _stream())
+                                      float(softmax_scale) if softmax_scale else 0.0, code, _stream())
     _lib.check("fsvd_attn_decode_densekv", rc)
     return out
 
@@ -404,24 +424,27 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, out: Optio
 
 
 def _rmsnorm_impl(x, weight, eps, out):
-    _need(x, "x"); _need(weight, "weight")
+    dt, code = _elem(x, "x")
+    _need(weight, "weight", dtype=dt)
     K = x.shape[-1]
     if weight.shape != (K,) or not weight.is_contiguous():
         raise ValueError(f"weight must be contiguous [{K}]")
     x2 = _rows(x, "x")
     if out is None:
         out = torch.empty_like(x, memory_format=torch.contiguous_format)
+    _need(out, "out", dtype=dt)
     o2 = _rows(out, "out")
     lib = _lib.load()
     rc = lib.fsvd_rmsnorm(x2.data_ptr(), x2.stride(0), weight.data_ptr(), float(eps), o2.data_ptr(), o2.stride(0),
-                          x2.shape[0], K, _stream())
+                          x2.shape[0], K, code, _stream())
     _lib.check("fsvd_rmsnorm", rc)
     return out
 
 
 def _expand_operands(p, u, heads, Dh, out, bias, head_stride):
-    """Checks of one head expansion; returns (B, M, R, coefficient strides)."""
-    _need(p, "p"); _need(u, "u"); _need(out, "out")
+    """Checks of one head expansion; returns (B, M, R, coefficient strides, element code)."""
+    dt, code = _elem(p, "p")
+    _need(u, "u", dtype=dt); _need(out, "out", dtype=dt)
     if p.dim() == 3:
         B, M, R = p.shape
         sp = (p.stride(0), p.stride(1), 0 if head_stride is None else int(head_stride))
@@ -439,16 +462,16 @@ def _expand_operands(p, u, heads, Dh, out, bias, head_stride):
     if out.dim() != 4 or out.shape[0] < B or out.shape[2] != heads or out.shape[3] != Dh:
         raise ValueError(f"out must be [B>={B}, rows, {heads}, {Dh}], got {tuple(out.shape)}")
     if bias is not None:
-        _need(bias, "bias")
+        _need(bias, "bias", dtype=dt)
         if bias.numel() != heads * Dh or not bias.is_contiguous():
             raise ValueError(f"bias must be contiguous [{heads * Dh}]")
-    return B, M, R, sp
+    return B, M, R, sp, code
 
 
-def _rope_tables(cos, sin, Dh):
+def _rope_tables(cos, sin, Dh, dt):
     if cos is None:
         return 0
-    _need(cos, "cos"); _need(sin, "sin")
+    _need(cos, "cos", dtype=dt); _need(sin, "sin", dtype=dt)
     if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2 or not cos.is_contiguous() or not sin.is_contiguous():
         raise ValueError(f"cos/sin must be contiguous [len, {Dh // 2}] tables")
     return cos.shape[0]
@@ -468,8 +491,8 @@ def lowrank_expand_heads(p: torch.Tensor, u: torch.Tensor, *, num_heads: int, he
 
 def _lowrank_expand_heads_impl(p, u, num_heads, head_dim, out, cos, sin, positions, bias, dst_by_position, head_stride):
     heads, Dh = int(num_heads), int(head_dim)
-    B, M, R, sp = _expand_operands(p, u, heads, Dh, out, bias, head_stride)
-    rope_len = _rope_tables(cos, sin, Dh)
+    B, M, R, sp, code = _expand_operands(p, u, heads, Dh, out, bias, head_stride)
+    rope_len = _rope_tables(cos, sin, Dh, p.dtype)
     if positions is not None:
         _need(positions, "positions", dtype=torch.int32)
         if positions.numel() != B:
@@ -477,7 +500,7 @@ def _lowrank_expand_heads_impl(p, u, num_heads, head_dim, out, cos, sin, positio
     lib = _lib.load()
     rc = lib.fsvd_lowrank_expand_heads(p.data_ptr(), sp[0], sp[1], sp[2], u.data_ptr(), u.stride(0), _ptr(bias), _ptr(cos), _ptr(sin),
                                        rope_len, _ptr(positions), out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
-                                       int(bool(dst_by_position)), out.shape[1], B, M, heads, Dh, R, _stream())
+                                       int(bool(dst_by_position)), out.shape[1], B, M, heads, Dh, R, code, _stream())
     _lib.check("fsvd_lowrank_expand_heads", rc)
     return out
 
@@ -507,16 +530,18 @@ def lowrank_expand_heads_multi(items, *, head_dim: int, cos: Optional[torch.Tens
     Dh = int(head_dim)
     if not 1 <= len(items) <= 3:
         raise ValueError(f"{len(items)} expansions (1..3)")
-    rope_len = _rope_tables(cos, sin, Dh)
+    rope_len = _rope_tables(cos, sin, Dh, items[0]["p"].dtype)
     descs = (_lib.ExpandDesc * len(items))()
-    shape = None
+    shape = code = None
     for d, it in zip(descs, items):
         heads, out, bias = int(it["num_heads"]), it["out"], it.get("bias")
-        B, M, R, sp = _expand_operands(it["p"], it["u"], heads, Dh, out, bias, it.get("head_stride"))
+        B, M, R, sp, c = _expand_operands(it["p"], it["u"], heads, Dh, out, bias, it.get("head_stride"))
         if shape is None:
-            shape = (B, M)
+            shape, code = (B, M), c
         elif shape != (B, M):
             raise ValueError(f"expansions of one call cover the same token rows: {shape} vs {(B, M)}")
+        elif c != code:
+            raise ValueError("expansions of one call are of one element type")
         if it.get("rotate") and cos is None:
             raise ValueError("rotate asked for without cos / sin")
         d.p, d.sp_b, d.sp_m, d.sp_h = it["p"].data_ptr(), sp[0], sp[1], sp[2]
@@ -530,7 +555,7 @@ def lowrank_expand_heads_multi(items, *, head_dim: int, cos: Optional[torch.Tens
         if positions.numel() != B:
             raise ValueError(f"positions must be int32 [{B}]")
     lib = _lib.load()
-    rc = lib.fsvd_lowrank_expand_heads_multi(descs, len(items), _ptr(cos), _ptr(sin), rope_len, _ptr(positions), B, M, Dh, _stream())
+    rc = lib.fsvd_lowrank_expand_heads_multi(descs, len(items), _ptr(cos), _ptr(sin), rope_len, _ptr(positions), B, M, Dh, code, _stream())
     _lib.check("fsvd_lowrank_expand_heads_multi", rc)
 
 
@@ -544,7 +569,8 @@ def attn_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, q_pos0: O
 
 
 def _attn_prefill_impl(q, k, v, q_pos0, causal, pad_mask, add_mask, out, softmax_scale):
-    _need(q, "q"); _need(k, "k"); _need(v, "v")
+    dt, code = _elem(q, "q")
+    _need(k, "k", dtype=dt); _need(v, "v", dtype=dt)
     if q.dim() != 4 or k.dim() != 4 or k.shape != v.shape or k.stride() != v.stride():
         raise ValueError(f"q must be [B,M,H,Dh] and k/v matching [B,S,Hk,Dh], got {tuple(q.shape)} {tuple(k.shape)} {tuple(v.shape)}")
     B, M, H, Dh = q.shape
@@ -554,7 +580,8 @@ def _attn_prefill_impl(q, k, v, q_pos0, causal, pad_mask, add_mask, out, softmax
     if q.stride(3) != 1 or k.stride(3) != 1:
         raise ValueError("q, k, v need unit stride on the last axis")
     if out is None:
-        out = torch.empty(B, M, H, Dh, device=q.device, dtype=_BF16)
+        out = torch.empty(B, M, H, Dh, device=q.device, dtype=dt)
+    _need(out, "out", dtype=dt)
     spm = sam_b = sam_q = 0
     if pad_mask is not None:
         if pad_mask.dtype != torch.uint8 or pad_mask.dim() != 2 or pad_mask.shape[0] != B or pad_mask.stride(1) != 1:
@@ -570,6 +597,6 @@ def _attn_prefill_impl(q, k, v, q_pos0, causal, pad_mask, add_mask, out, softmax
     rc = lib.fsvd_attn_prefill(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), k.data_ptr(), v.data_ptr(), k.stride(0),
                                k.stride(1), k.stride(2), _ptr(q_pos0), _ptr(pad_mask), spm, _ptr(add_mask), sam_b, sam_q,
                                out.data_ptr(), out.stride(0), out.stride(1), out.stride(2), B, M, H, Hk, Dh, S, int(bool(causal)),
-                               float(softmax_scale) if softmax_scale else 0.0, _stream())
+                               float(softmax_scale) if softmax_scale else 0.0, code, _stream())
     _lib.check("fsvd_attn_prefill", rc)
     return out

@@ -96,8 +96,8 @@ class FlashSVDRoPEAttention(nn.Module):
             raise ValueError(f"Expected Pk/Pv [B,Hk,M,R], got {tuple(f.Pk.shape)}/{tuple(f.Pv.shape)}")
         Bk, Hk, Mk, Rk = f.Pk.shape
         assert Bk == B and Mk == M and Rk == R, "Pk shape mismatch vs Pq"
-        if f.Pq.dtype != torch.bfloat16:
-            raise NotImplementedError(f"the MI355X prefill kernels compute in bfloat16; got {f.Pq.dtype}")
+        if f.Pq.dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"the MI355X prefill kernels compute in bfloat16 or float16; got {f.Pq.dtype}")
         if (f.bk is not None or f.bv is not None) and Hk != H:
             raise NotImplementedError("key/value biases indexed by query head need H == Hk")
         dev, dt = f.Pq.device, f.Pq.dtype

@@ -42,8 +42,8 @@ def _require_gpu(t: torch.Tensor, who: str) -> None:
     if not t.is_cuda:
         raise RuntimeError(f"{who} runs only on a GPU through libflashsvd_hip (got a {t.device} tensor); "
                            "there is no CPU path in this package")
-    if t.dtype != torch.bfloat16:
-        raise RuntimeError(f"{who} computes in bfloat16, got {t.dtype}")
+    if t.dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError(f"{who} computes in bfloat16 or float16, got {t.dtype}")
 
 
 class LlamaRMSNorm(nn.Module):
@@ -761,7 +761,7 @@ def patch_hf_llama_decoder_layer() -> bool:
 
     def forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
                 position_embeddings=None, **kwargs):
-        if not isinstance(self.mlp, SVD_LlamaMLP) or not hidden_states.is_cuda or hidden_states.dtype != torch.bfloat16:
+        if not isinstance(self.mlp, SVD_LlamaMLP) or not hidden_states.is_cuda or hidden_states.dtype not in (torch.bfloat16, torch.float16):
             return orig(self, hidden_states, attention_mask=attention_mask, position_ids=position_ids,
                         past_key_values=past_key_values, use_cache=use_cache, position_embeddings=position_embeddings, **kwargs)
         if _env_truthy("FLASH_SVD_MLP_CUDA_GRAPH") and os.getenv("FLASH_SVD_MLP_CUDA_GRAPH_SCOPE", "auto").strip().lower() == "mlp":

@@ -51,7 +51,7 @@ def _linear_out(x, weight, bias=None, norm_weight=None, eps=1e-6, residual=None,
 
 
 def _linear_fake(x, weight, bias=None, norm_weight=None, eps=1e-6, residual=None, cfg=0):
-    return x.new_empty((*x.shape[:-1], weight.shape[0]), dtype=_BF16)
+    return x.new_empty((*x.shape[:-1], weight.shape[0]))
 
 
 _define("linear(Tensor x, Tensor weight, Tensor? bias=None, Tensor? norm_weight=None, float eps=1e-6, Tensor? residual=None, "
@@ -72,7 +72,7 @@ def _swiglu_out(p, gate_u, up_u, up_off, mode=0, cfg=0, *, out):
 
 
 _define("swiglu_linear(Tensor p, Tensor gate_u, Tensor up_u, int up_off, int mode=0, int cfg=0) -> Tensor", _swiglu,
-        lambda p, gate_u, up_u, up_off, mode=0, cfg=0: p.new_empty((*p.shape[:-1], gate_u.shape[0]), dtype=_BF16))
+        lambda p, gate_u, up_u, up_off, mode=0, cfg=0: p.new_empty((*p.shape[:-1], gate_u.shape[0])))
 _define("swiglu_linear.out(Tensor p, Tensor gate_u, Tensor up_u, int up_off, int mode=0, int cfg=0, *, Tensor(a!) out) -> Tensor(a!)",
         _swiglu_out, lambda *a, out, **k: out)
 
@@ -109,7 +109,7 @@ def _qkv_out(p, q_u, k_u, v_u, cos, sin, positions, k_cache, v_cache, num_heads,
 
 def _qkv_fake(p, q_u, k_u, v_u, cos, sin, positions, k_cache, v_cache, num_heads, num_kv_heads, head_dim, cfg=0):
     rows = p.numel() // p.shape[-1]
-    return p.new_empty((rows, num_heads, head_dim), dtype=_BF16)
+    return p.new_empty((rows, num_heads, head_dim))
 
 
 _QKV_ARGS = ("Tensor p, Tensor q_u, Tensor k_u, Tensor v_u, Tensor? cos, Tensor? sin, Tensor positions, Tensor(a!) k_cache, "
@@ -136,7 +136,7 @@ def _attn_dense_out(q, k_cache, v_cache, cache_seqlens, k_new=None, v_new=None, 
 _AD_ARGS = ("Tensor q, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor cache_seqlens, Tensor? k_new=None, Tensor? v_new=None, "
             "Tensor? cos=None, Tensor? sin=None, int seqlen_add=0, int? nsplit=None, Tensor(c!)? workspace=None, "
             "float? softmax_scale=None, bool static_scratch=False")
-_define(f"attn_decode_densekv({_AD_ARGS}) -> Tensor", _attn_dense, lambda q, *a, **k: q.new_empty(q.shape, dtype=_BF16))
+_define(f"attn_decode_densekv({_AD_ARGS}) -> Tensor", _attn_dense, lambda q, *a, **k: q.new_empty(q.shape))
 _define(f"attn_decode_densekv.out({_AD_ARGS}, *, Tensor(d!) out) -> Tensor(d!)", _attn_dense_out, lambda *a, out, **k: out)
 
 
@@ -194,7 +194,7 @@ def _prefill_out(q, k, v, q_pos0=None, causal=True, pad_mask=None, add_mask=None
 
 _PF_ARGS = ("Tensor q, Tensor k, Tensor v, Tensor? q_pos0=None, bool causal=True, Tensor? pad_mask=None, Tensor? add_mask=None, "
             "float? softmax_scale=None")
-_define(f"rope_attn_prefill({_PF_ARGS}) -> Tensor", _prefill, lambda q, *a, **k: q.new_empty(q.shape, dtype=_BF16))
+_define(f"rope_attn_prefill({_PF_ARGS}) -> Tensor", _prefill, lambda q, *a, **k: q.new_empty(q.shape))
 _define(f"rope_attn_prefill.out({_PF_ARGS}, *, Tensor(a!) out) -> Tensor(a!)", _prefill_out, lambda *a, out, **k: out)
 
 

@@ -51,6 +51,14 @@ const char* fsvd_last_error(void);
  * split-K workspace inside hipBLASLt). */
 int fsvd_set_workspace(void* ws, size_t bytes, void* stream);
 
+/* The fused product path below (projections, SwiGLU pair, q / k / v of the current token, attention over the dense
+ * cache, RMSNorm, head expansion and prompt attention) computes in the 16-bit type its `dtype` argument names,
+ * FSVD_BF16 or FSVD_FP16: every tensor of a call is of that type ("bf16" in the formulas stands for it), sums are
+ * fp32, roundings are to nearest even at the same points in both.  The reference picks the type from its inputs the
+ * same way (kernels/attn/decode/densekv_reconstruct_triton.py:427-428; fp16 is the default of its dense cache,
+ * runtime/cache/attn_dense_kv.py:26, and the fallback of scripts/demo_support/api.py:161-165).  The int4 entries and the
+ * persistent decode step are bf16 only. */
+
 /* y[b,n] = (res[b,n] +) bf16( W[n,:] . norm(x[b,:]) (+ bias[n]) ),  W is an nn.Linear weight [N,K].
  * norm_w != NULL fuses the RMSNorm of x (w * bf16(x * rsqrt(mean(x^2)+eps))) in front.
  * Replaces the factor GEMVs the reference issues through torch: rank projection
@@ -60,13 +68,13 @@ int fsvd_set_workspace(void* ws, size_t bytes, void* stream);
  * (benchmark/mlp/bench_svd_llama_decode_graph.py:78-83).  cfg = 0 picks the tiling. */
 int fsvd_linear(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* bias,
                 const void* norm_w, float eps, const void* res, int64_t ldres,
-                void* y, int64_t ldy, int B, int N, int K, int cfg, void* stream);
+                void* y, int64_t ldy, int B, int N, int K, int cfg, int dtype, void* stream);
 
 /* h[b,n] = silu(gate_u[n,:] . p[b,0:R]) * (up_u[n,:] . p[b,up_off:up_off+R]),  gate_u/up_u [D,R].
  * mode 0 rounds like a chain of bf16 nn.Linear modules, mode 1 like the fused reference kernel
  * (h = bf16(silu(g32)*u32), kernels/mlp/decode/dual_split_triton.py:207). */
 int fsvd_swiglu_linear(const void* p, int64_t ldp, int64_t up_off, const void* gate_u, const void* up_u,
-                       int64_t ldw, void* h, int64_t ldh, int B, int D, int R, int mode, int cfg, void* stream);
+                       int64_t ldw, void* h, int64_t ldh, int B, int D, int R, int mode, int cfg, int dtype, void* stream);
 
 /* The same projection on group-wise int4 weights: y[b,n] = (res[b,n] +) bf16( sum_k norm(x)[b,k] * s[n,g(k)] *
  * (q[n,k] - z[n,g(k)]) (+ bias[n]) ).  qweight [N, ldq] bytes holds two columns per byte (even column in the low
@@ -100,7 +108,7 @@ int fsvd_qkv_rope_append(const void* p, int64_t ldp, const void* q_u, int64_t ld
                          const void* v_u, int64_t ldv, const void* cos, const void* sin, int rope_len,
                          const int32_t* positions, void* q_out, void* k_cache, void* v_cache,
                          int64_t sc_b, int64_t sc_s, int64_t sc_h,
-                         int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int S, int cfg, void* stream);
+                         int B, int H, int Hk, int Dh, int Rq, int Rk, int Rv, int S, int cfg, int dtype, void* stream);
 
 /* Bytes of scratch fsvd_attn_decode_densekv needs for nsplit > 1: a 256 KiB block of int32 arrival
  * counters followed by the fp32 partials.  The workspace must be zero-filled before its first use;
@@ -121,7 +129,7 @@ int fsvd_attn_decode_densekv(const void* q, int64_t sq_b, int64_t sq_h,
                              const void* cos, const void* sin, int rope_len,
                              void* out, int64_t so_b, int64_t so_h,
                              void* workspace, size_t workspace_bytes,
-                             int B, int H, int Hk, int Dh, int S, int nsplit, float scale, void* stream);
+                             int B, int H, int Hk, int Dh, int S, int nsplit, float scale, int dtype, void* stream);
 
 /* fsvd_attn_decode_densekv with the split scratch held by the library itself: no workspace argument and no device
  * allocation anywhere in the call.  No counterpart in the reference; it exists for callers that cannot allocate
@@ -138,11 +146,12 @@ int fsvd_attn_decode_densekv_static(const void* q, int64_t sq_b, int64_t sq_h,
                                     const int32_t* cache_seqlens, int seqlen_add,
                                     const void* cos, const void* sin, int rope_len,
                                     void* out, int64_t so_b, int64_t so_h,
-                                    int B, int H, int Hk, int Dh, int S, int nsplit, float scale, void* stream);
+                                    int B, int H, int Hk, int Dh, int S, int nsplit, float scale, int dtype, void* stream);
 
 /* y = w * bf16(x * rsqrt(mean(x^2)+eps)) over rows of length K.
  * benchmark/mlp/bench_svd_llama_decode_graph.py:78-83. */
-int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, void* stream);
+int fsvd_rmsnorm(const void* x, int64_t ldx, const void* w, float eps, void* y, int64_t ldy, int rows, int K, int dtype,
+                 void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Reference operand layouts ("x @ W", W is [K, N]).  dtype is FSVD_BF16 / FSVD_FP16 / FSVD_FP32;
@@ -250,7 +259,7 @@ int fsvd_rankkv_append(const void* pk, int64_t ldpk, const void* pv, int64_t ldp
 int fsvd_lowrank_expand_heads(const void* p, int64_t sp_b, int64_t sp_m, int64_t sp_h, const void* u, int64_t ldu,
                               const void* bias, const void* cos, const void* sin, int rope_len, const int32_t* positions,
                               void* y, int64_t sy_b, int64_t sy_m, int64_t sy_h, int dst_by_position, int dst_rows,
-                              int B, int M, int heads, int Dh, int R, void* stream);
+                              int B, int M, int heads, int Dh, int R, int dtype, void* stream);
 /* The q, k and v expansions of one prompt pass in one call: the same results as `n` calls of
  * fsvd_lowrank_expand_heads on the same token rows (one per descriptor; `rotate` selects whether that one gets the
  * rotation), and a single launch when every one of them takes the tiled kernel (128 token rows and more, rank a
@@ -266,13 +275,13 @@ typedef struct fsvd_expand_desc {
   int32_t dst_by_position, dst_rows, rsv0;
 } fsvd_expand_desc;
 int fsvd_lowrank_expand_heads_multi(const fsvd_expand_desc* desc, int n, const void* cos, const void* sin, int rope_len,
-                                    const int32_t* positions, int B, int M, int Dh, void* stream);
+                                    const int32_t* positions, int B, int M, int Dh, int dtype, void* stream);
 int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
                       const void* k, const void* v, int64_t sk_b, int64_t sk_s, int64_t sk_h,
                       const int32_t* q_pos0, const uint8_t* pad_mask, int64_t spm_b,
                       const float* add_mask, int64_t sam_b, int64_t sam_q,
                       void* out, int64_t so_b, int64_t so_m, int64_t so_h,
-                      int B, int M, int H, int Hk, int Dh, int S, int causal, float scale, void* stream);
+                      int B, int M, int H, int Hk, int Dh, int S, int causal, float scale, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Persistent decode step (batch 1): ONE launch walks a caller-built list of phases — embedding row,

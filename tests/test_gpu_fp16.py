@@ -1,0 +1,222 @@
+"""The fused product path in float16 (dtype code FSVD_FP16 through the C ABI) against the CPU oracle run in float16.
+
+The reference switches its kernels on the input dtype, its dense cache defaults to float16 and its model cast falls back
+to float16 (kernels/attn/decode/densekv_reconstruct_triton.py:427-428, runtime/cache/attn_dense_kv.py:26,
+scripts/demo_support/api.py:161-165).  Here every entry point of the path takes the element type as an argument; the
+kernels are the bf16 ones instantiated with the float16 conversions, V_DOT2_F32_F16 and V_MFMA_F32_16X16X32_F16.
+
+Tolerance: float16 carries three more mantissa bits than bfloat16, so the bar is a quarter of the bf16 one
+(max-abs 5e-3, max-rel 2.5e-3); where max|ref| >= 2 the absolute bound is two float16 ulps at max|ref| (one ulp is
+0.002 in [2, 4)).  Greedy tokens identical on configuration 1.
+"""
+import pytest
+import torch
+
+from oracle import flashsvd_oracle as O
+from tests.util import assert_close_bf16, model_from_oracle
+
+pytestmark = pytest.mark.gpu
+FP16 = torch.float16
+
+
+def rand_fp16(*shape, std=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * std).to(FP16)
+
+
+def close(got, ref, what):
+    assert got.dtype == FP16, f"{what}: result is {got.dtype}"
+    m = float(ref.float().abs().max())
+    return assert_close_bf16(got, ref, what, abs_tol=5e-3 if m < 2.0 else 2.0 * m * 2.0 ** -10, rel_tol=2.5e-3)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from flashsvd_amd import hip_ops
+    return hip_ops
+
+
+# one row (vector kernels), three rows and more (matrix cores: streamed, resident, K-split forms), prompt rows (tiles)
+@pytest.mark.parametrize("B,N,K", [(1, 3072, 4096), (1, 1536, 11008), (2, 257, 512), (1, 7, 100), (3, 512, 4096), (8, 3072, 4096),
+                                   (16, 1536, 11008), (32, 4096, 1536), (17, 100, 2048), (20, 8192, 6144), (100, 200, 1536),
+                                   (512, 3072, 4096), (129, 130, 192), (384, 1536, 11008), (2048, 4096, 256)])
+def test_linear(ops, B, N, K):
+    x, w = rand_fp16(B, K, seed=1), rand_fp16(N, K, std=0.02, seed=2)
+    bias, res = rand_fp16(N, std=0.1, seed=4), rand_fp16(B, N, seed=5)
+    close(ops.linear(x.cuda(), w.cuda()), O.lin(x, w), f"linear {B}x{N}x{K}")
+    close(ops.linear(x.cuda(), w.cuda(), bias.cuda(), residual=res.cuda()), res + O.lin(x, w, bias), f"linear + bias + residual {B}x{N}x{K}")
+
+
+@pytest.mark.parametrize("B", [1, 2, 8, 200])
+def test_linear_with_fused_norm_and_rmsnorm(ops, B):
+    N, K = 512, 4096
+    x, w = rand_fp16(B, K, seed=1), rand_fp16(N, K, std=0.02, seed=2)
+    nw = rand_fp16(K, seed=3) * 0.1 + 1
+    close(ops.rmsnorm(x.cuda(), nw.cuda(), 1e-6), O.rms_norm(x, nw, 1e-6), "rmsnorm")
+    close(ops.linear(x.cuda(), w.cuda(), norm_weight=nw.cuda(), eps=1e-6), O.lin(O.rms_norm(x, nw, 1e-6), w), "norm + linear")
+
+
+@pytest.mark.parametrize("B,D,R,mode", [(1, 11008, 1536, 0), (1, 11008, 1536, 1), (2, 100, 52, 1), (8, 11008, 1536, 0), (32, 1376, 256, 1),
+                                        (24, 14336, 2048, 0), (512, 11008, 1536, 0), (256, 1376, 256, 1)])
+def test_swiglu_linear(ops, B, D, R, mode):
+    p = rand_fp16(B, 2 * R, seed=1)
+    gu, uu = rand_fp16(D, R, std=0.05, seed=2), rand_fp16(D, R, std=0.05, seed=3)
+    h = ops.swiglu_linear(p.cuda(), gu.cuda(), uu.cuda(), up_off=R, mode=mode)
+    g, u = p[:, :R].float() @ gu.float().t(), p[:, R:].float() @ uu.float().t()
+    if mode == 0:
+        ref = torch.nn.functional.silu(g.to(FP16)) * u.to(FP16)
+    else:
+        ref = ((g * torch.sigmoid(g)) * u).to(FP16)
+    close(h, ref, f"swiglu mode {mode} at {B} rows")
+
+
+@pytest.mark.parametrize("B,H,Hk,Dh,Rq,Rk,Rv", [(1, 32, 32, 128, 1024, 1024, 1024), (2, 8, 2, 64, 128, 96, 72), (3, 4, 4, 64, 52, 52, 52)])
+def test_qkv_rope_append(ops, B, H, Hk, Dh, Rq, Rk, Rv):
+    S = 40
+    p = rand_fp16(B, Rq + Rk + Rv, seed=1)
+    qu, ku, vu = rand_fp16(H * Dh, Rq, std=0.05, seed=2), rand_fp16(Hk * Dh, Rk, std=0.05, seed=3), rand_fp16(Hk * Dh, Rv, std=0.05, seed=4)
+    cos, sin = O.rope_tables(S, Dh, dtype=FP16)
+    pos = torch.tensor([(7 * b + 5) % S for b in range(B)], dtype=torch.int32)
+    kc = torch.zeros(B, S, Hk, Dh, dtype=FP16, device="cuda")
+    vc = torch.zeros_like(kc)
+    q = ops.qkv_rope_append(p.cuda(), qu.cuda(), ku.cuda(), vu.cuda(), cos.cuda(), sin.cuda(), pos.cuda(), kc, vc,
+                            num_heads=H, num_kv_heads=Hk, head_dim=Dh)
+    pq, pk, pv = p[:, :Rq], p[:, Rq:Rq + Rk], p[:, Rq + Rk:]
+    for b in range(B):
+        c, s = cos[pos[b]], sin[pos[b]]
+        close(q[b], O.apply_rope(O.lin(pq[b:b + 1], qu).reshape(H, Dh), c, s), "q")
+        close(kc[b, pos[b]], O.apply_rope(O.lin(pk[b:b + 1], ku).reshape(Hk, Dh), c, s), "k row")
+        close(vc[b, pos[b]], O.lin(pv[b:b + 1], vu).reshape(Hk, Dh), "v row")
+
+
+@pytest.mark.parametrize("B,H,Hk,Dh,L,S,nsplit", [(1, 32, 32, 128, 513, 560, 8), (2, 8, 2, 64, 37, 64, 3), (2, 4, 4, 64, 100, 128, 1),
+                                                 (16, 32, 8, 128, 300, 320, 4), (16, 32, 16, 128, 130, 160, 2)])
+def test_attn_decode_densekv(ops, B, H, Hk, Dh, L, S, nsplit):
+    q = rand_fp16(B, H, Dh, seed=1)
+    kc, vc = rand_fp16(B, S, Hk, Dh, seed=2), rand_fp16(B, S, Hk, Dh, seed=3)
+    lens = torch.tensor([max(1, L - 3 * b) for b in range(B)], dtype=torch.int32)
+    out = ops.attn_decode_densekv(q.cuda(), kc.cuda(), vc.cuda(), lens.cuda(), nsplit=nsplit)
+    for b in range(B):
+        n = int(lens[b])
+        close(out[b:b + 1], O.dense_decode_attn(q[b:b + 1], kc[b:b + 1, :n], vc[b:b + 1, :n]), f"attention b={b}")
+
+
+def test_attn_decode_appends_and_rotates_the_new_token(ops):
+    B, H, Hk, Dh, S, n = 2, 8, 4, 128, 64, 21
+    q, kn, vn = rand_fp16(B, H, Dh, seed=1), rand_fp16(B, Hk, Dh, seed=2), rand_fp16(B, Hk, Dh, seed=3)
+    kc, vc = rand_fp16(B, S, Hk, Dh, seed=4), rand_fp16(B, S, Hk, Dh, seed=5)
+    cos, sin = O.rope_tables(S, Dh, dtype=FP16)
+    lens = torch.full((B,), n, dtype=torch.int32)
+    kg, vg = kc.cuda(), vc.cuda()
+    out = ops.attn_decode_densekv(q.cuda(), kg, vg, lens.cuda(), k_new=kn.cuda(), v_new=vn.cuda(), cos=cos.cuda(), sin=sin.cuda(), nsplit=2)
+    ref = O.flash_attn_with_kvcache(q[:, None], kc.clone(), vc.clone(), k=kn[:, None], v=vn[:, None], cache_seqlens=lens,
+                                    rotary_cos=cos, rotary_sin=sin)
+    close(out, ref[:, 0], "attention with append")
+
+
+@pytest.mark.parametrize("B,M,R", [(2, 40, 72), (1, 512, 1024), (2, 200, 128)])
+def test_expand_heads_and_prompt_attention(ops, B, M, R):
+    H, Hk, dh = 8, 4, 128
+    S = M + 24
+    cos, sin = O.rope_tables(S, dh, dtype=FP16)
+    pq, pk, pv = rand_fp16(B, M, R, seed=1), rand_fp16(B, M, R, seed=2), rand_fp16(B, M, R, seed=3)
+    uq, uk, uv = rand_fp16(H * dh, R, std=R ** -0.5, seed=4), rand_fp16(Hk * dh, R, std=R ** -0.5, seed=5), rand_fp16(Hk * dh, R, std=R ** -0.5, seed=6)
+    q = torch.empty(B, M, H, dh, dtype=FP16, device="cuda")
+    kc = torch.zeros(B, S, Hk, dh, dtype=FP16, device="cuda")
+    vc = torch.zeros_like(kc)
+    pos0 = torch.zeros(B, dtype=torch.int32, device="cuda")
+    ops.lowrank_expand_heads_multi(
+        [dict(p=pq.cuda(), u=uq.cuda(), num_heads=H, out=q, rotate=True),
+         dict(p=pk.cuda(), u=uk.cuda(), num_heads=Hk, out=kc, rotate=True, dst_by_position=True),
+         dict(p=pv.cuda(), u=uv.cuda(), num_heads=Hk, out=vc, rotate=False, dst_by_position=True)],
+        head_dim=dh, cos=cos.cuda(), sin=sin.cuda(), positions=pos0)
+    c, s = cos[:M][None, :, None], sin[:M][None, :, None]
+    q_ref = O.apply_rope(O.lin(pq, uq).reshape(B, M, H, dh), c, s)
+    k_ref = O.apply_rope(O.lin(pk, uk).reshape(B, M, Hk, dh), c, s)
+    v_ref = O.lin(pv, uv).reshape(B, M, Hk, dh)
+    close(q, q_ref, "q expansion")
+    close(kc[:, :M], k_ref, "k expansion into cache rows")
+    close(vc[:, :M], v_ref, "v expansion into cache rows")
+    single = torch.zeros_like(kc)
+    ops.lowrank_expand_heads(pk.cuda(), uk.cuda(), num_heads=Hk, head_dim=dh, out=single, cos=cos.cuda(), sin=sin.cuda(),
+                             positions=pos0, dst_by_position=True)
+    assert torch.equal(single.cpu(), kc.cpu()), "one expansion and the batched launch differ"
+    out = ops.attn_prefill(q_ref.cuda(), k_ref.cuda(), v_ref.cuda(), q_pos0=pos0, causal=True)
+    for m in (0, M // 3, M - 1):
+        close(out[:, m], O.dense_decode_attn(q_ref[:, m], k_ref[:, :m + 1], v_ref[:, :m + 1]), f"prompt attention row {m}")
+
+
+def test_mixed_element_types_are_refused(ops):
+    x, w = rand_fp16(1, 256, seed=1).cuda(), rand_fp16(64, 256, seed=2).cuda()
+    with pytest.raises(ValueError, match="must be torch.float16"):
+        ops.linear(x, w.to(torch.bfloat16))
+    with pytest.raises(ValueError, match="bfloat16 or torch.float16"):
+        ops.linear(x.float(), w.float())
+
+
+def _greedy(model, prompt, n_new, graph):
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    B, Lp = prompt.shape
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=Lp + n_new + 4, device="cuda", dtype=FP16)
+    out = model(prompt.cuda(), past_key_values=cache, cache_position=torch.arange(Lp))
+    hid = [out.hidden_states[:, -1].clone()]
+    tok = out.logits[:, -1].float().argmax(-1, keepdim=True)
+    toks = [tok.clone()]
+    dec = GraphedDecoder(model, cache, B)
+    dec.set_state(tok, Lp)
+    if graph:
+        dec.capture()
+    for _ in range(1, n_new):
+        toks.append((dec.step() if graph else dec.eager_step()).clone())
+        hid.append(dec.hidden.clone())
+    return torch.cat(toks, 1).cpu(), torch.stack(hid, 1).cpu(), cache
+
+
+@pytest.mark.parametrize("graph", [False, True])
+def test_config1_block_greedy_16_identical_in_float16(graph):
+    # configuration 1 of the reference (d 512, 8 x 64 heads, ffn 1376, ranks 128 / 256, prompt 128, 16 greedy steps)
+    mw, prompt = O.config_c1(FP16)
+    model = model_from_oracle(mw)
+    assert model.lm_head.weight.dtype == FP16
+    ref_tok, ref_hid, ref_cache = O.greedy_decode(mw, prompt, 16, "dense", return_hidden=True)
+    tok, hid, cache = _greedy(model, prompt, 16, graph)
+    assert torch.equal(tok, ref_tok), f"greedy tokens differ: gpu {tok.tolist()} oracle {ref_tok.tolist()}"
+    close(cache.key_cache[0][:, :128], ref_cache.k[0][:, :128], "K cache")
+    close(cache.value_cache[0][:, :128], ref_cache.v[0][:, :128], "V cache")
+    for s in range(16):
+        close(hid[:, s], ref_hid[:, s], f"hidden state at step {s}")
+
+
+def test_7b_width_layer_teacher_forced_in_float16():
+    """One 7B-width layer on the oracle's own layer input: 160 prompt rows (tiled kernels) and one decode token."""
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    mw = O.make_model(d=4096, n_heads=32, n_kv_heads=32, head_dim=128, ffn=11008, attn_rank=1024, mlp_rank=1536,
+                      n_layers=1, vocab=1000, dtype=FP16, seed=0)
+    model = model_from_oracle(mw)
+    T = 160
+    ids = torch.randint(0, 1000, (1, T + 1), generator=torch.Generator().manual_seed(1))
+    cos, sin = O.rope_tables(T + 8, 128, dtype=FP16)
+    x = mw.embed[ids]
+    oc = O.DenseCache(mw, 1, T + 8, FP16)
+    y_pre = O.block_forward(mw, 0, x[:, :T], 0, oc, cos, sin)
+    y_dec = O.block_forward(mw, 0, x[:, T:], T, oc, cos, sin)
+    gc = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=T + 8, device="cuda", dtype=FP16)
+    layer = model.model.layers[0]
+    g_pre = layer(x[:, :T].cuda(), past_key_values=gc, cache_position=torch.arange(T))
+    g_dec = layer(x[:, T:].cuda(), past_key_values=gc, cache_position=torch.tensor([T]))
+    close(g_pre, y_pre, "prompt rows")
+    close(g_dec, y_dec, "decode token")
+    close(gc.key_cache[0][:, :T + 1], oc.k[0][:, :T + 1], "K cache")
+    close(gc.value_cache[0][:, :T + 1], oc.v[0][:, :T + 1], "V cache")
+
+
+def test_persistent_step_refuses_float16():
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    from flashsvd_amd.step import PersistentDecoder
+    mw, _ = O.config_c1(FP16)
+    model = model_from_oracle(mw)
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=64, device="cuda", dtype=FP16)
+    with pytest.raises(ValueError, match="bf16 only"):
+        PersistentDecoder(model, cache)

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     for name in sorted(declared):
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
     assert declared == set(_lib.SIGNATURES), "ctypes signature table and header disagree"
-    assert lib.fsvd_version() >= 100
+    assert lib.fsvd_version() >= 101
     assert isinstance(lib.fsvd_last_error(), bytes)
     # pure host-side size queries
     assert lib.fsvd_attn_decode_workspace_bytes(1, 32, 128, 8) == 256 * 1024 + 32 * 8 * 130 * 4
@@ -33,13 +33,13 @@ def test_library_exports_every_declared_symbol():
 def test_null_pointer_and_shape_errors_come_back_as_status_codes():
     from flashsvd_amd import _lib
     lib = _lib.load()
-    rc = lib.fsvd_linear(None, 8, None, 8, None, None, 1e-6, None, 0, None, 8, 1, 8, 8, 0, None)
+    rc = lib.fsvd_linear(None, 8, None, 8, None, None, 1e-6, None, 0, None, 8, 1, 8, 8, 0, 0, None)
     assert rc == -4 and b"NULL" in lib.fsvd_last_error()
     buf = ctypes.create_string_buffer(64)  # never dereferenced: shape check fails first
     p = ctypes.addressof(buf)
-    rc = lib.fsvd_linear(p, 4, p, 8, None, None, 1e-6, None, 0, p, 8, 1, 8, 8, 0, None)
+    rc = lib.fsvd_linear(p, 4, p, 8, None, None, 1e-6, None, 0, p, 8, 1, 8, 8, 0, 0, None)
     assert rc == -1 and b"leading dimension" in lib.fsvd_last_error()
-    rc = lib.fsvd_swiglu_linear(p, 16, 8, p, p, 8, p, 8, 1, 8, 8, 7, 0, None)
+    rc = lib.fsvd_swiglu_linear(p, 16, 8, p, p, 8, p, 8, 1, 8, 8, 7, 0, 0, None)
     assert rc == -1
     with pytest.raises(_lib.FlashSVDHipError):
         _lib.check("fsvd_linear", -1)

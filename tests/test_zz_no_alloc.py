@@ -20,7 +20,7 @@ def _call(lib, static, q, kc, vc, lens, out, nsplit, ws=None):
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     head = (q.data_ptr(), q.stride(0), q.stride(1), kc.data_ptr(), vc.data_ptr(), kc.stride(0), kc.stride(1), kc.stride(2),
             None, 0, 0, None, 0, 0, lens.data_ptr(), 0, None, None, 0, out.data_ptr(), out.stride(0), out.stride(1))
-    tail = (B, H, Hk, Dh, S, nsplit, 0.0, stream)
+    tail = (B, H, Hk, Dh, S, nsplit, 0.0, 0, stream)
     if static:
         return lib.fsvd_attn_decode_densekv_static(*head, *tail)
     return lib.fsvd_attn_decode_densekv(*head, ws.data_ptr(), ws.numel() * ws.element_size(), *tail)
