@@ -64,6 +64,9 @@ def _parse():
     ap.add_argument("--quant", action="store_true",
                     help="the same model with every factor quantised to group-wise int4 (group 128): decode tok/s of both engines "
                          "and the bytes that cross HBM per token, as its own JSON line")
+    ap.add_argument("--fp16", action="store_true",
+                    help="the same model held in float16 through the per-operator engine (the resident step is bf16 only): "
+                         "warm prompt pass and decode tok/s")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device copy 10 times (the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counters are scaled against) and exit")
@@ -302,17 +305,18 @@ def kernel_legs(model, cache, dec):
     return legs
 
 
-def run_lowrank(args):
+def run_lowrank(args, dtype=None):
     import torch
     from flashsvd_amd import llama
     from flashsvd_amd.graphs import GraphedDecoder
     from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
 
+    dtype = dtype or torch.bfloat16
     cfg = dict(CFG, num_layers=args.layers)
-    model = llama.materialize(llama.build_model(**cfg), "cuda", torch.bfloat16, seed=0)
+    model = llama.materialize(llama.build_model(**cfg), "cuda", dtype, seed=0)
     B = 1
     max_len = PROMPT_LEN + args.warmup + args.steps + 8
-    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=torch.bfloat16)
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=dtype)
     prompt = torch.randint(0, cfg["vocab_size"], (B, PROMPT_LEN), generator=torch.Generator().manual_seed(1)).cuda()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -323,7 +327,7 @@ def run_lowrank(args):
     res = dict(prefill_s=t_prefill)
     # the first pass pays one-time set-up (weight packing, tables, kernel attributes): time warm passes as well
     reps = args.steps if args.prefill_only else 2
-    scratch = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=torch.bfloat16)
+    scratch = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=dtype)
     for _ in range(args.warmup if args.prefill_only else 1):
         model(prompt, past_key_values=scratch, cache_position=torch.arange(PROMPT_LEN), logits_to_keep=1)
     torch.cuda.synchronize()
@@ -357,6 +361,8 @@ def run_lowrank(args):
         torch.cuda.synchronize()
         t_decode = time.perf_counter() - t1
         res["graph"] = dict(tok_s=B * args.steps / t_decode, ms_per_step=t_decode * 1000.0 / args.steps)
+    if dtype != torch.bfloat16:
+        return res
     if args.engine in ("persistent", "both"):
         from flashsvd_amd.step import PersistentDecoder
         cache._seen_tokens = PROMPT_LEN
@@ -913,6 +919,13 @@ def main():
                           "unit": "tok/s", "n_gpus": 1, "steps": mp["decode"]["steps"], "dtype": "bf16", "data": "synthetic",
                           "config": {"workload": mp["model"] + "; prefill 8 x 2048, then decode batch 16 at context 4096", "layers": args.layers},
                           "model_pass": mp, "kernels": kern}))
+        return
+    if args.fp16:
+        args.engine = "graph"
+        lr = run_lowrank(args, torch.float16)
+        print(json.dumps({"metric": "decode tok/s, 7B-shape rank-0.5 bs1, float16, per-operator HIP graph", "value": lr["graph"]["tok_s"],
+                          "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": lr["graph"]["ms_per_step"],
+                          "dtype": "fp16", "data": "synthetic", "prefill": lr["prefill"]}))
         return
     lr = run_lowrank(args)
     if args.kernel_configs_only:

@@ -121,7 +121,7 @@ SIGNATURES = {
     "fsvd_attn_decode_rankkv": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64,
                                         c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                         c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
-                                        c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
+                                        c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_int, c_void_p]),
     "fsvd_attn_decode_rankkv_scores_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "fsvd_rankkv_append": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p,
                                    c_int, c_int, c_int, c_int, c_void_p]),

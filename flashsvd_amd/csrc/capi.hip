@@ -486,7 +486,7 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h, const voi
                             int64_t ldvu, const void* bv, const void* cos, const void* sin, int rope_len, int rotate_q,
                             const int32_t* cache_seqlens, int seqlen_add, float* ws_m, float* ws_l, float* ws_acc, void* out,
                             int64_t so_b, int64_t so_h, int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit,
-                            float scale, float* scores, size_t scores_bytes, void* stream) {
+                            float scale, float* scores, size_t scores_bytes, int dtype, void* stream) {
   const char* fn = "fsvd_attn_decode_rankkv";
   FSVD_REQUIRE_PTR(q, fn); FSVD_REQUIRE_PTR(pk_cache, fn); FSVD_REQUIRE_PTR(pv_cache, fn); FSVD_REQUIRE_PTR(k_u, fn);
   FSVD_REQUIRE_PTR(v_u, fn); FSVD_REQUIRE_PTR(cache_seqlens, fn); FSVD_REQUIRE_PTR(ws_m, fn); FSVD_REQUIRE_PTR(ws_l, fn);
@@ -506,6 +506,7 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h, const voi
     if ((reinterpret_cast<uintptr_t>(scores) & 15) != 0) { set_last_error("%s: the score buffer must be 16-byte aligned", fn); return kErrBadAlign; }
     a.scores = scores;
   }
+  a.dt = dtype;
   return launch_rank_decode(a, static_cast<hipStream_t>(stream));
 }
 

@@ -28,17 +28,17 @@
 
 namespace fsvd {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kRdThreads = 256;
 constexpr int kRdTileKeys = 64;   // 4 waves x 16 keys
 constexpr int kRdMaxChunks = 4;   // rank-space accumulator: R <= 4 * 512
 
-__device__ __forceinline__ bf16x8_t ld_frag(const uint16_t* p) {
-  return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(p));
+template <class F>
+__device__ __forceinline__ F ld_frag(const uint16_t* p) {
+  return __builtin_bit_cast(F, *reinterpret_cast<const u32x4_t*>(p));
 }
-__device__ __forceinline__ bf16x8_t zero_frag() { return __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u}); }
+template <class F>
+__device__ __forceinline__ F zero_frag() { return __builtin_bit_cast(F, u32x4_t{0u, 0u, 0u, 0u}); }
 
 // dynamic LDS of the partial kernel: k_u stages [stage][128 d][64 r] bf16 (two, or three in the deep form), reused for the
 // four waves' rank-space partials [4][kRdMaxChunks * 512] fp32 at the end; then the waves' Pk slots
@@ -60,8 +60,10 @@ template <int KS, bool PKL, bool DEEP, bool SC = false> struct RankDecodeLds {
 // SC (long caches, scratch registered): the kernel stops at the scores.  It writes s[b, key, h] = q_h . K_key * scale to
 // a.scores and leaves the softmax and the rank-space accumulation to rank_decode_softmax_kernel / rank_decode_pv_kernel,
 // which read every Pv row once for a group of heads instead of once per head.
-template <int REP, int KS, bool PKL, bool DEEP = false, bool SC = false>
+template <int DT, int REP, int KS, bool PKL, bool DEEP = false, bool SC = false>
 __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(RankDecodeArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   static_assert(!DEEP || (PKL && KS == 1), "the deep form is built for single sub-tiles with Pk through LDS");
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2;
   __shared__ float wm[4][REP], wl[4][REP];
@@ -99,10 +101,10 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   for (int i = tid; i < REP * HALF; i += kRdThreads) {
     const int g = i / HALF, d = i % HALF;
     const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)(h0 + g) * a.sq_h;
-    float x0 = bf16_bits_to_f32(qp[d]), x1 = bf16_bits_to_f32(qp[d + HALF]);
+    float x0 = E::val(qp[d]), x1 = E::val(qp[d + HALF]);
     if (a.rotate_q) {
       const int tp = min(max(n_keys - 1, 0), a.rope_len - 1);
-      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * HALF + d]), sn = bf16_bits_to_f32(a.sin[(int64_t)tp * HALF + d]);
+      const float c = E::val(a.cos[(int64_t)tp * HALF + d]), sn = E::val(a.sin[(int64_t)tp * HALF + d]);
       const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
       x0 = r0; x1 = r1;
     }
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
     const uint16_t* kug = ku_h + (int64_t)kd * a.ldku + kcol;
     const int nstep = (a.Rk + 63) / 64;
     u32x4_t kreg[4];
-    bf16x8_t af[KS][2];
+    frag_t af[KS][2];
     const auto load_ku = [&](int r0) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
 #pragma unroll
       for (int j = 0; j < KS; ++j)
 #pragma unroll
-        for (int k = 0; k < 2; ++k) af[j][k] = (r0 + k * 32 + lg * 8 < a.Rk) ? ld_frag(arow[j] + r0 + k * 32) : zero_frag();
+        for (int k = 0; k < 2; ++k) af[j][k] = (r0 + k * 32 + lg * 8 < a.Rk) ? ld_frag<frag_t>(arow[j] + r0 + k * 32) : zero_frag<frag_t>();
     };
     // PKL: lane -> key row lane / 8 (+ 8 per instruction) and the piece that belongs at LDS position lane % 8 of that row
     // (position p of row r holds piece p ^ r % 8: conflict-free 16-byte fragment reads)
@@ -199,7 +201,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
       for (int j = 0; j < KS; ++j)
 #pragma unroll
         for (int k = 0; k < 2; ++k)
-          af[j][k] = *reinterpret_cast<const bf16x8_t*>(myslot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
+          af[j][k] = *reinterpret_cast<const frag_t*>(myslot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
     };
     if constexpr (DEEP) {
       // lane -> LDS row wave * 32 + i * 8 + lane / 8 and position lane % 8 of a stage; the row holds head dimension kd(row)
@@ -234,7 +236,7 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int k = 0; k < 2; ++k)
-          af[0][k] = *reinterpret_cast<const bf16x8_t*>(myslot + (st & 1) * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
+          af[0][k] = *reinterpret_cast<const frag_t*>(myslot + (st & 1) * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
         __builtin_amdgcn_s_waitcnt(kNoVm | (0 << 8));            // fragments in registers: the slot is free again
         // everyone's pieces of chunk st are in, and stage (st - 1) % 3 is read out (its fragments fed matrix products that
         // precede this point).  The bare barrier instruction: __syncthreads() carries a fence that waits for ALL of the
@@ -246,11 +248,11 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         const int cur = st % 3;
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
-          bf16x8_t bf[NT];
+          frag_t bf[NT];
 #pragma unroll
-          for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+          for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
 #pragma unroll
-          for (int t = 0; t < NT; ++t) accs[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[0][k], bf[t], accs[0][t], 0, 0, 0);
+          for (int t = 0; t < NT; ++t) accs[0][t] = E::mfma(af[0][k], bf[t], accs[0][t]);
         }
       }
       __syncthreads();                                           // the last stages are read out before the next tile refills them
@@ -317,9 +319,9 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         for (int k = 0; k < 2; ++k) {
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
-            const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+            const frag_t bf = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
 #pragma unroll
-            for (int j = 0; j < KS; ++j) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][k], bf, accs[j][t], 0, 0, 0);
+            for (int j = 0; j < KS; ++j) accs[j][t] = E::mfma(af[j][k], bf, accs[j][t]);
           }
         }
       }
@@ -344,13 +346,13 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
       if (st + 1 < nstep) load_ku((st + 1) * 64);
 #pragma unroll
       for (int k = 0; k < 2; ++k) {
-        bf16x8_t bf[NT];
+        frag_t bf[NT];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+        for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
 #pragma unroll
         for (int j = 0; j < KS; ++j)
 #pragma unroll
-          for (int t = 0; t < NT; ++t) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][k], bf[t], accs[j][t], 0, 0, 0);
+          for (int t = 0; t < NT; ++t) accs[j][t] = E::mfma(af[j][k], bf[t], accs[j][t]);
       }
       if (st + 1 < nstep) {
         if (!PKL) load_pk((st + 1) * 64);          // lands while the chunk is handed over
@@ -371,8 +373,8 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         const int pos = min(wkey0 + lg * 4 + i, a.rope_len - 1);
         const uint2 cw = *reinterpret_cast<const uint2*>(a.cos + (int64_t)pos * HALF + lr * 4);
         const uint2 sw = *reinterpret_cast<const uint2*>(a.sin + (int64_t)pos * HALF + lr * 4);
-        const float cv[4] = {bf16_lo(cw.x), bf16_hi(cw.x), bf16_lo(cw.y), bf16_hi(cw.y)};
-        const float sv[4] = {bf16_lo(sw.x), bf16_hi(sw.x), bf16_lo(sw.y), bf16_hi(sw.y)};
+        const float cv[4] = {E::lo(cw.x), E::hi(cw.x), E::lo(cw.y), E::hi(cw.y)};
+        const float sv[4] = {E::lo(sw.x), E::hi(sw.x), E::lo(sw.y), E::hi(sw.y)};
 #pragma unroll
         for (int t = 0; t < NT / 2; ++t) {
           const float x0 = acc[t][i], x1 = acc[t + NT / 2][i];
@@ -433,10 +435,10 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
             const int key = min(wkey0 + kk, k1 - 1);   // p is 0 for clamped keys
             const u32x4_t v = *reinterpret_cast<const u32x4_t*>(pv_b + (int64_t)key * a.spv_s + r);
             const float pw = pk16[kk];
-            tacc[g][c][0] += pw * bf16_lo(v.x); tacc[g][c][1] += pw * bf16_hi(v.x);
-            tacc[g][c][2] += pw * bf16_lo(v.y); tacc[g][c][3] += pw * bf16_hi(v.y);
-            tacc[g][c][4] += pw * bf16_lo(v.z); tacc[g][c][5] += pw * bf16_hi(v.z);
-            tacc[g][c][6] += pw * bf16_lo(v.w); tacc[g][c][7] += pw * bf16_hi(v.w);
+            tacc[g][c][0] += pw * E::lo(v.x); tacc[g][c][1] += pw * E::hi(v.x);
+            tacc[g][c][2] += pw * E::lo(v.y); tacc[g][c][3] += pw * E::hi(v.y);
+            tacc[g][c][4] += pw * E::lo(v.z); tacc[g][c][5] += pw * E::hi(v.z);
+            tacc[g][c][6] += pw * E::lo(v.w); tacc[g][c][7] += pw * E::hi(v.w);
           }
         }
       }
@@ -482,8 +484,10 @@ template <int KS> struct RankPairLds {
   static constexpr int kSlot = KS * 2048;                        // Pk of KS sub-tiles x 16 keys x 128 bytes
   static constexpr int kBytes = 2 * kKu + 4 * 2 * kSlot;         // both heads' stages, then [pair of waves][2 slots]
 };
-template <int KS>
+template <int DT, int KS>
 __global__ __launch_bounds__(kRdPairThreads, 1) void rank_scores_pair_kernel(RankDecodeArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   static_assert(KS == 2 || KS == 4, "the two waves of a pair fill half of the sub-tiles each");
   constexpr int DH = 128, NT = DH / 16, HALF = DH / 2, KROW = 64;
   typedef RankPairLds<KS> Lds;
@@ -511,10 +515,10 @@ __global__ __launch_bounds__(kRdPairThreads, 1) void rank_scores_pair_kernel(Ran
   for (int i = tid; i < 2 * HALF; i += kRdPairThreads) {
     const int g = i / HALF, d = i % HALF;
     const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)(2 * gy + g) * a.sq_h;
-    float x0 = bf16_bits_to_f32(qp[d]), x1 = bf16_bits_to_f32(qp[d + HALF]);
+    float x0 = E::val(qp[d]), x1 = E::val(qp[d + HALF]);
     if (a.rotate_q) {
       const int tp = min(max(n_keys - 1, 0), a.rope_len - 1);
-      const float c = bf16_bits_to_f32(a.cos[(int64_t)tp * HALF + d]), sn = bf16_bits_to_f32(a.sin[(int64_t)tp * HALF + d]);
+      const float c = E::val(a.cos[(int64_t)tp * HALF + d]), sn = E::val(a.sin[(int64_t)tp * HALF + d]);
       const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
       x0 = r0; x1 = r1;
     }
@@ -584,19 +588,19 @@ __global__ __launch_bounds__(kRdPairThreads, 1) void rank_scores_pair_kernel(Ran
       __builtin_amdgcn_sched_barrier(0);
       const int cur = st & 1;
       const unsigned char* slot = slots + cur * Lds::kSlot;
-      bf16x8_t af[KS][2];
+      frag_t af[KS][2];
 #pragma unroll
       for (int j = 0; j < KS; ++j)
 #pragma unroll
         for (int k = 0; k < 2; ++k)
-          af[j][k] = *reinterpret_cast<const bf16x8_t*>(slot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
+          af[j][k] = *reinterpret_cast<const frag_t*>(slot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
 #pragma unroll
       for (int k = 0; k < 2; ++k) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-          const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+          const frag_t bf = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
 #pragma unroll
-          for (int j = 0; j < KS; ++j) accs[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[j][k], bf, accs[j][t], 0, 0, 0);
+          for (int j = 0; j < KS; ++j) accs[j][t] = E::mfma(af[j][k], bf, accs[j][t]);
         }
       }
     }
@@ -612,8 +616,8 @@ __global__ __launch_bounds__(kRdPairThreads, 1) void rank_scores_pair_kernel(Ran
           const int pos = min(wkey0 + lg * 4 + i, a.rope_len - 1);
           const uint2 cw = *reinterpret_cast<const uint2*>(a.cos + (int64_t)pos * HALF + lr * 4);
           const uint2 sw = *reinterpret_cast<const uint2*>(a.sin + (int64_t)pos * HALF + lr * 4);
-          const float cv[4] = {bf16_lo(cw.x), bf16_hi(cw.x), bf16_lo(cw.y), bf16_hi(cw.y)};
-          const float sv[4] = {bf16_lo(sw.x), bf16_hi(sw.x), bf16_lo(sw.y), bf16_hi(sw.y)};
+          const float cv[4] = {E::lo(cw.x), E::hi(cw.x), E::lo(cw.y), E::hi(cw.y)};
+          const float sv[4] = {E::lo(sw.x), E::hi(sw.x), E::lo(sw.y), E::hi(sw.y)};
 #pragma unroll
           for (int t = 0; t < NT / 2; ++t) {
             const float x0 = acc[t][i], x1 = acc[t + NT / 2][i];
@@ -647,7 +651,10 @@ __global__ __launch_bounds__(kRdPairThreads, 1) void rank_scores_pair_kernel(Ran
 // lo = bf16(p - hi), so that hi + lo carries p to 2^-17 and the consumer needs no arithmetic on them.  Keys between the end
 // of the cache row and the next multiple of 64 get weight 0.  grid (nsplit, H, B), 256 threads; rows of the score buffer
 // are a.score_ld floats apart (a multiple of 64).
+template <int DT>
 __global__ __launch_bounds__(kRdThreads) void rank_decode_softmax_kernel(RankDecodeArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   __shared__ float red[4];
   const int s = blockIdx.x, h = blockIdx.y, b = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int n_keys = a.seqlens[b] + a.seqlen_add;
@@ -688,8 +695,8 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_softmax_kernel(RankDec
     for (int i = 0; i < 8; ++i) {
       const float p = (k + i < k1) ? __expf((i < 4 ? x0[i] : x1[i - 4]) - M) : 0.f;
       l += p;
-      hi[i] = f32_to_bf16_bits(p);
-      lo[i] = f32_to_bf16_bits(p - bf16_bits_to_f32(hi[i]));
+      hi[i] = E::bits(p);
+      lo[i] = E::bits(p - E::val(hi[i]));
     }
     uint32_t* wp = reinterpret_cast<uint32_t*>(sp + k);
     *reinterpret_cast<u32x4_t*>(wp) = u32x4_t{hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)};
@@ -712,8 +719,10 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_softmax_kernel(RankDec
 // kernel left in the score buffer, 32 bytes per head and 8 keys) in LDS, two blocks ahead in registers; a lane gathers its
 // B fragment (8 keys of one column) with 2-byte LDS reads and takes its A fragments with 16-byte ones; two matrix
 // products per tile so that the sum keeps fp32 weights; fp32 accumulation in key order.
-template <int MT>
+template <int DT, int MT>
 __global__ __launch_bounds__(kRdThreads) void rank_decode_pv_kernel(RankDecodeArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   // LDS rows: 128 columns of a key in 260 bytes (8 rows apart = 8 banks apart: the four key groups of a fragment gather
   // from disjoint banks), the 64 keys of a head in 272 bytes (16 heads read 16 bytes each from disjoint banks)
   constexpr int KB = 64, NT = 2, PITCH = 260, WPITCH = 272, HT = 16 * MT;
@@ -783,11 +792,11 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_pv_kernel(RankDecodeAr
         for (int j = 0; j < 8; ++j) e[j] = *reinterpret_cast<const uint16_t*>(&tile[buf][(ks * 32 + lg * 8 + j) * PITCH + (wave * 32 + nt * 16 + lr) * 2]);
         const u32x4_t bw{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
                          (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
-        const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, bw);
+        const frag_t bf = __builtin_bit_cast(frag_t, bw);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[mt][0]), bf, acc[mt][nt], 0, 0, 0);
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, af[mt][1]), bf, acc[mt][nt], 0, 0, 0);
+          acc[mt][nt] = E::mfma(__builtin_bit_cast(frag_t, af[mt][0]), bf, acc[mt][nt]);
+          acc[mt][nt] = E::mfma(__builtin_bit_cast(frag_t, af[mt][1]), bf, acc[mt][nt]);
         }
       }
     }
@@ -834,7 +843,10 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_pv_kernel(RankDecodeAr
 // 128 / gridDim.z rows of v_u[h]; a wave takes four rows at a time with all of their loads in flight.  With one workgroup
 // per head and one row per wave at a time, a batch-1 call spent 36 us here on 32 compute units (8 MB of v_u, one load
 // latency per row).
+template <int DT>
 __global__ __launch_bounds__(kRdThreads) void rank_decode_merge_kernel(RankDecodeArgs a) {
+  typedef E16<DT> E;
+  typedef typename E::frag_t frag_t;
   constexpr int DH = 128, RW = 4, NIT = kRdMaxChunks;
   __shared__ __align__(16) float ts[kRdMaxChunks * 512];
   const int h = blockIdx.x, b = blockIdx.y;
@@ -900,16 +912,16 @@ __global__ __launch_bounds__(kRdThreads) void rank_decode_merge_kernel(RankDecod
       const f32x4_t t0 = *reinterpret_cast<const f32x4_t*>(&ts[r]), t1 = *reinterpret_cast<const f32x4_t*>(&ts[r + 4]);
 #pragma unroll
       for (int j = 0; j < RW; ++j)
-        acc[j] += t0[0] * bf16_lo(v[j][it].x) + t0[1] * bf16_hi(v[j][it].x) + t0[2] * bf16_lo(v[j][it].y) + t0[3] * bf16_hi(v[j][it].y) +
-                  t1[0] * bf16_lo(v[j][it].z) + t1[1] * bf16_hi(v[j][it].z) + t1[2] * bf16_lo(v[j][it].w) + t1[3] * bf16_hi(v[j][it].w);
+        acc[j] += t0[0] * E::lo(v[j][it].x) + t0[1] * E::hi(v[j][it].x) + t0[2] * E::lo(v[j][it].y) + t0[3] * E::hi(v[j][it].y) +
+                  t1[0] * E::lo(v[j][it].z) + t1[1] * E::hi(v[j][it].z) + t1[2] * E::lo(v[j][it].w) + t1[3] * E::hi(v[j][it].w);
     }
 #pragma unroll
     for (int j = 0; j < RW; ++j) {
       float o = wave_sum(acc[j]);
       if (lane == 0) {
         const int d = d0 + dd + j;
-        if (a.bv) o += bf16_bits_to_f32(a.bv[hk * DH + d]);
-        outp[d] = (uint16_t)f32_to_bf16_bits(o);
+        if (a.bv) o += E::val(a.bv[hk * DH + d]);
+        outp[d] = (uint16_t)E::bits(o);
       }
     }
   }
@@ -922,7 +934,8 @@ size_t rank_decode_scores_floats(int B, int H, int S, int64_t spv_h) {
   return n >= ((size_t)1 << 17) ? n : 0;
 }
 
-int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
+template <int DT>
+static int launch_rank_decode_t(const RankDecodeArgs& a, hipStream_t st) {
   const char* fn = "fsvd_attn_decode_rankkv";
   if (a.B <= 0 || a.H <= 0 || a.Hk <= 0 || a.H % a.Hk != 0 || a.S <= 0 || a.nsplit <= 0) {
     set_last_error("%s: bad shape B=%d H=%d Hk=%d S=%d nsplit=%d", fn, a.B, a.H, a.Hk, a.S, a.nsplit);
@@ -967,24 +980,24 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     constexpr int lds = RankDecodeLds<KS_, PKL_, DEEP_>::kBytes;                                                                    \
     static bool granted = false;                                                                                                    \
     if (!granted && lds >= 48 * 1024) {                                                                                             \
-      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_decode_partial_kernel<REP_, KS_, PKL_, DEEP_>),       \
+      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_decode_partial_kernel<DT, REP_, KS_, PKL_, DEEP_>),       \
                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);                                         \
       if (ea != hipSuccess) { set_last_error("%s: cannot reserve %d bytes of LDS: %s", fn, lds, hipGetErrorString(ea)); return kErrLaunch; } \
       granted = true;                                                                                                               \
     }                                                                                                                               \
-    hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, PKL_, DEEP_>), dim3(a.nsplit, GY_, a.B), block, lds, st, a);          \
+    hipLaunchKernelGGL((rank_decode_partial_kernel<DT, REP_, KS_, PKL_, DEEP_>), dim3(a.nsplit, GY_, a.B), block, lds, st, a);          \
   } while (0)
 #define FSVD_RD_LAUNCH_SC(REP_, KS_, PKL_, GY_)                                                                                      \
   do {                                                                                                                              \
     constexpr int lds = RankDecodeLds<KS_, PKL_, false, true>::kBytes;                                                              \
     static bool granted = false;                                                                                                    \
     if (!granted && lds >= 48 * 1024) {                                                                                             \
-      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_decode_partial_kernel<REP_, KS_, PKL_, false, true>), \
+      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_decode_partial_kernel<DT, REP_, KS_, PKL_, false, true>), \
                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);                                         \
       if (ea != hipSuccess) { set_last_error("%s: cannot reserve %d bytes of LDS: %s", fn, lds, hipGetErrorString(ea)); return kErrLaunch; } \
       granted = true;                                                                                                               \
     }                                                                                                                               \
-    hipLaunchKernelGGL((rank_decode_partial_kernel<REP_, KS_, PKL_, false, true>), dim3(a.nsplit, GY_, a.B), block, lds, st, a3);   \
+    hipLaunchKernelGGL((rank_decode_partial_kernel<DT, REP_, KS_, PKL_, false, true>), dim3(a.nsplit, GY_, a.B), block, lds, st, a3);   \
   } while (0)
 #define FSVD_RD_LAUNCH(REP_, KS_, GY_)                                                                                              \
   do {                                                                                                                              \
@@ -1004,12 +1017,12 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     constexpr int lds = RankPairLds<KS_>::kBytes;                                                                                   \
     static bool granted = false;                                                                                                    \
     if (!granted) {                                                                                                                 \
-      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_scores_pair_kernel<KS_>),                             \
+      hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(&rank_scores_pair_kernel<DT, KS_>),                             \
                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);                                         \
       if (ea != hipSuccess) { set_last_error("%s: cannot reserve %d bytes of LDS: %s", fn, lds, hipGetErrorString(ea)); return kErrLaunch; } \
       granted = true;                                                                                                               \
     }                                                                                                                               \
-    hipLaunchKernelGGL((rank_scores_pair_kernel<KS_>), dim3(a.nsplit, a.Hk / 2, a.B), dim3(kRdPairThreads), lds, st, a3);           \
+    hipLaunchKernelGGL((rank_scores_pair_kernel<DT, KS_>), dim3(a.nsplit, a.Hk / 2, a.B), dim3(kRdPairThreads), lds, st, a3);           \
   } while (0)
       if (per >= 256) FSVD_RD_LAUNCH_PAIR(4); else FSVD_RD_LAUNCH_PAIR(2);
 #undef FSVD_RD_LAUNCH_PAIR
@@ -1020,11 +1033,11 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
     else { if (pk3) FSVD_RD_LAUNCH_SC(1, 2, true, a.Hk * rep); else FSVD_RD_LAUNCH_SC(1, 2, false, a.Hk * rep); }
     hipError_t e3 = hipGetLastError();
     if (e3 != hipSuccess) { set_last_error("%s: score launch failed: %s", fn, hipGetErrorString(e3)); return kErrLaunch; }
-    hipLaunchKernelGGL(rank_decode_softmax_kernel, dim3(a.nsplit, a.H, a.B), block, 0, st, a3);
+    hipLaunchKernelGGL(rank_decode_softmax_kernel<DT>, dim3(a.nsplit, a.H, a.B), block, 0, st, a3);
     const int mt = a.H > 16 ? 2 : 1;
     const dim3 gpv((a.Rv + 127) / 128, a.nsplit * ((a.H + 16 * mt - 1) / (16 * mt)), a.B);
-    if (mt == 2) hipLaunchKernelGGL(rank_decode_pv_kernel<2>, gpv, block, 0, st, a3);
-    else hipLaunchKernelGGL(rank_decode_pv_kernel<1>, gpv, block, 0, st, a3);
+    if (mt == 2) hipLaunchKernelGGL((rank_decode_pv_kernel<DT, 2>), gpv, block, 0, st, a3);
+    else hipLaunchKernelGGL((rank_decode_pv_kernel<DT, 1>), gpv, block, 0, st, a3);
     e3 = hipGetLastError();
     if (e3 != hipSuccess) { set_last_error("%s: softmax / accumulation launch failed: %s", fn, hipGetErrorString(e3)); return kErrLaunch; }
   } else
@@ -1044,10 +1057,15 @@ int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
   // head-dimension slices: enough workgroups for two per compute unit, at most eight per head (16 rows each)
   int dz = 1;
   while (dz < 8 && (int64_t)a.H * a.B * dz < 512) dz *= 2;
-  hipLaunchKernelGGL(rank_decode_merge_kernel, dim3(a.H, a.B, dz), block, 0, st, a);
+  hipLaunchKernelGGL(rank_decode_merge_kernel<DT>, dim3(a.H, a.B, dz), block, 0, st, a);
   e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("%s: stage 2 launch failed: %s", fn, hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
+}
+
+int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st) {
+  if (a.dt != 0 && a.dt != 1) { set_last_error("fsvd_attn_decode_rankkv: dtype code %d (bf16 = 0 and fp16 = 1 are served)", a.dt); return kErrBadDtype; }
+  return a.dt == 1 ? launch_rank_decode_t<1>(a, st) : launch_rank_decode_t<0>(a, st);
 }
 
 // One token's rank coefficients into the caches: cache[b, positions[b], :] = row b (16-byte pieces; a row whose position

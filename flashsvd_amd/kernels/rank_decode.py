@@ -73,11 +73,16 @@ def rank_decode(q: torch.Tensor, pk_cache: torch.Tensor, pv_cache: torch.Tensor,
 def _rank_decode_impl(q, pk_cache, pv_cache, k_u, v_u, cos, sin, seqlens, num_kv_heads, seqlen_add, rotate_q, bv, nsplit,
                       ws_m, ws_l, ws_acc, out, softmax_scale):
     workspace = None if ws_m is None else (ws_m, ws_l, ws_acc)
-    for t, nm in ((q, "q"), (pk_cache, "pk_cache"), (pv_cache, "pv_cache"), (k_u, "k_u"), (v_u, "v_u")):
+    codes = {torch.bfloat16: 0, torch.float16: 1}      # FSVD_BF16, FSVD_FP16: q names the element type of the call
+    if q.dtype not in codes:
+        raise ValueError(f"rank-space decode computes in bfloat16 or float16; q is {q.dtype}")
+    for t, nm in ((q, "q"), (pk_cache, "pk_cache"), (pv_cache, "pv_cache"), (k_u, "k_u"), (v_u, "v_u"), (bv, "bv"), (cos, "cos"), (sin, "sin")):
+        if t is None:
+            continue
         if not t.is_cuda:
             raise ValueError(f"{nm} must be a GPU tensor")
-        if t.dtype != torch.bfloat16:
-            raise ValueError(f"rank-space decode is implemented for bfloat16 only; {nm} is {t.dtype}")
+        if t.dtype != q.dtype:
+            raise ValueError(f"rank-space decode: {nm} is {t.dtype}, q is {q.dtype}")
     B, H, Dh = q.shape
     Hk = int(num_kv_heads)
     if pk_cache.dim() == 3:
@@ -127,7 +132,7 @@ def _rank_decode_impl(q, pk_cache, pv_cache, k_u, v_u, cos, sin, seqlens, num_kv
         None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rope_len, int(bool(rotate_q)),
         seqlens.data_ptr(), int(seqlen_add), M.data_ptr(), L.data_ptr(), Acc.data_ptr(), out.data_ptr(), out.stride(0),
         out.stride(1), B, H, Hk, Dh, S, Rk, Rv, int(nsplit), float(softmax_scale) if softmax_scale else 0.0,
-        None if scores is None else scores.data_ptr(), need, stream())
+        None if scores is None else scores.data_ptr(), need, codes[q.dtype], stream())
     check("fsvd_attn_decode_rankkv", rc)
     return out
 
@@ -142,8 +147,8 @@ def rankkv_append(pk: torch.Tensor, pv: torch.Tensor, pk_cache: torch.Tensor, pv
 
 def _rankkv_append_impl(pk, pv, pk_cache, pv_cache, positions):
     for t, nm in ((pk, "pk"), (pv, "pv"), (pk_cache, "pk_cache"), (pv_cache, "pv_cache")):
-        if not t.is_cuda or t.dtype != torch.bfloat16:
-            raise ValueError(f"{nm} must be a bfloat16 GPU tensor")
+        if not t.is_cuda or t.dtype not in (torch.bfloat16, torch.float16) or t.dtype != pk.dtype:
+            raise ValueError(f"{nm} must be a bfloat16 or float16 GPU tensor of the rows' type")
         if t.stride(-1) != 1:
             raise ValueError(f"{nm} needs unit stride on the last axis")
     B, Rk = pk.shape

@@ -56,8 +56,9 @@ int fsvd_set_workspace(void* ws, size_t bytes, void* stream);
  * FSVD_BF16 or FSVD_FP16: every tensor of a call is of that type ("bf16" in the formulas stands for it), sums are
  * fp32, roundings are to nearest even at the same points in both.  The reference picks the type from its inputs the
  * same way (kernels/attn/decode/densekv_reconstruct_triton.py:427-428; fp16 is the default of its dense cache,
- * runtime/cache/attn_dense_kv.py:26, and the fallback of scripts/demo_support/api.py:161-165).  The int4 entries and the
- * persistent decode step are bf16 only. */
+ * runtime/cache/attn_dense_kv.py:26, and the fallback of scripts/demo_support/api.py:161-165).  So does the rank-space
+ * decode attention (fsvd_attn_decode_rankkv; fsvd_rankkv_append copies 16-bit patterns of either type).  The int4 entries
+ * and the persistent decode step are bf16 only. */
 
 /* y[b,n] = (res[b,n] +) bf16( W[n,:] . norm(x[b,:]) (+ bias[n]) ),  W is an nn.Linear weight [N,K].
  * norm_w != NULL fuses the RMSNorm of x (w * bf16(x * rsqrt(mean(x^2)+eps))) in front.
@@ -232,7 +233,7 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,
                             float* ws_m, float* ws_l, float* ws_acc,
                             void* out, int64_t so_b, int64_t so_h,
                             int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit, float scale,
-                            float* scores, size_t scores_bytes, void* stream);
+                            float* scores, size_t scores_bytes, int dtype, void* stream);
 
 /* One decoded token per batch row into a rank-space cache: pk_cache[b, positions[b], :] = pk[b, :] and the same for pv
  * (FlashSVDLegacySparseKVCache.update with one position per row, runtime/cache/attn_legacy_sparse_kv.py:113-169: two

@@ -212,6 +212,87 @@ def test_7b_width_layer_teacher_forced_in_float16():
     close(gc.value_cache[0][:, :T + 1], oc.v[0][:, :T + 1], "V cache")
 
 
+def _lin_layout(V):   # [heads,R,Dh] -> nn.Linear weight [heads*Dh, R]
+    h, r, d = V.shape
+    return V.transpose(1, 2).reshape(h * d, r).contiguous()
+
+
+# the one-kernel form (short caches, 1 / 2 / 4 query heads per kv head, deep and plain) and the three-launch form
+# (2^17 (head, key) pairs and more: pair, grouped and single-head score kernels)
+@pytest.mark.parametrize("B,H,Hk,L,S,Rk,Rv,nsplit", [(1, 32, 32, 512, 560, 1024, 1024, None), (2, 8, 2, 100, 128, 72, 40, 3),
+                                                    (2, 16, 4, 333, 400, 1664, 1664, 4), (2, 8, 4, 700, 720, 136, 264, 2),
+                                                    (4, 32, 32, 8200, 8200, 192, 200, 2), (4, 32, 8, 8200, 8200, 128, 64, 3), (12, 3, 3, 4000, 4000, 64, 64, 2)])
+def test_rank_space_decode_attention(B, H, Hk, L, S, Rk, Rv, nsplit):
+    from flashsvd_amd.kernels import rank_decode as RD
+    Dh = 128
+    cos, sin = O.rope_tables(S, Dh, dtype=FP16)
+    q = rand_fp16(B, H, Dh, seed=1)
+    Pk, Pv = rand_fp16(B, S, Rk, seed=2), rand_fp16(B, S, Rv, seed=3)
+    Vk, Vv = rand_fp16(Hk, Rk, Dh, std=Rk ** -0.5, seed=4), rand_fp16(Hk, Rv, Dh, std=Rv ** -0.5, seed=5)
+    lens = torch.tensor([max(1, min(L, S) - 17 * b) for b in range(B)], dtype=torch.int32)
+    out = RD.rank_decode(q.cuda(), Pk.cuda(), Pv.cuda(), _lin_layout(Vk).cuda(), _lin_layout(Vv).cuda(), cos.cuda(), sin.cuda(),
+                         lens.cuda(), num_kv_heads=Hk, nsplit=nsplit)
+    for b in (0, B - 1):
+        n = int(lens[b])
+        close(out[b:b + 1], O.rank_decode_attn(q[b:b + 1], Pk[b:b + 1, :n], Pv[b:b + 1, :n], Vk, Vv, cos[:n], sin[:n]), f"b={b} n={n}")
+
+
+def test_model_rank_cache_greedy_in_float16():
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.runtime.cache import FlashSVDLegacySparseKVCache
+    mw = O.make_model(d=256, n_heads=2, n_kv_heads=2, head_dim=128, ffn=512, attn_rank=64, mlp_rank=96, n_layers=2,
+                      vocab=500, dtype=FP16, seed=5, std=0.05)
+    prompt = torch.randint(0, 500, (1, 21), generator=torch.Generator().manual_seed(4))
+    n_new = 8
+    ref_tok, ref_hid, ref_cache = O.greedy_decode(mw, prompt, n_new, "rank", return_hidden=True)
+    model = model_from_oracle(mw)
+    cache = FlashSVDLegacySparseKVCache(model.config, max_batch_size=1, max_cache_len=40, device="cuda", dtype=FP16)
+    out = model(prompt.cuda(), past_key_values=cache, cache_position=torch.arange(21))
+    close(cache.key_cache[0][:, :21], ref_cache.pk[0][:, :21], "Pk cache layer 0")
+    # the rank path rounds at other points than the oracle's (fp32 K rebuild, V applied in rank space): hidden states
+    # are held to three times the float16 bar, tokens are teacher-forced
+    assert_close_bf16(out.hidden_states[:, -1], ref_hid[:, 0], "prefill hidden", abs_tol=1.5e-2, rel_tol=7.5e-3)
+    same = int(torch.equal(out.logits[:, -1].float().argmax(-1, keepdim=True).cpu(), ref_tok[:, :1]))
+    dec = GraphedDecoder(model, cache, 1)
+    dec.set_state(ref_tok[:, :1].cuda(), 21)
+    for s in range(1, n_new):
+        nxt = dec.eager_step().clone().cpu()
+        assert_close_bf16(dec.hidden, ref_hid[:, s], f"hidden step {s}", abs_tol=1.5e-2, rel_tol=7.5e-3)
+        same += int(torch.equal(nxt, ref_tok[:, s:s + 1]))
+        dec.tokens.copy_(ref_tok[:, s:s + 1])
+    assert same >= n_new - 1, f"only {same}/{n_new} teacher-forced tokens identical"
+
+
+def test_generate_text_after_the_float16_cast():
+    """The reference's own sequence: cast_model_for_inference(dtype="fp16"), then generate_text (scripts/demo_support/api.py:128-165,
+    238-322); the decode driver hands a float16 model to the per-operator engine."""
+    from flashsvd_amd import api
+
+    class Tok:
+        pad_token_id, eos_token_id, eos_token, pad_token = 0, None, "<eos>", "<pad>"
+
+        def __call__(self, text, return_tensors="pt", add_special_tokens=False):
+            return {"input_ids": torch.tensor([[1, 5, 7, 11, 13]], dtype=torch.long)}
+
+        def decode(self, ids, skip_special_tokens=False):
+            return " ".join(str(int(i)) for i in ids)
+
+    mw32, _ = O.config_c1(torch.float32)
+    mw16 = O.hold_weights_as(mw32, FP16)
+    mw16.embed, mw16.norm = mw32.embed.to(FP16), mw32.norm.to(FP16)
+    for b16, b32 in zip(mw16.blocks, mw32.blocks):
+        b16.ln1, b16.ln2 = b32.ln1.to(FP16), b32.ln2.to(FP16)
+    ref = O.greedy_decode(mw16, torch.tensor([[1, 5, 7, 11, 13]]), 6)
+    model = api.cast_model_for_inference(model_from_oracle(mw32), dtype="fp16", device="cuda")
+    assert next(model.parameters()).dtype == FP16
+    api.configure_runtime("flashsvd")
+    for graph in (False, True):
+        res = api.generate_text(model, Tok(), prompt="x", max_new_tokens=6, device="cuda", use_graph=graph)
+        assert res["completion_ids"] == ref[0].tolist()
+    out = api.decode_kvcache_eval(model, prompt_len=16, new_tokens=4, warmup=2, batch_size=2)
+    assert out["new_tokens"] == 4 and out["decode_tok_s"] > 0 and out["flashsvd_dense_cache"]
+
+
 def test_persistent_step_refuses_float16():
     from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
     from flashsvd_amd.step import PersistentDecoder

@@ -245,7 +245,7 @@ def test_rank_decode_rejects_unsupported(RD):
         RD.rank_decode(c(1, 2, 64), c(1, 8, 16), c(1, 8, 16), c(128, 16), c(128, 16), None, None, lens, num_kv_heads=2)
     with pytest.raises(FlashSVDHipError, match="multiples of 8"):
         RD.rank_decode(c(1, 2, 128), c(1, 8, 12), c(1, 8, 12), c(256, 12), c(256, 12), None, None, lens, num_kv_heads=2)
-    with pytest.raises(ValueError, match="bfloat16 only"):
+    with pytest.raises(ValueError, match="bfloat16 or float16"):
         RD.rank_decode(c(1, 2, 128).float(), c(1, 8, 16), c(1, 8, 16), c(256, 16), c(256, 16), None, None, lens, num_kv_heads=2)
 
 
