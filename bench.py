@@ -65,8 +65,7 @@ def _parse():
                     help="the same model with every factor quantised to group-wise int4 (group 128): decode tok/s of both engines "
                          "and the bytes that cross HBM per token, as its own JSON line")
     ap.add_argument("--fp16", action="store_true",
-                    help="the same model held in float16 through the per-operator engine (the resident step is bf16 only): "
-                         "warm prompt pass and decode tok/s")
+                    help="the same model held in float16: warm prompt pass and decode tok/s of both engines")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB device copy 10 times (the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counters are scaled against) and exit")
@@ -361,8 +360,6 @@ def run_lowrank(args, dtype=None):
         torch.cuda.synchronize()
         t_decode = time.perf_counter() - t1
         res["graph"] = dict(tok_s=B * args.steps / t_decode, ms_per_step=t_decode * 1000.0 / args.steps)
-    if dtype != torch.bfloat16:
-        return res
     if args.engine in ("persistent", "both"):
         from flashsvd_amd.step import PersistentDecoder
         cache._seen_tokens = PROMPT_LEN
@@ -392,7 +389,7 @@ def run_lowrank(args, dtype=None):
             # the same step with the rank projections folded into the u-factor phases (PersistentDecoder(composed=True)):
             # eight hand-offs per layer instead of ten, 6 % more bytes; reported beside the default form, never as the headline
             # value (its rank coefficients come from unrounded sums: closer to exact arithmetic, but not the reference's roundings)
-            scratch_c = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=torch.bfloat16)
+            scratch_c = FlashSVDV15DenseKVCache(model.config, max_batch_size=B, max_cache_len=max_len, device="cuda", dtype=dtype)
             model(prompt, past_key_values=scratch_c, cache_position=torch.arange(PROMPT_LEN), logits_to_keep=1)
             cdec = PersistentDecoder(model, scratch_c, composed=True)
             cdec.set_state(tok, PROMPT_LEN)
@@ -413,6 +410,8 @@ def run_lowrank(args, dtype=None):
             del cdec, scratch_c
     best = res.get("persistent") or res["graph"]
     res["tok_s"], res["ms_per_step"] = best["tok_s"], best["ms_per_step"]
+    if dtype != torch.bfloat16:
+        return res
     if not args.no_kernel_configs:
         res["kernel_configs"] = kernel_configs(model, cache, dec, args.layers)
     legs = kernel_legs(model, cache, dec)
@@ -921,11 +920,14 @@ def main():
                           "model_pass": mp, "kernels": kern}))
         return
     if args.fp16:
-        args.engine = "graph"
         lr = run_lowrank(args, torch.float16)
-        print(json.dumps({"metric": "decode tok/s, 7B-shape rank-0.5 bs1, float16, per-operator HIP graph", "value": lr["graph"]["tok_s"],
-                          "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": lr["graph"]["ms_per_step"],
-                          "dtype": "fp16", "data": "synthetic", "prefill": lr["prefill"]}))
+        line = {"metric": "decode tok/s, 7B-shape rank-0.5 bs1, float16", "value": lr["tok_s"], "unit": "tok/s", "n_gpus": 1,
+                "steps": args.steps, "warmup": args.warmup, "ms_per_step": lr["ms_per_step"], "dtype": "fp16", "data": "synthetic",
+                "prefill": lr["prefill"]}
+        for k in ("persistent", "persistent_composed", "graph"):
+            if k in lr:
+                line[k if k != "graph" else "per_operator_graph"] = {m: v for m, v in lr[k].items() if m != "phase_profile_us"}
+        print(json.dumps(line))
         return
     lr = run_lowrank(args)
     if args.kernel_configs_only:

@@ -89,6 +89,7 @@ class StepState(ctypes.Structure):
 PH_EMBED, PH_GEMV, _PH_RESERVED, PH_ATTN, PH_MERGE, PH_ARGMAX = range(6)
 EP_STORE, EP_RESID, EP_SWIGLU, EP_LOGITS, EP_F32 = range(5)
 PF_NOWAIT, PF_STAGE2, PF_SPLIT, PF_LEAD = 1, 2, 4, 8
+WBITS_FP16 = -16
 
 # name -> (restype, argtypes); mirrors include/flashsvd_hip.h declaration by declaration
 SIGNATURES = {

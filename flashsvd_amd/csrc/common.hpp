@@ -78,8 +78,15 @@ template <> struct E16<1> {
   static constexpr int code = 1;
   typedef f16x8_t frag_t;
   static __device__ __forceinline__ f32x4_t mfma(frag_t a, frag_t b, f32x4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
-  static __device__ __forceinline__ float val(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (unsigned short)h); }
-  static __device__ __forceinline__ float lo(uint32_t packed) { return val(packed & 0xffffu); }
+  // V_CVT_F32_F16 on the low half of a 32-bit register, written as an instruction: left to the compiler, the widening is
+  // folded into mixed-precision multiply-adds on 16-bit subregisters, which makes it copy whole register arrays whenever
+  // one element of them is rewritten (the step kernel's staging went from 150 registers to 256 with 780 spills)
+  static __device__ __forceinline__ float val(uint32_t h) {
+    float f;
+    asm("v_cvt_f32_f16 %0, %1" : "=v"(f) : "v"(h));
+    return f;
+  }
+  static __device__ __forceinline__ float lo(uint32_t packed) { return val(packed); }               // the instruction reads the low half
   static __device__ __forceinline__ float hi(uint32_t packed) { return val(packed >> 16); }
   static __device__ __forceinline__ uint32_t bits(float f) {
     return static_cast<uint32_t>(__builtin_bit_cast(unsigned short, static_cast<_Float16>(f)));

@@ -180,7 +180,7 @@ __device__ __forceinline__ void gemv_sz_table_addr(const GemvCtx& c, uint64_t (&
 // steps ahead (clamped to the last piece past the end, whose product is dropped).
 // GROUPED: the rows form three groups with their own inputs (q, k, v head expansion from [Pq | Pk | Pv]):
 // a row at or past g1 / g2 reads the second / third K-long part of the staged vector.
-template <int NMAT, bool GROUPED>
+template <class E, int NMAT, bool GROUPED>
 __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int g1, int g2, u32x4_t (&R)[kU], const uint16_t* xs,
                                             float* cp) {
   constexpr int SPB = kU / NMAT;                // steps per batch
@@ -205,7 +205,7 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
       int xo = mat * c.xk + kofs * 8;
       if (GROUPED) xo += ((row >= g1 ? 1 : 0) + (row >= g2 ? 1 : 0)) * c.K;
       const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xs + xo);
-      d[u] = dot8_bf16(R[u], xv, 0.f);
+      d[u] = E::dot8(R[u], xv, 0.f);
       if (REFILL) {
         const uint32_t in = min((uint32_t)((s0 + u / NMAT + SPB) * kT) + tid, last);
         R[u] = ld_stream(mat ? c.base1 : c.base0, in << 4);
@@ -236,6 +236,7 @@ __device__ __forceinline__ void gemv_stream(const GemvCtx& c, uint32_t m_kp, int
 // sums stay in the partial buffer, the window request at the end of the iteration fetches the first pieces of the phase
 // behind it, and that phase - which polls for its input only now, when the producers have long published - puts its own
 // partial sums behind these and publishes both.  Every step is full and the steps are a multiple of kU (host-checked).
+template <class E>
 __device__ __forceinline__ void lead_stream(const GemvCtx& a, uint32_t m_kp, u32x4_t (&R)[kU], const uint16_t* xs, float* cp) {
   const uint32_t tid = threadIdx.x;
   const int nA = a.nsteps;
@@ -250,7 +251,7 @@ __device__ __forceinline__ void lead_stream(const GemvCtx& a, uint32_t m_kp, u32
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
       const u32x4_t xv = *reinterpret_cast<const u32x4_t*>(xs + kofs * 8);
-      d[u] = dot8_bf16(R[u], xv, 0.f);
+      d[u] = E::dot8(R[u], xv, 0.f);
       if (REFILL) R[u] = ld_stream(a.base0, ((uint32_t)((s0 + u + kU) * kT) + tid) << 4);
       d[u] = row16_sum(d[u]);
       kofs += a.dk;
@@ -413,7 +414,7 @@ __device__ __forceinline__ void ld_coh128_round(u32x4_t (&v)[8], const uint64_t 
                : "memory");
 }
 #undef FSVD_LDC
-template <int NS>
+template <class E, int NS>
 __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uint32_t tin, const uint32_t* norm_w, float eps,
                                                  const fsvd_step_state* st, int limit, uint16_t* xs, float* red, bool q4, float* xsum) {
   static_assert(NS == 2 || NS == 8, "ld_coh128_round exists for rounds of 2 and of 8 loads");
@@ -456,7 +457,7 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
       if (q < nw128) {
         const uint32_t a0 = v[j].x & 0xffffu, a1 = v[j].y & 0xffffu, a2 = v[j].z & 0xffffu, a3 = v[j].w & 0xffffu;
         if (norm) {
-          const float f0 = bf16_bits_to_f32(a0), f1 = bf16_bits_to_f32(a1), f2 = bf16_bits_to_f32(a2), f3 = bf16_bits_to_f32(a3);
+          const float f0 = E::val(a0), f1 = E::val(a1), f2 = E::val(a2), f3 = E::val(a3);
           ss += (f0 * f0 + f1 * f1) + (f2 * f2 + f3 * f3);
           v[j].x = a0 | (a1 << 16);       // raw values; scaled once the sum is known
           v[j].y = a2 | (a3 << 16);
@@ -478,9 +479,9 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
         if (base + j * kT >= nw128) break;
         const int q = base + j * kT + tid;
         if (q < nw128) {
-          const float f0 = bf16_lo(v[j].x), f1 = bf16_hi(v[j].x), f2 = bf16_lo(v[j].y), f3 = bf16_hi(v[j].y);
-          stage_store_wide(xs, xsum, q, pack_bf16x2(bf16_lo(nwt[j].x) * round_bf16(f0 * rs), bf16_hi(nwt[j].x) * round_bf16(f1 * rs)),
-                           pack_bf16x2(bf16_lo(nwt[j].y) * round_bf16(f2 * rs), bf16_hi(nwt[j].y) * round_bf16(f3 * rs)), q4);
+          const float f0 = E::lo(v[j].x), f1 = E::hi(v[j].x), f2 = E::lo(v[j].y), f3 = E::hi(v[j].y);
+          stage_store_wide(xs, xsum, q, E::pack2(E::lo(nwt[j].x) * E::rnd(f0 * rs), E::hi(nwt[j].x) * E::rnd(f1 * rs)),
+                           E::pack2(E::lo(nwt[j].y) * E::rnd(f2 * rs), E::hi(nwt[j].y) * E::rnd(f3 * rs)), q4);
         }
       }
     }
@@ -493,7 +494,7 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
 // state itself.  One round of loads brings both; b goes to LDS as it is (at boff, for a phase that follows without a
 // hand-off) and gives rs = rsqrt(mean(b^2) + eps); a goes to LDS as bf16(a * rs) at 0: the RMSNorm of the hidden state
 // applied as a scalar behind the product (its weight vector is folded into the matrix).
-template <int NS>
+template <class E, int NS>
 __device__ __forceinline__ bool stage_pair(const void* a, int na, uint32_t ta, const void* b, int nb, uint32_t tb, int boff, float eps,
                                            const fsvd_step_state* st, int limit, uint16_t* xs, float* red) {
   const int tid = threadIdx.x;
@@ -532,7 +533,7 @@ __device__ __forceinline__ bool stage_pair(const void* a, int na, uint32_t ta, c
     const int q = (j - sa) * kT + tid;
     if (j >= sa && q < npb) {
       const uint32_t a0 = v[j].x & 0xffffu, a1 = v[j].y & 0xffffu, a2 = v[j].z & 0xffffu, a3 = v[j].w & 0xffffu;
-      const float f0 = bf16_bits_to_f32(a0), f1 = bf16_bits_to_f32(a1), f2 = bf16_bits_to_f32(a2), f3 = bf16_bits_to_f32(a3);
+      const float f0 = E::val(a0), f1 = E::val(a1), f2 = E::val(a2), f3 = E::val(a3);
       ss += (f0 * f0 + f1 * f1) + (f2 * f2 + f3 * f3);
       xb[q] = make_uint2(a0 | (a1 << 16), a2 | (a3 << 16));
     }
@@ -548,7 +549,7 @@ __device__ __forceinline__ bool stage_pair(const void* a, int na, uint32_t ta, c
 #pragma unroll
   for (int j = 0; j < NS; ++j) {
     const int q = j * kT + tid;
-    if (j < sa && q < npa) xa[q] = pack_bf16x2(__uint_as_float(v[j].x) * rs, __uint_as_float(v[j].z) * rs);
+    if (j < sa && q < npa) xa[q] = E::pack2(__uint_as_float(v[j].x) * rs, __uint_as_float(v[j].z) * rs);
   }
   return !fail;
 }
@@ -597,14 +598,15 @@ __device__ __forceinline__ void attn_issue(const AttnWork& a, int c0, u32x4_t (&
 #pragma unroll
   for (int u = 0; u < kU; ++u) R[u] = ld_stream(addr[u], 0);
 }
+template <class E>
 __device__ __forceinline__ void softmax_step(float sc, const u32x4_t& v, float& m, float& l, float (&acc)[8]) {
   const float m_new = fmaxf(m, sc);
   const float alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
   const float p = __expf(sc - m_new);
-  acc[0] = acc[0] * alpha + p * bf16_lo(v.x); acc[1] = acc[1] * alpha + p * bf16_hi(v.x);
-  acc[2] = acc[2] * alpha + p * bf16_lo(v.y); acc[3] = acc[3] * alpha + p * bf16_hi(v.y);
-  acc[4] = acc[4] * alpha + p * bf16_lo(v.z); acc[5] = acc[5] * alpha + p * bf16_hi(v.z);
-  acc[6] = acc[6] * alpha + p * bf16_lo(v.w); acc[7] = acc[7] * alpha + p * bf16_hi(v.w);
+  acc[0] = acc[0] * alpha + p * E::lo(v.x); acc[1] = acc[1] * alpha + p * E::hi(v.x);
+  acc[2] = acc[2] * alpha + p * E::lo(v.y); acc[3] = acc[3] * alpha + p * E::hi(v.y);
+  acc[4] = acc[4] * alpha + p * E::lo(v.z); acc[5] = acc[5] * alpha + p * E::hi(v.z);
+  acc[6] = acc[6] * alpha + p * E::lo(v.w); acc[7] = acc[7] * alpha + p * E::hi(v.w);
   l = l * alpha + p;
   m = m_new;
 }
@@ -643,9 +645,10 @@ __device__ __forceinline__ void raise_error(fsvd_step_state* st, int p, int w) {
 // [0] phase entered, [1] input staged, [2] weights consumed, [3] epilogue done
 // Q4: the list may hold int4 GEMV phases (wbits == 4); the build without them keeps the bf16 walk free of their code
 // CX: the list may hold the phases of the composed form (FSVD_PF_* flags, fp32 rows); likewise a build of its own
-template <bool TRACE, bool Q4, bool CX>
+template <bool TRACE, bool Q4, bool CX, int DT>
 __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __restrict__ phases, int nph, fsvd_step_state* st,
                                                          unsigned long long* trace, int trace_stride) {
+  typedef E16<DT> E;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw);
   float* cp = reinterpret_cast<float*>(smem_raw + (size_t)kMaxIn * 2);
@@ -696,7 +699,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       // the epilogue of the previous phase may still be reading the partial buffer in another wave (its LDS reads are
       // complete by the time that wave's stores have been issued, i.e. before it arrives here)
       __builtin_amdgcn_s_barrier();
-      lead_stream(gc, desc_u32(dv, FSVD_DW(m_kp)), R, xs + gc.xoff, cp);
+      lead_stream<E>(gc, desc_u32(dv, FSVD_DW(m_kp)), R, xs + gc.xoff, cp);
       lead_chunks = gc.pps >> 4;
       dvL = dv;
       if (TRACE && tr) tr[1] = tr[0];      // nothing staged
@@ -727,15 +730,15 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         const int n2 = DF_I(dv, in2_len);
         const int slots = ((in_len >> 1) + kT - 1) / kT + ((n2 >> 2) + kT - 1) / kT;
         if (slots <= 5)
-          ok = stage_pair<5>(inp, in_len, DF_TAG32(dv, in, epoch), DF_P(dv, in2), n2, DF_TAG16(dv, in2, epoch), DF_I(dv, in2_off),
+          ok = stage_pair<E, 5>(inp, in_len, DF_TAG32(dv, in, epoch), DF_P(dv, in2), n2, DF_TAG16(dv, in2, epoch), DF_I(dv, in2_off),
                              DF_F(dv, fparam), st, limit, xs, red);
         else
-          ok = stage_pair<8>(inp, in_len, DF_TAG32(dv, in, epoch), DF_P(dv, in2), n2, DF_TAG16(dv, in2, epoch), DF_I(dv, in2_off),
+          ok = stage_pair<E, 8>(inp, in_len, DF_TAG32(dv, in, epoch), DF_P(dv, in2), n2, DF_TAG16(dv, in2, epoch), DF_I(dv, in2_off),
                              DF_F(dv, fparam), st, limit, xs, red);
       } else if (in_len <= 2 * kT * 4) {
-        ok = stage_input_wide<2>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+        ok = stage_input_wide<E, 2>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
       } else {
-        ok = stage_input_wide<8>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
+        ok = stage_input_wide<E, 8>(inp, in_len, tin, nw, DF_F(dv, fparam), st, limit, xs, red, Q4 && gc.q4, xsum);
       }
       // Every load of the staging code has been consumed by now (and the window, requested before the polls, has landed
       // with them: loads complete in order).  The compiler's bookkeeping cannot see that for loads issued under a
@@ -770,11 +773,11 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         }
       } else if (gH > 0) {
         const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
-        gemv_stream<1, true>(gc, m_kp, g1, g2, R, xs + (CX ? gc.xoff : 0), cp);
+        gemv_stream<E, 1, true>(gc, m_kp, g1, g2, R, xs + (CX ? gc.xoff : 0), cp);
       } else if (gc.nmat == 1) {
-        gemv_stream<1, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cpm);
+        gemv_stream<E, 1, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cpm);
       } else {
-        gemv_stream<2, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cp);
+        gemv_stream<E, 2, false>(gc, m_kp, 0, 0, R, xs + (CX ? gc.xoff : 0), cp);
       }
       __syncthreads();
     } else if (type == FSVD_PH_ATTN) {
@@ -795,8 +798,8 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         float c = 1.f, sn = 0.f;
         if (role != 2 && cosT) {
           const int tp = min(max(pos, 0), DF_I(dv, rope_len) - 1);
-          c = bf16_bits_to_f32(cosT[(int64_t)tp * half + dd]);
-          sn = bf16_bits_to_f32(sinT[(int64_t)tp * half + dd]);
+          c = E::val(cosT[(int64_t)tp * half + dd]);
+          sn = E::val(sinT[(int64_t)tp * half + dd]);
         }
         // the two halves of a rotation pair in one trip through memory: both loads, then both tags
         uint32_t b0, b1;
@@ -807,14 +810,14 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           if ((v0 >> 16) == tq && (v1 >> 16) == tq) break;
           if (++spins > limit || ((spins & 1023) == 0 && ld_err(st) != 0)) { fail = true; break; }
         }
-        float x0 = bf16_bits_to_f32(b0), x1 = bf16_bits_to_f32(b1);
+        float x0 = E::val(b0), x1 = E::val(b1);
         if (role != 2 && cosT) {
           // eager bf16 arithmetic: one rounding per multiply and per add
-          const float r0 = round_bf16(round_bf16(x0 * c) - round_bf16(x1 * sn));
-          const float r1 = round_bf16(round_bf16(x1 * c) + round_bf16(x0 * sn));
+          const float r0 = E::rnd(E::rnd(x0 * c) - E::rnd(x1 * sn));
+          const float r1 = E::rnd(E::rnd(x1 * c) + E::rnd(x0 * sn));
           x0 = r0; x1 = r1;
         }
-        const uint16_t o0 = (uint16_t)f32_to_bf16_bits(x0), o1 = (uint16_t)f32_to_bf16_bits(x1);
+        const uint16_t o0 = (uint16_t)E::bits(x0), o1 = (uint16_t)E::bits(x1);
         xs[role * Dh + dd] = o0;
         xs[role * Dh + dd + half] = o1;
         if (role != 0 && aw.h == aw.hk * (aw.H / aw.Hk) && pos >= 0 && pos < DF_I(dv, S)) {
@@ -837,15 +840,15 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         if (c0 != aw.k0) attn_issue(aw, c0, R);
 #pragma unroll
         for (int u = 0; u < kUA; ++u) {
-          const float sc = row16_sum(dot8_bf16(R[u], qv, 0.f)) * scale;
-          if (c0 + u * kSlots + slot < aw.k1) softmax_step(sc, R[kUA + u], m_run, l_run, acc);
+          const float sc = row16_sum(E::dot8(R[u], qv, 0.f)) * scale;
+          if (c0 + u * kSlots + slot < aw.k1) softmax_step<E>(sc, R[kUA + u], m_run, l_run, acc);
         }
       }
       if (aw.newtok && slot == 0) {
         const u32x4_t kn = *reinterpret_cast<const u32x4_t*>(xs + Dh + part * 8);
         const u32x4_t vn = *reinterpret_cast<const u32x4_t*>(xs + 2 * Dh + part * 8);
-        const float sc = row16_sum(dot8_bf16(kn, qv, 0.f)) * scale;
-        softmax_step(sc, vn, m_run, l_run, acc);
+        const float sc = row16_sum(E::dot8(kn, qv, 0.f)) * scale;
+        softmax_step<E>(sc, vn, m_run, l_run, acc);
       }
       // park the key slots: cp[slot][Dh + 2]
       float* sl = cp + slot * (Dh + 2);
@@ -871,9 +874,9 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         uint16_t* logits = static_cast<uint16_t*>(DF_P(dv, plain_out));
         for (int ps = 0; ps < npass; ++ps) {
           const int t = min(ps * (kT / 8) + grp, gc.srows - 1);
-          const float v = round_bf16(row_sum8(cp, t, cpr));
+          const float v = E::rnd(row_sum8(cp, t, cpr));
           if (lead8 && ps * (kT / 8) + grp < gc.srows) {
-            logits[gc.r0 + t] = (uint16_t)f32_to_bf16_bits(v);
+            logits[gc.r0 + t] = (uint16_t)E::bits(v);
             if (v > best) { best = v; best_i = gc.r0 + t; }
           }
         }
@@ -889,7 +892,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         if (tid == 0) {
           for (int i = 1; i < kT / 64; ++i)
             if (red[i] > best || (red[i] == best && ired[i] < best_i)) { best = red[i]; best_i = ired[i]; }
-          const uint64_t word = ((uint64_t)((tout << 16) | f32_to_bf16_bits(best)) << 32) | (uint32_t)best_i;
+          const uint64_t word = ((uint64_t)((tout << 16) | E::bits(best)) << 32) | (uint32_t)best_i;
           __hip_atomic_store(static_cast<uint64_t*>(out) + w, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __syncthreads();   // `red` is reused by the argmax phase
@@ -907,17 +910,17 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           if (epi == FSVD_EP_SWIGLU) {
             float gv = row_sum8(cp, t, cpr), uv = row_sum8(cp, gc.srows + t, cpr);
             if (mode == 0) {
-              gv = round_bf16(gv);
-              uv = round_bf16(uv);
-              v = round_bf16(round_bf16(silu_f32(gv)) * uv);
+              gv = E::rnd(gv);
+              uv = E::rnd(uv);
+              v = E::rnd(E::rnd(silu_f32(gv)) * uv);
             } else {
-              v = round_bf16((gv * (1.0f / (1.0f + expf(-gv)))) * uv);
+              v = E::rnd((gv * (1.0f / (1.0f + expf(-gv)))) * uv);
             }
           } else {
-            v = round_bf16(row_sum8(cpm, t, cpr));
-            if (epi == FSVD_EP_RESID) v = round_bf16(bf16_bits_to_f32(resid & 0xffffu) + v);
+            v = E::rnd(row_sum8(cpm, t, cpr));
+            if (epi == FSVD_EP_RESID) v = E::rnd(E::val(resid & 0xffffu) + v);
           }
-          if (live) st_tag16(out, gc.r0 + t, tout, f32_to_bf16_bits(v));
+          if (live) st_tag16(out, gc.r0 + t, tout, E::bits(v));
         }
       }
       if (CX && lead_chunks != 0) {
@@ -1011,7 +1014,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           num += wi * cp[sp * per + tid];
           den += wi * cp[sp * per + cnt + 1];
         }
-        st_tag16(DF_P(dv, out0), o0 + tid, tout, f32_to_bf16_bits(den > 0.f ? num / den : 0.f));
+        st_tag16(DF_P(dv, out0), o0 + tid, tout, E::bits(den > 0.f ? num / den : 0.f));
       }
     } else if (type == FSVD_PH_ARGMAX) {
       // greedy token, state advance
@@ -1026,7 +1029,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
           for (;;) {
             const uint64_t v = ld_coh64(in, t);
             if ((uint32_t)(v >> 48) == tin) {
-              const float val = bf16_bits_to_f32((uint32_t)(v >> 32) & 0xffffu);
+              const float val = E::val((uint32_t)(v >> 32) & 0xffffu);
               const int idx = (int)(uint32_t)v;
               if (val > best || (val == best && idx < best_i)) { best = val; best_i = idx; }
               break;
@@ -1087,9 +1090,11 @@ int decode_step_workgroups() {
     set_last_error("fsvd_decode_step: cannot query the device");
     return 0;
   }
-  const void* fns[6] = {reinterpret_cast<const void*>(decode_step_kernel<false, false, false>), reinterpret_cast<const void*>(decode_step_kernel<true, false, false>),
-                        reinterpret_cast<const void*>(decode_step_kernel<false, true, false>), reinterpret_cast<const void*>(decode_step_kernel<true, true, false>),
-                        reinterpret_cast<const void*>(decode_step_kernel<false, false, true>), reinterpret_cast<const void*>(decode_step_kernel<true, false, true>)};
+  const void* fns[10] = {reinterpret_cast<const void*>(decode_step_kernel<false, false, false, 0>), reinterpret_cast<const void*>(decode_step_kernel<true, false, false, 0>),
+                         reinterpret_cast<const void*>(decode_step_kernel<false, true, false, 0>), reinterpret_cast<const void*>(decode_step_kernel<true, true, false, 0>),
+                         reinterpret_cast<const void*>(decode_step_kernel<false, false, true, 0>), reinterpret_cast<const void*>(decode_step_kernel<true, false, true, 0>),
+                         reinterpret_cast<const void*>(decode_step_kernel<false, false, false, 1>), reinterpret_cast<const void*>(decode_step_kernel<true, false, false, 1>),
+                         reinterpret_cast<const void*>(decode_step_kernel<false, false, true, 1>), reinterpret_cast<const void*>(decode_step_kernel<true, false, true, 1>)};
   for (const void* fn : fns) {
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSmemBytes) != hipSuccess) {
       set_last_error("fsvd_decode_step: the device refuses %zu bytes of dynamic LDS per workgroup", kSmemBytes);
@@ -1137,13 +1142,17 @@ static int gemv_in_len(const fsvd_phase& d) { return (d.H > 0 ? 3 : (d.shared_in
 int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
   if (nph < 2) return bad("a step needs at least two phases", 0);
   {
-    bool any_q4 = false, any_cx = false;
+    bool any_q4 = false, any_cx = false, any_f16 = false, any_b16 = false;
     for (int p = 0; p < nph; ++p) {
       if (ph[p].type != FSVD_PH_GEMV) continue;
       any_q4 = any_q4 || ph[p].wbits == 4;
+      any_f16 = any_f16 || ph[p].wbits == FSVD_WBITS_FP16;
+      any_b16 = any_b16 || ph[p].wbits == 0 || ph[p].wbits == 16;
       any_cx = any_cx || ph[p].flags != 0 || ph[p].epilogue == FSVD_EP_F32;
     }
     if (any_q4 && any_cx) return bad("a list holds int4 phases or phases of the composed form, not both (they run on different builds of the kernel)", 0);
+    // the element type belongs to the step: its vectors, tables and caches are all of one 16-bit type
+    if (any_f16 && (any_b16 || any_q4)) return bad("a list is float16 in every GEMV phase or in none (int4 phases take bf16 activations)", 0);
   }
 
   // Every tagged buffer with the phase that wrote it last.  `full`: every workgroup wrote part of it in that phase (a
@@ -1189,7 +1198,7 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         break;
       case FSVD_PH_GEMV: {
         if (d.nmat < 1 || d.nmat > 2 || !d.W[0] || (d.nmat == 2 && !d.W[1])) return bad("GEMV needs 1 or 2 matrices", p);
-        if (d.wbits != 0 && d.wbits != 16 && d.wbits != 4) return bad("wbits must be 0 / 16 (bf16) or 4", p);
+        if (d.wbits != 0 && d.wbits != 16 && d.wbits != 4 && d.wbits != FSVD_WBITS_FP16) return bad("wbits must be 0 / 16 (bf16), FSVD_WBITS_FP16 or 4", p);
         const bool q4 = d.wbits == 4;
         if (d.K <= 0 || d.K % (q4 ? 256 : 128) != 0) return bad(q4 ? "K must be a positive multiple of 256 for int4 weights" : "K must be a positive multiple of 128", p);
         if (q4) {
@@ -1382,16 +1391,18 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
 }
 
 // Which build of the kernel a list needs: 0 plain bf16, 1 with the int4 code (~5 % slower on a bf16 list), 2 with the
-// code of the composed form.  A build that meets a phase it was not compiled for raises the step's error flag.
+// code of the composed form; + 4 for a float16 list (plain or composed).  A build that meets a phase it was not compiled
+// for raises the step's error flag.
 int decode_step_build(const fsvd_phase* host, int nph) {
   if (!host) return 0;
-  int build = 0;
+  int build = 0, f16 = 0;
   for (int p = 0; p < nph; ++p) {
     if (host[p].type != FSVD_PH_GEMV) continue;
     if (host[p].wbits == 4) return 1;
+    if (host[p].wbits == FSVD_WBITS_FP16) f16 = 4;
     if (host[p].flags != 0 || host[p].epilogue == FSVD_EP_F32) build = 2;
   }
-  return build;
+  return build + f16;
 }
 
 int launch_decode_step(const fsvd_phase* dev, int nph, fsvd_step_state* st, unsigned long long* trace, int trace_stride, int build,
@@ -1400,15 +1411,19 @@ int launch_decode_step(const fsvd_phase* dev, int nph, fsvd_step_state* st, unsi
   if (nwg <= 0) return kErrLaunch;   // the reason is in the last-error text
   unsigned long long* tp = trace ? trace : nullptr;
   const int ts = trace ? trace_stride : 1;
-#define FSVD_LAUNCH(T, Q, C) hipLaunchKernelGGL((decode_step_kernel<T, Q, C>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, tp, ts)
+#define FSVD_LAUNCH(T, Q, C, D) hipLaunchKernelGGL((decode_step_kernel<T, Q, C, D>), dim3(nwg), dim3(kT), kSmemBytes, stream, dev, nph, st, tp, ts)
   if (trace) {
-    if (build == 1) FSVD_LAUNCH(true, true, false);
-    else if (build == 2) FSVD_LAUNCH(true, false, true);
-    else FSVD_LAUNCH(true, false, false);
+    if (build == 1) FSVD_LAUNCH(true, true, false, 0);
+    else if (build == 2) FSVD_LAUNCH(true, false, true, 0);
+    else if (build == 4) FSVD_LAUNCH(true, false, false, 1);
+    else if (build == 6) FSVD_LAUNCH(true, false, true, 1);
+    else FSVD_LAUNCH(true, false, false, 0);
   } else {
-    if (build == 1) FSVD_LAUNCH(false, true, false);
-    else if (build == 2) FSVD_LAUNCH(false, false, true);
-    else FSVD_LAUNCH(false, false, false);
+    if (build == 1) FSVD_LAUNCH(false, true, false, 0);
+    else if (build == 2) FSVD_LAUNCH(false, false, true, 0);
+    else if (build == 4) FSVD_LAUNCH(false, false, false, 1);
+    else if (build == 6) FSVD_LAUNCH(false, false, true, 1);
+    else FSVD_LAUNCH(false, false, false, 0);
   }
 #undef FSVD_LAUNCH
   hipError_t e = hipGetLastError();

@@ -64,20 +64,23 @@ class PersistentDecoder:
         inner = model.model
         cfg = model.config
         dev = model.lm_head.weight.device
-        if model.lm_head.weight.dtype != torch.bfloat16:
-            raise ValueError("PersistentDecoder is bf16 only")
-        # the kernel reinterprets every buffer it is pointed at as bf16 bits (int4 factors aside): refuse anything else
-        # here, so that the driver falls back to the per-operator engine instead of decoding garbage
-        if getattr(cache, "_dtype", torch.bfloat16) != torch.bfloat16:
-            raise ValueError(f"PersistentDecoder needs a bfloat16 KV cache, got {cache._dtype} "
-                             "(FlashSVDV15DenseKVCache defaults to float16: pass dtype=torch.bfloat16)")
-        if inner.embed_tokens.weight.dtype != torch.bfloat16 or inner.norm.weight.dtype != torch.bfloat16:
-            raise ValueError("PersistentDecoder needs a bfloat16 embedding table and final norm")
+        # one 16-bit element type for the whole step, named by the lm_head: bfloat16, or float16 (a model without int4
+        # factors).  The kernel reinterprets every buffer it is pointed at as bits of that type (int4 factors aside):
+        # anything else is refused here, so that the driver falls back to the per-operator engine instead of decoding garbage
+        edt = model.lm_head.weight.dtype
+        if edt not in (torch.bfloat16, torch.float16):
+            raise ValueError(f"PersistentDecoder computes in bfloat16 or float16, the model is {edt}")
+        self.dtype = edt
+        if getattr(cache, "_dtype", edt) != edt:
+            raise ValueError(f"PersistentDecoder needs a KV cache of the model's type {edt}, got {cache._dtype} "
+                             f"(FlashSVDV15DenseKVCache defaults to float16: pass dtype={edt})")
+        if inner.embed_tokens.weight.dtype != edt or inner.norm.weight.dtype != edt:
+            raise ValueError(f"PersistentDecoder needs the embedding table and final norm in the model's type {edt}")
         layers = list(inner.layers) if part == "model" else [inner.layers[layer_index]]
         for li, layer in enumerate(layers):
             for nm, p_ in layer.named_parameters():
-                if p_.is_floating_point() and p_.dtype != torch.bfloat16:
-                    raise ValueError(f"PersistentDecoder needs bfloat16 weights; layer {li} {nm} is {p_.dtype}")
+                if p_.is_floating_point() and p_.dtype != edt:
+                    raise ValueError(f"PersistentDecoder needs weights of one type ({edt}); layer {li} {nm} is {p_.dtype}")
         self.nwg = int(lib.fsvd_decode_step_workgroups())
         if self.nwg <= 0:
             raise RuntimeError((lib.fsvd_last_error() or b"").decode() or "fsvd_decode_step_workgroups: cannot query the device")
@@ -116,6 +119,8 @@ class PersistentDecoder:
                 if gs < m.in_features and (gs < 32 or gs & (gs - 1)):
                     raise ValueError(f"PersistentDecoder: int4 group size {gs} is not a power of two >= 32")
             layer_q4.append(True)
+        if any(layer_q4) and edt != torch.bfloat16:
+            raise ValueError("PersistentDecoder: int4 factors take bfloat16 activations; the model is float16")
         # Ranks may differ from layer to layer and, for bf16 factors, between q, k and v: the kernel wants one rank per
         # row group, a multiple of 128 (a lane group covers 128 elements of a row) and at least one row per workgroup,
         # so factors that do not fit are copied once into zero-padded twins (zero rows / columns contribute nothing:
@@ -149,10 +154,10 @@ class PersistentDecoder:
         self.PART, self.A = tagged64(H * nsplit * (Dh + 2)), tagged(H * Dh)
         self.PO, self.PM, self.HB, self.SB = tagged(Ro), tagged(2 * Rm), tagged(D), tagged(Rd)
         self.CAND = tagged64(self.nwg)
-        self.logits = torch.zeros(V, dtype=torch.bfloat16, device=dev)
+        self.logits = torch.zeros(V, dtype=edt, device=dev)
         self.token_log = torch.zeros(int(max_new_tokens), dtype=torch.int64, device=dev)
         self.state = torch.zeros(8, dtype=torch.int32, device=dev)   # fsvd_step_state
-        self.rope = cache.get_rope_tables(seqlen=S, head_dim=Dh, device=dev, dtype=torch.bfloat16)
+        self.rope = cache.get_rope_tables(seqlen=S, head_dim=Dh, device=dev, dtype=edt)
         cos, sin = self.rope
         self._keep = []   # tensors whose storage the phase list points into
 
@@ -172,12 +177,12 @@ class PersistentDecoder:
             return (lo | hi).contiguous()
 
         def pad_rows(w, n):       # zero rows below: outputs that are zero
-            out_ = torch.zeros(n, w.shape[1], dtype=torch.bfloat16, device=dev)
+            out_ = torch.zeros(n, w.shape[1], dtype=edt, device=dev)
             out_[:w.shape[0]] = w.data
             return out_
 
         def pad_cols(w, n):       # zero columns to the right: inputs that are multiplied by zero
-            out_ = torch.zeros(w.shape[0], n, dtype=torch.bfloat16, device=dev)
+            out_ = torch.zeros(w.shape[0], n, dtype=edt, device=dev)
             out_[:, :w.shape[1]] = w.data
             return out_
 
@@ -185,6 +190,8 @@ class PersistentDecoder:
                  flags=0, in_off=0, in2=None, in2_len=0, in2_off=0, rows0=0, aux2=None, out1=None):
             p = Phase()
             p.type, p.epilogue, p.N, p.K, p.nmat, p.mode = PH_GEMV, epi, N, K, nmat, mode
+            if edt == torch.float16:
+                p.wbits = _lib.WBITS_FP16     # in every GEMV phase: the step's element type
             if groups is not None:          # rows are q | k | v heads, each group reads its own K-long input
                 p.H, p.Hk, p.Dh = groups
             if q4 is not None:              # W holds (qweight, scales, zeros) triples; q4 = group size
@@ -254,8 +261,8 @@ class PersistentDecoder:
                 # unequal or unaligned q / k / v ranks: [q_v; k_v; v_v] with each block padded to rq rows, and the head bases
                 # with their columns padded to rq
                 aq, ak, av = at._qkv_rank_tuple()
-                pv = torch.zeros(3 * rq, d, dtype=torch.bfloat16, device=dev)
-                qu = torch.zeros((H + 2 * Hk) * Dh, rq, dtype=torch.bfloat16, device=dev)
+                pv = torch.zeros(3 * rq, d, dtype=edt, device=dev)
+                qu = torch.zeros((H + 2 * Hk) * Dh, rq, dtype=edt, device=dev)
                 for i, (m_v, m_u, r_, row0, rows) in enumerate(((at.q_v_proj, at.q_u_proj, aq, 0, H * Dh), (at.k_v_proj, at.k_u_proj, ak, H * Dh, Hk * Dh),
                                                                 (at.v_v_proj, at.v_u_proj, av, (H + Hk) * Dh, Hk * Dh))):
                     pv[i * rq:i * rq + r_] = m_v.weight.data
@@ -270,7 +277,7 @@ class PersistentDecoder:
             w_guv, w_gu, w_uu = mlp._packed_gu_v, mlp.gate_u_proj.weight, mlp.up_u_proj.weight
             if padded[l]["gu"]:
                 am = int(mlp.gate_v_proj.out_features)
-                w_guv = torch.zeros(2 * rm, d, dtype=torch.bfloat16, device=dev)
+                w_guv = torch.zeros(2 * rm, d, dtype=edt, device=dev)
                 w_guv[:am] = mlp.gate_v_proj.weight.data
                 w_guv[rm:rm + am] = mlp.up_v_proj.weight.data
                 w_gu, w_uu = pad_cols(w_gu, rm), pad_cols(w_uu, rm)
@@ -434,7 +441,7 @@ class PersistentDecoder:
             """W diag(norm) in fp32; as a bf16 matrix it is W itself when the norm weights are all one."""
             nw = norm.weight.data.float()
             wf = w.data.float() * nw[None, :]
-            return wf, (w if bool((nw == 1).all()) else wf.to(torch.bfloat16).contiguous())
+            return wf, (w if bool((nw == 1).all()) else wf.to(self.dtype).contiguous())
 
         bw = [bf16_weights(l) for l in range(L)]
         fq = [folded(bw[l]["qkv_v"], layers[l].input_layernorm) for l in range(L)]
@@ -446,7 +453,7 @@ class PersistentDecoder:
             w = bw[l]
             gu32, gu16 = folded(w["gu_v"], n2)
             # [o_u; [gate_v; up_v]' o_u] and [down_u; [q_v; k_v; v_v]'(next layer) down_u]: one stream each
-            cat_o = torch.cat([w["o_u"].data, (gu32 @ w["o_u"].data.float()).to(torch.bfloat16)]).contiguous()
+            cat_o = torch.cat([w["o_u"].data, (gu32 @ w["o_u"].data.float()).to(self.dtype)]).contiguous()
             if l == 0:
                 gemv("attn_rank_proj", [fq[0][1]], 3 * rq, d, xin, None, epi=EP_F32, out1=_tb(self.PRAW, L, 0))
             gemv("qkv_u", [w["qkv_u"]], (H + 2 * Hk) * Dh, rq, _tb(self.PRAW, L, l), _tb(self.QKV, L, l), groups=(H, Hk, Dh),
@@ -468,7 +475,7 @@ class PersistentDecoder:
                      flags=PF_NOWAIT | (PF_LEAD if self.leading else 0), in_off=off_m, out1=_tb(self.Q0, nq0, l))
             gemv("down_v", [w["down_v"]], rd, D, _tb(self.HB, L, l), _tb(self.SB, L, l))
             if l + 1 < L:
-                cat_d = torch.cat([w["down_u"].data, (fq[l + 1][0] @ w["down_u"].data.float()).to(torch.bfloat16)]).contiguous()
+                cat_d = torch.cat([w["down_u"].data, (fq[l + 1][0] @ w["down_u"].data.float()).to(self.dtype)]).contiguous()
                 gemv("down_u+attn_rank", [cat_d], d + 3 * rq_n, rd, _tb(self.SB, L, l), xout, epi=EP_RESID, aux=xmid, flags=PF_SPLIT,
                      rows0=d, aux2=_tb(self.Q0, nq0, l), out1=_tb(self.PRAW, L, l + 1))
             else:
@@ -584,6 +591,8 @@ class PersistentDecoder:
         """Final-layer hidden state of the last step, bf16 [hidden] (part "attention": the state after the attention
         half's residual add; part "mlp": after the MLP half's)."""
         buf = self.XB if getattr(self, "part", "model") == "attention" else self.XA
+        if getattr(self, "dtype", torch.bfloat16) == torch.float16:
+            return (buf & 0xFFFF).to(torch.int16).view(torch.float16)
         return ((buf & 0xFFFF) << 16).view(torch.float32).to(torch.bfloat16)
 
 

@@ -57,8 +57,9 @@ int fsvd_set_workspace(void* ws, size_t bytes, void* stream);
  * fp32, roundings are to nearest even at the same points in both.  The reference picks the type from its inputs the
  * same way (kernels/attn/decode/densekv_reconstruct_triton.py:427-428; fp16 is the default of its dense cache,
  * runtime/cache/attn_dense_kv.py:26, and the fallback of scripts/demo_support/api.py:161-165).  So does the rank-space
- * decode attention (fsvd_attn_decode_rankkv; fsvd_rankkv_append copies 16-bit patterns of either type).  The int4 entries
- * and the persistent decode step are bf16 only. */
+ * decode attention (fsvd_attn_decode_rankkv; fsvd_rankkv_append copies 16-bit patterns of either type).  The
+ * persistent decode step takes its type from its phase list (FSVD_WBITS_FP16); the int4 entries and int4 phases take
+ * bf16 activations only. */
 
 /* y[b,n] = (res[b,n] +) bf16( W[n,:] . norm(x[b,:]) (+ bias[n]) ),  W is an nn.Linear weight [N,K].
  * norm_w != NULL fuses the RMSNorm of x (w * bf16(x * rsqrt(mean(x^2)+eps))) in front.
@@ -314,6 +315,8 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
 #define FSVD_PH_MERGE 4   /* out0 = merged attention output from in = partials                               */
 #define FSVD_PH_ARGMAX 5  /* token = argmax of the per-workgroup candidates in `in`; advances the state      */
 
+#define FSVD_WBITS_FP16 (-16) /* fsvd_phase.wbits of a GEMV phase whose weights are float16 (see there)                */
+
 #define FSVD_EP_STORE 0   /* out0[n] = bf16(dot)                                                              */
 #define FSVD_EP_RESID 1   /* out0[n] = bf16(aux0[n] + bf16(dot))                                              */
 #define FSVD_EP_SWIGLU 2  /* nmat = 2: out0[n] = silu(W[0][n].in[0:K]) * (W[1][n].in[K:2K]), rounding `mode`  */
@@ -382,7 +385,8 @@ typedef struct fsvd_phase {
    * the fp16 scale bits of a group in the low half and (zero point + 128) in the high half; a group is
    * 32 << gshift columns.  K % 256 == 0.  Arithmetic as fsvd_linear_q4: y = sum_g s_g * sum_k x_k (q_k - z_g), fp32. */
   const void* qsz[2];
-  int32_t ldg, gshift, wbits;
+  int32_t ldg, gshift, wbits;   /* wbits also names the element type of a step: FSVD_WBITS_FP16 in EVERY GEMV phase of a list   */
+                                /* makes it a float16 step (vectors, tables, caches and weights float16; no int4 phases)     */
   int32_t shared_in;            /* nmat == 2: both matrices read the same K-long input (a dense gate / up pair) instead   */
                                 /* of in[0:K] and in[K:2K]                                                                 */
   /* derived by fsvd_decode_step_prepare (do not fill by hand): work items (rows, merge outputs) are

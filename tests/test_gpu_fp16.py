@@ -293,11 +293,65 @@ def test_generate_text_after_the_float16_cast():
     assert out["new_tokens"] == 4 and out["decode_tok_s"] > 0 and out["flashsvd_dense_cache"]
 
 
-def test_persistent_step_refuses_float16():
+@pytest.mark.parametrize("composed", [False, True], ids=["ten_phase", "composed"])
+def test_persistent_step_in_float16_teacher_forced_against_oracle(composed):
+    """The resident step over a float16 model (every GEMV phase carries FSVD_WBITS_FP16): a 3-layer GQA model of
+    head_dim 128, the oracle's tokens fed back, hidden states and logits against the oracle in float16 at the
+    multi-layer bound (three times the float16 bar), tokens tie-aware; then free-running against the per-operator
+    engine on the same model."""
+    from flashsvd_amd.graphs import GraphedDecoder
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    from flashsvd_amd.step import PersistentDecoder
+    mw = O.make_model(d=1024, n_heads=8, n_kv_heads=4, head_dim=128, ffn=2048, attn_rank=256, mlp_rank=384,
+                      n_layers=3, vocab=2048, dtype=FP16, seed=3)
+    prompt = torch.randint(0, 2048, (1, 37), generator=torch.Generator().manual_seed(5))
+    n_new, Lp = 12, 37
+    model = model_from_oracle(mw)
+    ref_tok, ref_hid, _, ref_logits = O.greedy_decode(mw, prompt, n_new, "dense", return_logits=True)
+
+    def prefill():
+        cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=Lp + n_new + 4, device="cuda", dtype=FP16)
+        out = model(prompt.cuda(), past_key_values=cache, cache_position=torch.arange(Lp))
+        return cache, out.logits[:, -1].float().argmax(-1, keepdim=True)
+
+    cache, tok0 = prefill()
+    assert int(tok0) == int(ref_tok[0, 0])
+    dec = PersistentDecoder(model, cache, composed=composed)
+    assert dec.dtype == FP16 and dec.composed == composed and dec.logits.dtype == FP16
+    n_equal = 0
+    for s_ in range(1, n_new):
+        dec.set_state(ref_tok[:, s_ - 1], Lp + s_ - 1)
+        dec.step(1)
+        g, o = int(dec.tokens()[0]), int(ref_tok[0, s_])
+        m = float(ref_hid[:, s_].float().abs().max())
+        assert_close_bf16(dec.hidden()[None].cpu(), ref_hid[:, s_], f"hidden state at step {s_}",
+                          abs_tol=3 * (5e-3 if m < 2.0 else 2.0 * m * 2.0 ** -10), rel_tol=7.5e-3)
+        rl = ref_logits[0, s_].float()
+        if g != o:    # only where the oracle itself holds the two candidates within float16 resolution of the hidden states
+            assert float(rl[o] - rl[g]) <= 5e-3 * float(rl.abs().max()), f"step {s_}: token {g} vs oracle {o}"
+        n_equal += int(g == o)
+    assert n_equal >= n_new - 3
+    # free-running: the resident step and the per-operator engine from the same prompt
+    cache_p, tok_p = prefill()
+    pdec = PersistentDecoder(model, cache_p, composed=composed)
+    pdec.set_state(tok_p, Lp)
+    pdec.step(n_new - 1)
+    cache_g, tok_g = prefill()
+    gdec = GraphedDecoder(model, cache_g, 1)
+    gdec.set_state(tok_g, Lp)
+    toks_g = torch.cat([gdec.eager_step().reshape(-1).cpu() for _ in range(n_new - 1)])
+    same = int((pdec.tokens().cpu() == toks_g).sum())
+    if composed:
+        assert same >= n_new - 3, f"composed form: {same}/{n_new - 1} tokens equal to the per-operator engine"
+    else:
+        assert same == n_new - 1, f"resident step {pdec.tokens().tolist()} vs per-operator engine {toks_g.tolist()}"
+
+
+def test_persistent_step_refuses_mixed_types():
     from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
     from flashsvd_amd.step import PersistentDecoder
     mw, _ = O.config_c1(FP16)
     model = model_from_oracle(mw)
-    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=64, device="cuda", dtype=FP16)
-    with pytest.raises(ValueError, match="bf16 only"):
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="KV cache of the model's type"):
         PersistentDecoder(model, cache)
