@@ -27,9 +27,9 @@ class _UV(nn.Module):
         return self.u_proj(self.v_proj(x))
 
 
-def _mw():
+def _mw(dtype=BF16):
     return O.make_model(d=256, n_heads=4, n_kv_heads=2, head_dim=128, ffn=512, attn_rank=64, mlp_rank=128, n_layers=2,
-                        vocab=400, dtype=BF16, seed=11, std=0.05)
+                        vocab=400, dtype=dtype, seed=11, std=0.05)
 
 
 def _hf_from_oracle(mw):
@@ -41,7 +41,7 @@ def _hf_from_oracle(mw):
     cfg = LlamaConfig(vocab_size=m["vocab"], hidden_size=m["d"], intermediate_size=m["ffn"], num_hidden_layers=m["n_layers"],
                       num_attention_heads=mw.n_heads, num_key_value_heads=mw.n_kv_heads, head_dim=mw.head_dim, rms_norm_eps=mw.eps,
                       attention_bias=False, mlp_bias=False, tie_word_embeddings=False, max_position_embeddings=256)
-    hf = LlamaForCausalLM(cfg).to(BF16).eval()
+    hf = LlamaForCausalLM(cfg).to(mw.embed.dtype).eval()
     with torch.no_grad():
         hf.model.embed_tokens.weight.copy_(mw.embed)
         hf.lm_head.weight.copy_(mw.lm_head)
@@ -64,7 +64,8 @@ def _decode(model, prompt, n_new):
     from flashsvd_amd import api
     from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
     Lp = prompt.shape[1]
-    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=Lp + n_new + 2, device="cuda", dtype=BF16)
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=Lp + n_new + 2, device="cuda",
+                                    dtype=model.lm_head.weight.dtype)
     assert api._can_use_manual_llama_decode_step(model)
     out = api._manual_llama_decode_step(model, prompt.cuda(), past_key_values=cache, cache_position=torch.arange(Lp))
     toks, logits = [], [out.logits[:, -1].clone()]
@@ -88,10 +89,11 @@ def unpatched():
     llama.LAYER_TAIL_GRAPH_ENABLED = keep
 
 
-def test_modules_inside_unmodified_hf_model(unpatched, monkeypatch):
+@pytest.mark.parametrize("dtype", [BF16, torch.float16], ids=["bf16", "fp16"])
+def test_modules_inside_unmodified_hf_model(unpatched, monkeypatch, dtype):
     from transformers.models.llama.modeling_llama import LlamaDecoderLayer, LlamaRMSNorm
     from flashsvd_amd import api, llama
-    mw = _mw()
+    mw = _mw(dtype)
     own = model_from_oracle(mw)
     hf = _hf_from_oracle(mw)
     lay = hf.model.layers[0]
