@@ -36,9 +36,10 @@ def _tb(t: torch.Tensor, uses: int, use: int) -> TagBuf:
 class PersistentDecoder:
     """``PersistentDecoder(model, cache)`` then ``set_state(token, position)``, ``step(n)``, ``tokens()``.
 
-    Requirements (checked): batch 1, bf16, dense KV cache, head_dim 128, hidden and intermediate sizes that are multiples
-    of 128, and a device whose compute-unit count is a multiple of the number of heads.  Factor ranks are free for bf16
-    factors (unequal q / k / v ranks, ranks that are not multiples of 128 or smaller than the workgroup count are served
+    Requirements (checked): batch 1, one 16-bit type throughout (bfloat16, or float16 for a model without int4 factors;
+    weights, norms, embedding and cache alike), dense KV cache, head_dim 128, hidden and intermediate sizes that are
+    multiples of 128, and a device whose compute-unit count is a multiple of the number of heads.  Factor ranks are free
+    for 16-bit factors (unequal q / k / v ranks, ranks that are not multiples of 128 or smaller than the workgroup count are served
     from zero-padded copies made once, at the cost of their memory); int4 layers need equal q / k / v ranks and row
     lengths that are multiples of 256.  Models outside these limits decode through ``graphs.GraphedDecoder``.
     """
@@ -588,7 +589,7 @@ class PersistentDecoder:
         return self.token_log[: self._host_steps].clone()
 
     def hidden(self) -> torch.Tensor:
-        """Final-layer hidden state of the last step, bf16 [hidden] (part "attention": the state after the attention
+        """Final-layer hidden state of the last step in the step's element type, [hidden] (part "attention": the state after the attention
         half's residual add; part "mlp": after the MLP half's)."""
         buf = self.XB if getattr(self, "part", "model") == "attention" else self.XA
         if getattr(self, "dtype", torch.bfloat16) == torch.float16:
