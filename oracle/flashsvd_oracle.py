@@ -9,7 +9,7 @@ reference implements with Triton kernels, cuBLAS calls and flash-attn, with ever
 floating-point rounding point written out.  Each function names the reference
 file:line it follows (paths relative to the reference checkout).
 
-Arithmetic contract used everywhere ("dtype" is torch.float32 or torch.bfloat16):
+Arithmetic contract used everywhere ("dtype" is torch.float32, torch.bfloat16 or torch.float16):
   * every matrix product accumulates in fp32 and is rounded once to ``dtype``
     (what a chain of ``nn.Linear`` modules does on an accelerator);
   * element-wise ops on ``dtype`` tensors round after every op, like eager PyTorch;

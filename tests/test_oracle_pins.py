@@ -37,19 +37,22 @@ def test_lowrank_pair_full_rank_is_dense_linear():
     assert torch.allclose(y, torch.nn.functional.linear(_rand(4, d, seed=5), W), atol=1e-5)
 
 
-def test_lin_bf16_rounds_once_from_fp32():
-    x, w = _rand(2, 64, dtype=torch.bfloat16), _rand(8, 64, dtype=torch.bfloat16)
+@pytest.mark.parametrize("dt,half_ulp", [(torch.bfloat16, 2 ** -8), (torch.float16, 2 ** -11)], ids=["bf16", "fp16"])
+def test_lin_16bit_rounds_once_from_fp32(dt, half_ulp):
+    x, w = _rand(2, 64, dtype=dt), _rand(8, 64, dtype=dt)
     exact = (x.double() @ w.double().t())
     y = O.lin(x, w)
-    assert y.dtype == torch.bfloat16
-    # one bf16 rounding of an (almost) exact sum: error <= 1/2 ulp (2^-9 relative) + fp32 noise
-    assert torch.all((y.double() - exact).abs() <= exact.abs() * 2 ** -8 + 1e-6)
+    assert y.dtype == dt
+    # one rounding of an (almost) exact sum to the 16-bit type: error <= 1/2 ulp (unit roundoff 2^-8 bf16, 2^-11 fp16) + fp32 noise;
+    # a second rounding on the way (e.g. through the other 16-bit type) would double it
+    assert torch.all((y.double() - exact).abs() <= exact.abs() * half_ulp * 1.02 + 1e-6)
+    assert torch.equal(y, (x.float() @ w.float().t()).to(dt))
 
 
 # ---------------------------------------------------------------- rmsnorm
 def test_rms_norm_matches_transformers():
     from transformers.models.llama.modeling_llama import LlamaRMSNorm
-    for dt in (torch.float32, torch.bfloat16):
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
         n = LlamaRMSNorm(32, eps=1e-6).to(dt)
         with torch.no_grad():
             n.weight.copy_(_rand(32, seed=3).to(dt))
@@ -89,7 +92,7 @@ def test_rope_invariants():
 def test_rope_matches_transformers_apply_rotary():
     from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
     Dh, T = 16, 6
-    for dt in (torch.float32, torch.bfloat16):
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
         cos_h, sin_h = O.rope_tables(T, Dh, dtype=dt)
         cos = torch.cat([cos_h, cos_h], -1)[None]
         sin = torch.cat([sin_h, sin_h], -1)[None]
@@ -97,7 +100,7 @@ def test_rope_matches_transformers_apply_rotary():
         k = _rand(1, 2, T, Dh, dtype=dt, seed=8)
         qe, ke = apply_rotary_pos_emb(q, k, cos, sin)
         mine = O.apply_rope(q, cos_h[None, None], sin_h[None, None])
-        assert torch.allclose(mine.float(), qe.float(), atol=0 if dt == torch.float32 else 2 ** -7 * 4)
+        assert torch.allclose(mine.float(), qe.float(), atol={torch.float32: 0, torch.bfloat16: 2 ** -7 * 4, torch.float16: 2 ** -10 * 4}[dt])
         if dt == torch.float32:
             assert torch.allclose(O.apply_rope_fp32(k, cos_h[None, None], sin_h[None, None]), ke, atol=1e-6)
 
@@ -300,12 +303,13 @@ def test_cached_greedy_decode_equals_full_recompute(cache_kind):
         seq = torch.cat([seq, nxt], 1)
 
 
-def test_rank_cache_and_dense_cache_agree_bf16():
-    mw = _tiny(torch.bfloat16)
+@pytest.mark.parametrize("dt,noise", [(torch.bfloat16, 0.15), (torch.float16, 0.02)], ids=["bf16", "fp16"])
+def test_rank_cache_and_dense_cache_agree_16bit(dt, noise):
+    mw = _tiny(dt)
     prompt = torch.randint(0, 50, (1, 8), generator=torch.Generator().manual_seed(6))
     _, hd, _ = O.greedy_decode(mw, prompt, 4, "dense", return_hidden=True)
     _, hr, _ = O.greedy_decode(mw, prompt, 4, "rank", return_hidden=True)
-    assert (hd.float() - hr.float()).abs().max() < 0.15  # bf16 noise only; same algebra
+    assert hd.dtype == dt and (hd.float() - hr.float()).abs().max() < noise  # rounding noise of the type only; same algebra
 
 
 # ---- group-wise int4 weights (src/quant/packed_quant_linear.py) --------------------------------
