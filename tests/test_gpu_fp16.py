@@ -147,6 +147,30 @@ def test_expand_heads_and_prompt_attention(ops, B, M, R):
         close(out[:, m], O.dense_decode_attn(q_ref[:, m], k_ref[:, :m + 1], v_ref[:, :m + 1]), f"prompt attention row {m}")
 
 
+@pytest.mark.parametrize("B,H,Hk,M,R,shared", [(1, 32, 32, 512, 1024, True), (2, 4, 2, 100, 40, False), (1, 8, 8, 333, 1664, True)])
+def test_rope_attention_module(B, H, Hk, M, R, shared):
+    """FlashSVDRoPEAttention (kernels/flashsvdropeattn.py, the reference's module interface) on float16 factors."""
+    from flashsvd_amd.kernels.flashsvdropeattn import FlashSVDRoPEAttention, QKVFactors
+
+    class Rot:
+        inv_freq = 1.0 / (10000.0 ** (torch.arange(0, 64, dtype=torch.float32) / 64))
+
+    dh = 128
+    if shared:
+        pq, pk, pv = (rand_fp16(B, 1, M, R, seed=i) for i in range(3))
+        Pq, Pk, Pv = pq.expand(B, H, M, R), pk.expand(B, Hk, M, R), pv.expand(B, Hk, M, R)
+    else:
+        Pq, Pk, Pv = rand_fp16(B, H, M, R, seed=0), rand_fp16(B, Hk, M, R, seed=1), rand_fp16(B, Hk, M, R, seed=2)
+    sc = R ** -0.5
+    Vq, Vk, Vv = rand_fp16(H, R, dh, std=sc, seed=3), rand_fp16(Hk, R, dh, std=sc, seed=4), rand_fp16(Hk, R, dh, std=sc, seed=5)
+    cos, sin = O.rope_tables(M, dh, dtype=FP16)
+    ref = O.rope_sdpa_prefill(Pq, Pk, Pv, Vq, Vk, Vv, cos, sin)
+    mod = FlashSVDRoPEAttention(H, dh, Rot(), bm=64, bn=64, br=64)
+    out = mod(QKVFactors(*[t.cuda() for t in (Pq, Pk, Pv, Vq, Vk, Vv)]), None, torch.arange(M, device="cuda")[None])
+    assert out.shape == (B, M, H, dh)
+    close(out, ref, "rope attention module")
+
+
 def test_mixed_element_types_are_refused(ops):
     x, w = rand_fp16(1, 256, seed=1).cuda(), rand_fp16(64, 256, seed=2).cuda()
     with pytest.raises(ValueError, match="must be torch.float16"):
