@@ -97,6 +97,8 @@ SIGNATURES = {
     "fsvd_last_error": (c_char_p, []),
     "fsvd_linear": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_float, c_void_p, c_int64,
                             c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "fsvd_linear_rankkv_append": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int, c_int, c_int, c_int,
+                                          c_int, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int, c_int, c_void_p]),
     "fsvd_swiglu_linear": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                                    c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_linear_q4": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p,

@@ -79,6 +79,24 @@ int fsvd_linear(const void* x, int64_t ldx, const void* W, int64_t ldw, const vo
   return launch_linear(a, cfg, static_cast<hipStream_t>(stream));
 }
 
+int fsvd_linear_rankkv_append(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* norm_w, float eps, void* y, int64_t ldy,
+                              int B, int Rq, int Rk, int Rv, int K, void* pk_cache, int64_t spk_b, int64_t spk_s, void* pv_cache,
+                              int64_t spv_b, int64_t spv_s, const int32_t* positions, int S, int dtype, void* stream) {
+  const char* fn = "fsvd_linear_rankkv_append";
+  FSVD_REQUIRE_PTR(x, fn); FSVD_REQUIRE_PTR(W, fn); FSVD_REQUIRE_PTR(y, fn); FSVD_REQUIRE_PTR(pk_cache, fn); FSVD_REQUIRE_PTR(pv_cache, fn);
+  FSVD_REQUIRE_PTR(positions, fn);
+  if (B <= 0 || B > 2) { set_last_error("%s: %d rows (one or two: more rows take fsvd_linear and fsvd_rankkv_append)", fn, B); return kErrBadShape; }
+  if (Rq < 0 || Rk <= 0 || Rv <= 0 || S <= 0) { set_last_error("%s: bad ranks / cache length (Rq=%d Rk=%d Rv=%d S=%d)", fn, Rq, Rk, Rv, S); return kErrBadShape; }
+  const int N = Rq + Rk + Rv;
+  if (ldx < K || ldw < K || ldy < N || spk_s < Rk || spv_s < Rv) { set_last_error("%s: a leading dimension is smaller than its row", fn); return kErrBadShape; }
+  LinearArgs a{cu16(x), ldx, cu16(W), ldw, nullptr, cu16(norm_w), eps, nullptr, 0, u16(y), ldy, B, N, K, dtype};
+  a.positions = positions;
+  a.app[0] = u16(pk_cache); a.app_sb[0] = spk_b; a.app_ss[0] = spk_s; a.app_n0[0] = Rq; a.app_n[0] = Rk;
+  a.app[1] = u16(pv_cache); a.app_sb[1] = spv_b; a.app_ss[1] = spv_s; a.app_n0[1] = Rq + Rk; a.app_n[1] = Rv;
+  a.app_S = S;
+  return launch_linear(a, 0, static_cast<hipStream_t>(stream));
+}
+
 int fsvd_swiglu_linear(const void* p, int64_t ldp, int64_t up_off, const void* gate_u, const void* up_u, int64_t ldw,
                        void* h, int64_t ldh, int B, int D, int R, int mode, int cfg, int dtype, void* stream) {
   FSVD_REQUIRE_PTR(p, "fsvd_swiglu_linear"); FSVD_REQUIRE_PTR(gate_u, "fsvd_swiglu_linear");

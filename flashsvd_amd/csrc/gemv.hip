@@ -253,7 +253,18 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(LinearArgs a) {
           if (a.bias) v += E::val(a.bias[n]);
           v = E::rnd(v);
           if (a.res) v = E::rnd(E::val(a.res[(int64_t)(b0 + b) * a.ldres + n]) + v);
-          a.y[(int64_t)(b0 + b) * a.ldy + n] = (uint16_t)E::bits(v);
+          const uint16_t bits = (uint16_t)E::bits(v);
+          a.y[(int64_t)(b0 + b) * a.ldy + n] = bits;
+          if (a.positions) {               // the same value into the cache row of this token (uniform branch: a kernel argument)
+            const int pos = a.positions[b0 + b];
+            if (pos >= 0 && pos < a.app_S) {
+#pragma unroll
+              for (int i = 0; i < 2; ++i) {
+                const int j = n - a.app_n0[i];
+                if (a.app[i] && j >= 0 && j < a.app_n[i]) a.app[i][(int64_t)(b0 + b) * a.app_sb[i] + (int64_t)pos * a.app_ss[i] + j] = bits;
+              }
+            }
+          }
         }
       }
   }
@@ -580,7 +591,10 @@ static int launch_linear_t(const LinearArgs& a, int cfg, hipStream_t st) {
 int launch_linear(const LinearArgs& a, int cfg, hipStream_t st) {
   if (a.B <= 0 || a.N <= 0 || a.K <= 0) { set_last_error("fsvd_linear: empty shape B=%d N=%d K=%d", a.B, a.N, a.K); return kErrBadShape; }
   if (a.dt != 0 && a.dt != 1) { set_last_error("fsvd_linear: dtype code %d (bf16 = 0 and fp16 = 1 are served)", a.dt); return kErrBadDtype; }
-  if (cfg == 0 && mfma_linear_applies(a)) return launch_linear_mfma(a, st);
+  if (cfg == 0 && mfma_linear_applies(a)) {
+    if (a.positions) { set_last_error("fsvd_linear_rankkv_append: %d rows take the matrix-core kernels, which have no append epilogue (one or two rows)", a.B); return kErrBadShape; }
+    return launch_linear_mfma(a, st);
+  }
   if (a.K > 32768) { set_last_error("fsvd_linear: K=%d exceeds the 32768 LDS staging limit", a.K); return kErrBadShape; }
   return a.dt == 1 ? launch_linear_t<1>(a, cfg, st) : launch_linear_t<0>(a, cfg, st);
 }

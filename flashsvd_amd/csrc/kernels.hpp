@@ -14,6 +14,14 @@ struct LinearArgs {
   uint16_t* y; int64_t ldy;              // [B, N]
   int B, N, K;
   int dt = 0;                            // element type: 0 bf16, 1 fp16
+  // optional second destination of two column ranges of y (one decoded token's coefficients into a rank-space cache):
+  // y[b, app_n0[i] + j], j < app_n[i], is also stored at app[i][b * app_sb[i] + positions[b] * app_ss[i] + j] when
+  // positions[b] lies in [0, app_S).  Served by the one- and two-row kernels only.
+  const int32_t* positions = nullptr;
+  uint16_t* app[2] = {nullptr, nullptr};
+  int64_t app_sb[2] = {0, 0}, app_ss[2] = {0, 0};
+  int app_n0[2] = {0, 0}, app_n[2] = {0, 0};
+  int app_S = 0;
 };
 
 struct SwigluArgs {

@@ -156,6 +156,46 @@ def _linear_impl(x, weight, bias, norm_weight, eps, residual, out, cfg):
     return out
 
 
+def linear_rankkv_append(x: torch.Tensor, weight: torch.Tensor, pk_cache: torch.Tensor, pv_cache: torch.Tensor, positions: torch.Tensor, *,
+                         ranks, norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6) -> torch.Tensor:
+    """The packed rank projection of one or two decoded tokens, ``p = norm(x) @ weight.T`` with ``weight = [q_v; k_v; v_v]``
+    and ``ranks = (rq, rk, rv)``, which also stores the Pk | Pv parts of every row at ``pk_cache[b, positions[b]]`` /
+    ``pv_cache[b, positions[b]]`` (caches [>=B, S, R]): ``linear`` followed by ``rankkv_append`` in one launch, same bits.
+    Custom operator flashsvd_hip::linear_rankkv_append (the caches are mutated arguments)."""
+    rq, rk, rv = (int(r) for r in ranks)
+    return _OPS.linear_rankkv_append.default(x, weight, pk_cache, pv_cache, positions, rq, rk, rv, norm_weight, float(eps))
+
+
+def _linear_rankkv_append_impl(x, weight, pk_cache, pv_cache, positions, rq, rk, rv, norm_weight, eps):
+    dt, code = _elem(x, "x")
+    _need(weight, "weight", dtype=dt); _need(pk_cache, "pk_cache", dtype=dt); _need(pv_cache, "pv_cache", dtype=dt)
+    _need(positions, "positions", dtype=torch.int32)
+    if weight.dim() != 2 or weight.stride(1) != 1 or weight.shape[0] != rq + rk + rv:
+        raise ValueError(f"weight must be [rq + rk + rv, K] = [{rq + rk + rv}, K] with unit inner stride, got {tuple(weight.shape)}")
+    K = weight.shape[1]
+    x2 = _rows(x, "x")
+    B = x2.shape[0]
+    if x2.shape[1] != K or B > 2:
+        raise ValueError(f"x must be one or two rows of {K} values, got {tuple(x.shape)}")
+    for c, r, nm in ((pk_cache, rk, "pk_cache"), (pv_cache, rv, "pv_cache")):
+        if c.dim() != 3 or c.shape[0] < B or c.shape[2] != r or c.stride(2) != 1 or c.shape[1] != pk_cache.shape[1]:
+            raise ValueError(f"{nm} must be [>={B}, S, {r}] with unit inner stride, got {tuple(c.shape)}")
+    if positions.numel() != B or not positions.is_contiguous():
+        raise ValueError(f"positions must be a contiguous int32 [{B}] tensor")
+    if norm_weight is not None:
+        _need(norm_weight, "norm_weight", dtype=dt)
+        if norm_weight.shape != (K,) or not norm_weight.is_contiguous():
+            raise ValueError(f"norm_weight must be a contiguous [{K}] tensor")
+    out = torch.empty(*x.shape[:-1], rq + rk + rv, device=x.device, dtype=dt)
+    o2 = _rows(out, "out")
+    rc = _lib.load().fsvd_linear_rankkv_append(x2.data_ptr(), x2.stride(0), weight.data_ptr(), weight.stride(0), _ptr(norm_weight), float(eps),
+                                               o2.data_ptr(), o2.stride(0), B, rq, rk, rv, K, pk_cache.data_ptr(), pk_cache.stride(0),
+                                               pk_cache.stride(1), pv_cache.data_ptr(), pv_cache.stride(0), pv_cache.stride(1),
+                                               positions.data_ptr(), int(pk_cache.shape[1]), code, _stream())
+    _lib.check("fsvd_linear_rankkv_append", rc)
+    return out
+
+
 def swiglu_linear(p: torch.Tensor, gate_u: torch.Tensor, up_u: torch.Tensor, *, up_off: int, mode: int = 0,
                   out: Optional[torch.Tensor] = None, cfg: int = 0) -> torch.Tensor:
     """h = silu(p[..., :R] @ gate_u.T) * (p[..., up_off:up_off+R] @ up_u.T); gate_u/up_u are [D, R].

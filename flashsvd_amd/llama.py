@@ -330,10 +330,14 @@ class SVD_LlamaAttention(nn.Module):
         pkc, pvc = cache.key_cache[self.layer_idx], cache.value_cache[self.layer_idx]
         if rope is None:
             rope = cache.get_rope_tables(seqlen=cache.max_cache_len, head_dim=Dh, device=x.device, dtype=x.dtype)
-        p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)       # [B, rq+rk+rv]
-        if rq % 8 == 0 and rk % 8 == 0 and rv % 8 == 0 and positions.dtype == torch.int32:
+        if B <= 2 and positions.dtype == torch.int32 and positions.is_contiguous() and pkc.dim() == 3:
+            # one or two tokens: the projection writes Pk | Pv into the cache rows from its own epilogue (one launch)
+            p = hip_ops.linear_rankkv_append(x, self._packed_qkv_v, pkc, pvc, positions, ranks=(rq, rk, rv), norm_weight=norm_weight, eps=eps)
+        elif rq % 8 == 0 and rk % 8 == 0 and rv % 8 == 0 and positions.dtype == torch.int32:
+            p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)       # [B, rq+rk+rv]
             rankkv_append(p[:, rq:rq + rk], p[:, rq + rk:], pkc, pvc, positions)      # one launch
         else:
+            p = hip_ops.linear(x, self._packed_qkv_v, norm_weight=norm_weight, eps=eps)
             rows = torch.arange(B, device=x.device)
             pos = positions.long()
             pkc[rows, pos] = p[:, rq:rq + rk]    # device-side scatter of the new coefficients (data movement only)

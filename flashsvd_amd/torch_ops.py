@@ -162,6 +162,16 @@ _define(f"attn_decode_rankkv({_AR_ARGS}) -> Tensor", _attn_rank, lambda q, *a, *
 _define(f"attn_decode_rankkv.out({_AR_ARGS}, *, Tensor(d!) out) -> Tensor(d!)", _attn_rank_out, lambda *a, out, **k: out)
 
 
+def _linear_rankkv_append(x, weight, pk_cache, pv_cache, positions, rq, rk, rv, norm_weight=None, eps=1e-6):
+    from . import hip_ops
+    return hip_ops._linear_rankkv_append_impl(x, weight, pk_cache, pv_cache, positions, rq, rk, rv, norm_weight, eps)
+
+
+_define("linear_rankkv_append(Tensor x, Tensor weight, Tensor(a!) pk_cache, Tensor(b!) pv_cache, Tensor positions, int rq, int rk, int rv, "
+        "Tensor? norm_weight=None, float eps=1e-6) -> Tensor", _linear_rankkv_append,
+        lambda x, weight, *a, **k: x.new_empty((*x.shape[:-1], weight.shape[0])))
+
+
 def _rankkv_append(pk, pv, pk_cache, pv_cache, positions):
     from .kernels import rank_decode as RD
     RD._rankkv_append_impl(pk, pv, pk_cache, pv_cache, positions)
@@ -233,5 +243,5 @@ _define("mlp_dual_split(Tensor PUp, Tensor PGate, Tensor GateU, Tensor UpU, Tens
         PUp.new_empty((PUp.shape[0], DownU.shape[1])))
 
 ops = getattr(torch.ops, NS)
-OP_NAMES = ("linear", "swiglu_linear", "rmsnorm", "qkv_rope_append", "attn_decode_densekv", "attn_decode_rankkv", "rankkv_append",
+OP_NAMES = ("linear", "swiglu_linear", "rmsnorm", "qkv_rope_append", "attn_decode_densekv", "attn_decode_rankkv", "rankkv_append", "linear_rankkv_append",
             "lowrank_expand_heads", "rope_attn_prefill", "reconstruct_qkv_token", "xw_linear", "mlp_dual_split")

@@ -236,6 +236,17 @@ int fsvd_attn_decode_rankkv(const void* q, int64_t sq_b, int64_t sq_h,
                             int B, int H, int Hk, int Dh, int S, int Rk, int Rv, int nsplit, float scale,
                             float* scores, size_t scores_bytes, int dtype, void* stream);
 
+/* The packed rank projection of a decoded token with the cache append in its epilogue, for one or two rows:
+ * y[b, :] = bf16( W . norm(x[b, :]) ) with W = [q_v; k_v; v_v] ([Rq + Rk + Rv, K], nn.Linear layout), and the Pk | Pv parts
+ * of y also stored at pk_cache[b, positions[b], :] / pv_cache[b, positions[b], :] (caches [B,S,R] with strides (sp*_b,
+ * sp*_s, 1); a row whose position is outside [0, S) is not appended).  One launch for `hidden @ packed_qkv_rank`
+ * (benchmark/attn/decode_compare.py:1538) plus FlashSVDLegacySparseKVCache.update
+ * (runtime/cache/attn_legacy_sparse_kv.py:113-169); the same bits as fsvd_linear followed by fsvd_rankkv_append. */
+int fsvd_linear_rankkv_append(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* norm_w, float eps, void* y,
+                              int64_t ldy, int B, int Rq, int Rk, int Rv, int K, void* pk_cache, int64_t spk_b, int64_t spk_s,
+                              void* pv_cache, int64_t spv_b, int64_t spv_s, const int32_t* positions, int S, int dtype,
+                              void* stream);
+
 /* One decoded token per batch row into a rank-space cache: pk_cache[b, positions[b], :] = pk[b, :] and the same for pv
  * (FlashSVDLegacySparseKVCache.update with one position per row, runtime/cache/attn_legacy_sparse_kv.py:113-169: two
  * index_copy_ calls there; one launch here).  Caches are [B,S,R] with strides (sp*_b, sp*_s, 1); a row whose position is

@@ -237,6 +237,29 @@ def test_rankkv_append_matches_index_copy(RD):
         RD.rankkv_append(p[:, 60:60 + Rk], p[:, 64 + Rk:], pkc, pvc, pos)
 
 
+@pytest.mark.parametrize("B,rq,rk,rv", [(1, 1024, 1024, 1024), (2, 72, 40, 136), (1, 64, 52, 52)])
+def test_projection_with_append_epilogue_equals_projection_then_append(RD, B, rq, rk, rv):
+    """fsvd_linear_rankkv_append: one launch, the bits of fsvd_linear followed by fsvd_rankkv_append (or by the indexed
+    copy, for ranks off the 8 grid), fused RMSNorm included; rows outside the cache are not appended."""
+    from flashsvd_amd import hip_ops
+    from flashsvd_amd._lib import FlashSVDHipError
+    K, S = 512, 24
+    x, w = rand_bf16(B, K, seed=1).cuda(), rand_bf16(rq + rk + rv, K, std=0.05, seed=2).cuda()
+    nw = (rand_bf16(K, seed=3) * 0.1 + 1).cuda()
+    pos = torch.tensor([5, 30][:B], dtype=torch.int32).cuda()       # the second row lies outside the cache
+    pkc = rand_bf16(B, S, rk, seed=4).cuda()
+    pvc = rand_bf16(B, S, rv, seed=5).cuda()
+    want_k, want_v = pkc.clone(), pvc.clone()
+    p_ref = hip_ops.linear(x, w, norm_weight=nw, eps=1e-6)
+    want_k[0, 5], want_v[0, 5] = p_ref[0, rq:rq + rk], p_ref[0, rq + rk:]
+    p = hip_ops.linear_rankkv_append(x, w, pkc, pvc, pos, ranks=(rq, rk, rv), norm_weight=nw, eps=1e-6)
+    assert torch.equal(p, p_ref) and torch.equal(pkc, want_k) and torch.equal(pvc, want_v)
+    assert_close_bf16(p, O.lin(O.rms_norm(x.cpu(), nw.cpu(), 1e-6), w.cpu()), "projection")
+    with pytest.raises(ValueError, match="one or two rows"):
+        hip_ops.linear_rankkv_append(rand_bf16(3, K).cuda(), w, rand_bf16(3, S, rk).cuda(), rand_bf16(3, S, rv).cuda(),
+                                     torch.zeros(3, dtype=torch.int32).cuda(), ranks=(rq, rk, rv))
+
+
 def test_rank_decode_rejects_unsupported(RD):
     from flashsvd_amd._lib import FlashSVDHipError
     c = lambda *s: rand_bf16(*s).cuda()
