@@ -759,14 +759,15 @@ def run_stress_model(steps: int = 8, warmup: int = 2, layers: int = 32):
     return {"model": f"{L}-layer 7B shape, attention rank {R}, MLP rank {RM}", "prefill": prefill, "decode": decode}
 
 
-def run_quant(args):
+def run_quant(args, dtype=None):
     """Config 4 with every factor linear as group-wise int4 (PackedQuantLinear, group 128, asymmetric): the persistent step
-    streams the packed nibbles (phases with wbits == 4), the per-operator graph uses fsvd_linear_q4 / fsvd_swiglu_linear_q4."""
+    streams the packed nibbles (int4 phases), the per-operator graph uses fsvd_linear_q4 / fsvd_swiglu_linear_q4.
+    ``dtype``: the type of the activations, the lm_head and the cache (bf16, or float16 with --fp16)."""
     import os
     import torch
     from flashsvd_amd import api, llama, quant as Q
     cfg = dict(CFG, num_layers=args.layers)
-    model = llama.materialize(llama.build_model(**cfg), "cuda", torch.bfloat16, seed=0)
+    model = llama.materialize(llama.build_model(**cfg), "cuda", dtype or torch.bfloat16, seed=0)
     n = Q.replace_linears_with_packed_quant_inplace(model, module_names=Q.factor_linear_names(model), bits=4, group_size=128, sym=False)
     torch.cuda.empty_cache()
     wbytes = 0
@@ -902,9 +903,10 @@ def main():
     from flashsvd_amd import _lib
     _lib.load()
     if args.quant:
-        q = run_quant(args)
+        q = run_quant(args, torch.float16 if args.fp16 else None)
+        act = "fp16" if args.fp16 else "bf16"
         print(json.dumps({"metric": "decode tok/s, 7B-shape rank-0.5 bs1, int4 factors (group 128)", "value": q["persistent"]["tok_s"], "unit": "tok/s",
-                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "int4 weights, bf16 activations, fp32 sums",
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": f"int4 weights, {act} activations, fp32 sums",
                           "data": "synthetic", "quant": q}))
         return
     if args.stress:

@@ -90,6 +90,7 @@ PH_EMBED, PH_GEMV, _PH_RESERVED, PH_ATTN, PH_MERGE, PH_ARGMAX = range(6)
 EP_STORE, EP_RESID, EP_SWIGLU, EP_LOGITS, EP_F32 = range(5)
 PF_NOWAIT, PF_STAGE2, PF_SPLIT, PF_LEAD = 1, 2, 4, 8
 WBITS_FP16 = -16
+WBITS_Q4_FP16 = -4
 
 # name -> (restype, argtypes); mirrors include/flashsvd_hip.h declaration by declaration
 SIGNATURES = {
@@ -102,10 +103,10 @@ SIGNATURES = {
     "fsvd_swiglu_linear": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
                                    c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_linear_q4": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p,
-                               c_float, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
-    "fsvd_dequant_q4": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
+                               c_float, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    "fsvd_dequant_q4": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "fsvd_swiglu_linear_q4": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                      c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+                                      c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fsvd_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                      c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int64, c_int64, c_int64,

@@ -48,7 +48,7 @@ static inline uint16_t* u16(void* p) { return static_cast<uint16_t*>(p); }
 
 extern "C" {
 
-int fsvd_version(void) { return 101; }
+int fsvd_version(void) { return 102; }
 const char* fsvd_last_error(void) { return g_last_error; }
 
 int fsvd_set_workspace(void* ws, size_t bytes, void* stream) {
@@ -112,28 +112,28 @@ int fsvd_swiglu_linear(const void* p, int64_t ldp, int64_t up_off, const void* g
 
 int fsvd_linear_q4(const void* x, int64_t ldx, const void* qweight, int64_t ldq, const void* scales, const void* zeros,
                    int64_t ldg, int group_size, const void* bias, const void* norm_w, float eps, const void* res,
-                   int64_t ldres, void* y, int64_t ldy, int B, int N, int K, void* stream) {
+                   int64_t ldres, void* y, int64_t ldy, int B, int N, int K, int dtype, void* stream) {
   const char* fn = "fsvd_linear_q4";
   FSVD_REQUIRE_PTR(x, fn); FSVD_REQUIRE_PTR(qweight, fn); FSVD_REQUIRE_PTR(scales, fn); FSVD_REQUIRE_PTR(zeros, fn);
   FSVD_REQUIRE_PTR(y, fn);
   if (ldx < K || ldy < N || (res && ldres < N)) { set_last_error("%s: leading dimension smaller than the row", fn); return kErrBadShape; }
   Q4Args a{cu16(x), ldx, 0, {static_cast<const uint8_t*>(qweight), nullptr}, ldq, {cu16(scales), nullptr},
            {static_cast<const int16_t*>(zeros), nullptr}, ldg, group_size, cu16(bias), cu16(norm_w), eps, cu16(res), ldres,
-           u16(y), ldy, B, N, K, 1, 0};
+           u16(y), ldy, B, N, K, 1, 0, dtype};
   return launch_linear_q4(a, static_cast<hipStream_t>(stream));
 }
 
 int fsvd_dequant_q4(const void* qweight, int64_t ldq, const void* scales, const void* zeros, int64_t ldg, int group_size,
-                    void* w, int64_t ldw, int N, int K, void* stream) {
+                    void* w, int64_t ldw, int N, int K, int dtype, void* stream) {
   const char* fn = "fsvd_dequant_q4";
   FSVD_REQUIRE_PTR(qweight, fn); FSVD_REQUIRE_PTR(scales, fn); FSVD_REQUIRE_PTR(zeros, fn); FSVD_REQUIRE_PTR(w, fn);
   return launch_dequant_q4(static_cast<const uint8_t*>(qweight), ldq, cu16(scales), static_cast<const int16_t*>(zeros), ldg,
-                           group_size, u16(w), ldw, N, K, static_cast<hipStream_t>(stream));
+                           group_size, u16(w), ldw, N, K, dtype, static_cast<hipStream_t>(stream));
 }
 
 int fsvd_swiglu_linear_q4(const void* p, int64_t ldp, int64_t up_off, const void* gate_q, const void* gate_scales,
                           const void* gate_zeros, const void* up_q, const void* up_scales, const void* up_zeros, int64_t ldq,
-                          int64_t ldg, int group_size, void* h, int64_t ldh, int B, int D, int R, int mode, void* stream) {
+                          int64_t ldg, int group_size, void* h, int64_t ldh, int B, int D, int R, int mode, int dtype, void* stream) {
   const char* fn = "fsvd_swiglu_linear_q4";
   FSVD_REQUIRE_PTR(p, fn); FSVD_REQUIRE_PTR(gate_q, fn); FSVD_REQUIRE_PTR(gate_scales, fn); FSVD_REQUIRE_PTR(gate_zeros, fn);
   FSVD_REQUIRE_PTR(up_q, fn); FSVD_REQUIRE_PTR(up_scales, fn); FSVD_REQUIRE_PTR(up_zeros, fn); FSVD_REQUIRE_PTR(h, fn);
@@ -144,7 +144,7 @@ int fsvd_swiglu_linear_q4(const void* p, int64_t ldp, int64_t up_off, const void
   }
   Q4Args a{cu16(p), ldp, up_off, {static_cast<const uint8_t*>(gate_q), static_cast<const uint8_t*>(up_q)}, ldq,
            {cu16(gate_scales), cu16(up_scales)}, {static_cast<const int16_t*>(gate_zeros), static_cast<const int16_t*>(up_zeros)},
-           ldg, group_size, nullptr, nullptr, 0.f, nullptr, 0, u16(h), ldh, B, D, R, 2, mode};
+           ldg, group_size, nullptr, nullptr, 0.f, nullptr, 0, u16(h), ldh, B, D, R, 2, mode, dtype};
   return launch_linear_q4(a, static_cast<hipStream_t>(stream));
 }
 

@@ -62,6 +62,11 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 template <int DT> struct E16;
 template <> struct E16<0> {
   static constexpr int code = 0;
+  // int4 streams: nib<S>(d) turns the nibbles at bits S and S + 16 of d into the patterns of two elements nib_off + n
+  // (exact in the element type) without a conversion: here 0x4300 | n = 128 + n.  one2 is the pair (1, 1).
+  static constexpr uint32_t one2 = 0x3f803f80u;
+  static constexpr int nib_off = 128;
+  template <int S> static __device__ __forceinline__ uint32_t nib(uint32_t d) { return ((d >> S) & 0x000f000fu) | 0x43004300u; }
   typedef bf16x8_t frag_t;
   static __device__ __forceinline__ f32x4_t mfma(frag_t a, frag_t b, f32x4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
   static __device__ __forceinline__ float lo(uint32_t packed) { return bf16_lo(packed); }
@@ -76,6 +81,13 @@ template <> struct E16<0> {
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 template <> struct E16<1> {
   static constexpr int code = 1;
+  // 0x4c00 | n << 6 = 16 + n: the nibble sits in the top of the mantissa, so the offset that the products carry (and
+  // that the row sum takes out again) stays small against the weights themselves
+  static constexpr uint32_t one2 = 0x3c003c00u;
+  static constexpr int nib_off = 16;
+  template <int S> static __device__ __forceinline__ uint32_t nib(uint32_t d) {
+    return ((S < 6 ? d << (S < 6 ? 6 - S : 0) : d >> (S < 6 ? 0 : S - 6)) & 0x03c003c0u) | 0x4c004c00u;
+  }
   typedef f16x8_t frag_t;
   static __device__ __forceinline__ f32x4_t mfma(frag_t a, frag_t b, f32x4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
   // V_CVT_F32_F16 on the low half of a 32-bit register, written as an instruction: left to the compiler, the widening is

@@ -126,10 +126,13 @@ struct GemvCtx {
   int q4, ldg, gshift;       // int4 weights: a piece is 32 columns; scale | zero words [N, ldg], group = 32 << gshift columns
   uint64_t sz0, sz1;         // byte addresses of the slab's scale | zero rows
 };
-template <bool Q4>
+// wbits of an int4 phase: 4 with bf16 activations, FSVD_WBITS_Q4_FP16 with float16 ones
+__host__ __device__ __forceinline__ bool is_q4_bits(int wbits) { return wbits == 4 || wbits == FSVD_WBITS_Q4_FP16; }
+// QB: the wbits value of an int4 phase in this build of the kernel (one compare on the walk)
+template <bool Q4, int QB>
 __device__ __forceinline__ void gemv_ctx(uint32_t dv, int w, GemvCtx& c) {
   c.K = DF_I(dv, K);
-  c.q4 = Q4 && DF_I(dv, wbits) == 4;
+  c.q4 = Q4 && DF_I(dv, wbits) == QB;
   c.kp = c.q4 ? c.K >> 5 : c.K >> 3;
   c.nmat = DF_I(dv, nmat);
   c.xk = DF_I(dv, shared_in) ? 0 : c.K;
@@ -269,8 +272,9 @@ __device__ __forceinline__ void lead_stream(const GemvCtx& a, uint32_t m_kp, u32
 // ---------------------------------------------------------------------------------------------
 // the same walk over group-wise int4 weights: a 16-byte piece is 32 columns, 8 consecutive lanes form a chunk of
 // 256 columns of one row (K % 256 == 0).  No weight becomes a float: OR-ing 0x4300 over a nibble n gives the bf16
-// pattern of 128 + n, V_DOT2_F32_BF16 multiplies two of them with two activations, and with X_p = sum of the piece's
-// activations the piece contributes s * (D_p - (z + 128) * X_p).  The activations sit in LDS in the order the masks
+// pattern of c + n with c = 128 (float16: 0x4c00 over n << 6, c = 16), the packed dot product multiplies two of them
+// with two activations, and with X_p = sum of the piece's activations the piece contributes
+// s * (D_p - (z + c) * X_p); the table holds z + c.  The activations sit in LDS in the order the masks
 // deliver the nibbles (columns 0,4 | 1,5 | 2,6 | 3,7 of every eight), X_p beside them (stage_store).
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ float row8_sum(float v) {
@@ -279,6 +283,7 @@ __device__ __forceinline__ float row8_sum(float v) {
   v += dpp_f32<0x141>(v);  // row_half_mirror
   return v;
 }
+template <class E>
 __device__ __forceinline__ float dot32_q4(const u32x4_t& q, const u32x4_t* xs) {
   float acc = 0.f;
   const uint32_t qd[4] = {q.x, q.y, q.z, q.w};
@@ -286,14 +291,14 @@ __device__ __forceinline__ float dot32_q4(const u32x4_t& q, const u32x4_t* xs) {
   for (int j = 0; j < 4; ++j) {
     const u32x4_t xv = xs[j];
     const uint32_t d = qd[j];
-    acc = dot2_bf16((d & 0x000f000fu) | 0x43004300u, xv.x, acc);
-    acc = dot2_bf16(((d >> 4) & 0x000f000fu) | 0x43004300u, xv.y, acc);
-    acc = dot2_bf16(((d >> 8) & 0x000f000fu) | 0x43004300u, xv.z, acc);
-    acc = dot2_bf16(((d >> 12) & 0x000f000fu) | 0x43004300u, xv.w, acc);
+    acc = E::dot2(E::template nib<0>(d), xv.x, acc);
+    acc = E::dot2(E::template nib<4>(d), xv.y, acc);
+    acc = E::dot2(E::template nib<8>(d), xv.z, acc);
+    acc = E::dot2(E::template nib<12>(d), xv.w, acc);
   }
   return acc;
 }
-template <int NMAT, bool GROUPED>
+template <class E, int NMAT, bool GROUPED>
 __device__ __forceinline__ void gemv_stream_q4(const GemvCtx& c, uint32_t m_kp, int g1, int g2, u32x4_t (&R)[kU], const uint32_t* sztab,
                                                const uint16_t* xs, const float* xsum, float* cp) {
   constexpr int SPB = kU / NMAT;                // steps per batch
@@ -314,7 +319,7 @@ __device__ __forceinline__ void gemv_stream_q4(const GemvCtx& c, uint32_t m_kp, 
       const int mat = u % NMAT;
       int sel = c.xk ? mat : 0;
       if (GROUPED) sel += (c.r0 + lrow >= g1 ? 1 : 0) + (c.r0 + lrow >= g2 ? 1 : 0);
-      const float dp = dot32_q4(R[u], reinterpret_cast<const u32x4_t*>(xs + sel * c.K + kofs * 32));
+      const float dp = dot32_q4<E>(R[u], reinterpret_cast<const u32x4_t*>(xs + sel * c.K + kofs * 32));
       const uint32_t sz = sztab[mat * szper + min(lrow, c.srows - 1) * c.ldg + (kofs >> c.gshift)];
       const float sc = (float)__builtin_bit_cast(_Float16, (unsigned short)(sz & 0xffffu));
       const float zz = (float)(int)(sz >> 16);
@@ -362,6 +367,7 @@ __device__ __forceinline__ float row_sum8(const float* cp, int row, int cpr) {
 // eight values of two neighbouring lanes (columns 0..3 and 4..7 of a group) are stored in the order the nibble masks
 // deliver the weights (columns 0,4 | 1,5 | 2,6 | 3,7) and the sum of every 32-column piece (8 lanes) is left in xsum,
 // added pairwise: columns, lane pairs, quads, halves.
+template <class E>
 __device__ __forceinline__ void stage_store_wide(uint16_t* xs, float* xsum, int q, uint32_t w0, uint32_t w1, bool q4) {
   uint2* xs64 = reinterpret_cast<uint2*>(xs);
   if (!q4) { xs64[q] = make_uint2(w0, w1); return; }
@@ -376,7 +382,7 @@ __device__ __forceinline__ void stage_store_wide(uint16_t* xs, float* xsum, int 
     out.y = (p1 >> 16) | (w1 & 0xffff0000u);
   }
   xs64[q] = out;                  // q and the lane have the same parity: words 0,1 of the group from the even lane, 2,3 from the odd
-  float s = (bf16_lo(w0) + bf16_hi(w0)) + (bf16_lo(w1) + bf16_hi(w1));
+  float s = (E::lo(w0) + E::hi(w0)) + (E::lo(w1) + E::hi(w1));
   s += dpp_f32<0xB1>(s);
   s += dpp_f32<0x4E>(s);
   s += dpp_f32<0x141>(s);
@@ -462,7 +468,7 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
           v[j].x = a0 | (a1 << 16);       // raw values; scaled once the sum is known
           v[j].y = a2 | (a3 << 16);
         } else {
-          stage_store_wide(xs, xsum, q, a0 | (a1 << 16), a2 | (a3 << 16), q4);
+          stage_store_wide<E>(xs, xsum, q, a0 | (a1 << 16), a2 | (a3 << 16), q4);
         }
       }
     }
@@ -480,7 +486,7 @@ __device__ __forceinline__ bool stage_input_wide(const void* in, int in_len, uin
         const int q = base + j * kT + tid;
         if (q < nw128) {
           const float f0 = E::lo(v[j].x), f1 = E::hi(v[j].x), f2 = E::lo(v[j].y), f3 = E::hi(v[j].y);
-          stage_store_wide(xs, xsum, q, E::pack2(E::lo(nwt[j].x) * E::rnd(f0 * rs), E::hi(nwt[j].x) * E::rnd(f1 * rs)),
+          stage_store_wide<E>(xs, xsum, q, E::pack2(E::lo(nwt[j].x) * E::rnd(f0 * rs), E::hi(nwt[j].x) * E::rnd(f1 * rs)),
                            E::pack2(E::lo(nwt[j].y) * E::rnd(f2 * rs), E::hi(nwt[j].y) * E::rnd(f3 * rs)), q4);
         }
       }
@@ -614,7 +620,7 @@ __device__ __forceinline__ void softmax_step(float sc, const u32x4_t& v, float& 
 // Addresses of the first window of the phase described by dv.  The loads themselves are issued at ONE
 // place in the kernel, straight into the window registers: a second issue site would make the compiler
 // merge two register sets, which it does by waiting for every load and copying.
-template <bool Q4>
+template <bool Q4, int QB>
 __device__ __forceinline__ void window_addresses(uint32_t dv, int w, int pos, uint64_t dummy, uint64_t (&addr)[kU], uint64_t (&addr_sz)[kSzLoads]) {
   const int type = DF_I(dv, type);
 #pragma unroll
@@ -623,7 +629,7 @@ __device__ __forceinline__ void window_addresses(uint32_t dv, int w, int pos, ui
   for (int j = 0; j < kSzLoads; ++j) addr_sz[j] = dummy;
   if (type == FSVD_PH_GEMV) {
     GemvCtx c;
-    gemv_ctx<Q4>(dv, w, c);
+    gemv_ctx<Q4, QB>(dv, w, c);
     if (c.nmat == 1) gemv_window_addr<1>(c, addr);
     else gemv_window_addr<2>(c, addr);
     if (Q4 && c.q4) gemv_sz_table_addr(c, addr_sz);
@@ -643,12 +649,13 @@ __device__ __forceinline__ void raise_error(fsvd_step_state* st, int p, int w) {
 
 // TRACE: workgroups 0, stride, 2*stride, ... record wall-clock ticks (100 MHz) per phase:
 // [0] phase entered, [1] input staged, [2] weights consumed, [3] epilogue done
-// Q4: the list may hold int4 GEMV phases (wbits == 4); the build without them keeps the bf16 walk free of their code
+// Q4: the list may hold int4 GEMV phases; the build without them keeps the 16-bit walk free of their code
 // CX: the list may hold the phases of the composed form (FSVD_PF_* flags, fp32 rows); likewise a build of its own
 template <bool TRACE, bool Q4, bool CX, int DT>
 __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __restrict__ phases, int nph, fsvd_step_state* st,
                                                          unsigned long long* trace, int trace_stride) {
   typedef E16<DT> E;
+  constexpr int QB = DT ? FSVD_WBITS_Q4_FP16 : 4;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw);
   float* cp = reinterpret_cast<float*>(smem_raw + (size_t)kMaxIn * 2);
@@ -691,11 +698,11 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
     // addresses of the next phase's first window, worked out now (behind the wait for this phase's input) so that the
     // request after publication is nothing but the loads
     uint64_t nxt[kU], nxt_sz[kSzLoads];
-    window_addresses<Q4>(dvB, w, pos, reinterpret_cast<uint64_t>(phases), nxt, nxt_sz);
+    window_addresses<Q4, QB>(dvB, w, pos, reinterpret_cast<uint64_t>(phases), nxt, nxt_sz);
 
     // ------------------------------------------------------------------ stage + stream
     if (CX && type == FSVD_PH_GEMV && (DF_I(dv, flags) & FSVD_PF_LEAD) != 0) {
-      gemv_ctx<false>(dv, w, gc);
+      gemv_ctx<false, 4>(dv, w, gc);
       // the epilogue of the previous phase may still be reading the partial buffer in another wave (its LDS reads are
       // complete by the time that wave's stores have been issued, i.e. before it arrives here)
       __builtin_amdgcn_s_barrier();
@@ -706,7 +713,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       type = -2;                           // no staging, no epilogue: on to the window request
     }
     if (type == FSVD_PH_GEMV) {
-      gemv_ctx<Q4>(dv, w, gc);
+      gemv_ctx<Q4, QB>(dv, w, gc);
       const int epi = DF_I(dv, epilogue);
       const int flags = CX ? DF_I(dv, flags) : 0;
       if (CX) rows0 = (flags & FSVD_PF_SPLIT) ? DF_I(dv, rows0) : (epi == FSVD_EP_F32 ? 0 : 0x7fffffff);
@@ -755,8 +762,8 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
 #pragma unroll
         for (int j = 0; j < kSzLoads; ++j) sztab[j * kT + tid] = SZ[j];
       }
-      // an int4 phase in the bf16 build, or a phase of the composed form in a build without it, is an error too
-      if (__syncthreads_or((ok && (Q4 || DF_I(dv, wbits) != 4) && (CX || (DF_I(dv, flags) == 0 && epi != FSVD_EP_F32))) ? 0 : 1)) {
+      // an int4 phase in a 16-bit build, or a phase of the composed form in a build without it, is an error too
+      if (__syncthreads_or((ok && (Q4 || DF_I(dv, wbits) != QB) && (CX || (DF_I(dv, flags) == 0 && epi != FSVD_EP_F32))) ? 0 : 1)) {
         raise_error(st, pm, w);
         return;
       }
@@ -765,11 +772,11 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
       if (Q4 && gc.q4) {
         if (gH > 0) {
           const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
-          gemv_stream_q4<1, true>(gc, m_kp, g1, g2, R, sztab, xs, xsum, cp);
+          gemv_stream_q4<E, 1, true>(gc, m_kp, g1, g2, R, sztab, xs, xsum, cp);
         } else if (gc.nmat == 1) {
-          gemv_stream_q4<1, false>(gc, m_kp, 0, 0, R, sztab, xs, xsum, cp);
+          gemv_stream_q4<E, 1, false>(gc, m_kp, 0, 0, R, sztab, xs, xsum, cp);
         } else {
-          gemv_stream_q4<2, false>(gc, m_kp, 0, 0, R, sztab, xs, xsum, cp);
+          gemv_stream_q4<E, 2, false>(gc, m_kp, 0, 0, R, sztab, xs, xsum, cp);
         }
       } else if (gH > 0) {
         const int g1 = gH * DF_I(dv, Dh), g2 = (gH + DF_I(dv, Hk)) * DF_I(dv, Dh);
@@ -927,7 +934,7 @@ __global__ __launch_bounds__(kT) void decode_step_kernel(const fsvd_phase* __res
         // the rows of the leading phase in front of this one: unrounded sums, taken by the lane groups from the top of the
         // workgroup down while those from the bottom up run this phase's epilogue
         GemvCtx fc;
-        gemv_ctx<false>(dvL, w, fc);
+        gemv_ctx<false, 4>(dvL, w, fc);
         const int t = kT / 8 - 1 - grp;
         if (t < fc.srows) {
           const float v = row_sum8(cp, t, fc.kp >> 4);
@@ -1090,11 +1097,12 @@ int decode_step_workgroups() {
     set_last_error("fsvd_decode_step: cannot query the device");
     return 0;
   }
-  const void* fns[10] = {reinterpret_cast<const void*>(decode_step_kernel<false, false, false, 0>), reinterpret_cast<const void*>(decode_step_kernel<true, false, false, 0>),
+  const void* fns[12] = {reinterpret_cast<const void*>(decode_step_kernel<false, false, false, 0>), reinterpret_cast<const void*>(decode_step_kernel<true, false, false, 0>),
                          reinterpret_cast<const void*>(decode_step_kernel<false, true, false, 0>), reinterpret_cast<const void*>(decode_step_kernel<true, true, false, 0>),
                          reinterpret_cast<const void*>(decode_step_kernel<false, false, true, 0>), reinterpret_cast<const void*>(decode_step_kernel<true, false, true, 0>),
                          reinterpret_cast<const void*>(decode_step_kernel<false, false, false, 1>), reinterpret_cast<const void*>(decode_step_kernel<true, false, false, 1>),
-                         reinterpret_cast<const void*>(decode_step_kernel<false, false, true, 1>), reinterpret_cast<const void*>(decode_step_kernel<true, false, true, 1>)};
+                         reinterpret_cast<const void*>(decode_step_kernel<false, false, true, 1>), reinterpret_cast<const void*>(decode_step_kernel<true, false, true, 1>),
+                         reinterpret_cast<const void*>(decode_step_kernel<false, true, false, 1>), reinterpret_cast<const void*>(decode_step_kernel<true, true, false, 1>)};
   for (const void* fn : fns) {
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSmemBytes) != hipSuccess) {
       set_last_error("fsvd_decode_step: the device refuses %zu bytes of dynamic LDS per workgroup", kSmemBytes);
@@ -1122,7 +1130,7 @@ int prepare_decode_step(fsvd_phase* ph, int nph, int nwg) {
     d.share_r = items % nwg;
     d.m_kp = 0;
     d.dk = 0;
-    const int pc = d.wbits == 4 ? 32 : 8;       // columns per 16-byte piece
+    const int pc = is_q4_bits(d.wbits) ? 32 : 8;   // columns per 16-byte piece
     if (d.type == FSVD_PH_GEMV && d.K >= pc) {
       d.m_kp = 0xffffffffu / (uint32_t)(d.K / pc) + 1u;
       d.dk = kT % (d.K / pc);
@@ -1145,14 +1153,14 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
     bool any_q4 = false, any_cx = false, any_f16 = false, any_b16 = false;
     for (int p = 0; p < nph; ++p) {
       if (ph[p].type != FSVD_PH_GEMV) continue;
-      any_q4 = any_q4 || ph[p].wbits == 4;
-      any_f16 = any_f16 || ph[p].wbits == FSVD_WBITS_FP16;
-      any_b16 = any_b16 || ph[p].wbits == 0 || ph[p].wbits == 16;
+      any_q4 = any_q4 || is_q4_bits(ph[p].wbits);
+      any_f16 = any_f16 || ph[p].wbits == FSVD_WBITS_FP16 || ph[p].wbits == FSVD_WBITS_Q4_FP16;
+      any_b16 = any_b16 || ph[p].wbits == 0 || ph[p].wbits == 16 || ph[p].wbits == 4;
       any_cx = any_cx || ph[p].flags != 0 || ph[p].epilogue == FSVD_EP_F32;
     }
     if (any_q4 && any_cx) return bad("a list holds int4 phases or phases of the composed form, not both (they run on different builds of the kernel)", 0);
     // the element type belongs to the step: its vectors, tables and caches are all of one 16-bit type
-    if (any_f16 && (any_b16 || any_q4)) return bad("a list is float16 in every GEMV phase or in none (int4 phases take bf16 activations)", 0);
+    if (any_f16 && any_b16) return bad("a list is float16 in every GEMV phase (FSVD_WBITS_FP16, FSVD_WBITS_Q4_FP16) or in none", 0);
   }
 
   // Every tagged buffer with the phase that wrote it last.  `full`: every workgroup wrote part of it in that phase (a
@@ -1185,7 +1193,7 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
       if (d.type == FSVD_PH_EMBED || d.type == FSVD_PH_GEMV) items = d.N;
       else if (d.type == FSVD_PH_MERGE) items = d.H * d.Dh;
       bool ok = d.share_q == items / nwg && d.share_r == items % nwg;
-      const int pc = d.wbits == 4 ? 32 : 8;
+      const int pc = is_q4_bits(d.wbits) ? 32 : 8;
       if (d.type == FSVD_PH_GEMV && d.K >= pc)
         ok = ok && d.m_kp == 0xffffffffu / (uint32_t)(d.K / pc) + 1u && d.dk == kT % (d.K / pc);
       if (!ok) return bad("derived fields missing: call fsvd_decode_step_prepare", p);
@@ -1198,8 +1206,9 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         break;
       case FSVD_PH_GEMV: {
         if (d.nmat < 1 || d.nmat > 2 || !d.W[0] || (d.nmat == 2 && !d.W[1])) return bad("GEMV needs 1 or 2 matrices", p);
-        if (d.wbits != 0 && d.wbits != 16 && d.wbits != 4 && d.wbits != FSVD_WBITS_FP16) return bad("wbits must be 0 / 16 (bf16), FSVD_WBITS_FP16 or 4", p);
-        const bool q4 = d.wbits == 4;
+        if (d.wbits != 0 && d.wbits != 16 && d.wbits != 4 && d.wbits != FSVD_WBITS_FP16 && d.wbits != FSVD_WBITS_Q4_FP16)
+          return bad("wbits must be 0 / 16 (bf16), 4 (int4 under bf16), FSVD_WBITS_FP16 or FSVD_WBITS_Q4_FP16", p);
+        const bool q4 = is_q4_bits(d.wbits);
         if (d.K <= 0 || d.K % (q4 ? 256 : 128) != 0) return bad(q4 ? "K must be a positive multiple of 256 for int4 weights" : "K must be a positive multiple of 128", p);
         if (q4) {
           if (!d.qsz[0] || (d.nmat == 2 && !d.qsz[1])) return bad("int4 GEMV needs the scale | zero words of every matrix", p);
@@ -1214,7 +1223,7 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
         const bool nowait = d.flags & FSVD_PF_NOWAIT, stage2 = d.flags & FSVD_PF_STAGE2, split = d.flags & FSVD_PF_SPLIT;
         const bool leading = d.flags & FSVD_PF_LEAD;
         const bool f32rows = split || d.epilogue == FSVD_EP_F32;
-        if ((d.flags != 0 || f32rows || d.in_off != 0) && q4) return bad("flags, fp32 rows and input offsets are for bf16 weights", p);
+        if ((d.flags != 0 || f32rows || d.in_off != 0) && q4) return bad("flags, fp32 rows and input offsets are for 16-bit weights", p);
         if (d.H > 0) {   // q | k | v row groups reading [Pq | Pk | Pv]
           if (d.nmat != 1 || d.epilogue != FSVD_EP_STORE || d.norm_w || split) return bad("grouped GEMV is a plain single-matrix store", p);
           if (d.Hk <= 0 || d.Dh <= 0 || d.N != (d.H + 2 * d.Hk) * d.Dh) return bad("grouped GEMV needs N = (H + 2*Hk) * Dh", p);
@@ -1235,7 +1244,7 @@ int validate_decode_step(const fsvd_phase* ph, int nph, int nwg) {
             if (((int64_t)(d.N / nwg) * (d.K / 8)) % (kT * kU) != 0) return bad("the slab of a leading phase must fill whole windows (rows per workgroup x K/8 a multiple of kT x kU)", p);
             if (p + 1 >= nph) return bad("a leading phase needs a phase behind it", p);
             const fsvd_phase& m = ph[p + 1];
-            if (m.type != FSVD_PH_GEMV || m.nmat != 1 || m.H > 0 || m.flags != 0 || m.wbits == 4 ||
+            if (m.type != FSVD_PH_GEMV || m.nmat != 1 || m.H > 0 || m.flags != 0 || is_q4_bits(m.wbits) ||
                 (m.epilogue != FSVD_EP_STORE && m.epilogue != FSVD_EP_RESID))
               return bad("the phase behind a leading phase must be a plain single-matrix bf16 GEMV that stores or adds a residual", p);
             if (d.in_off < gemv_in_len(m)) return bad("the staged input of a leading phase overlaps the input of the phase behind it", p);
@@ -1398,9 +1407,9 @@ int decode_step_build(const fsvd_phase* host, int nph) {
   int build = 0, f16 = 0;
   for (int p = 0; p < nph; ++p) {
     if (host[p].type != FSVD_PH_GEMV) continue;
-    if (host[p].wbits == 4) return 1;
-    if (host[p].wbits == FSVD_WBITS_FP16) f16 = 4;
-    if (host[p].flags != 0 || host[p].epilogue == FSVD_EP_F32) build = 2;
+    if (is_q4_bits(host[p].wbits)) build = 1;
+    if (host[p].wbits == FSVD_WBITS_FP16 || host[p].wbits == FSVD_WBITS_Q4_FP16) f16 = 4;
+    if (build != 1 && (host[p].flags != 0 || host[p].epilogue == FSVD_EP_F32)) build = 2;
   }
   return build + f16;
 }
@@ -1416,12 +1425,14 @@ int launch_decode_step(const fsvd_phase* dev, int nph, fsvd_step_state* st, unsi
     if (build == 1) FSVD_LAUNCH(true, true, false, 0);
     else if (build == 2) FSVD_LAUNCH(true, false, true, 0);
     else if (build == 4) FSVD_LAUNCH(true, false, false, 1);
+    else if (build == 5) FSVD_LAUNCH(true, true, false, 1);
     else if (build == 6) FSVD_LAUNCH(true, false, true, 1);
     else FSVD_LAUNCH(true, false, false, 0);
   } else {
     if (build == 1) FSVD_LAUNCH(false, true, false, 0);
     else if (build == 2) FSVD_LAUNCH(false, false, true, 0);
     else if (build == 4) FSVD_LAUNCH(false, false, false, 1);
+    else if (build == 5) FSVD_LAUNCH(false, true, false, 1);
     else if (build == 6) FSVD_LAUNCH(false, false, true, 1);
     else FSVD_LAUNCH(false, false, false, 0);
   }

@@ -196,10 +196,11 @@ struct Q4Args {
   const uint16_t* res; int64_t ldres;
   uint16_t* y; int64_t ldy;
   int B, N, K, nmat, mode;
+  int dt = 0;                                       // element type of x, bias, norm_w, res and y
 };
 int launch_linear_q4(const Q4Args& a, hipStream_t st);
 int launch_dequant_q4(const uint8_t* qw, int64_t ldq, const uint16_t* sc, const int16_t* zr, int64_t ldg, int group, uint16_t* w,
-                      int64_t ldw, int N, int K, hipStream_t st);
+                      int64_t ldw, int N, int K, int dt, hipStream_t st);
 int launch_qkv(const QkvArgs& a, int cfg, hipStream_t st);
 int launch_rmsnorm(const uint16_t* x, int64_t ldx, const uint16_t* w, float eps, uint16_t* y, int64_t ldy, int rows,
                    int K, int dt, hipStream_t st);

@@ -2,16 +2,17 @@
 //
 // Weights keep the layout of the quantised module (two columns per byte, even column in the low nibble;
 // fp16 scale and int16 zero point per group of columns), so a row of K columns is K/2 bytes: a quarter of
-// the bf16 stream.  The kernel must not spend the saved bytes on unpacking, so no weight is ever
-// converted to a float: OR-ing 0x4300 over a nibble n gives the bf16 bit pattern of 128 + n, and
-// V_DOT2_F32_BF16 multiplies two such weights with two bf16 activations straight from LDS.  With
-//     D_p = sum_k x_k * (128 + q_k)   over the 32 columns of a 16-byte piece p,
+// the 16-bit stream.  The kernel must not spend the saved bytes on unpacking, so no weight is ever
+// converted to a float: OR-ing 0x4300 over a nibble n gives the bf16 bit pattern of 128 + n (0x4c00 over n << 6: the
+// fp16 pattern of 16 + n), and V_DOT2_F32_{BF16,F16} multiplies two such weights with two activations of the same
+// type straight from LDS.  With c = 128 or 16,
+//     D_p = sum_k x_k * (c + q_k)     over the 32 columns of a 16-byte piece p,
 //     X_p = sum_k x_k                 (computed once per workgroup when x is staged),
-// the row is  y = sum_p s_g(p) * (D_p - (z_g(p) + 128) * X_p): two shift/mask operations and one dot per two
+// the row is  y = sum_p s_g(p) * (D_p - (z_g(p) + c) * X_p): two shift/mask operations and one dot per two
 // weights.  Activations are stored in LDS in the order the masks deliver the nibbles (columns 0,4 | 1,5 |
 // 2,6 | 3,7 of every eight).  Eight lanes share 256 columns of a row, fold their partial sums with DPP and
 // leave one value per 256 columns in LDS; a thread per output then adds the row's values in column order
-// (deterministic) and applies the epilogue of the bf16 kernels: bias, one rounding, residual, or SwiGLU.
+// (deterministic) and applies the epilogue of the 16-bit kernels: bias, one rounding, residual, or SwiGLU.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -32,6 +33,7 @@ __device__ __forceinline__ float row8_sum(float v) {
 }
 
 // 32 weights (four dwords of nibbles) against 32 activations in the permuted LDS order
+template <class E>
 __device__ __forceinline__ float dot32_q4(const u32x4_t& q, const u32x4_t* xs) {
   float acc = 0.f;
   const uint32_t qd[4] = {q.x, q.y, q.z, q.w};
@@ -39,16 +41,16 @@ __device__ __forceinline__ float dot32_q4(const u32x4_t& q, const u32x4_t* xs) {
   for (int j = 0; j < 4; ++j) {
     const u32x4_t xv = xs[j];
     const uint32_t d = qd[j];
-    acc = dot2_bf16((d & 0x000f000fu) | 0x43004300u, xv.x, acc);
-    acc = dot2_bf16(((d >> 4) & 0x000f000fu) | 0x43004300u, xv.y, acc);
-    acc = dot2_bf16(((d >> 8) & 0x000f000fu) | 0x43004300u, xv.z, acc);
-    acc = dot2_bf16(((d >> 12) & 0x000f000fu) | 0x43004300u, xv.w, acc);
+    acc = E::dot2(E::template nib<0>(d), xv.x, acc);
+    acc = E::dot2(E::template nib<4>(d), xv.y, acc);
+    acc = E::dot2(E::template nib<8>(d), xv.z, acc);
+    acc = E::dot2(E::template nib<12>(d), xv.w, acc);
   }
   return acc;
 }
 
 // NU pieces per thread of matrix m, starting at item i0: all loads first, then the products
-template <int BATCH, int NU>
+template <class E, int BATCH, int NU>
 __device__ __forceinline__ void q4_trip(const Q4Args& a, int m, int i0, int items, int r0, int PPR, int K, int nchunk,
                                         uint32_t ppr_magic, int gshift, const uint16_t* xs, const float* xsum, float* cp) {
   const int tid = threadIdx.x;
@@ -67,7 +69,7 @@ __device__ __forceinline__ void q4_trip(const Q4Args& a, int m, int i0, int item
     q[u] = __builtin_nontemporal_load((q4_gptr_t)(uintptr_t)(qw + n * a.ldq + (int64_t)piece[u] * 16));
     const int64_t gi = n * a.ldg + (piece[u] >> gshift);
     s[u] = half_bits_to_f32(sc[gi]);
-    zz[u] = (float)((int)zr[gi] + 128);
+    zz[u] = (float)((int)zr[gi] + E::nib_off);
   }
 #pragma unroll
   for (int u = 0; u < NU; ++u) {
@@ -75,7 +77,7 @@ __device__ __forceinline__ void q4_trip(const Q4Args& a, int m, int i0, int item
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
       const size_t xo = (size_t)m * BATCH + b;
-      const float d = dot32_q4(q[u], reinterpret_cast<const u32x4_t*>(xs + xo * K + (size_t)piece[u] * 32));
+      const float d = dot32_q4<E>(q[u], reinterpret_cast<const u32x4_t*>(xs + xo * K + (size_t)piece[u] * 32));
       const float part = row8_sum(s[u] * (d - zz[u] * xsum[xo * PPR + piece[u]]));
       if ((tid & 7) == 0 && i < items) cp[xo * nchunk + (i >> 3)] = part;
     }
@@ -83,15 +85,16 @@ __device__ __forceinline__ void q4_trip(const Q4Args& a, int m, int i0, int item
 }
 
 // BATCH activation rows, NMAT = 1 (linear) or 2 (gate and up of the SwiGLU, each with its own input)
-template <int BATCH, int NMAT>
+template <int DT, int BATCH, int NMAT>
 __global__ __launch_bounds__(kQT) void q4_linear_kernel(Q4Args a, int rows_per_wg, uint32_t ppr_magic, int gshift) {
+  typedef E16<DT> E;
   extern __shared__ __align__(16) unsigned char q4_smem[];
   const int tid = threadIdx.x;
   const int K = a.K, PPR = K >> 5, CPR = PPR >> 3;
   const int r0 = blockIdx.x * rows_per_wg;
   const int nrows = min(rows_per_wg, a.N - r0);
   if (nrows <= 0) return;
-  // LDS: activations (permuted bf16), piece sums, chunk partials, reduction scratch
+  // LDS: activations (permuted), piece sums, chunk partials, reduction scratch
   uint16_t* xs = reinterpret_cast<uint16_t*>(q4_smem);                          // [NMAT][BATCH][K]
   float* xsum = reinterpret_cast<float*>(xs + (size_t)NMAT * BATCH * K);         // [NMAT][BATCH][PPR]
   float* cp = xsum + (size_t)NMAT * BATCH * PPR;                                // [NMAT][BATCH][rows_per_wg * CPR]
@@ -108,12 +111,12 @@ __global__ __launch_bounds__(kQT) void q4_linear_kernel(Q4Args a, int rows_per_w
       }
       const uint16_t* src = a.x + (int64_t)b * a.ldx + (m ? a.up_off : 0);
       float rs = 0.f;
-      if (a.norm_w) {   // RMSNorm: w * bf16(x * rsqrt(mean(x^2) + eps)), sum in fp32
+      if (a.norm_w) {   // RMSNorm: w * round(x * rsqrt(mean(x^2) + eps)), sum in fp32
         float ss = 0.f;
         for (int k = tid * 8; k < K; k += kQT * 8) {
           const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + k);
-          const float a0 = bf16_lo(v.x), a1 = bf16_hi(v.x), a2 = bf16_lo(v.y), a3 = bf16_hi(v.y);
-          const float a4 = bf16_lo(v.z), a5 = bf16_hi(v.z), a6 = bf16_lo(v.w), a7 = bf16_hi(v.w);
+          const float a0 = E::lo(v.x), a1 = E::hi(v.x), a2 = E::lo(v.y), a3 = E::hi(v.y);
+          const float a4 = E::lo(v.z), a5 = E::hi(v.z), a6 = E::lo(v.w), a7 = E::hi(v.w);
           ss += ((a0 * a0 + a1 * a1) + (a2 * a2 + a3 * a3)) + ((a4 * a4 + a5 * a5) + (a6 * a6 + a7 * a7));
         }
         ss = wave_sum(ss);
@@ -129,10 +132,10 @@ __global__ __launch_bounds__(kQT) void q4_linear_kernel(Q4Args a, int rows_per_w
         u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + k);
         if (a.norm_w) {
           const u32x4_t g = *reinterpret_cast<const u32x4_t*>(a.norm_w + k);
-          v.x = pack_bf16x2(bf16_lo(g.x) * round_bf16(bf16_lo(v.x) * rs), bf16_hi(g.x) * round_bf16(bf16_hi(v.x) * rs));
-          v.y = pack_bf16x2(bf16_lo(g.y) * round_bf16(bf16_lo(v.y) * rs), bf16_hi(g.y) * round_bf16(bf16_hi(v.y) * rs));
-          v.z = pack_bf16x2(bf16_lo(g.z) * round_bf16(bf16_lo(v.z) * rs), bf16_hi(g.z) * round_bf16(bf16_hi(v.z) * rs));
-          v.w = pack_bf16x2(bf16_lo(g.w) * round_bf16(bf16_lo(v.w) * rs), bf16_hi(g.w) * round_bf16(bf16_hi(v.w) * rs));
+          v.x = E::pack2(E::lo(g.x) * E::rnd(E::lo(v.x) * rs), E::hi(g.x) * E::rnd(E::hi(v.x) * rs));
+          v.y = E::pack2(E::lo(g.y) * E::rnd(E::lo(v.y) * rs), E::hi(g.y) * E::rnd(E::hi(v.y) * rs));
+          v.z = E::pack2(E::lo(g.z) * E::rnd(E::lo(v.z) * rs), E::hi(g.z) * E::rnd(E::hi(v.z) * rs));
+          v.w = E::pack2(E::lo(g.w) * E::rnd(E::lo(v.w) * rs), E::hi(g.w) * E::rnd(E::hi(v.w) * rs));
         }
         // columns (0,1)(2,3)(4,5)(6,7) -> (0,4)(1,5)(2,6)(3,7)
         u32x4_t o;
@@ -151,10 +154,10 @@ __global__ __launch_bounds__(kQT) void q4_linear_kernel(Q4Args a, int rows_per_w
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const u32x4_t v = p[j];
-      s = dot2_bf16(0x3f803f80u, v.x, s);
-      s = dot2_bf16(0x3f803f80u, v.y, s);
-      s = dot2_bf16(0x3f803f80u, v.z, s);
-      s = dot2_bf16(0x3f803f80u, v.w, s);
+      s = E::dot2(E::one2, v.x, s);
+      s = E::dot2(E::one2, v.y, s);
+      s = E::dot2(E::one2, v.z, s);
+      s = E::dot2(E::one2, v.w, s);
     }
     xsum[o] = s;
   }
@@ -166,9 +169,9 @@ __global__ __launch_bounds__(kQT) void q4_linear_kernel(Q4Args a, int rows_per_w
   for (int m = 0; m < NMAT; ++m) {
     int i0 = 0;
     for (; i0 + kQT * kQUnroll <= items; i0 += kQT * kQUnroll)     // full trips: kQUnroll pieces in flight per thread
-      q4_trip<BATCH, kQUnroll>(a, m, i0, items, r0, PPR, K, nchunk, ppr_magic, gshift, xs, xsum, cp);
+      q4_trip<E, BATCH, kQUnroll>(a, m, i0, items, r0, PPR, K, nchunk, ppr_magic, gshift, xs, xsum, cp);
     for (; i0 < items; i0 += kQT)                                  // tail: one piece per thread
-      q4_trip<BATCH, 1>(a, m, i0, items, r0, PPR, K, nchunk, ppr_magic, gshift, xs, xsum, cp);
+      q4_trip<E, BATCH, 1>(a, m, i0, items, r0, PPR, K, nchunk, ppr_magic, gshift, xs, xsum, cp);
   }
   __syncthreads();
 
@@ -188,25 +191,27 @@ __global__ __launch_bounds__(kQT) void q4_linear_kernel(Q4Args a, int rows_per_w
     float out;
     if (NMAT == 2) {
       if (a.mode == 0) {
-        const float g = round_bf16(v[0]), up = round_bf16(v[NMAT - 1]);
-        out = round_bf16(round_bf16(silu_f32(g)) * up);
+        const float g = E::rnd(v[0]), up = E::rnd(v[NMAT - 1]);
+        out = E::rnd(E::rnd(silu_f32(g)) * up);
       } else {
-        out = round_bf16((v[0] * (1.0f / (1.0f + expf(-v[0])))) * v[NMAT - 1]);
+        out = E::rnd((v[0] * (1.0f / (1.0f + expf(-v[0])))) * v[NMAT - 1]);
       }
     } else {
       float t = v[0];
-      if (a.bias) t += bf16_bits_to_f32(a.bias[n]);
-      out = round_bf16(t);
-      if (a.res) out = round_bf16(bf16_bits_to_f32(a.res[(int64_t)b * a.ldres + n]) + out);
+      if (a.bias) t += E::val(a.bias[n]);
+      out = E::rnd(t);
+      if (a.res) out = E::rnd(E::val(a.res[(int64_t)b * a.ldres + n]) + out);
     }
-    a.y[(int64_t)b * a.ldy + n] = (uint16_t)f32_to_bf16_bits(out);
+    a.y[(int64_t)b * a.ldy + n] = (uint16_t)E::bits(out);
   }
 }
 
-// w[n, k] = bf16(s * (q - z)): the dense form of a quantised matrix (prefill runs on the matrix cores from it)
+// w[n, k] = round(s * (q - z)): the dense form of a quantised matrix (prefill runs on the matrix cores from it)
+template <int DT>
 __global__ __launch_bounds__(256) void q4_dequant_kernel(const uint8_t* __restrict__ qw, int64_t ldq, const uint16_t* __restrict__ sc,
                                                          const int16_t* __restrict__ zr, int64_t ldg, int group, uint16_t* __restrict__ w,
                                                          int64_t ldw, int N, int K) {
+  typedef E16<DT> E;
   const int64_t bytes_per_row = (K + 1) / 2;
   const int64_t total = (int64_t)N * bytes_per_row;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
@@ -214,20 +219,22 @@ __global__ __launch_bounds__(256) void q4_dequant_kernel(const uint8_t* __restri
     const int k = (int)(i - n * bytes_per_row) * 2;
     const uint32_t byte = qw[n * ldq + (k >> 1)];
     const int g0 = group > 0 ? k / group : 0, g1 = group > 0 ? (k + 1) / group : 0;
-    w[n * ldw + k] = (uint16_t)f32_to_bf16_bits(half_bits_to_f32(sc[n * ldg + g0]) * ((float)(int)(byte & 15u) - (float)zr[n * ldg + g0]));
+    w[n * ldw + k] = (uint16_t)E::bits(half_bits_to_f32(sc[n * ldg + g0]) * ((float)(int)(byte & 15u) - (float)zr[n * ldg + g0]));
     if (k + 1 < K)
-      w[n * ldw + k + 1] = (uint16_t)f32_to_bf16_bits(half_bits_to_f32(sc[n * ldg + g1]) * ((float)(int)(byte >> 4) - (float)zr[n * ldg + g1]));
+      w[n * ldw + k + 1] = (uint16_t)E::bits(half_bits_to_f32(sc[n * ldg + g1]) * ((float)(int)(byte >> 4) - (float)zr[n * ldg + g1]));
   }
 }
 
 int launch_dequant_q4(const uint8_t* qw, int64_t ldq, const uint16_t* sc, const int16_t* zr, int64_t ldg, int group, uint16_t* w,
-                      int64_t ldw, int N, int K, hipStream_t st) {
+                      int64_t ldw, int N, int K, int dt, hipStream_t st) {
+  if (dt != 0 && dt != 1) { set_last_error("fsvd_dequant_q4: dtype %d is neither bf16 (0) nor fp16 (1)", dt); return kErrBadDtype; }
   if (N <= 0 || K <= 0 || ldq < (K + 1) / 2 || ldw < K) { set_last_error("fsvd_dequant_q4: bad shape"); return kErrBadShape; }
   const int g = (group <= 0 || group >= K) ? 0 : group;
   if (g && ldg < (K + g - 1) / g) { set_last_error("fsvd_dequant_q4: scale rows shorter than the group count"); return kErrBadShape; }
   const int64_t total = (int64_t)N * ((K + 1) / 2);
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
-  hipLaunchKernelGGL(q4_dequant_kernel, dim3(blocks), dim3(256), 0, st, qw, ldq, sc, zr, ldg, g, w, ldw, N, K);
+  if (dt == 1) hipLaunchKernelGGL(q4_dequant_kernel<1>, dim3(blocks), dim3(256), 0, st, qw, ldq, sc, zr, ldg, g, w, ldw, N, K);
+  else hipLaunchKernelGGL(q4_dequant_kernel<0>, dim3(blocks), dim3(256), 0, st, qw, ldq, sc, zr, ldg, g, w, ldw, N, K);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("fsvd_dequant_q4: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
@@ -240,24 +247,35 @@ size_t q4_lds_bytes(int batch, int nmat, int K, int rows_per_wg) {
   return (size_t)nmat * batch * K * 2 + (size_t)nmat * batch * ppr * 4 + (size_t)nmat * batch * rows_per_wg * cpr * 4 + 8 * 4;
 }
 
-template <int BATCH, int NMAT>
+template <int DT, int BATCH, int NMAT>
 static int launch_q4_t(const Q4Args& a, int rows_per_wg, uint32_t magic, int gshift, size_t lds, hipStream_t st) {
   static size_t granted = 64 * 1024;   // dynamic LDS a kernel may use without asking
   if (lds > granted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&q4_linear_kernel<BATCH, NMAT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&q4_linear_kernel<DT, BATCH, NMAT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_last_error("fsvd_linear_q4: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return kErrLaunch; }
     granted = lds;
   }
   const int nwg = (a.N + rows_per_wg - 1) / rows_per_wg;
-  hipLaunchKernelGGL((q4_linear_kernel<BATCH, NMAT>), dim3(nwg), dim3(kQT), lds, st, a, rows_per_wg, magic, gshift);
+  hipLaunchKernelGGL((q4_linear_kernel<DT, BATCH, NMAT>), dim3(nwg), dim3(kQT), lds, st, a, rows_per_wg, magic, gshift);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_last_error("fsvd_linear_q4: launch failed: %s", hipGetErrorString(e)); return kErrLaunch; }
   return kOk;
 }
 
+template <int DT>
+static int launch_q4_batch(const Q4Args& a, int batch, int rows, uint32_t magic, int gshift, size_t lds, hipStream_t st) {
+  if (a.nmat == 1) return batch == 1 ? launch_q4_t<DT, 1, 1>(a, rows, magic, gshift, lds, st)
+                        : batch == 2 ? launch_q4_t<DT, 2, 1>(a, rows, magic, gshift, lds, st)
+                                     : launch_q4_t<DT, 4, 1>(a, rows, magic, gshift, lds, st);
+  return batch == 1 ? launch_q4_t<DT, 1, 2>(a, rows, magic, gshift, lds, st)
+       : batch == 2 ? launch_q4_t<DT, 2, 2>(a, rows, magic, gshift, lds, st)
+                    : launch_q4_t<DT, 4, 2>(a, rows, magic, gshift, lds, st);
+}
+
 int launch_linear_q4(const Q4Args& a0, hipStream_t st) {
   const char* fn = a0.nmat == 2 ? "fsvd_swiglu_linear_q4" : "fsvd_linear_q4";
+  if (a0.dt != 0 && a0.dt != 1) { set_last_error("%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, a0.dt); return kErrBadDtype; }
   if (a0.B <= 0 || a0.N <= 0 || a0.K <= 0 || (a0.nmat != 1 && a0.nmat != 2)) { set_last_error("%s: empty problem", fn); return kErrBadShape; }
   if (a0.K % 256) { set_last_error("%s: K = %d is not a multiple of 256 (pad the factor)", fn, a0.K); return kErrBadShape; }
   int gshift;
@@ -291,13 +309,8 @@ int launch_linear_q4(const Q4Args& a0, hipStream_t st) {
     const int batch = a.B == 1 ? 1 : (a.B == 2 ? 2 : 4);
     const size_t lds = q4_lds_bytes(batch, a.nmat, a.K, rows);
     if (lds > 160 * 1024) { set_last_error("%s: K = %d with %d rows needs %zu bytes of LDS", fn, a.K, a.B, lds); return kErrBadShape; }
-    int rc;
-    if (a.nmat == 1) rc = batch == 1 ? launch_q4_t<1, 1>(a, rows, magic, gshift, lds, st)
-                        : batch == 2 ? launch_q4_t<2, 1>(a, rows, magic, gshift, lds, st)
-                                     : launch_q4_t<4, 1>(a, rows, magic, gshift, lds, st);
-    else rc = batch == 1 ? launch_q4_t<1, 2>(a, rows, magic, gshift, lds, st)
-            : batch == 2 ? launch_q4_t<2, 2>(a, rows, magic, gshift, lds, st)
-                         : launch_q4_t<4, 2>(a, rows, magic, gshift, lds, st);
+    const int rc = a.dt == 1 ? launch_q4_batch<1>(a, batch, rows, magic, gshift, lds, st)
+                             : launch_q4_batch<0>(a, batch, rows, magic, gshift, lds, st);
     if (rc != kOk) return rc;
   }
   return kOk;

@@ -248,31 +248,32 @@ def linear_q4(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, zero
               bias: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
               residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = (residual +) linear(rmsnorm?(x), s * (q - z), bias) on group-wise int4 weights [N, K/2] bytes."""
-    _need(x, "x")
+    dt, code = _elem(x, "x")
     N, K = qweight.shape[0], x.shape[-1]
     group = _q4_check(qweight, scales, zeros, N, K, group_size, "linear_q4")
     x2 = _rows(x, "x")
     B = x2.shape[0]
     if out is None:
-        out = torch.empty(*x.shape[:-1], N, device=x.device, dtype=_BF16)
+        out = torch.empty(*x.shape[:-1], N, device=x.device, dtype=dt)
+    _need(out, "out", dtype=dt)
     o2 = out if out.dim() == 2 else _rows(out, "out")
     if o2.shape != (B, N) or o2.stride(1) != 1:
         raise ValueError("out must be a [rows, N] tensor with unit inner stride matching x")
     r2 = None
     if residual is not None:
-        _need(residual, "residual")
+        _need(residual, "residual", dtype=dt)
         r2 = _rows(residual, "residual")
         if r2.shape != (B, N):
             raise ValueError(f"residual shape {tuple(residual.shape)} does not match output [{B}, {N}]")
     for t, nm, n in ((bias, "bias", N), (norm_weight, "norm_weight", K)):
         if t is not None:
-            _need(t, nm)
+            _need(t, nm, dtype=dt)
             if t.shape != (n,) or not t.is_contiguous():
                 raise ValueError(f"{nm} must be a contiguous [{n}] tensor")
     lib = _lib.load()
     rc = lib.fsvd_linear_q4(x2.data_ptr(), x2.stride(0), qweight.data_ptr(), qweight.stride(0), scales.data_ptr(), zeros.data_ptr(),
                             scales.stride(0), group, _ptr(bias), _ptr(norm_weight), float(eps), _ptr(r2),
-                            0 if r2 is None else r2.stride(0), o2.data_ptr(), o2.stride(0), B, N, K, _stream())
+                            0 if r2 is None else r2.stride(0), o2.data_ptr(), o2.stride(0), B, N, K, code, _stream())
     _lib.check("fsvd_linear_q4", rc)
     return out
 
@@ -280,7 +281,7 @@ def linear_q4(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, zero
 def swiglu_linear_q4(p: torch.Tensor, gate: tuple, up: tuple, *, up_off: int, group_size: int, mode: int = 0,
                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """h = silu(p[..., :R] @ Wg.T) * (p[..., up_off:up_off+R] @ Wu.T); gate / up are (qweight, scales, zeros) of [D, R]."""
-    _need(p, "p")
+    dt, code = _elem(p, "p")
     (gq, gs, gz), (uq, us, uz) = gate, up
     D = gq.shape[0]
     R = 2 * gq.shape[1]
@@ -293,28 +294,30 @@ def swiglu_linear_q4(p: torch.Tensor, gate: tuple, up: tuple, *, up_off: int, gr
         raise ValueError("gate and up must share one layout")
     B = p2.shape[0]
     if out is None:
-        out = torch.empty(*p.shape[:-1], D, device=p.device, dtype=_BF16)
+        out = torch.empty(*p.shape[:-1], D, device=p.device, dtype=dt)
+    _need(out, "out", dtype=dt)
     o2 = _rows(out, "out")
     lib = _lib.load()
     rc = lib.fsvd_swiglu_linear_q4(p2.data_ptr(), p2.stride(0), int(up_off), gq.data_ptr(), gs.data_ptr(), gz.data_ptr(),
                                    uq.data_ptr(), us.data_ptr(), uz.data_ptr(), gq.stride(0), gs.stride(0), group,
-                                   o2.data_ptr(), o2.stride(0), B, D, R, int(mode), _stream())
+                                   o2.data_ptr(), o2.stride(0), B, D, R, int(mode), code, _stream())
     _lib.check("fsvd_swiglu_linear_q4", rc)
     return out
 
 
 def dequant_q4(qweight: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor, *, in_features: int, group_size: int,
-               out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """bf16 [N, K] = s * (q - z)."""
+               out: Optional[torch.Tensor] = None, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """[N, K] = s * (q - z), rounded once to ``dtype`` (bf16 or fp16; the type of ``out`` when that is given, else bf16)."""
     N, K = qweight.shape[0], int(in_features)
     group = _q4_check(qweight, scales, zeros, N, K, group_size, "dequant_q4")
     if out is None:
-        out = torch.empty(N, K, device=qweight.device, dtype=_BF16)
-    elif out.shape != (N, K) or out.dtype != _BF16 or out.stride(1) != 1:
-        raise ValueError(f"out must be a bf16 [{N}, {K}] tensor with unit inner stride")
+        out = torch.empty(N, K, device=qweight.device, dtype=dtype or _BF16)
+    dt, code = _elem(out, "out")
+    if out.shape != (N, K) or (dtype is not None and dt != dtype) or out.stride(1) != 1:
+        raise ValueError(f"out must be a {dtype or 'bf16 / fp16'} [{N}, {K}] tensor with unit inner stride")
     lib = _lib.load()
     rc = lib.fsvd_dequant_q4(qweight.data_ptr(), qweight.stride(0), scales.data_ptr(), zeros.data_ptr(), scales.stride(0), group,
-                             out.data_ptr(), out.stride(0), N, K, _stream())
+                             out.data_ptr(), out.stride(0), N, K, code, _stream())
     _lib.check("fsvd_dequant_q4", rc)
     return out
 

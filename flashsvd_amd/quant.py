@@ -5,13 +5,15 @@ same name (src/quant/packed_quant_linear.py:47-172: ``qweight`` uint8 with two i
 fp16 and ``zeros`` int16 per group of input columns, optional ``bias``), so a checkpoint written by the reference's
 quantisation scripts loads as it is.  On the GPU a 4-bit module runs on the packed bytes:
 
-* up to ``GEMV_ROWS`` activation rows (decode): ``fsvd_linear_q4`` streams the int4 rows, a quarter of the bf16 bytes;
-* more rows (prefill): the weight is expanded to bf16 by ``fsvd_dequant_q4`` into a scratch matrix that lives for the
-  call, and the matrix-core projection runs on it.
+* up to ``GEMV_ROWS`` activation rows (decode): ``fsvd_linear_q4`` streams the int4 rows, a quarter of the 16-bit bytes;
+* more rows (prefill): the weight is expanded to the activation type by ``fsvd_dequant_q4`` into a scratch matrix that
+  lives for the call, and the matrix-core projection runs on it.
+
+Activations are bf16 or fp16; the module computes in the type of its input.
 
 ``FLASH_SVD_QUANT_BACKEND`` (the reference's switch, :174-213) picks ``auto`` (the rule above), ``quant`` / ``int4`` /
 ``packed`` (always the int4 stream) or ``dense`` / ``cached_dense`` / ``fp16`` / ``dequant_cache`` (expand once, keep the
-bf16 matrix, run every call on it).  8-bit modules always take the dense route.  Quantising (``pack_weight``) is
+16-bit matrix, run every call on it).  8-bit modules always take the dense route.  Quantising (``pack_weight``) is
 offline preparation and runs in torch on whatever device the weight is on.
 
 ``replace_linears_with_packed_quant_inplace`` and ``extract_flashsvd_rank_map`` follow src/quant/common.py:80-149.
@@ -107,14 +109,14 @@ class PackedQuantLinear(nn.Module):
 
     # ---- dense form --------------------------------------------------------------------------------------
     def dequantize(self, *, dtype: Optional[torch.dtype] = None, device=None) -> torch.Tensor:
-        """scale * (q - zero), rounded once to ``dtype``.  4-bit buffers on the GPU with a bf16 result go through the
-        HIP expansion kernel; everything else is tensor arithmetic (tests, CPU tools)."""
+        """scale * (q - zero), rounded once to ``dtype``.  4-bit buffers on the GPU with a bf16 or fp16 result go through
+        the HIP expansion kernel; everything else is tensor arithmetic (tests, CPU tools)."""
         dtype = dtype or self.compute_dtype
         device = torch.device(device) if device is not None else self.qweight.device
-        if self.bits == 4 and dtype == torch.bfloat16 and device.type == "cuda" and self.qweight.is_cuda:
+        if self.bits == 4 and dtype in (torch.bfloat16, torch.float16) and device.type == "cuda" and self.qweight.is_cuda:
             from . import hip_ops
             return hip_ops.dequant_q4(self.qweight, self.scales, self.zeros, in_features=self.in_features,
-                                      group_size=self.group_size)
+                                      group_size=self.group_size, dtype=dtype)
         q = (unpack_int4(self.qweight, self.in_features) if self.bits == 4 else self.qweight).to(device=device, dtype=torch.float32)
         scales = self.scales.to(device=device, dtype=torch.float32)
         zeros = self.zeros.to(device=device, dtype=torch.float32)
@@ -137,10 +139,10 @@ class PackedQuantLinear(nn.Module):
             return "auto"
         raise ValueError(f"FLASH_SVD_QUANT_BACKEND={mode!r}: expected auto, quant or dense (there is no path without the GPU kernels)")
 
-    def _cached_dense(self) -> torch.Tensor:
-        key = (self.qweight.data_ptr(), self.scales.data_ptr(), self.qweight.device)
+    def _cached_dense(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+        key = (self.qweight.data_ptr(), self.scales.data_ptr(), self.qweight.device, dtype)
         if self._dense is None or self._dense[0] != key:
-            self._dense = (key, self.dequantize(dtype=torch.bfloat16))
+            self._dense = (key, self.dequantize(dtype=dtype))
         return self._dense[1]
 
     def streams_int4(self, rows: int) -> bool:
@@ -155,16 +157,20 @@ class PackedQuantLinear(nn.Module):
 
     def run(self, x: torch.Tensor, *, norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
             residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """The projection with the fused prologue / epilogue of the bf16 kernels."""
+        """The projection with the fused prologue / epilogue of the 16-bit kernels, in the type of ``x`` (bf16 or fp16)."""
         from . import hip_ops
         if not x.is_cuda:
             raise RuntimeError("PackedQuantLinear runs on the GPU kernels only; use dequantize() for CPU-side inspection")
         rows = x.numel() // max(1, x.shape[-1])
         if self.streams_int4(rows):
-            return hip_ops.linear_q4(x, self.qweight, self.scales, self.zeros, group_size=self.group_size, bias=self.bias,
+            bias = self.bias if self.bias is None or self.bias.dtype == x.dtype else self.bias.to(x.dtype)
+            return hip_ops.linear_q4(x, self.qweight, self.scales, self.zeros, group_size=self.group_size, bias=bias,
                                      norm_weight=norm_weight, eps=eps, residual=residual, out=out)
-        w = self._cached_dense() if self._backend() == "dense" else self.dequantize(dtype=torch.bfloat16)
-        return hip_ops.linear(x, w, self.bias, norm_weight=norm_weight, eps=eps, residual=residual, out=out)
+        if x.dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError(f"PackedQuantLinear computes in bfloat16 or float16, got {x.dtype}")
+        w = self._cached_dense(x.dtype) if self._backend() == "dense" else self.dequantize(dtype=x.dtype)
+        bias = self.bias if self.bias is None or self.bias.dtype == x.dtype else self.bias.to(x.dtype)
+        return hip_ops.linear(x, w, bias, norm_weight=norm_weight, eps=eps, residual=residual, out=out)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.run(x)

@@ -36,7 +36,7 @@ def _tb(t: torch.Tensor, uses: int, use: int) -> TagBuf:
 class PersistentDecoder:
     """``PersistentDecoder(model, cache)`` then ``set_state(token, position)``, ``step(n)``, ``tokens()``.
 
-    Requirements (checked): batch 1, one 16-bit type throughout (bfloat16, or float16 for a model without int4 factors;
+    Requirements (checked): batch 1, one 16-bit type throughout (bfloat16 or float16;
     weights, norms, embedding and cache alike), dense KV cache, head_dim 128, hidden and intermediate sizes that are
     multiples of 128, and a device whose compute-unit count is a multiple of the number of heads.  Factor ranks are free
     for 16-bit factors (unequal q / k / v ranks, ranks that are not multiples of 128 or smaller than the workgroup count are served
@@ -65,8 +65,8 @@ class PersistentDecoder:
         inner = model.model
         cfg = model.config
         dev = model.lm_head.weight.device
-        # one 16-bit element type for the whole step, named by the lm_head: bfloat16, or float16 (a model without int4
-        # factors).  The kernel reinterprets every buffer it is pointed at as bits of that type (int4 factors aside):
+        # one 16-bit element type for the whole step, named by the lm_head: bfloat16 or float16.
+        # The kernel reinterprets every buffer it is pointed at as bits of that type (int4 factors aside):
         # anything else is refused here, so that the driver falls back to the per-operator engine instead of decoding garbage
         edt = model.lm_head.weight.dtype
         if edt not in (torch.bfloat16, torch.float16):
@@ -120,8 +120,6 @@ class PersistentDecoder:
                 if gs < m.in_features and (gs < 32 or gs & (gs - 1)):
                     raise ValueError(f"PersistentDecoder: int4 group size {gs} is not a power of two >= 32")
             layer_q4.append(True)
-        if any(layer_q4) and edt != torch.bfloat16:
-            raise ValueError("PersistentDecoder: int4 factors take bfloat16 activations; the model is float16")
         # Ranks may differ from layer to layer and, for bf16 factors, between q, k and v: the kernel wants one rank per
         # row group, a multiple of 128 (a lane group covers 128 elements of a row) and at least one row per workgroup,
         # so factors that do not fit are copied once into zero-padded twins (zero rows / columns contribute nothing:
@@ -166,15 +164,17 @@ class PersistentDecoder:
         names: list[str] = []
 
         def sz_words(scales, zeros):
-            """uint32 [N, G]: fp16 scale bits in the low half, zero point + 128 in the high half (what a piece needs in one load)."""
+            """uint32 [N, G]: fp16 scale bits in the low half, zero point + c in the high half (what a piece needs in one
+            load); c = 128 in a bf16 step, 16 in a float16 one: the value a nibble's bit pattern is offset by."""
             if scales.dtype != torch.float16:
                 raise ValueError(f"int4 scales must be float16, got {scales.dtype}")
+            c = 16 if edt == torch.float16 else 128
             zmin, zmax = int(zeros.min()), int(zeros.max())
-            if zmin < -128 or zmax > 65535 - 128:
+            if zmin < -c or zmax > 65535 - c:
                 raise ValueError(f"int4 zero points {zmin}..{zmax} do not fit the unsigned 16-bit field of the packed "
-                                 "scale | zero word (zero + 128)")
+                                 f"scale | zero word (zero + {c})")
             lo = scales.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
-            hi = (zeros.to(torch.int32) + 128) << 16
+            hi = (zeros.to(torch.int32) + c) << 16
             return (lo | hi).contiguous()
 
         def pad_rows(w, n):       # zero rows below: outputs that are zero
@@ -197,7 +197,7 @@ class PersistentDecoder:
                 p.H, p.Hk, p.Dh = groups
             if q4 is not None:              # W holds (qweight, scales, zeros) triples; q4 = group size
                 gs = min(int(q4), K)
-                p.wbits, p.gshift = 4, int(math.log2(gs // 32))
+                p.wbits, p.gshift = (_lib.WBITS_Q4_FP16 if edt == torch.float16 else 4), int(math.log2(gs // 32))
                 for i, (qw, sc, zr) in enumerate(W):
                     G = (K + gs - 1) // gs
                     if tuple(qw.shape) != (N, K // 2) or not qw.is_contiguous() or tuple(sc.shape) != (N, G) or tuple(zr.shape) != (N, G):

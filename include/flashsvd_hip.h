@@ -58,8 +58,8 @@ int fsvd_set_workspace(void* ws, size_t bytes, void* stream);
  * same way (kernels/attn/decode/densekv_reconstruct_triton.py:427-428; fp16 is the default of its dense cache,
  * runtime/cache/attn_dense_kv.py:26, and the fallback of scripts/demo_support/api.py:161-165).  So does the rank-space
  * decode attention (fsvd_attn_decode_rankkv; fsvd_rankkv_append copies 16-bit patterns of either type).  The
- * persistent decode step takes its type from its phase list (FSVD_WBITS_FP16); the int4 entries and int4 phases take
- * bf16 activations only. */
+ * persistent decode step takes its type from its phase list (FSVD_WBITS_FP16, FSVD_WBITS_Q4_FP16); the int4 entries
+ * take activations of either type. */
 
 /* y[b,n] = (res[b,n] +) bf16( W[n,:] . norm(x[b,:]) (+ bias[n]) ),  W is an nn.Linear weight [N,K].
  * norm_w != NULL fuses the RMSNorm of x (w * bf16(x * rsqrt(mean(x^2)+eps))) in front.
@@ -78,26 +78,26 @@ int fsvd_linear(const void* x, int64_t ldx, const void* W, int64_t ldw, const vo
 int fsvd_swiglu_linear(const void* p, int64_t ldp, int64_t up_off, const void* gate_u, const void* up_u,
                        int64_t ldw, void* h, int64_t ldh, int B, int D, int R, int mode, int cfg, int dtype, void* stream);
 
-/* The same projection on group-wise int4 weights: y[b,n] = (res[b,n] +) bf16( sum_k norm(x)[b,k] * s[n,g(k)] *
+/* The same projection on group-wise int4 weights: y[b,n] = (res[b,n] +) round( sum_k norm(x)[b,k] * s[n,g(k)] *
  * (q[n,k] - z[n,g(k)]) (+ bias[n]) ).  qweight [N, ldq] bytes holds two columns per byte (even column in the low
  * nibble), scales fp16 and zeros int16 are [N, ldg] with one entry per group_size columns (a power of two >= 32;
  * <= 0 means one group per row): the buffers of the reference's PackedQuantLinear as they are
  * (src/quant/packed_quant_linear.py:18-26 packing, :126-172 quantisation, :284-299 dequantisation, :301-312 forward).
  * The sum runs on the un-rounded s * (q - z) in fp32, which the reference rounds to the activation type first.
- * K must be a multiple of 256; B rows go in slices of four. */
+ * K must be a multiple of 256; B rows go in slices of four.  dtype names the type of x, bias, norm_w, res and y. */
 int fsvd_linear_q4(const void* x, int64_t ldx, const void* qweight, int64_t ldq, const void* scales, const void* zeros,
                    int64_t ldg, int group_size, const void* bias, const void* norm_w, float eps, const void* res,
-                   int64_t ldres, void* y, int64_t ldy, int B, int N, int K, void* stream);
+                   int64_t ldres, void* y, int64_t ldy, int B, int N, int K, int dtype, void* stream);
 
-/* w[n,k] = bf16(s[n,g(k)] * (q[n,k] - z[n,g(k)])): PackedQuantLinear.dequantize for 4 bits and a bf16 result
+/* w[n,k] = round(s[n,g(k)] * (q[n,k] - z[n,g(k)])): PackedQuantLinear.dequantize for 4 bits and a result of type dtype
  * (src/quant/packed_quant_linear.py:284-299); any K and group size. */
 int fsvd_dequant_q4(const void* qweight, int64_t ldq, const void* scales, const void* zeros, int64_t ldg, int group_size,
-                    void* w, int64_t ldw, int N, int K, void* stream);
+                    void* w, int64_t ldw, int N, int K, int dtype, void* stream);
 
 /* fsvd_swiglu_linear on int4 gate_u / up_u [D, R] (same layout for both; rounding modes as above). */
 int fsvd_swiglu_linear_q4(const void* p, int64_t ldp, int64_t up_off, const void* gate_q, const void* gate_scales,
                           const void* gate_zeros, const void* up_q, const void* up_scales, const void* up_zeros, int64_t ldq,
-                          int64_t ldg, int group_size, void* h, int64_t ldh, int B, int D, int R, int mode, void* stream);
+                          int64_t ldg, int group_size, void* h, int64_t ldh, int B, int D, int R, int mode, int dtype, void* stream);
 
 /* Current-token q/k/v from packed rank coefficients p[b] = [Pq|Pk|Pv] and nn.Linear-layout
  * u_proj weights, rotate-half RoPE on q and k at positions[b] (eager bf16 arithmetic), q to
@@ -327,6 +327,7 @@ int fsvd_attn_prefill(const void* q, int64_t sq_b, int64_t sq_m, int64_t sq_h,
 #define FSVD_PH_ARGMAX 5  /* token = argmax of the per-workgroup candidates in `in`; advances the state      */
 
 #define FSVD_WBITS_FP16 (-16) /* fsvd_phase.wbits of a GEMV phase whose weights are float16 (see there)                */
+#define FSVD_WBITS_Q4_FP16 (-4) /* ... whose weights are int4 and whose activations are float16                         */
 
 #define FSVD_EP_STORE 0   /* out0[n] = bf16(dot)                                                              */
 #define FSVD_EP_RESID 1   /* out0[n] = bf16(aux0[n] + bf16(dot))                                              */
@@ -391,13 +392,14 @@ typedef struct fsvd_phase {
   fsvd_tagbuf in, aux0;         /* aux0: residual of EP_RESID                                                  */
   fsvd_tagbuf in2;              /* GEMV with FSVD_PF_STAGE2: the raw hidden state behind `in` (see the flag)   */
   fsvd_tagbuf out0;
-  /* GEMV over group-wise int4 weights (wbits == 4; 0 or 16 = bf16): W[m] is the packed matrix [N, K/2] bytes (two
-   * columns per byte, even column in the low nibble, as PackedQuantLinear.qweight); qsz[m] is uint32 [N, ldg] with
-   * the fp16 scale bits of a group in the low half and (zero point + 128) in the high half; a group is
-   * 32 << gshift columns.  K % 256 == 0.  Arithmetic as fsvd_linear_q4: y = sum_g s_g * sum_k x_k (q_k - z_g), fp32. */
+  /* GEMV over group-wise int4 weights (wbits == 4, or FSVD_WBITS_Q4_FP16 in a float16 step; 0 or 16 = bf16): W[m] is
+   * the packed matrix [N, K/2] bytes (two columns per byte, even column in the low nibble, as
+   * PackedQuantLinear.qweight); qsz[m] is uint32 [N, ldg] with the fp16 scale bits of a group in the low half and
+   * (zero point + 128) in the high half ((zero point + 16) in a float16 step); a group is 32 << gshift columns.  K % 256 == 0.  Arithmetic as fsvd_linear_q4: y = sum_g s_g * sum_k x_k (q_k - z_g), fp32. */
   const void* qsz[2];
-  int32_t ldg, gshift, wbits;   /* wbits also names the element type of a step: FSVD_WBITS_FP16 in EVERY GEMV phase of a list   */
-                                /* makes it a float16 step (vectors, tables, caches and weights float16; no int4 phases)     */
+  int32_t ldg, gshift, wbits;   /* wbits also names the element type of a step: FSVD_WBITS_FP16 (FSVD_WBITS_Q4_FP16 for an   */
+                                /* int4 phase) in EVERY GEMV phase of a list makes it a float16 step (vectors, tables,       */
+                                /* caches and 16-bit weights float16)                                                        */
   int32_t shared_in;            /* nmat == 2: both matrices read the same K-long input (a dense gate / up pair) instead   */
                                 /* of in[0:K] and in[K:2K]                                                                 */
   /* derived by fsvd_decode_step_prepare (do not fill by hand): work items (rows, merge outputs) are

@@ -379,3 +379,132 @@ def test_persistent_step_refuses_mixed_types():
     cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=64, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(ValueError, match="KV cache of the model's type"):
         PersistentDecoder(model, cache)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# group-wise int4 factors under float16 activations: the nibble patterns become float16 values 16 + n
+# ---------------------------------------------------------------------------------------------------------------------
+def _quant(N, K, group, sym=False, seed=0):
+    return O.quantize_weight(rand_fp16(N, K, std=0.05, seed=seed).float(), bits=4, group_size=group, sym=sym)
+
+
+def _ulp_check_f16(got, ref64, what, ulps=1.0):
+    """|got - ref| within ``ulps`` float16 steps at the magnitude of each reference value (the step at 1/32 of the largest
+    value for anything smaller: fp32 accumulation noise does not shrink with the result)."""
+    got, ref = got.double().cpu(), ref64
+    floor = float(ref.abs().max()) / 32.0
+    step = torch.clamp(ref.abs(), min=floor).log2().floor().exp2() * 2.0 ** -10
+    bad = (got - ref).abs() > ulps * step
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} values off by more than {ulps} ulp; worst " \
+                                f"{float(((got - ref).abs() / step).max()):.2f} ulp"
+
+
+@pytest.mark.parametrize("B,N,K,group", [(1, 4096, 1024, 128), (1, 1536, 11008, 128), (3, 1000, 512, 32), (4, 300, 256, -1),
+                                         (7, 520, 1024, 128)])
+def test_linear_q4(ops, B, N, K, group):
+    """Against the module's forward in float16 (weights rounded to float16 first) at the float16 bar, and against the
+    un-rounded sum_k x_k * s * (q - z) in float64, which is what the kernel adds up, within one float16 ulp."""
+    qw, sc, zr = _quant(N, K, group, seed=N + K)
+    x = rand_fp16(B, K, seed=1)
+    got = ops.linear_q4(x.cuda(), qw.cuda(), sc.cuda(), zr.cuda(), group_size=group)
+    close(got, O.quant_linear(x, qw, sc, zr, group_size=group), f"linear_q4 {B}x{N}x{K} g{group}")
+    w64 = O.dequantize_weight(qw, sc, zr, in_features=K, group_size=group, dtype=torch.float64)
+    _ulp_check_f16(got, x.double() @ w64.t(), f"linear_q4 closed form {B}x{N}x{K}")
+
+
+def test_linear_q4_symmetric_bias_norm_residual(ops):
+    B, N, K, group = 2, 768, 1024, 128
+    qw, sc, zr = _quant(N, K, group, sym=True, seed=5)
+    x, bias, res = rand_fp16(B, K, seed=2), rand_fp16(N, seed=3), rand_fp16(B, N, seed=6)
+    nw = (1 + rand_fp16(K, std=0.1, seed=4).float()).to(FP16)
+    out = torch.zeros(B, 2 * N, dtype=FP16, device="cuda")
+    ops.linear_q4(x.cuda(), qw.cuda(), sc.cuda(), zr.cuda(), group_size=group, bias=bias.cuda(), norm_weight=nw.cuda(), eps=1e-5,
+                  residual=res.cuda(), out=out[:, N:])
+    ref = (res.float() + O.quant_linear(O.rms_norm(x, nw, 1e-5), qw, sc, zr, bias, group_size=group).float()).to(FP16)
+    close(out[:, N:], ref, "q4 linear with norm, bias, residual")
+    assert float(out[:, :N].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("B,D,R", [(1, 11008, 1536), (2, 1376, 256)])
+def test_swiglu_q4(ops, mode, B, D, R):
+    gq, gs, gz = _quant(D, R, 128, seed=1)
+    uq, us, uz = _quant(D, R, 128, seed=2)
+    p = rand_fp16(B, 2 * R, seed=3)
+    got = ops.swiglu_linear_q4(p.cuda(), (gq.cuda(), gs.cuda(), gz.cuda()), (uq.cuda(), us.cuda(), uz.cuda()), up_off=R,
+                               group_size=128, mode=mode)
+    wg = O.dequantize_weight(gq, gs, gz, in_features=R, group_size=128, dtype=FP16).float()
+    wu = O.dequantize_weight(uq, us, uz, in_features=R, group_size=128, dtype=FP16).float()
+    g, u = p[:, :R].float() @ wg.t(), p[:, R:].float() @ wu.t()
+    if mode == 0:
+        g, u = g.to(FP16), u.to(FP16)
+        ref = torch.nn.functional.silu(g.float()).to(FP16) * u
+    else:
+        ref = ((g * torch.sigmoid(g)) * u).to(FP16)
+    close(got, ref, f"swiglu_q4 mode {mode}")
+
+
+def test_dequant_q4_is_bit_exact_in_float16(ops):
+    for N, K, group in ((64, 1024, 128), (33, 200, 40), (5, 7, -1), (16, 96, 32)):
+        qw, sc, zr = _quant(N, K, group, seed=K)
+        got = ops.dequant_q4(qw.cuda(), sc.cuda(), zr.cuda(), in_features=K, group_size=group, dtype=FP16)
+        assert got.dtype == FP16
+        assert torch.equal(got.cpu(), O.dequantize_weight(qw, sc, zr, in_features=K, group_size=group, dtype=FP16)), (N, K, group)
+    with pytest.raises(ValueError, match="bfloat16 or torch.float16"):
+        ops.dequant_q4(qw.cuda(), sc.cuda(), zr.cuda(), in_features=K, group_size=group, dtype=torch.float32)
+
+
+def test_quantized_float16_model_decodes_like_the_oracle_on_dequantized_weights(monkeypatch):
+    """Every factor linear of a small float16 model quantised to int4: prompt pass and teacher-forced decode through the
+    per-operator path and through the resident step (phases with FSVD_WBITS_Q4_FP16) against the oracle on the
+    dequantised float16 weights, at the multi-layer bound."""
+    from flashsvd_amd import _lib
+    from flashsvd_amd import quant as Q
+    from flashsvd_amd.runtime.cache import FlashSVDV15DenseKVCache
+    from flashsvd_amd.step import PersistentDecoder, make_persistent_decoder
+    mw = O.make_model(d=1024, n_heads=8, n_kv_heads=4, head_dim=128, ffn=2048, attn_rank=256, mlp_rank=512,
+                      n_layers=2, vocab=2048, dtype=FP16, seed=7)
+    model = model_from_oracle(mw)
+    n = Q.replace_linears_with_packed_quant_inplace(model, module_names=Q.factor_linear_names(model), bits=4, group_size=128, sym=False)
+    assert n == 28
+    for blk, layer in zip(mw.blocks, model.model.layers):
+        for name in ("q", "k", "v", "o"):
+            for f in ("u", "v"):
+                setattr(blk, f"{name}_{f}", getattr(layer.self_attn, f"{name}_{f}_proj").dequantize(dtype=FP16).cpu())
+        for name in ("gate", "up", "down"):
+            for f in ("u", "v"):
+                setattr(blk, f"{name}_{f}", getattr(layer.mlp, f"{name}_{f}_proj").dequantize(dtype=FP16).cpu())
+    prompt = torch.randint(0, 2048, (1, 19), generator=torch.Generator().manual_seed(8))
+    n_new, Lp = 6, 19
+    ref_tok, ref_hid, _ = O.greedy_decode(mw, prompt, n_new, "dense", return_hidden=True)
+
+    def bar(r):
+        m = float(r.abs().max())
+        return dict(abs_tol=3 * (5e-3 if m < 2.0 else 2.0 * m * 2.0 ** -10), rel_tol=7.5e-3)
+
+    cache = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=Lp + n_new + 4, device="cuda", dtype=FP16)
+    out = model(prompt.cuda(), past_key_values=cache, cache_position=torch.arange(Lp))
+    r0 = ref_hid[:, 0].float()
+    assert out.hidden_states.dtype == FP16
+    assert_close_bf16(out.hidden_states[:, -1], r0, "prompt pass hidden state", **bar(r0))
+    for s in range(1, n_new):
+        pos = torch.full((1,), Lp + s - 1, dtype=torch.int32, device="cuda")
+        _, h = model.decode_step(ref_tok[:, s - 1:s].cuda(), cache, pos, return_hidden=True)
+        r = ref_hid[:, s].float()
+        assert_close_bf16(h, r, f"decode hidden state {s}", **bar(r))
+    monkeypatch.setenv("FLASHSVD_AMD_DECODE_ENGINE", "auto")
+    cache2 = FlashSVDV15DenseKVCache(model.config, max_batch_size=1, max_cache_len=Lp + n_new + 4, device="cuda", dtype=FP16)
+    model(prompt.cuda(), past_key_values=cache2, cache_position=torch.arange(Lp))
+    dec = make_persistent_decoder(model, cache2, 1)
+    assert isinstance(dec, PersistentDecoder) and dec.dtype == FP16
+    wb = {int(ph.wbits) for ph in dec.host_phases if int(ph.type) == 1}
+    assert wb == {_lib.WBITS_Q4_FP16, _lib.WBITS_FP16}, wb
+    for s in range(1, n_new):
+        dec.set_state(ref_tok[:, s - 1], Lp + s - 1)
+        dec.step(1)
+        dec.check()
+        r = ref_hid[:, s].float()
+        assert_close_bf16(dec.hidden()[None].cpu(), r, f"resident step, hidden state {s}", **bar(r))
+    kb = bar(cache.key_cache[1].float().cpu())
+    assert_close_bf16(cache2.key_cache[1][:, :Lp + n_new - 1], cache.key_cache[1][:, :Lp + n_new - 1].cpu(),
+                      "K rows of layer 1 vs the per-operator path", **kb)

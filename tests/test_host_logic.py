@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     for name in sorted(declared):
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
     assert declared == set(_lib.SIGNATURES), "ctypes signature table and header disagree"
-    assert lib.fsvd_version() >= 101
+    assert lib.fsvd_version() >= 102
     assert isinstance(lib.fsvd_last_error(), bytes)
     # pure host-side size queries
     assert lib.fsvd_attn_decode_workspace_bytes(1, 32, 128, 8) == 256 * 1024 + 32 * 8 * 130 * 4
