@@ -41,7 +41,7 @@ def _heads_as_linear_layout(V: torch.Tensor) -> torch.Tensor:
 
 
 def _reconstruct_fast(Pq, Pk, Pv, Vq, Vk, Vv, bq, bk, bv):
-    """Shared coefficients (head stride 0), bf16: the head expansion of the product path on nn.Linear-layout twins of the
+    """Shared coefficients (head stride 0), bf16 or fp16: the head expansion of the product path on nn.Linear-layout twins of the
     bases — one launch (fsvd_qkv_rope_append without rotation, K and V written to one-row "caches") when there are no
     biases, else one fused-bias projection per matrix.  Same arithmetic as the reference kernels: fp32 sum (+ bias), one
     rounding (kernels/attn/decode/densekv_reconstruct_triton.py:170-237)."""
@@ -51,7 +51,7 @@ def _reconstruct_fast(Pq, Pk, Pv, Vq, Vk, Vv, bq, bk, bv):
     Hk, Rk, Rv, Dh = Pk.shape[1], Pk.shape[2], Pv.shape[2], Vq.shape[2]
     if os.getenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST", "1") == "0" or Dh not in (64, 128):
         return None
-    if any(t.dtype != torch.bfloat16 for t in (Pq, Pk, Pv, Vq, Vk, Vv)) or any(t.stride(1) != 0 or t.stride(2) != 1 for t in (Pq, Pk, Pv)):
+    if Pq.dtype not in (torch.bfloat16, torch.float16) or any(t.dtype != Pq.dtype for t in (Pk, Pv, Vq, Vk, Vv, bq, bk, bv) if t is not None) or any(t.stride(1) != 0 or t.stride(2) != 1 for t in (Pq, Pk, Pv)):
         return None
     if Rq % 8 or Rk % 8 or Rv % 8:
         return None

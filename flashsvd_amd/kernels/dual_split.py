@@ -104,13 +104,13 @@ def _run(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, b2, *, variant: int, BD: 
 
 
 def _fast_path_ok(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, variant, partials_fp32, s_out) -> bool:
-    """bf16, fp32 partial sums rounded once (v2 / v2_sm80 / pcat_s, and v1 with fp32 partials), no caller workspace:
+    """bf16 or fp16, fp32 partial sums rounded once (v2 / v2_sm80 / pcat_s, and v1 with fp32 partials), no caller workspace:
     the arithmetic of three product-path launches on nn.Linear-layout twins of the operands."""
     if os.getenv("FLASHSVD_AMD_REFERENCE_LAYOUT_FAST", "1") == "0":
         return False
     if s_out is not None or not (variant == 2 or (variant == 1 and partials_fp32)):
         return False
-    if any(t.dtype != torch.bfloat16 for t in (p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU)):
+    if p_up_2d.dtype not in (torch.bfloat16, torch.float16) or any(t.dtype != p_up_2d.dtype for t in (p_gate_2d, GateU, UpU, DownV, DownU)):
         return False
     R, D, Hd = p_up_2d.shape[1], GateU.shape[1], DownU.shape[1]
     return p_up_2d.stride(1) == 1 and p_gate_2d.stride(1) == 1 and R % 8 == 0 and D % 8 == 0 and Hd % 8 == 0
@@ -127,9 +127,9 @@ def _run_fast(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, b2):
     else:
         p = torch.cat([p_gate_2d, p_up_2d], dim=1)
     gate_u, up_u = linear_layout_of(GateU), linear_layout_of(UpU)          # [D, R]
-    h = hip_ops.swiglu_linear(p, gate_u, up_u, up_off=R, mode=1)           # h = bf16(silu(g32) * u32), dual_split_triton.py:207
+    h = hip_ops.swiglu_linear(p, gate_u, up_u, up_off=R, mode=1)           # h = round(silu(g32) * u32), dual_split_triton.py:207
     s = hip_ops.linear(h, linear_layout_of(DownV))                        # S: fp32 sum over D, one rounding (:719-720)
-    return hip_ops.linear(s, linear_layout_of(DownU), None if b2 is None else b2.to(torch.bfloat16).contiguous())
+    return hip_ops.linear(s, linear_layout_of(DownU), None if b2 is None else b2.to(s.dtype).contiguous())
 
 
 def _run_impl(p_up_2d, p_gate_2d, GateU, UpU, DownV, DownU, b2, variant, BD, partials_fp32, s_out):
