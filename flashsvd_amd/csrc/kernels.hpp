@@ -121,6 +121,7 @@ struct RankDecodeArgs {
   float scale;
   float* scores = nullptr; int64_t score_ld = 0;    // the caller's score buffer [B,H,ceil64(S)] fp32 or null; score_ld is set by the launcher
   int dt = 0;                                       // element type: 0 bf16, 1 fp16
+  int split_major = 0;                              // set by the launcher: the splits of a head are neighbours (else the heads of a split)
 };
 size_t rank_decode_scores_floats(int B, int H, int S, int64_t spv_h);
 int launch_rank_decode(const RankDecodeArgs& a, hipStream_t st);

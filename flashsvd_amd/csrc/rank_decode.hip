@@ -46,7 +46,7 @@ template <int KS, bool PKL, bool DEEP, bool SC = false> struct RankDecodeLds {
   static constexpr int kStages = (DEEP || (SC && PKL)) ? 3 : 2;
   static constexpr int kKu = kStages * 128 * 64 * 2, kTb = 4 * kRdMaxChunks * 512 * 4;
   static constexpr int kMain = kKu > kTb ? kKu : kTb;
-  static constexpr int kPkSlots = DEEP ? 2 : 1;
+  static constexpr int kPkSlots = DEEP ? 3 : 1;
   static constexpr int kBytes = kMain + (PKL ? 4 * kPkSlots * KS * 2048 : 0);
 };
 
@@ -79,13 +79,18 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   unsigned char* pkslot = rd_smem + Lds::kMain;                  // [wave][slot][sub-tile][16 keys][128 bytes]
   uint16_t (*kus)[DH][KROW] = reinterpret_cast<uint16_t (*)[DH][KROW]>(smem);
   float (*tbuf)[kRdMaxChunks * 512] = reinterpret_cast<float (*)[kRdMaxChunks * 512]>(smem);
-  float (*qs)[DH] = reinterpret_cast<float (*)[DH]>(smem);         // the queries, before the first k_u chunk takes the place
+  // the queries on their way to registers: in the k_u block before its first chunk takes the place; in the deep form,
+  // whose first chunks are already in flight by then, in the third Pk slot of wave 0 (first written for chunk 2)
+  constexpr bool kLate = DEEP && REP == 1;         // (with several heads per workgroup the registers do not reach)
+  float (*qs)[DH] = reinterpret_cast<float (*)[DH]>(kLate ? pkslot + 2 * KS * 2048 : smem);
 
   const int groups = a.H / a.Hk / REP;             // q-head groups per kv head handled by separate blocks
-  // the head groups of one key range (they read the same cache rows) are neighbours on one XCD
+  // neighbours on one XCD share an L2: the head groups of one key range (they read the same cache rows), or, when the
+  // head bases outweigh the cache rows of the call (short caches, small batches), the key ranges of one head group
   const int GY = gridDim.y;
   const int t = xcd_run_index(blockIdx.x + (int)gridDim.x * (blockIdx.y + GY * blockIdx.z), (int)gridDim.x * GY * gridDim.z);
-  const int gy = t % GY, s = (t / GY) % (int)gridDim.x, b = t / (GY * (int)gridDim.x);
+  const int gy = a.split_major ? (t / (int)gridDim.x) % GY : t % GY;
+  const int s = a.split_major ? t % (int)gridDim.x : (t / GY) % (int)gridDim.x, b = t / (GY * (int)gridDim.x);
   const int hk = gy / groups, grp = gy % groups;
   const int h0 = hk * (a.H / a.Hk) + grp * REP;    // first q head of this block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -97,27 +102,30 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
   per = (per + kRdTileKeys - 1) / kRdTileKeys * kRdTileKeys;
   const int k0 = min(s * per, n_keys), k1 = min(n_keys, k0 + per);
 
-  // queries of this block as fp32 in LDS, rotated at position n_keys-1 when asked to
-  for (int i = tid; i < REP * HALF; i += kRdThreads) {
-    const int g = i / HALF, d = i % HALF;
-    const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)(h0 + g) * a.sq_h;
-    float x0 = E::val(qp[d]), x1 = E::val(qp[d + HALF]);
-    if (a.rotate_q) {
-      const int tp = min(max(n_keys - 1, 0), a.rope_len - 1);
-      const float c = E::val(a.cos[(int64_t)tp * HALF + d]), sn = E::val(a.sin[(int64_t)tp * HALF + d]);
-      const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
-      x0 = r0; x1 = r1;
-    }
-    qs[g][d] = x0 * a.scale;
-    qs[g][d + HALF] = x1 * a.scale;
-  }
-  __syncthreads();
+  // queries of this block as fp32 through LDS into registers, rotated at position n_keys-1 when asked to
   float qv[REP][NT];
+  const auto load_queries = [&]() {
+    for (int i = tid; i < REP * HALF; i += kRdThreads) {
+      const int g = i / HALF, d = i % HALF;
+      const uint16_t* qp = a.q + (int64_t)b * a.sq_b + (int64_t)(h0 + g) * a.sq_h;
+      float x0 = E::val(qp[d]), x1 = E::val(qp[d + HALF]);
+      if (a.rotate_q) {
+        const int tp = min(max(n_keys - 1, 0), a.rope_len - 1);
+        const float c = E::val(a.cos[(int64_t)tp * HALF + d]), sn = E::val(a.sin[(int64_t)tp * HALF + d]);
+        const float r0 = x0 * c - x1 * sn, r1 = x0 * sn + x1 * c;
+        x0 = r0; x1 = r1;
+      }
+      qs[g][d] = x0 * a.scale;
+      qs[g][d + HALF] = x1 * a.scale;
+    }
+    __syncthreads();
 #pragma unroll
-  for (int g = 0; g < REP; ++g)
+    for (int g = 0; g < REP; ++g)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) qv[g][t] = qs[g][(t / 4) * HALF + lr * 4 + (t % 4)];
-  __syncthreads();                                                 // the queries are in registers: the LDS block is free
+      for (int t = 0; t < NT; ++t) qv[g][t] = qs[g][(t / 4) * HALF + lr * 4 + (t % 4)];
+    __syncthreads();                                               // the queries are in registers: the LDS block is free
+  };
+  if constexpr (!kLate) load_queries();                            // (else under the loads of the first chunk)
 
   const int nchunk = (a.Rv + 511) / 512;
   float m_run[REP], l_run[REP];
@@ -203,6 +211,20 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         for (int k = 0; k < 2; ++k)
           af[j][k] = *reinterpret_cast<const frag_t*>(myslot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
     };
+    // deep form, one head per workgroup: the rotation table rows of the wave's keys are requested ahead of the pass over
+    // r (they are needed right behind it, and a first read from memory takes as long as several chunks)
+    constexpr bool kTablesAhead = kLate;
+    uint2 cwp[4], swp[4];
+    if constexpr (kTablesAhead) {
+      if (a.cos) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int pos = min(kt + wave * 16 + lg * 4 + i, a.rope_len - 1);
+          cwp[i] = *reinterpret_cast<const uint2*>(a.cos + (int64_t)pos * HALF + lr * 4);
+          swp[i] = *reinterpret_cast<const uint2*>(a.sin + (int64_t)pos * HALF + lr * 4);
+        }
+      }
+    }
     if constexpr (DEEP) {
       // lane -> LDS row wave * 32 + i * 8 + lane / 8 and position lane % 8 of a stage; the row holds head dimension kd(row)
       // and its position p the piece p ^ row % 8 (the placement store_ku gives the register form)
@@ -221,38 +243,60 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
           __builtin_amdgcn_global_load_lds((gptr_t)(kusrc[i] + c * 64), (lptr_t)(smem + (c % 3) * (DH * KROW * 2) + (wave * 32 + i * 8) * 128), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
-          __builtin_amdgcn_global_load_lds((gptr_t)(prow[0][i] + c * 64), (lptr_t)(myslot + (c & 1) * 2048 + i * 1024), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((gptr_t)(prow[0][i] + c * 64), (lptr_t)(myslot + (c % 3) * 2048 + i * 1024), 16, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       };
       constexpr int kNoLgkm = (7 << 4) | (15 << 8);              // wait on the load counter only
-      constexpr int kNoVm = (7 << 4) | 15 | (3 << 14);           // wait on the LDS counter only
       // (the barrier that ended the previous tile freed every stage and slot)
       issue_group(0);
+      if constexpr (kLate) {
+        if (kt == k0) load_queries();                            // its barriers also wait for chunk 0, which it would have anyway
+      }
       if (nstep > 1) issue_group(1);
       for (int st = 0; st < nstep; ++st) {
         // chunk st has landed once only the group issued after it is outstanding
         if (st + 1 < nstep) __builtin_amdgcn_s_waitcnt(kNoLgkm | kGroup);
         else __builtin_amdgcn_s_waitcnt(kNoLgkm | 0);
         __builtin_amdgcn_sched_barrier(0);
+        // the wave's own Pk fragments: slot st % 3 is next written for chunk st + 3, requested in step st + 1 behind that
+        // step's reads, which these precede in the LDS queue
 #pragma unroll
         for (int k = 0; k < 2; ++k)
-          af[0][k] = *reinterpret_cast<const frag_t*>(myslot + (st & 1) * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
-        __builtin_amdgcn_s_waitcnt(kNoVm | (0 << 8));            // fragments in registers: the slot is free again
+          af[0][k] = *reinterpret_cast<const frag_t*>(myslot + (st % 3) * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
         // everyone's pieces of chunk st are in, and stage (st - 1) % 3 is read out (its fragments fed matrix products that
         // precede this point).  The bare barrier instruction: __syncthreads() carries a fence that waits for ALL of the
         // wave's loads, the chunks requested ahead included
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (st + 2 < nstep) issue_group(st + 2);
         const int cur = st % 3;
+        // all sixteen k_u fragments of the chunk are requested before the first product: read two at a time (what the
+        // compiler makes of a loop that reads and multiplies in turn), the chunk costs eight LDS round trips in a row,
+        // and with one key tile per workgroup nothing else is there to hide them; the requests for chunk st + 2 go out
+        // behind the reads, under their latency
+        // (with several heads per workgroup the rank-space sums leave no registers for that: half a chunk at a time)
+        if constexpr (REP == 1) {
+          frag_t bf[2][NT];
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-          frag_t bf[NT];
+          for (int k = 0; k < 2; ++k)
 #pragma unroll
-          for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+            for (int t = 0; t < NT; ++t) bf[k][t] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+          if (st + 2 < nstep) issue_group(st + 2);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int t = 0; t < NT; ++t) accs[0][t] = E::mfma(af[0][k], bf[t], accs[0][t]);
+          for (int k = 0; k < 2; ++k)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) accs[0][t] = E::mfma(af[0][k], bf[k][t], accs[0][t]);
+        } else {
+          if (st + 2 < nstep) issue_group(st + 2);
+#pragma unroll
+          for (int k = 0; k < 2; ++k) {
+            frag_t bf[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) bf[t] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+#pragma unroll
+            for (int t = 0; t < NT; ++t) accs[0][t] = E::mfma(af[0][k], bf[t], accs[0][t]);
+          }
         }
       }
       __syncthreads();                                           // the last stages are read out before the next tile refills them
@@ -371,8 +415,8 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int pos = min(wkey0 + lg * 4 + i, a.rope_len - 1);
-        const uint2 cw = *reinterpret_cast<const uint2*>(a.cos + (int64_t)pos * HALF + lr * 4);
-        const uint2 sw = *reinterpret_cast<const uint2*>(a.sin + (int64_t)pos * HALF + lr * 4);
+        const uint2 cw = kTablesAhead ? cwp[i] : *reinterpret_cast<const uint2*>(a.cos + (int64_t)pos * HALF + lr * 4);
+        const uint2 sw = kTablesAhead ? swp[i] : *reinterpret_cast<const uint2*>(a.sin + (int64_t)pos * HALF + lr * 4);
         const float cv[4] = {E::lo(cw.x), E::hi(cw.x), E::lo(cw.y), E::hi(cw.y)};
         const float sv[4] = {E::lo(sw.x), E::hi(sw.x), E::lo(sw.y), E::hi(sw.y)};
 #pragma unroll
@@ -424,6 +468,36 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) pk16[j * 4 + i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p[i]), j * 16));
+      if constexpr (REP == 1 && DEEP) {
+        // one head per workgroup, one key tile: eight rows of a 512-column chunk are requested together (left to the
+        // compiler, five or six rows are in flight at a time in a staggered chain of waits)
+#pragma unroll
+        for (int c = 0; c < kRdMaxChunks; ++c) {
+          const int r = c * 512 + lane * 8;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) tacc[g][c][i] *= alpha;
+          if (c < nchunk && r < a.Rv) {
+#pragma unroll
+            for (int k8 = 0; k8 < 16; k8 += 8) {
+              u32x4_t pvr[8];
+#pragma unroll
+              for (int kk = 0; kk < 8; ++kk) pvr[kk] = *reinterpret_cast<const u32x4_t*>(pv_b + (int64_t)min(wkey0 + k8 + kk, k1 - 1) * a.spv_s + r);
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int kk = 0; kk < 8; ++kk) {
+                const u32x4_t v = pvr[kk];
+                const float pw = pk16[k8 + kk];       // 0 for clamped keys
+                tacc[g][c][0] += pw * E::lo(v.x); tacc[g][c][1] += pw * E::hi(v.x);
+                tacc[g][c][2] += pw * E::lo(v.y); tacc[g][c][3] += pw * E::hi(v.y);
+                tacc[g][c][4] += pw * E::lo(v.z); tacc[g][c][5] += pw * E::hi(v.z);
+                tacc[g][c][6] += pw * E::lo(v.w); tacc[g][c][7] += pw * E::hi(v.w);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
+        }
+        continue;
+      }
 #pragma unroll
       for (int c = 0; c < kRdMaxChunks; ++c) {
         const int r = c * 512 + lane * 8;
@@ -964,6 +1038,10 @@ static int launch_rank_decode_t(const RankDecodeArgs& a, hipStream_t st) {
   // depends on the shape and on that argument alone, never on process state.
   const int64_t score_ld = ((int64_t)a.S + 63) / 64 * 64;
   const bool three = a.scores != nullptr && rank_decode_scores_floats(a.B, a.H, a.S, a.spv_h) != 0;
+  // the one-kernel form: which operand the neighbours on an XCD share.  Every workgroup of a head group reads that
+  // group's 128 x Rk rows of k_u, every workgroup of a key range the range's Pk rows: the larger set decides
+  RankDecodeArgs a1 = a;
+  a1.split_major = (int64_t)a.Hk * a.Dh > (int64_t)a.B * a.S && a.spk_h == 0 ? 1 : 0;
   RankDecodeArgs a3 = a;
   a3.scores = three ? a.scores : nullptr;
   a3.score_ld = score_ld;
@@ -985,7 +1063,7 @@ static int launch_rank_decode_t(const RankDecodeArgs& a, hipStream_t st) {
       if (ea != hipSuccess) { set_last_error("%s: cannot reserve %d bytes of LDS: %s", fn, lds, hipGetErrorString(ea)); return kErrLaunch; } \
       granted = true;                                                                                                               \
     }                                                                                                                               \
-    hipLaunchKernelGGL((rank_decode_partial_kernel<DT, REP_, KS_, PKL_, DEEP_>), dim3(a.nsplit, GY_, a.B), block, lds, st, a);          \
+    hipLaunchKernelGGL((rank_decode_partial_kernel<DT, REP_, KS_, PKL_, DEEP_>), dim3(a.nsplit, GY_, a.B), block, lds, st, a1);         \
   } while (0)
 #define FSVD_RD_LAUNCH_SC(REP_, KS_, PKL_, GY_)                                                                                      \
   do {                                                                                                                              \
