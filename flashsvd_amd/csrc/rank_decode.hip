@@ -668,15 +668,37 @@ __global__ __launch_bounds__(kRdPairThreads, 1) void rank_scores_pair_kernel(Ran
 #pragma unroll
         for (int k = 0; k < 2; ++k)
           af[j][k] = *reinterpret_cast<const frag_t*>(slot + j * 2048 + lr * 128 + (((k * 4 + lg) ^ (lr & 7)) * 16));
+      // k_u fragments two at a time, the next two requested before the products of the current two: left to itself the
+      // compiler reads a pair, waits for it and multiplies, and every pair pays an LDS round trip about as long as its
+      // 2 KS products (the launch then sits at half of the matrix cores' time by counter)
+      const auto rd_b = [&](int k, int t) {
+        return __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+      };
+      frag_t bq[2][2];
+      bq[0][0] = rd_b(0, 0);
+      bq[0][1] = rd_b(0, 1);
 #pragma unroll
-      for (int k = 0; k < 2; ++k) {
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const frag_t bf = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
-#pragma unroll
-          for (int j = 0; j < KS; ++j) accs[j][t] = E::mfma(af[j][k], bf, accs[j][t]);
+      for (int it = 0; it < NT; ++it) {            // item = (k, pair of tiles): k = it / 4, tiles 2 (it % 4), + 1
+        const int k = it / (NT / 2), t0 = 2 * (it % (NT / 2));
+        if (it + 1 < NT) {
+          const int kn = (it + 1) / (NT / 2), tn = 2 * ((it + 1) % (NT / 2));
+          bq[(it + 1) & 1][0] = rd_b(kn, tn);
+          bq[(it + 1) & 1][1] = rd_b(kn, tn + 1);
         }
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+          for (int j = 0; j < KS; ++j) accs[j][t0 + tt] = E::mfma(af[j][k], bq[it & 1][tt], accs[j][t0 + tt]);
       }
+      // the order asked of the scheduler: the Pk fragments and the first pair; then, seven times, the next pair's two
+      // reads in front of the current pair's 2 KS products; then the last pair's products
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * KS + 2, 0);
+#pragma unroll
+      for (int it = 0; it + 1 < NT; ++it) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * KS, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 2 * KS, 0);
     }
     __syncthreads();                               // the last chunk is read out before the next tile refills the stages
 #pragma unroll
