@@ -359,15 +359,34 @@ __global__ __launch_bounds__(kRdThreads, 2) void rank_decode_partial_kernel(Rank
         if (st + 2 < nstep) issue_ku(st + 2);
         __builtin_amdgcn_sched_barrier(0);
         const int cur = st % 3;
+        // k_u fragments two at a time, the next two requested before the products of the current two (as in
+        // rank_scores_pair_kernel: left to itself the compiler reads a pair, waits for it and multiplies)
+        const auto rd_b = [&](int k, int t) {
+          return __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
+        };
+        frag_t bq[2][2];
+        bq[0][0] = rd_b(0, 0);
+        bq[0][1] = rd_b(0, 1);
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-#pragma unroll
-          for (int t = 0; t < NT; ++t) {
-            const frag_t bf = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&kus[cur][t * 16 + lr][((k * 4 + lg) ^ (lr & 7)) * 8]));
-#pragma unroll
-            for (int j = 0; j < KS; ++j) accs[j][t] = E::mfma(af[j][k], bf, accs[j][t]);
+        for (int it = 0; it < NT; ++it) {          // item = (k, pair of tiles): k = it / 4, tiles 2 (it % 4), + 1
+          const int k = it / (NT / 2), t0 = 2 * (it % (NT / 2));
+          if (it + 1 < NT) {
+            const int kn = (it + 1) / (NT / 2), tn = 2 * ((it + 1) % (NT / 2));
+            bq[(it + 1) & 1][0] = rd_b(kn, tn);
+            bq[(it + 1) & 1][1] = rd_b(kn, tn + 1);
           }
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int j = 0; j < KS; ++j) accs[j][t0 + tt] = E::mfma(af[j][k], bq[it & 1][tt], accs[j][t0 + tt]);
         }
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);        // the first pair (the Pk fragments are in registers)
+#pragma unroll
+        for (int it = 0; it + 1 < NT; ++it) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 2 * KS, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * KS, 0);
       }
       __syncthreads();                             // the last stages are read out before the next tile refills them
     } else {
