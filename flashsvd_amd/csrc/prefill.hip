@@ -324,6 +324,11 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
   const int vko = (srow * 4) & 31;
   const int vcol = ((srow * 4) & 32) + 8 * ((vko & 15) >> 2) + 4 * (vko >> 4);
   u32x4_t kreg[4], vreg[4];
+  // the padding-mask bytes of a key tile travel with it: requested with the tile (threads 0-63, one key each), parked in
+  // LDS beside it, read from there four keys at a time (read from memory where they apply, each under its own test,
+  // they are sixteen memory round trips in a row per query block and tile)
+  __shared__ __align__(16) uint8_t pms[NG][BN];
+  uint8_t pmreg = 1;
   auto request = [&](int n0) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -331,6 +336,7 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
       kreg[j] = *reinterpret_cast<const u32x4_t*>(kb + (int64_t)kkey * a.sk_s + d0);
       vreg[j] = *reinterpret_cast<const u32x4_t*>(vb + (int64_t)vkey * a.sk_s + d0);
     }
+    if (a.pad_mask && tid < BN) pmreg = a.pad_mask[(int64_t)b * a.spm_b + min(n0 + tid, n_keys_all - 1)];
   };
   if (grp * BN < k_end) request(grp * BN);
 
@@ -339,6 +345,7 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
     const bool live = n0 < k_end;       // the second group may have no tile in the last round; it still meets the barriers
     __syncthreads();   // the previous tile's Ks / Vt are consumed
     if (live) {
+    if (a.pad_mask && tid < BN) pms[grp][tid] = pmreg;
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(&Ks[srow + 16 * j][d0]) = kreg[j];
     {
@@ -380,6 +387,11 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
     const bool plain = !a.pad_mask && !a.add_mask && !rows_ragged && n0 + BN <= n_keys_all &&
                        (!a.causal || n0 + BN - 1 <= q0 + m_base);
     frag_t ph[MI][2], pl[MI][2];     // P^T fragments (high part, residual) of the two 32-key steps
+    uint32_t pmw[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};   // mask bytes of keys n0 + 16 j + 4 lg + (0..3)
+    if (!plain && a.pad_mask) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pmw[j] = *reinterpret_cast<const uint32_t*>(&pms[grp][j * 16 + lg * 4]);
+    }
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi) {
       const int m = m_base + mi * 16 + lr;
@@ -394,7 +406,7 @@ __global__ __launch_bounds__(kPfThreads * NG, NG == 1 ? 2 : 1) void attn_prefill
             const int key = n0 + j * 16 + lg * 4 + i;
             bool ok = key < n_keys_all && m < a.M;
             if (a.causal) ok = ok && key <= qpos;
-            if (ok && a.pad_mask) ok = a.pad_mask[(int64_t)b * a.spm_b + key] != 0;
+            ok = ok && ((pmw[j] >> (8 * i)) & 0xffu) != 0;
             if (!ok) v = -INFINITY;                    // mask first, then the additive term, as the reference kernel
             else if (a.add_mask) v += a.add_mask[(int64_t)b * a.sam_b + (int64_t)m * a.sam_q + key];
           }
